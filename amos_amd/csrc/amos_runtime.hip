@@ -1,0 +1,399 @@
+// Host side of libamos_mi355x.so: descriptor validation, kernel-instance
+// dispatch, launch, timing.  The C ABI is declared in include/amos_mi355x.h.
+#include <hip/hip_runtime.h>
+
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+#include <mutex>
+#include <string>
+
+#include "amos_mi355x.h"
+#include "igemm_instances.h"
+#include "mapper.h"
+
+namespace amos {
+
+static thread_local char g_err[512] = "";
+
+int set_error(int code, const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_err, sizeof(g_err), fmt, ap);
+  va_end(ap);
+  return code;
+}
+
+#define HIP_TRY(expr)                                                                   \
+  do {                                                                                  \
+    hipError_t e_ = (expr);                                                             \
+    if (e_ != hipSuccess)                                                               \
+      return set_error(AMOS_ERR_HIP, "%s failed: %s", #expr, hipGetErrorString(e_));    \
+  } while (0)
+
+template <typename T>
+__global__ void fill_zero_kernel(T* p, int64_t rows, int64_t cols, int64_t ld) {
+  int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  int64_t n = rows * cols;
+  for (; idx < n; idx += (int64_t)gridDim.x * blockDim.x) p[(idx / cols) * ld + idx % cols] = 0;
+}
+
+// ---- kernel instance table (defined in inst_*.hip) -------------------------------------
+static Instance* pick(int dt, int rl, int cl, int ti, int tj) {
+  switch (dt * 2 + (rl == LD_STRIDED)) {
+    case DT_F16 * 2: return pick_f16_vec(cl, ti, tj);
+    case DT_F16 * 2 + 1: return pick_f16_strided(cl, ti, tj);
+    case DT_BF16 * 2: return pick_bf16_vec(cl, ti, tj);
+    case DT_BF16 * 2 + 1: return pick_bf16_strided(cl, ti, tj);
+    case DT_I8 * 2: return pick_i8_vec(cl, ti, tj);
+    case DT_I8 * 2 + 1: return pick_i8_strided(cl, ti, tj);
+  }
+  return nullptr;
+}
+
+// ---- descriptor -> launch plan --------------------------------------------------------
+struct Plan {
+  IgemmParams p;
+  int dt, rl, cl;
+  amos_kernel_config_t cfg;
+  int64_t batch;
+  int split;
+  // zero fill of the output before a split-K launch
+  int64_t fill_rows, fill_cols, fill_ld;
+};
+
+static int dtype_pair(int in_dtype, int out_dtype, int* dt) {
+  if (in_dtype == AMOS_F16 && out_dtype == AMOS_F32) { *dt = DT_F16; return 0; }
+  if (in_dtype == AMOS_BF16 && out_dtype == AMOS_F32) { *dt = DT_BF16; return 0; }
+  if (in_dtype == AMOS_I8 && out_dtype == AMOS_I32) { *dt = DT_I8; return 0; }
+  return set_error(AMOS_ERR_UNSUPPORTED,
+                   "unsupported dtype pair in=%d out=%d (f16->f32, bf16->f32, i8->i32 exist)",
+                   in_dtype, out_dtype);
+}
+
+static bool aligned16(const void* p) { return ((uintptr_t)p & 15) == 0; }
+
+static int fits_int(int64_t v) { return v > 0 && v < (int64_t)1 << 31; }
+
+static int plan_finish(Plan& pl, int op, const void* desc, const amos_kernel_config_t* cfg) {
+  amos_kernel_config_t c;
+  if (cfg && cfg->tile_i > 0 && cfg->tile_j > 0) {
+    c = *cfg;
+    if (c.split_k < 1) c.split_k = 1;
+  } else {
+    int rc = amos_default_config(op, desc, &c);
+    if (rc) return rc;
+    if (cfg && cfg->split_k > 0) c.split_k = cfg->split_k;
+  }
+  pl.cfg = c;
+  const int es = pl.dt == DT_I8 ? 1 : 2;
+  const int bke = 128 / es;
+  IgemmParams& p = pl.p;
+  p.k_tiles = (p.Kred + bke - 1) / bke;
+  int split = c.split_k;
+  if (split > p.k_tiles) split = p.k_tiles;
+  p.k_tiles_per_split = (p.k_tiles + split - 1) / split;
+  split = (p.k_tiles + p.k_tiles_per_split - 1) / p.k_tiles_per_split;
+  pl.split = split;
+  p.atomic_out = split > 1;
+  p.tiles_i = (p.I + c.tile_i - 1) / c.tile_i;
+  p.tiles_j = (p.J + c.tile_j - 1) / c.tile_j;
+  if ((int64_t)p.tiles_i * p.tiles_j >= ((int64_t)1 << 31))
+    return set_error(AMOS_ERR_BAD_ARG, "too many tiles");
+  if (split > 65535 || pl.batch > 65535)
+    return set_error(AMOS_ERR_UNSUPPORTED, "batch (%lld) or split_k (%d) above 65535",
+                     (long long)pl.batch, split);
+  return 0;
+}
+
+static int plan_gemm(Plan& pl, int op, const void* desc_any, const amos_gemm_desc_t* d,
+                     int64_t batch, int64_t sa, int64_t sb, int64_t sc,
+                     const amos_kernel_config_t* cfg, const void* A, const void* B, void* C) {
+  if (!d || !A || !B || !C) return set_error(AMOS_ERR_BAD_ARG, "null pointer argument");
+  if (!fits_int(d->M) || !fits_int(d->N) || !fits_int(d->K) || batch <= 0)
+    return set_error(AMOS_ERR_BAD_ARG, "extents must be in [1, 2^31): M=%lld N=%lld K=%lld batch=%lld",
+                     (long long)d->M, (long long)d->N, (long long)d->K, (long long)batch);
+  int rc = dtype_pair(d->in_dtype, d->out_dtype, &pl.dt);
+  if (rc) return rc;
+  const int64_t min_lda = d->trans_a ? d->M : d->K;
+  const int64_t min_ldb = d->trans_b ? d->K : d->N;
+  if (d->lda < min_lda || d->ldb < min_ldb || d->ldc < d->N)
+    return set_error(AMOS_ERR_BAD_ARG, "leading dimension too small (lda=%lld ldb=%lld ldc=%lld)",
+                     (long long)d->lda, (long long)d->ldb, (long long)d->ldc);
+  const int es = pl.dt == DT_I8 ? 1 : 2;
+  const int ce = 16 / es;
+  IgemmParams& p = pl.p;
+  memset(&p, 0, sizeof(p));
+  p.I = (int)d->M;
+  p.J = (int)d->N;
+  p.Kred = (int)d->K;
+  p.row_base = (const char*)A;
+  p.col_base = (const char*)B;
+  p.row_batch = sa;
+  p.col_batch = sb;
+  if (d->trans_a) { p.row_s_row = 1; p.row_s_k = d->lda; } else { p.row_s_row = d->lda; p.row_s_k = 1; }
+  if (d->trans_b) { p.col_s_row = d->ldb; p.col_s_k = 1; } else { p.col_s_row = 1; p.col_s_k = d->ldb; }
+  auto vec_ok = [&](const void* base, int64_t s_row, int64_t s_k, int64_t bstride) {
+    return s_k == 1 && aligned16(base) && (s_row % ce) == 0 && (d->K % ce) == 0 &&
+           (batch == 1 || (bstride % ce) == 0);
+  };
+  pl.rl = vec_ok(A, p.row_s_row, p.row_s_k, sa) ? LD_VEC : LD_STRIDED;
+  pl.cl = vec_ok(B, p.col_s_row, p.col_s_k, sb) ? LD_VEC : LD_STRIDED;
+  p.out = (char*)C;
+  p.out_si = d->ldc;
+  p.out_sjo = 0;
+  p.out_jmod = 0x7fffffff;
+  p.out_batch = sc;
+  pl.batch = batch;
+  pl.fill_rows = d->M;
+  pl.fill_cols = d->N;
+  pl.fill_ld = d->ldc;
+  return plan_finish(pl, op, desc_any, cfg);
+}
+
+static int conv_out_extent(int64_t in, int pad, int dil, int64_t k, int stride) {
+  int64_t eff = (k - 1) * dil + 1;
+  int64_t o = (in + 2 * (int64_t)pad - eff) / stride + 1;
+  if (in + 2 * (int64_t)pad < eff) return 0;
+  return (int)o;
+}
+
+static int plan_conv(Plan& pl, int op, const amos_conv_desc_t* d, const amos_kernel_config_t* cfg,
+                     const void* X, const void* Wt, void* Y) {
+  if (!d || !X || !Wt || !Y) return set_error(AMOS_ERR_BAD_ARG, "null pointer argument");
+  amos_conv_desc_t c = *d;
+  if (op == AMOS_OP_CONV2D) {
+    if (c.D > 1 || c.T > 1) return set_error(AMOS_ERR_BAD_ARG, "conv2d needs D = T = 1");
+    c.D = 1; c.T = 1; c.stride_d = 1; c.pad_d = 0; c.dil_d = 1;
+  }
+  if (c.N <= 0 || c.C <= 0 || c.D <= 0 || c.H <= 0 || c.W <= 0 || c.K <= 0 || c.T <= 0 ||
+      c.R <= 0 || c.S <= 0 || c.stride_d <= 0 || c.stride_h <= 0 || c.stride_w <= 0 ||
+      c.dil_d <= 0 || c.dil_h <= 0 || c.dil_w <= 0 || c.pad_d < 0 || c.pad_h < 0 || c.pad_w < 0)
+    return set_error(AMOS_ERR_BAD_ARG, "conv extents, strides and dilations must be positive, pads >= 0");
+  int rc = dtype_pair(c.in_dtype, c.out_dtype, &pl.dt);
+  if (rc) return rc;
+  int OD = conv_out_extent(c.D, c.pad_d, c.dil_d, c.T, c.stride_d);
+  int OP = conv_out_extent(c.H, c.pad_h, c.dil_h, c.R, c.stride_h);
+  int OQ = conv_out_extent(c.W, c.pad_w, c.dil_w, c.S, c.stride_w);
+  if (OD <= 0 || OP <= 0 || OQ <= 0)
+    return set_error(AMOS_ERR_BAD_ARG, "kernel window larger than the padded input");
+  int64_t J = c.N * OD * (int64_t)OP * OQ;
+  int64_t Kred = c.C * c.T * c.R * c.S;
+  int64_t per_image = c.C * c.D * c.H * c.W;
+  if (!fits_int(J) || !fits_int(Kred) || !fits_int(per_image) || !fits_int(c.K))
+    return set_error(AMOS_ERR_UNSUPPORTED, "conv extents above 2^31");
+  if ((c.T - 1) * c.dil_d >= 1024 || (c.R - 1) * c.dil_h >= 1024 || (c.S - 1) * c.dil_w >= 1024)
+    return set_error(AMOS_ERR_UNSUPPORTED, "dilated kernel extent above 1023");
+  const int es = pl.dt == DT_I8 ? 1 : 2;
+  const int ce = 16 / es;
+  IgemmParams& p = pl.p;
+  memset(&p, 0, sizeof(p));
+  p.I = (int)c.K;
+  p.J = (int)J;
+  p.Kred = (int)Kred;
+  p.row_base = (const char*)Wt;
+  p.row_s_row = Kred;
+  p.row_s_k = 1;
+  pl.rl = (aligned16(Wt) && Kred % ce == 0) ? LD_VEC : LD_STRIDED;
+  p.col_base = (const char*)X;
+  pl.cl = LD_CONV;
+  ConvGeom& g = p.g;
+  g.C = (int)c.C; g.D = (int)c.D; g.H = (int)c.H; g.W = (int)c.W;
+  g.T = (int)c.T; g.R = (int)c.R; g.S = (int)c.S;
+  g.sd = c.stride_d; g.sh = c.stride_h; g.sw = c.stride_w;
+  g.pd = c.pad_d; g.ph = c.pad_h; g.pw = c.pad_w;
+  g.dd = c.dil_d; g.dh = c.dil_h; g.dw = c.dil_w;
+  g.OD = OD; g.OP = OP; g.OQ = OQ;
+  g.use_mask = (c.T * c.R * c.S <= 64) ? 1 : 0;
+  int64_t odpq = (int64_t)OD * OP * OQ;
+  p.out = (char*)Y;
+  p.out_si = odpq;
+  p.out_sjo = c.K * odpq;
+  p.out_jmod = (int)odpq;
+  p.out_batch = 0;
+  pl.batch = 1;
+  pl.fill_rows = 1;
+  pl.fill_cols = c.N * c.K * odpq;
+  pl.fill_ld = pl.fill_cols;
+  return plan_finish(pl, op, d, cfg);
+}
+
+static int make_plan(Plan& pl, int op, const void* desc, const amos_kernel_config_t* cfg,
+                     const void* in0, const void* in1, void* out) {
+  switch (op) {
+    case AMOS_OP_GEMM:
+      return plan_gemm(pl, op, desc, (const amos_gemm_desc_t*)desc, 1, 0, 0, 0, cfg, in0, in1, out);
+    case AMOS_OP_BGEMM: {
+      const amos_bgemm_desc_t* b = (const amos_bgemm_desc_t*)desc;
+      if (!b) return set_error(AMOS_ERR_BAD_ARG, "null descriptor");
+      return plan_gemm(pl, op, desc, &b->g, b->batch, b->stride_a, b->stride_b, b->stride_c, cfg,
+                       in0, in1, out);
+    }
+    case AMOS_OP_CONV2D:
+    case AMOS_OP_CONV3D:
+      return plan_conv(pl, op, (const amos_conv_desc_t*)desc, cfg, in0, in1, out);
+  }
+  return set_error(AMOS_ERR_BAD_ARG, "unknown op %d", op);
+}
+
+static int resolve(const Plan& pl, Instance** out) {
+  Instance* inst = pick(pl.dt, pl.rl, pl.cl, pl.cfg.tile_i, pl.cfg.tile_j);
+  if (!inst)
+    return set_error(AMOS_ERR_INFEASIBLE, "no kernel instance with block tile %dx%d",
+                     pl.cfg.tile_i, pl.cfg.tile_j);
+  *out = inst;
+  return 0;
+}
+
+static int launch(const Plan& pl, hipStream_t stream) {
+  Instance* inst;
+  int rc = resolve(pl, &inst);
+  if (rc) return rc;
+  hipError_t attr_err = hipSuccess;
+  std::call_once(inst->once, [&] {
+    attr_err = hipFuncSetAttribute((const void*)inst->fn, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                   (int)inst->lds);
+  });
+  if (attr_err != hipSuccess)
+    return set_error(AMOS_ERR_HIP, "hipFuncSetAttribute(%s, %zu B LDS): %s", inst->name, inst->lds,
+                     hipGetErrorString(attr_err));
+  if (pl.split > 1) {
+    int64_t n = pl.fill_rows * pl.fill_cols * pl.batch;
+    int blocks = (int)((n + 255) / 256 < 4096 ? (n + 255) / 256 : 4096);
+    // batched outputs are contiguous per batch only when stride_c == M*ldc; fill per batch
+    for (int64_t b = 0; b < pl.batch; ++b) {
+      char* base = pl.p.out + b * pl.p.out_batch * 4;
+      if (pl.dt == DT_I8)
+        hipLaunchKernelGGL(fill_zero_kernel<int>, dim3(blocks), dim3(256), 0, stream, (int*)base,
+                           pl.fill_rows, pl.fill_cols, pl.fill_ld);
+      else
+        hipLaunchKernelGGL(fill_zero_kernel<float>, dim3(blocks), dim3(256), 0, stream,
+                           (float*)base, pl.fill_rows, pl.fill_cols, pl.fill_ld);
+    }
+  }
+  dim3 grid((unsigned)(pl.p.tiles_i * pl.p.tiles_j), (unsigned)pl.split, (unsigned)pl.batch);
+  hipLaunchKernelGGL(inst->fn, grid, dim3(256), inst->lds, stream, pl.p);
+  HIP_TRY(hipGetLastError());
+  return 0;
+}
+
+static int run_op(int op, const void* desc, const amos_kernel_config_t* cfg, const void* in0,
+                  const void* in1, void* out, void* stream) {
+  Plan pl;
+  int rc = make_plan(pl, op, desc, cfg, in0, in1, out);
+  if (rc) return rc;
+  return launch(pl, (hipStream_t)stream);
+}
+
+}  // namespace amos
+
+using namespace amos;
+
+extern "C" {
+
+int amos_version(void) { return AMOS_ABI_VERSION; }
+const char* amos_last_error(void) { return g_err; }
+
+int amos_device_info(amos_device_info_t* out) {
+  if (!out) return set_error(AMOS_ERR_BAD_ARG, "null pointer argument");
+  int dev = 0;
+  HIP_TRY(hipGetDevice(&dev));
+  hipDeviceProp_t prop;
+  HIP_TRY(hipGetDeviceProperties(&prop, dev));
+  memset(out, 0, sizeof(*out));
+  out->compute_units = prop.multiProcessorCount;
+  out->wave_size = prop.warpSize;
+  out->max_clock_khz = prop.clockRate;
+  out->lds_bytes_per_block = (int32_t)prop.sharedMemPerBlockOptin ? (int32_t)prop.sharedMemPerBlockOptin
+                                                                  : (int32_t)prop.sharedMemPerBlock;
+  out->hbm_bytes = (int64_t)prop.totalGlobalMem;
+  snprintf(out->arch, sizeof(out->arch), "%s", prop.gcnArchName);
+  double clk = prop.clockRate * 1e3;
+  out->peak_tflops_f16 = prop.multiProcessorCount * clk * 4096.0 / 1e12;
+  out->peak_tops_i8 = prop.multiProcessorCount * clk * 8192.0 / 1e12;
+  return 0;
+}
+
+int amos_gemm(const amos_gemm_desc_t* desc, const amos_kernel_config_t* cfg, const void* A,
+              const void* B, void* C, void* workspace, size_t ws_bytes, void* stream) {
+  (void)workspace; (void)ws_bytes;
+  return run_op(AMOS_OP_GEMM, desc, cfg, A, B, C, stream);
+}
+int amos_bgemm(const amos_bgemm_desc_t* desc, const amos_kernel_config_t* cfg, const void* A,
+               const void* B, void* C, void* workspace, size_t ws_bytes, void* stream) {
+  (void)workspace; (void)ws_bytes;
+  return run_op(AMOS_OP_BGEMM, desc, cfg, A, B, C, stream);
+}
+int amos_conv2d(const amos_conv_desc_t* desc, const amos_kernel_config_t* cfg, const void* X,
+                const void* Wt, void* Y, void* workspace, size_t ws_bytes, void* stream) {
+  (void)workspace; (void)ws_bytes;
+  return run_op(AMOS_OP_CONV2D, desc, cfg, X, Wt, Y, stream);
+}
+int amos_conv3d(const amos_conv_desc_t* desc, const amos_kernel_config_t* cfg, const void* X,
+                const void* Wt, void* Y, void* workspace, size_t ws_bytes, void* stream) {
+  (void)workspace; (void)ws_bytes;
+  return run_op(AMOS_OP_CONV3D, desc, cfg, X, Wt, Y, stream);
+}
+
+size_t amos_workspace_bytes(int op, const void* desc, const amos_kernel_config_t* cfg) {
+  (void)op; (void)desc; (void)cfg;
+  return 0;  // split-K accumulates straight into the (zero-filled) output
+}
+
+const char* amos_kernel_name(int op, const void* desc, const amos_kernel_config_t* cfg) {
+  // pointers only matter for their alignment here; use aligned dummies
+  static char dummy[16] __attribute__((aligned(16)));
+  Plan pl;
+  if (make_plan(pl, op, desc, cfg, dummy, dummy, dummy)) return nullptr;
+  Instance* inst;
+  if (resolve(pl, &inst)) return nullptr;
+  return inst->name;
+}
+
+int amos_time(int op, const void* desc, const amos_kernel_config_t* cfg, const void* in0,
+              const void* in1, void* out, void* workspace, size_t ws_bytes, void* stream_v,
+              int number, int repeat, int min_repeat_ms, double* out_seconds) {
+  (void)workspace; (void)ws_bytes;
+  if (!out_seconds || number < 1 || repeat < 1)
+    return set_error(AMOS_ERR_BAD_ARG, "amos_time needs number >= 1, repeat >= 1 and an output array");
+  hipStream_t stream = (hipStream_t)stream_v;
+  Plan pl;
+  int rc = make_plan(pl, op, desc, cfg, in0, in1, out);
+  if (rc) return rc;
+  rc = launch(pl, stream);  // warm-up
+  if (rc) return rc;
+  HIP_TRY(hipStreamSynchronize(stream));
+  hipEvent_t e0, e1;
+  HIP_TRY(hipEventCreate(&e0));
+  HIP_TRY(hipEventCreate(&e1));
+  long long n = number;  // like the reference, a grown `number` carries over to later repeats
+  for (int r = 0; r < repeat; ++r) {
+    double ms = 0.0;
+    for (;;) {
+      if (ms > 0.0) {
+        double want = (double)min_repeat_ms / (ms / (double)n) + 1.0;
+        double grown = (double)n * 1.618;
+        double nn = want > grown ? want : grown;
+        if (nn > 1e8) nn = 1e8;
+        n = (long long)nn;
+      }
+      HIP_TRY(hipEventRecord(e0, stream));
+      for (long long i = 0; i < n; ++i) {
+        rc = launch(pl, stream);
+        if (rc) return rc;
+      }
+      HIP_TRY(hipEventRecord(e1, stream));
+      HIP_TRY(hipEventSynchronize(e1));
+      float f = 0.f;
+      HIP_TRY(hipEventElapsedTime(&f, e0, e1));
+      ms = f;
+      if (ms >= (double)min_repeat_ms || n >= 100000000LL) break;
+    }
+    out_seconds[r] = ms * 1e-3 / (double)n;
+  }
+  (void)hipEventDestroy(e0);
+  (void)hipEventDestroy(e1);
+  return 0;
+}
+
+}  // extern "C"

@@ -1,0 +1,62 @@
+// Kernel-instance table: one translation unit per (dtype, row loader) pair keeps
+// the build parallel.  Each unit defines pick_<dtype>_<loader>(col loader, tile).
+#pragma once
+#include <mutex>
+#include <string>
+
+#include "igemm_kernel.h"
+
+namespace amos {
+
+typedef void (*igemm_fn)(const IgemmParams);
+
+struct Instance {
+  igemm_fn fn;
+  size_t lds;
+  const char* name;
+  std::once_flag once;  // guards the one-time LDS-size attribute call
+};
+
+template <int DT, int RL, int CL, int TI, int TJ>
+Instance* instance() {
+  static Instance inst;
+  static const char* dtn[] = {"f16", "bf16", "i8"};
+  static const char* ldn[] = {"vec", "strided", "im2col"};
+  static std::string name = std::string("amos_igemm<") + dtn[DT] + "," + ldn[RL] + "," + ldn[CL] +
+                            "," + std::to_string(64 * TI) + "x" + std::to_string(64 * TJ) + ">";
+  inst.fn = amos_igemm<DT, RL, CL, TI, TJ>;
+  inst.lds = igemm_lds_bytes<TI, TJ>();
+  inst.name = name.c_str();
+  return &inst;
+}
+
+template <int DT, int RL, int CL>
+Instance* pick_tile(int ti, int tj) {
+  if (ti == 64 && tj == 64) return instance<DT, RL, CL, 1, 1>();
+  if (ti == 128 && tj == 128) return instance<DT, RL, CL, 2, 2>();
+  if (ti == 256 && tj == 256) return instance<DT, RL, CL, 4, 4>();
+  if (ti == 128 && tj == 64) return instance<DT, RL, CL, 2, 1>();
+  if (ti == 64 && tj == 128) return instance<DT, RL, CL, 1, 2>();
+  if (ti == 256 && tj == 128) return instance<DT, RL, CL, 4, 2>();
+  if (ti == 128 && tj == 256) return instance<DT, RL, CL, 2, 4>();
+  return nullptr;
+}
+
+template <int DT, int RL>
+Instance* pick_col(int cl, int ti, int tj) {
+  switch (cl) {
+    case LD_VEC: return pick_tile<DT, RL, LD_VEC>(ti, tj);
+    case LD_STRIDED: return pick_tile<DT, RL, LD_STRIDED>(ti, tj);
+    case LD_CONV: return pick_tile<DT, RL, LD_CONV>(ti, tj);
+  }
+  return nullptr;
+}
+
+Instance* pick_f16_vec(int cl, int ti, int tj);
+Instance* pick_f16_strided(int cl, int ti, int tj);
+Instance* pick_bf16_vec(int cl, int ti, int tj);
+Instance* pick_bf16_strided(int cl, int ti, int tj);
+Instance* pick_i8_vec(int cl, int ti, int tj);
+Instance* pick_i8_strided(int cl, int ti, int tj);
+
+}  // namespace amos

@@ -1,0 +1,419 @@
+// Implicit-GEMM kernel family for gfx950 (MI355X), 64-lane wavefronts.
+//
+// One kernel template covers GEMM, batched GEMM and conv2d/conv3d.  The problem
+// is always   Out(i, j) = sum_k Row(i, k) * Col(j, k)
+// with i on the MFMA row side, j on the MFMA column side (the lane-fast,
+// hence coalesced, direction of the accumulator) and k the fused reduction:
+//
+//   GEMM   : i = m, j = n, Row = A, Col = B                 (C row-major)
+//   conv   : i = output channel, j = (image, od, op, oq) fused, k = (c, t, r, s)
+//            Row = weights KCTRS (k is contiguous there), Col = im2col view of
+//            NCDHW activations computed on the fly, Out = NKDPQ
+//
+// It is what the reference's generated "kernel2" does (global->shared copy,
+// load_matrix_sync, mma_sync chain, store_matrix_sync; reference: README.md:344-424,
+// python/tvm/auto_tensorize/tensorization_phases/schedulers/cuda_v2.py:582-825)
+// with the separate im2col, relayout and scatter kernels
+// (reference: src/auto_tensorize/compute_transform.cc:181-293,439-497) folded
+// into the loader and the epilogue.
+//
+// Block = 256 threads = 4 waves in a 2x2 arrangement; every wave owns TI x TJ
+// MFMA 32x32 accumulator tiles, so the block tile is (64*TI) x (64*TJ).
+// K advances 128 bytes per row per step (64 halves / 128 int8).  Tiles are staged
+// in LDS as rows of eight 16-byte chunks with an XOR swizzle of the chunk index,
+// double buffered with register prefetch of the next K step.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace amos {
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v16i __attribute__((ext_vector_type(16)));
+typedef float v16f __attribute__((ext_vector_type(16)));
+typedef _Float16 v8h __attribute__((ext_vector_type(8)));
+typedef __bf16 v8bf __attribute__((ext_vector_type(8)));
+
+enum { DT_F16 = 0, DT_BF16 = 1, DT_I8 = 2 };
+enum { LD_VEC = 0, LD_STRIDED = 1, LD_CONV = 2 };
+
+// v_mfma 32x32 with 32 bytes of K per row per issue.  Operand fragment layout:
+// lane l holds the 16 bytes  k-bytes [16*(l/32), 16*(l/32)+16)  of row (l%32) for
+// the first operand and of column (l%32) for the second; accumulator register r
+// of lane l is element (i = 8*(r/4) + 4*(l/32) + r%4, j = l%32).
+template <int DT>
+struct Mfma;
+template <>
+struct Mfma<DT_F16> {
+  typedef v16f acc_t;
+  typedef float out_t;
+  static constexpr int ES = 2;
+  static __device__ __forceinline__ acc_t run(v4i a, v4i b, acc_t c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(v8h, a),
+                                                  __builtin_bit_cast(v8h, b), c, 0, 0, 0);
+  }
+};
+template <>
+struct Mfma<DT_BF16> {
+  typedef v16f acc_t;
+  typedef float out_t;
+  static constexpr int ES = 2;
+  static __device__ __forceinline__ acc_t run(v4i a, v4i b, acc_t c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8bf, a),
+                                                   __builtin_bit_cast(v8bf, b), c, 0, 0, 0);
+  }
+};
+template <>
+struct Mfma<DT_I8> {
+  typedef v16i acc_t;
+  typedef int out_t;
+  static constexpr int ES = 1;
+  static __device__ __forceinline__ acc_t run(v4i a, v4i b, acc_t c) {
+    return __builtin_amdgcn_mfma_i32_32x32x32_i8(a, b, c, 0, 0, 0);
+  }
+};
+
+struct ConvGeom {
+  int C, D, H, W;
+  int T, R, S;
+  int sd, sh, sw;
+  int pd, ph, pw;
+  int dd, dh, dw;
+  int OD, OP, OQ;
+  int use_mask;  // T*R*S <= 64: per-row tap validity bitmask instead of compares
+};
+
+struct IgemmParams {
+  int I, J, Kred;         // extents in elements
+  int k_tiles;            // ceil(Kred / elements per K step)
+  int k_tiles_per_split;  // K steps one blockIdx.y handles
+  int tiles_i, tiles_j;
+  // row operand
+  const char* row_base;
+  int64_t row_s_row, row_s_k;   // element strides (LD_VEC: row_s_k == 1)
+  int64_t row_batch;            // elements between batches
+  // column operand
+  const char* col_base;
+  int64_t col_s_row, col_s_k;
+  int64_t col_batch;
+  ConvGeom g;                   // LD_CONV only
+  // output: element (i, j) at  i*out_si + (j / out_jmod)*out_sjo + j % out_jmod
+  char* out;
+  int64_t out_si, out_sjo;
+  int out_jmod;
+  int64_t out_batch;
+  int atomic_out;               // split-K: accumulate into a zeroed output
+};
+
+__device__ __forceinline__ int lds_chunk_offset(int row, int chunk) {
+  return row * 128 + ((chunk ^ ((row ^ (row >> 3)) & 7)) << 4);
+}
+
+// Workgroups are dealt round-robin to the 8 XCDs, each with its own L2.  Give
+// every XCD a contiguous range of logical tile ids, then walk tiles in column
+// groups so that concurrently running blocks share row / column panels.
+__device__ __forceinline__ void block_to_tile(int wg, int n_wg, int tiles_i, int tiles_j, int& ti,
+                                              int& tj) {
+  int logical = wg;
+  if ((n_wg & 7) == 0) logical = (wg & 7) * (n_wg >> 3) + (wg >> 3);
+  const int GROUP = 8;  // tile rows per group
+  int per_group = GROUP * tiles_j;
+  int gidx = logical / per_group;
+  int first_i = gidx * GROUP;
+  int rows_here = tiles_i - first_i < GROUP ? tiles_i - first_i : GROUP;
+  int in_group = logical - gidx * per_group;
+  ti = first_i + in_group % rows_here;
+  tj = in_group / rows_here;
+}
+
+template <int DT, int RL, int CL, int TI, int TJ>
+__global__ __launch_bounds__(256) void amos_igemm(const IgemmParams p) {
+  typedef Mfma<DT> MM;
+  typedef typename MM::acc_t acc_t;
+  typedef typename MM::out_t out_t;
+  constexpr int ES = MM::ES;
+  constexpr int CE = 16 / ES;     // elements per 16-byte chunk
+  constexpr int BKE = 128 / ES;   // elements of K per step
+  constexpr int BI = 64 * TI, BJ = 64 * TJ;
+  constexpr int NR = BI / 32, NC = BJ / 32;  // 16-byte chunks per thread per step
+  static_assert(RL != LD_CONV, "the row operand is never an im2col view");
+
+  extern __shared__ __attribute__((aligned(16))) char smem[];
+  char* const sR = smem;                       // [2][BI*128]
+  char* const sC = smem + 2 * BI * 128;        // [2][BJ*128]
+  int2* const sT = (int2*)(smem + 2 * (BI + BJ) * 128);  // [2][BKE] (LD_CONV)
+
+  const int t = threadIdx.x;
+  const int lane = t & 63;
+  const int wave = t >> 6;
+  const int wi = wave >> 1, wj = wave & 1;
+
+  int tile_i, tile_j;
+  block_to_tile(blockIdx.x, gridDim.x, p.tiles_i, p.tiles_j, tile_i, tile_j);
+  const int bi0 = tile_i * BI, bj0 = tile_j * BJ;
+  const int kt_begin = blockIdx.y * p.k_tiles_per_split;
+  int kt_end = kt_begin + p.k_tiles_per_split;
+  if (kt_end > p.k_tiles) kt_end = p.k_tiles;
+  const int64_t batch = blockIdx.z;
+
+  const char* const rbase = p.row_base + batch * p.row_batch * ES;
+  const char* const cbase = p.col_base + batch * p.col_batch * ES;
+
+  // ---- per-thread load slots -------------------------------------------------
+  // LD_VEC: chunk fastest across lanes (8 lanes cover one 128-byte row segment).
+  // LD_STRIDED / LD_CONV: row fastest across lanes (rows are the contiguous
+  // direction in memory), one fixed row per thread.
+  int r_row[NR], r_chunk[NR];
+#pragma unroll
+  for (int u = 0; u < NR; ++u) {
+    int item = t + 256 * u;
+    if (RL == LD_VEC) {
+      r_chunk[u] = item & 7;
+      r_row[u] = item >> 3;
+    } else {
+      r_row[u] = item % BI;
+      r_chunk[u] = item / BI;
+    }
+  }
+  int c_row[NC], c_chunk[NC];
+#pragma unroll
+  for (int u = 0; u < NC; ++u) {
+    int item = t + 256 * u;
+    if (CL == LD_VEC) {
+      c_chunk[u] = item & 7;
+      c_row[u] = item >> 3;
+    } else {
+      c_row[u] = item % BJ;
+      c_chunk[u] = item / BJ;
+    }
+  }
+
+  // im2col state of this thread's (single) column-operand row
+  int64_t cv_base = 0;
+  int cv_d0 = 0, cv_h0 = 0, cv_w0 = 0;
+  unsigned long long cv_mask = 0;
+  bool cv_valid = false;
+  if (CL == LD_CONV) {
+    int j = bj0 + c_row[0];
+    cv_valid = j < p.J;
+    int jj = cv_valid ? j : 0;
+    int opq = p.g.OP * p.g.OQ;
+    int img = jj / (p.g.OD * opq);
+    int rem = jj - img * (p.g.OD * opq);
+    int od = rem / opq;
+    rem -= od * opq;
+    int op = rem / p.g.OQ;
+    int oq = rem - op * p.g.OQ;
+    cv_d0 = od * p.g.sd - p.g.pd;
+    cv_h0 = op * p.g.sh - p.g.ph;
+    cv_w0 = oq * p.g.sw - p.g.pw;
+    cv_base = (int64_t)img * p.g.C * p.g.D * p.g.H * p.g.W +
+              ((int64_t)cv_d0 * p.g.H + cv_h0) * p.g.W + cv_w0;
+    if (p.g.use_mask && cv_valid) {
+      int tap = 0;
+      for (int tt = 0; tt < p.g.T; ++tt)
+        for (int rr = 0; rr < p.g.R; ++rr)
+          for (int ss = 0; ss < p.g.S; ++ss, ++tap) {
+            bool ok = (unsigned)(cv_d0 + tt * p.g.dd) < (unsigned)p.g.D &&
+                      (unsigned)(cv_h0 + rr * p.g.dh) < (unsigned)p.g.H &&
+                      (unsigned)(cv_w0 + ss * p.g.dw) < (unsigned)p.g.W;
+            if (ok) cv_mask |= 1ull << tap;
+          }
+    }
+  }
+
+  auto build_table = [&](int kt) {
+    if (CL == LD_CONV && t < BKE) {
+      int k = kt * BKE + t;
+      int2 e;
+      if (k < p.Kred) {
+        int rs = p.g.R * p.g.S;
+        int trs = p.g.T * rs;
+        int c = k / trs;
+        int tap = k - c * trs;
+        int tt = tap / rs;
+        int rem = tap - tt * rs;
+        int rr = rem / p.g.S;
+        int ss = rem - rr * p.g.S;
+        e.x = ((c * p.g.D + tt * p.g.dd) * p.g.H + rr * p.g.dh) * p.g.W + ss * p.g.dw;
+        e.y = p.g.use_mask ? tap : ((tt * p.g.dd) << 20 | (rr * p.g.dh) << 10 | (ss * p.g.dw));
+      } else {
+        e.x = 0;
+        e.y = p.g.use_mask ? 255 : -1;
+      }
+      sT[(kt & 1) * BKE + t] = e;
+    }
+  };
+
+  v4i rreg[NR], creg[NC];
+
+  auto load_elem = [&](const char* ptr, bool ok) -> unsigned {
+    if (ES == 2) return ok ? (unsigned)*(const unsigned short*)ptr : 0u;
+    return ok ? (unsigned)*(const unsigned char*)ptr : 0u;
+  };
+  auto pack = [&](const unsigned* e) -> v4i {
+    v4i v;
+    if (ES == 2) {
+      v.x = e[0] | (e[1] << 16);
+      v.y = e[2] | (e[3] << 16);
+      v.z = e[4] | (e[5] << 16);
+      v.w = e[6] | (e[7] << 16);
+    } else {
+      v.x = e[0] | (e[1] << 8) | (e[2] << 16) | (e[3] << 24);
+      v.y = e[4] | (e[5] << 8) | (e[6] << 16) | (e[7] << 24);
+      v.z = e[8] | (e[9] << 8) | (e[10] << 16) | (e[11] << 24);
+      v.w = e[12] | (e[13] << 8) | (e[14] << 16) | (e[15] << 24);
+    }
+    return v;
+  };
+
+  auto gload = [&](int kt) {
+    const int k0 = kt * BKE;
+#pragma unroll
+    for (int u = 0; u < NR; ++u) {
+      int row = bi0 + r_row[u];
+      int k = k0 + r_chunk[u] * CE;
+      if (RL == LD_VEC) {
+        v4i v = {0, 0, 0, 0};
+        if (row < p.I && k < p.Kred)
+          v = *(const v4i*)(rbase + ((int64_t)row * p.row_s_row + k) * ES);
+        rreg[u] = v;
+      } else {
+        unsigned e[CE];
+        const char* base = rbase + ((int64_t)row * p.row_s_row + (int64_t)k * p.row_s_k) * ES;
+#pragma unroll
+        for (int x = 0; x < CE; ++x)
+          e[x] = load_elem(base + (int64_t)x * p.row_s_k * ES, row < p.I && k + x < p.Kred);
+        rreg[u] = pack(e);
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < NC; ++u) {
+      int row = bj0 + c_row[u];
+      int k = k0 + c_chunk[u] * CE;
+      if (CL == LD_VEC) {
+        v4i v = {0, 0, 0, 0};
+        if (row < p.J && k < p.Kred)
+          v = *(const v4i*)(cbase + ((int64_t)row * p.col_s_row + k) * ES);
+        creg[u] = v;
+      } else if (CL == LD_STRIDED) {
+        unsigned e[CE];
+        const char* base = cbase + ((int64_t)row * p.col_s_row + (int64_t)k * p.col_s_k) * ES;
+#pragma unroll
+        for (int x = 0; x < CE; ++x)
+          e[x] = load_elem(base + (int64_t)x * p.col_s_k * ES, row < p.J && k + x < p.Kred);
+        creg[u] = pack(e);
+      } else {
+        unsigned e[CE];
+        const int2* tbl = sT + (kt & 1) * BKE + c_chunk[u] * CE;
+        const char* base = cbase + cv_base * ES;
+#pragma unroll
+        for (int x = 0; x < CE; ++x) {
+          int2 ent = tbl[x];
+          bool ok;
+          if (p.g.use_mask) {
+            ok = cv_valid && ent.y < 64 && ((cv_mask >> ent.y) & 1ull);
+          } else {
+            ok = cv_valid && ent.y >= 0 &&
+                 (unsigned)(cv_d0 + (ent.y >> 20)) < (unsigned)p.g.D &&
+                 (unsigned)(cv_h0 + ((ent.y >> 10) & 1023)) < (unsigned)p.g.H &&
+                 (unsigned)(cv_w0 + (ent.y & 1023)) < (unsigned)p.g.W;
+          }
+          e[x] = load_elem(base + (int64_t)ent.x * ES, ok);
+        }
+        creg[u] = pack(e);
+      }
+    }
+  };
+
+  auto lstore = [&](int buf) {
+    char* r = sR + buf * (BI * 128);
+    char* c = sC + buf * (BJ * 128);
+#pragma unroll
+    for (int u = 0; u < NR; ++u) *(v4i*)(r + lds_chunk_offset(r_row[u], r_chunk[u])) = rreg[u];
+#pragma unroll
+    for (int u = 0; u < NC; ++u) *(v4i*)(c + lds_chunk_offset(c_row[u], c_chunk[u])) = creg[u];
+  };
+
+  acc_t acc[TI][TJ];
+#pragma unroll
+  for (int a = 0; a < TI; ++a)
+#pragma unroll
+    for (int b = 0; b < TJ; ++b)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[a][b][r] = 0;
+
+  const int frag_row = lane & 31;
+  const int frag_half = lane >> 5;
+
+  auto compute = [&](int buf) {
+    const char* r = sR + buf * (BI * 128);
+    const char* c = sC + buf * (BJ * 128);
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks) {
+      v4i af[TI], bf[TJ];
+#pragma unroll
+      for (int a = 0; a < TI; ++a)
+        af[a] = *(const v4i*)(r + lds_chunk_offset((wi * TI + a) * 32 + frag_row, ks * 2 + frag_half));
+#pragma unroll
+      for (int b = 0; b < TJ; ++b)
+        bf[b] = *(const v4i*)(c + lds_chunk_offset((wj * TJ + b) * 32 + frag_row, ks * 2 + frag_half));
+#pragma unroll
+      for (int a = 0; a < TI; ++a)
+#pragma unroll
+        for (int b = 0; b < TJ; ++b) acc[a][b] = MM::run(af[a], bf[b], acc[a][b]);
+    }
+  };
+
+  // ---- main loop ---------------------------------------------------------------
+  if (kt_begin < kt_end) {
+    if (CL == LD_CONV) {
+      build_table(kt_begin);
+      __syncthreads();
+    }
+    gload(kt_begin);
+    if (CL == LD_CONV && kt_begin + 1 < kt_end) build_table(kt_begin + 1);
+    lstore(0);
+    __syncthreads();
+    for (int kt = kt_begin; kt < kt_end; ++kt) {
+      const int buf = (kt - kt_begin) & 1;
+      const bool more = kt + 1 < kt_end;
+      if (more) gload(kt + 1);
+      if (CL == LD_CONV && kt + 2 < kt_end) build_table(kt + 2);
+      compute(buf);
+      if (more) lstore(buf ^ 1);
+      __syncthreads();
+    }
+  }
+
+  // ---- epilogue: accumulators straight to the final layout -----------------------
+  out_t* const out = (out_t*)p.out + batch * p.out_batch;
+#pragma unroll
+  for (int b = 0; b < TJ; ++b) {
+    const int j = bj0 + (wj * TJ + b) * 32 + frag_row;
+    if (j >= p.J) continue;
+    const int jo = j / p.out_jmod;
+    const int64_t coff = (int64_t)jo * p.out_sjo + (j - jo * p.out_jmod);
+#pragma unroll
+    for (int a = 0; a < TI; ++a) {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int i = bi0 + (wi * TI + a) * 32 + 8 * (r >> 2) + 4 * frag_half + (r & 3);
+        if (i < p.I) {
+          out_t* dst = out + (int64_t)i * p.out_si + coff;
+          if (p.atomic_out)
+            atomicAdd(dst, acc[a][b][r]);
+          else
+            *dst = acc[a][b][r];
+        }
+      }
+    }
+  }
+}
+
+template <int TI, int TJ>
+constexpr size_t igemm_lds_bytes() {
+  return (size_t)2 * (64 * TI + 64 * TJ) * 128 + 2 * 128 * sizeof(int2);
+}
+
+}  // namespace amos

@@ -1,0 +1,162 @@
+// Per-shape mapping decisions.  The reference spreads these over
+// python/tvm/auto_tensorize/tensorization_phases/schedulers/cuda_v2.py (tile
+// factors), python/tvm/auto_tensorize/search/checker.py:43-82 with
+// src/auto_tensorize/utils.cc:31-57 (resource check) and a measured search
+// (python/tvm/auto_tensorize/search/parameter.py:386-459).  Here the choice is
+// analytical: a wave-quantisation + roofline estimate over the compiled tile
+// shapes.
+#include "mapper.h"
+
+#include <algorithm>
+#include <cmath>
+#include <cstring>
+
+namespace amos {
+
+static int64_t conv_out(int64_t in, int pad, int dil, int64_t k, int stride) {
+  int64_t eff = (k - 1) * dil + 1;
+  if (in + 2 * (int64_t)pad < eff) return 0;
+  return (in + 2 * (int64_t)pad - eff) / stride + 1;
+}
+
+int problem_of(int op, const void* desc, Problem* out) {
+  if (!desc || !out) return set_error(AMOS_ERR_BAD_ARG, "null descriptor");
+  memset(out, 0, sizeof(*out));
+  auto esize = [](int dt) { return dt == AMOS_I8 ? 1 : 2; };
+  switch (op) {
+    case AMOS_OP_GEMM:
+    case AMOS_OP_BGEMM: {
+      const amos_gemm_desc_t* g;
+      int64_t batch = 1;
+      if (op == AMOS_OP_BGEMM) {
+        const amos_bgemm_desc_t* b = (const amos_bgemm_desc_t*)desc;
+        g = &b->g;
+        batch = b->batch;
+      } else {
+        g = (const amos_gemm_desc_t*)desc;
+      }
+      if (g->M <= 0 || g->N <= 0 || g->K <= 0 || batch <= 0)
+        return set_error(AMOS_ERR_BAD_ARG, "non-positive GEMM extent");
+      out->I = g->M; out->J = g->N; out->K = g->K; out->batch = batch;
+      out->in_dtype = g->in_dtype;
+      out->in_bytes = batch * (g->M * g->K + g->K * g->N) * esize(g->in_dtype);
+      out->out_bytes = batch * g->M * g->N * 4;
+      return 0;
+    }
+    case AMOS_OP_CONV2D:
+    case AMOS_OP_CONV3D: {
+      const amos_conv_desc_t* c = (const amos_conv_desc_t*)desc;
+      int64_t D = op == AMOS_OP_CONV2D ? 1 : c->D, T = op == AMOS_OP_CONV2D ? 1 : c->T;
+      if (c->N <= 0 || c->C <= 0 || D <= 0 || c->H <= 0 || c->W <= 0 || c->K <= 0 || T <= 0 ||
+          c->R <= 0 || c->S <= 0 || c->stride_h <= 0 || c->stride_w <= 0 || c->dil_h <= 0 ||
+          c->dil_w <= 0)
+        return set_error(AMOS_ERR_BAD_ARG, "non-positive conv extent");
+      int64_t OD = op == AMOS_OP_CONV2D ? 1 : conv_out(D, c->pad_d, c->dil_d, T, c->stride_d);
+      int64_t OP = conv_out(c->H, c->pad_h, c->dil_h, c->R, c->stride_h);
+      int64_t OQ = conv_out(c->W, c->pad_w, c->dil_w, c->S, c->stride_w);
+      if (OD <= 0 || OP <= 0 || OQ <= 0)
+        return set_error(AMOS_ERR_BAD_ARG, "kernel window larger than the padded input");
+      out->I = c->K;
+      out->J = c->N * OD * OP * OQ;
+      out->K = c->C * T * c->R * c->S;
+      out->batch = 1;
+      out->in_dtype = c->in_dtype;
+      out->in_bytes = (c->N * c->C * D * c->H * c->W + c->K * out->K) * esize(c->in_dtype);
+      out->out_bytes = out->I * out->J * 4;
+      return 0;
+    }
+  }
+  return set_error(AMOS_ERR_BAD_ARG, "unknown op %d", op);
+}
+
+static const int kTiles[][2] = {{256, 256}, {256, 128}, {128, 256}, {128, 128},
+                                {128, 64},  {64, 128},  {64, 64}};
+
+static int64_t lds_bytes_of(int ti, int tj) { return 2ll * (ti + tj) * 128 + 2 * 128 * 8; }
+// accumulator registers per lane: (ti/2 x tj/2 wave tile) / 64 lanes
+static int64_t acc_regs_of(int ti, int tj) { return (int64_t)(ti / 2) * (tj / 2) / 64; }
+
+// Estimated seconds of one launch for a tile shape and split.  Three terms, the
+// largest wins: MFMA issue time of the busiest CU (wave quantisation of the grid
+// over 256 CUs, with an inner-loop efficiency that grows with the wave tile since
+// LDS reads per MFMA fall), HBM time for the algorithmic bytes (plus the partial
+// sums of a split-K launch), and a fixed launch floor.
+static double estimate_seconds(const Problem& pb, int ti, int tj, int split) {
+  const double es = pb.in_dtype == AMOS_I8 ? 1.0 : 2.0;
+  const double rate = (pb.in_dtype == AMOS_I8 ? Gfx950::kOpsPerClkCuI8 : Gfx950::kFlopsPerClkCuF16) *
+                      Gfx950::kClockGhz * 1e9;
+  const int64_t tiles = ((pb.I + ti - 1) / ti) * ((pb.J + tj - 1) / tj) * pb.batch * split;
+  const int per_cu = (int)std::min<int64_t>(Gfx950::kLdsBytes / lds_bytes_of(ti, tj), 2);
+  const int64_t slots = (int64_t)Gfx950::kComputeUnits * per_cu;
+  const int64_t rounds = (tiles + slots - 1) / slots;
+  const double bke = 128.0 / es;
+  const double ksteps = std::ceil(std::ceil((double)pb.K / bke) / split);
+  // LDS bytes read per MFMA flop fall with the wave tile; 0.85 is the ceiling we plan with
+  const double wave_i = ti / 2.0, wave_j = tj / 2.0;
+  const double eff = 0.85 * (wave_i * wave_j) / (wave_i * wave_j + 24.0 * (wave_i + wave_j));
+  const double tile_flop = 2.0 * ti * tj * ksteps * bke;
+  const double t_tile = tile_flop / (rate * eff) * per_cu;  // co-resident blocks share the CU
+  const double t_mfma = rounds * t_tile + 1.5e-6 /* prologue + epilogue */;
+  double bytes = (double)pb.in_bytes + (double)pb.out_bytes * (split > 1 ? 2.0 * split + 1.0 : 1.0);
+  const double t_hbm = bytes / Gfx950::kHbmBytesPerSec;
+  return std::max(t_mfma, t_hbm) + 2e-6;
+}
+
+}  // namespace amos
+
+using namespace amos;
+
+extern "C" {
+
+int amos_check_config(int op, const void* desc, const amos_kernel_config_t* cfg,
+                      int64_t* lds_bytes, int64_t* acc_regs) {
+  Problem pb;
+  int rc = problem_of(op, desc, &pb);
+  if (rc) return rc;
+  if (!cfg) return set_error(AMOS_ERR_BAD_ARG, "null config");
+  bool known = false;
+  for (auto& t : kTiles) known |= (t[0] == cfg->tile_i && t[1] == cfg->tile_j);
+  if (!known)
+    return set_error(AMOS_ERR_INFEASIBLE, "no kernel instance with block tile %dx%d", cfg->tile_i,
+                     cfg->tile_j);
+  int64_t lds = lds_bytes_of(cfg->tile_i, cfg->tile_j);
+  int64_t regs = acc_regs_of(cfg->tile_i, cfg->tile_j);
+  if (lds_bytes) *lds_bytes = lds;
+  if (acc_regs) *acc_regs = regs;
+  if (lds > Gfx950::kLdsBytes)
+    return set_error(AMOS_ERR_INFEASIBLE, "LDS over budget: %lld (required) vs. %d (given)",
+                     (long long)lds, Gfx950::kLdsBytes);
+  // accumulators + two operand fragments sets + prefetch registers must fit the file
+  int64_t prefetch = (cfg->tile_i + cfg->tile_j) / 32 * 4;
+  if (regs + prefetch + 64 > Gfx950::kVgprsPerLane)
+    return set_error(AMOS_ERR_INFEASIBLE, "registers over budget: %lld (required) vs. %d (given)",
+                     (long long)(regs + prefetch + 64), Gfx950::kVgprsPerLane);
+  if (cfg->split_k < 0) return set_error(AMOS_ERR_BAD_ARG, "negative split_k");
+  return 0;
+}
+
+int amos_default_config(int op, const void* desc, amos_kernel_config_t* out) {
+  Problem pb;
+  int rc = problem_of(op, desc, &pb);
+  if (rc) return rc;
+  if (!out) return set_error(AMOS_ERR_BAD_ARG, "null config");
+  memset(out, 0, sizeof(*out));
+  const double es = pb.in_dtype == AMOS_I8 ? 1.0 : 2.0;
+  const int k_tiles = (int)std::ceil((double)pb.K / (128.0 / es));
+  double best = 1e30;
+  for (auto& t : kTiles) {
+    for (int split = 1; split <= 16; split *= 2) {
+      if (split > 1 && (split > k_tiles / 4 || pb.batch > 1)) break;
+      double s = estimate_seconds(pb, t[0], t[1], split);
+      if (s < best * 0.98) {
+        best = s;
+        out->tile_i = t[0];
+        out->tile_j = t[1];
+        out->split_k = split;
+      }
+    }
+  }
+  return 0;
+}
+
+}  // extern "C"

@@ -1,0 +1,34 @@
+// Host-side mapper shared by the runtime and the C ABI: problem extents of an
+// op descriptor, resource check and per-shape kernel configuration.
+#pragma once
+#include <stdint.h>
+
+#include "amos_mi355x.h"
+
+namespace amos {
+
+int set_error(int code, const char* fmt, ...);
+
+// gfx950 limits the mapper plans against (one workgroup of 4 waves per CU slot)
+struct Gfx950 {
+  static constexpr int kComputeUnits = 256;
+  static constexpr int kXcds = 8;
+  static constexpr int kLdsBytes = 160 * 1024;      // per CU and per workgroup
+  static constexpr int kVgprsPerLane = 512;         // unified VGPR+AGPR file, one wave per SIMD
+  static constexpr int kWaveSize = 64;
+  static constexpr double kClockGhz = 2.4;
+  static constexpr double kFlopsPerClkCuF16 = 4096.0;
+  static constexpr double kOpsPerClkCuI8 = 8192.0;
+  static constexpr double kHbmBytesPerSec = 8e12;
+};
+
+// the implicit GEMM an op descriptor denotes: Out(i,j) = sum_k Row(i,k) Col(j,k), `batch` times
+struct Problem {
+  int64_t I, J, K, batch;
+  int in_dtype;
+  int64_t in_bytes, out_bytes;  // algorithmic bytes: every input read once, output written once
+};
+
+int problem_of(int op, const void* desc, Problem* out);
+
+}  // namespace amos

@@ -1,0 +1,197 @@
+"""Tensor-level entry points over the C ABI.
+
+PyTorch-ROCm only supplies device memory and the current stream here; every
+computation goes through libamos_mi355x.so.  There is no CPU or eager fallback:
+tensors that are not on a HIP device are rejected.
+"""
+import ctypes
+
+import torch
+
+from . import _lib
+from ._lib import (AMOS_OP_BGEMM, AMOS_OP_CONV2D, AMOS_OP_CONV3D, AMOS_OP_GEMM, BGemmDesc, ConvDesc,
+                   GemmDesc, KernelConfig, check)
+
+_IN_CODE = {torch.float16: _lib.AMOS_F16, torch.bfloat16: _lib.AMOS_BF16, torch.int8: _lib.AMOS_I8}
+_OUT_OF = {torch.float16: torch.float32, torch.bfloat16: torch.float32, torch.int8: torch.int32}
+_OUT_CODE = {torch.float32: _lib.AMOS_F32, torch.int32: _lib.AMOS_I32}
+
+
+def _need_device(*tensors):
+    for t in tensors:
+        if not isinstance(t, torch.Tensor) or not t.is_cuda:
+            raise RuntimeError("amos_amd runs on the GPU only: got a tensor on %s"
+                               % (getattr(t, "device", type(t)),))
+        if not t.is_contiguous():
+            raise ValueError("operands must be contiguous")
+
+
+def _stream_ptr(stream):
+    if stream is None:
+        stream = torch.cuda.current_stream()
+    return ctypes.c_void_p(stream.cuda_stream)
+
+
+def make_config(config):
+    """None | KernelConfig | dict(tile_i=, tile_j=, split_k=) -> KernelConfig or None"""
+    if config is None or isinstance(config, KernelConfig):
+        return config
+    c = KernelConfig()
+    c.tile_i = int(config.get("tile_i", 0))
+    c.tile_j = int(config.get("tile_j", 0))
+    c.split_k = int(config.get("split_k", 0))
+    return c
+
+
+def _cfg_ref(cfg):
+    return ctypes.byref(cfg) if cfg is not None else None
+
+
+def gemm_desc(M, N, K, in_dtype, trans_a=False, trans_b=False, lda=None, ldb=None, ldc=None):
+    d = GemmDesc()
+    d.M, d.N, d.K = M, N, K
+    d.in_dtype = _IN_CODE[in_dtype]
+    d.out_dtype = _OUT_CODE[_OUT_OF[in_dtype]]
+    d.trans_a, d.trans_b = int(trans_a), int(trans_b)
+    d.lda = lda if lda is not None else (M if trans_a else K)
+    d.ldb = ldb if ldb is not None else (K if trans_b else N)
+    d.ldc = ldc if ldc is not None else N
+    return d
+
+
+def conv_desc(x_shape, w_shape, in_dtype, stride, pad, dil):
+    """x_shape NCDHW, w_shape KCTRS; stride / pad / dil are 3-tuples"""
+    d = ConvDesc()
+    d.N, d.C, d.D, d.H, d.W = x_shape
+    d.K, _, d.T, d.R, d.S = w_shape
+    d.stride_d, d.stride_h, d.stride_w = stride
+    d.pad_d, d.pad_h, d.pad_w = pad
+    d.dil_d, d.dil_h, d.dil_w = dil
+    d.in_dtype = _IN_CODE[in_dtype]
+    d.out_dtype = _OUT_CODE[_OUT_OF[in_dtype]]
+    return d
+
+
+def _tup(v, n, unit=None):
+    if isinstance(v, (tuple, list)):
+        assert len(v) == n
+        return tuple(int(t) for t in v)
+    return (int(v),) * n
+
+
+def conv_out_shape(x_shape, w_shape, stride, pad, dil):
+    out = []
+    for ext, k, s, p, d in zip(x_shape[2:], w_shape[2:], stride, pad, dil):
+        out.append((ext + 2 * p - ((k - 1) * d + 1)) // s + 1)
+    return (x_shape[0], w_shape[0]) + tuple(out)
+
+
+def gemm(a, b, trans_a=False, trans_b=False, out=None, config=None, stream=None):
+    """C[M,N] = A(m,k) B(k,n); a is [M,K] ([K,M] if trans_a), b is [K,N] ([N,K] if trans_b)."""
+    _need_device(a, b)
+    M, K = (a.shape[1], a.shape[0]) if trans_a else a.shape
+    N = b.shape[0] if trans_b else b.shape[1]
+    if (b.shape[1] if trans_b else b.shape[0]) != K or a.dtype != b.dtype:
+        raise ValueError("operand shapes / dtypes do not agree")
+    if out is None:
+        out = torch.empty((M, N), dtype=_OUT_OF[a.dtype], device=a.device)
+    _need_device(out)
+    d = gemm_desc(M, N, K, a.dtype, trans_a, trans_b)
+    cfg = make_config(config)
+    check(_lib.load().amos_gemm(ctypes.byref(d), _cfg_ref(cfg), a.data_ptr(), b.data_ptr(),
+                                out.data_ptr(), None, 0, _stream_ptr(stream)))
+    return out
+
+
+def bgemm_desc(batch, M, N, K, in_dtype, trans_a=False, trans_b=False):
+    d = BGemmDesc()
+    d.batch = batch
+    d.g = gemm_desc(M, N, K, in_dtype, trans_a, trans_b)
+    d.stride_a, d.stride_b, d.stride_c = M * K, K * N, M * N
+    return d
+
+
+def bgemm(a, b, trans_a=False, trans_b=False, out=None, config=None, stream=None):
+    """batched GEMM; a is [B,M,K] ([B,K,M] if trans_a), b is [B,K,N] ([B,N,K] if trans_b)."""
+    _need_device(a, b)
+    B = a.shape[0]
+    M, K = (a.shape[2], a.shape[1]) if trans_a else a.shape[1:]
+    N = b.shape[1] if trans_b else b.shape[2]
+    if b.shape[0] != B or (b.shape[2] if trans_b else b.shape[1]) != K or a.dtype != b.dtype:
+        raise ValueError("operand shapes / dtypes do not agree")
+    if out is None:
+        out = torch.empty((B, M, N), dtype=_OUT_OF[a.dtype], device=a.device)
+    _need_device(out)
+    d = bgemm_desc(B, M, N, K, a.dtype, trans_a, trans_b)
+    cfg = make_config(config)
+    check(_lib.load().amos_bgemm(ctypes.byref(d), _cfg_ref(cfg), a.data_ptr(), b.data_ptr(),
+                                 out.data_ptr(), None, 0, _stream_ptr(stream)))
+    return out
+
+
+def conv2d(x, w, stride=1, pad=0, dil=1, out=None, config=None, stream=None):
+    """x NCHW, w KCRS -> NKPQ"""
+    _need_device(x, w)
+    st, pd, dl = (1,) + _tup(stride, 2), (0,) + _tup(pad, 2), (1,) + _tup(dil, 2)
+    xs = (x.shape[0], x.shape[1], 1, x.shape[2], x.shape[3])
+    ws = (w.shape[0], w.shape[1], 1, w.shape[2], w.shape[3])
+    if x.shape[1] != w.shape[1] or x.dtype != w.dtype:
+        raise ValueError("operand shapes / dtypes do not agree")
+    oshape = conv_out_shape(xs, ws, st, pd, dl)
+    if out is None:
+        out = torch.empty((oshape[0], oshape[1], oshape[3], oshape[4]), dtype=_OUT_OF[x.dtype],
+                          device=x.device)
+    _need_device(out)
+    d = conv_desc(xs, ws, x.dtype, st, pd, dl)
+    cfg = make_config(config)
+    check(_lib.load().amos_conv2d(ctypes.byref(d), _cfg_ref(cfg), x.data_ptr(), w.data_ptr(),
+                                  out.data_ptr(), None, 0, _stream_ptr(stream)))
+    return out
+
+
+def conv3d(x, w, stride=1, pad=0, dil=1, out=None, config=None, stream=None):
+    """x NCDHW, w KCTRS -> NKDPQ"""
+    _need_device(x, w)
+    st, pd, dl = _tup(stride, 3), _tup(pad, 3), _tup(dil, 3)
+    if x.shape[1] != w.shape[1] or x.dtype != w.dtype:
+        raise ValueError("operand shapes / dtypes do not agree")
+    oshape = conv_out_shape(tuple(x.shape), tuple(w.shape), st, pd, dl)
+    if out is None:
+        out = torch.empty(oshape, dtype=_OUT_OF[x.dtype], device=x.device)
+    _need_device(out)
+    d = conv_desc(tuple(x.shape), tuple(w.shape), x.dtype, st, pd, dl)
+    cfg = make_config(config)
+    check(_lib.load().amos_conv3d(ctypes.byref(d), _cfg_ref(cfg), x.data_ptr(), w.data_ptr(),
+                                  out.data_ptr(), None, 0, _stream_ptr(stream)))
+    return out
+
+
+def time_op(op, desc, in0, in1, out, config=None, number=100, repeat=1, min_repeat_ms=150, stream=None):
+    """mean seconds per launch, `repeat` values (time_evaluator semantics)"""
+    _need_device(in0, in1, out)
+    cfg = make_config(config)
+    res = (ctypes.c_double * repeat)()
+    check(_lib.load().amos_time(op, ctypes.byref(desc), _cfg_ref(cfg), in0.data_ptr(), in1.data_ptr(),
+                                out.data_ptr(), None, 0, _stream_ptr(stream), number, repeat,
+                                min_repeat_ms, res))
+    return list(res)
+
+
+def default_config(op, desc):
+    cfg = KernelConfig()
+    check(_lib.load().amos_default_config(op, ctypes.byref(desc), ctypes.byref(cfg)))
+    return cfg
+
+
+def kernel_name(op, desc, config=None):
+    cfg = make_config(config)
+    name = _lib.load().amos_kernel_name(op, ctypes.byref(desc), _cfg_ref(cfg))
+    if name is None:
+        raise _lib.AmosError(-3, _lib.load().amos_last_error().decode())
+    return name.decode()
+
+
+def device_info():
+    info = _lib.DeviceInfo()
+    check(_lib.load().amos_device_info(ctypes.byref(info)))
+    return info

@@ -1,0 +1,281 @@
+"""HIP path vs the CPU oracle on the same seeded inputs, through the C ABI.
+
+Bars: int8 -> int32 bit-exact against exact integer arithmetic; fp16 / bf16 within
+max-rel-err 1e-2 and mean-rel-err 1e-3 of the fp32-accumulated CPU result (relative
+error with the denominator floored at 1e-2 * rms(ref), oracle.cpu_oracle.rel_errors).
+The te_literal loop nest rounds every product to the input dtype, as the reference's llvm
+build does, so it sits 2^-11 (fp16) or 2^-8 (bf16) per product away from any matrix-core
+result; it is compared with the reference's own tolerances: allclose(atol=rtol=1e-2) for
+fp16 (reference: README.md:334), atol=rtol=1e-1 for bf16 (reference:
+tests/python/auto_tensorize/manual_mapping_conv2d_fp16fp32_tensorcore.py:114), both scaled
+by max(1, rms) of the output, and mean-rel-err <= 1e-3 for fp16 on the config-sized cases.
+"""
+import numpy as np
+import pytest
+
+from conftest import make_operand, to_device
+from oracle import cpu_oracle as co
+
+pytestmark = pytest.mark.gpu
+
+MAX_REL, MEAN_REL = 1e-2, 1e-3
+
+
+def check_float(got, ref, what):
+    mx, mean = co.rel_errors(got, ref)
+    assert mx <= MAX_REL and mean <= MEAN_REL, "%s: max_rel=%.3e mean_rel=%.3e" % (what, mx, mean)
+
+
+def check_literal(got, lit, dtype, what, mean_bar=None):
+    if dtype == "int8":
+        assert np.array_equal(got, lit), what
+        return
+    tol = 1e-2 if dtype == "float16" else 1e-1
+    scale = max(1.0, float(np.sqrt(np.mean(lit.astype(np.float64) ** 2))))
+    assert np.allclose(got, lit, atol=tol * scale, rtol=tol), "%s: max abs diff %.3e (scale %.2f)" % (
+        what, float(np.abs(got - lit).max()), scale)
+    if mean_bar is not None:
+        assert co.rel_errors(got, lit)[1] <= mean_bar, what
+
+
+def check(got, ref, dtype, what):
+    if dtype == "int8":
+        assert got.dtype == np.int32
+        bad = int((got != ref).sum())
+        assert bad == 0, "%s: %d of %d int32 outputs differ" % (what, bad, got.size)
+    else:
+        check_float(got, ref, what)
+
+
+GEMM_SHAPES = [(64, 64, 64), (128, 256, 192), (200, 136, 72), (33, 17, 19), (1, 1, 1), (300, 70, 520)]
+
+
+@pytest.mark.parametrize("dtype", ["float16", "bfloat16", "int8"])
+@pytest.mark.parametrize("trans", [(0, 0), (0, 1), (1, 0), (1, 1)])
+@pytest.mark.parametrize("shape", GEMM_SHAPES)
+def test_gemm_small(gpu, dtype, trans, shape):
+    from amos_amd import ops
+    M, N, K = shape
+    ta, tb = trans
+    rng = np.random.default_rng(hash((M, N, K, ta, tb)) % 2**32)
+    a = make_operand(rng, (K, M) if ta else (M, K), dtype)
+    b = make_operand(rng, (N, K) if tb else (K, N), dtype)
+    got = ops.gemm(to_device(a, dtype), to_device(b, dtype), ta, tb).cpu().numpy()
+    ref = co.lib_gemm(a, b, dtype, ta, tb, acc="float64")
+    check(got, ref, dtype, "gemm %s %s %s vs exact" % (dtype, trans, shape))
+    lit = co.te_literal_gemm(a, b, dtype, ta, tb, mode="exact" if dtype == "int8" else "te_literal")
+    check_literal(got, lit, dtype, "gemm %s %s %s vs te_literal" % (dtype, trans, shape))
+
+
+TILES = [(64, 64), (128, 128), (256, 256), (128, 64), (64, 128), (256, 128), (128, 256)]
+
+
+@pytest.mark.parametrize("dtype", ["float16", "int8"])
+@pytest.mark.parametrize("tile", TILES)
+@pytest.mark.parametrize("split", [1, 3])
+def test_gemm_every_tile(gpu, dtype, tile, split):
+    from amos_amd import ops
+    M, N, K = 520, 392, 1096
+    rng = np.random.default_rng(7)
+    a = make_operand(rng, (M, K), dtype)
+    b = make_operand(rng, (N, K), dtype)
+    cfg = dict(tile_i=tile[0], tile_j=tile[1], split_k=split)
+    got = ops.gemm(to_device(a, dtype), to_device(b, dtype), False, True, config=cfg).cpu().numpy()
+    ref = co.lib_gemm(a, b, dtype, False, True, acc="float64")
+    check(got, ref, dtype, "gemm tile %s split %d" % (tile, split))
+
+
+def test_gemm_config1_512(gpu):
+    """fp16 GEMM 512^3, inputs U[-1,1], against the full te_literal loop nest"""
+    from amos_amd import ops
+    rng = np.random.default_rng(0)
+    a = make_operand(rng, (512, 512), "float16")
+    b = make_operand(rng, (512, 512), "float16")
+    got = ops.gemm(to_device(a, "float16"), to_device(b, "float16")).cpu().numpy()
+    check_float(got, co.lib_gemm(a, b, "float16", acc="float32"), "C1 vs fp32 matmul")
+    check_literal(got, co.te_literal_gemm(a, b, "float16", threads=8), "float16", "C1 vs te_literal", MEAN_REL)
+
+
+def test_gemm_config2_8192(gpu):
+    """fp16 GEMM 8192^3, row-major A, column-major B: slabs of rows against the oracle,
+    plus linearity C(A, B) + C(A2, B) == C(A + A2, B) on exactly representable operands."""
+    import torch
+    from amos_amd import ops
+    n = 8192
+    rng = np.random.default_rng(0)
+    a = make_operand(rng, (n, n), "float16")
+    b = make_operand(rng, (n, n), "float16")
+    da, db = to_device(a, "float16"), to_device(b, "float16")
+    got = ops.gemm(da, db, False, True)
+    g = got.cpu().numpy()
+    rows = np.r_[0:4, 4093:4099, 8188:8192]
+    ref = co.lib_gemm(a[rows], b, "float16", False, True, acc="float64")
+    check_float(g[rows], ref, "C2 rows vs fp64")
+    lit = co.te_literal_gemm(np.ascontiguousarray(a[rows[:4]]), b, "float16", False, True, threads=8)
+    check_literal(g[rows[:4]], lit, "float16", "C2 rows vs te_literal", MEAN_REL)
+    # column sums: sum_m C[m, n] == (sum_m A[m, :]) . B[n, :]  -- touches every output once
+    colsum = got.double().sum(dim=0).cpu().numpy()
+    want = (a.astype(np.float64).sum(axis=0))[None, :] @ b.astype(np.float64).T
+    mx, mean = co.rel_errors(colsum, want[0])
+    assert mx < 1e-2 and mean < 1e-3, (mx, mean)
+    # small integers: every product and partial sum is exact in fp16 x fp16 -> fp32
+    ai = rng.integers(-2, 3, size=(n, n)).astype(np.float16)
+    bi = rng.integers(-2, 3, size=(n, n)).astype(np.float16)
+    gi = ops.gemm(to_device(ai, "float16"), to_device(bi, "float16"), False, True)
+    wi = torch.from_numpy(ai).cuda().float() @ torch.from_numpy(bi).cuda().float().T
+    assert torch.equal(gi, wi)
+
+
+def test_bgemm_small(gpu):
+    from amos_amd import ops
+    rng = np.random.default_rng(3)
+    for dtype in ["float16", "bfloat16", "int8"]:
+        for (B, M, N, K, ta, tb) in [(3, 70, 50, 40, 0, 1), (2, 64, 64, 64, 0, 0), (5, 17, 9, 33, 1, 1)]:
+            a = make_operand(rng, (B, K, M) if ta else (B, M, K), dtype, "normal")
+            b = make_operand(rng, (B, N, K) if tb else (B, K, N), dtype, "normal")
+            got = ops.bgemm(to_device(a, dtype), to_device(b, dtype), ta, tb).cpu().numpy()
+            check(got, co.lib_gemm(a, b, dtype, ta, tb, acc="float64"), dtype, "bgemm %s" % dtype)
+            lit = co.te_literal_bgemm(a, b, dtype, ta, tb, mode="exact" if dtype == "int8" else "te_literal")
+            check_literal(got, lit, dtype, "bgemm te_literal %s" % dtype)
+
+
+def test_bgemm_config5a(gpu):
+    """fp16 batched GEMM 192 x (512x512x64), scores = Q K^T, N(0,1) inputs: full check"""
+    from amos_amd import ops
+    rng = np.random.default_rng(0)
+    q = make_operand(rng, (192, 512, 64), "float16", "normal")
+    k = make_operand(rng, (192, 512, 64), "float16", "normal")
+    got = ops.bgemm(to_device(q, "float16"), to_device(k, "float16"), False, True).cpu().numpy()
+    check_float(got, co.lib_gemm(q, k, "float16", False, True, acc="float32"), "C5a vs fp32")
+    lit = co.te_literal_bgemm(q, k, "float16", False, True, batches=(0, 4), threads=8)
+    check_literal(got[:4], lit[:4], "float16", "C5a vs te_literal (4 batches)", MEAN_REL)
+
+
+CONV2D_CASES = [
+    # N, C, H, W, K, R, S, stride, pad, dil
+    (1, 16, 8, 8, 16, 3, 3, 1, 1, 1),
+    (2, 24, 14, 14, 40, 3, 3, 1, 1, 1),
+    (3, 7, 9, 11, 5, 3, 2, 2, 1, 1),
+    (2, 16, 15, 15, 32, 3, 3, 1, 2, 2),
+    (1, 3, 32, 32, 8, 7, 7, 2, 3, 1),
+    (2, 64, 7, 7, 64, 1, 1, 1, 0, 1),
+    (2, 32, 10, 10, 16, 1, 1, 2, 0, 1),
+    (1, 8, 5, 5, 4, 5, 5, 1, 0, 1),
+    (1, 4, 12, 12, 4, 9, 9, 1, 4, 1),   # 81 taps: compare path instead of the tap bitmask
+]
+
+
+@pytest.mark.parametrize("dtype", ["float16", "bfloat16", "int8"])
+@pytest.mark.parametrize("case", CONV2D_CASES)
+def test_conv2d_small(gpu, dtype, case):
+    from amos_amd import ops
+    N, C, H, W, K, R, S, st, pd, dl = case
+    rng = np.random.default_rng(hash(case) % 2**32)
+    x = make_operand(rng, (N, C, H, W), dtype)
+    w = make_operand(rng, (K, C, R, S), dtype)
+    got = ops.conv2d(to_device(x, dtype), to_device(w, dtype), st, pd, dl).cpu().numpy()
+    ref = co.lib_conv2d(x, w, dtype, st, pd, dl, acc="float64")
+    check(got, ref, dtype, "conv2d %s %s" % (dtype, case))
+    lit = co.te_literal_conv2d(x, w, dtype, st, pd, dl, mode="exact" if dtype == "int8" else "te_literal")
+    check_literal(got, lit, dtype, "conv2d te_literal %s %s" % (dtype, case))
+
+
+@pytest.mark.parametrize("tile", TILES)
+def test_conv2d_every_tile(gpu, tile):
+    from amos_amd import ops
+    rng = np.random.default_rng(11)
+    x = make_operand(rng, (3, 40, 13, 13), "int8")
+    w = make_operand(rng, (72, 40, 3, 3), "int8")
+    for split in (1, 2):
+        cfg = dict(tile_i=tile[0], tile_j=tile[1], split_k=split)
+        got = ops.conv2d(to_device(x, "int8"), to_device(w, "int8"), 1, 1, 1, config=cfg).cpu().numpy()
+        check(got, co.lib_conv2d(x, w, "int8", 1, 1, 1), "int8", "conv2d tile %s split %d" % (tile, split))
+
+
+def test_conv2d_config3(gpu):
+    """fp16 conv2d N32 C256 14x14 K256 3x3 s1 p1; X ~ U[0,1], W ~ N(0, 0.05)"""
+    from amos_amd import ops
+    rng = np.random.default_rng(0)
+    x = rng.uniform(0, 1, size=(32, 256, 14, 14)).astype(np.float32).astype(np.float16)
+    w = (rng.standard_normal(size=(256, 256, 3, 3)) * 0.05).astype(np.float32).astype(np.float16)
+    got = ops.conv2d(to_device(x, "float16"), to_device(w, "float16"), 1, 1, 1).cpu().numpy()
+    check_float(got, co.lib_conv2d(x, w, "float16", 1, 1, 1, acc="float32"), "C3 vs fp32")
+    lit = co.te_literal_conv2d(x, w, "float16", 1, 1, 1, images=(0, 2), threads=8)
+    check_literal(got[:2], lit[:2], "float16", "C3 vs te_literal (2 images)", MEAN_REL)
+
+
+def test_conv2d_config4_int8(gpu):
+    """int8 conv2d N64 C128 28x28 K128 3x3 s1 p1: bit-exact on the whole tensor"""
+    from amos_amd import ops
+    rng = np.random.default_rng(0)
+    x = rng.integers(-128, 128, size=(64, 128, 28, 28)).astype(np.int8)
+    w = rng.integers(-64, 64, size=(128, 128, 3, 3)).astype(np.int8)
+    got = ops.conv2d(to_device(x, "int8"), to_device(w, "int8"), 1, 1, 1).cpu().numpy()
+    ref = co.lib_conv2d(x, w, "int8", 1, 1, 1)
+    assert got.dtype == np.int32 and np.array_equal(got, ref)
+    lit = co.te_literal_conv2d(x, w, "int8", 1, 1, 1, mode="exact", images=(0, 1), threads=8)
+    assert np.array_equal(got[:1], lit[:1])
+
+
+CONV3D_CASES = [
+    # N, C, D, H, W, K, T, R, S, stride, pad, dil
+    (1, 8, 4, 6, 6, 8, 3, 3, 3, 1, 1, 1),
+    (2, 5, 5, 7, 9, 12, 3, 2, 3, (1, 2, 1), (1, 0, 2), (1, 1, 2)),
+    (1, 16, 6, 6, 6, 16, 1, 1, 1, 1, 0, 1),
+    (1, 4, 8, 8, 8, 8, 2, 2, 2, 2, 0, 1),
+]
+
+
+@pytest.mark.parametrize("dtype", ["float16", "int8"])
+@pytest.mark.parametrize("case", CONV3D_CASES)
+def test_conv3d_small(gpu, dtype, case):
+    from amos_amd import ops
+    N, C, D, H, W, K, T, R, S, st, pd, dl = case
+    rng = np.random.default_rng(5)
+    x = make_operand(rng, (N, C, D, H, W), dtype, "normal")
+    w = make_operand(rng, (K, C, T, R, S), dtype, "normal")
+    got = ops.conv3d(to_device(x, dtype), to_device(w, dtype), st, pd, dl).cpu().numpy()
+    check(got, co.lib_conv3d(x, w, dtype, st, pd, dl, acc="float64"), dtype, "conv3d %s" % (case,))
+    lit = co.te_literal_conv3d(x, w, dtype, st, pd, dl, mode="exact" if dtype == "int8" else "te_literal")
+    check_literal(got, lit, dtype, "conv3d te_literal %s" % (case,))
+
+
+def test_conv3d_config5b(gpu):
+    """fp16 conv3d N8 C64 D16 56x56 K64 3x3x3 s1 p1, N(0,1): one image against the library
+    form, plus the batch-shift property (image n of the batched call == the same image alone)."""
+    import torch
+    from amos_amd import ops
+    rng = np.random.default_rng(0)
+    x = make_operand(rng, (8, 64, 16, 56, 56), "float16", "normal")
+    w = make_operand(rng, (64, 64, 3, 3, 3), "float16", "normal")
+    dx, dw = to_device(x, "float16"), to_device(w, "float16")
+    got = ops.conv3d(dx, dw, 1, 1, 1)
+    ref0 = co.lib_conv3d(x[5:6], w, "float16", 1, 1, 1, acc="float32")
+    check_float(got[5:6].cpu().numpy(), ref0, "C5b image 5 vs fp32")
+    # same tiling and no split-K => the same accumulation order => bitwise equal
+    cfg = dict(tile_i=64, tile_j=128, split_k=1)
+    full = ops.conv3d(dx, dw, 1, 1, 1, config=cfg)
+    alone = ops.conv3d(dx[2:3].contiguous(), dw, 1, 1, 1, config=cfg)
+    assert torch.equal(alone[0], full[2])
+    check_float(full[5:6].cpu().numpy(), ref0, "C5b image 5 vs fp32 (64x128)")
+
+
+def test_errors(gpu):
+    import torch
+    from amos_amd import _lib, ops
+    a = torch.zeros((8, 8), dtype=torch.float16, device="cuda")
+    with pytest.raises(_lib.AmosError) as e:
+        ops.gemm(a, a, config=dict(tile_i=96, tile_j=64, split_k=1))
+    assert e.value.code == _lib.AMOS_ERR_INFEASIBLE
+    with pytest.raises(RuntimeError):
+        ops.gemm(a.cpu(), a.cpu())
+
+
+def test_time_evaluator(gpu):
+    import torch
+    from amos_amd import _lib, ops
+    a = torch.randn((512, 512), device="cuda").half()
+    out = torch.empty((512, 512), device="cuda")
+    d = ops.gemm_desc(512, 512, 512, torch.float16)
+    res = ops.time_op(_lib.AMOS_OP_GEMM, d, a, a, out, number=10, repeat=3, min_repeat_ms=5)
+    assert len(res) == 3 and all(0 < r < 1e-2 for r in res)
