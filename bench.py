@@ -1,0 +1,205 @@
+"""Headline benchmark: fp16 GEMM M=N=K=8192, fp32 accumulate, row-major A, column-major B,
+on one MI355X, next to the CPU restatement of the reference's llvm path timed in the same run.
+
+  python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--report FILE]
+
+A step is one launch of the GEMM over device-resident operands.  Prints ONE JSON line.
+`--report FILE` additionally times every configuration of the path (GEMM, batched GEMM,
+conv2d fp16 / int8, conv3d) and writes a per-config table as JSON to FILE.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+METRIC = "TFLOP/s + % of MFMA peak per op (fp16 conv2d/GEMM, int8 TOP/s), 1 MI355X"
+PEAK_F16_TFLOPS = 2500.0   # published dense fp16 MFMA peak of MI355X
+PEAK_I8_TOPS = 5000.0      # published dense int8 peak
+PEAK_HBM_GBS = 8000.0      # published HBM3E bandwidth
+
+
+def cpu_baseline_gemm(a, b, seconds_budget=12.0):
+    """te_literal loop nest (single thread, as TVM's default schedule) on a slab of rows of the
+    same 8192^3 workload, scaled linearly; plus an all-core OpenMP run of a larger slab."""
+    from oracle import cpu_oracle as co
+    n = a.shape[0]
+    flop_row = 2.0 * n * n
+    t0 = time.perf_counter()
+    co.te_literal_gemm(a, b, "float16", False, True, rows=(0, 1), threads=1)
+    t_row = time.perf_counter() - t0
+    rows1 = int(max(2, min(64, seconds_budget / max(t_row, 1e-6))))
+    t0 = time.perf_counter()
+    co.te_literal_gemm(a, b, "float16", False, True, rows=(0, rows1), threads=1)
+    t1 = time.perf_counter() - t0
+    cores = min(co.load().oracle_max_threads(), int(os.environ.get("OMP_NUM_THREADS", "16")), 16)
+    rowsn = rows1 * cores
+    t0 = time.perf_counter()
+    co.te_literal_gemm(a, b, "float16", False, True, rows=(0, rowsn), threads=cores)
+    tn = time.perf_counter() - t0
+    return {
+        "value": rows1 * flop_row / t1 / 1e12, "unit": "TFLOP/s", "cores": 1, "kind": "port",
+        "sample": "rows [0,%d) of the 8192^3 GEMM, te_literal loop nest (fp16 product rounded to "
+                  "fp16, fp32 sequential accumulate), gcc -O3, %.1f s; extrapolated_from=%.5f"
+                  % (rows1, t1, rows1 / n),
+        "all_cores": {"value": rowsn * flop_row / tn / 1e12, "unit": "TFLOP/s", "cores": cores,
+                      "sample": "rows [0,%d), OpenMP over rows, %.1f s" % (rowsn, tn)},
+    }
+
+
+def _timed(fn):
+    t0 = time.perf_counter()
+    fn()
+    return time.perf_counter() - t0
+
+
+def run_all_configs(cpu=True):
+    """Every configuration of the path: GPU ms, TFLOP/s (TOP/s), % of the MFMA peak, % of the
+    HBM roof for the algorithmic bytes, which roof binds, and the te_literal CPU loop nest
+    (1 thread and all cores) on a slab of the same workload, linearly scaled."""
+    import numpy as np
+    import torch
+    from amos_amd import _lib, ops
+    from oracle import cpu_oracle as co
+    cores = min(co.load().oracle_max_threads(), int(os.environ.get("OMP_NUM_THREADS", "16")), 16)
+    rng = np.random.default_rng(0)
+    f16 = lambda x: x.astype(np.float32).astype(np.float16)
+    rows = []
+
+    def gpu_time(op, desc, i0, i1, out):
+        cfg = ops.default_config(op, desc)
+        t = ops.time_op(op, desc, i0, i1, out, config=cfg, number=20, repeat=3, min_repeat_ms=100)
+        return min(t), cfg
+
+    def add(name, op, desc, hin, dtype, flop, nbytes, out_shape, cpu_fn, frac):
+        tin = [torch.from_numpy(h).cuda() for h in hin]
+        out = torch.empty(out_shape, dtype=torch.int32 if dtype == "int8" else torch.float32,
+                          device="cuda")
+        sec, cfg = gpu_time(op, desc, tin[0], tin[1], out)
+        peak = PEAK_I8_TOPS if dtype == "int8" else PEAK_F16_TFLOPS
+        t_mfma, t_hbm = flop / (peak * 1e12), nbytes / (PEAK_HBM_GBS * 1e9)
+        row = {"config": name, "kernel": ops.kernel_name(op, desc, cfg), "split_k": cfg.split_k,
+               "gpu_us": sec * 1e6, "tflops": flop / sec / 1e12,
+               "pct_mfma_peak": 100 * t_mfma / sec, "pct_hbm_roof": 100 * t_hbm / sec,
+               "bound": "mfma" if t_mfma >= t_hbm else "hbm", "flop": flop, "bytes": nbytes}
+        if cpu:
+            t1 = _timed(lambda: cpu_fn(1, False))
+            tn = _timed(lambda: cpu_fn(cores, True))
+            row["cpu"] = {"kind": "port (te_literal loop nest, gcc -O3)",
+                          "threads1_tflops": flop * frac[0] / t1 / 1e12,
+                          "threadsN_tflops": flop * frac[1] / tn / 1e12, "cores": cores,
+                          "extrapolated_from": list(frac)}
+        rows.append(row)
+        del tin, out
+        torch.cuda.empty_cache()
+
+    # C2 fp16 GEMM 8192^3
+    n = 8192
+    a, b = f16(rng.uniform(-1, 1, (n, n))), f16(rng.uniform(-1, 1, (n, n)))
+    add("C2 fp16 GEMM 8192^3 (ntn)", _lib.AMOS_OP_GEMM, ops.gemm_desc(n, n, n, torch.float16, False, True),
+        [a, b], "float16", 2.0 * n ** 3, 2 * n * n * 2 + n * n * 4, (n, n),
+        lambda th, big: co.te_literal_gemm(a, b, "float16", False, True, rows=(0, 8 * th), threads=th),
+        (8 / n, 8 * cores / n))
+    # C3 fp16 conv2d
+    x = f16(rng.uniform(0, 1, (32, 256, 14, 14)))
+    w = f16(rng.standard_normal((256, 256, 3, 3)) * 0.05)
+    add("C3 fp16 conv2d N32 C256 14x14 K256 3x3", _lib.AMOS_OP_CONV2D,
+        ops.conv_desc((32, 256, 1, 14, 14), (256, 256, 1, 3, 3), torch.float16, (1, 1, 1), (0, 1, 1), (1, 1, 1)),
+        [x, w], "float16", 2.0 * 6272 * 256 * 2304, 10813440, (32, 256, 14, 14),
+        lambda th, big: co.te_literal_conv2d(x, w, "float16", 1, 1, 1, images=(0, 2 * th), threads=th),
+        (2 / 32, min(32, 2 * cores) / 32))
+    # C4 int8 conv2d
+    xi = rng.integers(-128, 128, (64, 128, 28, 28)).astype(np.int8)
+    wi = rng.integers(-64, 64, (128, 128, 3, 3)).astype(np.int8)
+    add("C4 int8 conv2d N64 C128 28x28 K128 3x3", _lib.AMOS_OP_CONV2D,
+        ops.conv_desc((64, 128, 1, 28, 28), (128, 128, 1, 3, 3), torch.int8, (1, 1, 1), (0, 1, 1), (1, 1, 1)),
+        [xi, wi], "int8", 2.0 * 50176 * 128 * 1152, 32260096, (64, 128, 28, 28),
+        lambda th, big: co.te_literal_conv2d(xi, wi, "int8", 1, 1, 1, mode="exact", images=(0, th), threads=th),
+        (1 / 64, cores / 64))
+    # C5a fp16 batched GEMM
+    q, k = f16(rng.standard_normal((192, 512, 64))), f16(rng.standard_normal((192, 512, 64)))
+    add("C5a fp16 bGEMM 192x(512x512x64) (ntn)", _lib.AMOS_OP_BGEMM,
+        ops.bgemm_desc(192, 512, 512, 64, torch.float16, False, True), [q, k], "float16",
+        2.0 * 192 * 512 * 512 * 64, 226492416, (192, 512, 512),
+        lambda th, big: co.te_literal_bgemm(q, k, "float16", False, True, batches=(0, 4 * th), threads=th),
+        (4 / 192, 4 * cores / 192))
+    # C5b fp16 conv3d
+    x3, w3 = f16(rng.standard_normal((8, 64, 16, 56, 56))), f16(rng.standard_normal((64, 64, 3, 3, 3)))
+    x3s = np.ascontiguousarray(x3[:1, :, :4])   # CPU slab: one image, 4 of 16 depth slices
+    add("C5b fp16 conv3d N8 C64 D16 56x56 K64 3x3x3", _lib.AMOS_OP_CONV3D,
+        ops.conv_desc((8, 64, 16, 56, 56), (64, 64, 3, 3, 3), torch.float16, (1, 1, 1), (1, 1, 1), (1, 1, 1)),
+        [x3, w3], "float16", 2.0 * 401408 * 64 * 1728, 154361856, (8, 64, 16, 56, 56),
+        lambda th, big: co.te_literal_conv3d(x3s, w3, "float16", 1, 1, 1, threads=th),
+        (1 / 32, 1 / 32))
+    return rows
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=100)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU-baseline leg")
+    ap.add_argument("--report", default=None, help="also time every config, write JSON here")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py measures the one-GPU kernel path; --gpus %d is not supported "
+                 "(this build has no multi-GPU path)" % args.gpus)
+
+    import numpy as np
+    import torch
+    from amos_amd import _lib, ops
+    if not torch.cuda.is_available():
+        sys.exit("bench.py needs a GPU")
+    n = 8192
+    rng = np.random.default_rng(0)
+    a = rng.uniform(-1, 1, (n, n)).astype(np.float32).astype(np.float16)
+    b = rng.uniform(-1, 1, (n, n)).astype(np.float32).astype(np.float16)   # stored [N, K]
+    da, db = torch.from_numpy(a).cuda(), torch.from_numpy(b).cuda()
+    dc = torch.empty((n, n), dtype=torch.float32, device="cuda")
+    desc = ops.gemm_desc(n, n, n, torch.float16, False, True)
+    cfg = ops.default_config(_lib.AMOS_OP_GEMM, desc)
+    flop = 2.0 * n ** 3
+
+    for _ in range(args.warmup):
+        ops.gemm(da, db, False, True, out=dc, config=cfg)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        ops.gemm(da, db, False, True, out=dc, config=cfg)
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    ms_per_step = elapsed / args.steps * 1e3
+    value = flop / (elapsed / args.steps) / 1e12
+
+    # dominant (only) kernel: mean launch duration from HIP events on the launch stream
+    per_launch = ops.time_op(_lib.AMOS_OP_GEMM, desc, da, db, dc, config=cfg, number=args.steps,
+                             repeat=1, min_repeat_ms=0)[0]
+    achieved = flop / per_launch / 1e12
+    line = {
+        "metric": METRIC, "value": value, "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": ms_per_step, "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "f16", "data": "synthetic",
+        "config": {"workload": "fp16 GEMM M=N=K=8192, fp32 accumulate, row-major A, column-major B "
+                               "(BASELINE configs[1])",
+                   "kernel": ops.kernel_name(_lib.AMOS_OP_GEMM, desc, cfg),
+                   "tile": "%dx%d" % (cfg.tile_i, cfg.tile_j), "split_k": cfg.split_k,
+                   "pct_of_mfma_peak": 100.0 * value / PEAK_F16_TFLOPS},
+        "roofline": {"bound": "mfma", "achieved": achieved, "peak": PEAK_F16_TFLOPS,
+                     "unit": "TFLOP/s", "frac": achieved / PEAK_F16_TFLOPS, "traffic": None,
+                     "kernel_us": per_launch * 1e6},
+    }
+    if not args.no_cpu:
+        line["cpu_baseline"] = cpu_baseline_gemm(a, b)
+    if args.report:
+        with open(args.report, "w") as f:
+            json.dump(run_all_configs(cpu=not args.no_cpu), f, indent=1)
+    print(json.dumps(line), flush=True)
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,103 @@
+"""The C-ABI library loads and exports what include/amos_mi355x.h declares; host-side
+validation, resource check and mapper defaults (no kernel is launched here)."""
+import ctypes
+import os
+import re
+
+import pytest
+
+from amos_amd import _lib
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def header_functions():
+    text = open(os.path.join(ROOT, "include", "amos_mi355x.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(amos_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_every_declared_symbol_is_exported():
+    lib = _lib.load()
+    names = header_functions()
+    assert len(names) >= 12
+    for n in names:
+        assert hasattr(lib, n), "libamos_mi355x.so does not export %s" % n
+    assert sorted(_lib.EXPORTS) == names
+    assert lib.amos_version() == 1
+
+
+def test_struct_sizes_match_header():
+    assert ctypes.sizeof(_lib.GemmDesc) == 3 * 8 + 4 * 4 + 3 * 8
+    assert ctypes.sizeof(_lib.BGemmDesc) == 8 + ctypes.sizeof(_lib.GemmDesc) + 3 * 8
+    assert ctypes.sizeof(_lib.ConvDesc) == 9 * 8 + 11 * 4 + 4
+    assert ctypes.sizeof(_lib.KernelConfig) == 32
+
+
+def gemm_desc(M, N, K, ind=_lib.AMOS_F16, outd=_lib.AMOS_F32, ta=0, tb=0):
+    d = _lib.GemmDesc()
+    d.M, d.N, d.K, d.in_dtype, d.out_dtype, d.trans_a, d.trans_b = M, N, K, ind, outd, ta, tb
+    d.lda, d.ldb, d.ldc = (M if ta else K), (K if tb else N), N
+    return d
+
+
+def test_bad_arguments_are_reported():
+    lib = _lib.load()
+    d = gemm_desc(16, 16, 16)
+    buf = ctypes.create_string_buffer(64)
+    rc = lib.amos_gemm(ctypes.byref(d), None, None, buf, buf, None, 0, None)
+    assert rc == _lib.AMOS_ERR_BAD_ARG and b"null" in lib.amos_last_error()
+    d2 = gemm_desc(0, 16, 16)
+    assert lib.amos_gemm(ctypes.byref(d2), None, buf, buf, buf, None, 0, None) == _lib.AMOS_ERR_BAD_ARG
+    d3 = gemm_desc(16, 16, 16, _lib.AMOS_F16, _lib.AMOS_I32)
+    assert lib.amos_gemm(ctypes.byref(d3), None, buf, buf, buf, None, 0, None) == _lib.AMOS_ERR_UNSUPPORTED
+    d4 = gemm_desc(16, 16, 16)
+    d4.lda = 8
+    assert lib.amos_gemm(ctypes.byref(d4), None, buf, buf, buf, None, 0, None) == _lib.AMOS_ERR_BAD_ARG
+    with pytest.raises(_lib.AmosError):
+        _lib.check(rc)
+
+
+def test_check_config_budget():
+    lib = _lib.load()
+    d = gemm_desc(1024, 1024, 1024)
+    lds, regs = ctypes.c_int64(), ctypes.c_int64()
+    cfg = _lib.KernelConfig(256, 256, 1)
+    assert lib.amos_check_config(0, ctypes.byref(d), ctypes.byref(cfg), ctypes.byref(lds), ctypes.byref(regs)) == 0
+    assert lds.value == 2 * (256 + 256) * 128 + 2048 and lds.value <= 160 * 1024 and regs.value == 256
+    bad = _lib.KernelConfig(96, 64, 1)
+    assert lib.amos_check_config(0, ctypes.byref(d), ctypes.byref(bad), None, None) == _lib.AMOS_ERR_INFEASIBLE
+
+
+def test_default_config_is_a_compiled_instance():
+    lib = _lib.load()
+    cfg = _lib.KernelConfig()
+    for (M, N, K) in [(8192, 8192, 8192), (512, 512, 512), (64, 64, 4096), (33, 17, 19), (100000, 64, 64)]:
+        d = gemm_desc(M, N, K, tb=1)
+        assert lib.amos_default_config(0, ctypes.byref(d), ctypes.byref(cfg)) == 0
+        assert lib.amos_check_config(0, ctypes.byref(d), ctypes.byref(cfg), None, None) == 0
+        name = lib.amos_kernel_name(0, ctypes.byref(d), ctypes.byref(cfg))
+        assert name is not None and name.startswith(b"amos_igemm<f16,")
+    d = gemm_desc(8192, 8192, 8192, tb=1)
+    lib.amos_default_config(0, ctypes.byref(d), ctypes.byref(cfg))
+    assert (cfg.tile_i, cfg.tile_j, cfg.split_k) == (256, 256, 1)
+
+
+def test_kernel_name_reflects_layout():
+    lib = _lib.load()
+    cfg = _lib.KernelConfig(128, 128, 1)
+    assert lib.amos_kernel_name(0, ctypes.byref(gemm_desc(256, 256, 256, tb=1)), ctypes.byref(cfg)) == \
+        b"amos_igemm<f16,vec,vec,128x128>"
+    assert lib.amos_kernel_name(0, ctypes.byref(gemm_desc(256, 256, 256)), ctypes.byref(cfg)) == \
+        b"amos_igemm<f16,vec,strided,128x128>"
+    assert lib.amos_kernel_name(0, ctypes.byref(gemm_desc(256, 256, 255, tb=1)), ctypes.byref(cfg)) == \
+        b"amos_igemm<f16,strided,strided,128x128>"
+    c = _lib.ConvDesc()
+    c.N, c.C, c.D, c.H, c.W, c.K, c.T, c.R, c.S = 2, 16, 1, 8, 8, 16, 1, 3, 3
+    c.stride_d = c.stride_h = c.stride_w = 1
+    c.dil_d = c.dil_h = c.dil_w = 1
+    c.pad_h = c.pad_w = 1
+    c.in_dtype, c.out_dtype = _lib.AMOS_I8, _lib.AMOS_I32
+    assert lib.amos_kernel_name(2, ctypes.byref(c), ctypes.byref(cfg)) == b"amos_igemm<i8,vec,im2col,128x128>"
+    c.R = 20   # window larger than the padded input
+    assert lib.amos_kernel_name(2, ctypes.byref(c), ctypes.byref(cfg)) is None
