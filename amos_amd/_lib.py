@@ -8,6 +8,8 @@ LIB_PATH = os.path.join(_HERE, "libamos_mi355x.so")
 AMOS_F16, AMOS_BF16, AMOS_I8, AMOS_F32, AMOS_I32 = range(5)
 AMOS_OP_GEMM, AMOS_OP_BGEMM, AMOS_OP_CONV2D, AMOS_OP_CONV3D = range(4)
 
+AMOS_PIPE_AUTO, AMOS_PIPE_STAGED, AMOS_PIPE_DIRECT4, AMOS_PIPE_DIRECT8 = range(4)
+
 AMOS_ERR_BAD_ARG = -1
 AMOS_ERR_UNSUPPORTED = -2
 AMOS_ERR_INFEASIBLE = -3
@@ -46,7 +48,8 @@ class ConvDesc(ctypes.Structure):
 
 
 class KernelConfig(ctypes.Structure):
-    _fields_ = [("tile_i", _i32), ("tile_j", _i32), ("split_k", _i32), ("reserved", _i32 * 5)]
+    _fields_ = [("tile_i", _i32), ("tile_j", _i32), ("split_k", _i32), ("pipeline", _i32),
+                ("reserved", _i32 * 4)]
 
 
 class AmosError(RuntimeError):

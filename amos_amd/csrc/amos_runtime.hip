@@ -9,6 +9,7 @@
 #include <string>
 
 #include "amos_mi355x.h"
+#include "gemm_tn_kernel.h"
 #include "igemm_instances.h"
 #include "mapper.h"
 
@@ -60,6 +61,9 @@ struct Plan {
   int split;
   // zero fill of the output before a split-K launch
   int64_t fill_rows, fill_cols, fill_ld;
+  // direct-to-LDS GEMM pipeline (0 = not used, else waves per block)
+  int tn_waves;
+  GemmTnParams tn;
 };
 
 static int dtype_pair(int in_dtype, int out_dtype, int* dt) {
@@ -148,7 +152,33 @@ static int plan_gemm(Plan& pl, int op, const void* desc_any, const amos_gemm_des
   pl.fill_rows = d->M;
   pl.fill_cols = d->N;
   pl.fill_ld = d->ldc;
-  return plan_finish(pl, op, desc_any, cfg);
+  rc = plan_finish(pl, op, desc_any, cfg);
+  if (rc) return rc;
+  // direct-to-LDS pipeline: both operands K-contiguous and 16-byte aligned, whole K steps,
+  // 32-bit byte offsets inside a 256-row tile
+  const int bke = 128 / es;
+  const bool tn_ok = pl.rl == LD_VEC && pl.cl == LD_VEC && d->K % bke == 0 && pl.split == 1 &&
+                     256 * d->lda * es + 128 < ((int64_t)1 << 32) &&
+                     256 * d->ldb * es + 128 < ((int64_t)1 << 32);
+  const int pipe = pl.cfg.pipeline;
+  if (pipe == AMOS_PIPE_DIRECT4 || pipe == AMOS_PIPE_DIRECT8) {
+    if (!tn_ok || pl.cfg.tile_i != 256 || pl.cfg.tile_j != 256)
+      return set_error(AMOS_ERR_INFEASIBLE,
+                       "direct-to-LDS pipeline needs K-contiguous 16-byte aligned operands, "
+                       "K %% %d == 0, tile 256x256 and split_k 1", bke);
+    pl.tn_waves = pipe == AMOS_PIPE_DIRECT4 ? 4 : 8;
+  } else if (pipe == AMOS_PIPE_AUTO && tn_ok && pl.cfg.tile_i == 256 && pl.cfg.tile_j == 256) {
+    pl.tn_waves = 8;  // measured a few percent ahead of 4 waves on the 8192^3 fp16 GEMM
+  }
+  if (pl.tn_waves) {
+    GemmTnParams& q = pl.tn;
+    q.a = (const char*)A; q.b = (const char*)B; q.c = (char*)C;
+    q.I = p.I; q.J = p.J; q.K = p.Kred;
+    q.lda = d->lda; q.ldb = d->ldb; q.ldc = d->ldc;
+    q.batch_a = sa; q.batch_b = sb; q.batch_c = sc;
+    q.tiles_i = p.tiles_i; q.tiles_j = p.tiles_j;
+  }
+  return 0;
 }
 
 static int conv_out_extent(int64_t in, int pad, int dil, int64_t k, int stride) {
@@ -220,6 +250,7 @@ static int plan_conv(Plan& pl, int op, const amos_conv_desc_t* d, const amos_ker
 
 static int make_plan(Plan& pl, int op, const void* desc, const amos_kernel_config_t* cfg,
                      const void* in0, const void* in1, void* out) {
+  pl.tn_waves = 0;
   switch (op) {
     case AMOS_OP_GEMM:
       return plan_gemm(pl, op, desc, (const amos_gemm_desc_t*)desc, 1, 0, 0, 0, cfg, in0, in1, out);
@@ -245,7 +276,25 @@ static int resolve(const Plan& pl, Instance** out) {
   return 0;
 }
 
+static int launch_tn(const Plan& pl, hipStream_t stream) {
+  TnInstance* inst = pick_gemm_tn(pl.dt, pl.tn_waves);
+  if (!inst) return set_error(AMOS_ERR_INFEASIBLE, "no direct-to-LDS instance");
+  hipError_t attr_err = hipSuccess;
+  std::call_once(inst->once, [&] {
+    attr_err = hipFuncSetAttribute((const void*)inst->fn, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                   (int)inst->lds);
+  });
+  if (attr_err != hipSuccess)
+    return set_error(AMOS_ERR_HIP, "hipFuncSetAttribute(%s): %s", inst->name,
+                     hipGetErrorString(attr_err));
+  dim3 grid((unsigned)(pl.tn.tiles_i * pl.tn.tiles_j), 1, (unsigned)pl.batch);
+  hipLaunchKernelGGL(inst->fn, grid, dim3(inst->threads), inst->lds, stream, pl.tn);
+  HIP_TRY(hipGetLastError());
+  return 0;
+}
+
 static int launch(const Plan& pl, hipStream_t stream) {
+  if (pl.tn_waves) return launch_tn(pl, stream);
   Instance* inst;
   int rc = resolve(pl, &inst);
   if (rc) return rc;
@@ -345,6 +394,10 @@ const char* amos_kernel_name(int op, const void* desc, const amos_kernel_config_
   static char dummy[16] __attribute__((aligned(16)));
   Plan pl;
   if (make_plan(pl, op, desc, cfg, dummy, dummy, dummy)) return nullptr;
+  if (pl.tn_waves) {
+    TnInstance* tn = pick_gemm_tn(pl.dt, pl.tn_waves);
+    return tn ? tn->name : nullptr;
+  }
   Instance* inst;
   if (resolve(pl, &inst)) return nullptr;
   return inst->name;

@@ -1,0 +1,176 @@
+// GEMM / batched GEMM with both operands K-contiguous ("ntn": A[M,K], B stored [N,K]),
+// the layout v_mfma wants: every lane's operand fragment is 16 contiguous bytes of K.
+//
+// Block tile 256x256, K step 128 bytes per row (64 halves / 128 int8), two LDS
+// stages of 64 KB.  Differences to the generic implicit-GEMM kernel:
+//   * global -> LDS copies are direct (global_load_lds_dwordx4): no staging
+//     registers, no ds_write; the XOR swizzle of the LDS layout is applied on the
+//     global-address side (a wave instruction fills 1 KB of LDS linearly, lane l
+//     fetches the 16-byte chunk that belongs at that position);
+//   * operand fragments are double buffered in registers: the ds_reads of K
+//     sub-step s+1 are in flight while the MFMAs of sub-step s issue;
+//   * one barrier per K step; the copies for step kt+2 are issued right after it and
+//     have a whole step to land.
+// Rows beyond M / N are clamped to the last valid row on load (their products only
+// reach outputs that are never stored); K must be a multiple of the K step.
+//
+// Role in the reference: the "kernel2" main loop that
+// python/tvm/auto_tensorize/tensorization_phases/schedulers/cuda_v2.py:582-825
+// schedules (cache_read to shared, load_matrix_sync, mma_sync, store_matrix_sync;
+// README.md:369-424) -- there with synchronous copies and no double buffering.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "igemm_kernel.h"
+
+namespace amos {
+
+struct GemmTnParams {
+  const char* a;   // row operand, [I][lda] elements, K contiguous
+  const char* b;   // column operand, [J][ldb]
+  char* c;         // [I][ldc] fp32 / int32
+  int I, J, K;
+  int64_t lda, ldb, ldc;
+  int64_t batch_a, batch_b, batch_c;  // elements between batches
+  int tiles_i, tiles_j;
+};
+
+#define AMOS_GLOBAL_PTR(p) ((const __attribute__((address_space(1))) void*)(p))
+#define AMOS_LDS_PTR(p) ((__attribute__((address_space(3))) void*)(p))
+
+template <int DT, int WI, int WJ>
+__global__ __launch_bounds__(64 * WI * WJ) void amos_gemm_tn(const GemmTnParams p) {
+  typedef Mfma<DT> MM;
+  typedef typename MM::acc_t acc_t;
+  typedef typename MM::out_t out_t;
+  constexpr int ES = MM::ES;
+  constexpr int BKE = 128 / ES;
+  constexpr int NW = WI * WJ;
+  constexpr int TI = 256 / (32 * WI), TJ = 256 / (32 * WJ);
+  constexpr int OPER = 256 * 128;      // bytes of one operand tile
+  constexpr int STAGE = 2 * OPER;      // A tile then B tile
+  constexpr int CH = 64 / NW;          // 1 KB copy chunks per wave per K step
+
+  extern __shared__ __attribute__((aligned(16))) char smem[];
+
+  const int t = threadIdx.x;
+  const int lane = t & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(t >> 6);
+  const int wi = wave / WJ, wj = wave % WJ;
+
+  int tile_i, tile_j;
+  block_to_tile(blockIdx.x, gridDim.x, p.tiles_i, p.tiles_j, tile_i, tile_j);
+  const int bi0 = tile_i * 256, bj0 = tile_j * 256;
+  const int64_t batch = blockIdx.z;
+  const char* const abase = p.a + (batch * p.batch_a + (int64_t)bi0 * p.lda) * ES;
+  const char* const bbase = p.b + (batch * p.batch_b + (int64_t)bj0 * p.ldb) * ES;
+
+  // ---- copy slots: chunk q of this wave covers tile rows [8*qq, 8*qq+8) of A (q < 32) or B
+  unsigned g_off[CH];   // byte offset from the operand's tile base, K step 0
+#pragma unroll
+  for (int u = 0; u < CH; ++u) {
+    const int q = wave + NW * u;       // 0..63, uniform per wave
+    const int qq = q & 31;
+    const int row = qq * 8 + (lane >> 3);
+    const int chunk = (lane & 7) ^ ((row ^ (row >> 3)) & 7);
+    if (q < 32) {
+      int r = bi0 + row < p.I ? row : p.I - 1 - bi0;
+      g_off[u] = (unsigned)r * (unsigned)(p.lda * ES) + chunk * 16;
+    } else {
+      int r = bj0 + row < p.J ? row : p.J - 1 - bj0;
+      g_off[u] = (unsigned)r * (unsigned)(p.ldb * ES) + chunk * 16;
+    }
+  }
+
+  auto issue_copies = [&](int kt, int stage) {
+    const char* ak = abase + (int64_t)kt * 128;
+    const char* bk = bbase + (int64_t)kt * 128;
+    char* s = smem + stage * STAGE;
+#pragma unroll
+    for (int u = 0; u < CH; ++u) {
+      const int q = wave + NW * u;
+      const char* src = (q < 32 ? ak : bk) + g_off[u];
+      __builtin_amdgcn_global_load_lds(AMOS_GLOBAL_PTR(src), AMOS_LDS_PTR(s + q * 1024), 16, 0, 0);
+    }
+  };
+
+  // ---- fragment read offsets: row = tile_row0 + a*32 + lane%32, chunk = 2*ks + lane/32
+  const int frag_row = lane & 31, frag_half = lane >> 5;
+  int a_off[2][4], b_off[2][4];   // [a & 1][ks]: the swizzle term flips with the parity of a
+#pragma unroll
+  for (int par = 0; par < 2; ++par)
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks) {
+      a_off[par][ks] = lds_chunk_offset(wi * TI * 32 + par * 32 + frag_row, ks * 2 + frag_half);
+      b_off[par][ks] = OPER + lds_chunk_offset(wj * TJ * 32 + par * 32 + frag_row, ks * 2 + frag_half);
+    }
+
+  acc_t acc[TI][TJ];
+#pragma unroll
+  for (int a = 0; a < TI; ++a)
+#pragma unroll
+    for (int b = 0; b < TJ; ++b)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[a][b][r] = 0;
+
+  v4i af[2][TI], bf[2][TJ];
+  auto read_frags = [&](int stage, int ks, int slot) {
+    const char* s = smem + stage * STAGE;
+#pragma unroll
+    for (int a = 0; a < TI; ++a)
+      af[slot][a] = *(const v4i*)(s + a_off[a & 1][ks] + (a >> 1) * (64 * 128));
+#pragma unroll
+    for (int b = 0; b < TJ; ++b)
+      bf[slot][b] = *(const v4i*)(s + b_off[b & 1][ks] + (b >> 1) * (64 * 128));
+  };
+  auto mma = [&](int slot) {
+#pragma unroll
+    for (int a = 0; a < TI; ++a)
+#pragma unroll
+      for (int b = 0; b < TJ; ++b) acc[a][b] = MM::run(af[slot][a], bf[slot][b], acc[a][b]);
+  };
+
+  const int KT = p.K / BKE;
+  issue_copies(0, 0);
+  if (KT > 1) issue_copies(1, 1);
+  // stage 0 must have landed; stage 1 may still be in flight, but a counter wait cannot
+  // tell them apart cheaply here, so wait for both once
+  asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");
+  read_frags(0, 0, 0);
+
+  for (int kt = 0; kt < KT; ++kt) {
+    const int st = kt & 1;
+    read_frags(st, 1, 1);
+    mma(0);
+    read_frags(st, 2, 0);
+    mma(1);
+    read_frags(st, 3, 1);
+    mma(0);
+    // every ds_read of this stage has been issued; once they and this wave's copies of the
+    // other stage are complete, meet the other waves: after the barrier the other stage
+    // is fully written and this stage is free to be overwritten
+    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+    if (kt + 2 < KT) issue_copies(kt + 2, st);
+    if (kt + 1 < KT) read_frags(st ^ 1, 0, 0);
+    mma(1);
+  }
+
+  // ---- epilogue ---------------------------------------------------------------------
+  out_t* const out = (out_t*)p.c + batch * p.batch_c;
+#pragma unroll
+  for (int b = 0; b < TJ; ++b) {
+    const int j = bj0 + (wj * TJ + b) * 32 + frag_row;
+    if (j >= p.J) continue;
+#pragma unroll
+    for (int a = 0; a < TI; ++a) {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int i = bi0 + (wi * TI + a) * 32 + 8 * (r >> 2) + 4 * frag_half + (r & 3);
+        if (i < p.I) out[(int64_t)i * p.ldc + j] = acc[a][b][r];
+      }
+    }
+  }
+}
+
+}  // namespace amos

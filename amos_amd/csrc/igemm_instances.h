@@ -52,6 +52,18 @@ Instance* pick_col(int cl, int ti, int tj) {
   return nullptr;
 }
 
+struct GemmTnParams;
+typedef void (*gemm_tn_fn)(const GemmTnParams);
+struct TnInstance {
+  gemm_tn_fn fn;
+  size_t lds;
+  int threads;
+  const char* name;
+  std::once_flag once;
+};
+// direct-to-LDS GEMM (defined in inst_gemm_tn.hip); waves = 4 or 8
+TnInstance* pick_gemm_tn(int dt, int waves);
+
 Instance* pick_f16_vec(int cl, int ti, int tj);
 Instance* pick_f16_strided(int cl, int ti, int tj);
 Instance* pick_bf16_vec(int cl, int ti, int tj);

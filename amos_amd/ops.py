@@ -40,6 +40,7 @@ def make_config(config):
     c.tile_i = int(config.get("tile_i", 0))
     c.tile_j = int(config.get("tile_j", 0))
     c.split_k = int(config.get("split_k", 0))
+    c.pipeline = int(config.get("pipeline", 0))
     return c
 
 

@@ -122,9 +122,16 @@ typedef struct {
  */
 typedef struct {
   int32_t tile_i, tile_j;   /* block tile of the MFMA row / column operand: 64, 128 or 256 */
-  int32_t split_k;          /* >= 1; > 1 needs workspace                                    */
-  int32_t reserved[5];
+  int32_t split_k;          /* >= 1: blocks along the fused reduction                       */
+  int32_t pipeline;         /* AMOS_PIPE_*; 0 = mapper's choice                             */
+  int32_t reserved[4];
 } amos_kernel_config_t;
+
+/* how tiles travel from HBM to the MFMA operands */
+#define AMOS_PIPE_AUTO 0
+#define AMOS_PIPE_STAGED 1    /* global -> registers -> LDS, any layout, ragged K             */
+#define AMOS_PIPE_DIRECT4 2   /* global -> LDS direct copies, 256x256 tile, 4 waves           */
+#define AMOS_PIPE_DIRECT8 3   /* same with 8 waves (two per SIMD)                             */
 
 int amos_version(void);
 const char* amos_last_error(void);

@@ -85,6 +85,37 @@ def test_gemm_every_tile(gpu, dtype, tile, split):
     check(got, ref, dtype, "gemm tile %s split %d" % (tile, split))
 
 
+@pytest.mark.parametrize("dtype", ["float16", "bfloat16", "int8"])
+@pytest.mark.parametrize("pipeline", [2, 3])   # direct-to-LDS copies, 4 and 8 waves
+@pytest.mark.parametrize("shape", [(256, 256, 128), (512, 768, 1024), (300, 520, 384), (1, 257, 128)])
+def test_gemm_direct_pipeline(gpu, dtype, pipeline, shape):
+    from amos_amd import _lib, ops
+    M, N, K = shape
+    rng = np.random.default_rng(M * 7 + N * 3 + K)
+    a = make_operand(rng, (M, K), dtype)
+    b = make_operand(rng, (N, K), dtype)
+    cfg = dict(tile_i=256, tile_j=256, split_k=1, pipeline=pipeline)
+    d = ops.gemm_desc(M, N, K, to_device(a, dtype).dtype, False, True)
+    assert "amos_gemm_tn" in ops.kernel_name(_lib.AMOS_OP_GEMM, d, cfg)
+    got = ops.gemm(to_device(a, dtype), to_device(b, dtype), False, True, config=cfg).cpu().numpy()
+    check(got, co.lib_gemm(a, b, dtype, False, True, acc="float64"), dtype,
+          "direct gemm %s pipe %d %s" % (dtype, pipeline, shape))
+    # batched through the same kernel
+    ab = make_operand(rng, (3, M, K), dtype)
+    bb = make_operand(rng, (3, N, K), dtype)
+    gb = ops.bgemm(to_device(ab, dtype), to_device(bb, dtype), False, True, config=cfg).cpu().numpy()
+    check(gb, co.lib_gemm(ab, bb, dtype, False, True, acc="float64"), dtype, "direct bgemm")
+
+
+def test_gemm_direct_pipeline_rejects_ragged_k(gpu):
+    import torch
+    from amos_amd import _lib, ops
+    a = torch.zeros((256, 72), dtype=torch.float16, device="cuda")
+    with pytest.raises(_lib.AmosError) as e:
+        ops.gemm(a, a, False, True, config=dict(tile_i=256, tile_j=256, split_k=1, pipeline=2))
+    assert e.value.code == _lib.AMOS_ERR_INFEASIBLE
+
+
 def test_gemm_config1_512(gpu):
     """fp16 GEMM 512^3, inputs U[-1,1], against the full te_literal loop nest"""
     from amos_amd import ops
