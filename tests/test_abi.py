@@ -32,6 +32,7 @@ def test_struct_sizes_match_header():
     assert ctypes.sizeof(_lib.BGemmDesc) == 8 + ctypes.sizeof(_lib.GemmDesc) + 3 * 8
     assert ctypes.sizeof(_lib.ConvDesc) == 9 * 8 + 11 * 4 + 4
     assert ctypes.sizeof(_lib.KernelConfig) == 32
+    assert _lib.KernelConfig.pipeline.offset == 12
 
 
 def gemm_desc(M, N, K, ind=_lib.AMOS_F16, outd=_lib.AMOS_F32, ta=0, tb=0):
@@ -77,10 +78,14 @@ def test_default_config_is_a_compiled_instance():
         assert lib.amos_default_config(0, ctypes.byref(d), ctypes.byref(cfg)) == 0
         assert lib.amos_check_config(0, ctypes.byref(d), ctypes.byref(cfg), None, None) == 0
         name = lib.amos_kernel_name(0, ctypes.byref(d), ctypes.byref(cfg))
-        assert name is not None and name.startswith(b"amos_igemm<f16,")
+        assert name is not None and (name.startswith(b"amos_igemm<f16,") or name.startswith(b"amos_gemm_tn<f16,"))
     d = gemm_desc(8192, 8192, 8192, tb=1)
     lib.amos_default_config(0, ctypes.byref(d), ctypes.byref(cfg))
     assert (cfg.tile_i, cfg.tile_j, cfg.split_k) == (256, 256, 1)
+    # aligned K-contiguous operands at 256x256 take the direct-to-LDS pipeline
+    assert lib.amos_kernel_name(0, ctypes.byref(d), ctypes.byref(cfg)) == b"amos_gemm_tn<f16,256x256,8w>"
+    staged = _lib.KernelConfig(256, 256, 1, _lib.AMOS_PIPE_STAGED)
+    assert lib.amos_kernel_name(0, ctypes.byref(d), ctypes.byref(staged)) == b"amos_igemm<f16,vec,vec,256x256>"
 
 
 def test_kernel_name_reflects_layout():
