@@ -9,6 +9,7 @@
 #include <string>
 
 #include "amos_mi355x.h"
+#include "conv_fprop_kernel.h"
 #include "gemm_tn_kernel.h"
 #include "igemm_instances.h"
 #include "mapper.h"
@@ -64,6 +65,10 @@ struct Plan {
   // direct-to-LDS GEMM pipeline (0 = not used, else waves per block)
   int tn_waves;
   GemmTnParams tn;
+  // patch-staged convolution (0 = not used)
+  int conv_ups;
+  ConvFpropParams cv;
+  size_t conv_lds;
 };
 
 static int dtype_pair(int in_dtype, int out_dtype, int* dt) {
@@ -188,8 +193,50 @@ static int conv_out_extent(int64_t in, int pad, int dil, int64_t k, int stride) 
   return (int)o;
 }
 
+// worst case over the J tiles of the patch a block stages: LDS positions and slices touched
+static void conv_patch_extent(int64_t J, int OPQ, int OQ, int BJ, int sh, int R, int dh, int Wp,
+                              int* max_pos, int* max_seg) {
+  *max_pos = 0;
+  *max_seg = 0;
+  const int64_t tiles = (J + BJ - 1) / BJ;
+  // the pattern of (tile start mod OPQ) repeats after OPQ / gcd(BJ, OPQ) tiles
+  int64_t a = BJ, b = OPQ;
+  while (b) { int64_t r = a % b; a = b; b = r; }
+  int64_t period = OPQ / a + 1;
+  const int64_t scan = tiles < period ? tiles : period;
+  for (int64_t tj = 0; tj <= scan; ++tj) {
+    int64_t t2 = tj == scan ? tiles - 1 : tj;   // the ragged last tile too
+    int64_t j0 = t2 * BJ, j1 = j0 + BJ - 1 < J - 1 ? j0 + BJ - 1 : J - 1;
+    int64_t sa = j0 / OPQ, sb = j1 / OPQ;
+    int pos = 0;
+    for (int64_t sl = sa; sl <= sb; ++sl) {
+      int64_t lo = j0 > sl * OPQ ? j0 : sl * OPQ;
+      int64_t hi = j1 < (sl + 1) * OPQ - 1 ? j1 : (sl + 1) * OPQ - 1;
+      int pa = (int)((lo - sl * OPQ) / OQ), pb = (int)((hi - sl * OPQ) / OQ);
+      pos += ((pb - pa) * sh + (R - 1) * dh + 1) * Wp;
+    }
+    if (pos > *max_pos) *max_pos = pos;
+    if ((int)(sb - sa + 1) > *max_seg) *max_seg = (int)(sb - sa + 1);
+  }
+}
+
+// workspace of the patch-staged pipeline: [packed weights | 256 zero bytes | NDHWC activations]
+static int64_t conv_packed_bytes(const amos_conv_desc_t& c, int op) {
+  int64_t T = op == AMOS_OP_CONV2D ? 1 : c.T;
+  int es = c.in_dtype == AMOS_I8 ? 1 : 2;
+  if (c.C <= 0 || (c.C * es) % 128 != 0) return 0;
+  return (c.K * T * c.R * c.S * c.C * es + 255) / 256 * 256;
+}
+static int64_t conv_workspace_bytes(const amos_conv_desc_t& c, int op) {
+  int64_t packed = conv_packed_bytes(c, op);
+  if (packed == 0) return 0;
+  int64_t D = op == AMOS_OP_CONV2D ? 1 : c.D;
+  int es = c.in_dtype == AMOS_I8 ? 1 : 2;
+  return packed + 256 + c.N * c.C * D * c.H * c.W * es;
+}
+
 static int plan_conv(Plan& pl, int op, const amos_conv_desc_t* d, const amos_kernel_config_t* cfg,
-                     const void* X, const void* Wt, void* Y) {
+                     const void* X, const void* Wt, void* Y, void* workspace, size_t ws_bytes) {
   if (!d || !X || !Wt || !Y) return set_error(AMOS_ERR_BAD_ARG, "null pointer argument");
   amos_conv_desc_t c = *d;
   if (op == AMOS_OP_CONV2D) {
@@ -245,12 +292,113 @@ static int plan_conv(Plan& pl, int op, const amos_conv_desc_t* d, const amos_ker
   pl.fill_rows = 1;
   pl.fill_cols = c.N * c.K * odpq;
   pl.fill_ld = pl.fill_cols;
-  return plan_finish(pl, op, d, cfg);
+  rc = plan_finish(pl, op, d, cfg);
+  if (rc) return rc;
+
+  // ---- patch-staged pipeline: channels fill whole 128-byte K steps, the relaid operands fit
+  // the workspace, the patch of a tile fits LDS next to a ring of weight tiles
+  const int pipe = pl.cfg.pipeline;
+  if (pipe == AMOS_PIPE_STAGED) return 0;
+  const char* why = nullptr;
+  const int64_t packed = conv_packed_bytes(c, op);
+  const int64_t need_ws = conv_workspace_bytes(c, op);
+  const int BI = pl.cfg.tile_i, BJ = pl.cfg.tile_j;
+  int max_pos = 0, max_seg = 0, nsw = 0, pls = 0;
+  size_t lds = 0;
+  const int RS = (int)(c.R * c.S);
+  const int Wp = (OQ - 1) * c.stride_w + ((int)c.S - 1) * c.dil_w + 1;
+  const bool tile_ok = (BI == 64 && (BJ == 64 || BJ == 128 || BJ == 256)) ||
+                       (BI == 128 && (BJ == 64 || BJ == 128 || BJ == 256)) ||
+                       (BI == 256 && (BJ == 64 || BJ == 128));
+  if (packed == 0) why = "C * element size is not a multiple of 128 bytes";
+  else if (packed >= ((int64_t)1 << 32)) why = "packed weights above 4 GiB";
+  else if (c.N * c.D * c.H * c.W >= ((int64_t)1 << 31) || J >= ((int64_t)1 << 31) - 512)
+    why = "more than 2^31 input or output positions";
+  else if (c.D + 2 * (int64_t)c.pad_d + c.T * c.dil_d >= 30000) why = "depth extent above 30000";
+  else if (!workspace || ws_bytes < (size_t)need_ws || ((uintptr_t)workspace & 255))
+    why = "workspace smaller than amos_workspace_bytes() or not 256-byte aligned";
+  else if (!tile_ok) why = "no patch-staged instance with this block tile";
+  if (!why) {
+    conv_patch_extent(J, OP * OQ, OQ, BJ, c.stride_h, (int)c.R, c.dil_h, Wp, &max_pos, &max_seg);
+    max_pos = (max_pos + 7) & ~7;
+    const size_t budget = (size_t)160 * 1024 - 512;
+    const size_t patch = (size_t)2 * max_pos * 128 + (size_t)max_pos * 8;
+    const size_t wstage = (size_t)BI * 128;
+    if (max_seg > kConvMaxSeg) why = "a tile spans more than 4 image slices";
+    else if (max_pos >= 4096) why = "input patch of a tile has 4096 or more positions";
+    else if (patch + 2 * wstage > budget) why = "input patch of a tile does not fit LDS";
+    else {
+      nsw = (int)((budget - patch) / wstage);
+      if (nsw > 8) nsw = 8;
+      if (nsw > RS + 1) nsw = RS + 1;
+      // The next patch is copied during the taps of the current one.  A copy issued on tap u
+      // is complete for everybody at the barrier of the patch's last tap only if u <= RS-2
+      // and it is older than the weight tiles still allowed in flight there: u <= RS+1-nsw.
+      int taps = RS + 2 - nsw < RS - 1 ? RS + 2 - nsw : RS - 1;
+      const int64_t macro_steps = c.T * (c.C * es / 128);
+      int split = pl.cfg.split_k < 1 ? 1 : pl.cfg.split_k;
+      const bool one_macro = (macro_steps + split - 1) / split <= 1;   // no next patch at all
+      if (taps < 1 && !one_macro) why = "1x1 window with several channel chunks per block";
+      if (taps < 1) taps = 1;
+      const int per_wave = ((max_pos / 8) + 3) / 4;
+      pls = (per_wave + taps - 1) / taps;
+      if (pls < 1) pls = 1;
+      lds = (size_t)nsw * wstage + patch;
+    }
+  }
+  if (why) {
+    if (pipe == AMOS_PIPE_PATCH)
+      return set_error(AMOS_ERR_INFEASIBLE, "patch-staged convolution not applicable: %s", why);
+    return 0;   // register-staged implicit GEMM handles it
+  }
+  pl.conv_ups = 1;
+  pl.conv_lds = lds;
+  ConvFpropParams& q = pl.cv;
+  memset(&q, 0, sizeof(q));
+  q.x = (const char*)X; q.w = (const char*)Wt; q.y = (char*)Y;
+  q.wp = (char*)workspace;
+  q.zeros = (char*)workspace + packed;
+  q.xt = (char*)workspace + packed + 256;
+  q.N = (int)c.N; q.C = (int)c.C; q.D = (int)c.D; q.H = (int)c.H; q.W = (int)c.W; q.K = (int)c.K;
+  q.T = (int)c.T; q.R = (int)c.R; q.S = (int)c.S;
+  q.sd = c.stride_d; q.sh = c.stride_h; q.sw = c.stride_w;
+  q.pd = c.pad_d; q.ph = c.pad_h; q.pw = c.pad_w;
+  q.dd = c.dil_d; q.dh = c.dil_h; q.dw = c.dil_w;
+  q.OD = OD; q.OP = OP; q.OQ = OQ;
+  q.J = (int)J;
+  q.Wp = Wp;
+  q.max_pos = max_pos;
+  q.nsw = nsw;
+  q.pls = pls;
+  q.c_chunks = (int)(c.C * es / 128);
+  q.macro_steps = (int)c.T * q.c_chunks;
+  int split = pl.cfg.split_k < 1 ? 1 : pl.cfg.split_k;
+  if (split > q.macro_steps) split = q.macro_steps;
+  q.macro_per_split = (q.macro_steps + split - 1) / split;
+  split = (q.macro_steps + q.macro_per_split - 1) / q.macro_per_split;
+  pl.split = split;
+  q.atomic_out = split > 1;
+  q.tiles_i = (int)((c.K + BI - 1) / BI);
+  q.tiles_j = (int)((J + BJ - 1) / BJ);
+  q.zero_words = split > 1 ? c.N * c.K * odpq : 0;
+  q.fd_opq = make_fast_div((uint32_t)(OP * OQ));
+  q.fd_oq = make_fast_div((uint32_t)OQ);
+  q.fd_od = make_fast_div((uint32_t)OD);
+  q.fd_wp = make_fast_div((uint32_t)Wp);
+  q.fd_odpq = make_fast_div((uint32_t)odpq);
+  q.fd_cc = make_fast_div((uint32_t)q.c_chunks);
+  const int64_t welems = c.K * c.T * c.R * c.S * c.C;
+  q.prep_w_blocks = (int)((welems + 2047) / 2048 < 1024 ? (welems + 2047) / 2048 : 1024);
+  q.prep_x_blocks = (int)(c.N * c.D * (((int64_t)c.H * c.W + 63) / 64) * (c.C / 64));
+  q.prep_z_blocks = q.zero_words ? (int)((q.zero_words + 4095) / 4096 < 2048 ? (q.zero_words + 4095) / 4096 : 2048) : 0;
+  return 0;
 }
 
 static int make_plan(Plan& pl, int op, const void* desc, const amos_kernel_config_t* cfg,
-                     const void* in0, const void* in1, void* out) {
+                     const void* in0, const void* in1, void* out, void* workspace = nullptr,
+                     size_t ws_bytes = 0) {
   pl.tn_waves = 0;
+  pl.conv_ups = 0;
   switch (op) {
     case AMOS_OP_GEMM:
       return plan_gemm(pl, op, desc, (const amos_gemm_desc_t*)desc, 1, 0, 0, 0, cfg, in0, in1, out);
@@ -262,7 +410,7 @@ static int make_plan(Plan& pl, int op, const void* desc, const amos_kernel_confi
     }
     case AMOS_OP_CONV2D:
     case AMOS_OP_CONV3D:
-      return plan_conv(pl, op, (const amos_conv_desc_t*)desc, cfg, in0, in1, out);
+      return plan_conv(pl, op, (const amos_conv_desc_t*)desc, cfg, in0, in1, out, workspace, ws_bytes);
   }
   return set_error(AMOS_ERR_BAD_ARG, "unknown op %d", op);
 }
@@ -293,8 +441,34 @@ static int launch_tn(const Plan& pl, hipStream_t stream) {
   return 0;
 }
 
+static ConvInstance* pick_conv(int dt, int ti, int tj) {
+  if (dt == DT_F16) return pick_conv_f16(ti, tj);
+  if (dt == DT_BF16) return pick_conv_bf16(ti, tj);
+  return pick_conv_i8(ti, tj);
+}
+
+static int launch_conv(const Plan& pl, hipStream_t stream) {
+  ConvInstance* inst = pick_conv(pl.dt, pl.cfg.tile_i, pl.cfg.tile_j);
+  if (!inst) return set_error(AMOS_ERR_INFEASIBLE, "no patch-staged convolution instance");
+  hipError_t attr_err = hipSuccess;
+  std::call_once(inst->once, [&] {
+    attr_err = hipFuncSetAttribute((const void*)inst->fn, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                   160 * 1024 - 512);
+  });
+  if (attr_err != hipSuccess)
+    return set_error(AMOS_ERR_HIP, "hipFuncSetAttribute(%s): %s", inst->name,
+                     hipGetErrorString(attr_err));
+  const ConvFpropParams& q = pl.cv;
+  launch_conv_prepare(pl.dt == DT_I8 ? 1 : 2, q, stream);
+  dim3 grid((unsigned)(q.tiles_i * q.tiles_j), (unsigned)pl.split, 1);
+  hipLaunchKernelGGL(inst->fn, grid, dim3(256), pl.conv_lds, stream, q);
+  HIP_TRY(hipGetLastError());
+  return 0;
+}
+
 static int launch(const Plan& pl, hipStream_t stream) {
   if (pl.tn_waves) return launch_tn(pl, stream);
+  if (pl.conv_ups) return launch_conv(pl, stream);
   Instance* inst;
   int rc = resolve(pl, &inst);
   if (rc) return rc;
@@ -327,9 +501,9 @@ static int launch(const Plan& pl, hipStream_t stream) {
 }
 
 static int run_op(int op, const void* desc, const amos_kernel_config_t* cfg, const void* in0,
-                  const void* in1, void* out, void* stream) {
+                  const void* in1, void* out, void* workspace, size_t ws_bytes, void* stream) {
   Plan pl;
-  int rc = make_plan(pl, op, desc, cfg, in0, in1, out);
+  int rc = make_plan(pl, op, desc, cfg, in0, in1, out, workspace, ws_bytes);
   if (rc) return rc;
   return launch(pl, (hipStream_t)stream);
 }
@@ -365,35 +539,41 @@ int amos_device_info(amos_device_info_t* out) {
 
 int amos_gemm(const amos_gemm_desc_t* desc, const amos_kernel_config_t* cfg, const void* A,
               const void* B, void* C, void* workspace, size_t ws_bytes, void* stream) {
-  (void)workspace; (void)ws_bytes;
-  return run_op(AMOS_OP_GEMM, desc, cfg, A, B, C, stream);
+  return run_op(AMOS_OP_GEMM, desc, cfg, A, B, C, workspace, ws_bytes, stream);
 }
 int amos_bgemm(const amos_bgemm_desc_t* desc, const amos_kernel_config_t* cfg, const void* A,
                const void* B, void* C, void* workspace, size_t ws_bytes, void* stream) {
-  (void)workspace; (void)ws_bytes;
-  return run_op(AMOS_OP_BGEMM, desc, cfg, A, B, C, stream);
+  return run_op(AMOS_OP_BGEMM, desc, cfg, A, B, C, workspace, ws_bytes, stream);
 }
 int amos_conv2d(const amos_conv_desc_t* desc, const amos_kernel_config_t* cfg, const void* X,
                 const void* Wt, void* Y, void* workspace, size_t ws_bytes, void* stream) {
-  (void)workspace; (void)ws_bytes;
-  return run_op(AMOS_OP_CONV2D, desc, cfg, X, Wt, Y, stream);
+  return run_op(AMOS_OP_CONV2D, desc, cfg, X, Wt, Y, workspace, ws_bytes, stream);
 }
 int amos_conv3d(const amos_conv_desc_t* desc, const amos_kernel_config_t* cfg, const void* X,
                 const void* Wt, void* Y, void* workspace, size_t ws_bytes, void* stream) {
-  (void)workspace; (void)ws_bytes;
-  return run_op(AMOS_OP_CONV3D, desc, cfg, X, Wt, Y, stream);
+  return run_op(AMOS_OP_CONV3D, desc, cfg, X, Wt, Y, workspace, ws_bytes, stream);
 }
 
 size_t amos_workspace_bytes(int op, const void* desc, const amos_kernel_config_t* cfg) {
-  (void)op; (void)desc; (void)cfg;
-  return 0;  // split-K accumulates straight into the (zero-filled) output
+  // GEMM: none (split-K accumulates straight into the zero-filled output).
+  // conv: room for the weights repacked to K,(TRS),C when the patch-staged pipeline applies.
+  (void)cfg;
+  if (!desc || (op != AMOS_OP_CONV2D && op != AMOS_OP_CONV3D)) return 0;
+  return (size_t)conv_workspace_bytes(*(const amos_conv_desc_t*)desc, op);
 }
 
 const char* amos_kernel_name(int op, const void* desc, const amos_kernel_config_t* cfg) {
   // pointers only matter for their alignment here; use aligned dummies
   static char dummy[16] __attribute__((aligned(16)));
   Plan pl;
-  if (make_plan(pl, op, desc, cfg, dummy, dummy, dummy)) return nullptr;
+  // a workspace "large enough" so that the name is the one a caller who provides
+  // amos_workspace_bytes() gets
+  static char dummy_ws[256] __attribute__((aligned(256)));
+  if (make_plan(pl, op, desc, cfg, dummy, dummy, dummy, dummy_ws, (size_t)-1)) return nullptr;
+  if (pl.conv_ups) {
+    ConvInstance* ci = pick_conv(pl.dt, pl.cfg.tile_i, pl.cfg.tile_j);
+    return ci ? ci->name : nullptr;
+  }
   if (pl.tn_waves) {
     TnInstance* tn = pick_gemm_tn(pl.dt, pl.tn_waves);
     return tn ? tn->name : nullptr;
@@ -406,12 +586,11 @@ const char* amos_kernel_name(int op, const void* desc, const amos_kernel_config_
 int amos_time(int op, const void* desc, const amos_kernel_config_t* cfg, const void* in0,
               const void* in1, void* out, void* workspace, size_t ws_bytes, void* stream_v,
               int number, int repeat, int min_repeat_ms, double* out_seconds) {
-  (void)workspace; (void)ws_bytes;
   if (!out_seconds || number < 1 || repeat < 1)
     return set_error(AMOS_ERR_BAD_ARG, "amos_time needs number >= 1, repeat >= 1 and an output array");
   hipStream_t stream = (hipStream_t)stream_v;
   Plan pl;
-  int rc = make_plan(pl, op, desc, cfg, in0, in1, out);
+  int rc = make_plan(pl, op, desc, cfg, in0, in1, out, workspace, ws_bytes);
   if (rc) return rc;
   rc = launch(pl, stream);  // warm-up
   if (rc) return rc;

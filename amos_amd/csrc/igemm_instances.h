@@ -39,6 +39,8 @@ Instance* pick_tile(int ti, int tj) {
   if (ti == 64 && tj == 128) return instance<DT, RL, CL, 1, 2>();
   if (ti == 256 && tj == 128) return instance<DT, RL, CL, 4, 2>();
   if (ti == 128 && tj == 256) return instance<DT, RL, CL, 2, 4>();
+  if (ti == 256 && tj == 64) return instance<DT, RL, CL, 4, 1>();
+  if (ti == 64 && tj == 256) return instance<DT, RL, CL, 1, 4>();
   return nullptr;
 }
 
@@ -63,6 +65,44 @@ struct TnInstance {
 };
 // direct-to-LDS GEMM (defined in inst_gemm_tn.hip); waves = 4 or 8
 TnInstance* pick_gemm_tn(int dt, int waves);
+
+// patch-staged convolution (defined in inst_conv_*.hip)
+struct ConvFpropParams;
+typedef void (*conv_fprop_fn)(const ConvFpropParams);
+struct ConvInstance {
+  conv_fprop_fn fn;
+  const char* name;
+  std::once_flag once;
+};
+ConvInstance* pick_conv_f16(int ti, int tj);
+ConvInstance* pick_conv_bf16(int ti, int tj);
+ConvInstance* pick_conv_i8(int ti, int tj);
+void launch_conv_prepare(int es, const ConvFpropParams& p, hipStream_t stream);
+
+#ifdef AMOS_CONV_FPROP_KERNEL_INCLUDED
+template <int DT, int TI, int TJ>
+ConvInstance* conv_instance() {
+  static ConvInstance inst;
+  static const char* dtn[] = {"f16", "bf16", "i8"};
+  static std::string name = std::string("amos_conv_fprop<") + dtn[DT] + "," + std::to_string(64 * TI) +
+                            "x" + std::to_string(64 * TJ) + ">";
+  inst.fn = amos_conv_fprop<DT, TI, TJ>;
+  inst.name = name.c_str();
+  return &inst;
+}
+template <int DT>
+ConvInstance* pick_conv_tile(int ti, int tj) {
+  if (ti == 64 && tj == 64) return conv_instance<DT, 1, 1>();
+  if (ti == 128 && tj == 64) return conv_instance<DT, 2, 1>();
+  if (ti == 64 && tj == 128) return conv_instance<DT, 1, 2>();
+  if (ti == 128 && tj == 128) return conv_instance<DT, 2, 2>();
+  if (ti == 256 && tj == 64) return conv_instance<DT, 4, 1>();
+  if (ti == 256 && tj == 128) return conv_instance<DT, 4, 2>();
+  if (ti == 128 && tj == 256) return conv_instance<DT, 2, 4>();
+  if (ti == 64 && tj == 256) return conv_instance<DT, 1, 4>();
+  return nullptr;
+}
+#endif
 
 Instance* pick_f16_vec(int cl, int ti, int tj);
 Instance* pick_f16_strided(int cl, int ti, int tj);

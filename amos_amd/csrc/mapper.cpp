@@ -70,7 +70,7 @@ int problem_of(int op, const void* desc, Problem* out) {
 }
 
 static const int kTiles[][2] = {{256, 256}, {256, 128}, {128, 256}, {128, 128},
-                                {128, 64},  {64, 128},  {64, 64}};
+                                {256, 64},  {128, 64},  {64, 128},  {64, 64},   {64, 256}};
 
 static int64_t lds_bytes_of(int ti, int tj) { return 2ll * (ti + tj) * 128 + 2 * 128 * 8; }
 // accumulator registers per lane: (ti/2 x tj/2 wave tile) / 64 lanes

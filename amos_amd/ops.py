@@ -130,6 +130,16 @@ def bgemm(a, b, trans_a=False, trans_b=False, out=None, config=None, stream=None
     return out
 
 
+def _workspace(op, desc, cfg, device):
+    """device scratch of amos_workspace_bytes() (conv: repacked weights); (tensor, ptr, bytes)"""
+    need = _lib.load().amos_workspace_bytes(op, ctypes.byref(desc), _cfg_ref(cfg))
+    if need == 0:
+        return None, None, 0
+    ws = torch.empty(need + 256, dtype=torch.uint8, device=device)
+    ptr = (ws.data_ptr() + 255) // 256 * 256
+    return ws, ptr, need
+
+
 def conv2d(x, w, stride=1, pad=0, dil=1, out=None, config=None, stream=None):
     """x NCHW, w KCRS -> NKPQ"""
     _need_device(x, w)
@@ -145,8 +155,9 @@ def conv2d(x, w, stride=1, pad=0, dil=1, out=None, config=None, stream=None):
     _need_device(out)
     d = conv_desc(xs, ws, x.dtype, st, pd, dl)
     cfg = make_config(config)
+    ws, ws_ptr, ws_bytes = _workspace(AMOS_OP_CONV2D, d, cfg, x.device)
     check(_lib.load().amos_conv2d(ctypes.byref(d), _cfg_ref(cfg), x.data_ptr(), w.data_ptr(),
-                                  out.data_ptr(), None, 0, _stream_ptr(stream)))
+                                  out.data_ptr(), ws_ptr, ws_bytes, _stream_ptr(stream)))
     return out
 
 
@@ -162,8 +173,9 @@ def conv3d(x, w, stride=1, pad=0, dil=1, out=None, config=None, stream=None):
     _need_device(out)
     d = conv_desc(tuple(x.shape), tuple(w.shape), x.dtype, st, pd, dl)
     cfg = make_config(config)
+    ws, ws_ptr, ws_bytes = _workspace(AMOS_OP_CONV3D, d, cfg, x.device)
     check(_lib.load().amos_conv3d(ctypes.byref(d), _cfg_ref(cfg), x.data_ptr(), w.data_ptr(),
-                                  out.data_ptr(), None, 0, _stream_ptr(stream)))
+                                  out.data_ptr(), ws_ptr, ws_bytes, _stream_ptr(stream)))
     return out
 
 
@@ -172,8 +184,9 @@ def time_op(op, desc, in0, in1, out, config=None, number=100, repeat=1, min_repe
     _need_device(in0, in1, out)
     cfg = make_config(config)
     res = (ctypes.c_double * repeat)()
+    ws, ws_ptr, ws_bytes = _workspace(op, desc, cfg, in0.device)
     check(_lib.load().amos_time(op, ctypes.byref(desc), _cfg_ref(cfg), in0.data_ptr(), in1.data_ptr(),
-                                out.data_ptr(), None, 0, _stream_ptr(stream), number, repeat,
+                                out.data_ptr(), ws_ptr, ws_bytes, _stream_ptr(stream), number, repeat,
                                 min_repeat_ms, res))
     return list(res)
 

@@ -132,6 +132,8 @@ typedef struct {
 #define AMOS_PIPE_STAGED 1    /* global -> registers -> LDS, any layout, ragged K             */
 #define AMOS_PIPE_DIRECT4 2   /* global -> LDS direct copies, 256x256 tile, 4 waves           */
 #define AMOS_PIPE_DIRECT8 3   /* same with 8 waves (two per SIMD)                             */
+#define AMOS_PIPE_PATCH 4     /* conv: input patch staged once per channel chunk, weights     */
+                              /* repacked into the workspace; needs amos_workspace_bytes()    */
 
 int amos_version(void);
 const char* amos_last_error(void);
@@ -146,6 +148,8 @@ int amos_default_config(int op, const void* desc, amos_kernel_config_t* out);
  * returns AMOS_ERR_INFEASIBLE when over budget */
 int amos_check_config(int op, const void* desc, const amos_kernel_config_t* cfg,
                       int64_t* lds_bytes, int64_t* acc_regs);
+/* bytes of device scratch the op's fastest pipeline wants (conv: repacked weights); calls
+ * that get less fall back to the register-staged pipeline, which needs none */
 size_t amos_workspace_bytes(int op, const void* desc, const amos_kernel_config_t* cfg);
 
 /* the runnable kernels: replace `func(A, B, C)` of the module tvm.build returns

@@ -67,7 +67,7 @@ def test_gemm_small(gpu, dtype, trans, shape):
     check_literal(got, lit, dtype, "gemm %s %s %s vs te_literal" % (dtype, trans, shape))
 
 
-TILES = [(64, 64), (128, 128), (256, 256), (128, 64), (64, 128), (256, 128), (128, 256)]
+TILES = [(64, 64), (128, 128), (256, 256), (128, 64), (64, 128), (256, 128), (128, 256), (256, 64), (64, 256)]
 
 
 @pytest.mark.parametrize("dtype", ["float16", "int8"])
@@ -221,6 +221,54 @@ def test_conv2d_every_tile(gpu, tile):
         cfg = dict(tile_i=tile[0], tile_j=tile[1], split_k=split)
         got = ops.conv2d(to_device(x, "int8"), to_device(w, "int8"), 1, 1, 1, config=cfg).cpu().numpy()
         check(got, co.lib_conv2d(x, w, "int8", 1, 1, 1), "int8", "conv2d tile %s split %d" % (tile, split))
+
+
+PATCH_CONV_CASES = [
+    # N, C, D, H, W, K, T, R, S, stride, pad, dil   (C * element size is a multiple of 128 bytes)
+    (2, 128, 1, 14, 14, 96, 1, 3, 3, (1, 1, 1), (0, 1, 1), (1, 1, 1)),
+    (5, 128, 1, 7, 7, 40, 1, 3, 3, (1, 1, 1), (0, 1, 1), (1, 1, 1)),     # tiles straddle images
+    (2, 256, 1, 9, 11, 64, 1, 3, 2, (1, 2, 1), (0, 1, 0), (1, 1, 2)),    # stride, dilation
+    (3, 128, 1, 8, 8, 130, 1, 1, 1, (1, 1, 1), (0, 0, 0), (1, 1, 1)),    # 1x1, ragged K tile
+    (1, 128, 1, 20, 20, 32, 1, 5, 5, (1, 1, 1), (0, 2, 2), (1, 1, 1)),
+    (1, 128, 1, 13, 13, 16, 1, 3, 3, (1, 2, 2), (0, 0, 0), (1, 1, 1)),   # valid conv, stride 2
+    (2, 128, 4, 6, 6, 24, 3, 3, 3, (1, 1, 1), (1, 1, 1), (1, 1, 1)),     # conv3d
+    (1, 128, 5, 5, 7, 48, 2, 3, 2, (2, 1, 1), (1, 0, 1), (2, 1, 1)),     # conv3d stride / dilation in depth
+]
+
+
+@pytest.mark.parametrize("dtype", ["float16", "bfloat16", "int8"])
+@pytest.mark.parametrize("case", PATCH_CONV_CASES)
+def test_conv_patch_pipeline(gpu, dtype, case):
+    """patch-staged convolution (pipeline 4): every tile shape, with and without split-K"""
+    from amos_amd import _lib, ops
+    N, C, D, H, W, K, T, R, S, st, pd, dl = case
+    rng = np.random.default_rng(hash(case) % 2**32)
+    x = make_operand(rng, (N, C, D, H, W), dtype, "normal")
+    w = make_operand(rng, (K, C, T, R, S), dtype, "normal")
+    ref = co.lib_conv3d(x, w, dtype, st, pd, dl, acc="float64")
+    dx, dw = to_device(x, dtype), to_device(w, dtype)
+    for tile in [(64, 64), (128, 64), (64, 128), (128, 128), (256, 64), (256, 128), (128, 256), (64, 256)]:
+        for split in (1, 2):
+            cfg = dict(tile_i=tile[0], tile_j=tile[1], split_k=split, pipeline=_lib.AMOS_PIPE_PATCH)
+            try:
+                if D == 1 and T == 1:
+                    got = ops.conv2d(dx[:, :, 0], dw[:, :, 0], st[1:], pd[1:], dl[1:], config=cfg)[:, :, None]
+                else:
+                    got = ops.conv3d(dx, dw, st, pd, dl, config=cfg)
+            except _lib.AmosError as e:
+                # a tile that spans too many slices or a patch too large: reported, never silent
+                assert e.code == _lib.AMOS_ERR_INFEASIBLE and "not applicable" in str(e)
+                continue
+            check(got.cpu().numpy(), ref, dtype, "patch conv %s %s tile %s split %d" % (dtype, case, tile, split))
+
+
+def test_conv_patch_is_the_default_when_applicable(gpu):
+    import torch
+    from amos_amd import _lib, ops
+    d = ops.conv_desc((32, 256, 1, 14, 14), (256, 256, 1, 3, 3), torch.float16, (1, 1, 1), (0, 1, 1), (1, 1, 1))
+    assert ops.kernel_name(_lib.AMOS_OP_CONV2D, d).startswith("amos_conv_fprop<f16,")
+    d = ops.conv_desc((2, 24, 1, 14, 14), (40, 24, 1, 3, 3), torch.float16, (1, 1, 1), (0, 1, 1), (1, 1, 1))
+    assert ops.kernel_name(_lib.AMOS_OP_CONV2D, d).startswith("amos_igemm<f16,")
 
 
 def test_conv2d_config3(gpu):
