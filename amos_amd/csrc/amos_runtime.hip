@@ -193,48 +193,6 @@ static int conv_out_extent(int64_t in, int pad, int dil, int64_t k, int stride) 
   return (int)o;
 }
 
-// worst case over the J tiles of the patch a block stages: LDS positions and slices touched
-static void conv_patch_extent(int64_t J, int OPQ, int OQ, int BJ, int sh, int R, int dh, int Wp,
-                              int* max_pos, int* max_seg) {
-  *max_pos = 0;
-  *max_seg = 0;
-  const int64_t tiles = (J + BJ - 1) / BJ;
-  // the pattern of (tile start mod OPQ) repeats after OPQ / gcd(BJ, OPQ) tiles
-  int64_t a = BJ, b = OPQ;
-  while (b) { int64_t r = a % b; a = b; b = r; }
-  int64_t period = OPQ / a + 1;
-  const int64_t scan = tiles < period ? tiles : period;
-  for (int64_t tj = 0; tj <= scan; ++tj) {
-    int64_t t2 = tj == scan ? tiles - 1 : tj;   // the ragged last tile too
-    int64_t j0 = t2 * BJ, j1 = j0 + BJ - 1 < J - 1 ? j0 + BJ - 1 : J - 1;
-    int64_t sa = j0 / OPQ, sb = j1 / OPQ;
-    int pos = 0;
-    for (int64_t sl = sa; sl <= sb; ++sl) {
-      int64_t lo = j0 > sl * OPQ ? j0 : sl * OPQ;
-      int64_t hi = j1 < (sl + 1) * OPQ - 1 ? j1 : (sl + 1) * OPQ - 1;
-      int pa = (int)((lo - sl * OPQ) / OQ), pb = (int)((hi - sl * OPQ) / OQ);
-      pos += ((pb - pa) * sh + (R - 1) * dh + 1) * Wp;
-    }
-    if (pos > *max_pos) *max_pos = pos;
-    if ((int)(sb - sa + 1) > *max_seg) *max_seg = (int)(sb - sa + 1);
-  }
-}
-
-// workspace of the patch-staged pipeline: [packed weights | 256 zero bytes | NDHWC activations]
-static int64_t conv_packed_bytes(const amos_conv_desc_t& c, int op) {
-  int64_t T = op == AMOS_OP_CONV2D ? 1 : c.T;
-  int es = c.in_dtype == AMOS_I8 ? 1 : 2;
-  if (c.C <= 0 || (c.C * es) % 128 != 0) return 0;
-  return (c.K * T * c.R * c.S * c.C * es + 255) / 256 * 256;
-}
-static int64_t conv_workspace_bytes(const amos_conv_desc_t& c, int op) {
-  int64_t packed = conv_packed_bytes(c, op);
-  if (packed == 0) return 0;
-  int64_t D = op == AMOS_OP_CONV2D ? 1 : c.D;
-  int es = c.in_dtype == AMOS_I8 ? 1 : 2;
-  return packed + 256 + c.N * c.C * D * c.H * c.W * es;
-}
-
 static int plan_conv(Plan& pl, int op, const amos_conv_desc_t* d, const amos_kernel_config_t* cfg,
                      const void* X, const void* Wt, void* Y, void* workspace, size_t ws_bytes) {
   if (!d || !X || !Wt || !Y) return set_error(AMOS_ERR_BAD_ARG, "null pointer argument");
@@ -299,53 +257,18 @@ static int plan_conv(Plan& pl, int op, const amos_conv_desc_t* d, const amos_ker
   // the workspace, the patch of a tile fits LDS next to a ring of weight tiles
   const int pipe = pl.cfg.pipeline;
   if (pipe == AMOS_PIPE_STAGED) return 0;
-  const char* why = nullptr;
+  const int BI = pl.cfg.tile_i, BJ = pl.cfg.tile_j;
   const int64_t packed = conv_packed_bytes(c, op);
   const int64_t need_ws = conv_workspace_bytes(c, op);
-  const int BI = pl.cfg.tile_i, BJ = pl.cfg.tile_j;
-  int max_pos = 0, max_seg = 0, nsw = 0, pls = 0;
-  size_t lds = 0;
   const int RS = (int)(c.R * c.S);
   const int Wp = (OQ - 1) * c.stride_w + ((int)c.S - 1) * c.dil_w + 1;
-  const bool tile_ok = (BI == 64 && (BJ == 64 || BJ == 128 || BJ == 256)) ||
-                       (BI == 128 && (BJ == 64 || BJ == 128 || BJ == 256)) ||
-                       (BI == 256 && (BJ == 64 || BJ == 128));
-  if (packed == 0) why = "C * element size is not a multiple of 128 bytes";
-  else if (packed >= ((int64_t)1 << 32)) why = "packed weights above 4 GiB";
-  else if (c.N * c.D * c.H * c.W >= ((int64_t)1 << 31) || J >= ((int64_t)1 << 31) - 512)
-    why = "more than 2^31 input or output positions";
-  else if (c.D + 2 * (int64_t)c.pad_d + c.T * c.dil_d >= 30000) why = "depth extent above 30000";
-  else if (!workspace || ws_bytes < (size_t)need_ws || ((uintptr_t)workspace & 255))
+  ConvPatchPlan pp = conv_patch_plan(c, op, BI, BJ, pl.cfg.split_k);
+  const char* why = pp.why;
+  if (!why && (!workspace || ws_bytes < (size_t)need_ws || ((uintptr_t)workspace & 255)))
     why = "workspace smaller than amos_workspace_bytes() or not 256-byte aligned";
-  else if (!tile_ok) why = "no patch-staged instance with this block tile";
-  if (!why) {
-    conv_patch_extent(J, OP * OQ, OQ, BJ, c.stride_h, (int)c.R, c.dil_h, Wp, &max_pos, &max_seg);
-    max_pos = (max_pos + 7) & ~7;
-    const size_t budget = (size_t)160 * 1024 - 512;
-    const size_t patch = (size_t)2 * max_pos * 128 + (size_t)max_pos * 8;
-    const size_t wstage = (size_t)BI * 128;
-    if (max_seg > kConvMaxSeg) why = "a tile spans more than 4 image slices";
-    else if (max_pos >= 4096) why = "input patch of a tile has 4096 or more positions";
-    else if (patch + 2 * wstage > budget) why = "input patch of a tile does not fit LDS";
-    else {
-      nsw = (int)((budget - patch) / wstage);
-      if (nsw > 8) nsw = 8;
-      if (nsw > RS + 1) nsw = RS + 1;
-      // The next patch is copied during the taps of the current one.  A copy issued on tap u
-      // is complete for everybody at the barrier of the patch's last tap only if u <= RS-2
-      // and it is older than the weight tiles still allowed in flight there: u <= RS+1-nsw.
-      int taps = RS + 2 - nsw < RS - 1 ? RS + 2 - nsw : RS - 1;
-      const int64_t macro_steps = c.T * (c.C * es / 128);
-      int split = pl.cfg.split_k < 1 ? 1 : pl.cfg.split_k;
-      const bool one_macro = (macro_steps + split - 1) / split <= 1;   // no next patch at all
-      if (taps < 1 && !one_macro) why = "1x1 window with several channel chunks per block";
-      if (taps < 1) taps = 1;
-      const int per_wave = ((max_pos / 8) + 3) / 4;
-      pls = (per_wave + taps - 1) / taps;
-      if (pls < 1) pls = 1;
-      lds = (size_t)nsw * wstage + patch;
-    }
-  }
+  const int max_pos = pp.max_pos, nsw = pp.nsw, pls = pp.pls;
+  const size_t lds = pp.lds;
+  (void)RS;
   if (why) {
     if (pipe == AMOS_PIPE_PATCH)
       return set_error(AMOS_ERR_INFEASIBLE, "patch-staged convolution not applicable: %s", why);

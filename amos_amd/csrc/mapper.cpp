@@ -69,6 +69,104 @@ int problem_of(int op, const void* desc, Problem* out) {
   return set_error(AMOS_ERR_BAD_ARG, "unknown op %d", op);
 }
 
+// worst case over the J tiles of the patch a block stages: LDS positions and slices touched
+static void conv_patch_extent(int64_t J, int OPQ, int OQ, int BJ, int sh, int R, int dh, int Wp,
+                              int* max_pos, int* max_seg) {
+  *max_pos = 0;
+  *max_seg = 0;
+  const int64_t tiles = (J + BJ - 1) / BJ;
+  // the pattern of (tile start mod OPQ) repeats after OPQ / gcd(BJ, OPQ) tiles
+  int64_t a = BJ, b = OPQ;
+  while (b) { int64_t r = a % b; a = b; b = r; }
+  int64_t period = OPQ / a + 1;
+  const int64_t scan = tiles < period ? tiles : period;
+  for (int64_t tj = 0; tj <= scan; ++tj) {
+    int64_t t2 = tj == scan ? tiles - 1 : tj;   // the ragged last tile too
+    int64_t j0 = t2 * BJ, j1 = j0 + BJ - 1 < J - 1 ? j0 + BJ - 1 : J - 1;
+    int64_t sa = j0 / OPQ, sb = j1 / OPQ;
+    int pos = 0;
+    for (int64_t sl = sa; sl <= sb; ++sl) {
+      int64_t lo = j0 > sl * OPQ ? j0 : sl * OPQ;
+      int64_t hi = j1 < (sl + 1) * OPQ - 1 ? j1 : (sl + 1) * OPQ - 1;
+      int pa = (int)((lo - sl * OPQ) / OQ), pb = (int)((hi - sl * OPQ) / OQ);
+      pos += ((pb - pa) * sh + (R - 1) * dh + 1) * Wp;
+    }
+    if (pos > *max_pos) *max_pos = pos;
+    if ((int)(sb - sa + 1) > *max_seg) *max_seg = (int)(sb - sa + 1);
+  }
+}
+
+// workspace of the patch-staged pipeline: [packed weights | 256 zero bytes | NDHWC activations]
+int64_t conv_packed_bytes(const amos_conv_desc_t& c, int op) {
+  int64_t T = op == AMOS_OP_CONV2D ? 1 : c.T;
+  int es = c.in_dtype == AMOS_I8 ? 1 : 2;
+  if (c.C <= 0 || (c.C * es) % 128 != 0) return 0;
+  return (c.K * T * c.R * c.S * c.C * es + 255) / 256 * 256;
+}
+int64_t conv_workspace_bytes(const amos_conv_desc_t& c, int op) {
+  int64_t packed = conv_packed_bytes(c, op);
+  if (packed == 0) return 0;
+  int64_t D = op == AMOS_OP_CONV2D ? 1 : c.D;
+  int es = c.in_dtype == AMOS_I8 ? 1 : 2;
+  return packed + 256 + c.N * c.C * D * c.H * c.W * es;
+}
+
+
+ConvPatchPlan conv_patch_plan(const amos_conv_desc_t& cin, int op, int BI, int BJ, int split_k) {
+  ConvPatchPlan pp = {nullptr, 0, 0, 0, 0, 0};
+  amos_conv_desc_t c = cin;
+  if (op == AMOS_OP_CONV2D) { c.D = 1; c.T = 1; c.stride_d = 1; c.pad_d = 0; c.dil_d = 1; }
+  const int es = c.in_dtype == AMOS_I8 ? 1 : 2;
+  const int64_t OD = conv_out(c.D, c.pad_d, c.dil_d, c.T, c.stride_d);
+  const int64_t OP = conv_out(c.H, c.pad_h, c.dil_h, c.R, c.stride_h);
+  const int64_t OQ = conv_out(c.W, c.pad_w, c.dil_w, c.S, c.stride_w);
+  const int64_t J = c.N * OD * OP * OQ;
+  const int64_t packed = conv_packed_bytes(c, op);
+  const int RS = (int)(c.R * c.S);
+  const int Wp = (int)((OQ - 1) * c.stride_w + (c.S - 1) * c.dil_w + 1);
+  const bool tile_ok = (BI == 64 && (BJ == 64 || BJ == 128 || BJ == 256)) ||
+                       (BI == 128 && (BJ == 64 || BJ == 128 || BJ == 256)) ||
+                       (BI == 256 && (BJ == 64 || BJ == 128));
+  if (OD <= 0 || OP <= 0 || OQ <= 0) { pp.why = "empty output"; return pp; }
+  if (packed == 0) { pp.why = "C * element size is not a multiple of 128 bytes"; return pp; }
+  if (packed >= ((int64_t)1 << 32)) { pp.why = "packed weights above 4 GiB"; return pp; }
+  if (c.N * c.D * c.H * c.W >= ((int64_t)1 << 31) || J >= ((int64_t)1 << 31) - 512) {
+    pp.why = "more than 2^31 input or output positions";
+    return pp;
+  }
+  if (c.D + 2 * (int64_t)c.pad_d + c.T * c.dil_d >= 30000) { pp.why = "depth extent above 30000"; return pp; }
+  if (!tile_ok) { pp.why = "no patch-staged instance with this block tile"; return pp; }
+  int max_pos = 0, max_seg = 0;
+  conv_patch_extent(J, (int)(OP * OQ), (int)OQ, BJ, c.stride_h, (int)c.R, c.dil_h, Wp, &max_pos, &max_seg);
+  max_pos = (max_pos + 7) & ~7;
+  const size_t budget = (size_t)160 * 1024 - 512;
+  const size_t patch = (size_t)2 * max_pos * 128 + (size_t)max_pos * 8;
+  const size_t wstage = (size_t)BI * 128;
+  pp.max_pos = max_pos;
+  pp.max_seg = max_seg;
+  if (max_seg > kConvMaxSegHost) { pp.why = "a tile spans more than 4 image slices"; return pp; }
+  if (max_pos >= 4096) { pp.why = "input patch of a tile has 4096 or more positions"; return pp; }
+  if (patch + 2 * wstage > budget) { pp.why = "input patch of a tile does not fit LDS"; return pp; }
+  int nsw = (int)((budget - patch) / wstage);
+  if (nsw > 8) nsw = 8;
+  if (nsw > RS + 1) nsw = RS + 1;
+  // The next patch is copied during the taps of the current one.  A copy issued on tap u is
+  // complete for everybody at the barrier of the patch's last tap only if u <= RS-2 and it is
+  // older than the weight tiles still allowed in flight there: u <= RS+1-nsw.
+  int taps = RS + 2 - nsw < RS - 1 ? RS + 2 - nsw : RS - 1;
+  const int64_t macro_steps = c.T * (c.C * es / 128);
+  const int split = split_k < 1 ? 1 : split_k;
+  const bool one_macro = (macro_steps + split - 1) / split <= 1;   // no next patch at all
+  if (taps < 1 && !one_macro) { pp.why = "1x1 window with several channel chunks per block"; return pp; }
+  if (taps < 1) taps = 1;
+  const int per_wave = ((max_pos / 8) + 3) / 4;
+  pp.pls = (per_wave + taps - 1) / taps;
+  if (pp.pls < 1) pp.pls = 1;
+  pp.nsw = nsw;
+  pp.lds = (size_t)nsw * wstage + patch;
+  return pp;
+}
+
 static const int kTiles[][2] = {{256, 256}, {256, 128}, {128, 256}, {128, 128},
                                 {256, 64},  {128, 64},  {64, 128},  {64, 64},   {64, 256}};
 
@@ -144,6 +242,33 @@ int amos_default_config(int op, const void* desc, amos_kernel_config_t* out) {
   const double es = pb.in_dtype == AMOS_I8 ? 1.0 : 2.0;
   const int k_tiles = (int)std::ceil((double)pb.K / (128.0 / es));
   double best = 1e30;
+  if (op == AMOS_OP_CONV2D || op == AMOS_OP_CONV3D) {
+    // patch-staged pipeline where it applies: blocks of one per CU, a K step costs its MFMA
+    // issue time plus a per-step instruction overhead that does not shrink with the tile;
+    // split-K pays for atomic accumulation into the output
+    const amos_conv_desc_t& c = *(const amos_conv_desc_t*)desc;
+    const int64_t T = op == AMOS_OP_CONV2D ? 1 : c.T;
+    const double steps_all = (double)T * c.R * c.S * std::ceil(c.C * es / 128.0);
+    for (auto& t : kTiles) {
+      for (int split = 1; split <= 4; split *= 2) {
+        ConvPatchPlan pp = conv_patch_plan(c, op, t[0], t[1], split);
+        if (pp.why) continue;
+        const double blocks = std::ceil((double)pb.I / t[0]) * std::ceil((double)pb.J / t[1]) * split;
+        const double rounds = std::ceil(blocks / Gfx950::kComputeUnits);
+        const double steps = std::ceil(steps_all / split);
+        const double mfma_per_step = (t[0] / 64.0) * (t[1] / 64.0) * 4.0 * 32.0;
+        const double cycles = rounds * (steps * (mfma_per_step + 600.0) + 4000.0);
+        double s = cycles / (2.1e9) + (split > 1 ? (double)pb.out_bytes * split / 1.2e12 : 0.0);
+        if (s < best * 0.98) {
+          best = s;
+          out->tile_i = t[0];
+          out->tile_j = t[1];
+          out->split_k = split;
+        }
+      }
+    }
+    if (best < 1e30) return 0;
+  }
   for (auto& t : kTiles) {
     for (int split = 1; split <= 16; split *= 2) {
       if (split > 1 && (split > k_tiles / 4 || pb.batch > 1)) break;
