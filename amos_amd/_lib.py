@@ -52,6 +52,13 @@ class KernelConfig(ctypes.Structure):
                 ("reserved", _i32 * 4)]
 
 
+class ComputeC(ctypes.Structure):
+    _fields_ = [("n_tokens", _i32), ("tokens", ctypes.POINTER(_i32)), ("n_iters", _i32),
+                ("iter_kinds", ctypes.POINTER(_i32)), ("iter_extents", ctypes.POINTER(_i64)),
+                ("n_loads", _i32), ("load_ndim", ctypes.POINTER(_i32)),
+                ("coeffs", ctypes.POINTER(_i64))]
+
+
 class AmosError(RuntimeError):
     """A C-ABI call returned a negative code; `.code` holds it."""
 
@@ -63,8 +70,8 @@ class AmosError(RuntimeError):
 # every symbol include/amos_mi355x.h declares
 EXPORTS = [
     "amos_version", "amos_last_error", "amos_device_info", "amos_default_config",
-    "amos_check_config", "amos_workspace_bytes", "amos_gemm", "amos_bgemm", "amos_conv2d",
-    "amos_conv3d", "amos_time", "amos_kernel_name",
+    "amos_check_config", "amos_workspace_bytes", "amos_estimate_seconds", "amos_gemm", "amos_bgemm", "amos_conv2d",
+    "amos_conv3d", "amos_time", "amos_kernel_name", "amos_match", "amos_enumerate_mappings",
 ]
 
 _lib = None
@@ -88,6 +95,8 @@ def load():
                                       ctypes.POINTER(_i64), ctypes.POINTER(_i64)]
     lib.amos_workspace_bytes.argtypes = [ctypes.c_int, vp, ctypes.POINTER(KernelConfig)]
     lib.amos_workspace_bytes.restype = sz
+    lib.amos_estimate_seconds.argtypes = [ctypes.c_int, vp, ctypes.POINTER(KernelConfig),
+                                          ctypes.POINTER(ctypes.c_double)]
     for name, desc in (("amos_gemm", GemmDesc), ("amos_bgemm", BGemmDesc), ("amos_conv2d", ConvDesc),
                        ("amos_conv3d", ConvDesc)):
         fn = getattr(lib, name)
@@ -98,6 +107,11 @@ def load():
                               ctypes.POINTER(ctypes.c_double)]
     lib.amos_kernel_name.argtypes = [ctypes.c_int, vp, ctypes.POINTER(KernelConfig)]
     lib.amos_kernel_name.restype = ctypes.c_char_p
+    lib.amos_match.argtypes = [ctypes.POINTER(ComputeC), ctypes.POINTER(ComputeC),
+                               ctypes.POINTER(_i32), _i32]
+    lib.amos_enumerate_mappings.argtypes = [_i32, _i32, ctypes.POINTER(_i32), ctypes.POINTER(_i64),
+                                            ctypes.POINTER(_i64), ctypes.POINTER(ctypes.c_uint8),
+                                            ctypes.POINTER(ctypes.c_uint8), _i32]
     _lib = lib
     return lib
 

@@ -1,0 +1,256 @@
+"""From a matched TE compute to an operator descriptor of the C ABI.
+
+The reference lowers the mapped compute through TVM's schedule, TIR passes and CUDA code
+generator (python/tvm/auto_tensorize/tensorization_phases/schedulers/cuda_v2.py:398-854,
+src/target/source/codegen_c.cc:733-772).  Here the kernels exist already; lowering means
+recognising which of them a compute is -- GEMM (any of the four operand transpositions),
+batched GEMM, NCHW conv2d or NCDHW conv3d with their padding stage -- and reading strides,
+dilations, paddings and layouts off the affine index expressions.  A compute that matches
+an intrinsic but has no kernel raises NoKernelError; nothing falls back to another device.
+"""
+from .. import _lib, te
+
+
+class NoKernelError(RuntimeError):
+    pass
+
+
+class LoweredOp(object):
+    """kind: 'gemm' | 'bgemm' | 'conv2d' | 'conv3d'; `inputs` are the two placeholder tensors
+    in kernel argument order (row/A operand first for GEMM, activations first for conv);
+    `output` the result tensor."""
+
+    def __init__(self, kind, op_code, desc, inputs, output, attrs):
+        self.kind = kind
+        self.op_code = op_code
+        self.desc = desc
+        self.inputs = inputs
+        self.output = output
+        self.attrs = attrs
+
+    def flops(self):
+        a = self.attrs
+        if self.kind in ("gemm", "bgemm"):
+            return 2.0 * a.get("batch", 1) * a["M"] * a["N"] * a["K"]
+        return 2.0 * a["J"] * a["K_out"] * a["K_red"]
+
+    def __str__(self):
+        return "%s %s" % (self.kind, {k: v for k, v in self.attrs.items()})
+
+
+def _single_var(form, iters):
+    """affine form that is exactly one iteration variable (coefficient 1, constant 0)"""
+    if form is None:
+        return None
+    coef, const = form
+    if const != 0 or len(coef) != 1:
+        return None
+    (v, c), = coef.items()
+    if c != 1:
+        return None
+    for iv in iters:
+        if iv.var is v:
+            return iv
+    return None
+
+
+def _strip_cast(e):
+    while isinstance(e, te.Cast):
+        e = e.value
+    return e
+
+
+def _product_loads(main_op):
+    body = main_op.body[0]
+    if not isinstance(body, te.Reduce):
+        raise NoKernelError("main op is not a sum reduction")
+    src = _strip_cast(body.source)
+    if not isinstance(src, te.Mul):
+        raise NoKernelError("reduction source is not a product")
+    l0, l1 = _strip_cast(src.a), _strip_cast(src.b)
+    if not (isinstance(l0, te.ProducerLoad) and isinstance(l1, te.ProducerLoad)):
+        raise NoKernelError("product operands are not tensor loads")
+    return l0, l1
+
+
+_DT = {"float16": _lib.AMOS_F16, "bfloat16": _lib.AMOS_BF16, "int8": _lib.AMOS_I8,
+       "float32": _lib.AMOS_F32, "int32": _lib.AMOS_I32}
+
+
+def _dtype_pair(l0, l1, out):
+    if l0.dtype != l1.dtype or (l0.dtype, out.dtype) not in (("float16", "float32"), ("bfloat16", "float32"),
+                                                            ("int8", "int32")):
+        raise NoKernelError("no kernel for dtypes %s x %s -> %s" % (l0.dtype, l1.dtype, out.dtype))
+    return _DT[l0.dtype], _DT[out.dtype]
+
+
+def _lower_gemm(main_op, l0, l1, iters, forms0, forms1):
+    spatial, reduce_ = list(main_op.axis), list(main_op.reduce_axis)
+    if len(reduce_) != 1 or len(spatial) not in (2, 3):
+        return None
+    k = reduce_[0]
+    v0 = [_single_var(f, iters) for f in forms0]
+    v1 = [_single_var(f, iters) for f in forms1]
+    if any(v is None for v in v0 + v1) or len(v0) != len(spatial) or len(v1) != len(spatial):
+        return None
+    batch = spatial[0] if len(spatial) == 3 else None
+    x, y = spatial[-2], spatial[-1]
+    if batch is not None and (v0[0] is not batch or v1[0] is not batch):
+        return None
+    d0, d1 = v0[-2:], v1[-2:]
+
+    def has(d, iv):
+        return any(e is iv for e in d)
+
+    if has(d0, x) and has(d1, y) and not has(d0, y) and not has(d1, x):
+        la, lb, da, db = l0, l1, d0, d1
+    elif has(d1, x) and has(d0, y) and not has(d1, y) and not has(d0, x):
+        la, lb, da, db = l1, l0, d1, d0
+    else:
+        return None
+    if not (has(da, k) and has(db, k)):
+        return None
+    if not (isinstance(la.tensor.op, te.PlaceholderOp) and isinstance(lb.tensor.op, te.PlaceholderOp)):
+        raise NoKernelError("GEMM operands must be placeholders")
+    trans_a = 0 if da[0] is x else 1          # [x, k] row-major A, [k, x] transposed
+    trans_b = 0 if db[0] is k else 1          # [k, y] row-major B, [y, k] column-major B
+    M, N, K = int(x.dom.extent), int(y.dom.extent), int(k.dom.extent)
+    ind, outd = _dtype_pair(la, lb, main_op.output(0))
+    g = _lib.GemmDesc()
+    g.M, g.N, g.K, g.in_dtype, g.out_dtype, g.trans_a, g.trans_b = M, N, K, ind, outd, trans_a, trans_b
+    g.lda, g.ldb, g.ldc = (M if trans_a else K), (K if trans_b else N), N
+    attrs = dict(M=M, N=N, K=K, trans_a=trans_a, trans_b=trans_b, dtype=la.dtype)
+    if batch is None:
+        return LoweredOp("gemm", _lib.AMOS_OP_GEMM, g, [la.tensor, lb.tensor], main_op.output(0), attrs)
+    b = _lib.BGemmDesc()
+    b.batch = int(batch.dom.extent)
+    b.g = g
+    b.stride_a, b.stride_b, b.stride_c = M * K, K * N, M * N
+    attrs["batch"] = b.batch
+    return LoweredOp("bgemm", _lib.AMOS_OP_BGEMM, b, [la.tensor, lb.tensor], main_op.output(0), attrs)
+
+
+def _pad_stage(tensor):
+    """tensor made by the padding compute -> (source placeholder, pads per spatial dim)"""
+    op = tensor.op
+    if isinstance(op, te.PlaceholderOp):
+        return tensor, [0] * (len(tensor.shape) - 2)
+    if not isinstance(op, te.ComputeOp) or op.reduce_axis:
+        raise NoKernelError("activation operand is neither a placeholder nor a padding stage")
+    body = op.body[0]
+    if not isinstance(body, te.Select) or not isinstance(_strip_cast(body.then_value), te.ProducerLoad):
+        raise NoKernelError("unrecognised stage %s in front of the convolution" % op.name)
+    zero = body.else_value
+    if not isinstance(zero, (te.IntImm, te.FloatImm)) or zero.value != 0:
+        raise NoKernelError("padding value is not zero")
+    load = _strip_cast(body.then_value)
+    src = load.tensor
+    if not isinstance(src.op, te.PlaceholderOp):
+        raise NoKernelError("padding stage does not read a placeholder")
+    variables = [iv.var for iv in op.axis]
+    pads = []
+    for d, idx in enumerate(load.indices):
+        form = te.affine_form(idx, variables)
+        if form is None or len(form[0]) != 1 or list(form[0].items())[0] != (variables[d], 1):
+            raise NoKernelError("padding stage permutes or scales indices")
+        pad = -form[1]
+        if d < 2:
+            if pad != 0:
+                raise NoKernelError("padding on the batch or channel dimension")
+        else:
+            if pad < 0 or int(op.output(0).shape[d]) != int(src.shape[d]) + 2 * pad:
+                raise NoKernelError("padding stage is not symmetric zero padding")
+            pads.append(pad)
+    return src, pads
+
+
+def _lower_conv(main_op, l0, l1, iters, forms0, forms1):
+    spatial, reduce_ = list(main_op.axis), list(main_op.reduce_axis)
+    nsp = len(spatial) - 2                     # 2 or 3 spatial output dims
+    if nsp not in (2, 3) or len(reduce_) != nsp + 1:
+        return None
+    n_iv, k_iv, out_sp = spatial[0], spatial[1], spatial[2:]
+    rc, red_sp = reduce_[0], reduce_[1:]
+
+    def try_roles(lx, fx, lw, fw):
+        if len(fx) != nsp + 2 or len(fw) != nsp + 2:
+            return None
+        wv = [_single_var(f, iters) for f in fw]
+        if wv[0] is not k_iv or wv[1] is not rc or any(a is not b for a, b in zip(wv[2:], red_sp)):
+            return None
+        if _single_var(fx[0], iters) is not n_iv or _single_var(fx[1], iters) is not rc:
+            return None
+        strides, dils = [], []
+        for d in range(nsp):
+            f = fx[2 + d]
+            if f is None:
+                return None
+            coef, const = f
+            if const != 0 or set(coef.keys()) != {out_sp[d].var, red_sp[d].var}:
+                # a 1-wide window has a reduce axis of extent 1 that may be folded away
+                if const != 0 or set(coef.keys()) - {out_sp[d].var, red_sp[d].var}:
+                    return None
+            strides.append(int(coef.get(out_sp[d].var, 1)))
+            dils.append(int(coef.get(red_sp[d].var, 1)))
+            if strides[-1] < 1 or dils[-1] < 1:
+                return None
+        return strides, dils
+
+    roles = try_roles(l0, forms0, l1, forms1)
+    lx, lw = l0, l1
+    if roles is None:
+        roles = try_roles(l1, forms1, l0, forms0)
+        lx, lw = l1, l0
+    if roles is None:
+        return None
+    strides, dils = roles
+    src, pads = _pad_stage(lx.tensor)
+    if not isinstance(lw.tensor.op, te.PlaceholderOp):
+        raise NoKernelError("convolution weights must be a placeholder")
+    xs, ws = [int(s) for s in src.shape], [int(s) for s in lw.tensor.shape]
+    for d in range(nsp):
+        if int(red_sp[d].dom.extent) != ws[2 + d]:
+            raise NoKernelError("reduce extent %d differs from the kernel window %d"
+                                % (int(red_sp[d].dom.extent), ws[2 + d]))
+        want = (xs[2 + d] + 2 * pads[d] - ((ws[2 + d] - 1) * dils[d] + 1)) // strides[d] + 1
+        if int(out_sp[d].dom.extent) != want:
+            raise NoKernelError("output extent %d is not what stride / padding / dilation give (%d)"
+                                % (int(out_sp[d].dom.extent), want))
+    if xs[1] != ws[1] or int(rc.dom.extent) != xs[1]:
+        raise NoKernelError("grouped convolution has no kernel")
+    ind, outd = _dtype_pair(lx, lw, main_op.output(0))
+    c = _lib.ConvDesc()
+    if nsp == 2:
+        xs5, ws5 = [xs[0], xs[1], 1, xs[2], xs[3]], [ws[0], ws[1], 1, ws[2], ws[3]]
+        st, pd, dl = [1] + strides, [0] + pads, [1] + dils
+    else:
+        xs5, ws5, st, pd, dl = xs, ws, strides, pads, dils
+    c.N, c.C, c.D, c.H, c.W = xs5
+    c.K, _, c.T, c.R, c.S = ws5
+    c.stride_d, c.stride_h, c.stride_w = st
+    c.pad_d, c.pad_h, c.pad_w = pd
+    c.dil_d, c.dil_h, c.dil_w = dl
+    c.in_dtype, c.out_dtype = ind, outd
+    out_shape = [int(s) for s in main_op.output(0).shape]
+    J = out_shape[0]
+    for e in out_shape[2:]:
+        J *= e
+    attrs = dict(x_shape=xs, w_shape=ws, stride=strides, pad=pads, dil=dils, dtype=lx.dtype, J=J,
+                 K_out=ws[0], K_red=ws[1] * (ws5[2] * ws5[3] * ws5[4]))
+    kind, code = ("conv2d", _lib.AMOS_OP_CONV2D) if nsp == 2 else ("conv3d", _lib.AMOS_OP_CONV3D)
+    return LoweredOp(kind, code, c, [src, lw.tensor], main_op.output(0), attrs)
+
+
+def lower_main_op(main_op):
+    """ComputeOp that matched a GEMM-like intrinsic -> LoweredOp"""
+    l0, l1 = _product_loads(main_op)
+    iters = list(main_op.axis) + list(main_op.reduce_axis)
+    variables = [iv.var for iv in iters]
+    forms0 = [te.affine_form(i, variables) for i in l0.indices]
+    forms1 = [te.affine_form(i, variables) for i in l1.indices]
+    for fn in (_lower_gemm, _lower_conv):
+        low = fn(main_op, l0, l1, iters, forms0, forms1)
+        if low is not None:
+            return low
+    raise NoKernelError("access pattern of %s is neither GEMM, batched GEMM, NCHW conv2d nor NCDHW conv3d"
+                        % main_op.name)

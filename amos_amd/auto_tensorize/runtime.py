@@ -1,0 +1,141 @@
+"""The runnable module: what `build(sch, args, target)` returns.
+
+Stands where tvm.build + tvm.runtime.Module stand in the reference
+(python/tvm/auto_tensorize/auto_tensorize.py:294-301, src/runtime/cuda/cuda_module.cc:105-172):
+`func(*arrays)` takes the arrays in `inputs + outputs` order, launches on the current
+stream and returns without synchronising; `time_evaluator` follows
+src/runtime/rpc/rpc_module.cc:341-399.  Arrays are device tensors; there is no host path.
+"""
+import numpy as np
+import torch
+
+from .. import ops
+from .measure import _TORCH_DTYPE
+
+
+class NDArray(object):
+    """device array with the asnumpy() / shape / dtype face of tvm.nd.NDArray"""
+
+    def __init__(self, tensor, dtype_name):
+        self.tensor = tensor
+        self.dtype = dtype_name
+
+    @property
+    def shape(self): return tuple(self.tensor.shape)
+
+    def asnumpy(self):
+        t = self.tensor
+        if t.dtype == torch.bfloat16:
+            return t.float().cpu().numpy()
+        return t.cpu().numpy()
+
+    numpy = asnumpy
+
+
+class Context(object):
+    def __init__(self, target, dev_id=0):
+        self.target, self.dev_id = target, dev_id
+        self.device = torch.device("cuda", dev_id)
+
+    def sync(self):
+        torch.cuda.synchronize(self.device)
+
+
+def context(target="hip", dev_id=0):
+    return Context(target, dev_id)
+
+
+def array(np_array, ctx=None, dtype=None):
+    """host numpy array -> device array; dtype names 'float16', 'bfloat16', 'int8', 'float32', 'int32'"""
+    if not torch.cuda.is_available():
+        raise RuntimeError("device arrays need a GPU: no HIP device is visible")
+    dev = ctx.device if ctx is not None else torch.device("cuda", 0)
+    name = dtype or str(np_array.dtype)
+    if name == "bfloat16":
+        t = torch.from_numpy(np.ascontiguousarray(np_array, dtype=np.float32)).to(dev).to(torch.bfloat16)
+    else:
+        t = torch.from_numpy(np.ascontiguousarray(np_array)).to(dev)
+        if name in _TORCH_DTYPE and t.dtype != _TORCH_DTYPE[name]:
+            t = t.to(_TORCH_DTYPE[name])
+    return NDArray(t, name)
+
+
+class _Source(object):
+    def __init__(self, mod): self.mod = mod
+
+    def get_source(self):
+        return self.mod.get_source()
+
+
+class TimeResult(object):
+    def __init__(self, results):
+        self.results = list(results)
+        self.mean = sum(results) / len(results)
+
+
+class Module(object):
+    entry_name = "default_function"
+
+    def __init__(self, lowered, params, arg_tensors):
+        self.lowered = lowered
+        self.params = params
+        # positions of (in0, in1, out) among the caller's arguments
+        ids = [id(t) for t in arg_tensors]
+        try:
+            self.arg_index = [ids.index(id(lowered.inputs[0])), ids.index(id(lowered.inputs[1])),
+                              ids.index(id(lowered.output))]
+        except ValueError:
+            raise ValueError("build() args must hold the compute's two inputs and its output tensor")
+        self.imported_modules = [_Source(self)]
+
+    def _pick(self, arrays):
+        if len(arrays) <= max(self.arg_index):
+            raise ValueError("expected %d arrays (inputs + outputs)" % (max(self.arg_index) + 1))
+        out = []
+        for i in self.arg_index:
+            a = arrays[i]
+            out.append(a.tensor if isinstance(a, NDArray) else a)
+        return out
+
+    def _run(self, in0, in1, out):
+        low, cfg = self.lowered, self.params.to_config() if self.params is not None else None
+        a = low.attrs
+        if low.kind == "gemm":
+            ops.gemm(in0, in1, a["trans_a"], a["trans_b"], out=out, config=cfg)
+        elif low.kind == "bgemm":
+            ops.bgemm(in0, in1, a["trans_a"], a["trans_b"], out=out, config=cfg)
+        elif low.kind == "conv2d":
+            ops.conv2d(in0, in1, a["stride"], a["pad"], a["dil"], out=out, config=cfg)
+        else:
+            ops.conv3d(in0, in1, a["stride"], a["pad"], a["dil"], out=out, config=cfg)
+
+    def __call__(self, *arrays):
+        self._run(*self._pick(arrays))
+
+    def time_evaluator(self, func_name=None, ctx=None, number=10, repeat=1, min_repeat_ms=0):
+        def evaluator(*arrays):
+            in0, in1, out = self._pick(arrays)
+            cfg = self.params.to_config() if self.params is not None else None
+            return TimeResult(ops.time_op(self.lowered.op_code, self.lowered.desc, in0, in1, out, config=cfg,
+                                          number=number, repeat=repeat, min_repeat_ms=min_repeat_ms))
+        return evaluator
+
+    def get_source(self):
+        """what was chosen: the kernel instance and its configuration (the kernels are
+        hand-written HIP in libamos_mi355x.so, not generated text)"""
+        cfg = self.params.to_config() if self.params is not None else None
+        name = ops.kernel_name(self.lowered.op_code, self.lowered.desc, cfg)
+        return "// %s\n// %s\n// config: %s\n" % (name, self.lowered, self.params)
+
+
+def build(sch, args, target="hip", target_host=None, name="default_function"):
+    """schedule (with a kernel config applied by a ScheduleApplier) -> runnable Module"""
+    lowered = getattr(sch, "lowered", None)
+    if lowered is None:
+        from .lowering import lower_main_op
+        from .. import te
+        mains = [op for op in sch.outputs if isinstance(op, te.ComputeOp) and op.reduce_axis]
+        if not mains:
+            raise ValueError("nothing to build: apply a schedule from auto_tensorize first")
+        lowered = lower_main_op(mains[0])
+    return Module(lowered, getattr(sch, "kernel_config", None), list(args))

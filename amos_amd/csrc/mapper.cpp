@@ -200,6 +200,25 @@ static double estimate_seconds(const Problem& pb, int ti, int tj, int split) {
   return std::max(t_mfma, t_hbm) + 2e-6;
 }
 
+// Patch-staged convolution: blocks of one per CU; a K step costs its MFMA issue time plus a
+// per-step instruction overhead that does not shrink with the tile; split-K pays for atomic
+// accumulation into the output.  Returns <= 0 where the pipeline does not apply.
+static double conv_patch_estimate(const amos_conv_desc_t& c, int op, const Problem& pb, int ti, int tj,
+                                  int split) {
+  ConvPatchPlan pp = conv_patch_plan(c, op, ti, tj, split);
+  if (pp.why) return -1.0;
+  const double es = pb.in_dtype == AMOS_I8 ? 1.0 : 2.0;
+  const int64_t T = op == AMOS_OP_CONV2D ? 1 : c.T;
+  const double steps_all = (double)T * c.R * c.S * std::ceil(c.C * es / 128.0);
+  const double blocks = std::ceil((double)pb.I / ti) * std::ceil((double)pb.J / tj) * split;
+  const double rounds = std::ceil(blocks / Gfx950::kComputeUnits);
+  const double steps = std::ceil(steps_all / split);
+  const double mfma_per_step = (ti / 64.0) * (tj / 64.0) * 4.0 * 32.0;
+  const double cycles = rounds * (steps * (mfma_per_step + 600.0) + 4000.0);
+  const double relayout = ((double)pb.in_bytes * 2.0) / 2.5e12 + 3e-6;
+  return cycles / 2.1e9 + relayout + (split > 1 ? (double)pb.out_bytes * split / 1.2e12 : 0.0);
+}
+
 }  // namespace amos
 
 using namespace amos;
@@ -233,6 +252,22 @@ int amos_check_config(int op, const void* desc, const amos_kernel_config_t* cfg,
   return 0;
 }
 
+int amos_estimate_seconds(int op, const void* desc, const amos_kernel_config_t* cfg, double* seconds) {
+  Problem pb;
+  int rc = problem_of(op, desc, &pb);
+  if (rc) return rc;
+  if (!cfg || !seconds) return set_error(AMOS_ERR_BAD_ARG, "null pointer argument");
+  rc = amos_check_config(op, desc, cfg, nullptr, nullptr);
+  if (rc) return rc;
+  const int split = cfg->split_k < 1 ? 1 : cfg->split_k;
+  if ((op == AMOS_OP_CONV2D || op == AMOS_OP_CONV3D) && cfg->pipeline != AMOS_PIPE_STAGED) {
+    double s = conv_patch_estimate(*(const amos_conv_desc_t*)desc, op, pb, cfg->tile_i, cfg->tile_j, split);
+    if (s > 0) { *seconds = s; return 0; }
+  }
+  *seconds = estimate_seconds(pb, cfg->tile_i, cfg->tile_j, split);
+  return 0;
+}
+
 int amos_default_config(int op, const void* desc, amos_kernel_config_t* out) {
   Problem pb;
   int rc = problem_of(op, desc, &pb);
@@ -247,19 +282,10 @@ int amos_default_config(int op, const void* desc, amos_kernel_config_t* out) {
     // issue time plus a per-step instruction overhead that does not shrink with the tile;
     // split-K pays for atomic accumulation into the output
     const amos_conv_desc_t& c = *(const amos_conv_desc_t*)desc;
-    const int64_t T = op == AMOS_OP_CONV2D ? 1 : c.T;
-    const double steps_all = (double)T * c.R * c.S * std::ceil(c.C * es / 128.0);
     for (auto& t : kTiles) {
       for (int split = 1; split <= 4; split *= 2) {
-        ConvPatchPlan pp = conv_patch_plan(c, op, t[0], t[1], split);
-        if (pp.why) continue;
-        const double blocks = std::ceil((double)pb.I / t[0]) * std::ceil((double)pb.J / t[1]) * split;
-        const double rounds = std::ceil(blocks / Gfx950::kComputeUnits);
-        const double steps = std::ceil(steps_all / split);
-        const double mfma_per_step = (t[0] / 64.0) * (t[1] / 64.0) * 4.0 * 32.0;
-        const double cycles = rounds * (steps * (mfma_per_step + 600.0) + 4000.0);
-        double s = cycles / (2.1e9) + (split > 1 ? (double)pb.out_bytes * split / 1.2e12 : 0.0);
-        if (s < best * 0.98) {
+        const double s = conv_patch_estimate(c, op, pb, t[0], t[1], split);
+        if (s > 0 && s < best * 0.98) {
           best = s;
           out->tile_i = t[0];
           out->tile_j = t[1];

@@ -151,6 +151,11 @@ int amos_check_config(int op, const void* desc, const amos_kernel_config_t* cfg,
 /* bytes of device scratch the op's fastest pipeline wants (conv: repacked weights); calls
  * that get less fall back to the register-staged pipeline, which needs none */
 size_t amos_workspace_bytes(int op, const void* desc, const amos_kernel_config_t* cfg);
+/* the mapper's analytical estimate (seconds per launch) for a config: wave quantisation of the
+ * grid over the CUs against MFMA issue time, HBM time for the algorithmic bytes, a launch floor
+ * (stands where the reference ranks candidates with its analytical model,
+ *  python/tvm/auto_tensorize/backend/tenet_integrate.py:168-202) */
+int amos_estimate_seconds(int op, const void* desc, const amos_kernel_config_t* cfg, double* seconds);
 
 /* the runnable kernels: replace `func(A, B, C)` of the module tvm.build returns
  * (reference: python/tvm/auto_tensorize/auto_tensorize.py:294-301,
@@ -179,6 +184,58 @@ int amos_time(int op, const void* desc, const amos_kernel_config_t* cfg, const v
  * "amos_igemm<f16,vec,vec,256x256>"; replaces func.imported_modules[0].get_source()
  * as the way to see what was chosen (reference: README.md:340). */
 const char* amos_kernel_name(int op, const void* desc, const amos_kernel_config_t* cfg);
+
+/* ---- the mapper: which loops of a compute can sit on the intrinsic's axes ------------------ */
+
+/*
+ * A compute as the matcher sees it: the structure of its body and, for every tensor
+ * load in it, the index expressions in affine form over the compute's iteration
+ * variables (spatial ones first, then reduce).
+ *   tokens      the body in prefix order, one per node: (kind << 8) | dtype code, with
+ *               kind 1 reduce, 2 cast, 3 mul, 4 add, 5 sub, 6 load, 7 select, 8 constant,
+ *               9 anything else; index expressions are not part of the token stream
+ *   iter_kinds  0 = spatial, 2 = reduce (TVM's IterVarType numbering)
+ *   load_ndim   dimensions of each load, in token order
+ *   coeffs      for every load and every dimension a row of n_iters + 2 values:
+ *               the n_iters coefficients, the constant term, and 1 if the index is affine
+ *               (0 = opaque: no variable that occurs in it can be mapped)
+ */
+typedef struct {
+  int32_t n_tokens;
+  const int32_t* tokens;
+  int32_t n_iters;
+  const int32_t* iter_kinds;
+  const int64_t* iter_extents;
+  int32_t n_loads;
+  const int32_t* load_ndim;
+  const int64_t* coeffs;
+} amos_compute_t;
+
+/*
+ * Match points of `target` against the intrinsic `intrin`: every injective assignment of
+ * the intrinsic's iteration variables to target variables of the same kind such that, load
+ * by load, each intrinsic index equals a distinct target index dimension up to a positive
+ * factor and a constant once unmapped variables are set to 0, and every other dimension
+ * is constant.  Writes n_iters(intrin) target variable ids per point into `points`, in
+ * enumeration order; returns the number of points (which may exceed max_points: only
+ * max_points are written), 0 if the bodies do not line up, negative on a bad argument.
+ * (reference: src/auto_tensorize/matcher.cc:47-310, include/tvm/auto_tensorize/matcher.h:42-331)
+ */
+int amos_match(const amos_compute_t* target, const amos_compute_t* intrin, int32_t* points,
+               int32_t max_points);
+
+/*
+ * Mappings = non-empty subsets of the match points.  Two subsets that put the same sets of
+ * loops on every intrinsic axis are one mapping (the first in binary counting order, first
+ * point = most significant bit, is kept); with more than 15 points only single points whose
+ * extents equal the intrinsic's and the all-ones subset are considered.  For each mapping
+ * `feasible` says whether every fused extent reaches the intrinsic's extent.  Returns the
+ * number of mappings (rows of n_points bytes in `bits`).
+ * (reference: python/tvm/auto_tensorize/tensorization_phases/compute_transform.py:115-207,427-499)
+ */
+int amos_enumerate_mappings(int32_t n_points, int32_t n_axes, const int32_t* points,
+                            const int64_t* target_extents, const int64_t* intrin_extents,
+                            uint8_t* bits, uint8_t* feasible, int32_t max_mappings);
 
 #ifdef __cplusplus
 }

@@ -1,0 +1,96 @@
+"""The reference's script flow on the GPU: TE compute -> auto_tensorize -> schedule ->
+build -> func(A, B, C), checked against the CPU oracle (reference flow: README.md:174-340,
+benchmark/amos/mapping_gemm_tensorcore.py:18-85)."""
+import json
+
+import numpy as np
+import pytest
+
+import amos_amd.tvm as tvm
+from amos_amd.tvm import auto_tensorize as at
+from oracle import cpu_oracle as co
+from test_mapper import conv2d, gemm
+
+pytestmark = pytest.mark.gpu
+
+
+def test_conv2d_tutorial_flow(gpu, tmp_path, capsys):
+    N, C, H, W, K, R, S, stride, padding, dilation = 2, 128, 14, 14, 64, 3, 3, 1, 1, 1
+    A, B, Conv = conv2d(N, C, H, W, K, R, S, stride, padding, dilation)
+    target_dag = at.compute_dag_from_tensors([Conv])
+    target = "hip"
+    measure_opt = at.MeasureOptions(target=target, timeout=10, number=5, min_repeat_ms=5)
+    log = str(tmp_path / "conv2d_tutorial.log")
+    result = at.auto_tensorize(target_dag, target, log, measure_opt, trials=6)
+    assert result.defined()
+    lines = [json.loads(l) for l in open(log)]
+    assert len(lines) == 6 and all(set(l) == {"record", "value"} for l in lines)
+    assert 1 / result.perf == pytest.approx(max(l["value"] for l in lines))
+    # reload from the log, as the reference's scripts do
+    result.sch_gen.load_from_file(log, clear=True)
+    entry = result.sch_gen.get_best_entry()
+    params, value = entry.record, 1 / entry.value
+    cost = at.evaluate_params(result.sch_app, params, measure_opt, dump=False)
+    assert 0 < cost < 1e3 and value > 0
+    # retrieve schedule from the record, build, run
+    schedule_app = result.sch_app
+    inputs = schedule_app.target_dag.get_inputs()
+    args = inputs + list(schedule_app.target_dag.tensors)
+    sch = tvm.te.create_schedule([x.op for x in schedule_app.target_dag.tensors])
+    sch = schedule_app.apply(sch, params)
+    func = tvm.build(sch, args, target)
+    rng = np.random.default_rng(0)
+    A_np = rng.uniform(-10, 10, [int(x) for x in A.shape]).astype(A.dtype)
+    B_np = rng.uniform(-10, 10, [int(x) for x in B.shape]).astype(B.dtype)
+    Conv_np = np.zeros([int(x) for x in Conv.shape], dtype=Conv.dtype)
+    ctx = tvm.context(target, 0)
+    A_tvm, B_tvm, Conv_tvm = tvm.nd.array(A_np, ctx), tvm.nd.array(B_np, ctx), tvm.nd.array(Conv_np, ctx)
+    func(A_tvm, B_tvm, Conv_tvm)
+    ctx.sync()
+    golden = co.lib_conv2d(A_np, B_np, "float16", stride, padding, dilation, acc="float32")
+    tvm.testing.assert_allclose(golden, Conv_tvm.asnumpy(), atol=1e-2 * float(golden.std()), rtol=1e-2)
+    mx, mean = co.rel_errors(Conv_tvm.asnumpy(), golden)
+    assert mx <= 1e-2 and mean <= 1e-3
+    assert "amos_" in func.imported_modules[0].get_source()
+    t = func.time_evaluator(func.entry_name, ctx, number=5, min_repeat_ms=5)(A_tvm, B_tvm, Conv_tvm).mean
+    assert 0 < t < 1e-2
+
+
+@pytest.mark.parametrize("ta,tb", [(0, 0), (0, 1), (1, 1)])
+def test_gemm_script_flow(gpu, tmp_path, ta, tb):
+    M, N, K = 384, 256, 320
+    A, B, C = gemm(M, N, K, ta=ta, tb=tb)
+    dag = at.compute_dag_from_tensors([C])
+    opt = at.MeasureOptions(target="hip", timeout=100, number=5, min_repeat_ms=5)
+    result = at.auto_tensorize(dag, "hip", str(tmp_path / "gemm.log"), opt, trials=4)
+    assert result.defined()
+    sch, args = at.get_schedule(result.sch_app, result.params)
+    func = tvm.build(sch, args, "hip")
+    rng = np.random.default_rng(1)
+    a = rng.uniform(-1, 1, [int(s) for s in A.shape]).astype(np.float16)
+    b = rng.uniform(-1, 1, [int(s) for s in B.shape]).astype(np.float16)
+    ctx = tvm.context("hip", 0)
+    c = tvm.nd.array(np.zeros((M, N), dtype=np.float32), ctx)
+    func(tvm.nd.array(a, ctx), tvm.nd.array(b, ctx), c)
+    mx, mean = co.rel_errors(c.asnumpy(), co.lib_gemm(a, b, "float16", ta, tb, acc="float32"))
+    assert mx <= 1e-2 and mean <= 1e-3
+
+
+def test_v4_explores_the_realised_mappings(gpu, tmp_path, capsys):
+    A, B, Conv = conv2d(4, 128, 14, 14, 128, 3, 3, 1, 1, 1, dtype="int8", out_dtype="int32", exact_int=True)
+    opt = at.MeasureOptions(target="hip", number=3, min_repeat_ms=2)
+    res = at.auto_tensorize_v4(at.compute_dag_from_tensors([Conv]), "hip", "conv.log", opt,
+                               schedule_log_dir=str(tmp_path / "logs"), trials=40, repeat_rounds=1,
+                               search_group_size=1)
+    out = capsys.readouterr().out
+    assert res.defined() and "Round 1, Match 1, Mapping" in out and "New weights" in out
+    assert "No kernel instance realises this mapping; skipped." in out
+    sch, args = at.get_schedule(res.sch_app, res.params)
+    func = tvm.build(sch, args, "hip")
+    rng = np.random.default_rng(2)
+    a = rng.integers(-128, 128, [int(s) for s in A.shape]).astype(np.int8)
+    b = rng.integers(-64, 64, [int(s) for s in B.shape]).astype(np.int8)
+    ctx = tvm.context("hip", 0)
+    y = tvm.nd.array(np.zeros([int(s) for s in Conv.shape], dtype=np.int32), ctx)
+    func(tvm.nd.array(a, ctx), tvm.nd.array(b, ctx), y)
+    assert np.array_equal(y.asnumpy(), co.lib_conv2d(a, b, "int8", 1, 1, 1))

@@ -1,0 +1,329 @@
+"""Matcher, mapping enumeration, policies, lowering and the log format, pinned against what the
+reference's README prints for its conv2d tutorial (tests/golden/readme_conv2d_mappings.json),
+a tuning log it ships, and brute-force evaluation of the TE computes.  No GPU needed."""
+import json
+import os
+
+import numpy as np
+import pytest
+
+from amos_amd import _lib, te
+from amos_amd.te import tir
+from amos_amd import auto_tensorize as at
+from amos_amd.auto_tensorize import hw_abs_dag as dagmod
+from amos_amd.auto_tensorize.hw_abstraction import MFMABase, register_abstraction
+from oracle import cpu_oracle as co
+from oracle import te_interp
+
+GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+
+
+def conv2d(N, C, H, W, K, R, S, stride, padding, dilation, dtype="float16", out_dtype="float32", exact_int=False):
+    """the tutorial's compute (reference: README.md:131-165)"""
+    kH, kW = (R - 1) * dilation + 1, (S - 1) * dilation + 1
+    pH, pW = H + 2 * padding, W + 2 * padding
+    A = te.placeholder([N, C, H, W], dtype=dtype, name="A")
+    B = te.placeholder([K, C, R, S], dtype=dtype, name="B")
+    Pad = te.compute([N, C, pH, pW], lambda n, c, h, w: tir.if_then_else(
+        tir.all(h >= padding, h - padding < H, w >= padding, w - padding < W),
+        A[n, c, h - padding, w - padding], tir.const(0.0, A.dtype)), name="Pad")
+    rc = te.reduce_axis([0, C], name="rc")
+    rr = te.reduce_axis([0, R], name="rr")
+    rs = te.reduce_axis([0, S], name="rs")
+    P, Q = (pH - kH) // stride + 1, (pW - kW) // stride + 1
+
+    def body(n, k, p, q):
+        a = Pad[n, rc, p * stride + rr * dilation, q * stride + rs * dilation]
+        b = B[k, rc, rr, rs]
+        prod = a.astype(out_dtype) * b.astype(out_dtype) if exact_int else (a * b).astype(out_dtype)
+        return te.sum(prod, axis=[rc, rr, rs])
+
+    Conv = te.compute([N, K, P, Q], body, name="Conv")
+    return A, B, Conv
+
+
+def gemm(M, N, K, dtype="float16", out="float32", ta=False, tb=False, batch=None):
+    pre = [batch] if batch else []
+    A = te.placeholder(pre + ([K, M] if ta else [M, K]), dtype=dtype, name="A")
+    B = te.placeholder(pre + ([N, K] if tb else [K, N]), dtype=dtype, name="B")
+    rk = te.reduce_axis([0, K], name="k")
+
+    def la(b, i): return A[tuple(b) + ((rk, i) if ta else (i, rk))]
+    def lb(b, j): return B[tuple(b) + ((j, rk) if tb else (rk, j))]
+    if batch:
+        C = te.compute([batch, M, N], lambda b, i, j: te.sum((la([b], i) * lb([b], j)).astype(out), axis=rk), name="C")
+    else:
+        C = te.compute([M, N], lambda i, j: te.sum((la([], i) * lb([], j)).astype(out), axis=rk), name="C")
+    return A, B, C
+
+
+# ---- a test-only intrinsic with the reference's Tensor Core shapes, to replay the README ----------
+@pytest.fixture(scope="module")
+def wmma_like_target():
+    @register_abstraction("readme_test", "wmma_fp16_fp32::mma", override=True)
+    class Mma(MFMABase):
+        in_dtype, out_dtype = "float16", "float32"
+
+    class WmmaLike(dagmod.MFMADag):
+        mnemonic = "wmma_fp16_fp32"
+        mma_mnemonic = "wmma_fp16_fp32::mma"
+        shape_keys = ("16x16x16", "32x8x16", "8x32x16")
+
+        def __init__(self):
+            self.mma = Mma()
+
+    dagmod.register_hw_abs_dag("readme_test", "wmma_fp16_fp32", override=True)(WmmaLike)
+    yield "readme_test"
+    dagmod.HW_ABS_DAG_REGISTER_POOL.remove("readme_test", "wmma_fp16_fp32")
+
+
+def names(axis_map):
+    return {k.var.name: [t.var.name for t in v] for k, v in axis_map.items()}
+
+
+def test_readme_conv2d_matchings_and_mappings(wmma_like_target, capsys):
+    gold = json.load(open(os.path.join(GOLDEN, "readme_conv2d_mappings.json")))
+    L = gold["layer"]
+    A, B, Conv = conv2d(L["N"], L["C"], L["H"], L["W"], L["K"], L["R"], L["S"], L["stride"], L["padding"], L["dilation"])
+    dag = at.compute_dag_from_tensors([Conv])
+    assert [op.name for op in dag.op_lst] == ["Pad", "Conv"]
+    assert [t.name for t in dag.get_inputs()] == ["A", "B"]
+    matches = at.get_match_results(dag, wmma_like_target)
+    assert [str(m) for m in matches] == gold["matchings"]
+    for m in matches:
+        assert names(m.axis_map) == gold["axis_map"]
+        assert list(m.main_op_map.values())[0].name == "Conv"
+    chosen, record = at.all_fit(matches)
+    assert str(chosen) == gold["selected"]
+    assert record.vmap_choice[0] == [1] * 7
+    mappings = at.MappingGenerator(chosen).get_all()
+    assert len(mappings) == gold["num_mappings"]
+    assert "Totally 35 different mappings for this matching" in capsys.readouterr().out
+    app = at.MappingApplier(chosen, strict=True)
+    infeasible, feasible = [], []
+    for r in mappings:
+        try:
+            app.apply(r)
+            feasible.append(list(r.vmap_choice[0]))
+        except RuntimeError:
+            infeasible.append(list(r.vmap_choice[0]))
+    assert infeasible == gold["infeasible"]
+    assert len(feasible) == gold["num_feasible"]
+    assert feasible[0] == gold["first_explored_mapping"]
+    assert str(mappings[0]) == '{"vmap": [[0, 0, 0, 0, 0, 0, 1], -1]}' and mappings[1].as_key() == "(0,0,0,0,0,1,0)"
+    # non-strict mode accepts every mapping and flags padding instead
+    lax = at.MappingApplier(chosen, strict=False)
+    assert all(lax.apply(r).need_padding == (list(r.vmap_choice[0]) in infeasible) for r in mappings)
+    # trial budget of the tutorial run: 1200 trials, 10 rounds, 1 matching, 20 equal weights
+    t = gold["trials"]
+    assert t["total"] // t["rounds"] // 1 == t["per_matching"]
+    assert int(np.ceil(t["per_matching"] * (1.0 / gold["num_feasible"]))) == t["per_mapping"]
+
+
+def test_mfma_registry_and_matches():
+    keys = [c().get_name() for c in at.query_hw_abs_dag("hip")]
+    assert keys == ["mfma_f16_f32", "mfma_bf16_f32", "mfma_i8_i32", "mfma_i8_i32_wrapped_spelling"]
+    assert [c().get_name() for c in at.query_hw_abs_dag("rocm")] == keys
+    assert at.query_hw_abs_dag("cuda") == []
+    A, B, C = gemm(64, 48, 32)
+    ms = at.get_match_results(at.compute_dag_from_tensors([C]), "hip")
+    assert [str(m) for m in ms] == ["MatchResult(hw_abs_dag:mfma_f16_f32, compute:%s, shape:%s)" % (c, s)
+                                    for c in ("nnn", "ntn", "tnn", "ttn") for s in ("32x32x16", "16x16x32")]
+    assert names(ms[0].axis_map) == {"i": ["i"], "j": ["j"], "rk": ["k"]}
+    # bf16 and int8 computes reach their own DAGs only
+    _, _, Cb = gemm(64, 48, 32, dtype="bfloat16")
+    assert {m.hw_abs_dag.get_name() for m in at.get_match_results(at.compute_dag_from_tensors([Cb]), "hip")} == {"mfma_bf16_f32"}
+    _, _, Ci = gemm(64, 48, 32, dtype="int8", out="int32")
+    assert {m.hw_abs_dag.get_name() for m in at.get_match_results(at.compute_dag_from_tensors([Ci]), "hip")} == \
+        {"mfma_i8_i32_wrapped_spelling"}
+    _, _, Conv = conv2d(2, 16, 8, 8, 16, 3, 3, 1, 1, 1, dtype="int8", out_dtype="int32", exact_int=True)
+    assert {m.hw_abs_dag.get_name() for m in at.get_match_results(at.compute_dag_from_tensors([Conv]), "hip")} == {"mfma_i8_i32"}
+
+
+def test_batched_gemm_batch_axis_is_a_time_loop():
+    A, B, C = gemm(32, 32, 64, tb=True, batch=6)
+    ms = at.get_match_results(at.compute_dag_from_tensors([C]), "hip")
+    assert names(ms[0].axis_map) == {"i": ["i"], "j": ["j"], "rk": ["k"]}
+    state = at.MappingApplier(ms[0]).apply(at.MappingGenerator(ms[0], verbose_init=False).get_all()[0])
+    assert [a.var.name for a in state.time_loops] == ["b"]
+
+
+def test_conv3d_has_13_match_points():
+    N, C, D, H, W, K, T, R, S = 2, 16, 6, 8, 8, 16, 3, 3, 3
+    A = te.placeholder([N, C, D, H, W], dtype="float16", name="A")
+    Wt = te.placeholder([K, C, T, R, S], dtype="float16", name="W")
+    rc, rd, rr, rs = (te.reduce_axis([0, e], name=n) for e, n in ((C, "rc"), (T, "rd"), (R, "rr"), (S, "rs")))
+    Y = te.compute([N, K, D - 2, H - 2, W - 2], lambda n, k, d, p, q: te.sum(
+        (A[n, rc, d + rd, p + rr, q + rs] * Wt[k, rc, rd, rr, rs]).astype("float32"), axis=[rc, rd, rr, rs]), name="Y")
+    m = at.get_match_results(at.compute_dag_from_tensors([Y]), "hip")[0]
+    nm = names(m.axis_map)
+    pts = set(zip(nm["i"], nm["j"], nm["rk"]))
+    want = {(i, "k", r) for i in "ndpq" for r in ("rc", "rd", "rr", "rs")} - {("d", "k", "rd"), ("p", "k", "rr"), ("q", "k", "rs")}
+    assert len(nm["i"]) == 13 and pts == want
+    low = at.lower_main_op(Y.op)
+    assert low.kind == "conv3d" and low.attrs["stride"] == [1, 1, 1] and low.attrs["pad"] == [0, 0, 0]
+
+
+def test_enumeration_rule_above_15_points():
+    """more than 15 points: single points whose extents equal the intrinsic's, plus all ones"""
+    import ctypes
+    n_points, n_axes = 16, 3
+    pts = []
+    for p in range(n_points):
+        pts += [p, 16, 17]                 # i differs per point, j and rk shared
+    ext = [32 if p in (3, 9) else 8 for p in range(16)] + [32, 16]
+    flat = (ctypes.c_int32 * len(pts))(*pts)
+    text = (ctypes.c_int64 * len(ext))(*ext)
+    iext = (ctypes.c_int64 * 3)(32, 32, 16)
+    bits = (ctypes.c_uint8 * (32 * n_points))()
+    feas = (ctypes.c_uint8 * 32)()
+    n = _lib.load().amos_enumerate_mappings(n_points, n_axes, flat, text, iext, bits, feas, 32)
+    rows = [[bits[m * n_points + i] for i in range(n_points)] for m in range(n)]
+    assert n == 3 and rows[0] == [int(i == 3) for i in range(16)] and rows[1] == [int(i == 9) for i in range(16)]
+    assert rows[2] == [1] * 16 and list(feas[:3]) == [1, 1, 1]
+
+
+@pytest.mark.parametrize("ta,tb", [(0, 0), (0, 1), (1, 0), (1, 1)])
+@pytest.mark.parametrize("dtype", ["float16", "int8"])
+def test_lowered_gemm_means_what_the_compute_says(ta, tb, dtype):
+    M, N, K = 5, 4, 6
+    A, B, C = gemm(M, N, K, dtype=dtype, out="int32" if dtype == "int8" else "float32", ta=ta, tb=tb)
+    low = at.lower_main_op(C.op)
+    assert low.kind == "gemm" and (low.attrs["trans_a"], low.attrs["trans_b"]) == (ta, tb)
+    assert (low.desc.M, low.desc.N, low.desc.K, low.desc.lda, low.desc.ldb, low.desc.ldc) == \
+        (M, N, K, M if ta else K, K if tb else N, N)
+    rng = np.random.default_rng(1)
+    a = rng.integers(-5, 6, [int(s) for s in A.shape]).astype(np.int8 if dtype == "int8" else np.float16)
+    b = rng.integers(-5, 6, [int(s) for s in B.shape]).astype(a.dtype)
+    want = te_interp.evaluate(C, {"A": a, "B": b})
+    feeds = {low.inputs[0].name: a if low.inputs[0] is A else b, low.inputs[1].name: b if low.inputs[1] is B else a}
+    got = co.te_literal_gemm(feeds[low.inputs[0].name], feeds[low.inputs[1].name], dtype,
+                             bool(low.attrs["trans_a"]), bool(low.attrs["trans_b"]), mode="exact")
+    assert np.array_equal(got, want)
+
+
+def test_lowered_gemm_with_swapped_operands():
+    """C[i, j] = sum_k B[k, j] * A[i, k]: the row operand is the second factor"""
+    M, N, K = 4, 3, 5
+    A = te.placeholder([M, K], dtype="float16", name="A")
+    B = te.placeholder([K, N], dtype="float16", name="B")
+    rk = te.reduce_axis([0, K], name="k")
+    C = te.compute([M, N], lambda i, j: te.sum((B[rk, j] * A[i, rk]).astype("float32"), axis=rk), name="C")
+    low = at.lower_main_op(C.op)
+    assert [t.name for t in low.inputs] == ["A", "B"] and (low.attrs["trans_a"], low.attrs["trans_b"]) == (0, 0)
+
+
+CONV_LOWER_CASES = [(2, 3, 7, 6, 4, 3, 3, 1, 1, 1), (1, 2, 9, 9, 3, 3, 3, 2, 1, 1), (1, 2, 9, 8, 2, 3, 3, 1, 2, 2),
+                    (1, 3, 6, 6, 2, 1, 1, 1, 0, 1), (1, 2, 8, 8, 2, 3, 3, 2, 0, 1)]
+
+
+@pytest.mark.parametrize("case", CONV_LOWER_CASES)
+def test_lowered_conv2d_means_what_the_compute_says(case):
+    N, C, H, W, K, R, S, st, pd, dl = case
+    A, B, Conv = conv2d(N, C, H, W, K, R, S, st, pd, dl, dtype="int8", out_dtype="int32", exact_int=True)
+    low = at.lower_main_op(Conv.op)
+    assert low.kind == "conv2d" and low.attrs["stride"] == [st, st] and low.attrs["pad"] == [pd, pd] and low.attrs["dil"] == [dl, dl]
+    assert [t.name for t in low.inputs] == ["A", "B"]
+    rng = np.random.default_rng(2)
+    a = rng.integers(-9, 10, (N, C, H, W)).astype(np.int8)
+    b = rng.integers(-9, 10, (K, C, R, S)).astype(np.int8)
+    want = te_interp.evaluate(Conv, {"A": a, "B": b})
+    got = co.te_literal_conv2d(a, b, "int8", low.attrs["stride"], low.attrs["pad"], low.attrs["dil"], mode="exact")
+    assert np.array_equal(got, want)
+
+
+def test_no_kernel_for_other_layouts():
+    # NHWC activations match the intrinsic but have no kernel
+    N, H, W, C, K = 2, 6, 6, 8, 8
+    A = te.placeholder([N, H, W, C], dtype="float16", name="A")
+    B = te.placeholder([K, C, 3, 3], dtype="float16", name="B")
+    rc, rr, rs = te.reduce_axis([0, C], "rc"), te.reduce_axis([0, 3], "rr"), te.reduce_axis([0, 3], "rs")
+    Y = te.compute([N, K, H - 2, W - 2], lambda n, k, p, q: te.sum(
+        (A[n, p + rr, q + rs, rc] * B[k, rc, rr, rs]).astype("float32"), axis=[rc, rr, rs]), name="Y")
+    assert at.get_match_results(at.compute_dag_from_tensors([Y]), "hip")
+    with pytest.raises(at.NoKernelError):
+        at.lower_main_op(Y.op)
+    # fp16 accumulate has no instruction
+    _, _, C16 = gemm(32, 32, 32, out="float16")
+    assert at.get_match_results(at.compute_dag_from_tensors([C16]), "hip") == []
+
+
+def test_auto_tensorize_plumbing_config1_on_cpu(tmp_path, capsys):
+    """fp16 GEMM 512^3: TE compute -> match -> mapping -> schedule object -> descriptor, no GPU;
+    the CPU result of the same compute comes from the oracle"""
+    A, B, C = gemm(512, 512, 512)
+    dag = at.compute_dag_from_tensors([C])
+    opt = at.MeasureOptions(target="hip", timeout=100, number=200, min_repeat_ms=500)
+    res = at.auto_tensorize(dag, "hip", str(tmp_path / "gemm.log"), opt, trials=0)
+    out = capsys.readouterr().out
+    assert "Possible matchings:" in out and "Selected matching:" in out and "Axis mapping:" in out
+    assert res.defined() and res.perf > 0 and opt.target == "hip"
+    sch, args = at.get_schedule(res.sch_app, res.params)
+    assert [t.name for t in args] == ["A", "B", "C"] and sch.lowered.kind == "gemm"
+    cfg = res.params.to_config()
+    assert _lib.load().amos_check_config(0, __import__("ctypes").byref(sch.lowered.desc), __import__("ctypes").byref(cfg), None, None) == 0
+    rng = np.random.default_rng(0)
+    a = rng.uniform(-1, 1, (512, 512)).astype(np.float16)
+    b = rng.uniform(-1, 1, (512, 512)).astype(np.float16)
+    lit = co.te_literal_gemm(a, b, "float16", threads=8)
+    mx, mean = co.rel_errors(lit, co.lib_gemm(a, b, "float16", acc="float64"))
+    assert mean < 1e-3
+    with pytest.raises(RuntimeError):
+        at.auto_tensorize(dag, "cuda", "", opt, trials=0)
+
+
+def test_v4_pure_test_mode_lists_infeasible_mappings(tmp_path, capsys):
+    A, B, Conv = conv2d(1, 128, 28, 28, 128, 3, 3, 1, 1, 1)
+    opt = at.MeasureOptions(target="hip")
+    res = at.auto_tensorize_v4(at.compute_dag_from_tensors([Conv]), "hip", "conv.log", opt,
+                               schedule_log_dir=str(tmp_path / "logs"), trials=0)
+    out = capsys.readouterr().out
+    assert "Catch an infeasible mapping:" in out and "Pure testing mode..." in out and "Num mapping:" in out
+    assert res.defined() and res.mapping is not None
+    # the two mappings the kernel family realises: channels only on rk (patch staging), or all
+    # reduce loops fused on rk (im2col staging); both put n, p, q on i
+    # (the enumeration keeps the first bit vector of each distinct set of fused loops)
+    m = at.all_fit(at.get_match_results(at.compute_dag_from_tensors([Conv]), "hip"))[0]
+    fused = {k: set(v) for k, v in at.MappingApplier(m, strict=False).apply(res.mapping).fused_names().items()}
+    assert fused["i"] == {"n", "p", "q"} and fused["j"] == {"k"}
+    assert fused["rk"] in ({"rc"}, {"rc", "rr", "rs"})
+
+
+def test_log_format_and_reference_fixture(tmp_path):
+    from amos_amd.auto_tensorize.schedule import KernelParams, read_log
+    rows = read_log(os.path.join(GOLDEN, "a100_conv2d_1_256_14_14_256_3_3_mapping_0010010.log"))
+    assert len(rows) == 13 and set(rows[0][0].keys()) >= {"inline", "vectorize", "spatial_factors", "reduce_factors"}
+    best = max(v for _, v in rows)
+    assert abs(1 / best * 1e3 - 0.049993) < 1e-5      # ms, the figure quoted for this layer
+    A, B, C = gemm(256, 256, 256, tb=True)
+    m = at.get_match_results(at.compute_dag_from_tensors([C]), "hip")[0]
+    log = str(tmp_path / "t.log")
+    gen = at.MI355XScheduleGenerator(m, None, log_file=log, verbose_init=False)
+    gen.feedback(KernelParams(128, 128, 1, 0), 1 / 20e-6)
+    gen.feedback(KernelParams(256, 256, 1, 0), 1 / 10e-6)
+    gen.feedback(KernelParams(64, 64, 2, 1), 1 / 30e-6)
+    lines = [json.loads(l) for l in open(log)]
+    assert lines[1] == {"record": {"tile_i": 256, "tile_j": 256, "split_k": 1, "pipeline": 0}, "value": 1 / 10e-6}
+    gen2 = at.MI355XScheduleGenerator(m, None, log_file=str(tmp_path / "u.log"), verbose_init=False)
+    gen2.load_from_file(log)
+    e = gen2.get_best_entry()
+    assert e.record.to_json() == lines[1]["record"] and gen2.num_entries() == 3 and 1 / e.value == pytest.approx(10e-6)
+    # every candidate the sweep proposes resolves to a compiled kernel instance
+    cands = gen.candidates()
+    assert len(cands) > 8 and str(cands[0]) == str(KernelParams(256, 256, 1, 0)) or len(cands) > 8
+
+
+def test_measure_options_defaults():
+    o = at.MeasureOptions()
+    assert (o.target, o.timeout, o.number, o.repeat, o.min_repeat_ms, o.dev_id) == ("llvm", 10, 100, 1, 150, 0)
+
+
+def test_fragment_layout_is_a_bijection():
+    from amos_amd.auto_tensorize.hw_abstraction import mfma_fragment_layout
+    for key in ("32x32x16", "16x16x32", "32x32x32", "16x16x64"):
+        m, n, k = (int(x) for x in key.split("x"))
+        lay = mfma_fragment_layout(key)
+        a = {lay["a"](l, e) for l in range(64) for e in range(lay["k_per_lane"])}
+        d = {lay["d"](l, r) for l in range(64) for r in range(lay["acc_regs"])}
+        assert a == {(i, kk) for i in range(m) for kk in range(k)}
+        assert d == {(i, j) for i in range(m) for j in range(n)}
