@@ -21,6 +21,9 @@ METRIC = "TFLOP/s + % of MFMA peak per op (fp16 conv2d/GEMM, int8 TOP/s), 1 MI35
 PEAK_F16_TFLOPS = 2500.0   # published dense fp16 MFMA peak of MI355X
 PEAK_I8_TOPS = 5000.0      # published dense int8 peak
 PEAK_HBM_GBS = 8000.0      # published HBM3E bandwidth
+# bytes beyond L2 per launch, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this command,
+# each scaled by the same counter's reading for a 256 MiB device copy (x2.0 and x1.0)
+MEASURED_TRAFFIC = {"amos_gemm_tn<f16,256x256,8w>": 870610 * 1024 * 2.0 + 262140 * 1024 * 1.0}
 
 
 def cpu_baseline_gemm(a, b, seconds_budget=12.0):
@@ -145,6 +148,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU-baseline leg")
     ap.add_argument("--report", default=None, help="also time every config, write JSON here")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run a 256 MiB device copy, the known-size kernel that rocprofv3's "
+                         "FETCH_SIZE / WRITE_SIZE readings are scaled by")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures the one-GPU kernel path; --gpus %d is not supported "
@@ -164,6 +170,14 @@ def main():
     desc = ops.gemm_desc(n, n, n, torch.float16, False, True)
     cfg = ops.default_config(_lib.AMOS_OP_GEMM, desc)
     flop = 2.0 * n ** 3
+
+    if args.calibrate_copy:
+        src = torch.empty(256 << 20, dtype=torch.uint8, device="cuda").random_()
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
 
     for _ in range(args.warmup):
         ops.gemm(da, db, False, True, out=dc, config=cfg)
@@ -190,7 +204,8 @@ def main():
                    "tile": "%dx%d" % (cfg.tile_i, cfg.tile_j), "split_k": cfg.split_k,
                    "pct_of_mfma_peak": 100.0 * value / PEAK_F16_TFLOPS},
         "roofline": {"bound": "mfma", "achieved": achieved, "peak": PEAK_F16_TFLOPS,
-                     "unit": "TFLOP/s", "frac": achieved / PEAK_F16_TFLOPS, "traffic": None,
+                     "unit": "TFLOP/s", "frac": achieved / PEAK_F16_TFLOPS,
+                     "traffic": MEASURED_TRAFFIC.get(ops.kernel_name(_lib.AMOS_OP_GEMM, desc, cfg)),
                      "kernel_us": per_launch * 1e6},
     }
     if not args.no_cpu:
