@@ -69,6 +69,7 @@ struct Plan {
   int conv_ups;
   ConvFpropParams cv;
   size_t conv_lds;
+  int conv_occ;
 };
 
 static int dtype_pair(int in_dtype, int out_dtype, int* dt) {
@@ -267,6 +268,7 @@ static int plan_conv(Plan& pl, int op, const amos_conv_desc_t* d, const amos_ker
   if (!why && (!workspace || ws_bytes < (size_t)need_ws || ((uintptr_t)workspace & 255)))
     why = "workspace smaller than amos_workspace_bytes() or not 256-byte aligned";
   const int max_pos = pp.max_pos, nsw = pp.nsw, pls = pp.pls;
+  pl.conv_occ = pp.occ;
   const size_t lds = pp.lds;
   (void)RS;
   if (why) {
@@ -293,6 +295,7 @@ static int plan_conv(Plan& pl, int op, const amos_conv_desc_t* d, const amos_ker
   q.max_pos = max_pos;
   q.nsw = nsw;
   q.pls = pls;
+  q.xbufs = pp.xbufs;
   q.c_chunks = (int)(c.C * es / 128);
   q.macro_steps = (int)c.T * q.c_chunks;
   int split = pl.cfg.split_k < 1 ? 1 : pl.cfg.split_k;
@@ -310,8 +313,10 @@ static int plan_conv(Plan& pl, int op, const amos_conv_desc_t* d, const amos_ker
   q.fd_wp = make_fast_div((uint32_t)Wp);
   q.fd_odpq = make_fast_div((uint32_t)odpq);
   q.fd_cc = make_fast_div((uint32_t)q.c_chunks);
+  q.fd_c = make_fast_div((uint32_t)c.C);
   const int64_t welems = c.K * c.T * c.R * c.S * c.C;
-  q.prep_w_blocks = (int)((welems + 2047) / 2048 < 1024 ? (welems + 2047) / 2048 : 1024);
+  (void)welems;
+  q.prep_w_blocks = (int)(c.K < 1024 ? c.K : 1024);
   q.prep_x_blocks = (int)(c.N * c.D * (((int64_t)c.H * c.W + 63) / 64) * (c.C / 64));
   q.prep_z_blocks = q.zero_words ? (int)((q.zero_words + 4095) / 4096 < 2048 ? (q.zero_words + 4095) / 4096 : 2048) : 0;
   return 0;
@@ -364,14 +369,14 @@ static int launch_tn(const Plan& pl, hipStream_t stream) {
   return 0;
 }
 
-static ConvInstance* pick_conv(int dt, int ti, int tj) {
-  if (dt == DT_F16) return pick_conv_f16(ti, tj);
-  if (dt == DT_BF16) return pick_conv_bf16(ti, tj);
-  return pick_conv_i8(ti, tj);
+static ConvInstance* pick_conv(int dt, int ti, int tj, int occ) {
+  if (dt == DT_F16) return pick_conv_f16(ti, tj, occ);
+  if (dt == DT_BF16) return pick_conv_bf16(ti, tj, occ);
+  return pick_conv_i8(ti, tj, occ);
 }
 
 static int launch_conv(const Plan& pl, hipStream_t stream) {
-  ConvInstance* inst = pick_conv(pl.dt, pl.cfg.tile_i, pl.cfg.tile_j);
+  ConvInstance* inst = pick_conv(pl.dt, pl.cfg.tile_i, pl.cfg.tile_j, pl.conv_occ);
   if (!inst) return set_error(AMOS_ERR_INFEASIBLE, "no patch-staged convolution instance");
   hipError_t attr_err = hipSuccess;
   std::call_once(inst->once, [&] {
@@ -494,7 +499,7 @@ const char* amos_kernel_name(int op, const void* desc, const amos_kernel_config_
   static char dummy_ws[256] __attribute__((aligned(256)));
   if (make_plan(pl, op, desc, cfg, dummy, dummy, dummy, dummy_ws, (size_t)-1)) return nullptr;
   if (pl.conv_ups) {
-    ConvInstance* ci = pick_conv(pl.dt, pl.cfg.tile_i, pl.cfg.tile_j);
+    ConvInstance* ci = pick_conv(pl.dt, pl.cfg.tile_i, pl.cfg.tile_j, pl.conv_occ);
     return ci ? ci->name : nullptr;
   }
   if (pl.tn_waves) {

@@ -76,12 +76,13 @@ struct ConvFpropParams {
   int max_pos;       // LDS positions reserved per patch buffer (multiple of 8)
   int nsw;           // weight ring stages (>= 2)
   int pls;           // patch copy instructions per wave per K step
+  int xbufs;         // patch buffers: 2, or 1 when a block handles a single (depth tap, channel chunk)
   int c_chunks;      // C*ES / 128
   int macro_steps;   // T * c_chunks
   int macro_per_split;
   int tiles_i, tiles_j;
   int atomic_out;
-  FastDiv fd_opq, fd_oq, fd_od, fd_wp, fd_odpq, fd_cc;   // divisions by OP*OQ, OQ, OD, Wp, OD*OP*OQ, c_chunks
+  FastDiv fd_opq, fd_oq, fd_od, fd_wp, fd_odpq, fd_cc, fd_c;   // divisions by OP*OQ, OQ, OD, Wp, OD*OP*OQ, c_chunks, C
   // prepare kernel work split (in blocks)
   int prep_w_blocks, prep_x_blocks, prep_z_blocks;
   int64_t zero_words;
@@ -95,15 +96,19 @@ __global__ __launch_bounds__(256) void amos_conv_prepare(const ConvFpropParams p
   int b = blockIdx.x;
   const int TRS = p.T * p.R * p.S;
   if (b < p.prep_w_blocks) {
-    // wp[k][tap][c] = w[k][c][tap]; idx walks the OUTPUT order so writes coalesce
-    const int64_t n = (int64_t)p.K * p.C * TRS;
+    // wp[k][tap][c] = w[k][c][tap]: one block per output channel k (grid-strided); the
+    // k-th slab of C*TRS elements is read contiguously into LDS-free registers by walking the
+    // OUTPUT order (writes coalesce, reads stay inside one 1-2 KB slab that L1 holds)
     const T* w = (const T*)p.w;
     T* wp = (T*)p.wp;
-    for (int64_t idx = (int64_t)b * 256 + t; idx < n; idx += (int64_t)p.prep_w_blocks * 256) {
-      int64_t k = idx / ((int64_t)p.C * TRS);
-      int rem = (int)(idx - k * (int64_t)p.C * TRS);
-      int tap = rem / p.C, c = rem - tap * p.C;
-      wp[idx] = w[(k * p.C + c) * TRS + tap];
+    const int slab = p.C * TRS;
+    for (int k = b; k < p.K; k += p.prep_w_blocks) {
+      const T* src = w + (int64_t)k * slab;
+      T* dst = wp + (int64_t)k * slab;
+      for (int o = t; o < slab; o += 256) {
+        const int tap = fast_div(o, p.fd_c), c = o - tap * p.C;
+        dst[o] = src[c * TRS + tap];
+      }
     }
     if (b == 0 && t < 32) ((int*)p.zeros)[t] = 0;
     return;
@@ -157,8 +162,9 @@ __device__ __forceinline__ void wait_vmcnt_le(int n) {
 }
 
 // ---- launch 2: the convolution -----------------------------------------------------------------
-template <int DT, int TI, int TJ>
-__global__ __launch_bounds__(256) void amos_conv_fprop(const ConvFpropParams p) {
+// OCC = workgroups the compiler must leave room for on a CU (register budget 512 / OCC per lane)
+template <int DT, int TI, int TJ, int OCC>
+__global__ __launch_bounds__(256, OCC) void amos_conv_fprop(const ConvFpropParams p) {
   typedef Mfma<DT> MM;
   typedef typename MM::acc_t acc_t;
   typedef typename MM::out_t out_t;
@@ -169,8 +175,8 @@ __global__ __launch_bounds__(256) void amos_conv_fprop(const ConvFpropParams p) 
 
   extern __shared__ __attribute__((aligned(16))) char smem[];
   char* const sW = smem;                                            // [nsw][BI*128]
-  char* const sX = smem + (size_t)p.nsw * WSTAGE;                   // [2][max_pos*128]
-  int2* const sTab = (int2*)(sX + 2 * (size_t)p.max_pos * 128);     // [max_pos] position table
+  char* const sX = smem + (size_t)p.nsw * WSTAGE;                   // [xbufs][max_pos*128]
+  int2* const sTab = (int2*)(sX + (size_t)p.xbufs * p.max_pos * 128);   // [max_pos] position table
 
   const int t = threadIdx.x;
   const int lane = t & 63;
@@ -320,28 +326,39 @@ __global__ __launch_bounds__(256) void amos_conv_fprop(const ConvFpropParams p) 
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[a][b][r] = 0;
 
-  v4i af[2][TI], bf[2][TJ];
-  unsigned xb[TJ], xsw[TJ];   // per column: LDS address of its position at the current tap, swizzle term
-  auto set_tap = [&](unsigned xbuf_lds, int dpos) {
+  // Operand fragments of a whole K step (4 sub-steps) are read one step ahead: with wave tiles
+  // this small, the MFMAs of one sub-step are too few to cover the LDS latency of the next.
+  v4i af[2][4][TI], bf[2][4][TJ];
+  auto read_step = [&](unsigned wstage_off, unsigned xbuf_lds, int dpos, int slot) {
+    unsigned xb[TJ], xsw[TJ];   // per column: LDS address of its position at this tap, swizzle term
 #pragma unroll
     for (int b = 0; b < TJ; ++b) {
       const int pos = col_pos[b] + dpos;
       xb[b] = xbuf_lds + (unsigned)pos * 128;
       xsw[b] = (unsigned)((pos ^ (pos >> 3)) & 7) << 4;
     }
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks) {
+#pragma unroll
+      for (int a = 0; a < TI; ++a)
+        af[slot][ks][a] = *(const v4i*)AMOS_LDS_PTR_FROM(a_off[a & 1][ks] + wstage_off + (a >> 1) * (64 * 128));
+#pragma unroll
+      for (int b = 0; b < TJ; ++b) bf[slot][ks][b] = *(const v4i*)AMOS_LDS_PTR_FROM(xb[b] + (kh[ks] ^ xsw[b]));
+    }
   };
-  auto read_frags = [&](unsigned wstage_off, int ks, int slot) {
+  auto mma_step = [&](int slot) {
 #pragma unroll
-    for (int a = 0; a < TI; ++a)
-      af[slot][a] = *(const v4i*)AMOS_LDS_PTR_FROM(a_off[a & 1][ks] + wstage_off + (a >> 1) * (64 * 128));
+    for (int ks = 0; ks < 4; ++ks)
 #pragma unroll
-    for (int b = 0; b < TJ; ++b) bf[slot][b] = *(const v4i*)AMOS_LDS_PTR_FROM(xb[b] + (kh[ks] ^ xsw[b]));
+      for (int a = 0; a < TI; ++a)
+#pragma unroll
+        for (int b = 0; b < TJ; ++b) acc[a][b] = MM::run(af[slot][ks][a], bf[slot][ks][b], acc[a][b]);
   };
-  auto mma = [&](int slot) {
-#pragma unroll
-    for (int a = 0; a < TI; ++a)
-#pragma unroll
-      for (int b = 0; b < TJ; ++b) acc[a][b] = MM::run(af[slot][a], bf[slot][b], acc[a][b]);
+  // wait until at most `later` weight tiles (the youngest) are still in flight
+  auto wait_weights = [&](int later) {
+    if (later >= 2) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * WCH) : "memory");
+    else if (later == 1) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(WCH) : "memory");
+    else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   };
 
   // ---- prologue: the whole first patch, the first NSW weight tiles -------------------------------
@@ -349,47 +366,43 @@ __global__ __launch_bounds__(256) void amos_conv_fprop(const ConvFpropParams p) 
   if (n_steps > 0) {
     for (int v = 0; v < n_pl; ++v) issue_patch(m_begin, 0, v);
     while (iw_step < NSW && iw_step < n_steps) issue_next_weights();
-    wait_vmcnt_le(WCH * (iw_step - 1));   // patch and tile 0 landed
+    wait_weights(iw_step - 1);   // patch and tile 0 landed (NSW <= 4: never more than 3 later tiles)
     asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
-    set_tap(x_lds, 0);
-    read_frags(0, 0, 0);
+    read_step(0, x_lds, 0, 0);
   }
 
   // current K step: macro step index mi (of this block), tap = (tr, ts), ring stage
   int mi = 0, tap = 0, tr = 0, ts = 0, stage = 0;
-  for (int step = 0; step < n_steps; ++step) {
-    const unsigned wst = (unsigned)stage * WSTAGE;
-    read_frags(wst, 1, 1);
-    mma(0);
-    read_frags(wst, 2, 0);
-    mma(1);
-    read_frags(wst, 3, 1);
-    mma(0);
-    // Every read of this step's weight stage (and, on a patch's last tap, of the patch) has
-    // been issued.  Wait for them and for this wave's copies of the next weight tile, then
-    // meet: afterwards the next tile is complete everywhere and this stage is free.
-    const int later = iw_step - (step + 2);   // weight tiles issued after tile step+1
-    wait_vmcnt_le(WCH * (later < 0 ? 0 : later));
+  auto one_step = [&](int step, int slot) {
+    // This wave's reads of the current step's operands (issued a step ago) and its copies of the
+    // next weight tile are complete; after the barrier that holds for every wave: the next tile
+    // (and, past a patch's last tap, the next patch) may be read, the current stage overwritten.
+    wait_weights(iw_step - (step + 2));   // weight tiles issued after tile step+1
     asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
     // Patch of the next (depth tap, channel chunk): a few copies per step on the early taps,
     // issued BEFORE this step's weight tile so that they are older than a tile that is
     // waited for before the patch is first read.
     if (mi + 1 < n_macro && tap * p.pls < n_pl) {
       const int v_end = (tap + 1) * p.pls < n_pl ? (tap + 1) * p.pls : n_pl;
-      for (int v = tap * p.pls; v < v_end; ++v) issue_patch(m_begin + mi + 1, (mi + 1) & 1, v);
+      for (int v = tap * p.pls; v < v_end; ++v) issue_patch(m_begin + mi + 1, (mi + 1) & (p.xbufs - 1), v);
     }
     if (iw_step < n_steps) issue_next_weights();   // tile step+NSW into the stage just freed
-    // next K step
+    // operands of the next K step, then the MFMAs of this one
     ++tap;
     if (++ts == p.S) { ts = 0; ++tr; }
     if (tap == RS) { tap = 0; tr = 0; ++mi; }
     if (++stage == NSW) stage = 0;
-    if (step + 1 < n_steps) {
-      set_tap(x_lds + (unsigned)(mi & 1) * (unsigned)xbuf_bytes, tr * p.dh * p.Wp + ts * p.dw);
-      read_frags((unsigned)stage * WSTAGE, 0, 0);
-    }
-    mma(1);
+    if (step + 1 < n_steps)
+      read_step((unsigned)stage * WSTAGE, x_lds + (unsigned)(mi & (p.xbufs - 1)) * (unsigned)xbuf_bytes,
+                tr * p.dh * p.Wp + ts * p.dw, slot ^ 1);
+    mma_step(slot);
+  };
+  int step = 0;
+  for (; step + 1 < n_steps; step += 2) {
+    one_step(step, 0);
+    one_step(step + 1, 1);
   }
+  if (step < n_steps) one_step(step, 0);
 
   // ---- epilogue: Y[(n*K + i)*ODPQ + (od*OPQ + opq)] ---------------------------------------------
   out_t* const out = (out_t*)p.y;

@@ -74,32 +74,39 @@ struct ConvInstance {
   const char* name;
   std::once_flag once;
 };
-ConvInstance* pick_conv_f16(int ti, int tj);
-ConvInstance* pick_conv_bf16(int ti, int tj);
-ConvInstance* pick_conv_i8(int ti, int tj);
+ConvInstance* pick_conv_f16(int ti, int tj, int occ);
+ConvInstance* pick_conv_bf16(int ti, int tj, int occ);
+ConvInstance* pick_conv_i8(int ti, int tj, int occ);
 void launch_conv_prepare(int es, const ConvFpropParams& p, hipStream_t stream);
 
 #ifdef AMOS_CONV_FPROP_KERNEL_INCLUDED
-template <int DT, int TI, int TJ>
+template <int DT, int TI, int TJ, int OCC>
 ConvInstance* conv_instance() {
   static ConvInstance inst;
   static const char* dtn[] = {"f16", "bf16", "i8"};
   static std::string name = std::string("amos_conv_fprop<") + dtn[DT] + "," + std::to_string(64 * TI) +
-                            "x" + std::to_string(64 * TJ) + ">";
-  inst.fn = amos_conv_fprop<DT, TI, TJ>;
+                            "x" + std::to_string(64 * TJ) + (OCC == 2 ? ",occ2>" : ">");
+  inst.fn = amos_conv_fprop<DT, TI, TJ, OCC>;
   inst.name = name.c_str();
   return &inst;
 }
 template <int DT>
-ConvInstance* pick_conv_tile(int ti, int tj) {
-  if (ti == 64 && tj == 64) return conv_instance<DT, 1, 1>();
-  if (ti == 128 && tj == 64) return conv_instance<DT, 2, 1>();
-  if (ti == 64 && tj == 128) return conv_instance<DT, 1, 2>();
-  if (ti == 128 && tj == 128) return conv_instance<DT, 2, 2>();
-  if (ti == 256 && tj == 64) return conv_instance<DT, 4, 1>();
-  if (ti == 256 && tj == 128) return conv_instance<DT, 4, 2>();
-  if (ti == 128 && tj == 256) return conv_instance<DT, 2, 4>();
-  if (ti == 64 && tj == 256) return conv_instance<DT, 1, 4>();
+ConvInstance* pick_conv_tile(int ti, int tj, int occ) {
+  if (occ == 2) {
+    if (ti == 64 && tj == 64) return conv_instance<DT, 1, 1, 2>();
+    if (ti == 128 && tj == 64) return conv_instance<DT, 2, 1, 2>();
+    if (ti == 64 && tj == 128) return conv_instance<DT, 1, 2, 2>();
+    if (ti == 128 && tj == 128) return conv_instance<DT, 2, 2, 2>();
+    return nullptr;
+  }
+  if (ti == 64 && tj == 64) return conv_instance<DT, 1, 1, 1>();
+  if (ti == 128 && tj == 64) return conv_instance<DT, 2, 1, 1>();
+  if (ti == 64 && tj == 128) return conv_instance<DT, 1, 2, 1>();
+  if (ti == 128 && tj == 128) return conv_instance<DT, 2, 2, 1>();
+  if (ti == 256 && tj == 64) return conv_instance<DT, 4, 1, 1>();
+  if (ti == 256 && tj == 128) return conv_instance<DT, 4, 2, 1>();
+  if (ti == 128 && tj == 256) return conv_instance<DT, 2, 4, 1>();
+  if (ti == 64 && tj == 256) return conv_instance<DT, 1, 4, 1>();
   return nullptr;
 }
 #endif

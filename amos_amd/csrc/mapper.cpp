@@ -113,7 +113,7 @@ int64_t conv_workspace_bytes(const amos_conv_desc_t& c, int op) {
 
 
 ConvPatchPlan conv_patch_plan(const amos_conv_desc_t& cin, int op, int BI, int BJ, int split_k) {
-  ConvPatchPlan pp = {nullptr, 0, 0, 0, 0, 0};
+  ConvPatchPlan pp = {nullptr, 0, 0, 0, 0, 0, 0, 0};
   amos_conv_desc_t c = cin;
   if (op == AMOS_OP_CONV2D) { c.D = 1; c.T = 1; c.stride_d = 1; c.pad_d = 0; c.dil_d = 1; }
   const int es = c.in_dtype == AMOS_I8 ? 1 : 2;
@@ -140,7 +140,11 @@ ConvPatchPlan conv_patch_plan(const amos_conv_desc_t& cin, int op, int BI, int B
   conv_patch_extent(J, (int)(OP * OQ), (int)OQ, BJ, c.stride_h, (int)c.R, c.dil_h, Wp, &max_pos, &max_seg);
   max_pos = (max_pos + 7) & ~7;
   const size_t budget = (size_t)160 * 1024 - 512;
-  const size_t patch = (size_t)2 * max_pos * 128 + (size_t)max_pos * 8;
+  const int64_t macro_steps = c.T * (c.C * es / 128);
+  const int split = split_k < 1 ? 1 : split_k;
+  const bool one_macro = (macro_steps + split - 1) / split <= 1;   // no next patch at all
+  pp.xbufs = one_macro ? 1 : 2;
+  const size_t patch = (size_t)pp.xbufs * max_pos * 128 + (size_t)max_pos * 8;
   const size_t wstage = (size_t)BI * 128;
   pp.max_pos = max_pos;
   pp.max_seg = max_seg;
@@ -148,15 +152,12 @@ ConvPatchPlan conv_patch_plan(const amos_conv_desc_t& cin, int op, int BI, int B
   if (max_pos >= 4096) { pp.why = "input patch of a tile has 4096 or more positions"; return pp; }
   if (patch + 2 * wstage > budget) { pp.why = "input patch of a tile does not fit LDS"; return pp; }
   int nsw = (int)((budget - patch) / wstage);
-  if (nsw > 8) nsw = 8;
+  if (nsw > 4) nsw = 4;   // the kernel's wait accounting covers up to two tiles in flight behind the next
   if (nsw > RS + 1) nsw = RS + 1;
   // The next patch is copied during the taps of the current one.  A copy issued on tap u is
   // complete for everybody at the barrier of the patch's last tap only if u <= RS-2 and it is
   // older than the weight tiles still allowed in flight there: u <= RS+1-nsw.
   int taps = RS + 2 - nsw < RS - 1 ? RS + 2 - nsw : RS - 1;
-  const int64_t macro_steps = c.T * (c.C * es / 128);
-  const int split = split_k < 1 ? 1 : split_k;
-  const bool one_macro = (macro_steps + split - 1) / split <= 1;   // no next patch at all
   if (taps < 1 && !one_macro) { pp.why = "1x1 window with several channel chunks per block"; return pp; }
   if (taps < 1) taps = 1;
   const int per_wave = ((max_pos / 8) + 3) / 4;
@@ -164,6 +165,24 @@ ConvPatchPlan conv_patch_plan(const amos_conv_desc_t& cin, int op, int BI, int B
   if (pp.pls < 1) pp.pls = 1;
   pp.nsw = nsw;
   pp.lds = (size_t)nsw * wstage + patch;
+  pp.occ = 1;
+  // two workgroups per CU when both fit: 80 KB of LDS each, accumulators + two steps of operand
+  // fragments within 256 registers (tiles up to 128x128); pointless when every block already has
+  // a CU to itself
+  const int64_t blocks = ((c.K + BI - 1) / BI) * ((J + BJ - 1) / BJ) * split;
+  if (BI <= 128 && BJ <= 128 && blocks > Gfx950::kComputeUnits) {
+    int nsw2 = nsw;
+    while (nsw2 > 2 && (size_t)nsw2 * wstage + patch > (size_t)79 * 1024) --nsw2;
+    if ((size_t)nsw2 * wstage + patch <= (size_t)79 * 1024) {
+      pp.occ = 2;
+      pp.nsw = nsw2;
+      pp.lds = (size_t)nsw2 * wstage + patch;
+      int taps2 = RS + 2 - nsw2 < RS - 1 ? RS + 2 - nsw2 : RS - 1;
+      if (taps2 < 1) taps2 = 1;
+      pp.pls = (per_wave + taps2 - 1) / taps2;
+      if (pp.pls < 1) pp.pls = 1;
+    }
+  }
   return pp;
 }
 
@@ -211,10 +230,12 @@ static double conv_patch_estimate(const amos_conv_desc_t& c, int op, const Probl
   const int64_t T = op == AMOS_OP_CONV2D ? 1 : c.T;
   const double steps_all = (double)T * c.R * c.S * std::ceil(c.C * es / 128.0);
   const double blocks = std::ceil((double)pb.I / ti) * std::ceil((double)pb.J / tj) * split;
-  const double rounds = std::ceil(blocks / Gfx950::kComputeUnits);
+  // two resident workgroups take turns on the matrix cores while their per-step instruction
+  // overheads overlap
+  const double rounds = std::ceil(blocks / (Gfx950::kComputeUnits * (double)pp.occ));
   const double steps = std::ceil(steps_all / split);
   const double mfma_per_step = (ti / 64.0) * (tj / 64.0) * 4.0 * 32.0;
-  const double cycles = rounds * (steps * (mfma_per_step + 600.0) + 4000.0);
+  const double cycles = rounds * (steps * (pp.occ * mfma_per_step + (pp.occ == 2 ? 500.0 : 600.0)) + 4000.0);
   const double relayout = ((double)pb.in_bytes * 2.0) / 2.5e12 + 3e-6;
   return cycles / 2.1e9 + relayout + (split > 1 ? (double)pb.out_bytes * split / 1.2e12 : 0.0);
 }

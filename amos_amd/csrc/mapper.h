@@ -39,6 +39,8 @@ struct ConvPatchPlan {
   int max_seg;       // image slices a tile may touch
   int nsw;           // weight ring stages
   int pls;           // patch copies per wave per K step
+  int xbufs;         // patch buffers (1 when a block runs a single macro step)
+  int occ;           // workgroups per CU the instance is built for (2 when LDS and registers allow)
   size_t lds;        // dynamic LDS bytes of the block
 };
 int64_t conv_packed_bytes(const amos_conv_desc_t& c, int op);
