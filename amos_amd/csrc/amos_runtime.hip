@@ -270,7 +270,6 @@ static int plan_conv(Plan& pl, int op, const amos_conv_desc_t* d, const amos_ker
   const int max_pos = pp.max_pos, nsw = pp.nsw, pls = pp.pls;
   pl.conv_occ = pp.occ;
   const size_t lds = pp.lds;
-  (void)RS;
   if (why) {
     if (pipe == AMOS_PIPE_PATCH)
       return set_error(AMOS_ERR_INFEASIBLE, "patch-staged convolution not applicable: %s", why);
@@ -284,6 +283,7 @@ static int plan_conv(Plan& pl, int op, const amos_conv_desc_t* d, const amos_ker
   q.wp = (char*)workspace;
   q.zeros = (char*)workspace + packed;
   q.xt = (char*)workspace + packed + 256;
+  q.steps = (char*)workspace + packed + 256 + conv_relaid_bytes(c, op);
   q.N = (int)c.N; q.C = (int)c.C; q.D = (int)c.D; q.H = (int)c.H; q.W = (int)c.W; q.K = (int)c.K;
   q.T = (int)c.T; q.R = (int)c.R; q.S = (int)c.S;
   q.sd = c.stride_d; q.sh = c.stride_h; q.sw = c.stride_w;
@@ -296,8 +296,12 @@ static int plan_conv(Plan& pl, int op, const amos_conv_desc_t* d, const amos_ker
   q.nsw = nsw;
   q.pls = pls;
   q.xbufs = pp.xbufs;
+  q.sx_off = nsw * BI * 128;
+  q.tab_off = q.sx_off + pp.xbufs * max_pos * 128;
+  q.dump_off = q.tab_off + max_pos * 8;
   q.c_chunks = (int)(c.C * es / 128);
   q.macro_steps = (int)c.T * q.c_chunks;
+  q.total_steps = q.macro_steps * RS;
   int split = pl.cfg.split_k < 1 ? 1 : pl.cfg.split_k;
   if (split > q.macro_steps) split = q.macro_steps;
   q.macro_per_split = (q.macro_steps + split - 1) / split;
@@ -369,23 +373,29 @@ static int launch_tn(const Plan& pl, hipStream_t stream) {
   return 0;
 }
 
-static ConvInstance* pick_conv(int dt, int ti, int tj, int occ) {
-  if (dt == DT_F16) return pick_conv_f16(ti, tj, occ);
-  if (dt == DT_BF16) return pick_conv_bf16(ti, tj, occ);
-  return pick_conv_i8(ti, tj, occ);
+static ConvInstance* pick_conv(int dt, int ti, int tj, int pls, int occ) {
+  if (dt == DT_F16) return pick_conv_f16(ti, tj, pls, occ);
+  if (dt == DT_BF16) return pick_conv_bf16(ti, tj, pls, occ);
+  return pick_conv_i8(ti, tj, pls, occ);
 }
 
 static int launch_conv(const Plan& pl, hipStream_t stream) {
-  ConvInstance* inst = pick_conv(pl.dt, pl.cfg.tile_i, pl.cfg.tile_j, pl.conv_occ);
+  ConvInstance* inst = pick_conv(pl.dt, pl.cfg.tile_i, pl.cfg.tile_j, pl.cv.pls, pl.conv_occ);
   if (!inst) return set_error(AMOS_ERR_INFEASIBLE, "no patch-staged convolution instance");
   hipError_t attr_err = hipSuccess;
   std::call_once(inst->once, [&] {
     attr_err = hipFuncSetAttribute((const void*)inst->fn, hipFuncAttributeMaxDynamicSharedMemorySize,
                                    160 * 1024 - 512);
+    // the kernel addresses its dynamic LDS from byte 0
+    hipFuncAttributes fa;
+    if (attr_err == hipSuccess) attr_err = hipFuncGetAttributes(&fa, (const void*)inst->fn);
+    if (attr_err == hipSuccess && fa.sharedSizeBytes != 0) inst->static_lds = (int)fa.sharedSizeBytes;
   });
   if (attr_err != hipSuccess)
     return set_error(AMOS_ERR_HIP, "hipFuncSetAttribute(%s): %s", inst->name,
                      hipGetErrorString(attr_err));
+  if (inst->static_lds)
+    return set_error(AMOS_ERR_HIP, "%s was built with %d bytes of static LDS", inst->name, inst->static_lds);
   const ConvFpropParams& q = pl.cv;
   launch_conv_prepare(pl.dt == DT_I8 ? 1 : 2, q, stream);
   dim3 grid((unsigned)(q.tiles_i * q.tiles_j), (unsigned)pl.split, 1);
@@ -499,7 +509,7 @@ const char* amos_kernel_name(int op, const void* desc, const amos_kernel_config_
   static char dummy_ws[256] __attribute__((aligned(256)));
   if (make_plan(pl, op, desc, cfg, dummy, dummy, dummy, dummy_ws, (size_t)-1)) return nullptr;
   if (pl.conv_ups) {
-    ConvInstance* ci = pick_conv(pl.dt, pl.cfg.tile_i, pl.cfg.tile_j, pl.conv_occ);
+    ConvInstance* ci = pick_conv(pl.dt, pl.cfg.tile_i, pl.cfg.tile_j, pl.cv.pls, pl.conv_occ);
     return ci ? ci->name : nullptr;
   }
   if (pl.tn_waves) {

@@ -60,6 +60,7 @@ __device__ __forceinline__ int fast_div(int n, const FastDiv& f) {
 }
 
 #define AMOS_LDS_PTR_FROM(off) ((const __attribute__((address_space(3))) char*)(size_t)(off))
+#define AMOS_LDS_PTR_RW(off) ((__attribute__((address_space(3))) char*)(size_t)(off))
 
 struct ConvFpropParams {
   const char* x;     // original NCDHW activations (prepare kernel input)
@@ -73,10 +74,13 @@ struct ConvFpropParams {
   int OD, OP, OQ;
   int J;             // N*OD*OP*OQ
   int Wp;            // patch columns: (OQ-1)*sw + (S-1)*dw + 1
-  int max_pos;       // LDS positions reserved per patch buffer (multiple of 8)
+  int max_pos;       // LDS positions reserved per patch buffer (multiple of 64)
   int nsw;           // weight ring stages (>= 2)
-  int pls;           // patch copy instructions per wave per K step
+  int pls;           // patch copy instructions per wave per K step (the instance's PL)
   int xbufs;         // patch buffers: 2, or 1 when a block handles a single (depth tap, channel chunk)
+  int sx_off, tab_off, dump_off;   // LDS byte offsets: patch buffers, position table, dump line
+  int total_steps;   // macro_steps * R * S
+  void* steps;       // [total_steps + 1] step table (workspace), written by the prepare kernel
   int c_chunks;      // C*ES / 128
   int macro_steps;   // T * c_chunks
   int macro_per_split;
@@ -89,6 +93,54 @@ struct ConvFpropParams {
 };
 
 // ---- launch 1: relayout ---------------------------------------------------------------------
+// Step table: what differs between the K steps of amos_conv_fprop, 8 words per step
+// g = macro step * R*S + tap (macro step = (depth tap, channel chunk)):
+//   [0] byte offset, inside a packed weight row, of the tile FETCHED during step g (that of step
+//       g + nsw)            [7] the same for step g's own tile
+//   [1] LDS offset the fragments of step g+1 read their patch at (buffer + tap shift)
+//   [2] source offset of macro step m+1 from the zero block, [3] its depth shift - 32768
+//   [4] first patch copy of step g | first patch copy of step g+1 << 16
+//   [5] macro step m of g    [6] LDS offset of the patch buffer of macro step m+1
+__device__ __forceinline__ void conv_write_steps(const ConvFpropParams& p, int es, int t) {
+  const int RS = p.R * p.S, total = p.total_steps;
+  const unsigned pos_bytes = (unsigned)p.C * es;
+  const unsigned xbuf_bytes = (unsigned)p.max_pos * 128u;
+  int* const tb = (int*)p.steps;
+  auto wk_of = [&](int g) {
+    if (g > total - 1) g = total - 1;
+    const int m = g / RS, tap = g - m * RS;
+    const int tt = m / p.c_chunks, cc = m - tt * p.c_chunks;
+    return (unsigned)(tt * RS + tap) * pos_bytes + (unsigned)cc * 128u;
+  };
+  for (int g = t; g <= total; g += 256) {
+    const int gc = g < total - 1 ? g : total - 1;
+    const int m = gc / RS, tap = gc - m * RS;
+    const int g1 = g + 1 < total - 1 ? g + 1 : total - 1;
+    const int m1 = g1 / RS, tap1 = g1 - m1 * RS;
+    const int tr = tap1 / p.S, ts = tap1 - tr * p.S;
+    unsigned po = 0;
+    int pdb = -32768;
+    if (m + 1 < p.macro_steps) {
+      const int tt = (m + 1) / p.c_chunks, cc = (m + 1) - tt * p.c_chunks;
+      po = 256u + (unsigned)(tt * p.dd * p.H * p.W) * pos_bytes + (unsigned)cc * 128u;
+      pdb = tt * p.dd - 32768;
+    }
+    int v0 = tap * p.pls, v0n = (tap + 1 == RS ? 0 : tap + 1) * p.pls;
+    if (v0 > 0x7ff0) v0 = 0x7ff0;
+    if (v0n > 0x7ff0) v0n = 0x7ff0;
+    int* const e = tb + (int64_t)g * 8;
+    e[0] = (int)wk_of(g + p.nsw);
+    e[1] = (int)((unsigned)p.sx_off + (unsigned)(m1 & (p.xbufs - 1)) * xbuf_bytes +
+                 (unsigned)(tr * p.dh * p.Wp + ts * p.dw) * 128u);
+    e[2] = (int)po;
+    e[3] = pdb;
+    e[4] = v0 | (v0n << 16);
+    e[5] = m;
+    e[6] = (int)((unsigned)p.sx_off + (unsigned)((m + 1) & (p.xbufs - 1)) * xbuf_bytes);
+    e[7] = (int)wk_of(g);
+  }
+}
+
 template <typename T>
 __global__ __launch_bounds__(256) void amos_conv_prepare(const ConvFpropParams p) {
   __shared__ T tile[64][64 + 2];
@@ -110,7 +162,10 @@ __global__ __launch_bounds__(256) void amos_conv_prepare(const ConvFpropParams p
         dst[o] = src[c * TRS + tap];
       }
     }
-    if (b == 0 && t < 32) ((int*)p.zeros)[t] = 0;
+    if (b == 0) {
+      if (t < 64) ((int*)p.zeros)[t] = 0;
+      conv_write_steps(p, (int)sizeof(T), t);
+    }
     return;
   }
   b -= p.prep_w_blocks;
@@ -151,19 +206,29 @@ __global__ __launch_bounds__(256) void amos_conv_prepare(const ConvFpropParams p
 __device__ __forceinline__ void wait_vmcnt_le(int n) {
   if (n <= 0) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   else if (n < 2) asm volatile("s_waitcnt vmcnt(1)" ::: "memory");
-  else if (n < 4) asm volatile("s_waitcnt vmcnt(2)" ::: "memory");
+  else if (n < 3) asm volatile("s_waitcnt vmcnt(2)" ::: "memory");
+  else if (n < 4) asm volatile("s_waitcnt vmcnt(3)" ::: "memory");
   else if (n < 6) asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
   else if (n < 8) asm volatile("s_waitcnt vmcnt(6)" ::: "memory");
-  else if (n < 12) asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
+  else if (n < 10) asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
+  else if (n < 12) asm volatile("s_waitcnt vmcnt(10)" ::: "memory");
   else if (n < 16) asm volatile("s_waitcnt vmcnt(12)" ::: "memory");
-  else if (n < 24) asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
+  else if (n < 20) asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
+  else if (n < 24) asm volatile("s_waitcnt vmcnt(20)" ::: "memory");
   else if (n < 32) asm volatile("s_waitcnt vmcnt(24)" ::: "memory");
   else asm volatile("s_waitcnt vmcnt(32)" ::: "memory");
 }
 
 // ---- launch 2: the convolution -----------------------------------------------------------------
+// Every K step does exactly the same work, so that its body is one straight run of instructions the
+// MFMAs can overlap: PL patch copies (of the next macro step's patch; copies a wave has no use for
+// fetch zeros into a dump line), one weight tile (steps past the end re-fetch the last tile), the
+// operand fragments of the next step, the MFMAs of this one.  What differs between steps is read
+// from the step table with one scalar load a step ahead.  With all steps alike, the number of
+// copies in flight behind the tile a step waits for is the same at every step.
+//
 // OCC = workgroups the compiler must leave room for on a CU (register budget 512 / OCC per lane)
-template <int DT, int TI, int TJ, int OCC>
+template <int DT, int TI, int TJ, int PL, int OCC>
 __global__ __launch_bounds__(256, OCC) void amos_conv_fprop(const ConvFpropParams p) {
   typedef Mfma<DT> MM;
   typedef typename MM::acc_t acc_t;
@@ -173,10 +238,11 @@ __global__ __launch_bounds__(256, OCC) void amos_conv_fprop(const ConvFpropParam
   constexpr int WCH = BI / 32;    // 1 KB weight copy instructions per wave per K step
   constexpr int WSTAGE = BI * 128;
 
-  extern __shared__ __attribute__((aligned(16))) char smem[];
-  char* const sW = smem;                                            // [nsw][BI*128]
-  char* const sX = smem + (size_t)p.nsw * WSTAGE;                   // [xbufs][max_pos*128]
-  int2* const sTab = (int2*)(sX + (size_t)p.xbufs * p.max_pos * 128);   // [max_pos] position table
+  // dynamic LDS: [nsw][BI*128] weight ring | [xbufs][max_pos*128] patches (at sx_off, 8 KB
+  // multiples) | [max_pos] position table (tab_off) | 1 KB dump line (dump_off)
+  // All LDS addressing below is by byte offset from 0: the kernel has no static LDS, so its
+  // dynamic LDS starts there (the host checks the kernel's static LDS size before the first launch).
+  extern __shared__ __attribute__((aligned(1024))) char smem[];
 
   const int t = threadIdx.x;
   const int lane = t & 63;
@@ -189,13 +255,13 @@ __global__ __launch_bounds__(256, OCC) void amos_conv_fprop(const ConvFpropParam
   const int m_begin = blockIdx.y * p.macro_per_split;
   int m_end = m_begin + p.macro_per_split;
   if (m_end > p.macro_steps) m_end = p.macro_steps;
-  const int n_macro = m_end - m_begin;
   const int RS = p.R * p.S;
   const int OPQ = p.OP * p.OQ;
   const int HW = p.H * p.W;
-  const int n_steps = n_macro * RS;
+  const int n_steps = (m_end - m_begin) * RS;
   const int NSW = p.nsw;
-  const size_t xbuf_bytes = (size_t)p.max_pos * 128;
+  const unsigned xbuf_bytes = (unsigned)p.max_pos * 128u;
+  const unsigned pos_bytes = (unsigned)p.C * ES;
 
   // ---- segments of this tile (wave-uniform scalars) -------------------------------------------
   const int j_last = (bj0 + BJ - 1 < p.J ? bj0 + BJ - 1 : p.J - 1);
@@ -223,22 +289,26 @@ __global__ __launch_bounds__(256, OCC) void amos_conv_fprop(const ConvFpropParam
   const int npos = seg_pos0[kConvMaxSeg];
   const int npos8 = (npos + 7) & ~7;
 
-  // position table: {position index in NDHWC for depth tap 0, (h,w outside ? sign bit) | d0 + 32768}
-  for (int pos = t; pos < npos8; pos += 256) {
-    int g_pos0 = 0, g_pa = seg_pa[0], g_base = seg_base[0], g_d0 = seg_d0[0];
+  // position table: {byte offset of the position's channels in NDHWC at depth tap 0 (modulo 2^32;
+  // a depth shift is added before use), d0 + 32768, or 0 when (h, w) lies outside the image}
+  {
+    int2* const sTab = (int2*)(smem + p.tab_off);
+    for (int pos = t; pos < npos8; pos += 256) {
+      int g_pos0 = 0, g_pa = seg_pa[0], g_base = seg_base[0], g_d0 = seg_d0[0];
 #pragma unroll
-    for (int g = 1; g < kConvMaxSeg; ++g)
-      if (g < nseg && pos >= seg_pos0[g]) { g_pos0 = seg_pos0[g]; g_pa = seg_pa[g]; g_base = seg_base[g]; g_d0 = seg_d0[g]; }
-    const int rel = pos - g_pos0;
-    const int hr = fast_div(rel, p.fd_wp);
-    const int wc = rel - hr * p.Wp;
-    const int h = g_pa * p.sh - p.ph + hr, w = wc - p.pw;
-    const bool ok = pos < npos && (unsigned)h < (unsigned)p.H && (unsigned)w < (unsigned)p.W;
-    sTab[pos] = int2{g_base + h * p.W + w, (ok ? 0 : (int)0x80000000) | (g_d0 + 32768)};
+      for (int g = 1; g < kConvMaxSeg; ++g)
+        if (g < nseg && pos >= seg_pos0[g]) { g_pos0 = seg_pos0[g]; g_pa = seg_pa[g]; g_base = seg_base[g]; g_d0 = seg_d0[g]; }
+      const int rel = pos - g_pos0;
+      const int hr = fast_div(rel, p.fd_wp);
+      const int wc = rel - hr * p.Wp;
+      const int h = g_pa * p.sh - p.ph + hr, w = wc - p.pw;
+      const bool ok = pos < npos && (unsigned)h < (unsigned)p.H && (unsigned)w < (unsigned)p.W;
+      sTab[pos] = int2{(int)((unsigned)(g_base + h * p.W + w) * pos_bytes), ok ? g_d0 + 32768 : 0};
+    }
   }
 
   // ---- weight copy slots ---------------------------------------------------------------------
-  const int64_t w_row_bytes = (int64_t)p.T * RS * p.C * ES;
+  const unsigned w_row_bytes = (unsigned)(p.T * RS) * pos_bytes;
   unsigned w_off[WCH];
 #pragma unroll
   for (int u = 0; u < WCH; ++u) {
@@ -246,54 +316,47 @@ __global__ __launch_bounds__(256, OCC) void amos_conv_fprop(const ConvFpropParam
     const int row = q * 8 + (lane >> 3);
     const int chunk = (lane & 7) ^ ((row ^ (row >> 3)) & 7);
     const int r = bi0 + row < p.K ? bi0 + row : p.K - 1;
-    w_off[u] = (unsigned)r * (unsigned)w_row_bytes + chunk * 16;
+    w_off[u] = (unsigned)r * w_row_bytes + chunk * 16;
   }
-  // next weight tile to issue: (macro step, tap), its ring stage and its (uniform) source
-  int iw_m = m_begin, iw_tap = 0, iw_stage = 0, iw_step = 0;
-  const int64_t tap_bytes = (int64_t)p.C * ES;
-  auto macro_weight_src = [&](int m) {
-    const int tt = fast_div(m, p.fd_cc), cc = m - tt * p.c_chunks;
-    return p.wp + ((int64_t)tt * RS * tap_bytes + (int64_t)cc * 128);
-  };
-  const char* iw_src = macro_weight_src(m_begin);
-  auto issue_next_weights = [&]() {
-    char* s = sW + iw_stage * WSTAGE;
+  // weight tile whose K slice starts wk bytes into a packed weight row -> ring stage at stage_off
+  // (32-bit offsets from the packed weights: the host keeps them under 4 GiB)
+  auto issue_weights = [&](unsigned wk, unsigned stage_off) {
 #pragma unroll
     for (int u = 0; u < WCH; ++u)
-      __builtin_amdgcn_global_load_lds(AMOS_GLOBAL_PTR(iw_src + w_off[u]), AMOS_LDS_PTR(s + (wave + 4 * u) * 1024),
-                                       16, 0, 0);
-    ++iw_step;
-    iw_src += tap_bytes;
-    if (++iw_tap == RS) { iw_tap = 0; ++iw_m; iw_src = macro_weight_src(iw_m); }
-    if (++iw_stage == NSW) iw_stage = 0;
+      __builtin_amdgcn_global_load_lds(AMOS_GLOBAL_PTR(p.wp + (size_t)(w_off[u] + wk)),
+                                       AMOS_LDS_PTR_RW(stage_off + (unsigned)(wave + 4 * u) * 1024), 16, 0, 0);
   };
 
-  // ---- patch copies: instruction v of this wave fills positions [8q, 8q+8), q = wave + 4v -------
+  // ---- patch copies: copy v of this wave fills positions [8q, 8q+8), q = wave + 4v ---------------
   const int n_chunks8 = npos8 >> 3;
   const int n_pl = n_chunks8 > wave ? (n_chunks8 - wave + 3) >> 2 : 0;   // copies this wave owns per patch
-  const unsigned tab_lds = (unsigned)(size_t)AMOS_LDS_PTR(sTab) + (unsigned)(lane >> 3) * 8;
-  const int64_t pos_bytes = (int64_t)p.C * ES;
-  // patch of macro step m into buffer `buf`: uniform part of the source and the depth shift
-  auto issue_patch = [&](int m, int buf, int v) {
-    const int tt = fast_div(m, p.fd_cc), cc = m - tt * p.c_chunks;
-    const int q = wave + 4 * v;
-    // The table is read with an explicit ds_read: next to outstanding global -> LDS copies
-    // the compiler would otherwise wait for all of them before any LDS load it cannot
-    // tell apart from their destinations.
+  const unsigned tab_lane = (unsigned)p.tab_off + (unsigned)(lane >> 3) * 8;
+  // 16-byte chunk a lane fetches: the swizzle of the LDS position it fills (8 KB-aligned buffers)
+  const unsigned lane_c16 = (unsigned)((lane & 7) ^ (lane >> 3)) << 4;
+  // The table is read with an explicit ds_read the compiler does not see as a memory access: next
+  // to outstanding global -> LDS copies it would otherwise wait for all of them before an LDS
+  // load it cannot tell apart from their destinations.  The caller waits (lgkmcnt) before use.
+  auto read_tab = [&](int v) {
+    int vq = v < n_pl - 1 ? v : n_pl - 1;
+    if (vq < 0) vq = 0;
     int2 e;
-    asm volatile("ds_read_b64 %0, %1\n\ts_waitcnt lgkmcnt(0)" : "=v"(e) : "v"(tab_lds + (unsigned)q * 64) : "memory");
-    const int pos = q * 8 + (lane >> 3);
-    const int d = (e.y & 0xffff) - 32768 + tt * p.dd;
-    const bool ok = e.y >= 0 && (unsigned)d < (unsigned)p.D;
-    const int chunk = (lane & 7) ^ ((pos ^ (pos >> 3)) & 7);
-    const char* base = p.xt + ((int64_t)tt * p.dd * HW * pos_bytes + (int64_t)cc * 128);
-    const char* src = ok ? base + ((int64_t)e.x * pos_bytes + chunk * 16) : p.zeros + chunk * 16;
-    char* dst = sX + (size_t)buf * xbuf_bytes + q * 1024;
-    __builtin_amdgcn_global_load_lds(AMOS_GLOBAL_PTR(src), AMOS_LDS_PTR(dst), 16, 0, 0);
+    asm volatile("ds_read_b64 %0, %1" : "=v"(e) : "v"(tab_lane + (unsigned)(wave + 4 * vq) * 64));
+    return e;
   };
+  // one copy: table entry e of the lane's position; po = the macro step's uniform source offset
+  // from the zero block, pdb = its depth shift - 32768, cq = the lane's chunk for the LDS line
+  // being filled; depth_limit = D, or 0 for a copy that only moves zeros
+  auto patch_copy = [&](int2 e, unsigned cq, unsigned po, int pdb, unsigned dst_off, unsigned depth_limit) {
+    const int d = e.y + pdb;
+    const unsigned src = (unsigned)e.x + po + cq;
+    const unsigned voff = (unsigned)d < depth_limit ? src : cq;
+    __builtin_amdgcn_global_load_lds(AMOS_GLOBAL_PTR(p.zeros + (size_t)voff), AMOS_LDS_PTR_RW(dst_off), 16, 0, 0);
+  };
+  // q & 7 = (wave & 3) + 4 * (v & 1): two chunk patterns per lane
+  const unsigned lane_cq[2] = {lane_c16 ^ ((unsigned)wave << 4), lane_c16 ^ ((unsigned)(wave + 4) << 4)};
 
   // ---- this lane's output columns -> patch positions ---------------------------------------------
-  int col_pos[TJ];
+  unsigned col_byte[TJ];
 #pragma unroll
   for (int b = 0; b < TJ; ++b) {
     int j = bj0 + (wj * TJ + b) * 32 + frag_row;
@@ -304,7 +367,7 @@ __global__ __launch_bounds__(256, OCC) void amos_conv_fprop(const ConvFpropParam
 #pragma unroll
     for (int g = 1; g < kConvMaxSeg; ++g)
       if (sl - sl_a == g) { g_pos0 = seg_pos0[g]; g_pa = seg_pa[g]; }
-    col_pos[b] = g_pos0 + (op - g_pa) * p.sh * p.Wp + oq * p.sw;
+    col_byte[b] = (unsigned)(g_pos0 + (op - g_pa) * p.sh * p.Wp + oq * p.sw) * 128u;
   }
   // LDS byte offsets: weights by (parity of the 32-row tile, sub-step), the lane's chunk per sub-step
   unsigned a_off[2][4], kh[4];
@@ -313,10 +376,8 @@ __global__ __launch_bounds__(256, OCC) void amos_conv_fprop(const ConvFpropParam
     kh[ks] = (unsigned)(ks * 2 + frag_half) << 4;
 #pragma unroll
     for (int par = 0; par < 2; ++par)
-      a_off[par][ks] = (unsigned)(size_t)AMOS_LDS_PTR(sW) +
-                       lds_chunk_offset(wi * TI * 32 + par * 32 + frag_row, ks * 2 + frag_half);
+      a_off[par][ks] = (unsigned)lds_chunk_offset(wi * TI * 32 + par * 32 + frag_row, ks * 2 + frag_half);
   }
-  const unsigned x_lds = (unsigned)(size_t)AMOS_LDS_PTR(sX);
 
   acc_t acc[TI][TJ];
 #pragma unroll
@@ -329,13 +390,13 @@ __global__ __launch_bounds__(256, OCC) void amos_conv_fprop(const ConvFpropParam
   // Operand fragments of a whole K step (4 sub-steps) are read one step ahead: with wave tiles
   // this small, the MFMAs of one sub-step are too few to cover the LDS latency of the next.
   v4i af[2][4][TI], bf[2][4][TJ];
-  auto read_step = [&](unsigned wstage_off, unsigned xbuf_lds, int dpos, int slot) {
+  // xo: LDS offset of the patch buffer plus the tap's shift, 128 bytes per position
+  auto read_step = [&](unsigned wstage_off, unsigned xo, int slot) {
     unsigned xb[TJ], xsw[TJ];   // per column: LDS address of its position at this tap, swizzle term
 #pragma unroll
     for (int b = 0; b < TJ; ++b) {
-      const int pos = col_pos[b] + dpos;
-      xb[b] = xbuf_lds + (unsigned)pos * 128;
-      xsw[b] = (unsigned)((pos ^ (pos >> 3)) & 7) << 4;
+      xb[b] = col_byte[b] + xo;
+      xsw[b] = ((xb[b] >> 3) ^ (xb[b] >> 6)) & 0x70;   // ((pos ^ pos >> 3) & 7) << 4, pos = byte / 128
     }
 #pragma unroll
     for (int ks = 0; ks < 4; ++ks) {
@@ -354,56 +415,131 @@ __global__ __launch_bounds__(256, OCC) void amos_conv_fprop(const ConvFpropParam
 #pragma unroll
         for (int b = 0; b < TJ; ++b) acc[a][b] = MM::run(af[slot][ks][a], bf[slot][ks][b], acc[a][b]);
   };
-  // wait until at most `later` weight tiles (the youngest) are still in flight
-  auto wait_weights = [&](int later) {
-    if (later >= 2) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * WCH) : "memory");
-    else if (later == 1) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(WCH) : "memory");
-    else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-  };
+
+  // step table, read with scalar loads
+  typedef int v8i_t __attribute__((ext_vector_type(8)));
+  const __attribute__((address_space(4))) v8i_t* const tbl =
+      (const __attribute__((address_space(4))) v8i_t*)p.steps;
+  int g = m_begin * RS;   // table index of the current step
+  int2 pt[PL > 0 ? PL : 1];   // table entries of the patch copies of the coming step
 
   // ---- prologue: the whole first patch, the first NSW weight tiles -------------------------------
   __syncthreads();   // position table visible
+  v8i_t cur = tbl[g];
   if (n_steps > 0) {
-    for (int v = 0; v < n_pl; ++v) issue_patch(m_begin, 0, v);
-    while (iw_step < NSW && iw_step < n_steps) issue_next_weights();
-    wait_weights(iw_step - 1);   // patch and tile 0 landed (NSW <= 4: never more than 3 later tiles)
-    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
-    read_step(0, x_lds, 0, 0);
+    {
+      const int tt = fast_div(m_begin, p.fd_cc), cc = m_begin - tt * p.c_chunks;
+      const unsigned po = 256u + (unsigned)(tt * p.dd * HW) * pos_bytes + (unsigned)cc * 128u;
+      const unsigned buf = (unsigned)p.sx_off + (unsigned)(m_begin & (p.xbufs - 1)) * xbuf_bytes;
+      for (int v = 0; v < n_pl; ++v) {
+        const int q = wave + 4 * v;
+        int2 e = read_tab(v);
+        asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(e));
+        patch_copy(e, lane_cq[v & 1], po, tt * p.dd - 32768, buf + (unsigned)q * 1024, (unsigned)p.D);
+      }
+      // tile u, each later one behind as many (dummy) patch copies as a step issues ahead of its tile
+      const unsigned last = (unsigned)(p.total_steps - 1);
+      for (int u = 0; u < NSW; ++u) {
+        if (u > 0)
+#pragma unroll
+          for (int x = 0; x < PL; ++x) patch_copy(int2{0, 0}, lane_cq[0], 0u, 0, (unsigned)p.dump_off, 0u);
+        const unsigned gu = (unsigned)(g + u) < last ? (unsigned)(g + u) : last;
+        issue_weights((unsigned)tbl[gu][7], (unsigned)u * WSTAGE);
+      }
+      wait_vmcnt_le((NSW - 1) * (PL + WCH));   // first patch and tile 0 landed
+      asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+      read_step(0, buf, 0);
+#pragma unroll
+      for (int x = 0; x < PL; ++x) pt[x] = read_tab(x);
+    }
   }
 
-  // current K step: macro step index mi (of this block), tap = (tr, ts), ring stage
-  int mi = 0, tap = 0, tr = 0, ts = 0, stage = 0;
-  auto one_step = [&](int step, int slot) {
-    // This wave's reads of the current step's operands (issued a step ago) and its copies of the
-    // next weight tile are complete; after the barrier that holds for every wave: the next tile
-    // (and, past a patch's last tap, the next patch) may be read, the current stage overwritten.
-    wait_weights(iw_step - (step + 2));   // weight tiles issued after tile step+1
-    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
-    // Patch of the next (depth tap, channel chunk): a few copies per step on the early taps,
-    // issued BEFORE this step's weight tile so that they are older than a tile that is
-    // waited for before the patch is first read.
-    if (mi + 1 < n_macro && tap * p.pls < n_pl) {
-      const int v_end = (tap + 1) * p.pls < n_pl ? (tap + 1) * p.pls : n_pl;
-      for (int v = tap * p.pls; v < v_end; ++v) issue_patch(m_begin + mi + 1, (mi + 1) & (p.xbufs - 1), v);
-    }
-    if (iw_step < n_steps) issue_next_weights();   // tile step+NSW into the stage just freed
-    // operands of the next K step, then the MFMAs of this one
-    ++tap;
-    if (++ts == p.S) { ts = 0; ++tr; }
-    if (tap == RS) { tap = 0; tr = 0; ++mi; }
-    if (++stage == NSW) stage = 0;
-    if (step + 1 < n_steps)
-      read_step((unsigned)stage * WSTAGE, x_lds + (unsigned)(mi & (p.xbufs - 1)) * (unsigned)xbuf_bytes,
-                tr * p.dh * p.Wp + ts * p.dw, slot ^ 1);
+  // cur = {wk of the tile fetched during this step, xo of the NEXT step's fragments, po and pdb of
+  //        the next macro step, v0 | v0 of the next step << 16, macro step, LDS offset of the next
+  //        macro step's patch buffer, wk of this step's own tile}
+  unsigned istage = 0;   // ring stage (byte offset) this step's fetch goes to = the stage step-1 read
+  v8i_t nxt = cur;
+#ifdef AMOS_CONV_TIMING
+  unsigned long long tacc[3] = {0, 0, 0}, tC = 0;
+  auto now = [] { unsigned long long tt; asm volatile("s_memtime %0\n\ts_waitcnt lgkmcnt(0)" : "=s"(tt)::"memory"); return tt; };
+  tC = now();
+  const unsigned long long tstart = tC;
+#endif
+  auto one_step = [&](int slot, const v8i_t& e, v8i_t& e_next) {
+#ifdef AMOS_CONV_TIMING
+    const unsigned long long tA = now();
+    tacc[0] += tA - tC;
+#endif
+    // This wave's reads of the current step's operands (issued a step ago) are complete, and so
+    // are its copies of everything older than the youngest NSW-2 steps' worth: the next weight
+    // tile and, at a macro step's last tap, the next patch.  After the barrier that holds for
+    // every wave.
+    if (NSW >= 4) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * (PL + WCH)) : "memory");
+    else if (NSW == 3) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(PL + WCH) : "memory");
+    else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+#ifdef AMOS_CONV_TIMING
+    const unsigned long long tB = now();
+    tacc[1] += tB - tA;
+#endif
+    // (the table entries read a step ago are tied to the wait, so that nothing uses them before it)
+    if (PL == 4)
+      asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" : "+v"(pt[0]), "+v"(pt[1]), "+v"(pt[PL > 2 ? 2 : 0]), "+v"(pt[PL > 2 ? 3 : 0])::"memory");
+    else if (PL == 2)
+      asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" : "+v"(pt[0]), "+v"(pt[PL > 1 ? 1 : 0])::"memory");
+    else
+      asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+#ifdef AMOS_CONV_TIMING
+    tC = now();
+    tacc[2] += tC - tB;
+#endif
+    // (every word of the entry stays live up to here: a register of the tuple that is reused
+    // earlier makes the compiler wait for the scalar load right after issuing it)
+    asm volatile("" ::"s"(e[0]), "s"(e[1]), "s"(e[2]), "s"(e[3]), "s"(e[4]), "s"(e[5]), "s"(e[6]), "s"(e[7]));
+    // operands of the next K step first: LDS is the busiest unit of a step, the MFMAs of this step
+    // (whose operands are in registers already) run while it delivers
+    const unsigned rstage = istage + WSTAGE == (unsigned)NSW * WSTAGE ? 0u : istage + WSTAGE;
+    read_step(rstage, (unsigned)e[1], slot ^ 1);
     mma_step(slot);
+    // patch of the next (depth tap, channel chunk): BEFORE this step's weight tile, so that the
+    // copies are older than a tile that is waited for before the patch is first read
+    if (PL > 0) {
+      const int n_live = e[5] + 1 < m_end ? n_pl : 0;
+      const int v0 = e[4] & 0xffff;   // even: copies per step come in twos
+      const unsigned dst0 = (unsigned)e[6] + (unsigned)wave * 1024 + (unsigned)v0 * 4096;
+#pragma unroll
+      for (int x = 0; x < PL; ++x) {
+        const bool live = v0 + x < n_live;
+        patch_copy(pt[x], lane_cq[x & 1], (unsigned)e[2], e[3], live ? dst0 + x * 4096 : (unsigned)p.dump_off,
+                   live ? (unsigned)p.D : 0u);
+      }
+    }
+    issue_weights((unsigned)e[0], istage);   // tile step+NSW into the stage just freed
+    istage = rstage;
+    if (PL > 0) {
+      const int v0n = (int)((unsigned)e[4] >> 16);
+#pragma unroll
+      for (int x = 0; x < PL; ++x) pt[x] = read_tab(v0n + x);
+    }
+    // the next step's table entry, last: it has until the top of the next step to arrive
+    __builtin_amdgcn_sched_barrier(0);
+    ++g;
+    e_next = tbl[g];
   };
   int step = 0;
   for (; step + 1 < n_steps; step += 2) {
-    one_step(step, 0);
-    one_step(step + 1, 1);
+    one_step(0, cur, nxt);
+    one_step(1, nxt, cur);
   }
-  if (step < n_steps) one_step(step, 0);
+  if (step < n_steps) one_step(0, cur, nxt);
 
+#ifdef AMOS_CONV_TIMING
+  const unsigned long long tloop = now();
+  if ((blockIdx.x == 0 || blockIdx.x == 77) && blockIdx.y == 0 && t == 0) {
+    unsigned* dbg = (unsigned*)(p.zeros + 128) + (blockIdx.x ? 8 : 0);
+    dbg[0] = (unsigned)tacc[0]; dbg[1] = (unsigned)tacc[1]; dbg[2] = (unsigned)tacc[2];
+    dbg[3] = (unsigned)(tloop - tstart); dbg[4] = (unsigned)n_steps;
+  }
+#endif
   // ---- epilogue: Y[(n*K + i)*ODPQ + (od*OPQ + opq)] ---------------------------------------------
   out_t* const out = (out_t*)p.y;
   const int ODPQ = p.OD * OPQ;
@@ -435,6 +571,8 @@ __global__ __launch_bounds__(256, OCC) void amos_conv_fprop(const ConvFpropParam
       }
     }
   }
+  // the re-fetched tiles of the last steps still target this block's LDS
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 }
 
 }  // namespace amos

@@ -96,19 +96,26 @@ static void conv_patch_extent(int64_t J, int OPQ, int OQ, int BJ, int sh, int R,
   }
 }
 
-// workspace of the patch-staged pipeline: [packed weights | 256 zero bytes | NDHWC activations]
+// workspace of the patch-staged pipeline:
+// [packed weights | 256 zero bytes | NDHWC activations | step table, 32 bytes per K step + 1]
 int64_t conv_packed_bytes(const amos_conv_desc_t& c, int op) {
   int64_t T = op == AMOS_OP_CONV2D ? 1 : c.T;
   int es = c.in_dtype == AMOS_I8 ? 1 : 2;
   if (c.C <= 0 || (c.C * es) % 128 != 0) return 0;
   return (c.K * T * c.R * c.S * c.C * es + 255) / 256 * 256;
 }
+int64_t conv_relaid_bytes(const amos_conv_desc_t& c, int op) {
+  int64_t D = op == AMOS_OP_CONV2D ? 1 : c.D;
+  int es = c.in_dtype == AMOS_I8 ? 1 : 2;
+  return (c.N * c.C * D * c.H * c.W * es + 255) / 256 * 256;
+}
 int64_t conv_workspace_bytes(const amos_conv_desc_t& c, int op) {
   int64_t packed = conv_packed_bytes(c, op);
   if (packed == 0) return 0;
-  int64_t D = op == AMOS_OP_CONV2D ? 1 : c.D;
+  int64_t T = op == AMOS_OP_CONV2D ? 1 : c.T;
   int es = c.in_dtype == AMOS_I8 ? 1 : 2;
-  return packed + 256 + c.N * c.C * D * c.H * c.W * es;
+  int64_t steps = T * c.R * c.S * (c.C * es / 128);
+  return packed + 256 + conv_relaid_bytes(c, op) + (steps + 1) * 32;
 }
 
 
@@ -130,57 +137,71 @@ ConvPatchPlan conv_patch_plan(const amos_conv_desc_t& cin, int op, int BI, int B
   if (OD <= 0 || OP <= 0 || OQ <= 0) { pp.why = "empty output"; return pp; }
   if (packed == 0) { pp.why = "C * element size is not a multiple of 128 bytes"; return pp; }
   if (packed >= ((int64_t)1 << 32)) { pp.why = "packed weights above 4 GiB"; return pp; }
+  if (conv_relaid_bytes(c, op) + 256 >= ((int64_t)1 << 32)) { pp.why = "activations above 4 GiB"; return pp; }
   if (c.N * c.D * c.H * c.W >= ((int64_t)1 << 31) || J >= ((int64_t)1 << 31) - 512) {
     pp.why = "more than 2^31 input or output positions";
     return pp;
   }
   if (c.D + 2 * (int64_t)c.pad_d + c.T * c.dil_d >= 30000) { pp.why = "depth extent above 30000"; return pp; }
   if (!tile_ok) { pp.why = "no patch-staged instance with this block tile"; return pp; }
-  int max_pos = 0, max_seg = 0;
-  conv_patch_extent(J, (int)(OP * OQ), (int)OQ, BJ, c.stride_h, (int)c.R, c.dil_h, Wp, &max_pos, &max_seg);
-  max_pos = (max_pos + 7) & ~7;
+  int real_pos = 0, max_seg = 0;
+  conv_patch_extent(J, (int)(OP * OQ), (int)OQ, BJ, c.stride_h, (int)c.R, c.dil_h, Wp, &real_pos, &max_seg);
+  real_pos = (real_pos + 7) & ~7;
+  // patch buffers start at multiples of 8 KB, so that the LDS swizzle of a position can be
+  // taken from its address
+  const int max_pos = (real_pos + 63) & ~63;
   const size_t budget = (size_t)160 * 1024 - 512;
   const int64_t macro_steps = c.T * (c.C * es / 128);
   const int split = split_k < 1 ? 1 : split_k;
   const bool one_macro = (macro_steps + split - 1) / split <= 1;   // no next patch at all
   pp.xbufs = one_macro ? 1 : 2;
-  const size_t patch = (size_t)pp.xbufs * max_pos * 128 + (size_t)max_pos * 8;
+  // patch buffers, position table, dump line
+  const size_t patch = (size_t)pp.xbufs * max_pos * 128 + (size_t)max_pos * 8 + 1024;
   const size_t wstage = (size_t)BI * 128;
   pp.max_pos = max_pos;
   pp.max_seg = max_seg;
   if (max_seg > kConvMaxSegHost) { pp.why = "a tile spans more than 4 image slices"; return pp; }
   if (max_pos >= 4096) { pp.why = "input patch of a tile has 4096 or more positions"; return pp; }
   if (patch + 2 * wstage > budget) { pp.why = "input patch of a tile does not fit LDS"; return pp; }
-  int nsw = (int)((budget - patch) / wstage);
-  if (nsw > 4) nsw = 4;   // the kernel's wait accounting covers up to two tiles in flight behind the next
-  if (nsw > RS + 1) nsw = RS + 1;
-  // The next patch is copied during the taps of the current one.  A copy issued on tap u is
-  // complete for everybody at the barrier of the patch's last tap only if u <= RS-2 and it is
-  // older than the weight tiles still allowed in flight there: u <= RS+1-nsw.
-  int taps = RS + 2 - nsw < RS - 1 ? RS + 2 - nsw : RS - 1;
-  if (taps < 1 && !one_macro) { pp.why = "1x1 window with several channel chunks per block"; return pp; }
-  if (taps < 1) taps = 1;
-  const int per_wave = ((max_pos / 8) + 3) / 4;
-  pp.pls = (per_wave + taps - 1) / taps;
-  if (pp.pls < 1) pp.pls = 1;
-  pp.nsw = nsw;
-  pp.lds = (size_t)nsw * wstage + patch;
+  const int per_wave = ((real_pos / 8) + 3) / 4;   // patch copies of the busiest wave
+  // Ring depth and patch copies per step for an LDS budget.  The next patch is copied during the
+  // taps of the current one; a copy issued on tap u has landed for everybody at the barrier of
+  // the patch's last tap only if it is older than the nsw-2 steps' worth of copies still allowed
+  // in flight there: u <= RS - nsw.  Kernel instances exist for 0, 2 and 4 copies per step.
+  auto fit = [&](size_t lds_budget, int* nsw_out, int* pls_out) -> const char* {
+    if (patch + 2 * wstage > lds_budget) return "input patch of a tile does not fit LDS";
+    int nsw = (int)((lds_budget - patch) / wstage);
+    if (nsw > 4) nsw = 4;
+    if (nsw > RS + 1) nsw = RS + 1;
+    if (nsw < 2) nsw = 2;
+    if (one_macro) { *nsw_out = nsw; *pls_out = 0; return nullptr; }
+    for (; nsw >= 2; --nsw) {
+      const int taps = RS + 1 - nsw;
+      if (taps < 1) continue;
+      const int pls = (per_wave + taps - 1) / taps;
+      if (pls > 4) continue;
+      *nsw_out = nsw;
+      *pls_out = pls <= 2 ? 2 : 4;
+      return nullptr;
+    }
+    return RS == 1 ? "1x1 window with several channel chunks per block"
+                   : "input patch too large to prefetch behind the window's taps";
+  };
+  pp.why = fit(budget, &pp.nsw, &pp.pls);
+  if (pp.why) return pp;
+  pp.lds = (size_t)pp.nsw * wstage + patch;
   pp.occ = 1;
   // two workgroups per CU when both fit: 80 KB of LDS each, accumulators + two steps of operand
   // fragments within 256 registers (tiles up to 128x128); pointless when every block already has
   // a CU to itself
   const int64_t blocks = ((c.K + BI - 1) / BI) * ((J + BJ - 1) / BJ) * split;
   if (BI <= 128 && BJ <= 128 && blocks > Gfx950::kComputeUnits) {
-    int nsw2 = nsw;
-    while (nsw2 > 2 && (size_t)nsw2 * wstage + patch > (size_t)79 * 1024) --nsw2;
-    if ((size_t)nsw2 * wstage + patch <= (size_t)79 * 1024) {
+    int nsw2 = 0, pls2 = 0;
+    if (!fit((size_t)79 * 1024, &nsw2, &pls2)) {
       pp.occ = 2;
       pp.nsw = nsw2;
+      pp.pls = pls2;
       pp.lds = (size_t)nsw2 * wstage + patch;
-      int taps2 = RS + 2 - nsw2 < RS - 1 ? RS + 2 - nsw2 : RS - 1;
-      if (taps2 < 1) taps2 = 1;
-      pp.pls = (per_wave + taps2 - 1) / taps2;
-      if (pp.pls < 1) pp.pls = 1;
     }
   }
   return pp;

@@ -35,15 +35,16 @@ int problem_of(int op, const void* desc, Problem* out);
 constexpr int kConvMaxSegHost = 4;
 struct ConvPatchPlan {
   const char* why;   // nullptr = applicable, else the reason it is not
-  int max_pos;       // LDS positions per patch buffer (multiple of 8)
+  int max_pos;       // LDS positions per patch buffer (multiple of 64)
   int max_seg;       // image slices a tile may touch
   int nsw;           // weight ring stages
-  int pls;           // patch copies per wave per K step
+  int pls;           // patch copies per wave per K step: 0 (single macro step), 2 or 4
   int xbufs;         // patch buffers (1 when a block runs a single macro step)
   int occ;           // workgroups per CU the instance is built for (2 when LDS and registers allow)
   size_t lds;        // dynamic LDS bytes of the block
 };
 int64_t conv_packed_bytes(const amos_conv_desc_t& c, int op);
+int64_t conv_relaid_bytes(const amos_conv_desc_t& c, int op);
 int64_t conv_workspace_bytes(const amos_conv_desc_t& c, int op);
 ConvPatchPlan conv_patch_plan(const amos_conv_desc_t& c, int op, int BI, int BJ, int split_k);
 
