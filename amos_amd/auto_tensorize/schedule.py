@@ -104,7 +104,7 @@ def mapping_of_pipeline(match_result, pipeline):
     names = {ia.var.name: [t.var.name for t in lst] for ia, lst in match_result.axis_map.items()}
     rk_key = [k for k in names if k.startswith("r")][0]
     n_points = len(names[rk_key])
-    if pipeline == _lib.AMOS_PIPE_PATCH:
+    if pipeline in (_lib.AMOS_PIPE_PATCH, _lib.AMOS_PIPE_PATCH8):
         first = names[rk_key][0]      # the channel axis sorts first among reduce axes (rc < rd < rr < rs)
         return [1 if names[rk_key][p] == first else 0 for p in range(n_points)]
     return [1] * n_points
@@ -207,7 +207,7 @@ class MI355XScheduleGenerator(object):
             add(KernelParams(d.tile_i, d.tile_j, d.split_k, 0))
         is_conv = low.kind in ("conv2d", "conv3d")
         pipes = pipelines if pipelines is not None else (
-            [_lib.AMOS_PIPE_PATCH, _lib.AMOS_PIPE_STAGED] if is_conv else [_lib.AMOS_PIPE_AUTO, _lib.AMOS_PIPE_STAGED])
+            [_lib.AMOS_PIPE_PATCH, _lib.AMOS_PIPE_PATCH8, _lib.AMOS_PIPE_STAGED] if is_conv else [_lib.AMOS_PIPE_AUTO, _lib.AMOS_PIPE_STAGED])
         for pipe in pipes:
             for ti, tj in _TILES:
                 for split in (1, 2, 4, 8):

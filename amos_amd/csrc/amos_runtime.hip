@@ -70,6 +70,7 @@ struct Plan {
   ConvFpropParams cv;
   size_t conv_lds;
   int conv_occ;
+  int conv_waves;
 };
 
 static int dtype_pair(int in_dtype, int out_dtype, int* dt) {
@@ -263,15 +264,17 @@ static int plan_conv(Plan& pl, int op, const amos_conv_desc_t* d, const amos_ker
   const int64_t need_ws = conv_workspace_bytes(c, op);
   const int RS = (int)(c.R * c.S);
   const int Wp = (OQ - 1) * c.stride_w + ((int)c.S - 1) * c.dil_w + 1;
-  ConvPatchPlan pp = conv_patch_plan(c, op, BI, BJ, pl.cfg.split_k);
+  ConvPatchPlan pp = conv_patch_plan(c, op, BI, BJ, pl.cfg.split_k,
+                                     pipe == AMOS_PIPE_PATCH ? 4 : pipe == AMOS_PIPE_PATCH8 ? 8 : 0);
   const char* why = pp.why;
   if (!why && (!workspace || ws_bytes < (size_t)need_ws || ((uintptr_t)workspace & 255)))
     why = "workspace smaller than amos_workspace_bytes() or not 256-byte aligned";
   const int max_pos = pp.max_pos, nsw = pp.nsw, pls = pp.pls;
   pl.conv_occ = pp.occ;
+  pl.conv_waves = pp.waves;
   const size_t lds = pp.lds;
   if (why) {
-    if (pipe == AMOS_PIPE_PATCH)
+    if (pipe == AMOS_PIPE_PATCH || pipe == AMOS_PIPE_PATCH8)
       return set_error(AMOS_ERR_INFEASIBLE, "patch-staged convolution not applicable: %s", why);
     return 0;   // register-staged implicit GEMM handles it
   }
@@ -319,9 +322,9 @@ static int plan_conv(Plan& pl, int op, const amos_conv_desc_t* d, const amos_ker
   q.fd_cc = make_fast_div((uint32_t)q.c_chunks);
   q.fd_c = make_fast_div((uint32_t)c.C);
   const int64_t welems = c.K * c.T * c.R * c.S * c.C;
-  (void)welems;
-  q.prep_w_blocks = (int)(c.K < 1024 ? c.K : 1024);
-  q.prep_x_blocks = (int)(c.N * c.D * (((int64_t)c.H * c.W + 63) / 64) * (c.C / 64));
+  q.fd_slab = make_fast_div((uint32_t)(c.C * c.T * c.R * c.S));
+  q.prep_w_blocks = (int)((welems + 1023) / 1024 < 2048 ? (welems + 1023) / 1024 : 2048);
+  q.prep_x_blocks = (int)(c.N * c.D * (((int64_t)c.H * c.W + 63) / 64) * (c.C * es / 128));
   q.prep_z_blocks = q.zero_words ? (int)((q.zero_words + 4095) / 4096 < 2048 ? (q.zero_words + 4095) / 4096 : 2048) : 0;
   return 0;
 }
@@ -373,14 +376,14 @@ static int launch_tn(const Plan& pl, hipStream_t stream) {
   return 0;
 }
 
-static ConvInstance* pick_conv(int dt, int ti, int tj, int pls, int occ) {
-  if (dt == DT_F16) return pick_conv_f16(ti, tj, pls, occ);
-  if (dt == DT_BF16) return pick_conv_bf16(ti, tj, pls, occ);
-  return pick_conv_i8(ti, tj, pls, occ);
+static ConvInstance* pick_conv(int dt, int ti, int tj, int waves, int pls, int occ) {
+  if (dt == DT_F16) return pick_conv_f16(ti, tj, waves, pls, occ);
+  if (dt == DT_BF16) return pick_conv_bf16(ti, tj, waves, pls, occ);
+  return pick_conv_i8(ti, tj, waves, pls, occ);
 }
 
 static int launch_conv(const Plan& pl, hipStream_t stream) {
-  ConvInstance* inst = pick_conv(pl.dt, pl.cfg.tile_i, pl.cfg.tile_j, pl.cv.pls, pl.conv_occ);
+  ConvInstance* inst = pick_conv(pl.dt, pl.cfg.tile_i, pl.cfg.tile_j, pl.conv_waves, pl.cv.pls, pl.conv_occ);
   if (!inst) return set_error(AMOS_ERR_INFEASIBLE, "no patch-staged convolution instance");
   hipError_t attr_err = hipSuccess;
   std::call_once(inst->once, [&] {
@@ -399,7 +402,7 @@ static int launch_conv(const Plan& pl, hipStream_t stream) {
   const ConvFpropParams& q = pl.cv;
   launch_conv_prepare(pl.dt == DT_I8 ? 1 : 2, q, stream);
   dim3 grid((unsigned)(q.tiles_i * q.tiles_j), (unsigned)pl.split, 1);
-  hipLaunchKernelGGL(inst->fn, grid, dim3(256), pl.conv_lds, stream, q);
+  hipLaunchKernelGGL(inst->fn, grid, dim3(inst->threads), pl.conv_lds, stream, q);
   HIP_TRY(hipGetLastError());
   return 0;
 }
@@ -509,7 +512,7 @@ const char* amos_kernel_name(int op, const void* desc, const amos_kernel_config_
   static char dummy_ws[256] __attribute__((aligned(256)));
   if (make_plan(pl, op, desc, cfg, dummy, dummy, dummy, dummy_ws, (size_t)-1)) return nullptr;
   if (pl.conv_ups) {
-    ConvInstance* ci = pick_conv(pl.dt, pl.cfg.tile_i, pl.cfg.tile_j, pl.cv.pls, pl.conv_occ);
+    ConvInstance* ci = pick_conv(pl.dt, pl.cfg.tile_i, pl.cfg.tile_j, pl.conv_waves, pl.cv.pls, pl.conv_occ);
     return ci ? ci->name : nullptr;
   }
   if (pl.tn_waves) {

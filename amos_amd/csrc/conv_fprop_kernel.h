@@ -86,7 +86,7 @@ struct ConvFpropParams {
   int macro_per_split;
   int tiles_i, tiles_j;
   int atomic_out;
-  FastDiv fd_opq, fd_oq, fd_od, fd_wp, fd_odpq, fd_cc, fd_c;   // divisions by OP*OQ, OQ, OD, Wp, OD*OP*OQ, c_chunks, C
+  FastDiv fd_opq, fd_oq, fd_od, fd_wp, fd_odpq, fd_cc, fd_c, fd_slab;   // divisions by OP*OQ, OQ, OD, Wp, OD*OP*OQ, c_chunks, C, C*T*R*S
   // prepare kernel work split (in blocks)
   int prep_w_blocks, prep_x_blocks, prep_z_blocks;
   int64_t zero_words;
@@ -143,24 +143,33 @@ __device__ __forceinline__ void conv_write_steps(const ConvFpropParams& p, int e
 
 template <typename T>
 __global__ __launch_bounds__(256) void amos_conv_prepare(const ConvFpropParams p) {
-  __shared__ T tile[64][64 + 2];
+  __shared__ __attribute__((aligned(16))) T tile[64][128 / sizeof(T) + 8 / sizeof(T)];
   const int t = threadIdx.x;
   int b = blockIdx.x;
   const int TRS = p.T * p.R * p.S;
   if (b < p.prep_w_blocks) {
-    // wp[k][tap][c] = w[k][c][tap]: one block per output channel k (grid-strided); the
-    // k-th slab of C*TRS elements is read contiguously into LDS-free registers by walking the
-    // OUTPUT order (writes coalesce, reads stay inside one 1-2 KB slab that L1 holds)
+    // wp[k][tap][c] = w[k][c][tap], walking the OUTPUT order (writes coalesce, the gathered
+    // reads of a wave stay inside one channel's C*TRS slab); four independent elements per
+    // thread so that the loads overlap
     const T* w = (const T*)p.w;
     T* wp = (T*)p.wp;
     const int slab = p.C * TRS;
-    for (int k = b; k < p.K; k += p.prep_w_blocks) {
-      const T* src = w + (int64_t)k * slab;
-      T* dst = wp + (int64_t)k * slab;
-      for (int o = t; o < slab; o += 256) {
+    const int64_t total = (int64_t)p.K * slab;
+    for (int64_t base = (int64_t)b * 1024; base < total; base += (int64_t)p.prep_w_blocks * 1024) {
+      T v[4];
+      int64_t of[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        of[u] = base + t + 256 * u;
+        const int64_t oc = of[u] < total ? of[u] : total - 1;
+        const int k = fast_div((int)oc, p.fd_slab);   // the host keeps the packed weights under 2^31 elements
+        const int o = (int)(oc - (int64_t)k * slab);
         const int tap = fast_div(o, p.fd_c), c = o - tap * p.C;
-        dst[o] = src[c * TRS + tap];
+        v[u] = w[(int64_t)k * slab + c * TRS + tap];
       }
+#pragma unroll
+      for (int u = 0; u < 4; ++u)
+        if (of[u] < total) wp[of[u]] = v[u];
     }
     if (b == 0) {
       if (t < 64) ((int*)p.zeros)[t] = 0;
@@ -170,28 +179,49 @@ __global__ __launch_bounds__(256) void amos_conv_prepare(const ConvFpropParams p
   }
   b -= p.prep_w_blocks;
   if (b < p.prep_x_blocks) {
-    // xt[slice][s][c] = x[n][c][d][s] through a 64(c) x 64(s) LDS tile
+    // xt[slice][s][c] = x[n][c][d][s] through an LDS tile of 128 bytes of channels x 64
+    // positions, moved 8 bytes per lane on both sides where the rows of x are 8-byte aligned
+    constexpr int ES = (int)sizeof(T);
+    constexpr int CT = 128 / ES;          // channels per tile
+    constexpr int VE = 8 / ES;            // elements per 8-byte access
+    constexpr int PITCH = CT + VE;        // LDS row (one position) in elements: 136 bytes
+    constexpr int LTR = 64 / VE;          // loading threads per channel row
+    constexpr int LROWS = 256 / LTR;      // channel rows per pass
+    T* const tl = &tile[0][0];
+    static_assert(sizeof(tile) >= (size_t)64 * PITCH * ES, "transpose tile");
     const int HW = p.H * p.W;
-    const int s_tiles = (HW + 63) / 64, c_tiles = p.C / 64;
+    const int s_tiles = (HW + 63) / 64, c_tiles = p.C / CT;
     const int per_slice = s_tiles * c_tiles;
     const int slice = b / per_slice;
     const int rem = b - slice * per_slice;
     const int st = rem / c_tiles, ct = rem - st * c_tiles;
     const int n = slice / p.D, d = slice - n * p.D;
-    const int tx = t & 63, ty = t >> 6;
     const T* x = (const T*)p.x;
     T* xt = (T*)p.xt;
-    const int s = st * 64 + tx;
+    const bool vec = ((((uintptr_t)x) | (uintptr_t)((int64_t)HW * ES)) & 7) == 0;
+    const int ls = (t % LTR) * VE, lc = t / LTR;   // this thread's positions / channel row in a pass
 #pragma unroll
-    for (int r = 0; r < 16; ++r) {
-      const int c = ct * 64 + ty + 4 * r;
-      if (s < HW) tile[ty + 4 * r][tx] = x[(((int64_t)n * p.C + c) * p.D + d) * HW + s];
+    for (int r = 0; r < CT / LROWS; ++r) {
+      const int cl = lc + LROWS * r;
+      const int sg = st * 64 + ls;
+      const T* src = x + ((((int64_t)n * p.C + ct * CT + cl) * p.D + d) * HW + sg);
+      T v[VE];
+      if (vec && sg + VE <= HW) {
+        *(uint2*)v = *(const uint2*)src;
+      } else {
+#pragma unroll
+        for (int e = 0; e < VE; ++e) v[e] = sg + e < HW ? src[e] : (T)0;
+      }
+#pragma unroll
+      for (int e = 0; e < VE; ++e) tl[(ls + e) * PITCH + cl] = v[e];
     }
     __syncthreads();
+    const int oc = (t % 16) * VE, os = t / 16;   // 16 lanes x 8 bytes = one position's 128 bytes
 #pragma unroll
-    for (int r = 0; r < 16; ++r) {
-      const int so = st * 64 + ty + 4 * r;
-      if (so < HW) xt[((int64_t)slice * HW + so) * p.C + ct * 64 + tx] = tile[tx][ty + 4 * r];
+    for (int r = 0; r < 4; ++r) {
+      const int sl = os + 16 * r, so = st * 64 + sl;
+      if (so < HW)
+        *(uint2*)(xt + ((int64_t)slice * HW + so) * p.C + ct * CT + oc) = *(const uint2*)(tl + sl * PITCH + oc);
     }
     return;
   }
@@ -228,14 +258,22 @@ __device__ __forceinline__ void wait_vmcnt_le(int n) {
 // copies in flight behind the tile a step waits for is the same at every step.
 //
 // OCC = workgroups the compiler must leave room for on a CU (register budget 512 / OCC per lane)
-template <int DT, int TI, int TJ, int PL, int OCC>
-__global__ __launch_bounds__(256, OCC) void amos_conv_fprop(const ConvFpropParams p) {
+//
+// BI64 x BJ64 = block tile in units of 64; NW = 4 or 8 waves.  A SIMD issues one instruction of a
+// wave every ~4 cycles, and a step of a small wave tile is ~100 instructions around a handful of
+// MFMAs: with 8 waves a SIMD holds two instruction streams and interleaves them.
+template <int DT, int BI64, int BJ64, int NW, int PL, int OCC>
+__global__ __launch_bounds__(64 * NW, OCC) void amos_conv_fprop(const ConvFpropParams p) {
   typedef Mfma<DT> MM;
   typedef typename MM::acc_t acc_t;
   typedef typename MM::out_t out_t;
   constexpr int ES = MM::ES;
-  constexpr int BI = 64 * TI, BJ = 64 * TJ;
-  constexpr int WCH = BI / 32;    // 1 KB weight copy instructions per wave per K step
+  constexpr int BI = 64 * BI64, BJ = 64 * BJ64;
+  constexpr int WJ = NW == 4 ? 2 : (BJ >= 128 ? 4 : 2), WI = NW / WJ;   // wave grid
+  constexpr int TI = BI / (32 * WI), TJ = BJ / (32 * WJ);               // 32x32 tiles per wave
+  static_assert(TI >= 1 && TJ >= 1 && TI * WI * 32 == BI && TJ * WJ * 32 == BJ, "wave tile");
+  constexpr int WCH = BI / 8 / NW;    // 1 KB weight copy instructions per wave per K step
+  static_assert(WCH >= 1 && WCH * NW * 8 == BI, "weight copies");
   constexpr int WSTAGE = BI * 128;
 
   // dynamic LDS: [nsw][BI*128] weight ring | [xbufs][max_pos*128] patches (at sx_off, 8 KB
@@ -247,7 +285,7 @@ __global__ __launch_bounds__(256, OCC) void amos_conv_fprop(const ConvFpropParam
   const int t = threadIdx.x;
   const int lane = t & 63;
   const int wave = __builtin_amdgcn_readfirstlane(t >> 6);
-  const int wi = wave >> 1, wj = wave & 1;
+  const int wi = wave / WJ, wj = wave % WJ;
   const int frag_row = lane & 31, frag_half = lane >> 5;
 
   const int tile_j = blockIdx.x / p.tiles_i, tile_i = blockIdx.x - tile_j * p.tiles_i;
@@ -262,6 +300,41 @@ __global__ __launch_bounds__(256, OCC) void amos_conv_fprop(const ConvFpropParam
   const int NSW = p.nsw;
   const unsigned xbuf_bytes = (unsigned)p.max_pos * 128u;
   const unsigned pos_bytes = (unsigned)p.C * ES;
+
+  // ---- weight copy slots ---------------------------------------------------------------------
+  const unsigned w_row_bytes = (unsigned)(p.T * RS) * pos_bytes;
+  unsigned w_off[WCH];
+#pragma unroll
+  for (int u = 0; u < WCH; ++u) {
+    const int q = wave + NW * u;   // 1 KB chunk = 8 rows
+    const int row = q * 8 + (lane >> 3);
+    const int chunk = (lane & 7) ^ ((row ^ (row >> 3)) & 7);
+    const int r = bi0 + row < p.K ? bi0 + row : p.K - 1;
+    w_off[u] = (unsigned)r * w_row_bytes + chunk * 16;
+  }
+  // weight tile whose K slice starts wk bytes into a packed weight row -> ring stage at stage_off
+  // (32-bit offsets from the packed weights: the host keeps them under 4 GiB)
+  auto issue_weights = [&](unsigned wk, unsigned stage_off) {
+#pragma unroll
+    for (int u = 0; u < WCH; ++u)
+      __builtin_amdgcn_global_load_lds(AMOS_GLOBAL_PTR(p.wp + (size_t)(w_off[u] + wk)),
+                                       AMOS_LDS_PTR_RW(stage_off + (unsigned)(wave + NW * u) * 1024), 16, 0, 0);
+  };
+
+  // step table, read with scalar loads
+  typedef int v8i_t __attribute__((ext_vector_type(8)));
+  const __attribute__((address_space(4))) v8i_t* const tbl =
+      (const __attribute__((address_space(4))) v8i_t*)p.steps;
+  int g = m_begin * RS;   // table index of the current step
+  // the first NSW weight tiles go out before anything else: they need no set-up, and their
+  // latency covers the position table and the first patch
+  if (n_steps > 0) {
+    const unsigned last = (unsigned)(p.total_steps - 1);
+    for (int u = 0; u < NSW; ++u) {
+      const unsigned gu = (unsigned)(g + u) < last ? (unsigned)(g + u) : last;
+      issue_weights((unsigned)tbl[gu][7], (unsigned)u * WSTAGE);
+    }
+  }
 
   // ---- segments of this tile (wave-uniform scalars) -------------------------------------------
   const int j_last = (bj0 + BJ - 1 < p.J ? bj0 + BJ - 1 : p.J - 1);
@@ -293,7 +366,7 @@ __global__ __launch_bounds__(256, OCC) void amos_conv_fprop(const ConvFpropParam
   // a depth shift is added before use), d0 + 32768, or 0 when (h, w) lies outside the image}
   {
     int2* const sTab = (int2*)(smem + p.tab_off);
-    for (int pos = t; pos < npos8; pos += 256) {
+    for (int pos = t; pos < npos8; pos += 64 * NW) {
       int g_pos0 = 0, g_pa = seg_pa[0], g_base = seg_base[0], g_d0 = seg_d0[0];
 #pragma unroll
       for (int g = 1; g < kConvMaxSeg; ++g)
@@ -307,29 +380,9 @@ __global__ __launch_bounds__(256, OCC) void amos_conv_fprop(const ConvFpropParam
     }
   }
 
-  // ---- weight copy slots ---------------------------------------------------------------------
-  const unsigned w_row_bytes = (unsigned)(p.T * RS) * pos_bytes;
-  unsigned w_off[WCH];
-#pragma unroll
-  for (int u = 0; u < WCH; ++u) {
-    const int q = wave + 4 * u;   // 1 KB chunk = 8 rows
-    const int row = q * 8 + (lane >> 3);
-    const int chunk = (lane & 7) ^ ((row ^ (row >> 3)) & 7);
-    const int r = bi0 + row < p.K ? bi0 + row : p.K - 1;
-    w_off[u] = (unsigned)r * w_row_bytes + chunk * 16;
-  }
-  // weight tile whose K slice starts wk bytes into a packed weight row -> ring stage at stage_off
-  // (32-bit offsets from the packed weights: the host keeps them under 4 GiB)
-  auto issue_weights = [&](unsigned wk, unsigned stage_off) {
-#pragma unroll
-    for (int u = 0; u < WCH; ++u)
-      __builtin_amdgcn_global_load_lds(AMOS_GLOBAL_PTR(p.wp + (size_t)(w_off[u] + wk)),
-                                       AMOS_LDS_PTR_RW(stage_off + (unsigned)(wave + 4 * u) * 1024), 16, 0, 0);
-  };
-
-  // ---- patch copies: copy v of this wave fills positions [8q, 8q+8), q = wave + 4v ---------------
+  // ---- patch copies: copy v of this wave fills positions [8q, 8q+8), q = wave + NW*v -------------
   const int n_chunks8 = npos8 >> 3;
-  const int n_pl = n_chunks8 > wave ? (n_chunks8 - wave + 3) >> 2 : 0;   // copies this wave owns per patch
+  const int n_pl = n_chunks8 > wave ? (n_chunks8 - wave + NW - 1) / NW : 0;   // copies this wave owns per patch
   const unsigned tab_lane = (unsigned)p.tab_off + (unsigned)(lane >> 3) * 8;
   // 16-byte chunk a lane fetches: the swizzle of the LDS position it fills (8 KB-aligned buffers)
   const unsigned lane_c16 = (unsigned)((lane & 7) ^ (lane >> 3)) << 4;
@@ -340,7 +393,7 @@ __global__ __launch_bounds__(256, OCC) void amos_conv_fprop(const ConvFpropParam
     int vq = v < n_pl - 1 ? v : n_pl - 1;
     if (vq < 0) vq = 0;
     int2 e;
-    asm volatile("ds_read_b64 %0, %1" : "=v"(e) : "v"(tab_lane + (unsigned)(wave + 4 * vq) * 64));
+    asm volatile("ds_read_b64 %0, %1" : "=v"(e) : "v"(tab_lane + (unsigned)(wave + NW * vq) * 64));
     return e;
   };
   // one copy: table entry e of the lane's position; po = the macro step's uniform source offset
@@ -352,8 +405,8 @@ __global__ __launch_bounds__(256, OCC) void amos_conv_fprop(const ConvFpropParam
     const unsigned voff = (unsigned)d < depth_limit ? src : cq;
     __builtin_amdgcn_global_load_lds(AMOS_GLOBAL_PTR(p.zeros + (size_t)voff), AMOS_LDS_PTR_RW(dst_off), 16, 0, 0);
   };
-  // q & 7 = (wave & 3) + 4 * (v & 1): two chunk patterns per lane
-  const unsigned lane_cq[2] = {lane_c16 ^ ((unsigned)wave << 4), lane_c16 ^ ((unsigned)(wave + 4) << 4)};
+  // q & 7 = (wave + NW * (v & 1)) & 7: two chunk patterns per lane (one with 8 waves)
+  const unsigned lane_cq[2] = {lane_c16 ^ ((unsigned)(wave & 7) << 4), lane_c16 ^ ((unsigned)((wave + NW) & 7) << 4)};
 
   // ---- this lane's output columns -> patch positions ---------------------------------------------
   unsigned col_byte[TJ];
@@ -416,11 +469,6 @@ __global__ __launch_bounds__(256, OCC) void amos_conv_fprop(const ConvFpropParam
         for (int b = 0; b < TJ; ++b) acc[a][b] = MM::run(af[slot][ks][a], bf[slot][ks][b], acc[a][b]);
   };
 
-  // step table, read with scalar loads
-  typedef int v8i_t __attribute__((ext_vector_type(8)));
-  const __attribute__((address_space(4))) v8i_t* const tbl =
-      (const __attribute__((address_space(4))) v8i_t*)p.steps;
-  int g = m_begin * RS;   // table index of the current step
   int2 pt[PL > 0 ? PL : 1];   // table entries of the patch copies of the coming step
 
   // ---- prologue: the whole first patch, the first NSW weight tiles -------------------------------
@@ -431,22 +479,22 @@ __global__ __launch_bounds__(256, OCC) void amos_conv_fprop(const ConvFpropParam
       const int tt = fast_div(m_begin, p.fd_cc), cc = m_begin - tt * p.c_chunks;
       const unsigned po = 256u + (unsigned)(tt * p.dd * HW) * pos_bytes + (unsigned)cc * 128u;
       const unsigned buf = (unsigned)p.sx_off + (unsigned)(m_begin & (p.xbufs - 1)) * xbuf_bytes;
-      for (int v = 0; v < n_pl; ++v) {
-        const int q = wave + 4 * v;
-        int2 e = read_tab(v);
-        asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(e));
-        patch_copy(e, lane_cq[v & 1], po, tt * p.dd - 32768, buf + (unsigned)q * 1024, (unsigned)p.D);
-      }
-      // tile u, each later one behind as many (dummy) patch copies as a step issues ahead of its tile
-      const unsigned last = (unsigned)(p.total_steps - 1);
-      for (int u = 0; u < NSW; ++u) {
-        if (u > 0)
+      for (int v = 0; v < n_pl; v += 4) {   // four table entries per LDS round trip
+        int2 e[4];
 #pragma unroll
-          for (int x = 0; x < PL; ++x) patch_copy(int2{0, 0}, lane_cq[0], 0u, 0, (unsigned)p.dump_off, 0u);
-        const unsigned gu = (unsigned)(g + u) < last ? (unsigned)(g + u) : last;
-        issue_weights((unsigned)tbl[gu][7], (unsigned)u * WSTAGE);
+        for (int x = 0; x < 4; ++x) e[x] = read_tab(v + x);
+        asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(e[0]), "+v"(e[1]), "+v"(e[2]), "+v"(e[3]));
+#pragma unroll
+        for (int x = 0; x < 4; ++x) {
+          const bool live = v + x < n_pl;
+          patch_copy(e[x], lane_cq[x & 1], po, tt * p.dd - 32768,
+                     live ? buf + (unsigned)(wave + NW * (v + x)) * 1024 : (unsigned)p.dump_off,
+                     live ? (unsigned)p.D : 0u);
+        }
       }
-      wait_vmcnt_le((NSW - 1) * (PL + WCH));   // first patch and tile 0 landed
+      // everything issued so far has landed before the first step: its wait then allows the
+      // youngest nsw-2 steps' worth of copies in flight, and there are none yet
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
       asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
       read_step(0, buf, 0);
 #pragma unroll
@@ -459,17 +507,7 @@ __global__ __launch_bounds__(256, OCC) void amos_conv_fprop(const ConvFpropParam
   //        macro step's patch buffer, wk of this step's own tile}
   unsigned istage = 0;   // ring stage (byte offset) this step's fetch goes to = the stage step-1 read
   v8i_t nxt = cur;
-#ifdef AMOS_CONV_TIMING
-  unsigned long long tacc[3] = {0, 0, 0}, tC = 0;
-  auto now = [] { unsigned long long tt; asm volatile("s_memtime %0\n\ts_waitcnt lgkmcnt(0)" : "=s"(tt)::"memory"); return tt; };
-  tC = now();
-  const unsigned long long tstart = tC;
-#endif
   auto one_step = [&](int slot, const v8i_t& e, v8i_t& e_next) {
-#ifdef AMOS_CONV_TIMING
-    const unsigned long long tA = now();
-    tacc[0] += tA - tC;
-#endif
     // This wave's reads of the current step's operands (issued a step ago) are complete, and so
     // are its copies of everything older than the youngest NSW-2 steps' worth: the next weight
     // tile and, at a macro step's last tap, the next patch.  After the barrier that holds for
@@ -477,10 +515,6 @@ __global__ __launch_bounds__(256, OCC) void amos_conv_fprop(const ConvFpropParam
     if (NSW >= 4) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * (PL + WCH)) : "memory");
     else if (NSW == 3) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(PL + WCH) : "memory");
     else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-#ifdef AMOS_CONV_TIMING
-    const unsigned long long tB = now();
-    tacc[1] += tB - tA;
-#endif
     // (the table entries read a step ago are tied to the wait, so that nothing uses them before it)
     if (PL == 4)
       asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" : "+v"(pt[0]), "+v"(pt[1]), "+v"(pt[PL > 2 ? 2 : 0]), "+v"(pt[PL > 2 ? 3 : 0])::"memory");
@@ -488,10 +522,6 @@ __global__ __launch_bounds__(256, OCC) void amos_conv_fprop(const ConvFpropParam
       asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" : "+v"(pt[0]), "+v"(pt[PL > 1 ? 1 : 0])::"memory");
     else
       asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
-#ifdef AMOS_CONV_TIMING
-    tC = now();
-    tacc[2] += tC - tB;
-#endif
     // (every word of the entry stays live up to here: a register of the tuple that is reused
     // earlier makes the compiler wait for the scalar load right after issuing it)
     asm volatile("" ::"s"(e[0]), "s"(e[1]), "s"(e[2]), "s"(e[3]), "s"(e[4]), "s"(e[5]), "s"(e[6]), "s"(e[7]));
@@ -504,12 +534,12 @@ __global__ __launch_bounds__(256, OCC) void amos_conv_fprop(const ConvFpropParam
     // copies are older than a tile that is waited for before the patch is first read
     if (PL > 0) {
       const int n_live = e[5] + 1 < m_end ? n_pl : 0;
-      const int v0 = e[4] & 0xffff;   // even: copies per step come in twos
-      const unsigned dst0 = (unsigned)e[6] + (unsigned)wave * 1024 + (unsigned)v0 * 4096;
+      const int v0 = e[4] & 0xffff;   // even with 4 waves: their copies per step come in twos
+      const unsigned dst0 = (unsigned)e[6] + (unsigned)wave * 1024 + (unsigned)v0 * (NW * 1024);
 #pragma unroll
       for (int x = 0; x < PL; ++x) {
         const bool live = v0 + x < n_live;
-        patch_copy(pt[x], lane_cq[x & 1], (unsigned)e[2], e[3], live ? dst0 + x * 4096 : (unsigned)p.dump_off,
+        patch_copy(pt[x], lane_cq[x & 1], (unsigned)e[2], e[3], live ? dst0 + x * (NW * 1024) : (unsigned)p.dump_off,
                    live ? (unsigned)p.D : 0u);
       }
     }
@@ -532,14 +562,6 @@ __global__ __launch_bounds__(256, OCC) void amos_conv_fprop(const ConvFpropParam
   }
   if (step < n_steps) one_step(0, cur, nxt);
 
-#ifdef AMOS_CONV_TIMING
-  const unsigned long long tloop = now();
-  if ((blockIdx.x == 0 || blockIdx.x == 77) && blockIdx.y == 0 && t == 0) {
-    unsigned* dbg = (unsigned*)(p.zeros + 128) + (blockIdx.x ? 8 : 0);
-    dbg[0] = (unsigned)tacc[0]; dbg[1] = (unsigned)tacc[1]; dbg[2] = (unsigned)tacc[2];
-    dbg[3] = (unsigned)(tloop - tstart); dbg[4] = (unsigned)n_steps;
-  }
-#endif
   // ---- epilogue: Y[(n*K + i)*ODPQ + (od*OPQ + opq)] ---------------------------------------------
   out_t* const out = (out_t*)p.y;
   const int ODPQ = p.OD * OPQ;

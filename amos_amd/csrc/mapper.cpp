@@ -119,8 +119,22 @@ int64_t conv_workspace_bytes(const amos_conv_desc_t& c, int op) {
 }
 
 
-ConvPatchPlan conv_patch_plan(const amos_conv_desc_t& cin, int op, int BI, int BJ, int split_k) {
-  ConvPatchPlan pp = {nullptr, 0, 0, 0, 0, 0, 0, 0};
+static ConvPatchPlan conv_patch_plan_waves(const amos_conv_desc_t& cin, int op, int BI, int BJ, int split_k,
+                                           int waves);
+
+// waves: 4, 8, or 0 = 8 where that applies and four waves would leave a CU with a single workgroup
+ConvPatchPlan conv_patch_plan(const amos_conv_desc_t& c, int op, int BI, int BJ, int split_k, int waves) {
+  if (waves == 4 || waves == 8) return conv_patch_plan_waves(c, op, BI, BJ, split_k, waves);
+  ConvPatchPlan p4 = conv_patch_plan_waves(c, op, BI, BJ, split_k, 4);
+  if (!p4.why && p4.occ == 2) return p4;
+  ConvPatchPlan p8 = conv_patch_plan_waves(c, op, BI, BJ, split_k, 8);
+  return p8.why ? p4 : p8;
+}
+
+static ConvPatchPlan conv_patch_plan_waves(const amos_conv_desc_t& cin, int op, int BI, int BJ, int split_k,
+                                           int waves) {
+  ConvPatchPlan pp = {nullptr, 0, 0, 0, 0, 0, 0, 0, 0};
+  pp.waves = waves;
   amos_conv_desc_t c = cin;
   if (op == AMOS_OP_CONV2D) { c.D = 1; c.T = 1; c.stride_d = 1; c.pad_d = 0; c.dil_d = 1; }
   const int es = c.in_dtype == AMOS_I8 ? 1 : 2;
@@ -131,12 +145,14 @@ ConvPatchPlan conv_patch_plan(const amos_conv_desc_t& cin, int op, int BI, int B
   const int64_t packed = conv_packed_bytes(c, op);
   const int RS = (int)(c.R * c.S);
   const int Wp = (int)((OQ - 1) * c.stride_w + (c.S - 1) * c.dil_w + 1);
-  const bool tile_ok = (BI == 64 && (BJ == 64 || BJ == 128 || BJ == 256)) ||
-                       (BI == 128 && (BJ == 64 || BJ == 128 || BJ == 256)) ||
-                       (BI == 256 && (BJ == 64 || BJ == 128));
+  const bool tile_ok = waves == 8 ? ((BI == 128 && (BJ == 64 || BJ == 128 || BJ == 256)) ||
+                                     (BI == 64 && BJ == 128) || (BI == 256 && BJ == 128))
+                                  : ((BI == 64 && (BJ == 64 || BJ == 128 || BJ == 256)) ||
+                                     (BI == 128 && (BJ == 64 || BJ == 128 || BJ == 256)) ||
+                                     (BI == 256 && (BJ == 64 || BJ == 128)));
   if (OD <= 0 || OP <= 0 || OQ <= 0) { pp.why = "empty output"; return pp; }
   if (packed == 0) { pp.why = "C * element size is not a multiple of 128 bytes"; return pp; }
-  if (packed >= ((int64_t)1 << 32)) { pp.why = "packed weights above 4 GiB"; return pp; }
+  if (packed >= ((int64_t)1 << 31)) { pp.why = "packed weights above 2 GiB"; return pp; }
   if (conv_relaid_bytes(c, op) + 256 >= ((int64_t)1 << 32)) { pp.why = "activations above 4 GiB"; return pp; }
   if (c.N * c.D * c.H * c.W >= ((int64_t)1 << 31) || J >= ((int64_t)1 << 31) - 512) {
     pp.why = "more than 2^31 input or output positions";
@@ -163,11 +179,12 @@ ConvPatchPlan conv_patch_plan(const amos_conv_desc_t& cin, int op, int BI, int B
   if (max_seg > kConvMaxSegHost) { pp.why = "a tile spans more than 4 image slices"; return pp; }
   if (max_pos >= 4096) { pp.why = "input patch of a tile has 4096 or more positions"; return pp; }
   if (patch + 2 * wstage > budget) { pp.why = "input patch of a tile does not fit LDS"; return pp; }
-  const int per_wave = ((real_pos / 8) + 3) / 4;   // patch copies of the busiest wave
+  const int per_wave = ((real_pos / 8) + waves - 1) / waves;   // patch copies of the busiest wave
   // Ring depth and patch copies per step for an LDS budget.  The next patch is copied during the
   // taps of the current one; a copy issued on tap u has landed for everybody at the barrier of
   // the patch's last tap only if it is older than the nsw-2 steps' worth of copies still allowed
-  // in flight there: u <= RS - nsw.  Kernel instances exist for 0, 2 and 4 copies per step.
+  // in flight there: u <= RS - nsw.  Kernel instances exist for 0, 2 and 4 copies per step
+  // (4 waves), 0, 1 and 2 (8 waves).
   auto fit = [&](size_t lds_budget, int* nsw_out, int* pls_out) -> const char* {
     if (patch + 2 * wstage > lds_budget) return "input patch of a tile does not fit LDS";
     int nsw = (int)((lds_budget - patch) / wstage);
@@ -179,9 +196,9 @@ ConvPatchPlan conv_patch_plan(const amos_conv_desc_t& cin, int op, int BI, int B
       const int taps = RS + 1 - nsw;
       if (taps < 1) continue;
       const int pls = (per_wave + taps - 1) / taps;
-      if (pls > 4) continue;
+      if (pls > (waves == 8 ? 2 : 4)) continue;
       *nsw_out = nsw;
-      *pls_out = pls <= 2 ? 2 : 4;
+      *pls_out = waves == 8 ? pls : (pls <= 2 ? 2 : 4);
       return nullptr;
     }
     return RS == 1 ? "1x1 window with several channel chunks per block"
@@ -195,7 +212,7 @@ ConvPatchPlan conv_patch_plan(const amos_conv_desc_t& cin, int op, int BI, int B
   // fragments within 256 registers (tiles up to 128x128); pointless when every block already has
   // a CU to itself
   const int64_t blocks = ((c.K + BI - 1) / BI) * ((J + BJ - 1) / BJ) * split;
-  if (BI <= 128 && BJ <= 128 && blocks > Gfx950::kComputeUnits) {
+  if (waves == 4 && BI <= 128 && BJ <= 128 && blocks > Gfx950::kComputeUnits) {
     int nsw2 = 0, pls2 = 0;
     if (!fit((size_t)79 * 1024, &nsw2, &pls2)) {
       pp.occ = 2;
@@ -245,8 +262,9 @@ static double estimate_seconds(const Problem& pb, int ti, int tj, int split) {
 // accumulation into the output.  Returns <= 0 where the pipeline does not apply.
 static double conv_patch_estimate(const amos_conv_desc_t& c, int op, const Problem& pb, int ti, int tj,
                                   int split) {
-  ConvPatchPlan pp = conv_patch_plan(c, op, ti, tj, split);
+  ConvPatchPlan pp = conv_patch_plan(c, op, ti, tj, split, 0);
   if (pp.why) return -1.0;
+  const bool two_streams = pp.occ == 2 || pp.waves == 8;   // two waves per SIMD
   const double es = pb.in_dtype == AMOS_I8 ? 1.0 : 2.0;
   const int64_t T = op == AMOS_OP_CONV2D ? 1 : c.T;
   const double steps_all = (double)T * c.R * c.S * std::ceil(c.C * es / 128.0);
@@ -256,7 +274,7 @@ static double conv_patch_estimate(const amos_conv_desc_t& c, int op, const Probl
   const double rounds = std::ceil(blocks / (Gfx950::kComputeUnits * (double)pp.occ));
   const double steps = std::ceil(steps_all / split);
   const double mfma_per_step = (ti / 64.0) * (tj / 64.0) * 4.0 * 32.0;
-  const double cycles = rounds * (steps * (pp.occ * mfma_per_step + (pp.occ == 2 ? 500.0 : 600.0)) + 4000.0);
+  const double cycles = rounds * (steps * (pp.occ * mfma_per_step + (two_streams ? 500.0 : 600.0)) + 4000.0);
   const double relayout = ((double)pb.in_bytes * 2.0) / 2.5e12 + 3e-6;
   return cycles / 2.1e9 + relayout + (split > 1 ? (double)pb.out_bytes * split / 1.2e12 : 0.0);
 }

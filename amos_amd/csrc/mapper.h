@@ -41,11 +41,12 @@ struct ConvPatchPlan {
   int pls;           // patch copies per wave per K step: 0 (single macro step), 2 or 4
   int xbufs;         // patch buffers (1 when a block runs a single macro step)
   int occ;           // workgroups per CU the instance is built for (2 when LDS and registers allow)
+  int waves;         // waves per workgroup: 4 or 8
   size_t lds;        // dynamic LDS bytes of the block
 };
 int64_t conv_packed_bytes(const amos_conv_desc_t& c, int op);
 int64_t conv_relaid_bytes(const amos_conv_desc_t& c, int op);
 int64_t conv_workspace_bytes(const amos_conv_desc_t& c, int op);
-ConvPatchPlan conv_patch_plan(const amos_conv_desc_t& c, int op, int BI, int BJ, int split_k);
+ConvPatchPlan conv_patch_plan(const amos_conv_desc_t& c, int op, int BI, int BJ, int split_k, int waves);
 
 }  // namespace amos

@@ -133,7 +133,9 @@ typedef struct {
 #define AMOS_PIPE_DIRECT4 2   /* global -> LDS direct copies, 256x256 tile, 4 waves           */
 #define AMOS_PIPE_DIRECT8 3   /* same with 8 waves (two per SIMD)                             */
 #define AMOS_PIPE_PATCH 4     /* conv: input patch staged once per channel chunk, weights     */
-                              /* repacked into the workspace; needs amos_workspace_bytes()    */
+                              /* repacked into the workspace; needs amos_workspace_bytes();   */
+                              /* 4 waves per workgroup                                        */
+#define AMOS_PIPE_PATCH8 5    /* same with 8 waves (two per SIMD)                             */
 
 int amos_version(void);
 const char* amos_last_error(void);

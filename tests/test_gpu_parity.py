@@ -239,7 +239,7 @@ PATCH_CONV_CASES = [
 @pytest.mark.parametrize("dtype", ["float16", "bfloat16", "int8"])
 @pytest.mark.parametrize("case", PATCH_CONV_CASES)
 def test_conv_patch_pipeline(gpu, dtype, case):
-    """patch-staged convolution (pipeline 4): every tile shape, with and without split-K"""
+    """patch-staged convolution (4 and 8 waves): every tile shape, with and without split-K"""
     from amos_amd import _lib, ops
     N, C, D, H, W, K, T, R, S, st, pd, dl = case
     rng = np.random.default_rng(hash(case) % 2**32)
@@ -247,9 +247,11 @@ def test_conv_patch_pipeline(gpu, dtype, case):
     w = make_operand(rng, (K, C, T, R, S), dtype, "normal")
     ref = co.lib_conv3d(x, w, dtype, st, pd, dl, acc="float64")
     dx, dw = to_device(x, dtype), to_device(w, dtype)
-    for tile in [(64, 64), (128, 64), (64, 128), (128, 128), (256, 64), (256, 128), (128, 256), (64, 256)]:
-        for split in (1, 2):
-            cfg = dict(tile_i=tile[0], tile_j=tile[1], split_k=split, pipeline=_lib.AMOS_PIPE_PATCH)
+    tiles = [(64, 64), (128, 64), (64, 128), (128, 128), (256, 64), (256, 128), (128, 256), (64, 256)]
+    for tile, split, pipe in [(t, s, p) for t in tiles for s in (1, 2)
+                              for p in (_lib.AMOS_PIPE_PATCH, _lib.AMOS_PIPE_PATCH8)]:
+        if True:
+            cfg = dict(tile_i=tile[0], tile_j=tile[1], split_k=split, pipeline=pipe)
             try:
                 if D == 1 and T == 1:
                     got = ops.conv2d(dx[:, :, 0], dw[:, :, 0], st[1:], pd[1:], dl[1:], config=cfg)[:, :, None]
@@ -259,7 +261,8 @@ def test_conv_patch_pipeline(gpu, dtype, case):
                 # a tile that spans too many slices or a patch too large: reported, never silent
                 assert e.code == _lib.AMOS_ERR_INFEASIBLE and "not applicable" in str(e)
                 continue
-            check(got.cpu().numpy(), ref, dtype, "patch conv %s %s tile %s split %d" % (dtype, case, tile, split))
+            check(got.cpu().numpy(), ref, dtype,
+                  "patch conv %s %s tile %s split %d pipeline %d" % (dtype, case, tile, split, pipe))
 
 
 def test_conv_patch_is_the_default_when_applicable(gpu):
