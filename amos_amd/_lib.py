@@ -52,6 +52,14 @@ class KernelConfig(ctypes.Structure):
                 ("reserved", _i32 * 4)]
 
 
+AMOS_EPI_NONE, AMOS_EPI_ADD = 0, 1
+
+
+class Epilogue(ctypes.Structure):
+    _fields_ = [("kind", _i32), ("dtype", _i32), ("operand", ctypes.c_void_p), ("ld", _i64),
+                ("stride", _i64)]
+
+
 class ComputeC(ctypes.Structure):
     _fields_ = [("n_tokens", _i32), ("tokens", ctypes.POINTER(_i32)), ("n_iters", _i32),
                 ("iter_kinds", ctypes.POINTER(_i32)), ("iter_extents", ctypes.POINTER(_i64)),
@@ -71,7 +79,8 @@ class AmosError(RuntimeError):
 EXPORTS = [
     "amos_version", "amos_last_error", "amos_device_info", "amos_default_config",
     "amos_check_config", "amos_workspace_bytes", "amos_estimate_seconds", "amos_gemm", "amos_bgemm", "amos_conv2d",
-    "amos_conv3d", "amos_time", "amos_kernel_name", "amos_match", "amos_enumerate_mappings",
+    "amos_conv3d", "amos_run_fused", "amos_time", "amos_time_fused", "amos_kernel_name", "amos_match",
+    "amos_enumerate_mappings",
 ]
 
 _lib = None
@@ -105,6 +114,11 @@ def load():
     lib.amos_time.argtypes = [ctypes.c_int, vp, ctypes.POINTER(KernelConfig), vp, vp, vp, vp, sz, vp,
                               ctypes.c_int, ctypes.c_int, ctypes.c_int,
                               ctypes.POINTER(ctypes.c_double)]
+    lib.amos_run_fused.argtypes = [ctypes.c_int, vp, ctypes.POINTER(KernelConfig), ctypes.POINTER(Epilogue),
+                                   vp, vp, vp, vp, sz, vp]
+    lib.amos_time_fused.argtypes = [ctypes.c_int, vp, ctypes.POINTER(KernelConfig), ctypes.POINTER(Epilogue),
+                                    vp, vp, vp, vp, sz, vp, ctypes.c_int, ctypes.c_int, ctypes.c_int,
+                                    ctypes.POINTER(ctypes.c_double)]
     lib.amos_kernel_name.argtypes = [ctypes.c_int, vp, ctypes.POINTER(KernelConfig)]
     lib.amos_kernel_name.restype = ctypes.c_char_p
     lib.amos_match.argtypes = [ctypes.POINTER(ComputeC), ctypes.POINTER(ComputeC),

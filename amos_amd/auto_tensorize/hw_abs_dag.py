@@ -180,3 +180,46 @@ class MFMAInt8Int32WrappedSpelling(MFMADag):
     mma_mnemonic = "mfma_i8_i32::mma_wrapped_spelling"
     shape_keys = ("32x32x32", "16x16x64")
     wrapped_spelling = True
+
+
+class MFMABiasDag(MFMADag):
+    """load_a, load_b -> mma, load_bias -> bias -> store: the DAG with an element-wise stage
+    behind the MMA.  Like the reference's WMMAFp16Fp32Bias (hw_abs_dag/cuda/wmma_fp16_bias.py:11-56)
+    it is NOT registered: query_hw_abs_dag() and the matching counts of the tutorial flow do not
+    see it.  A compute with such a tail still matches the plain DAG on its main op, and lowering
+    fuses the tail into the kernel (lowering.py)."""
+    edges = {"mma": ["load_a", "load_b"], "bias": ["mma", "load_bias"], "store": ["bias"]}
+    anchor_point = "bias"
+    bias_dtype = None
+
+    def __init__(self):
+        super().__init__()
+        self.hw_abs_dict = dict(self.hw_abs_dict)
+        self.hw_abs_dict["load_bias"] = HW_ABS_REGISTER_POOL.find("hip", "mfma::lds_load")
+        self.hw_abs_dict["bias"] = HW_ABS_REGISTER_POOL.find("hip", "mfma::add_bias")
+        self.input_dtypes = dict(self.input_dtypes, load_bias=[self.bias_dtype],
+                                 bias=[self.mma.out_dtype, self.bias_dtype], store=[self.mma.out_dtype])
+        self.output_dtypes = dict(self.output_dtypes, load_bias=[self.bias_dtype], bias=[self.mma.out_dtype])
+
+    def get_effective_compute_dag(self, compute_key, shape_key):
+        """two ops: the MMA (op_lst[0]) and the element-wise addition behind it (op_lst[1])"""
+        _, outs = self.get_main_compute_expression(compute_key, shape_key)
+        m, n, _ = self.get_problem_size(shape_key)
+        shape = [int(x) for x in outs[0].shape]
+        _, tail = self.hw_abs_dict["bias"]().get_compute_expression_with_inputs(
+            [outs[0]], [shape, shape], [shape], [self.mma.out_dtype, self.bias_dtype], [self.mma.out_dtype])
+        return compute_dag_from_tensors(tail), outs
+
+
+class MFMAFp16Fp32Bias(MFMABiasDag):
+    mnemonic = "mfma_f16_f32_bias"
+    mma_mnemonic = "mfma_f16_f32::mma"
+    shape_keys = ("32x32x16", "16x16x32")
+    bias_dtype = "float16"
+
+
+class MFMAInt8Int32Bias(MFMABiasDag):
+    mnemonic = "mfma_i8_i32_bias"
+    mma_mnemonic = "mfma_i8_i32::mma"
+    shape_keys = ("32x32x32", "16x16x64")
+    bias_dtype = "int32"

@@ -245,5 +245,29 @@ class GlobalStore(MemoryAbstraction):
     target = "hip"
 
 
+@register_abstraction("hip", "mfma::add_bias")
+class MFMAAddBias(ElementwiseComputeAbstraction):
+    """C = A + B.astype(out) on the accumulator registers of a wavefront: the tail a kernel
+    fuses into its store.  Replaces nvcuda::wmma::add_bias
+    (hw_abstraction/cuda/wmma_bias.py:12-80)."""
+    target = "hip"
+
+    def get_compute_expression(self, input_shapes, output_shapes, input_dtypes, output_dtypes, problem_size=None):
+        assert len(input_shapes) == 2 and len(output_shapes) == 1
+        A = te.placeholder(input_shapes[0], name="A", dtype=input_dtypes[0])
+        _, outs = self.get_compute_expression_with_inputs([A], input_shapes, output_shapes, input_dtypes,
+                                                          output_dtypes, problem_size)
+        return [A, outs[0].op.input_tensors[1]], outs
+
+    def get_compute_expression_with_inputs(self, inputs, input_shapes, output_shapes, input_dtypes,
+                                           output_dtypes, problem_size=None):
+        (A,) = inputs
+        B = te.placeholder(input_shapes[1], name="B", dtype=input_dtypes[1])
+        same = input_dtypes[1] == output_dtypes[0]
+        C = te.compute(output_shapes[0],
+                       lambda *idx: A(*idx) + (B(*idx) if same else B(*idx).astype(output_dtypes[0])), name="C")
+        return [A, B], [C]
+
+
 register_abstraction("hip", "mfma::lds_load")(LdsLoad)
 register_abstraction("hip", "mfma::global_store")(GlobalStore)

@@ -27,6 +27,7 @@ class LoweredOp(object):
         self.inputs = inputs
         self.output = output
         self.attrs = attrs
+        self.add_input = None    # tensor D of a fused tail  output = main + D.astype(out), else None
 
     def flops(self):
         a = self.attrs
@@ -35,7 +36,8 @@ class LoweredOp(object):
         return 2.0 * a["J"] * a["K_out"] * a["K_red"]
 
     def __str__(self):
-        return "%s %s" % (self.kind, {k: v for k, v in self.attrs.items()})
+        tail = " + %s" % self.add_input.name if self.add_input is not None else ""
+        return "%s%s %s" % (self.kind, tail, {k: v for k, v in self.attrs.items()})
 
 
 def _single_var(form, iters):
@@ -241,8 +243,53 @@ def _lower_conv(main_op, l0, l1, iters, forms0, forms1):
     return LoweredOp(kind, code, c, [src, lw.tensor], main_op.output(0), attrs)
 
 
-def lower_main_op(main_op):
-    """ComputeOp that matched a GEMM-like intrinsic -> LoweredOp"""
+def _fuse_tail(low, main_op, target_dag):
+    """The element-wise stage behind the main op, if any, becomes the kernel's fused tail.
+    The reference keeps such stages in IntrinMatchResult.elem_op_map and maps them with the
+    main op (intrin_match.py:24-42, tests/python/auto_tensorize/test_compute_transform_gemm.py:7-23,
+    "E = C + D"); the kernels here add one operand of the output's shape on the accumulators."""
+    readers = [op for op in target_dag.op_lst if any(t.op is main_op for t in op.input_tensors)]
+    if not readers:
+        return low
+    if len(readers) > 1:
+        raise NoKernelError("the main op feeds %d stages; one element-wise tail can be fused" % len(readers))
+    tail = readers[0]
+    if any(any(t.op is tail for t in op.input_tensors) for op in target_dag.op_lst):
+        raise NoKernelError("a chain of stages behind the main op has no fused kernel")
+    body = tail.body[0] if not tail.reduce_axis else None
+    if not isinstance(body, te.Add):
+        raise NoKernelError("stage %s behind the main op is not an element-wise addition" % tail.name)
+    loads = [_strip_cast(body.a), _strip_cast(body.b)]
+    if not all(isinstance(l, te.ProducerLoad) for l in loads):
+        raise NoKernelError("stage %s does not add two tensor elements" % tail.name)
+    main_load = [l for l in loads if l.tensor.op is main_op]
+    other = [l for l in loads if l.tensor.op is not main_op]
+    if len(main_load) != 1 or len(other) != 1 or not isinstance(other[0].tensor.op, te.PlaceholderOp):
+        raise NoKernelError("stage %s must add the main op's result and a placeholder" % tail.name)
+    variables = [iv.var for iv in tail.axis]
+    for l in loads:
+        if len(l.indices) != len(variables) or any(i is not v for i, v in zip(l.indices, variables)):
+            raise NoKernelError("stage %s permutes or offsets indices" % tail.name)
+    d = other[0].tensor
+    out = tail.output(0)
+    if [int(x) for x in d.shape] != [int(x) for x in out.shape] or out.dtype != low.output.dtype:
+        raise NoKernelError("the added tensor must have the output's shape and the sum its type")
+    ok = ("int32",) if out.dtype == "int32" else ("float32", "float16", "bfloat16")
+    if d.dtype not in ok:
+        raise NoKernelError("cannot add a %s tensor to a %s result" % (d.dtype, out.dtype))
+    low.add_input = d
+    low.output = out
+    return low
+
+
+def lower_main_op(main_op, target_dag=None):
+    """ComputeOp that matched a GEMM-like intrinsic -> LoweredOp; with the compute DAG it
+    belongs to, an element-wise addition behind it is fused into the kernel"""
+    low = _lower_main_op(main_op)
+    return _fuse_tail(low, main_op, target_dag) if target_dag is not None else low
+
+
+def _lower_main_op(main_op):
     l0, l1 = _product_loads(main_op)
     iters = list(main_op.axis) + list(main_op.reduce_axis)
     variables = [iv.var for iv in iters]

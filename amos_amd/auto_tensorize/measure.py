@@ -55,13 +55,27 @@ def random_device_arrays(lowered, dev_id=0, seed=0):
     return arrays[0], arrays[1], out
 
 
+def random_add_array(lowered, dev_id=0, seed=1):
+    """the operand of a fused tail (None without one), filled like the inputs"""
+    t = getattr(lowered, "add_input", None)
+    if t is None:
+        return None
+    dev = torch.device("cuda", dev_id)
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(seed)
+    shape = [int(s) for s in t.shape]
+    if t.dtype == "int32":
+        return torch.randint(-(1 << 16), 1 << 16, shape, dtype=torch.int32, device=dev, generator=gen)
+    return (torch.rand(shape, device=dev, generator=gen) * 2 - 1).to(_TORCH_DTYPE[t.dtype])
+
+
 def evaluate_params_on_device(lowered, params, measure_opt):
     """milliseconds per launch of one kernel configuration"""
     from .. import ops
     in0, in1, out = random_device_arrays(lowered, measure_opt.dev_id)
     secs = ops.time_op(lowered.op_code, lowered.desc, in0, in1, out, config=params.to_config(),
                        number=measure_opt.number, repeat=max(1, measure_opt.repeat),
-                       min_repeat_ms=measure_opt.min_repeat_ms)
+                       min_repeat_ms=measure_opt.min_repeat_ms, add=random_add_array(lowered, measure_opt.dev_id))
     return sum(secs) / len(secs) * 1e3
 
 

@@ -79,13 +79,15 @@ class Module(object):
     def __init__(self, lowered, params, arg_tensors):
         self.lowered = lowered
         self.params = params
-        # positions of (in0, in1, out) among the caller's arguments
+        # positions of (in0, in1, out[, added tensor of a fused tail]) among the caller's arguments
         ids = [id(t) for t in arg_tensors]
         try:
             self.arg_index = [ids.index(id(lowered.inputs[0])), ids.index(id(lowered.inputs[1])),
                               ids.index(id(lowered.output))]
+            if getattr(lowered, "add_input", None) is not None:
+                self.arg_index.append(ids.index(id(lowered.add_input)))
         except ValueError:
-            raise ValueError("build() args must hold the compute's two inputs and its output tensor")
+            raise ValueError("build() args must hold the compute's inputs and its output tensor")
         self.imported_modules = [_Source(self)]
 
     def _pick(self, arrays):
@@ -97,27 +99,29 @@ class Module(object):
             out.append(a.tensor if isinstance(a, NDArray) else a)
         return out
 
-    def _run(self, in0, in1, out):
+    def _run(self, in0, in1, out, add=None):
         low, cfg = self.lowered, self.params.to_config() if self.params is not None else None
         a = low.attrs
         if low.kind == "gemm":
-            ops.gemm(in0, in1, a["trans_a"], a["trans_b"], out=out, config=cfg)
+            ops.gemm(in0, in1, a["trans_a"], a["trans_b"], out=out, config=cfg, add=add)
         elif low.kind == "bgemm":
-            ops.bgemm(in0, in1, a["trans_a"], a["trans_b"], out=out, config=cfg)
+            ops.bgemm(in0, in1, a["trans_a"], a["trans_b"], out=out, config=cfg, add=add)
         elif low.kind == "conv2d":
-            ops.conv2d(in0, in1, a["stride"], a["pad"], a["dil"], out=out, config=cfg)
+            ops.conv2d(in0, in1, a["stride"], a["pad"], a["dil"], out=out, config=cfg, add=add)
         else:
-            ops.conv3d(in0, in1, a["stride"], a["pad"], a["dil"], out=out, config=cfg)
+            ops.conv3d(in0, in1, a["stride"], a["pad"], a["dil"], out=out, config=cfg, add=add)
 
     def __call__(self, *arrays):
         self._run(*self._pick(arrays))
 
     def time_evaluator(self, func_name=None, ctx=None, number=10, repeat=1, min_repeat_ms=0):
         def evaluator(*arrays):
-            in0, in1, out = self._pick(arrays)
+            picked = self._pick(arrays)
+            in0, in1, out = picked[:3]
             cfg = self.params.to_config() if self.params is not None else None
             return TimeResult(ops.time_op(self.lowered.op_code, self.lowered.desc, in0, in1, out, config=cfg,
-                                          number=number, repeat=repeat, min_repeat_ms=min_repeat_ms))
+                                          number=number, repeat=repeat, min_repeat_ms=min_repeat_ms,
+                                          add=picked[3] if len(picked) > 3 else None))
         return evaluator
 
     def get_source(self):
@@ -134,8 +138,10 @@ def build(sch, args, target="hip", target_host=None, name="default_function"):
     if lowered is None:
         from .lowering import lower_main_op
         from .. import te
-        mains = [op for op in sch.outputs if isinstance(op, te.ComputeOp) and op.reduce_axis]
+        from .hw_abstraction import compute_dag_from_tensors
+        dag = compute_dag_from_tensors([op.output(0) for op in sch.outputs])
+        mains = [op for op in dag.op_lst if op.reduce_axis]
         if not mains:
             raise ValueError("nothing to build: apply a schedule from auto_tensorize first")
-        lowered = lower_main_op(mains[0])
+        lowered = lower_main_op(mains[0], dag)
     return Module(lowered, getattr(sch, "kernel_config", None), list(args))

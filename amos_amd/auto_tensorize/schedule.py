@@ -116,7 +116,7 @@ class MI355XScheduleGenerator(object):
         self.match_result = intrin_match_result
         self.state = new_state
         main_op = list(intrin_match_result.main_op_map.values())[0]
-        self.lowered = lower_main_op(main_op)
+        self.lowered = lower_main_op(main_op, getattr(intrin_match_result, "target_dag", None))
         self.log_file = log_file
         self.verbose_init = verbose_init
         self.entries = []

@@ -441,10 +441,42 @@ static int launch(const Plan& pl, hipStream_t stream) {
   return 0;
 }
 
-static int run_op(int op, const void* desc, const amos_kernel_config_t* cfg, const void* in0,
-                  const void* in1, void* out, void* workspace, size_t ws_bytes, void* stream) {
+// fused tail operation: validate it against the planned op and hand it to whichever kernel runs
+static int plan_epilogue(Plan& pl, int op, const void* desc, const amos_epilogue_t* e) {
+  EpiParams ep = {nullptr, 0, 0, EPI_NONE};
+  if (e && e->kind != AMOS_EPI_NONE) {
+    if (e->kind != AMOS_EPI_ADD) return set_error(AMOS_ERR_UNSUPPORTED, "unknown epilogue kind %d", e->kind);
+    if (!e->operand) return set_error(AMOS_ERR_BAD_ARG, "epilogue operand is null");
+    const bool int_out = pl.dt == DT_I8;
+    if (int_out ? e->dtype != AMOS_I32
+                : (e->dtype != AMOS_F32 && e->dtype != AMOS_F16 && e->dtype != AMOS_BF16))
+      return set_error(AMOS_ERR_UNSUPPORTED, "epilogue operand dtype %d does not go with the output type "
+                       "(int32 output: int32; fp32 output: fp32, fp16 or bf16)", e->dtype);
+    ep.ptr = (const char*)e->operand;
+    ep.dt = e->dtype == AMOS_F16 ? EPI_F16 : e->dtype == AMOS_BF16 ? EPI_BF16 : EPI_OUT_TYPE;
+    if (op == AMOS_OP_GEMM || op == AMOS_OP_BGEMM) {
+      const amos_gemm_desc_t& g = op == AMOS_OP_GEMM ? *(const amos_gemm_desc_t*)desc
+                                                     : ((const amos_bgemm_desc_t*)desc)->g;
+      ep.si = e->ld > 0 ? e->ld : g.N;
+      if (ep.si < g.N) return set_error(AMOS_ERR_BAD_ARG, "epilogue ld %lld below N", (long long)e->ld);
+      ep.batch = e->stride > 0 ? e->stride : g.M * ep.si;
+    } else {
+      ep.si = pl.p.out_si;   // D is laid out like the output, NKDPQ
+    }
+  }
+  pl.p.epi = ep;
+  pl.tn.epi = ep;
+  pl.cv.epi = ep;
+  return 0;
+}
+
+static int run_op(int op, const void* desc, const amos_kernel_config_t* cfg, const amos_epilogue_t* epi,
+                  const void* in0, const void* in1, void* out, void* workspace, size_t ws_bytes,
+                  void* stream) {
   Plan pl;
   int rc = make_plan(pl, op, desc, cfg, in0, in1, out, workspace, ws_bytes);
+  if (rc) return rc;
+  rc = plan_epilogue(pl, op, desc, epi);
   if (rc) return rc;
   return launch(pl, (hipStream_t)stream);
 }
@@ -480,19 +512,27 @@ int amos_device_info(amos_device_info_t* out) {
 
 int amos_gemm(const amos_gemm_desc_t* desc, const amos_kernel_config_t* cfg, const void* A,
               const void* B, void* C, void* workspace, size_t ws_bytes, void* stream) {
-  return run_op(AMOS_OP_GEMM, desc, cfg, A, B, C, workspace, ws_bytes, stream);
+  return run_op(AMOS_OP_GEMM, desc, cfg, nullptr, A, B, C, workspace, ws_bytes, stream);
 }
 int amos_bgemm(const amos_bgemm_desc_t* desc, const amos_kernel_config_t* cfg, const void* A,
                const void* B, void* C, void* workspace, size_t ws_bytes, void* stream) {
-  return run_op(AMOS_OP_BGEMM, desc, cfg, A, B, C, workspace, ws_bytes, stream);
+  return run_op(AMOS_OP_BGEMM, desc, cfg, nullptr, A, B, C, workspace, ws_bytes, stream);
 }
 int amos_conv2d(const amos_conv_desc_t* desc, const amos_kernel_config_t* cfg, const void* X,
                 const void* Wt, void* Y, void* workspace, size_t ws_bytes, void* stream) {
-  return run_op(AMOS_OP_CONV2D, desc, cfg, X, Wt, Y, workspace, ws_bytes, stream);
+  return run_op(AMOS_OP_CONV2D, desc, cfg, nullptr, X, Wt, Y, workspace, ws_bytes, stream);
 }
 int amos_conv3d(const amos_conv_desc_t* desc, const amos_kernel_config_t* cfg, const void* X,
                 const void* Wt, void* Y, void* workspace, size_t ws_bytes, void* stream) {
-  return run_op(AMOS_OP_CONV3D, desc, cfg, X, Wt, Y, workspace, ws_bytes, stream);
+  return run_op(AMOS_OP_CONV3D, desc, cfg, nullptr, X, Wt, Y, workspace, ws_bytes, stream);
+}
+
+int amos_run_fused(int op, const void* desc, const amos_kernel_config_t* cfg,
+                   const amos_epilogue_t* epilogue, const void* in0, const void* in1, void* out,
+                   void* workspace, size_t ws_bytes, void* stream) {
+  if (op != AMOS_OP_GEMM && op != AMOS_OP_BGEMM && op != AMOS_OP_CONV2D && op != AMOS_OP_CONV3D)
+    return set_error(AMOS_ERR_BAD_ARG, "unknown op %d", op);
+  return run_op(op, desc, cfg, epilogue, in0, in1, out, workspace, ws_bytes, stream);
 }
 
 size_t amos_workspace_bytes(int op, const void* desc, const amos_kernel_config_t* cfg) {
@@ -527,11 +567,21 @@ const char* amos_kernel_name(int op, const void* desc, const amos_kernel_config_
 int amos_time(int op, const void* desc, const amos_kernel_config_t* cfg, const void* in0,
               const void* in1, void* out, void* workspace, size_t ws_bytes, void* stream_v,
               int number, int repeat, int min_repeat_ms, double* out_seconds) {
+  return amos_time_fused(op, desc, cfg, nullptr, in0, in1, out, workspace, ws_bytes, stream_v, number,
+                         repeat, min_repeat_ms, out_seconds);
+}
+
+int amos_time_fused(int op, const void* desc, const amos_kernel_config_t* cfg,
+                    const amos_epilogue_t* epilogue, const void* in0, const void* in1, void* out,
+                    void* workspace, size_t ws_bytes, void* stream_v, int number, int repeat,
+                    int min_repeat_ms, double* out_seconds) {
   if (!out_seconds || number < 1 || repeat < 1)
     return set_error(AMOS_ERR_BAD_ARG, "amos_time needs number >= 1, repeat >= 1 and an output array");
   hipStream_t stream = (hipStream_t)stream_v;
   Plan pl;
   int rc = make_plan(pl, op, desc, cfg, in0, in1, out, workspace, ws_bytes);
+  if (rc) return rc;
+  rc = plan_epilogue(pl, op, desc, epilogue);
   if (rc) return rc;
   rc = launch(pl, stream);  // warm-up
   if (rc) return rc;

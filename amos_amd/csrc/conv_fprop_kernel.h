@@ -90,6 +90,7 @@ struct ConvFpropParams {
   // prepare kernel work split (in blocks)
   int prep_w_blocks, prep_x_blocks, prep_z_blocks;
   int64_t zero_words;
+  EpiParams epi;     // fused tail: Y = acc + cast(D), D laid out like Y
 };
 
 // ---- launch 1: relayout ---------------------------------------------------------------------
@@ -576,6 +577,16 @@ __global__ __launch_bounds__(64 * NW, OCC) void amos_conv_fprop(const ConvFpropP
     for (int a = 0; a < TI; ++a) {
       const int i0 = bi0 + (wi * TI + a) * 32 + 4 * frag_half;
       out_t* const dst0 = out + (int64_t)i0 * ODPQ + coff;
+      if (p.epi.dt != EPI_NONE && blockIdx.y == 0) {   // one K split adds D; all loads first
+        out_t dv[16];
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int i = i0 + 8 * (r >> 2) + (r & 3);
+          dv[r] = epi_value<out_t>(p.epi, (int64_t)(i < p.K ? i : p.K - 1) * ODPQ + coff);
+        }
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[a][b][r] += dv[r];
+      }
       if (full) {
 #pragma unroll
         for (int r = 0; r < 16; ++r) dst0[(int64_t)(8 * (r >> 2) + (r & 3)) * ODPQ] = acc[a][b][r];

@@ -34,6 +34,7 @@ struct GemmTnParams {
   int64_t lda, ldb, ldc;
   int64_t batch_a, batch_b, batch_c;  // elements between batches
   int tiles_i, tiles_j;
+  EpiParams epi;   // fused tail: C = acc + cast(D), D[i][j] at i*epi.si + j
 };
 
 #define AMOS_GLOBAL_PTR(p) ((const __attribute__((address_space(1))) void*)(p))
@@ -164,6 +165,16 @@ __global__ __launch_bounds__(64 * WI * WJ) void amos_gemm_tn(const GemmTnParams 
     if (j >= p.J) continue;
 #pragma unroll
     for (int a = 0; a < TI; ++a) {
+      if (p.epi.dt != EPI_NONE) {   // all sixteen loads of the tile in flight before the first addition
+        out_t dv[16];
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int i = bi0 + (wi * TI + a) * 32 + 8 * (r >> 2) + 4 * frag_half + (r & 3);
+          dv[r] = epi_value<out_t>(p.epi, batch * p.epi.batch + (int64_t)(i < p.I ? i : p.I - 1) * p.epi.si + j);
+        }
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[a][b][r] += dv[r];
+      }
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
         const int i = bi0 + (wi * TI + a) * 32 + 8 * (r >> 2) + 4 * frag_half + (r & 3);

@@ -73,6 +73,29 @@ struct Mfma<DT_I8> {
   }
 };
 
+// Tail operation fused into the store: out = acc + cast(D), D an operand of the output's shape
+// (reference: the element-wise stage after the main op, hw_abstraction/cuda/wmma_bias.py:12-80,
+// tests/python/auto_tensorize/test_compute_transform_gemm.py:7-23 "E = C + D").
+enum { EPI_NONE = 0, EPI_OUT_TYPE = 1, EPI_F16 = 2, EPI_BF16 = 3 };
+struct EpiParams {
+  const char* ptr;     // D
+  int64_t si;          // elements between output rows i in D
+  int64_t batch;       // elements between batches in D
+  int dt;              // EPI_*: element type of D (EPI_OUT_TYPE = fp32 / int32 like the output)
+};
+template <typename out_t>
+__device__ __forceinline__ out_t epi_value(const EpiParams& e, int64_t idx);
+template <>
+__device__ __forceinline__ float epi_value<float>(const EpiParams& e, int64_t idx) {
+  if (e.dt == EPI_F16) return (float)((const _Float16*)e.ptr)[idx];
+  if (e.dt == EPI_BF16) return __builtin_bit_cast(float, (unsigned)((const unsigned short*)e.ptr)[idx] << 16);
+  return ((const float*)e.ptr)[idx];
+}
+template <>
+__device__ __forceinline__ int epi_value<int>(const EpiParams& e, int64_t idx) {
+  return ((const int*)e.ptr)[idx];
+}
+
 struct ConvGeom {
   int C, D, H, W;
   int T, R, S;
@@ -103,6 +126,7 @@ struct IgemmParams {
   int out_jmod;
   int64_t out_batch;
   int atomic_out;               // split-K: accumulate into a zeroed output
+  EpiParams epi;                // D is indexed like the output, with its own row stride
 };
 
 __device__ __forceinline__ int lds_chunk_offset(int row, int chunk) {
@@ -388,6 +412,7 @@ __global__ __launch_bounds__(256) void amos_igemm(const IgemmParams p) {
 
   // ---- epilogue: accumulators straight to the final layout -----------------------
   out_t* const out = (out_t*)p.out + batch * p.out_batch;
+  const bool add_d = p.epi.dt != EPI_NONE && blockIdx.y == 0;   // one K split adds D
 #pragma unroll
   for (int b = 0; b < TJ; ++b) {
     const int j = bj0 + (wj * TJ + b) * 32 + frag_row;
@@ -396,6 +421,16 @@ __global__ __launch_bounds__(256) void amos_igemm(const IgemmParams p) {
     const int64_t coff = (int64_t)jo * p.out_sjo + (j - jo * p.out_jmod);
 #pragma unroll
     for (int a = 0; a < TI; ++a) {
+      if (add_d) {   // all sixteen loads of the tile in flight before the first addition
+        out_t dv[16];
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int i = bi0 + (wi * TI + a) * 32 + 8 * (r >> 2) + 4 * frag_half + (r & 3);
+          dv[r] = epi_value<out_t>(p.epi, batch * p.epi.batch + (int64_t)(i < p.I ? i : p.I - 1) * p.epi.si + coff);
+        }
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[a][b][r] += dv[r];
+      }
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
         const int i = bi0 + (wi * TI + a) * 32 + 8 * (r >> 2) + 4 * frag_half + (r & 3);

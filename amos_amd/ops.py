@@ -48,6 +48,28 @@ def _cfg_ref(cfg):
     return ctypes.byref(cfg) if cfg is not None else None
 
 
+def make_epilogue(add, out_shape, out_dtype):
+    """None | tensor of the output's shape -> Epilogue (out = acc + add) or None.  `add` is fp32,
+    fp16 or bf16 for fp32 outputs, int32 for int32 outputs."""
+    if add is None:
+        return None
+    _need_device(add)
+    if tuple(add.shape) != tuple(out_shape):
+        raise ValueError("the added operand has shape %s, the output %s" % (tuple(add.shape), tuple(out_shape)))
+    codes = {torch.float32: _lib.AMOS_F32, torch.float16: _lib.AMOS_F16, torch.bfloat16: _lib.AMOS_BF16,
+             torch.int32: _lib.AMOS_I32}
+    ok = (torch.int32,) if out_dtype == torch.int32 else (torch.float32, torch.float16, torch.bfloat16)
+    if add.dtype not in ok:
+        raise ValueError("cannot add a %s operand to a %s output" % (add.dtype, out_dtype))
+    e = _lib.Epilogue()
+    e.kind, e.dtype, e.operand, e.ld, e.stride = _lib.AMOS_EPI_ADD, codes[add.dtype], add.data_ptr(), 0, 0
+    return e
+
+
+def _epi_ref(e):
+    return ctypes.byref(e) if e is not None else None
+
+
 def gemm_desc(M, N, K, in_dtype, trans_a=False, trans_b=False, lda=None, ldb=None, ldc=None):
     d = GemmDesc()
     d.M, d.N, d.K = M, N, K
@@ -87,8 +109,8 @@ def conv_out_shape(x_shape, w_shape, stride, pad, dil):
     return (x_shape[0], w_shape[0]) + tuple(out)
 
 
-def gemm(a, b, trans_a=False, trans_b=False, out=None, config=None, stream=None):
-    """C[M,N] = A(m,k) B(k,n); a is [M,K] ([K,M] if trans_a), b is [K,N] ([N,K] if trans_b)."""
+def gemm(a, b, trans_a=False, trans_b=False, out=None, config=None, stream=None, add=None):
+    """C[M,N] = A(m,k) B(k,n) (+ add[M,N]); a is [M,K] ([K,M] if trans_a), b is [K,N] ([N,K] if trans_b)."""
     _need_device(a, b)
     M, K = (a.shape[1], a.shape[0]) if trans_a else a.shape
     N = b.shape[0] if trans_b else b.shape[1]
@@ -99,8 +121,9 @@ def gemm(a, b, trans_a=False, trans_b=False, out=None, config=None, stream=None)
     _need_device(out)
     d = gemm_desc(M, N, K, a.dtype, trans_a, trans_b)
     cfg = make_config(config)
-    check(_lib.load().amos_gemm(ctypes.byref(d), _cfg_ref(cfg), a.data_ptr(), b.data_ptr(),
-                                out.data_ptr(), None, 0, _stream_ptr(stream)))
+    epi = make_epilogue(add, (M, N), out.dtype)
+    check(_lib.load().amos_run_fused(AMOS_OP_GEMM, ctypes.byref(d), _cfg_ref(cfg), _epi_ref(epi), a.data_ptr(),
+                                     b.data_ptr(), out.data_ptr(), None, 0, _stream_ptr(stream)))
     return out
 
 
@@ -112,7 +135,7 @@ def bgemm_desc(batch, M, N, K, in_dtype, trans_a=False, trans_b=False):
     return d
 
 
-def bgemm(a, b, trans_a=False, trans_b=False, out=None, config=None, stream=None):
+def bgemm(a, b, trans_a=False, trans_b=False, out=None, config=None, stream=None, add=None):
     """batched GEMM; a is [B,M,K] ([B,K,M] if trans_a), b is [B,K,N] ([B,N,K] if trans_b)."""
     _need_device(a, b)
     B = a.shape[0]
@@ -125,8 +148,9 @@ def bgemm(a, b, trans_a=False, trans_b=False, out=None, config=None, stream=None
     _need_device(out)
     d = bgemm_desc(B, M, N, K, a.dtype, trans_a, trans_b)
     cfg = make_config(config)
-    check(_lib.load().amos_bgemm(ctypes.byref(d), _cfg_ref(cfg), a.data_ptr(), b.data_ptr(),
-                                 out.data_ptr(), None, 0, _stream_ptr(stream)))
+    epi = make_epilogue(add, (B, M, N), out.dtype)
+    check(_lib.load().amos_run_fused(AMOS_OP_BGEMM, ctypes.byref(d), _cfg_ref(cfg), _epi_ref(epi), a.data_ptr(),
+                                     b.data_ptr(), out.data_ptr(), None, 0, _stream_ptr(stream)))
     return out
 
 
@@ -140,8 +164,8 @@ def _workspace(op, desc, cfg, device):
     return ws, ptr, need
 
 
-def conv2d(x, w, stride=1, pad=0, dil=1, out=None, config=None, stream=None):
-    """x NCHW, w KCRS -> NKPQ"""
+def conv2d(x, w, stride=1, pad=0, dil=1, out=None, config=None, stream=None, add=None):
+    """x NCHW, w KCRS -> NKPQ (+ add of the output's shape)"""
     _need_device(x, w)
     st, pd, dl = (1,) + _tup(stride, 2), (0,) + _tup(pad, 2), (1,) + _tup(dil, 2)
     xs = (x.shape[0], x.shape[1], 1, x.shape[2], x.shape[3])
@@ -156,13 +180,14 @@ def conv2d(x, w, stride=1, pad=0, dil=1, out=None, config=None, stream=None):
     d = conv_desc(xs, ws, x.dtype, st, pd, dl)
     cfg = make_config(config)
     ws, ws_ptr, ws_bytes = _workspace(AMOS_OP_CONV2D, d, cfg, x.device)
-    check(_lib.load().amos_conv2d(ctypes.byref(d), _cfg_ref(cfg), x.data_ptr(), w.data_ptr(),
-                                  out.data_ptr(), ws_ptr, ws_bytes, _stream_ptr(stream)))
+    epi = make_epilogue(add, tuple(out.shape), out.dtype)
+    check(_lib.load().amos_run_fused(AMOS_OP_CONV2D, ctypes.byref(d), _cfg_ref(cfg), _epi_ref(epi), x.data_ptr(),
+                                     w.data_ptr(), out.data_ptr(), ws_ptr, ws_bytes, _stream_ptr(stream)))
     return out
 
 
-def conv3d(x, w, stride=1, pad=0, dil=1, out=None, config=None, stream=None):
-    """x NCDHW, w KCTRS -> NKDPQ"""
+def conv3d(x, w, stride=1, pad=0, dil=1, out=None, config=None, stream=None, add=None):
+    """x NCDHW, w KCTRS -> NKDPQ (+ add of the output's shape)"""
     _need_device(x, w)
     st, pd, dl = _tup(stride, 3), _tup(pad, 3), _tup(dil, 3)
     if x.shape[1] != w.shape[1] or x.dtype != w.dtype:
@@ -174,20 +199,23 @@ def conv3d(x, w, stride=1, pad=0, dil=1, out=None, config=None, stream=None):
     d = conv_desc(tuple(x.shape), tuple(w.shape), x.dtype, st, pd, dl)
     cfg = make_config(config)
     ws, ws_ptr, ws_bytes = _workspace(AMOS_OP_CONV3D, d, cfg, x.device)
-    check(_lib.load().amos_conv3d(ctypes.byref(d), _cfg_ref(cfg), x.data_ptr(), w.data_ptr(),
-                                  out.data_ptr(), ws_ptr, ws_bytes, _stream_ptr(stream)))
+    epi = make_epilogue(add, tuple(out.shape), out.dtype)
+    check(_lib.load().amos_run_fused(AMOS_OP_CONV3D, ctypes.byref(d), _cfg_ref(cfg), _epi_ref(epi), x.data_ptr(),
+                                     w.data_ptr(), out.data_ptr(), ws_ptr, ws_bytes, _stream_ptr(stream)))
     return out
 
 
-def time_op(op, desc, in0, in1, out, config=None, number=100, repeat=1, min_repeat_ms=150, stream=None):
+def time_op(op, desc, in0, in1, out, config=None, number=100, repeat=1, min_repeat_ms=150, stream=None,
+            add=None):
     """mean seconds per launch, `repeat` values (time_evaluator semantics)"""
     _need_device(in0, in1, out)
     cfg = make_config(config)
     res = (ctypes.c_double * repeat)()
     ws, ws_ptr, ws_bytes = _workspace(op, desc, cfg, in0.device)
-    check(_lib.load().amos_time(op, ctypes.byref(desc), _cfg_ref(cfg), in0.data_ptr(), in1.data_ptr(),
-                                out.data_ptr(), ws_ptr, ws_bytes, _stream_ptr(stream), number, repeat,
-                                min_repeat_ms, res))
+    epi = make_epilogue(add, tuple(out.shape), out.dtype)
+    check(_lib.load().amos_time_fused(op, ctypes.byref(desc), _cfg_ref(cfg), _epi_ref(epi), in0.data_ptr(),
+                                      in1.data_ptr(), out.data_ptr(), ws_ptr, ws_bytes, _stream_ptr(stream),
+                                      number, repeat, min_repeat_ms, res))
     return list(res)
 
 

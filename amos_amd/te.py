@@ -309,7 +309,10 @@ _AXIS_NAMES = "ijklmnopqrstuvwxyz"
 
 def compute(shape, fcompute, name="compute", tag="", attrs=None):
     shape = [int(s) for s in shape]
-    params = list(inspect.signature(fcompute).parameters)
+    sig = inspect.signature(fcompute).parameters
+    params = list(sig)
+    if len(params) == 1 and sig[params[0]].kind == inspect.Parameter.VAR_POSITIONAL:
+        params = ["i%d" % d for d in range(len(shape))]     # lambda *indices, as TVM names them
     if len(params) != len(shape):
         raise ValueError("fcompute takes %d indices for a %d-d output" % (len(params), len(shape)))
     axis = [IterVar((0, ext), pname) for pname, ext in zip(params, shape)]

@@ -73,23 +73,27 @@ def run_all_configs(cpu=True):
     f16 = lambda x: x.astype(np.float32).astype(np.float16)
     rows = []
 
-    def gpu_time(op, desc, i0, i1, out):
+    def gpu_time(op, desc, i0, i1, out, fused=None):
         cfg = ops.default_config(op, desc)
-        t = ops.time_op(op, desc, i0, i1, out, config=cfg, number=20, repeat=3, min_repeat_ms=100)
+        t = ops.time_op(op, desc, i0, i1, out, config=cfg, number=20, repeat=3, min_repeat_ms=100, add=fused)
         return min(t), cfg
 
-    def add(name, op, desc, hin, dtype, flop, nbytes, out_shape, cpu_fn, frac):
+    def add(name, op, desc, hin, dtype, flop, nbytes, out_shape, cpu_fn, frac, fused_tail=False):
         tin = [torch.from_numpy(h).cuda() for h in hin]
         out = torch.empty(out_shape, dtype=torch.int32 if dtype == "int8" else torch.float32,
                           device="cuda")
-        sec, cfg = gpu_time(op, desc, tin[0], tin[1], out)
+        # fused tail out = acc + D: D has the output's shape and type, read once more
+        fused = torch.ones_like(out) if fused_tail else None
+        if fused_tail:
+            nbytes += out.numel() * 4
+        sec, cfg = gpu_time(op, desc, tin[0], tin[1], out, fused)
         peak = PEAK_I8_TOPS if dtype == "int8" else PEAK_F16_TFLOPS
         t_mfma, t_hbm = flop / (peak * 1e12), nbytes / (PEAK_HBM_GBS * 1e9)
         row = {"config": name, "kernel": ops.kernel_name(op, desc, cfg), "split_k": cfg.split_k,
                "gpu_us": sec * 1e6, "tflops": flop / sec / 1e12,
                "pct_mfma_peak": 100 * t_mfma / sec, "pct_hbm_roof": 100 * t_hbm / sec,
                "bound": "mfma" if t_mfma >= t_hbm else "hbm", "flop": flop, "bytes": nbytes}
-        if cpu:
+        if cpu and cpu_fn is not None:
             t1 = _timed(lambda: cpu_fn(1, False))
             tn = _timed(lambda: cpu_fn(cores, True))
             row["cpu"] = {"kind": "port (te_literal loop nest, gcc -O3)",
@@ -107,6 +111,9 @@ def run_all_configs(cpu=True):
         [a, b], "float16", 2.0 * n ** 3, 2 * n * n * 2 + n * n * 4, (n, n),
         lambda th, big: co.te_literal_gemm(a, b, "float16", False, True, rows=(0, 8 * th), threads=th),
         (8 / n, 8 * cores / n))
+    add("C2 + D: fp16 GEMM 8192^3 with the fused tail E = C + D (D fp32)", _lib.AMOS_OP_GEMM,
+        ops.gemm_desc(n, n, n, torch.float16, False, True), [a, b], "float16", 2.0 * n ** 3,
+        2 * n * n * 2 + n * n * 4, (n, n), None, None, fused_tail=True)
     # C3 fp16 conv2d
     x = f16(rng.uniform(0, 1, (32, 256, 14, 14)))
     w = f16(rng.standard_normal((256, 256, 3, 3)) * 0.05)
@@ -115,6 +122,9 @@ def run_all_configs(cpu=True):
         [x, w], "float16", 2.0 * 6272 * 256 * 2304, 10813440, (32, 256, 14, 14),
         lambda th, big: co.te_literal_conv2d(x, w, "float16", 1, 1, 1, images=(0, 2 * th), threads=th),
         (2 / 32, min(32, 2 * cores) / 32))
+    add("C3 + D: fp16 conv2d with the fused tail (D fp32, NKPQ)", _lib.AMOS_OP_CONV2D,
+        ops.conv_desc((32, 256, 1, 14, 14), (256, 256, 1, 3, 3), torch.float16, (1, 1, 1), (0, 1, 1), (1, 1, 1)),
+        [x, w], "float16", 2.0 * 6272 * 256 * 2304, 10813440, (32, 256, 14, 14), None, None, fused_tail=True)
     # C4 int8 conv2d
     xi = rng.integers(-128, 128, (64, 128, 28, 28)).astype(np.int8)
     wi = rng.integers(-64, 64, (128, 128, 3, 3)).astype(np.int8)

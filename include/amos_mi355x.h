@@ -171,6 +171,27 @@ int amos_conv2d(const amos_conv_desc_t* desc, const amos_kernel_config_t* cfg, c
 int amos_conv3d(const amos_conv_desc_t* desc, const amos_kernel_config_t* cfg, const void* X,
                 const void* Wt, void* Y, void* workspace, size_t ws_bytes, void* stream);
 
+/* A tail operation fused into the store of the accumulators.  AMOS_EPI_ADD: out = acc + cast(D),
+ * D an operand with the output's shape: GEMM / batched GEMM [M][ld] (ld 0 = N) with `stride`
+ * elements between batches (0 = M*ld); convolution NKDPQ, contiguous.  D is fp32, fp16 or bf16
+ * for fp32 outputs and int32 for int32 outputs.  (reference: the element-wise stage behind the
+ * main op, python/tvm/auto_tensorize/hw_abstraction/cuda/wmma_bias.py:12-80 and
+ * tests/python/auto_tensorize/test_compute_transform_gemm.py:7-23, "E = C + D") */
+#define AMOS_EPI_NONE 0
+#define AMOS_EPI_ADD 1
+typedef struct {
+  int32_t kind;          /* AMOS_EPI_* */
+  int32_t dtype;         /* amos_dtype_t of the operand */
+  const void* operand;   /* device pointer */
+  int64_t ld;
+  int64_t stride;
+} amos_epilogue_t;
+/* any of the four ops with a fused tail (epilogue NULL = none); in0, in1, out as in the op's own
+ * entry point */
+int amos_run_fused(int op, const void* desc, const amos_kernel_config_t* cfg,
+                   const amos_epilogue_t* epilogue, const void* in0, const void* in1, void* out,
+                   void* workspace, size_t ws_bytes, void* stream);
+
 /*
  * Mean seconds per launch, measured the way the reference's time_evaluator does
  * (reference: src/runtime/rpc/rpc_module.cc:355-388): one warm-up launch, then
@@ -181,6 +202,11 @@ int amos_conv3d(const amos_conv_desc_t* desc, const amos_kernel_config_t* cfg, c
 int amos_time(int op, const void* desc, const amos_kernel_config_t* cfg, const void* in0,
               const void* in1, void* out, void* workspace, size_t ws_bytes, void* stream,
               int number, int repeat, int min_repeat_ms, double* out_seconds);
+
+int amos_time_fused(int op, const void* desc, const amos_kernel_config_t* cfg,
+                    const amos_epilogue_t* epilogue, const void* in0, const void* in1, void* out,
+                    void* workspace, size_t ws_bytes, void* stream, int number, int repeat,
+                    int min_repeat_ms, double* out_seconds);
 
 /* name of the kernel instance a (desc, cfg) pair dispatches to, e.g.
  * "amos_igemm<f16,vec,vec,256x256>"; replaces func.imported_modules[0].get_source()

@@ -94,3 +94,39 @@ def test_v4_explores_the_realised_mappings(gpu, tmp_path, capsys):
     y = tvm.nd.array(np.zeros([int(s) for s in Conv.shape], dtype=np.int32), ctx)
     func(tvm.nd.array(a, ctx), tvm.nd.array(b, ctx), y)
     assert np.array_equal(y.asnumpy(), co.lib_conv2d(a, b, "int8", 1, 1, 1))
+
+
+def test_gemm_with_elementwise_tail(gpu, tmp_path):
+    """E = C + D behind the GEMM, the compute of the reference's
+    tests/python/auto_tensorize/test_compute_transform_gemm.py:7-23, through the script flow:
+    the tail is fused into the kernel and D becomes the module's third input"""
+    M, N, K = 256, 192, 320
+    A = tvm.te.placeholder([M, K], dtype="float16", name="A")
+    B = tvm.te.placeholder([K, N], dtype="float16", name="B")
+    tk = tvm.te.reduce_axis([0, K], name="tk")
+    C = tvm.te.compute([M, N], lambda ti, tj: tvm.te.sum((A[ti, tk] * B[tk, tj]).astype("float32"), axis=tk),
+                       name="C")
+    D = tvm.te.placeholder([M, N], dtype="float32", name="D")
+    E = tvm.te.compute([M, N], lambda si, sj: C[si, sj] + D[si, sj], name="E")
+    dag = at.compute_dag_from_tensors([E])
+    opt = at.MeasureOptions(target="hip", timeout=100, number=5, min_repeat_ms=5)
+    result = at.auto_tensorize(dag, "hip", str(tmp_path / "gemm_tail.log"), opt, trials=4)
+    assert result.defined()
+    assert result.sch_app.lowered.add_input is D
+    sch, args = at.get_schedule(result.sch_app, result.params)
+    assert [t.name for t in args] == ["A", "B", "D", "E"]
+    func = tvm.build(sch, args, "hip")
+    rng = np.random.default_rng(2)
+    a = rng.uniform(-1, 1, (M, K)).astype(np.float16)
+    b = rng.uniform(-1, 1, (K, N)).astype(np.float16)
+    d = rng.uniform(-1, 1, (M, N)).astype(np.float32)
+    ctx = tvm.context("hip", 0)
+    e = tvm.nd.array(np.zeros((M, N), dtype=np.float32), ctx)
+    func(tvm.nd.array(a, ctx), tvm.nd.array(b, ctx), tvm.nd.array(d, ctx), e)
+    ctx.sync()
+    ref = co.lib_gemm(a, b, "float16", 0, 0, acc="float64") + d
+    mx, mean = co.rel_errors(e.asnumpy(), ref)
+    assert mx <= 1e-2 and mean <= 1e-3
+    t = func.time_evaluator(func.entry_name, ctx, number=5, min_repeat_ms=5)(
+        tvm.nd.array(a, ctx), tvm.nd.array(b, ctx), tvm.nd.array(d, ctx), e).mean
+    assert 0 < t < 1e-2

@@ -8,6 +8,7 @@ import numpy as np
 import pytest
 
 from amos_amd import _lib, te
+import amos_amd.tvm as tvm
 from amos_amd.te import tir
 from amos_amd import auto_tensorize as at
 from amos_amd.auto_tensorize import hw_abs_dag as dagmod
@@ -327,3 +328,59 @@ def test_fragment_layout_is_a_bijection():
         d = {lay["d"](l, r) for l in range(64) for r in range(lay["acc_regs"])}
         assert a == {(i, kk) for i in range(m) for kk in range(k)}
         assert d == {(i, j) for i in range(m) for j in range(n)}
+
+
+# ---- element-wise tail behind the main op (reference: tests/python/auto_tensorize/
+# test_compute_transform_gemm.py:7-23, hw_abs_dag/cuda/wmma_fp16_bias.py) ---------------------
+def _gemm_with_tail(M, N, K, d_dtype="float32", tail="add"):
+    A = tvm.te.placeholder([M, K], dtype="float16", name="A")
+    B = tvm.te.placeholder([K, N], dtype="float16", name="B")
+    tk = tvm.te.reduce_axis([0, K], name="tk")
+    C = tvm.te.compute([M, N], lambda ti, tj: tvm.te.sum((A[ti, tk] * B[tk, tj]).astype("float32"), axis=tk),
+                       name="C")
+    D = tvm.te.placeholder([M, N], dtype=d_dtype, name="D")
+
+    def body(si, sj):
+        d = D[si, sj] if d_dtype == "float32" else D[si, sj].astype("float32")
+        return C[si, sj] + d if tail == "add" else C[si, sj] * d
+    E = tvm.te.compute([M, N], body, name="E")
+    return A, B, D, E
+
+
+def test_tail_addition_is_fused_at_lowering():
+    from amos_amd.auto_tensorize.lowering import NoKernelError, lower_main_op
+    for d_dtype in ("float32", "float16", "bfloat16"):
+        A, B, D, E = _gemm_with_tail(128, 128, 128, d_dtype)
+        dag = at.compute_dag_from_tensors([E])
+        assert [op.name for op in dag.op_lst] == ["C", "E"]
+        # the tail does not change what matches: the main op alone, as for the plain GEMM
+        results = at.get_match_results(dag, "hip")
+        assert len(results) == 8 and all(list(r.main_op_map.values())[0] is dag.op_lst[0] for r in results)
+        low = lower_main_op(dag.op_lst[0], dag)
+        assert low.kind == "gemm" and low.add_input is D and low.output is E
+        assert [t.name for t in dag.get_inputs()] == ["A", "B", "D"]
+    A, B, D, E = _gemm_with_tail(128, 128, 128, tail="mul")
+    dag = at.compute_dag_from_tensors([E])
+    with pytest.raises(NoKernelError, match="not an element-wise addition"):
+        lower_main_op(dag.op_lst[0], dag)
+    A, B, D, E = _gemm_with_tail(128, 128, 128, "int32")
+    with pytest.raises(NoKernelError, match="cannot add"):
+        dag = at.compute_dag_from_tensors([E])
+        lower_main_op(dag.op_lst[0], dag)
+
+
+def test_bias_dag_is_unregistered_and_has_two_ops():
+    dag_cls = at.MFMAFp16Fp32Bias
+    assert dag_cls not in at.query_hw_abs_dag("hip")
+    hw = dag_cls()
+    assert hw.get_name() == "mfma_f16_f32_bias" and hw.anchor_point == "bias"
+    assert hw.edges["bias"] == ["mma", "load_bias"] and hw.edges["store"] == ["bias"]
+    intrin_dag, main = hw.get_effective_compute_dag("nnn", "32x32x16")
+    assert len(intrin_dag.op_lst) == 2 and intrin_dag.op_lst[0] is main[0].op
+    # the mapping the reference's test4 states by hand: main op <-> C, element-wise op <-> E
+    A, B, D, E = _gemm_with_tail(128, 128, 128, "float16")
+    target = at.compute_dag_from_tensors([E])
+    main_op_map = {intrin_dag.op_lst[0]: target.op_lst[0]}
+    elem_op_map = {intrin_dag.op_lst[1]: target.op_lst[1]}
+    assert at.intrinsic_match(target.op_lst[0], intrin_dag.op_lst[0])
+    assert len(main_op_map) == 1 and len(elem_op_map) == 1
