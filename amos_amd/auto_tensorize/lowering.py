@@ -132,6 +132,134 @@ def _lower_gemm(main_op, l0, l1, iters, forms0, forms1):
     return LoweredOp("bgemm", _lib.AMOS_OP_BGEMM, b, [la.tensor, lb.tensor], main_op.output(0), attrs)
 
 
+def _row_major_strides(shape):
+    strides, acc = [], 1
+    for ext in reversed([int(x) for x in shape]):
+        strides.append(acc)
+        acc *= ext
+    return list(reversed(strides))
+
+
+def _flat_address(load, variables):
+    """Element offset of a tensor load inside the PLACEHOLDER it ultimately reads, as an affine
+    form ({Var: coefficient}, constant) of `variables`.  Pure view stages in between -- computes
+    without a reduction whose body is one load with affine indices, the reshapes of
+    benchmark/amos/mapping_batchedfc_tensorcore.py:14-22 -- are substituted away.  None when
+    the chain is not affine or changes values."""
+    forms = [te.affine_form(i, variables) for i in load.indices]
+    if any(f is None for f in forms):
+        return None
+    op = load.tensor.op
+    if isinstance(op, te.PlaceholderOp):
+        coef, const = {}, 0
+        for f, stride in zip(forms, _row_major_strides(load.tensor.shape)):
+            for v, c in f[0].items():
+                coef[v] = coef.get(v, 0) + c * stride
+            const += f[1] * stride
+        return load.tensor, {v: c for v, c in coef.items() if c != 0}, const
+    if not isinstance(op, te.ComputeOp) or op.reduce_axis:
+        return None
+    inner = op.body[0]
+    if isinstance(inner, te.Cast) and inner.dtype == inner.value.dtype:
+        inner = inner.value
+    if not isinstance(inner, te.ProducerLoad) or inner.dtype != load.dtype:
+        return None
+    view_vars = [iv.var for iv in op.axis]
+    res = _flat_address(inner, view_vars)
+    if res is None:
+        return None
+    src, icoef, iconst = res
+    coef, const = {}, iconst
+    for vv, f in zip(view_vars, forms):       # substitute view variable := the load's index form
+        c = icoef.get(vv, 0)
+        if c == 0:
+            continue
+        for v, cc in f[0].items():
+            coef[v] = coef.get(v, 0) + c * cc
+        const += c * f[1]
+    return src, {v: c for v, c in coef.items() if c != 0}, const
+
+
+def _lower_strided_gemm(main_op, l0, l1):
+    """GEMM, batched GEMM and their strided relatives (GEMV, batched FC over channel groups,
+    operands read through reshaping stages) from the flat addresses of the two loads: a spatial
+    iteration variable in one operand only is M or N, in both it is the batch; leading
+    dimensions and batch strides are the coefficients.  (reference computes:
+    benchmark/amos/mapping_gemm_tensorcore.py:7-15, mapping_gemv_tensorcore.py:7-16,
+    mapping_batchedfc_tensorcore.py:7-37)"""
+    spatial, reduce_ = list(main_op.axis), list(main_op.reduce_axis)
+    if len(reduce_) != 1:
+        return None
+    variables = [iv.var for iv in spatial + reduce_]
+    r0, r1 = _flat_address(l0, variables), _flat_address(l1, variables)
+    if r0 is None or r1 is None or r0[2] != 0 or r1[2] != 0:
+        return None
+    k = reduce_[0]
+    if k.var not in r0[1] or k.var not in r1[1]:
+        return None
+    live = [iv for iv in spatial if int(iv.dom.extent) > 1]
+    in0 = [iv for iv in live if iv.var in r0[1]]
+    in1 = [iv for iv in live if iv.var in r1[1]]
+    batch = [iv for iv in in0 if any(iv is j for j in in1)]
+    only0 = [iv for iv in in0 if not any(iv is j for j in batch)]
+    only1 = [iv for iv in in1 if not any(iv is j for j in batch)]
+    if len(batch) > 1 or len(only0) > 1 or len(only1) > 1 or len(batch) + len(only0) + len(only1) != len(live):
+        return None
+    out_strides = dict(zip([iv.var for iv in spatial], _row_major_strides(main_op.output(0).shape)))
+
+    def roles(ra, rb, m_iv, n_iv):
+        """A-side / B-side description with (m_iv from ra, n_iv from rb), or None"""
+        K = int(k.dom.extent)
+        M = int(m_iv.dom.extent) if m_iv is not None else 1
+        N = int(n_iv.dom.extent) if n_iv is not None else 1
+        a_m = ra[1].get(m_iv.var, 0) if m_iv is not None else 0
+        a_k = ra[1][k.var]
+        b_n = rb[1].get(n_iv.var, 0) if n_iv is not None else 0
+        b_k = rb[1][k.var]
+        if a_k == 1 and (M == 1 or a_m >= K):
+            trans_a, lda = 0, (a_m if M > 1 else K)
+        elif (a_m == 1 or M == 1) and a_k >= M:
+            trans_a, lda = 1, a_k
+        else:
+            return None
+        if b_k == 1 and (N == 1 or b_n >= K):
+            trans_b, ldb = 1, (b_n if N > 1 else K)
+        elif (b_n == 1 or N == 1) and b_k >= N:
+            trans_b, ldb = 0, b_k
+        else:
+            return None
+        c_m = out_strides[m_iv.var] if m_iv is not None else N
+        c_n = out_strides[n_iv.var] if n_iv is not None else 1
+        if (N > 1 and c_n != 1) or (M > 1 and c_m < N):
+            return None
+        return dict(M=M, N=N, K=K, trans_a=trans_a, trans_b=trans_b, lda=lda, ldb=ldb, ldc=c_m if M > 1 else N)
+
+    m_iv = only0[0] if only0 else None
+    n_iv = only1[0] if only1 else None
+    la, lb, ra, rb = l0, l1, r0, r1
+    g = roles(ra, rb, m_iv, n_iv)
+    if g is None:       # the other operand supplies the output rows
+        la, lb, ra, rb, m_iv, n_iv = l1, l0, r1, r0, n_iv, m_iv
+        g = roles(ra, rb, m_iv, n_iv)
+    if g is None:
+        return None
+    ind, outd = _dtype_pair(la, lb, main_op.output(0))
+    d = _lib.GemmDesc()
+    d.M, d.N, d.K, d.in_dtype, d.out_dtype = g["M"], g["N"], g["K"], ind, outd
+    d.trans_a, d.trans_b, d.lda, d.ldb, d.ldc = g["trans_a"], g["trans_b"], g["lda"], g["ldb"], g["ldc"]
+    attrs = dict(M=g["M"], N=g["N"], K=g["K"], trans_a=g["trans_a"], trans_b=g["trans_b"], dtype=la.dtype,
+                 lda=g["lda"], ldb=g["ldb"], ldc=g["ldc"])
+    if not batch:
+        return LoweredOp("gemm", _lib.AMOS_OP_GEMM, d, [ra[0], rb[0]], main_op.output(0), attrs)
+    b_iv = batch[0]
+    bd = _lib.BGemmDesc()
+    bd.batch = int(b_iv.dom.extent)
+    bd.g = d
+    bd.stride_a, bd.stride_b, bd.stride_c = ra[1][b_iv.var], rb[1][b_iv.var], out_strides[b_iv.var]
+    attrs.update(batch=bd.batch, stride_a=bd.stride_a, stride_b=bd.stride_b, stride_c=bd.stride_c)
+    return LoweredOp("bgemm", _lib.AMOS_OP_BGEMM, bd, [ra[0], rb[0]], main_op.output(0), attrs)
+
+
 def _pad_stage(tensor):
     """tensor made by the padding compute -> (source placeholder, pads per spatial dim)"""
     op = tensor.op
@@ -168,8 +296,8 @@ def _pad_stage(tensor):
 
 def _lower_conv(main_op, l0, l1, iters, forms0, forms1):
     spatial, reduce_ = list(main_op.axis), list(main_op.reduce_axis)
-    nsp = len(spatial) - 2                     # 2 or 3 spatial output dims
-    if nsp not in (2, 3) or len(reduce_) != nsp + 1:
+    nsp = len(spatial) - 2                     # 1, 2 or 3 spatial output dims
+    if nsp not in (1, 2, 3) or len(reduce_) != nsp + 1:
         return None
     n_iv, k_iv, out_sp = spatial[0], spatial[1], spatial[2:]
     rc, red_sp = reduce_[0], reduce_[1:]
@@ -222,7 +350,10 @@ def _lower_conv(main_op, l0, l1, iters, forms0, forms1):
         raise NoKernelError("grouped convolution has no kernel")
     ind, outd = _dtype_pair(lx, lw, main_op.output(0))
     c = _lib.ConvDesc()
-    if nsp == 2:
+    if nsp == 1:      # conv1d (benchmark/amos/mapping_conv1d_tensorcore.py:25-42) = conv2d with H = R = 1
+        xs5, ws5 = [xs[0], xs[1], 1, 1, xs[2]], [ws[0], ws[1], 1, 1, ws[2]]
+        st, pd, dl = [1, 1] + strides, [0, 0] + pads, [1, 1] + dils
+    elif nsp == 2:
         xs5, ws5 = [xs[0], xs[1], 1, xs[2], xs[3]], [ws[0], ws[1], 1, ws[2], ws[3]]
         st, pd, dl = [1] + strides, [0] + pads, [1] + dils
     else:
@@ -239,8 +370,39 @@ def _lower_conv(main_op, l0, l1, iters, forms0, forms1):
         J *= e
     attrs = dict(x_shape=xs, w_shape=ws, stride=strides, pad=pads, dil=dils, dtype=lx.dtype, J=J,
                  K_out=ws[0], K_red=ws[1] * (ws5[2] * ws5[3] * ws5[4]))
-    kind, code = ("conv2d", _lib.AMOS_OP_CONV2D) if nsp == 2 else ("conv3d", _lib.AMOS_OP_CONV3D)
+    kind, code = ("conv2d", _lib.AMOS_OP_CONV2D) if nsp <= 2 else ("conv3d", _lib.AMOS_OP_CONV3D)
     return LoweredOp(kind, code, c, [src, lw.tensor], main_op.output(0), attrs)
+
+
+def _numel(shape):
+    n = 1
+    for e in shape:
+        n *= int(e)
+    return n
+
+
+def _dense_output(low):
+    """the kernel writes the main op's tensor contiguously (no padding between rows / batches)"""
+    if low.kind == "gemm":
+        return low.desc.ldc == low.desc.N
+    if low.kind == "bgemm":
+        return low.desc.g.ldc == low.desc.g.N and low.desc.stride_c == low.desc.g.M * low.desc.g.N
+    return True
+
+
+def _flat_address_of_compute(load, producer_op, variables):
+    """offset of a load of `producer_op`'s (row-major) result, affine in `variables`"""
+    if load.tensor.op is not producer_op:
+        return None
+    forms = [te.affine_form(i, variables) for i in load.indices]
+    if any(f is None for f in forms):
+        return None
+    coef, const = {}, 0
+    for f, stride in zip(forms, _row_major_strides(load.tensor.shape)):
+        for v, c in f[0].items():
+            coef[v] = coef.get(v, 0) + c * stride
+        const += f[1] * stride
+    return {v: c for v, c in coef.items() if c != 0}, const
 
 
 def _fuse_tail(low, main_op, target_dag):
@@ -257,6 +419,17 @@ def _fuse_tail(low, main_op, target_dag):
     if any(any(t.op is tail for t in op.input_tensors) for op in target_dag.op_lst):
         raise NoKernelError("a chain of stages behind the main op has no fused kernel")
     body = tail.body[0] if not tail.reduce_axis else None
+    if isinstance(_strip_cast(body), te.ProducerLoad) and _strip_cast(body).dtype == low.output.dtype:
+        # a reshape of the result (mapping_gemv_tensorcore.py:15, D[i] = C[i, 0]): same memory
+        variables = [iv.var for iv in tail.axis]
+        res = _flat_address_of_compute(_strip_cast(body), main_op, variables)
+        want = dict(zip(variables, _row_major_strides(tail.output(0).shape)))
+        want = {v: c for v, c in want.items() if int([iv for iv in tail.axis if iv.var is v][0].dom.extent) > 1}
+        if res is not None and res[1] == 0 and {v: c for v, c in res[0].items()} == want and \
+                _numel(tail.output(0).shape) == _numel(main_op.output(0).shape) and _dense_output(low):
+            low.output = tail.output(0)
+            return low
+        raise NoKernelError("stage %s behind the main op is neither a reshape nor an addition" % tail.name)
     if not isinstance(body, te.Add):
         raise NoKernelError("stage %s behind the main op is not an element-wise addition" % tail.name)
     loads = [_strip_cast(body.a), _strip_cast(body.b)]
@@ -295,6 +468,9 @@ def _lower_main_op(main_op):
     variables = [iv.var for iv in iters]
     forms0 = [te.affine_form(i, variables) for i in l0.indices]
     forms1 = [te.affine_form(i, variables) for i in l1.indices]
+    low = _lower_strided_gemm(main_op, l0, l1)
+    if low is not None:
+        return low
     for fn in (_lower_gemm, _lower_conv):
         low = fn(main_op, l0, l1, iters, forms0, forms1)
         if low is not None:

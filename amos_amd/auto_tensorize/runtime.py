@@ -100,16 +100,8 @@ class Module(object):
         return out
 
     def _run(self, in0, in1, out, add=None):
-        low, cfg = self.lowered, self.params.to_config() if self.params is not None else None
-        a = low.attrs
-        if low.kind == "gemm":
-            ops.gemm(in0, in1, a["trans_a"], a["trans_b"], out=out, config=cfg, add=add)
-        elif low.kind == "bgemm":
-            ops.bgemm(in0, in1, a["trans_a"], a["trans_b"], out=out, config=cfg, add=add)
-        elif low.kind == "conv2d":
-            ops.conv2d(in0, in1, a["stride"], a["pad"], a["dil"], out=out, config=cfg, add=add)
-        else:
-            ops.conv3d(in0, in1, a["stride"], a["pad"], a["dil"], out=out, config=cfg, add=add)
+        cfg = self.params.to_config() if self.params is not None else None
+        ops.run_desc(self.lowered.op_code, self.lowered.desc, in0, in1, out, config=cfg, add=add)
 
     def __call__(self, *arrays):
         self._run(*self._pick(arrays))

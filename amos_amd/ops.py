@@ -205,6 +205,32 @@ def conv3d(x, w, stride=1, pad=0, dil=1, out=None, config=None, stream=None, add
     return out
 
 
+def _epilogue_for(op, desc, add, out):
+    """Epilogue for an operand laid out like the output the descriptor describes"""
+    if add is None:
+        return None
+    if add.numel() != out.numel():
+        raise ValueError("the added operand has %d elements, the output %d" % (add.numel(), out.numel()))
+    epi = make_epilogue(add, tuple(add.shape), out.dtype)
+    if op == AMOS_OP_GEMM:
+        epi.ld = desc.ldc
+    elif op == AMOS_OP_BGEMM:
+        epi.ld, epi.stride = desc.g.ldc, desc.stride_c
+    return epi
+
+
+def run_desc(op, desc, in0, in1, out, config=None, stream=None, add=None):
+    """launch an op from its C descriptor (leading dimensions and batch strides as the descriptor
+    says; the tensors only supply the device memory)"""
+    _need_device(in0, in1, out)
+    cfg = make_config(config)
+    ws, ws_ptr, ws_bytes = _workspace(op, desc, cfg, in0.device)
+    epi = _epilogue_for(op, desc, add, out)
+    check(_lib.load().amos_run_fused(op, ctypes.byref(desc), _cfg_ref(cfg), _epi_ref(epi), in0.data_ptr(),
+                                     in1.data_ptr(), out.data_ptr(), ws_ptr, ws_bytes, _stream_ptr(stream)))
+    return out
+
+
 def time_op(op, desc, in0, in1, out, config=None, number=100, repeat=1, min_repeat_ms=150, stream=None,
             add=None):
     """mean seconds per launch, `repeat` values (time_evaluator semantics)"""
@@ -212,7 +238,7 @@ def time_op(op, desc, in0, in1, out, config=None, number=100, repeat=1, min_repe
     cfg = make_config(config)
     res = (ctypes.c_double * repeat)()
     ws, ws_ptr, ws_bytes = _workspace(op, desc, cfg, in0.device)
-    epi = make_epilogue(add, tuple(out.shape), out.dtype)
+    epi = _epilogue_for(op, desc, add, out)
     check(_lib.load().amos_time_fused(op, ctypes.byref(desc), _cfg_ref(cfg), _epi_ref(epi), in0.data_ptr(),
                                       in1.data_ptr(), out.data_ptr(), ws_ptr, ws_bytes, _stream_ptr(stream),
                                       number, repeat, min_repeat_ms, res))

@@ -9,7 +9,7 @@ import pytest
 import amos_amd.tvm as tvm
 from amos_amd.tvm import auto_tensorize as at
 from oracle import cpu_oracle as co
-from test_mapper import conv2d, gemm
+from test_mapper import batched_fc, conv1d, conv2d, gemm, gemv
 
 pytestmark = pytest.mark.gpu
 
@@ -130,3 +130,69 @@ def test_gemm_with_elementwise_tail(gpu, tmp_path):
     t = func.time_evaluator(func.entry_name, ctx, number=5, min_repeat_ms=5)(
         tvm.nd.array(a, ctx), tvm.nd.array(b, ctx), tvm.nd.array(d, ctx), e).mean
     assert 0 < t < 1e-2
+
+
+def _run_script_flow(tensors, feeds, tmp_path, name, **kwargs):
+    """auto_tensorize -> get_schedule -> build -> func(*arrays); returns the output array"""
+    dag = at.compute_dag_from_tensors([tensors[-1]])
+    opt = at.MeasureOptions(target="hip", timeout=100, number=5, min_repeat_ms=5)
+    result = at.auto_tensorize(dag, "hip", str(tmp_path / (name + ".log")), opt, trials=4, **kwargs)
+    assert result.defined()
+    sch, args = at.get_schedule(result.sch_app, result.params)
+    func = tvm.build(sch, args, "hip")
+    ctx = tvm.context("hip", 0)
+    arrays = [tvm.nd.array(feeds[t.name], ctx) for t in args[:-1]]
+    out = tvm.nd.array(np.zeros([int(s) for s in args[-1].shape], dtype=args[-1].dtype), ctx)
+    func(*arrays, out)
+    ctx.sync()
+    return out.asnumpy(), result
+
+
+def test_gemv_script_flow(gpu, tmp_path):
+    """reference compute: benchmark/amos/mapping_gemv_tensorcore.py:7-16 (GEMM with N = 1 and a
+    reshaping stage behind it)"""
+    M, K = 1000, 520
+    A, B, D = gemv(M, K)
+    rng = np.random.default_rng(5)
+    a = rng.uniform(-1, 1, (M, K)).astype(np.float16)
+    b = rng.uniform(-1, 1, (K, 1)).astype(np.float16)
+    with pytest.raises(RuntimeError, match="infeasible"):   # N = 1 < 16: the strict rule of the reference
+        _run_script_flow([A, B, D], {"A": a, "B": b}, tmp_path, "gemv_strict")
+    got, result = _run_script_flow([A, B, D], {"A": a, "B": b}, tmp_path, "gemv", transform_strict=False)
+    assert got.shape == (M,) and result.sch_app.lowered.kind == "gemm"
+    ref = (a.astype(np.float64) @ b.astype(np.float64))[:, 0]
+    mx, mean = co.rel_errors(got, ref)
+    assert mx <= 1e-2 and mean <= 1e-3
+
+
+def test_batched_fc_script_flow(gpu, tmp_path):
+    """reference compute: benchmark/amos/mapping_batchedfc_tensorcore.py:7-37 (channel groups
+    read through reshaping stages: a batched GEMM with strided batches)"""
+    N, I, O, groups = 96, 512, 384, 4
+    A, B, F = batched_fc(N, I, O, groups)
+    rng = np.random.default_rng(6)
+    a = rng.uniform(-1, 1, (N, I)).astype(np.float16)
+    b = rng.uniform(-1, 1, (O, I // groups)).astype(np.float16)
+    got, result = _run_script_flow([A, B, F], {"A": a, "B": b}, tmp_path, "bfc")
+    assert result.sch_app.lowered.kind == "bgemm"
+    a64 = a.astype(np.float64).reshape(N, groups, I // groups)
+    b64 = b.astype(np.float64).reshape(groups, O // groups, I // groups)
+    ref = np.einsum("ngc,gkc->ngk", a64, b64)
+    mx, mean = co.rel_errors(got, ref)
+    assert got.shape == (N, groups, O // groups) and mx <= 1e-2 and mean <= 1e-3
+
+
+@pytest.mark.parametrize("C", [64, 24])    # patch-staged and register-staged kernels
+def test_conv1d_script_flow(gpu, tmp_path, C):
+    """reference compute: benchmark/amos/mapping_conv1d_tensorcore.py:7-42"""
+    N, L, K, KL, stride, padding, dilation = 4, 200, 48, 5, 2, 2, 1
+    A, B, Out = conv1d(N, C, L, K, KL, stride, padding, dilation)
+    rng = np.random.default_rng(7)
+    a = rng.uniform(-1, 1, (N, C, L)).astype(np.float16)
+    b = rng.uniform(-1, 1, (K, C, KL)).astype(np.float16)
+    got, result = _run_script_flow([A, B, Out], {"A": a, "B": b}, tmp_path, "conv1d")
+    assert result.sch_app.lowered.kind == "conv2d"
+    ref = co.lib_conv2d(a[:, :, None, :], b[:, :, None, :], "float16", (1, stride), (0, padding), (1, dilation),
+                        acc="float64")[:, :, 0, :]
+    mx, mean = co.rel_errors(got, ref)
+    assert got.shape == ref.shape and mx <= 1e-2 and mean <= 1e-3

@@ -384,3 +384,106 @@ def test_bias_dag_is_unregistered_and_has_two_ops():
     elem_op_map = {intrin_dag.op_lst[1]: target.op_lst[1]}
     assert at.intrinsic_match(target.op_lst[0], intrin_dag.op_lst[0])
     assert len(main_op_map) == 1 and len(elem_op_map) == 1
+
+
+# ---- more operators through the same lowering (reference: benchmark/amos/mapping_gemv_tensorcore.py:7-16,
+# mapping_batchedfc_tensorcore.py:7-37, mapping_conv1d_tensorcore.py:7-42) --------------------------
+def gemv(M, K, in_dtype="float16", out_dtype="float32"):
+    A = te.placeholder([M, K], dtype=in_dtype, name="A")
+    B = te.placeholder([K, 1], dtype=in_dtype, name="B")
+    rk = te.reduce_axis([0, K], name="k")
+    C = te.compute([M, 1], lambda i, j: te.sum((A[i, rk] * B[rk, j]).astype(out_dtype), axis=rk), name="C")
+    D = te.compute([M], lambda i: C[i, 0], name="D")
+    return A, B, D
+
+
+def batched_fc(N, I, O, groups, in_dtype="float16", out_dtype="float32"):
+    cpg, ocpg = I // groups, O // groups
+    A = te.placeholder([N, I], dtype=in_dtype, name="A")
+    B = te.placeholder([O, cpg], dtype=in_dtype, name="B")
+    A_reshaped = te.compute([N, groups, cpg], lambda n, c_o, c_i: A[n, c_o * cpg + c_i])
+    B_reshaped = te.compute([groups, ocpg, cpg], lambda k_o, k_i, c: B[k_o * ocpg + k_i, c])
+    rc = te.reduce_axis([0, cpg], name="rc")
+    BFC = te.compute([N, groups, ocpg], lambda n, k_o, k_i: te.sum(
+        (A_reshaped[n, k_o, rc] * B_reshaped[k_o, k_i, rc]).astype(out_dtype), axis=[rc]), name="BatchedFC")
+    return A, B, BFC
+
+
+def conv1d(N, C, L, K, KL, stride, padding, dilation, in_dtype="float16", out_dtype="float32"):
+    A = te.placeholder([N, C, L], dtype=in_dtype, name="A")
+    B = te.placeholder([K, C, KL], dtype=in_dtype, name="B")
+    out_len = (L + 2 * padding - dilation * (KL - 1) - 1) // stride + 1
+    rc = te.reduce_axis((0, C), name="rc")
+    rl = te.reduce_axis((0, KL), name="rl")
+    padded = te.compute((N, C, L + 2 * padding), lambda b, c, l: tir.if_then_else(
+        tir.all(l >= padding, l < L + padding), A[b, c, l - padding], tir.const(0, A.dtype)))
+    conved = te.compute((N, K, out_len), lambda b, k, l: te.sum(
+        (padded[b, rc, l * stride + rl * dilation] * B[k, rc, rl]).astype(out_dtype), axis=[rc, rl]))
+    return A, B, conved
+
+
+def gemm_from_desc(low, a, b):
+    """what the C descriptor of a lowered GEMM / batched GEMM says, evaluated with numpy on the
+    flat operand buffers (float64)"""
+    d = low.desc.g if low.kind == "bgemm" else low.desc
+    batch, sa, sb, sc = (low.desc.batch, low.desc.stride_a, low.desc.stride_b, low.desc.stride_c) \
+        if low.kind == "bgemm" else (1, 0, 0, 0)
+    a, b = a.astype(np.float64).ravel(), b.astype(np.float64).ravel()
+    out = np.zeros(max(1, (batch - 1) * sc + (d.M - 1) * d.ldc + d.N))
+    for g in range(batch):
+        for i in range(d.M):
+            for j in range(d.N):
+                ai = [g * sa + (k * d.lda + i if d.trans_a else i * d.lda + k) for k in range(d.K)]
+                bi = [g * sb + (j * d.ldb + k if d.trans_b else k * d.ldb + j) for k in range(d.K)]
+                out[g * sc + i * d.ldc + j] = float(np.dot(a[ai], b[bi]))
+    return out
+
+
+@pytest.mark.parametrize("build", [lambda: gemv(24, 40), lambda: batched_fc(6, 32, 24, 4),
+                                   lambda: gemm(20, 12, 16, ta=True, tb=True, batch=3)])
+def test_strided_gemm_lowering_keeps_the_meaning(build):
+    from amos_amd.auto_tensorize.lowering import lower_main_op
+    A, B, Out = build()
+    dag = at.compute_dag_from_tensors([Out])
+    main = [op for op in dag.op_lst if op.reduce_axis][0]
+    low = lower_main_op(main, dag)
+    assert low.kind in ("gemm", "bgemm") and [t.name for t in low.inputs] == ["A", "B"] and low.output is Out
+    rng = np.random.default_rng(3)
+    a = rng.integers(-4, 5, [int(s) for s in A.shape]).astype(np.float64)
+    b = rng.integers(-4, 5, [int(s) for s in B.shape]).astype(np.float64)
+    want = te_interp.evaluate(Out, {"A": a, "B": b})
+    got = gemm_from_desc(low, a, b)
+    assert got.size == want.size and np.array_equal(got, want.ravel())
+
+
+def test_gemv_and_batched_fc_descriptors():
+    from amos_amd.auto_tensorize.lowering import lower_main_op
+    A, B, D = gemv(256, 512)
+    dag = at.compute_dag_from_tensors([D])
+    low = lower_main_op(dag.op_lst[0], dag)
+    g = low.desc
+    assert (low.kind, g.M, g.N, g.K, g.trans_a, g.trans_b, g.lda, g.ldc) == ("gemm", 256, 1, 512, 0, 1, 512, 1)
+    A, B, F = batched_fc(64, 512, 256, 4)
+    dag = at.compute_dag_from_tensors([F])
+    low = lower_main_op([op for op in dag.op_lst if op.reduce_axis][0], dag)
+    d = low.desc
+    assert (low.kind, d.batch, d.g.M, d.g.N, d.g.K) == ("bgemm", 4, 64, 64, 128)
+    assert (d.g.trans_a, d.g.trans_b, d.g.lda, d.g.ldb, d.g.ldc) == (0, 1, 512, 128, 256)
+    assert (d.stride_a, d.stride_b, d.stride_c) == (128, 64 * 128, 64)
+
+
+def test_conv1d_lowers_to_conv2d_with_unit_height():
+    from amos_amd.auto_tensorize.lowering import lower_main_op
+    A, B, Out = conv1d(2, 16, 30, 8, 3, 2, 1, 2)
+    dag = at.compute_dag_from_tensors([Out])
+    low = lower_main_op([op for op in dag.op_lst if op.reduce_axis][0], dag)
+    c = low.desc
+    assert low.kind == "conv2d" and (c.N, c.C, c.D, c.H, c.W, c.K, c.T, c.R, c.S) == (2, 16, 1, 1, 30, 8, 1, 1, 3)
+    assert (c.stride_h, c.stride_w, c.pad_h, c.pad_w, c.dil_h, c.dil_w) == (1, 2, 0, 1, 1, 2)
+    rng = np.random.default_rng(4)
+    a = rng.integers(-3, 4, (2, 16, 30)).astype(np.float64)
+    b = rng.integers(-3, 4, (8, 16, 3)).astype(np.float64)
+    want = te_interp.evaluate(Out, {"A": a, "B": b})
+    ref = co.lib_conv2d(a[:, :, None, :].astype(np.float16), b[:, :, None, :].astype(np.float16), "float16",
+                        (1, 2), (0, 1), (1, 2), acc="float64")
+    assert np.array_equal(ref[:, :, 0, :], want)
