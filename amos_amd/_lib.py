@@ -44,7 +44,7 @@ class ConvDesc(ctypes.Structure):
                 ("stride_d", _i32), ("stride_h", _i32), ("stride_w", _i32),
                 ("pad_d", _i32), ("pad_h", _i32), ("pad_w", _i32),
                 ("dil_d", _i32), ("dil_h", _i32), ("dil_w", _i32),
-                ("in_dtype", _i32), ("out_dtype", _i32)]
+                ("in_dtype", _i32), ("out_dtype", _i32), ("groups", _i32), ("reserved", _i32)]
 
 
 class KernelConfig(ctypes.Structure):

@@ -391,17 +391,32 @@ def _dense_output(low):
 
 
 def _flat_address_of_compute(load, producer_op, variables):
-    """offset of a load of `producer_op`'s (row-major) result, affine in `variables`"""
+    """offset of a load of `producer_op`'s (row-major) result, affine in `variables`.  An index
+    pair (v // c, v % c) whose strides are (c*s, s) counts as v*s: the split of one axis in two
+    that mapping_groupedconv2d_tensorcore.py:53-57 undoes behind its main op."""
     if load.tensor.op is not producer_op:
         return None
-    forms = [te.affine_form(i, variables) for i in load.indices]
-    if any(f is None for f in forms):
-        return None
-    coef, const = {}, 0
-    for f, stride in zip(forms, _row_major_strides(load.tensor.shape)):
+    coef, const, div, mod = {}, 0, {}, {}
+    for idx, stride in zip(load.indices, _row_major_strides(load.tensor.shape)):
+        e = _strip_cast(idx)
+        if isinstance(e, (te.FloorDiv, te.FloorMod)) and isinstance(e.a, te.Var) and isinstance(e.b, te.IntImm) \
+                and any(e.a is v for v in variables):
+            bucket = div if isinstance(e, te.FloorDiv) else mod
+            key = (e.a, int(e.b.value))
+            bucket[key] = bucket.get(key, 0) + stride
+            continue
+        f = te.affine_form(idx, variables)
+        if f is None:
+            return None
         for v, c in f[0].items():
             coef[v] = coef.get(v, 0) + c * stride
         const += f[1] * stride
+    if set(div) != set(mod):
+        return None
+    for (v, c), s_mod in mod.items():
+        if div[(v, c)] != c * s_mod:
+            return None
+        coef[v] = coef.get(v, 0) + s_mod
     return {v: c for v, c in coef.items() if c != 0}, const
 
 
@@ -455,6 +470,129 @@ def _fuse_tail(low, main_op, target_dag):
     return low
 
 
+def _resolve_dims(load, variables):
+    """(tensor, per-dimension affine index forms in `variables`) of the first tensor behind `load`
+    that is not a pure view stage; None if an index is not affine"""
+    forms = [te.affine_form(i, variables) for i in load.indices]
+    if any(f is None for f in forms):
+        return None
+    op = load.tensor.op
+    if isinstance(op, te.ComputeOp) and not op.reduce_axis:
+        inner = op.body[0]
+        if isinstance(inner, te.Cast) and inner.dtype == inner.value.dtype:
+            inner = inner.value
+        if isinstance(inner, te.ProducerLoad) and inner.dtype == load.dtype:
+            view_vars = [iv.var for iv in op.axis]
+            res = _resolve_dims(inner, view_vars)
+            if res is None:
+                return None
+            tensor, inner_forms = res
+            out = []
+            for icoef, iconst in inner_forms:       # substitute view variable := the load's index form
+                coef, const = {}, iconst
+                for vv, f in zip(view_vars, forms):
+                    c = icoef.get(vv, 0)
+                    for v, cc in f[0].items():
+                        coef[v] = coef.get(v, 0) + c * cc
+                    const += c * f[1]
+                out.append(({v: c for v, c in coef.items() if c != 0}, const))
+            return tensor, out
+    return load.tensor, forms
+
+
+def _lower_grouped_conv(main_op, l0, l1):
+    """Grouped and depthwise convolution as the reference spells them
+    (benchmark/amos/mapping_groupedconv2d_tensorcore.py:7-60, mapping_depthwiseconv2d_tensorcore.py:7-48):
+    output [N, groups, K/groups, spatial...], the activations' channel index is
+    group * (C/groups) + rc (or the group alone when C/groups = 1), the weights are read through a
+    reshaping stage.  Lowered to the convolution descriptor with `groups`."""
+    spatial, reduce_ = list(main_op.axis), list(main_op.reduce_axis)
+    nsp = len(spatial) - 3
+    if nsp not in (1, 2, 3) or len(reduce_) not in (nsp, nsp + 1):
+        return None
+    n_iv, g_iv, k_iv, out_sp = spatial[0], spatial[1], spatial[2], spatial[3:]
+    rc = reduce_[0] if len(reduce_) == nsp + 1 else None
+    red_sp = reduce_[1:] if rc is not None else reduce_
+    variables = [iv.var for iv in spatial + reduce_]
+    G, Kg = int(g_iv.dom.extent), int(k_iv.dom.extent)
+    Cg = int(rc.dom.extent) if rc is not None else 1
+
+    def try_roles(lx, lw):
+        rx, rw = _resolve_dims(lx, variables), _flat_address(lw, variables)
+        if rx is None or rw is None or rw[2] != 0:
+            return None
+        xt, fx = rx
+        if len(fx) != nsp + 2 or fx[0] != ({n_iv.var: 1}, 0):
+            return None
+        want_c = {g_iv.var: Cg}
+        if rc is not None:
+            want_c[rc.var] = 1
+        if fx[1] != (want_c, 0):
+            return None
+        strides, dils = [], []
+        for d in range(nsp):
+            coef, const = fx[2 + d]
+            if const != 0 or set(coef) - {out_sp[d].var, red_sp[d].var}:
+                return None
+            strides.append(int(coef.get(out_sp[d].var, 1)))
+            dils.append(int(coef.get(red_sp[d].var, 1)))
+        # weights: a dense [K][Cg][window...] placeholder, however it is reshaped on the way
+        win = [int(r.dom.extent) for r in red_sp]
+        trs = 1
+        for e in win:
+            trs *= e
+        want = {g_iv.var: Kg * Cg * trs, k_iv.var: Cg * trs}
+        if rc is not None:
+            want[rc.var] = trs
+        acc = 1
+        for r in reversed(red_sp):
+            want[r.var] = acc
+            acc *= int(r.dom.extent)
+        want = {v: c for v, c in want.items() if c != 0 and
+                int([iv for iv in spatial + reduce_ if iv.var is v][0].dom.extent) > 1}
+        got = {v: c for v, c in rw[1].items()
+               if int([iv for iv in spatial + reduce_ if iv.var is v][0].dom.extent) > 1}
+        if got != want or _numel(rw[0].shape) != G * Kg * Cg * trs:
+            return None
+        return xt, rw[0], strides, dils, win
+
+    roles, lx, lw = try_roles(l0, l1), l0, l1
+    if roles is None:
+        roles, lx, lw = try_roles(l1, l0), l1, l0
+    if roles is None:
+        return None
+    xt, wt, strides, dils, win = roles
+    src, pads = _pad_stage(xt)
+    xs = [int(s) for s in src.shape]
+    if xs[1] != G * Cg:
+        raise NoKernelError("activations have %d channels, the compute reads %d groups of %d" % (xs[1], G, Cg))
+    for d in range(nsp):
+        want = (xs[2 + d] + 2 * pads[d] - ((win[d] - 1) * dils[d] + 1)) // strides[d] + 1
+        if int(out_sp[d].dom.extent) != want:
+            raise NoKernelError("output extent %d is not what stride / padding / dilation give (%d)"
+                                % (int(out_sp[d].dom.extent), want))
+    ind, outd = _dtype_pair(lx, lw, main_op.output(0))
+    c = _lib.ConvDesc()
+    lead = 3 - nsp
+    xs5 = xs[:2] + [1] * lead + xs[2:]
+    ws5 = [G * Kg, Cg] + [1] * lead + win
+    st, pd, dl = [1] * lead + strides, [0] * lead + pads, [1] * lead + dils
+    c.N, c.C, c.D, c.H, c.W = xs5
+    c.K, _, c.T, c.R, c.S = ws5
+    c.stride_d, c.stride_h, c.stride_w = st
+    c.pad_d, c.pad_h, c.pad_w = pd
+    c.dil_d, c.dil_h, c.dil_w = dl
+    c.in_dtype, c.out_dtype = ind, outd
+    c.groups = G
+    J = xs[0]
+    for iv in out_sp:
+        J *= int(iv.dom.extent)
+    attrs = dict(x_shape=xs, w_shape=[G * Kg, Cg] + win, stride=strides, pad=pads, dil=dils, dtype=lx.dtype,
+                 J=J, K_out=G * Kg, K_red=Cg * _numel(win), groups=G)
+    kind, code = ("conv2d", _lib.AMOS_OP_CONV2D) if nsp <= 2 else ("conv3d", _lib.AMOS_OP_CONV3D)
+    return LoweredOp(kind, code, c, [src, wt], main_op.output(0), attrs)
+
+
 def lower_main_op(main_op, target_dag=None):
     """ComputeOp that matched a GEMM-like intrinsic -> LoweredOp; with the compute DAG it
     belongs to, an element-wise addition behind it is fused into the kernel"""
@@ -468,9 +606,10 @@ def _lower_main_op(main_op):
     variables = [iv.var for iv in iters]
     forms0 = [te.affine_form(i, variables) for i in l0.indices]
     forms1 = [te.affine_form(i, variables) for i in l1.indices]
-    low = _lower_strided_gemm(main_op, l0, l1)
-    if low is not None:
-        return low
+    for fn in (_lower_strided_gemm, _lower_grouped_conv):
+        low = fn(main_op, l0, l1)
+        if low is not None:
+            return low
     for fn in (_lower_gemm, _lower_conv):
         low = fn(main_op, l0, l1, iters, forms0, forms1)
         if low is not None:

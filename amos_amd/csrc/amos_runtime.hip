@@ -62,6 +62,7 @@ struct Plan {
   int split;
   // zero fill of the output before a split-K launch
   int64_t fill_rows, fill_cols, fill_ld;
+  int fill_once;
   // direct-to-LDS GEMM pipeline (0 = not used, else waves per block)
   int tn_waves;
   GemmTnParams tn;
@@ -209,13 +210,18 @@ static int plan_conv(Plan& pl, int op, const amos_conv_desc_t* d, const amos_ker
     return set_error(AMOS_ERR_BAD_ARG, "conv extents, strides and dilations must be positive, pads >= 0");
   int rc = dtype_pair(c.in_dtype, c.out_dtype, &pl.dt);
   if (rc) return rc;
+  const int64_t G = c.groups > 1 ? c.groups : 1;
+  if (c.C % G || c.K % G)
+    return set_error(AMOS_ERR_BAD_ARG, "groups (%lld) must divide C (%lld) and K (%lld)", (long long)G,
+                     (long long)c.C, (long long)c.K);
+  const int64_t Cg = c.C / G, Kg = c.K / G;
   int OD = conv_out_extent(c.D, c.pad_d, c.dil_d, c.T, c.stride_d);
   int OP = conv_out_extent(c.H, c.pad_h, c.dil_h, c.R, c.stride_h);
   int OQ = conv_out_extent(c.W, c.pad_w, c.dil_w, c.S, c.stride_w);
   if (OD <= 0 || OP <= 0 || OQ <= 0)
     return set_error(AMOS_ERR_BAD_ARG, "kernel window larger than the padded input");
   int64_t J = c.N * OD * (int64_t)OP * OQ;
-  int64_t Kred = c.C * c.T * c.R * c.S;
+  int64_t Kred = Cg * c.T * c.R * c.S;
   int64_t per_image = c.C * c.D * c.H * c.W;
   if (!fits_int(J) || !fits_int(Kred) || !fits_int(per_image) || !fits_int(c.K))
     return set_error(AMOS_ERR_UNSUPPORTED, "conv extents above 2^31");
@@ -225,17 +231,19 @@ static int plan_conv(Plan& pl, int op, const amos_conv_desc_t* d, const amos_ker
   const int ce = 16 / es;
   IgemmParams& p = pl.p;
   memset(&p, 0, sizeof(p));
-  p.I = (int)c.K;
+  p.I = (int)Kg;
   p.J = (int)J;
   p.Kred = (int)Kred;
   p.row_base = (const char*)Wt;
   p.row_s_row = Kred;
   p.row_s_k = 1;
+  p.row_batch = Kg * Kred;                        // group g: its Kg output channels' weights ...
+  p.col_batch = Cg * c.D * c.H * c.W;             // ... its Cg input channels of every image ...
   pl.rl = (aligned16(Wt) && Kred % ce == 0) ? LD_VEC : LD_STRIDED;
   p.col_base = (const char*)X;
   pl.cl = LD_CONV;
   ConvGeom& g = p.g;
-  g.C = (int)c.C; g.D = (int)c.D; g.H = (int)c.H; g.W = (int)c.W;
+  g.C = (int)Cg; g.Cimg = (int)c.C; g.D = (int)c.D; g.H = (int)c.H; g.W = (int)c.W;
   g.T = (int)c.T; g.R = (int)c.R; g.S = (int)c.S;
   g.sd = c.stride_d; g.sh = c.stride_h; g.sw = c.stride_w;
   g.pd = c.pad_d; g.ph = c.pad_h; g.pw = c.pad_w;
@@ -247,11 +255,12 @@ static int plan_conv(Plan& pl, int op, const amos_conv_desc_t* d, const amos_ker
   p.out_si = odpq;
   p.out_sjo = c.K * odpq;
   p.out_jmod = (int)odpq;
-  p.out_batch = 0;
-  pl.batch = 1;
+  p.out_batch = Kg * odpq;                        // ... its Kg channels of every output image
+  pl.batch = G;
   pl.fill_rows = 1;
   pl.fill_cols = c.N * c.K * odpq;
   pl.fill_ld = pl.fill_cols;
+  pl.fill_once = 1;                               // the whole output in one fill, not per group
   rc = plan_finish(pl, op, d, cfg);
   if (rc) return rc;
 
@@ -334,6 +343,7 @@ static int make_plan(Plan& pl, int op, const void* desc, const amos_kernel_confi
                      size_t ws_bytes = 0) {
   pl.tn_waves = 0;
   pl.conv_ups = 0;
+  pl.fill_once = 0;
   switch (op) {
     case AMOS_OP_GEMM:
       return plan_gemm(pl, op, desc, (const amos_gemm_desc_t*)desc, 1, 0, 0, 0, cfg, in0, in1, out);
@@ -425,7 +435,7 @@ static int launch(const Plan& pl, hipStream_t stream) {
     int64_t n = pl.fill_rows * pl.fill_cols * pl.batch;
     int blocks = (int)((n + 255) / 256 < 4096 ? (n + 255) / 256 : 4096);
     // batched outputs are contiguous per batch only when stride_c == M*ldc; fill per batch
-    for (int64_t b = 0; b < pl.batch; ++b) {
+    for (int64_t b = 0; b < (pl.fill_once ? 1 : pl.batch); ++b) {
       char* base = pl.p.out + b * pl.p.out_batch * 4;
       if (pl.dt == DT_I8)
         hipLaunchKernelGGL(fill_zero_kernel<int>, dim3(blocks), dim3(256), 0, stream, (int*)base,
@@ -462,6 +472,7 @@ static int plan_epilogue(Plan& pl, int op, const void* desc, const amos_epilogue
       ep.batch = e->stride > 0 ? e->stride : g.M * ep.si;
     } else {
       ep.si = pl.p.out_si;   // D is laid out like the output, NKDPQ
+      ep.batch = pl.p.out_batch;
     }
   }
   pl.p.epi = ep;

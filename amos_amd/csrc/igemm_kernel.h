@@ -97,7 +97,8 @@ __device__ __forceinline__ int epi_value<int>(const EpiParams& e, int64_t idx) {
 }
 
 struct ConvGeom {
-  int C, D, H, W;
+  int C, D, H, W;   // C = channels that are reduced over (of one group)
+  int Cimg;         // channels between images in memory (all groups)
   int T, R, S;
   int sd, sh, sw;
   int pd, ph, pw;
@@ -231,7 +232,7 @@ __global__ __launch_bounds__(256) void amos_igemm(const IgemmParams p) {
     cv_d0 = od * p.g.sd - p.g.pd;
     cv_h0 = op * p.g.sh - p.g.ph;
     cv_w0 = oq * p.g.sw - p.g.pw;
-    cv_base = (int64_t)img * p.g.C * p.g.D * p.g.H * p.g.W +
+    cv_base = (int64_t)img * p.g.Cimg * p.g.D * p.g.H * p.g.W +
               ((int64_t)cv_d0 * p.g.H + cv_h0) * p.g.W + cv_w0;
     if (p.g.use_mask && cv_valid) {
       int tap = 0;

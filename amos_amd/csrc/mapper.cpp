@@ -56,13 +56,16 @@ int problem_of(int op, const void* desc, Problem* out) {
       int64_t OQ = conv_out(c->W, c->pad_w, c->dil_w, c->S, c->stride_w);
       if (OD <= 0 || OP <= 0 || OQ <= 0)
         return set_error(AMOS_ERR_BAD_ARG, "kernel window larger than the padded input");
-      out->I = c->K;
+      const int64_t G = c->groups > 1 ? c->groups : 1;
+      if (c->C % G || c->K % G)
+        return set_error(AMOS_ERR_BAD_ARG, "groups (%lld) must divide C and K", (long long)G);
+      out->I = c->K / G;
       out->J = c->N * OD * OP * OQ;
-      out->K = c->C * T * c->R * c->S;
-      out->batch = 1;
+      out->K = c->C / G * T * c->R * c->S;
+      out->batch = G;
       out->in_dtype = c->in_dtype;
       out->in_bytes = (c->N * c->C * D * c->H * c->W + c->K * out->K) * esize(c->in_dtype);
-      out->out_bytes = out->I * out->J * 4;
+      out->out_bytes = c->K * out->J * 4;
       return 0;
     }
   }
@@ -111,7 +114,7 @@ int64_t conv_relaid_bytes(const amos_conv_desc_t& c, int op) {
 }
 int64_t conv_workspace_bytes(const amos_conv_desc_t& c, int op) {
   int64_t packed = conv_packed_bytes(c, op);
-  if (packed == 0) return 0;
+  if (packed == 0 || c.groups > 1) return 0;
   int64_t T = op == AMOS_OP_CONV2D ? 1 : c.T;
   int es = c.in_dtype == AMOS_I8 ? 1 : 2;
   int64_t steps = T * c.R * c.S * (c.C * es / 128);
@@ -151,6 +154,7 @@ static ConvPatchPlan conv_patch_plan_waves(const amos_conv_desc_t& cin, int op, 
                                      (BI == 128 && (BJ == 64 || BJ == 128 || BJ == 256)) ||
                                      (BI == 256 && (BJ == 64 || BJ == 128)));
   if (OD <= 0 || OP <= 0 || OQ <= 0) { pp.why = "empty output"; return pp; }
+  if (c.groups > 1) { pp.why = "grouped convolution runs on the register-staged kernel"; return pp; }
   if (packed == 0) { pp.why = "C * element size is not a multiple of 128 bytes"; return pp; }
   if (packed >= ((int64_t)1 << 31)) { pp.why = "packed weights above 2 GiB"; return pp; }
   if (conv_relaid_bytes(c, op) + 256 >= ((int64_t)1 << 32)) { pp.why = "activations above 4 GiB"; return pp; }

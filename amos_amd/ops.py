@@ -82,11 +82,15 @@ def gemm_desc(M, N, K, in_dtype, trans_a=False, trans_b=False, lda=None, ldb=Non
     return d
 
 
-def conv_desc(x_shape, w_shape, in_dtype, stride, pad, dil):
-    """x_shape NCDHW, w_shape KCTRS; stride / pad / dil are 3-tuples"""
+def conv_desc(x_shape, w_shape, in_dtype, stride, pad, dil, groups=1):
+    """x_shape NCDHW, w_shape K,(C/groups),T,R,S; stride / pad / dil are 3-tuples"""
     d = ConvDesc()
     d.N, d.C, d.D, d.H, d.W = x_shape
-    d.K, _, d.T, d.R, d.S = w_shape
+    d.K, cg, d.T, d.R, d.S = w_shape
+    if cg * groups != d.C:
+        raise ValueError("weights have %d channels per group, activations %d channels in %d groups"
+                         % (cg, d.C, groups))
+    d.groups = groups
     d.stride_d, d.stride_h, d.stride_w = stride
     d.pad_d, d.pad_h, d.pad_w = pad
     d.dil_d, d.dil_h, d.dil_w = dil
@@ -164,20 +168,20 @@ def _workspace(op, desc, cfg, device):
     return ws, ptr, need
 
 
-def conv2d(x, w, stride=1, pad=0, dil=1, out=None, config=None, stream=None, add=None):
-    """x NCHW, w KCRS -> NKPQ (+ add of the output's shape)"""
+def conv2d(x, w, stride=1, pad=0, dil=1, out=None, config=None, stream=None, add=None, groups=1):
+    """x NCHW, w K,(C/groups),R,S -> NKPQ (+ add of the output's shape)"""
     _need_device(x, w)
     st, pd, dl = (1,) + _tup(stride, 2), (0,) + _tup(pad, 2), (1,) + _tup(dil, 2)
     xs = (x.shape[0], x.shape[1], 1, x.shape[2], x.shape[3])
     ws = (w.shape[0], w.shape[1], 1, w.shape[2], w.shape[3])
-    if x.shape[1] != w.shape[1] or x.dtype != w.dtype:
+    if x.shape[1] != w.shape[1] * groups or x.dtype != w.dtype:
         raise ValueError("operand shapes / dtypes do not agree")
     oshape = conv_out_shape(xs, ws, st, pd, dl)
     if out is None:
         out = torch.empty((oshape[0], oshape[1], oshape[3], oshape[4]), dtype=_OUT_OF[x.dtype],
                           device=x.device)
     _need_device(out)
-    d = conv_desc(xs, ws, x.dtype, st, pd, dl)
+    d = conv_desc(xs, ws, x.dtype, st, pd, dl, groups)
     cfg = make_config(config)
     ws, ws_ptr, ws_bytes = _workspace(AMOS_OP_CONV2D, d, cfg, x.device)
     epi = make_epilogue(add, tuple(out.shape), out.dtype)
@@ -186,17 +190,17 @@ def conv2d(x, w, stride=1, pad=0, dil=1, out=None, config=None, stream=None, add
     return out
 
 
-def conv3d(x, w, stride=1, pad=0, dil=1, out=None, config=None, stream=None, add=None):
-    """x NCDHW, w KCTRS -> NKDPQ (+ add of the output's shape)"""
+def conv3d(x, w, stride=1, pad=0, dil=1, out=None, config=None, stream=None, add=None, groups=1):
+    """x NCDHW, w K,(C/groups),T,R,S -> NKDPQ (+ add of the output's shape)"""
     _need_device(x, w)
     st, pd, dl = _tup(stride, 3), _tup(pad, 3), _tup(dil, 3)
-    if x.shape[1] != w.shape[1] or x.dtype != w.dtype:
+    if x.shape[1] != w.shape[1] * groups or x.dtype != w.dtype:
         raise ValueError("operand shapes / dtypes do not agree")
     oshape = conv_out_shape(tuple(x.shape), tuple(w.shape), st, pd, dl)
     if out is None:
         out = torch.empty(oshape, dtype=_OUT_OF[x.dtype], device=x.device)
     _need_device(out)
-    d = conv_desc(tuple(x.shape), tuple(w.shape), x.dtype, st, pd, dl)
+    d = conv_desc(tuple(x.shape), tuple(w.shape), x.dtype, st, pd, dl, groups)
     cfg = make_config(config)
     ws, ws_ptr, ws_bytes = _workspace(AMOS_OP_CONV3D, d, cfg, x.device)
     epi = make_epilogue(add, tuple(out.shape), out.dtype)

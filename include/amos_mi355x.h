@@ -31,7 +31,7 @@
 extern "C" {
 #endif
 
-#define AMOS_ABI_VERSION 1
+#define AMOS_ABI_VERSION 2
 
 /* error codes */
 #define AMOS_OK 0
@@ -102,8 +102,12 @@ typedef struct {
  * Y[n,k,od,op,oq] = sum_{c,t,r,s} X[n,c, od*sd+t*dd-pd, op*sh+r*dh-ph, oq*sw+s*dw-pw] * Wt[k,c,t,r,s]
  * with out-of-range X reads = 0.  X is NCDHW, Wt is KCTRS, Y is NKDPQ, all dense.
  * conv2d is the D = T = 1, sd = dd = 1, pd = 0 case.
+ * groups > 1: channel group g of X (C/groups channels) meets output channels
+ * [g*K/groups, (g+1)*K/groups) only; Wt is [K][C/groups][T][R][S].  groups = C is the
+ * depthwise convolution with K/C outputs per channel.
  * (reference computes: benchmark/amos/mapping_conv2d_tensorcore.py:7-42,
- *  benchmark/amos/mapping_conv3d_tensorcore.py:7-55)
+ *  benchmark/amos/mapping_conv3d_tensorcore.py:7-55, mapping_groupedconv2d_tensorcore.py:7-60,
+ *  mapping_depthwiseconv2d_tensorcore.py:7-48)
  */
 typedef struct {
   int64_t N, C, D, H, W;
@@ -112,6 +116,8 @@ typedef struct {
   int32_t pad_d, pad_h, pad_w;
   int32_t dil_d, dil_h, dil_w;
   int32_t in_dtype, out_dtype;
+  int32_t groups;        /* 0 or 1 = ordinary convolution */
+  int32_t reserved;
 } amos_conv_desc_t;
 
 /*

@@ -24,13 +24,14 @@ def test_every_declared_symbol_is_exported():
     for n in names:
         assert hasattr(lib, n), "libamos_mi355x.so does not export %s" % n
     assert sorted(_lib.EXPORTS) == names
-    assert lib.amos_version() == 1
+    assert lib.amos_version() == 2
 
 
 def test_struct_sizes_match_header():
     assert ctypes.sizeof(_lib.GemmDesc) == 3 * 8 + 4 * 4 + 3 * 8
     assert ctypes.sizeof(_lib.BGemmDesc) == 8 + ctypes.sizeof(_lib.GemmDesc) + 3 * 8
-    assert ctypes.sizeof(_lib.ConvDesc) == 9 * 8 + 11 * 4 + 4
+    assert ctypes.sizeof(_lib.ConvDesc) == 9 * 8 + 13 * 4 + 4 and _lib.ConvDesc.groups.offset == 9 * 8 + 11 * 4
+    assert ctypes.sizeof(_lib.Epilogue) == 32 and _lib.Epilogue.operand.offset == 8
     assert ctypes.sizeof(_lib.KernelConfig) == 32
     assert _lib.KernelConfig.pipeline.offset == 12
 

@@ -9,7 +9,8 @@ import pytest
 import amos_amd.tvm as tvm
 from amos_amd.tvm import auto_tensorize as at
 from oracle import cpu_oracle as co
-from test_mapper import batched_fc, conv1d, conv2d, gemm, gemv
+from test_mapper import (batched_fc, conv1d, conv2d, depthwise_conv2d, gemm, gemv, grouped_conv2d,
+                         grouped_conv_reference)
 
 pytestmark = pytest.mark.gpu
 
@@ -194,5 +195,27 @@ def test_conv1d_script_flow(gpu, tmp_path, C):
     assert result.sch_app.lowered.kind == "conv2d"
     ref = co.lib_conv2d(a[:, :, None, :], b[:, :, None, :], "float16", (1, stride), (0, padding), (1, dilation),
                         acc="float64")[:, :, 0, :]
+    mx, mean = co.rel_errors(got, ref)
+    assert got.shape == ref.shape and mx <= 1e-2 and mean <= 1e-3
+
+
+@pytest.mark.parametrize("kind", ["grouped", "depthwise"])
+def test_grouped_conv_script_flow(gpu, tmp_path, kind):
+    """reference computes: benchmark/amos/mapping_groupedconv2d_tensorcore.py:7-60,
+    mapping_depthwiseconv2d_tensorcore.py:7-48"""
+    if kind == "grouped":
+        N, C, H, W, K, R, S, stride, padding, groups = 4, 64, 14, 14, 128, 3, 3, 1, 1, 4
+        A, B, Out = grouped_conv2d(N, C, H, W, K, R, S, stride, padding, groups)
+    else:
+        N, C, H, W, K, R, S, stride, padding = 2, 32, 14, 14, 64, 3, 3, 2, 1
+        groups = C
+        A, B, Out = depthwise_conv2d(N, C, H, W, K, R, S, stride, padding)
+    rng = np.random.default_rng(9)
+    a = rng.uniform(-1, 1, [int(s) for s in A.shape]).astype(np.float16)
+    b = rng.uniform(-1, 1, [int(s) for s in B.shape]).astype(np.float16)
+    got, result = _run_script_flow([A, B, Out], {"A": a, "B": b}, tmp_path, kind, transform_strict=False)
+    low = result.sch_app.lowered
+    assert low.kind == "conv2d" and low.desc.groups == groups
+    ref = grouped_conv_reference(a, b, stride, padding, groups)
     mx, mean = co.rel_errors(got, ref)
     assert got.shape == ref.shape and mx <= 1e-2 and mean <= 1e-3

@@ -124,3 +124,42 @@ def test_epilogue_errors(gpu):
     rc = lib.amos_run_fused(_lib.AMOS_OP_GEMM, ctypes.byref(d), None, ctypes.byref(e), a.data_ptr(), a.data_ptr(),
                             out.data_ptr(), None, 0, None)
     assert rc == _lib.AMOS_ERR_BAD_ARG and b"below N" in lib.amos_last_error()
+
+
+GROUPED_CASES = [
+    # N, C, D, H, W, K, T, R, S, stride, pad, dil, groups
+    (2, 64, 1, 12, 12, 96, 1, 3, 3, (1, 1, 1), (0, 1, 1), (1, 1, 1), 4),
+    (3, 24, 1, 9, 7, 24, 1, 3, 3, (1, 2, 1), (0, 1, 1), (1, 1, 1), 24),     # depthwise
+    (2, 16, 1, 8, 8, 48, 1, 3, 3, (1, 1, 1), (0, 1, 1), (1, 1, 1), 16),     # depthwise, 3 outputs per channel
+    (1, 32, 3, 6, 6, 16, 2, 3, 3, (1, 1, 1), (1, 1, 1), (1, 1, 1), 2),      # grouped conv3d
+]
+
+
+@pytest.mark.parametrize("dtype", ["float16", "bfloat16", "int8"])
+@pytest.mark.parametrize("case", GROUPED_CASES)
+def test_grouped_conv(gpu, dtype, case):
+    """grouped and depthwise convolution (reference computes:
+    benchmark/amos/mapping_groupedconv2d_tensorcore.py:7-60, mapping_depthwiseconv2d_tensorcore.py:7-48)
+    against the oracle run once per group, with and without split-K and a fused addition"""
+    from amos_amd import _lib, ops
+    N, C, D, H, W, K, T, R, S, st, pd, dl, G = case
+    rng = np.random.default_rng(hash(case) % 2**32)
+    x = make_operand(rng, (N, C, D, H, W), dtype, "normal")
+    w = make_operand(rng, (K, C // G, T, R, S), dtype, "normal")
+    cg, kg = C // G, K // G
+    ref = np.concatenate([co.lib_conv3d(np.ascontiguousarray(x[:, g * cg:(g + 1) * cg]),
+                                        np.ascontiguousarray(w[g * kg:(g + 1) * kg]), dtype, st, pd, dl,
+                                        acc="float64") for g in range(G)], axis=1)
+    dx, dw = to_device(x, dtype), to_device(w, dtype)
+    for cfg in (None, dict(tile_i=64, tile_j=64, split_k=2)):
+        if D == 1 and T == 1:
+            got = ops.conv2d(dx[:, :, 0], dw[:, :, 0], st[1:], pd[1:], dl[1:], config=cfg, groups=G)[:, :, None]
+        else:
+            got = ops.conv3d(dx, dw, st, pd, dl, config=cfg, groups=G)
+        check(got.cpu().numpy(), ref, dtype, "grouped conv %s %s cfg %s" % (dtype, case, cfg))
+    d_host, d_dev = make_d(rng, ref.shape, dtype, d_types(dtype)[0])
+    got = ops.conv3d(dx, dw, st, pd, dl, groups=G, add=d_dev).cpu().numpy()
+    want = (ref.astype(np.int64) + d_host).astype(np.int32) if dtype == "int8" else ref + d_host
+    check(got, want, dtype, "grouped conv + D %s %s" % (dtype, case))
+    with pytest.raises(_lib.AmosError, match="not applicable"):
+        ops.conv3d(dx, dw, st, pd, dl, groups=G, config=dict(tile_i=64, tile_j=64, split_k=1, pipeline=4))

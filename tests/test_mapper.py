@@ -487,3 +487,77 @@ def test_conv1d_lowers_to_conv2d_with_unit_height():
     ref = co.lib_conv2d(a[:, :, None, :].astype(np.float16), b[:, :, None, :].astype(np.float16), "float16",
                         (1, 2), (0, 1), (1, 2), acc="float64")
     assert np.array_equal(ref[:, :, 0, :], want)
+
+
+def grouped_conv2d(N, C, H, W, K, R, S, stride, padding, groups, in_dtype="float16", out_dtype="float32"):
+    """reference: benchmark/amos/mapping_groupedconv2d_tensorcore.py:7-60"""
+    pH, pW = H + 2 * padding, W + 2 * padding
+    A = te.placeholder([N, C, H, W], dtype=in_dtype, name="A")
+    B = te.placeholder([K, C // groups, R, S], dtype=in_dtype, name="B")
+    Pad = te.compute([N, C, pH, pW], lambda n, c, h, w: tir.if_then_else(
+        tir.all(h >= padding, h - padding < H, w >= padding, w - padding < W),
+        A[n, c, h - padding, w - padding], tir.const(0.0, A.dtype)), name="Pad")
+    A_reshaped = te.compute([N, groups, C // groups, pH, pW],
+                            lambda n, c_o, c_i, r, s: Pad[n, c_o * (C // groups) + c_i, r, s])
+    B_reshaped = te.compute([groups, K // groups, C // groups, R, S],
+                            lambda k_o, k_i, c, r, s: B[k_o * (K // groups) + k_i, c, r, s])
+    rc = te.reduce_axis([0, C // groups], name="rc")
+    rr = te.reduce_axis([0, R], name="rr")
+    rs = te.reduce_axis([0, S], name="rs")
+    P, Q = (pH - R) // stride + 1, (pW - S) // stride + 1
+    Conv = te.compute([N, groups, K // groups, P, Q], lambda n, k_o, k_i, p, q: te.sum(
+        (A_reshaped[n, k_o, rc, p * stride + rr, q * stride + rs] * B_reshaped[k_o, k_i, rc, rr, rs]).astype(out_dtype),
+        axis=[rc, rr, rs]), name="Conv")
+    Reshaped = te.compute([N, K, P, Q], lambda n, k, p, q: Conv[n, k // (K // groups), k % (K // groups), p, q],
+                          name="Reshaped")
+    return A, B, Reshaped
+
+
+def depthwise_conv2d(N, C, H, W, K, R, S, stride, padding, in_dtype="float16", out_dtype="float32"):
+    """reference: benchmark/amos/mapping_depthwiseconv2d_tensorcore.py:7-48"""
+    pH, pW = H + 2 * padding, W + 2 * padding
+    A = te.placeholder([N, C, H, W], dtype=in_dtype, name="A")
+    B = te.placeholder([K, R, S], dtype=in_dtype, name="B")
+    Pad = te.compute([N, C, pH, pW], lambda n, c, h, w: tir.if_then_else(
+        tir.all(h >= padding, h - padding < H, w >= padding, w - padding < W),
+        A[n, c, h - padding, w - padding], tir.const(0.0, A.dtype)), name="Pad")
+    B_reshaped = te.compute([C, K // C, R, S], lambda k_o, k_i, r, s: B[k_o * (K // C) + k_i, r, s])
+    rr = te.reduce_axis([0, R], name="rr")
+    rs = te.reduce_axis([0, S], name="rs")
+    P, Q = (pH - R) // stride + 1, (pW - S) // stride + 1
+    Conv = te.compute([N, C, K // C, P, Q], lambda n, k_o, k_i, p, q: te.sum(
+        (Pad[n, k_o, p * stride + rr, q * stride + rs] * B_reshaped[k_o, k_i, rr, rs]).astype(out_dtype),
+        axis=[rr, rs]), name="Conv")
+    Reshaped = te.compute([N, K, P, Q], lambda n, k, p, q: Conv[n, k // (K // C), k % (K // C), p, q],
+                          name="Reshaped")
+    return A, B, Reshaped
+
+
+def grouped_conv_reference(a, b, stride, padding, groups):
+    cg, kg = a.shape[1] // groups, b.shape[0] // groups
+    b4 = b.reshape(b.shape[0], cg, b.shape[-2], b.shape[-1])
+    return np.concatenate([co.lib_conv2d(np.ascontiguousarray(a[:, g * cg:(g + 1) * cg]).astype(np.float16),
+                                         np.ascontiguousarray(b4[g * kg:(g + 1) * kg]).astype(np.float16),
+                                         "float16", stride, padding, 1, acc="float64") for g in range(groups)], axis=1)
+
+
+@pytest.mark.parametrize("build,groups", [(lambda: grouped_conv2d(2, 8, 6, 7, 12, 3, 3, 2, 1, 4), 4),
+                                          (lambda: depthwise_conv2d(2, 6, 7, 6, 12, 3, 2, 1, 1), 6)])
+def test_grouped_and_depthwise_conv_lowering(build, groups):
+    from amos_amd.auto_tensorize.lowering import lower_main_op
+    A, B, Out = build()
+    dag = at.compute_dag_from_tensors([Out])
+    main = [op for op in dag.op_lst if op.reduce_axis][0]
+    assert at.get_match_results(dag, "hip")          # the 5-d main op matches the MFMA intrinsic
+    low = lower_main_op(main, dag)
+    assert low.kind == "conv2d" and low.desc.groups == groups and low.output is Out
+    assert [t.name for t in low.inputs] == ["A", "B"]
+    rng = np.random.default_rng(8)
+    a = rng.integers(-3, 4, [int(s) for s in A.shape]).astype(np.float64)
+    b = rng.integers(-3, 4, [int(s) for s in B.shape]).astype(np.float64)
+    want = te_interp.evaluate(Out, {"A": a, "B": b})
+    c = low.desc
+    assert (c.N, c.C, c.H, c.W, c.K, c.R, c.S) == (a.shape[0], a.shape[1], a.shape[2], a.shape[3], b.shape[0],
+                                                   b.shape[-2], b.shape[-1])
+    got = grouped_conv_reference(a, b, (c.stride_h, c.stride_w), (c.pad_h, c.pad_w), groups)
+    assert np.array_equal(got, want)
