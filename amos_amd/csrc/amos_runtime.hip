@@ -72,6 +72,7 @@ struct Plan {
   size_t conv_lds;
   int conv_occ;
   int conv_waves;
+  int conv_w9;
 };
 
 static int dtype_pair(int in_dtype, int out_dtype, int* dt) {
@@ -274,13 +275,15 @@ static int plan_conv(Plan& pl, int op, const amos_conv_desc_t* d, const amos_ker
   const int RS = (int)(c.R * c.S);
   const int Wp = (OQ - 1) * c.stride_w + ((int)c.S - 1) * c.dil_w + 1;
   ConvPatchPlan pp = conv_patch_plan(c, op, BI, BJ, pl.cfg.split_k,
-                                     pipe == AMOS_PIPE_PATCH ? 4 : pipe == AMOS_PIPE_PATCH8 ? 8 : 0);
+                                     pipe == AMOS_PIPE_PATCH ? 4 : pipe == AMOS_PIPE_PATCH8 ? 8 : 0,
+                                     !(pl.cfg.reserved[0] & AMOS_FLAG_NO_UNROLLED_TAPS));
   const char* why = pp.why;
   if (!why && (!workspace || ws_bytes < (size_t)need_ws || ((uintptr_t)workspace & 255)))
     why = "workspace smaller than amos_workspace_bytes() or not 256-byte aligned";
   const int max_pos = pp.max_pos, nsw = pp.nsw, pls = pp.pls;
   pl.conv_occ = pp.occ;
   pl.conv_waves = pp.waves;
+  pl.conv_w9 = pp.w9;
   const size_t lds = pp.lds;
   if (why) {
     if (pipe == AMOS_PIPE_PATCH || pipe == AMOS_PIPE_PATCH8)
@@ -386,14 +389,14 @@ static int launch_tn(const Plan& pl, hipStream_t stream) {
   return 0;
 }
 
-static ConvInstance* pick_conv(int dt, int ti, int tj, int waves, int pls, int occ) {
-  if (dt == DT_F16) return pick_conv_f16(ti, tj, waves, pls, occ);
-  if (dt == DT_BF16) return pick_conv_bf16(ti, tj, waves, pls, occ);
-  return pick_conv_i8(ti, tj, waves, pls, occ);
+static ConvInstance* pick_conv(int dt, int ti, int tj, int waves, int pls, int occ, int w9) {
+  if (dt == DT_F16) return pick_conv_f16(ti, tj, waves, pls, occ, w9);
+  if (dt == DT_BF16) return pick_conv_bf16(ti, tj, waves, pls, occ, w9);
+  return pick_conv_i8(ti, tj, waves, pls, occ, w9);
 }
 
 static int launch_conv(const Plan& pl, hipStream_t stream) {
-  ConvInstance* inst = pick_conv(pl.dt, pl.cfg.tile_i, pl.cfg.tile_j, pl.conv_waves, pl.cv.pls, pl.conv_occ);
+  ConvInstance* inst = pick_conv(pl.dt, pl.cfg.tile_i, pl.cfg.tile_j, pl.conv_waves, pl.cv.pls, pl.conv_occ, pl.conv_w9);
   if (!inst) return set_error(AMOS_ERR_INFEASIBLE, "no patch-staged convolution instance");
   hipError_t attr_err = hipSuccess;
   std::call_once(inst->once, [&] {
@@ -563,7 +566,7 @@ const char* amos_kernel_name(int op, const void* desc, const amos_kernel_config_
   static char dummy_ws[256] __attribute__((aligned(256)));
   if (make_plan(pl, op, desc, cfg, dummy, dummy, dummy, dummy_ws, (size_t)-1)) return nullptr;
   if (pl.conv_ups) {
-    ConvInstance* ci = pick_conv(pl.dt, pl.cfg.tile_i, pl.cfg.tile_j, pl.conv_waves, pl.cv.pls, pl.conv_occ);
+    ConvInstance* ci = pick_conv(pl.dt, pl.cfg.tile_i, pl.cfg.tile_j, pl.conv_waves, pl.cv.pls, pl.conv_occ, pl.conv_w9);
     return ci ? ci->name : nullptr;
   }
   if (pl.tn_waves) {

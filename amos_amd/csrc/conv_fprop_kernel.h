@@ -263,7 +263,17 @@ __device__ __forceinline__ void wait_vmcnt_le(int n) {
 // BI64 x BJ64 = block tile in units of 64; NW = 4 or 8 waves.  A SIMD issues one instruction of a
 // wave every ~4 cycles, and a step of a small wave tile is ~100 instructions around a handful of
 // MFMAs: with 8 waves a SIMD holds two instruction streams and interleaves them.
-template <int DT, int BI64, int BJ64, int NW, int PL, int OCC>
+//
+// W9 = 1: the window has nine taps per macro step (3x3, also 3x3x3 per depth tap) and the ring
+// three stages.  The tap loop is unrolled, so ring stages, patch buffers, patch read addresses
+// per tap, copy slots and wait counts are compile-time or precomputed registers, and a step is
+// about half the instructions of the table-driven one.  The patch buffers are a fixed distance
+// apart (it must fit the 16-bit offset field of ds_read): 56 KB next to 64-row weight tiles, 48 KB
+// next to 128-row ones.
+constexpr unsigned conv_w9_xbuf(int bi) { return bi <= 64 ? 56 * 1024 : 48 * 1024; }
+template <int N> struct IntC { static constexpr int value = N; };
+
+template <int DT, int BI64, int BJ64, int NW, int PL, int OCC, int W9 = 0>
 __global__ __launch_bounds__(64 * NW, OCC) void amos_conv_fprop(const ConvFpropParams p) {
   typedef Mfma<DT> MM;
   typedef typename MM::acc_t acc_t;
@@ -479,7 +489,7 @@ __global__ __launch_bounds__(64 * NW, OCC) void amos_conv_fprop(const ConvFpropP
     {
       const int tt = fast_div(m_begin, p.fd_cc), cc = m_begin - tt * p.c_chunks;
       const unsigned po = 256u + (unsigned)(tt * p.dd * HW) * pos_bytes + (unsigned)cc * 128u;
-      const unsigned buf = (unsigned)p.sx_off + (unsigned)(m_begin & (p.xbufs - 1)) * xbuf_bytes;
+      const unsigned buf = (unsigned)p.sx_off + (W9 ? 0u : (unsigned)(m_begin & (p.xbufs - 1)) * xbuf_bytes);
       for (int v = 0; v < n_pl; v += 4) {   // four table entries per LDS round trip
         int2 e[4];
 #pragma unroll
@@ -498,8 +508,6 @@ __global__ __launch_bounds__(64 * NW, OCC) void amos_conv_fprop(const ConvFpropP
       asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
       asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
       read_step(0, buf, 0);
-#pragma unroll
-      for (int x = 0; x < PL; ++x) pt[x] = read_tab(x);
     }
   }
 
@@ -513,6 +521,14 @@ __global__ __launch_bounds__(64 * NW, OCC) void amos_conv_fprop(const ConvFpropP
     // are its copies of everything older than the youngest NSW-2 steps' worth: the next weight
     // tile and, at a macro step's last tap, the next patch.  After the barrier that holds for
     // every wave.
+    // The table entries of this step's patch copies: read here, waited for and tied to the barrier
+    // statement below.  (An explicit ds_read's result must not be live across a loop edge: the
+    // compiler does not know it arrives late and may copy the register before it has.)
+    if (PL > 0) {
+      const int v0 = e[4] & 0xffff;
+#pragma unroll
+      for (int x = 0; x < PL; ++x) pt[x] = read_tab(v0 + x);
+    }
     if (NSW >= 4) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * (PL + WCH)) : "memory");
     else if (NSW == 3) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(PL + WCH) : "memory");
     else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
@@ -546,22 +562,110 @@ __global__ __launch_bounds__(64 * NW, OCC) void amos_conv_fprop(const ConvFpropP
     }
     issue_weights((unsigned)e[0], istage);   // tile step+NSW into the stage just freed
     istage = rstage;
-    if (PL > 0) {
-      const int v0n = (int)((unsigned)e[4] >> 16);
-#pragma unroll
-      for (int x = 0; x < PL; ++x) pt[x] = read_tab(v0n + x);
-    }
     // the next step's table entry, last: it has until the top of the next step to arrive
     __builtin_amdgcn_sched_barrier(0);
     ++g;
     e_next = tbl[g];
   };
-  int step = 0;
-  for (; step + 1 < n_steps; step += 2) {
-    one_step(0, cur, nxt);
-    one_step(1, nxt, cur);
+  if constexpr (!W9) {
+    int step = 0;
+    for (; step + 1 < n_steps; step += 2) {
+      one_step(0, cur, nxt);
+      one_step(1, nxt, cur);
+    }
+    if (step < n_steps) one_step(0, cur, nxt);
+  } else {
+    // ---- nine unrolled taps per macro step ------------------------------------------------------
+    // patch read addresses per tap (buffer 0): position shift and swizzle term folded in
+    unsigned baddr[9][TJ][4];
+    {
+      int tr = 0, ts = 0;
+#pragma unroll
+      for (int tap = 0; tap < 9; ++tap) {
+        const unsigned shift = (unsigned)p.sx_off + (unsigned)(tr * p.dh * p.Wp + ts * p.dw) * 128u;
+#pragma unroll
+        for (int b = 0; b < TJ; ++b) {
+          const unsigned xb = col_byte[b] + shift;
+          const unsigned key = ((xb >> 3) ^ (xb >> 6)) & 0x70;
+#pragma unroll
+          for (int ks = 0; ks < 4; ++ks) baddr[tap][b][ks] = xb + (kh[ks] ^ key);
+        }
+        if (++ts == p.S) { ts = 0; ++tr; }
+      }
+    }
+    const int n_macro = m_end - m_begin;
+    auto wk_of_macro = [&](int m) {
+      if (m > p.macro_steps - 1) m = p.macro_steps - 1;
+      const int tt = fast_div(m, p.fd_cc), cc = m - tt * p.c_chunks;
+      return (unsigned)(tt * 9) * pos_bytes + (unsigned)cc * 128u;
+    };
+    // one K step: TAP of the macro step in patch buffer BUF
+    auto step9 = [&](auto tap_c, auto buf_c, unsigned wk_cur, unsigned wk_nxt, int n_live, unsigned po, int pdb) {
+      constexpr int TAP = decltype(tap_c)::value, BUF = decltype(buf_c)::value;
+      constexpr int SLOT = (TAP + BUF) & 1;            // nine steps per macro step: the parity flips with BUF
+      if constexpr (PL > 0 && TAP <= 6) {
+#pragma unroll
+        for (int x = 0; x < PL; ++x) pt[x] = read_tab(TAP * PL + x);
+      }
+      // the copies of the previous step may still be in flight: WCH of the weight tile, PL of the
+      // patch if that step was one of the taps 0..6 that fetch it
+      asm volatile("s_waitcnt vmcnt(%0)" ::"n"(WCH + ((TAP >= 1 && TAP <= 7) ? PL : 0)) : "memory");
+      if (PL == 2)
+        asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" : "+v"(pt[0]), "+v"(pt[PL > 1 ? 1 : 0])::"memory");
+      else if (PL == 1)
+        asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" : "+v"(pt[0])::"memory");
+      else
+        asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+      // operands of the next K step
+      // (PL = 0: a block runs one macro step and has one patch buffer; its last read is unused)
+      constexpr int TN = TAP == 8 ? 0 : TAP + 1, BN = (TAP == 8 && PL > 0) ? BUF ^ 1 : BUF;
+#pragma unroll
+      for (int ks = 0; ks < 4; ++ks) {
+#pragma unroll
+        for (int a = 0; a < TI; ++a)
+          af[SLOT ^ 1][ks][a] = *(const v4i*)AMOS_LDS_PTR_FROM(a_off[a & 1][ks] + (unsigned)((TN % 3) * WSTAGE + (a >> 1) * (64 * 128)));
+#pragma unroll
+        for (int b = 0; b < TJ; ++b)
+          bf[SLOT ^ 1][ks][b] = *(const v4i*)AMOS_LDS_PTR_FROM(baddr[TN][b][ks] + (unsigned)BN * conv_w9_xbuf(BI));
+      }
+      mma_step(SLOT);
+      // patch of the next macro step, on taps 0..6, before this step's weight tile
+      if constexpr (PL > 0 && TAP <= 6) {
+#pragma unroll
+        for (int x = 0; x < PL; ++x) {
+          const int v = TAP * PL + x;
+          const bool live = v < n_live;
+          const unsigned dst = (unsigned)p.sx_off + (unsigned)(BUF ^ 1) * conv_w9_xbuf(BI) + (unsigned)(wave + NW * v) * 1024;
+          patch_copy(pt[x], lane_cq[v & 1], po, pdb, live ? dst : (unsigned)p.dump_off, live ? (unsigned)p.D : 0u);
+        }
+      }
+      // weight tile of the step three ahead, into the stage the previous step read
+      constexpr int NT = TAP + 3;
+      issue_weights(NT < 9 ? wk_cur + (unsigned)NT * pos_bytes : wk_nxt + (unsigned)(NT - 9) * pos_bytes,
+                    (unsigned)((TAP % 3) * WSTAGE));
+    };
+    auto macro9 = [&](auto buf_c, int mi) {
+      const int m = m_begin + mi;
+      const unsigned wk_cur = wk_of_macro(m), wk_nxt = wk_of_macro(m + 1);
+      const int n_live = m + 1 < m_end ? n_pl : 0;
+      const int tt1 = fast_div(m + 1, p.fd_cc), cc1 = (m + 1) - tt1 * p.c_chunks;
+      const unsigned po = 256u + (unsigned)(tt1 * p.dd * HW) * pos_bytes + (unsigned)cc1 * 128u;
+      const int pdb = tt1 * p.dd - 32768;
+      step9(IntC<0>{}, buf_c, wk_cur, wk_nxt, n_live, po, pdb);
+      step9(IntC<1>{}, buf_c, wk_cur, wk_nxt, n_live, po, pdb);
+      step9(IntC<2>{}, buf_c, wk_cur, wk_nxt, n_live, po, pdb);
+      step9(IntC<3>{}, buf_c, wk_cur, wk_nxt, n_live, po, pdb);
+      step9(IntC<4>{}, buf_c, wk_cur, wk_nxt, n_live, po, pdb);
+      step9(IntC<5>{}, buf_c, wk_cur, wk_nxt, n_live, po, pdb);
+      step9(IntC<6>{}, buf_c, wk_cur, wk_nxt, n_live, po, pdb);
+      step9(IntC<7>{}, buf_c, wk_cur, wk_nxt, n_live, po, pdb);
+      step9(IntC<8>{}, buf_c, wk_cur, wk_nxt, n_live, po, pdb);
+    };
+    for (int mi = 0; mi < n_macro; mi += 2) {
+      macro9(IntC<0>{}, mi);
+      if (mi + 1 < n_macro) macro9(IntC<1>{}, mi + 1);
+    }
   }
-  if (step < n_steps) one_step(0, cur, nxt);
 
   // ---- epilogue: Y[(n*K + i)*ODPQ + (od*OPQ + opq)] ---------------------------------------------
   out_t* const out = (out_t*)p.y;

@@ -76,20 +76,20 @@ struct ConvInstance {
   std::once_flag once;
   int static_lds = 0;   // must stay 0: the kernel addresses dynamic LDS from byte 0
 };
-ConvInstance* pick_conv_f16(int ti, int tj, int waves, int pls, int occ);
-ConvInstance* pick_conv_bf16(int ti, int tj, int waves, int pls, int occ);
-ConvInstance* pick_conv_i8(int ti, int tj, int waves, int pls, int occ);
+ConvInstance* pick_conv_f16(int ti, int tj, int waves, int pls, int occ, int w9);
+ConvInstance* pick_conv_bf16(int ti, int tj, int waves, int pls, int occ, int w9);
+ConvInstance* pick_conv_i8(int ti, int tj, int waves, int pls, int occ, int w9);
 void launch_conv_prepare(int es, const ConvFpropParams& p, hipStream_t stream);
 
 #ifdef AMOS_CONV_FPROP_KERNEL_INCLUDED
-template <int DT, int TI, int TJ, int NW, int PL, int OCC>
+template <int DT, int TI, int TJ, int NW, int PL, int OCC, int W9 = 0>
 ConvInstance* conv_instance() {
   static ConvInstance inst;
   static const char* dtn[] = {"f16", "bf16", "i8"};
   static std::string name = std::string("amos_conv_fprop<") + dtn[DT] + "," + std::to_string(64 * TI) +
                             "x" + std::to_string(64 * TJ) + "," + std::to_string(NW) + "w,pl" +
-                            std::to_string(PL) + (OCC == 2 ? ",occ2>" : ">");
-  inst.fn = amos_conv_fprop<DT, TI, TJ, NW, PL, OCC>;
+                            std::to_string(PL) + (OCC == 2 ? ",occ2" : "") + (W9 ? ",9taps>" : ">");
+  inst.fn = amos_conv_fprop<DT, TI, TJ, NW, PL, OCC, W9>;
   inst.name = name.c_str();
   inst.threads = 64 * NW;
   return &inst;
@@ -122,10 +122,24 @@ ConvInstance* pick_conv_tile8(int ti, int tj) {
   if (ti == 128 && tj == 256) return conv_instance<DT, 2, 4, 8, PL, 1>();
   return nullptr;
 }
+template <int DT, int PL>
+ConvInstance* pick_conv_tile9(int ti, int tj) {
+  if (ti == 128 && tj == 64) return conv_instance<DT, 2, 1, 8, PL, 1, 1>();
+  if (ti == 64 && tj == 128) return conv_instance<DT, 1, 2, 8, PL, 1, 1>();
+  if (ti == 128 && tj == 128) return conv_instance<DT, 2, 2, 8, PL, 1, 1>();
+  return nullptr;
+}
 // waves = 4 or 8; pls = patch copies per wave per K step the plan asks for: 0, 2 or 4 with 4
-// waves, 0, 1 or 2 with 8
+// waves, 0, 1 or 2 with 8; w9 = the instance with nine unrolled taps
 template <int DT>
-ConvInstance* pick_conv_tile(int ti, int tj, int waves, int pls, int occ) {
+ConvInstance* pick_conv_tile(int ti, int tj, int waves, int pls, int occ, int w9) {
+  if (w9) {
+    if (waves != 8 || occ != 1) return nullptr;
+    if (pls == 0) return pick_conv_tile9<DT, 0>(ti, tj);
+    if (pls == 1) return pick_conv_tile9<DT, 1>(ti, tj);
+    if (pls == 2) return pick_conv_tile9<DT, 2>(ti, tj);
+    return nullptr;
+  }
   if (waves == 8) {
     if (occ != 1) return nullptr;
     if (pls == 0) return pick_conv_tile8<DT, 0>(ti, tj);

@@ -123,20 +123,23 @@ int64_t conv_workspace_bytes(const amos_conv_desc_t& c, int op) {
 
 
 static ConvPatchPlan conv_patch_plan_waves(const amos_conv_desc_t& cin, int op, int BI, int BJ, int split_k,
-                                           int waves);
+                                           int waves, bool allow_w9);
 
 // waves: 4, 8, or 0 = 8 where that applies and four waves would leave a CU with a single workgroup
-ConvPatchPlan conv_patch_plan(const amos_conv_desc_t& c, int op, int BI, int BJ, int split_k, int waves) {
-  if (waves == 4 || waves == 8) return conv_patch_plan_waves(c, op, BI, BJ, split_k, waves);
-  ConvPatchPlan p4 = conv_patch_plan_waves(c, op, BI, BJ, split_k, 4);
+// (or where the unrolled 3x3 instance applies, which exists with 8 waves)
+ConvPatchPlan conv_patch_plan(const amos_conv_desc_t& c, int op, int BI, int BJ, int split_k, int waves,
+                              bool allow_w9) {
+  if (waves == 4 || waves == 8) return conv_patch_plan_waves(c, op, BI, BJ, split_k, waves, allow_w9);
+  ConvPatchPlan p8 = conv_patch_plan_waves(c, op, BI, BJ, split_k, 8, allow_w9);
+  if (!p8.why && p8.w9) return p8;
+  ConvPatchPlan p4 = conv_patch_plan_waves(c, op, BI, BJ, split_k, 4, allow_w9);
   if (!p4.why && p4.occ == 2) return p4;
-  ConvPatchPlan p8 = conv_patch_plan_waves(c, op, BI, BJ, split_k, 8);
   return p8.why ? p4 : p8;
 }
 
 static ConvPatchPlan conv_patch_plan_waves(const amos_conv_desc_t& cin, int op, int BI, int BJ, int split_k,
-                                           int waves) {
-  ConvPatchPlan pp = {nullptr, 0, 0, 0, 0, 0, 0, 0, 0};
+                                           int waves, bool allow_w9) {
+  ConvPatchPlan pp = {nullptr, 0, 0, 0, 0, 0, 0, 0, 0, 0};
   pp.waves = waves;
   amos_conv_desc_t c = cin;
   if (op == AMOS_OP_CONV2D) { c.D = 1; c.T = 1; c.stride_d = 1; c.pad_d = 0; c.dil_d = 1; }
@@ -208,6 +211,23 @@ static ConvPatchPlan conv_patch_plan_waves(const amos_conv_desc_t& cin, int op, 
     return RS == 1 ? "1x1 window with several channel chunks per block"
                    : "input patch too large to prefetch behind the window's taps";
   };
+  // the instance with the nine taps unrolled: 8 waves, three ring stages, patch buffers a fixed
+  // 48 KB (56 KB next to 64-row weight tiles) apart, the next patch fetched on taps 0..6 with at
+  // most two copies per wave and step
+  if (allow_w9 && waves == 8 && RS == 9 && BI <= 128 && BJ <= 128 && !(BI == 64 && BJ == 64)) {
+    const int max_pos9 = one_macro ? max_pos : (BI <= 64 ? 448 : 384);
+    const size_t patch9 = (size_t)pp.xbufs * max_pos9 * 128 + (size_t)max_pos9 * 8 + 1024;
+    const int pls9 = one_macro ? 0 : (per_wave + 6) / 7;
+    if (real_pos <= max_pos9 && 3 * wstage + patch9 <= budget && pls9 <= 2) {
+      pp.w9 = 1;
+      pp.nsw = 3;
+      pp.pls = pls9;
+      pp.max_pos = max_pos9;
+      pp.occ = 1;
+      pp.lds = 3 * wstage + patch9;
+      return pp;
+    }
+  }
   pp.why = fit(budget, &pp.nsw, &pp.pls);
   if (pp.why) return pp;
   pp.lds = (size_t)pp.nsw * wstage + patch;

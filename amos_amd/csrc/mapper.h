@@ -42,11 +42,13 @@ struct ConvPatchPlan {
   int xbufs;         // patch buffers (1 when a block runs a single macro step)
   int occ;           // workgroups per CU the instance is built for (2 when LDS and registers allow)
   int waves;         // waves per workgroup: 4 or 8
+  int w9;            // the instance with the nine taps of a 3x3 window unrolled
   size_t lds;        // dynamic LDS bytes of the block
 };
 int64_t conv_packed_bytes(const amos_conv_desc_t& c, int op);
 int64_t conv_relaid_bytes(const amos_conv_desc_t& c, int op);
 int64_t conv_workspace_bytes(const amos_conv_desc_t& c, int op);
-ConvPatchPlan conv_patch_plan(const amos_conv_desc_t& c, int op, int BI, int BJ, int split_k, int waves);
+ConvPatchPlan conv_patch_plan(const amos_conv_desc_t& c, int op, int BI, int BJ, int split_k, int waves,
+                              bool allow_w9 = true);
 
 }  // namespace amos

@@ -41,6 +41,7 @@ def make_config(config):
     c.tile_j = int(config.get("tile_j", 0))
     c.split_k = int(config.get("split_k", 0))
     c.pipeline = int(config.get("pipeline", 0))
+    c.reserved[0] = int(config.get("flags", 0))
     return c
 
 

@@ -130,8 +130,12 @@ typedef struct {
   int32_t tile_i, tile_j;   /* block tile of the MFMA row / column operand: 64, 128 or 256 */
   int32_t split_k;          /* >= 1: blocks along the fused reduction                       */
   int32_t pipeline;         /* AMOS_PIPE_*; 0 = mapper's choice                             */
-  int32_t reserved[4];
+  int32_t reserved[4];      /* [0]: AMOS_FLAG_* bits; the rest 0                            */
 } amos_kernel_config_t;
+
+/* conv: do not use the instances whose 3x3 window taps are unrolled (they are preferred where
+ * they apply; the flag lets a sweep time the table-driven ones) */
+#define AMOS_FLAG_NO_UNROLLED_TAPS 1
 
 /* how tiles travel from HBM to the MFMA operands */
 #define AMOS_PIPE_AUTO 0

@@ -248,10 +248,11 @@ def test_conv_patch_pipeline(gpu, dtype, case):
     ref = co.lib_conv3d(x, w, dtype, st, pd, dl, acc="float64")
     dx, dw = to_device(x, dtype), to_device(w, dtype)
     tiles = [(64, 64), (128, 64), (64, 128), (128, 128), (256, 64), (256, 128), (128, 256), (64, 256)]
-    for tile, split, pipe in [(t, s, p) for t in tiles for s in (1, 2)
-                              for p in (_lib.AMOS_PIPE_PATCH, _lib.AMOS_PIPE_PATCH8)]:
+    # (pipeline, flags): 4 waves; 8 waves with the 3x3 taps unrolled where that applies; 8 waves table-driven
+    variants = [(_lib.AMOS_PIPE_PATCH, 0), (_lib.AMOS_PIPE_PATCH8, 0), (_lib.AMOS_PIPE_PATCH8, 1)]
+    for tile, split, (pipe, flags) in [(t, s, v) for t in tiles for s in (1, 2) for v in variants]:
         if True:
-            cfg = dict(tile_i=tile[0], tile_j=tile[1], split_k=split, pipeline=pipe)
+            cfg = dict(tile_i=tile[0], tile_j=tile[1], split_k=split, pipeline=pipe, flags=flags)
             try:
                 if D == 1 and T == 1:
                     got = ops.conv2d(dx[:, :, 0], dw[:, :, 0], st[1:], pd[1:], dl[1:], config=cfg)[:, :, None]
@@ -262,7 +263,7 @@ def test_conv_patch_pipeline(gpu, dtype, case):
                 assert e.code == _lib.AMOS_ERR_INFEASIBLE and "not applicable" in str(e)
                 continue
             check(got.cpu().numpy(), ref, dtype,
-                  "patch conv %s %s tile %s split %d pipeline %d" % (dtype, case, tile, split, pipe))
+                  "patch conv %s %s tile %s split %d pipeline %d flags %d" % (dtype, case, tile, split, pipe, flags))
 
 
 def test_conv_patch_is_the_default_when_applicable(gpu):
