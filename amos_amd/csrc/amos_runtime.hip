@@ -42,6 +42,11 @@ __global__ void fill_zero_kernel(T* p, int64_t rows, int64_t cols, int64_t ld) {
 
 // ---- kernel instance table (defined in inst_*.hip) -------------------------------------
 static Instance* pick(int dt, int rl, int cl, int ti, int tj) {
+  if (rl == LD_TVEC) {
+    if (dt == DT_F16) return pick_f16_tvec(cl, ti, tj);
+    if (dt == DT_BF16) return pick_bf16_tvec(cl, ti, tj);
+    return nullptr;
+  }
   switch (dt * 2 + (rl == LD_STRIDED)) {
     case DT_F16 * 2: return pick_f16_vec(cl, ti, tj);
     case DT_F16 * 2 + 1: return pick_f16_strided(cl, ti, tj);
@@ -150,8 +155,19 @@ static int plan_gemm(Plan& pl, int op, const void* desc_any, const amos_gemm_des
     return s_k == 1 && aligned16(base) && (s_row % ce) == 0 && (d->K % ce) == 0 &&
            (batch == 1 || (bstride % ce) == 0);
   };
-  pl.rl = vec_ok(A, p.row_s_row, p.row_s_k, sa) ? LD_VEC : LD_STRIDED;
-  pl.cl = vec_ok(B, p.col_s_row, p.col_s_k, sb) ? LD_VEC : LD_STRIDED;
+  // rows contiguous instead of K (a transposed A, a row-major B), 16-bit elements: vector loads
+  // along the rows, transposed in registers
+  auto tvec_ok = [&](const void* base, int64_t s_row, int64_t s_k, int64_t bstride, int64_t rows) {
+    return es == 2 && s_row == 1 && (s_k % 8) == 0 && aligned16(base) && (rows % 8) == 0 &&
+           (batch == 1 || (bstride % 8) == 0);
+  };
+  pl.rl = vec_ok(A, p.row_s_row, p.row_s_k, sa) ? LD_VEC
+          : tvec_ok(A, p.row_s_row, p.row_s_k, sa, d->M) ? LD_TVEC : LD_STRIDED;
+  pl.cl = vec_ok(B, p.col_s_row, p.col_s_k, sb) ? LD_VEC
+          : tvec_ok(B, p.col_s_row, p.col_s_k, sb, d->N) ? LD_TVEC : LD_STRIDED;
+  // a tvec loader runs next to vec or tvec only: with a strided partner both take element loads
+  if ((pl.rl == LD_TVEC && pl.cl == LD_STRIDED) || (pl.cl == LD_TVEC && pl.rl == LD_STRIDED))
+    pl.rl = pl.rl == LD_VEC ? LD_VEC : LD_STRIDED, pl.cl = pl.cl == LD_VEC ? LD_VEC : LD_STRIDED;
   p.out = (char*)C;
   p.out_si = d->ldc;
   p.out_sjo = 0;

@@ -21,7 +21,7 @@ template <int DT, int RL, int CL, int TI, int TJ>
 Instance* instance() {
   static Instance inst;
   static const char* dtn[] = {"f16", "bf16", "i8"};
-  static const char* ldn[] = {"vec", "strided", "im2col"};
+  static const char* ldn[] = {"vec", "strided", "im2col", "tvec"};
   static std::string name = std::string("amos_igemm<") + dtn[DT] + "," + ldn[RL] + "," + ldn[CL] +
                             "," + std::to_string(64 * TI) + "x" + std::to_string(64 * TJ) + ">";
   inst.fn = amos_igemm<DT, RL, CL, TI, TJ>;
@@ -50,7 +50,18 @@ Instance* pick_col(int cl, int ti, int tj) {
     case LD_VEC: return pick_tile<DT, RL, LD_VEC>(ti, tj);
     case LD_STRIDED: return pick_tile<DT, RL, LD_STRIDED>(ti, tj);
     case LD_CONV: return pick_tile<DT, RL, LD_CONV>(ti, tj);
+    case LD_TVEC:
+      // 16-bit types, next to a vec or tvec row loader
+      if constexpr (DT != DT_I8 && RL != LD_STRIDED) return pick_tile<DT, RL, LD_TVEC>(ti, tj);
+      return nullptr;
   }
+  return nullptr;
+}
+// row loader tvec: column loaders vec and tvec
+template <int DT>
+Instance* pick_col_tvec(int cl, int ti, int tj) {
+  if (cl == LD_VEC) return pick_tile<DT, LD_TVEC, LD_VEC>(ti, tj);
+  if (cl == LD_TVEC) return pick_tile<DT, LD_TVEC, LD_TVEC>(ti, tj);
   return nullptr;
 }
 
@@ -154,6 +165,8 @@ ConvInstance* pick_conv_tile(int ti, int tj, int waves, int pls, int occ, int w9
 }
 #endif
 
+Instance* pick_f16_tvec(int cl, int ti, int tj);
+Instance* pick_bf16_tvec(int cl, int ti, int tj);
 Instance* pick_f16_vec(int cl, int ti, int tj);
 Instance* pick_f16_strided(int cl, int ti, int tj);
 Instance* pick_bf16_vec(int cl, int ti, int tj);

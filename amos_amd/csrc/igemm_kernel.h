@@ -35,7 +35,10 @@ typedef _Float16 v8h __attribute__((ext_vector_type(8)));
 typedef __bf16 v8bf __attribute__((ext_vector_type(8)));
 
 enum { DT_F16 = 0, DT_BF16 = 1, DT_I8 = 2 };
-enum { LD_VEC = 0, LD_STRIDED = 1, LD_CONV = 2 };
+// LD_VEC: K contiguous, 16-byte loads.  LD_STRIDED: any strides, element loads.  LD_CONV: im2col
+// gather.  LD_TVEC (16-bit types): ROWS contiguous (a transposed A, a row-major B): vector loads
+// along the rows, transposed in registers on the way to LDS.
+enum { LD_VEC = 0, LD_STRIDED = 1, LD_CONV = 2, LD_TVEC = 3 };
 
 // v_mfma 32x32 with 32 bytes of K per row per issue.  Operand fragment layout:
 // lane l holds the 16 bytes  k-bytes [16*(l/32), 16*(l/32)+16)  of row (l%32) for
@@ -95,6 +98,8 @@ template <>
 __device__ __forceinline__ int epi_value<int>(const EpiParams& e, int64_t idx) {
   return ((const int*)e.ptr)[idx];
 }
+
+template <int N> struct NSlots { static constexpr int value = N; };
 
 struct ConvGeom {
   int C, D, H, W;   // C = channels that are reduced over (of one group)
@@ -195,6 +200,9 @@ __global__ __launch_bounds__(256) void amos_igemm(const IgemmParams p) {
     if (RL == LD_VEC) {
       r_chunk[u] = item & 7;
       r_row[u] = item >> 3;
+    } else if (RL == LD_TVEC) {     // thread = (group of NR adjacent rows, K chunk): one row per slot
+      r_row[u] = (t & 31) * NR + u;
+      r_chunk[u] = t >> 5;
     } else {
       r_row[u] = item % BI;
       r_chunk[u] = item / BI;
@@ -207,6 +215,9 @@ __global__ __launch_bounds__(256) void amos_igemm(const IgemmParams p) {
     if (CL == LD_VEC) {
       c_chunk[u] = item & 7;
       c_row[u] = item >> 3;
+    } else if (CL == LD_TVEC) {
+      c_row[u] = (t & 31) * NC + u;
+      c_chunk[u] = t >> 5;
     } else {
       c_row[u] = item % BJ;
       c_chunk[u] = item / BJ;
@@ -292,10 +303,48 @@ __global__ __launch_bounds__(256) void amos_igemm(const IgemmParams p) {
     return v;
   };
 
+  // LD_TVEC: the thread's N adjacent rows (2*N contiguous bytes) at 8 consecutive k -> N chunks
+  // of 8 k each.  Rows come in groups that are entirely inside or outside the operand (the host
+  // takes this loader only for row extents that are multiples of 8), k is checked per load.
+  auto tvec_load = [&](const char* base, int64_t s_k, int row0, int rows, int k0c, v4i* dst, auto n_c) {
+    constexpr int N = decltype(n_c)::value;     // 2, 4 or 8 rows per thread
+    unsigned in[8][N / 2];
+#pragma unroll
+    for (int x = 0; x < 8; ++x) {
+      const bool ok = row0 < rows && k0c + x < p.Kred;
+      const char* src = base + ((int64_t)(k0c + x) * s_k + row0) * 2;
+      if (N == 8) {
+        v4i v = {0, 0, 0, 0};
+        if (ok) v = *(const v4i*)src;
+        in[x][0] = v.x; in[x][1 % (N / 2)] = v.y; in[x][2 % (N / 2)] = v.z; in[x][3 % (N / 2)] = v.w;
+      } else if (N == 4) {
+        int2 v = {0, 0};
+        if (ok) v = *(const int2*)src;
+        in[x][0] = v.x; in[x][1 % (N / 2)] = v.y;
+      } else {
+        in[x][0] = ok ? *(const unsigned*)src : 0u;
+      }
+    }
+#pragma unroll
+    for (int r = 0; r < N; ++r) {
+      const unsigned sel = (r & 1) ? 0x07060302u : 0x05040100u;   // high / low halves of (b, a)
+      v4i o;
+      o.x = (int)__builtin_amdgcn_perm(in[1][r / 2], in[0][r / 2], sel);
+      o.y = (int)__builtin_amdgcn_perm(in[3][r / 2], in[2][r / 2], sel);
+      o.z = (int)__builtin_amdgcn_perm(in[5][r / 2], in[4][r / 2], sel);
+      o.w = (int)__builtin_amdgcn_perm(in[7][r / 2], in[6][r / 2], sel);
+      dst[r] = o;
+    }
+  };
+
   auto gload = [&](int kt) {
     const int k0 = kt * BKE;
+    if (RL == LD_TVEC)
+      tvec_load(rbase, p.row_s_k, bi0 + r_row[0], p.I, k0 + r_chunk[0] * CE, rreg, NSlots<NR>{});
+    if (CL == LD_TVEC)
+      tvec_load(cbase, p.col_s_k, bj0 + c_row[0], p.J, k0 + c_chunk[0] * CE, creg, NSlots<NC>{});
 #pragma unroll
-    for (int u = 0; u < NR; ++u) {
+    for (int u = 0; u < (RL == LD_TVEC ? 0 : NR); ++u) {
       int row = bi0 + r_row[u];
       int k = k0 + r_chunk[u] * CE;
       if (RL == LD_VEC) {
@@ -313,7 +362,7 @@ __global__ __launch_bounds__(256) void amos_igemm(const IgemmParams p) {
       }
     }
 #pragma unroll
-    for (int u = 0; u < NC; ++u) {
+    for (int u = 0; u < (CL == LD_TVEC ? 0 : NC); ++u) {
       int row = bj0 + c_row[u];
       int k = k0 + c_chunk[u] * CE;
       if (CL == LD_VEC) {

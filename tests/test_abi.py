@@ -94,8 +94,16 @@ def test_kernel_name_reflects_layout():
     cfg = _lib.KernelConfig(128, 128, 1)
     assert lib.amos_kernel_name(0, ctypes.byref(gemm_desc(256, 256, 256, tb=1)), ctypes.byref(cfg)) == \
         b"amos_igemm<f16,vec,vec,128x128>"
+    # row-major B: rows (n) contiguous, vector loads transposed in registers ...
     assert lib.amos_kernel_name(0, ctypes.byref(gemm_desc(256, 256, 256)), ctypes.byref(cfg)) == \
+        b"amos_igemm<f16,vec,tvec,128x128>"
+    assert lib.amos_kernel_name(0, ctypes.byref(gemm_desc(256, 256, 256, ta=1)), ctypes.byref(cfg)) == \
+        b"amos_igemm<f16,tvec,tvec,128x128>"
+    # ... unless N is not a multiple of 8, or the type is 8-bit: element loads
+    assert lib.amos_kernel_name(0, ctypes.byref(gemm_desc(256, 252, 256)), ctypes.byref(cfg)) == \
         b"amos_igemm<f16,vec,strided,128x128>"
+    assert lib.amos_kernel_name(0, ctypes.byref(gemm_desc(256, 256, 256, _lib.AMOS_I8, _lib.AMOS_I32)),
+                                ctypes.byref(cfg)) == b"amos_igemm<i8,vec,strided,128x128>"
     assert lib.amos_kernel_name(0, ctypes.byref(gemm_desc(256, 256, 255, tb=1)), ctypes.byref(cfg)) == \
         b"amos_igemm<f16,strided,strided,128x128>"
     c = _lib.ConvDesc()

@@ -107,6 +107,35 @@ def test_gemm_direct_pipeline(gpu, dtype, pipeline, shape):
     check(gb, co.lib_gemm(ab, bb, dtype, False, True, acc="float64"), dtype, "direct bgemm")
 
 
+@pytest.mark.parametrize("dtype", ["float16", "bfloat16"])
+@pytest.mark.parametrize("trans", [(0, 0), (1, 0), (1, 1)])
+@pytest.mark.parametrize("tile", TILES)
+def test_gemm_row_contiguous_operands(gpu, dtype, trans, tile):
+    """operands whose ROWS are contiguous (row-major B, transposed A) take vector loads along the
+    rows and are transposed in registers; ragged K, row extents that are multiples of 8 but not
+    of the tile, split-K, batches"""
+    from amos_amd import _lib, ops
+    M, N, K = 520, 392, 1104      # K: whole 16-byte chunks, not whole 64-element steps
+    ta, tb = trans
+    rng = np.random.default_rng(11)
+    a = make_operand(rng, (K, M) if ta else (M, K), dtype)
+    b = make_operand(rng, (N, K) if tb else (K, N), dtype)
+    da, db = to_device(a, dtype), to_device(b, dtype)
+    d = ops.gemm_desc(M, N, K, da.dtype, ta, tb)
+    cfg = dict(tile_i=tile[0], tile_j=tile[1], split_k=1)
+    name = ops.kernel_name(_lib.AMOS_OP_GEMM, d, cfg)
+    assert name.startswith("amos_igemm<") and "tvec" in name, name
+    ref = co.lib_gemm(a, b, dtype, ta, tb, acc="float64")
+    for split in (1, 3):
+        got = ops.gemm(da, db, ta, tb, config=dict(cfg, split_k=split)).cpu().numpy()
+        check(got, ref, dtype, "%s %s tile %s split %d" % (name, trans, tile, split))
+    if tile == (128, 128):
+        ab = make_operand(rng, (3, K, M) if ta else (3, M, K), dtype)
+        bb = make_operand(rng, (3, N, K) if tb else (3, K, N), dtype)
+        gb = ops.bgemm(to_device(ab, dtype), to_device(bb, dtype), ta, tb, config=cfg).cpu().numpy()
+        check(gb, co.lib_gemm(ab, bb, dtype, ta, tb, acc="float64"), dtype, "batched %s" % name)
+
+
 def test_gemm_direct_pipeline_rejects_ragged_k(gpu):
     import torch
     from amos_amd import _lib, ops
