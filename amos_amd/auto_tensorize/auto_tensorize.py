@@ -238,7 +238,9 @@ def auto_tensorize_v4(target_dag, target, schedule_log_file, measure_opt, schedu
                 else:
                     if key not in cache:
                         try:
-                            gen = MI355XScheduleGenerator(match_result, new_state, log_file=log)
+                            gen = MI355XScheduleGenerator(
+                                match_result, new_state, log_file=log,
+                                perf_percentage=perf_percentage if enable_perf_model else 1.0)
                         except NoKernelError as e:
                             print("No kernel for this compute:", e, flush=True)
                             gen = None

@@ -124,6 +124,8 @@ class MI355XScheduleGenerator(object):
         self._open_log()
         self._candidates = None
         self._cursor = 0
+        # fraction of the model-ranked candidates the sweep may measure (1.0 = all)
+        self.perf_percentage = float(kwargs.get("perf_percentage", 1.0))
 
     # ---- log ------------------------------------------------------------------------------
     def _open_log(self):
@@ -204,16 +206,25 @@ class MI355XScheduleGenerator(object):
 
         d = _lib.KernelConfig()
         if lib.amos_default_config(low.op_code, ctypes.byref(low.desc), ctypes.byref(d)) == 0:
-            add(KernelParams(d.tile_i, d.tile_j, d.split_k, 0))
+            add(KernelParams(d.tile_i, d.tile_j, d.split_k, d.pipeline))
         is_conv = low.kind in ("conv2d", "conv3d")
         pipes = pipelines if pipelines is not None else (
             [_lib.AMOS_PIPE_PATCH, _lib.AMOS_PIPE_PATCH8, _lib.AMOS_PIPE_STAGED] if is_conv else [_lib.AMOS_PIPE_AUTO, _lib.AMOS_PIPE_STAGED])
+        first = len(out)
         for pipe in pipes:
             for ti, tj in _TILES:
                 for split in (1, 2, 4, 8):
                     if split > 1 and low.kind == "bgemm":
                         continue
                     add(KernelParams(ti, tj, split, pipe))
+        # The sweep visits candidates in the order of the analytical model (the mapper's own
+        # choice stays first), so that a small trial budget is spent on the likely winners; the
+        # reference ranks candidates with its performance model the same way before measuring
+        # (auto_tensorize.py:1018-1035, backend/tenet_integrate.py:168-202).
+        out[first:] = sorted(out[first:], key=self.estimate)
+        if self.perf_percentage < 1.0:
+            keep = max(1, int(round(len(out) * self.perf_percentage)))
+            out = out[:keep]
         if pipelines is None:
             self._candidates = out
         return out

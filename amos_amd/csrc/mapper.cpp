@@ -39,6 +39,18 @@ int problem_of(int op, const void* desc, Problem* out) {
         return set_error(AMOS_ERR_BAD_ARG, "non-positive GEMM extent");
       out->I = g->M; out->J = g->N; out->K = g->K; out->batch = batch;
       out->in_dtype = g->in_dtype;
+      {
+        const int es = esize(g->in_dtype), ce = 16 / es;
+        auto loader = [&](bool k_contiguous, int64_t ld, int64_t rows) {
+          if (k_contiguous) return (ld % ce == 0 && g->K % ce == 0) ? 0 : 1;
+          return (es == 2 && ld % 8 == 0 && rows % 8 == 0) ? 3 : 1;
+        };
+        out->row_loader = loader(!g->trans_a, g->lda, g->M);
+        out->col_loader = loader(g->trans_b != 0, g->ldb, g->N);
+        if ((out->row_loader == 3 && out->col_loader == 1) || (out->col_loader == 3 && out->row_loader == 1))
+          out->row_loader = out->row_loader == 0 ? 0 : 1, out->col_loader = out->col_loader == 0 ? 0 : 1;
+        out->direct_ok = out->row_loader == 0 && out->col_loader == 0 && g->K % (128 / es) == 0;
+      }
       out->in_bytes = batch * (g->M * g->K + g->K * g->N) * esize(g->in_dtype);
       out->out_bytes = batch * g->M * g->N * 4;
       return 0;
@@ -66,6 +78,8 @@ int problem_of(int op, const void* desc, Problem* out) {
       out->in_dtype = c->in_dtype;
       out->in_bytes = (c->N * c->C * D * c->H * c->W + c->K * out->K) * esize(c->in_dtype);
       out->out_bytes = c->K * out->J * 4;
+      out->row_loader = (out->K % (16 / esize(c->in_dtype)) == 0) ? 0 : 1;
+      out->col_loader = 2;
       return 0;
     }
   }
@@ -255,50 +269,83 @@ static int64_t lds_bytes_of(int ti, int tj) { return 2ll * (ti + tj) * 128 + 2 *
 // accumulator registers per lane: (ti/2 x tj/2 wave tile) / 64 lanes
 static int64_t acc_regs_of(int ti, int tj) { return (int64_t)(ti / 2) * (tj / 2) / 64; }
 
-// Estimated seconds of one launch for a tile shape and split.  Three terms, the
-// largest wins: MFMA issue time of the busiest CU (wave quantisation of the grid
-// over 256 CUs, with an inner-loop efficiency that grows with the wave tile since
-// LDS reads per MFMA fall), HBM time for the algorithmic bytes (plus the partial
-// sums of a split-K launch), and a fixed launch floor.
-static double estimate_seconds(const Problem& pb, int ti, int tj, int split) {
+// Estimated seconds of one launch of the register-staged kernel (or, for a 256x256 tile on
+// eligible operands, the direct-to-LDS GEMM kernel) for a tile shape and split.  A model of the
+// kernel's own structure with measured constants (profiles/mapper_model_calibration.md):
+//   * a workgroup advances one 128-byte K step in L1(tile) microseconds when it has a CU to itself;
+//   * a CU saturated with co-resident workgroups completes one workgroup-step every tau(tile)
+//     microseconds (tau < L1: the loads of one workgroup hide behind the MFMAs of another);
+//   * a CU that holds c workgroups therefore needs max(L1, c * tau) per step of all of them, and
+//     the busiest CU has ceil(workgroups / CUs) of them, at most occ(tile) at a time;
+//   * operands that are not loaded as 16-byte vectors along K slow both constants down;
+//   * split-K adds the zero fill and the atomic read-modify-writes of the output.
+struct TileCost { int ti, tj, occ; double tau_us, alone_us; };
+static const TileCost kTileCost[] = {
+    {256, 256, 1, 2.45, 2.75}, {256, 128, 1, 1.38, 1.55}, {128, 256, 1, 1.46, 1.65},
+    {128, 128, 2, 0.654, 1.03}, {256, 64, 1, 1.09, 1.17}, {128, 64, 3, 0.394, 0.69},
+    {64, 128, 3, 0.403, 0.69},  {64, 64, 4, 0.24, 0.50},  {64, 256, 1, 1.26, 1.22}};
+static const TileCost kDirectCost = {256, 256, 1, 1.95, 1.65};   // amos_gemm_tn, 8 waves
+
+static double loader_factor(int loader) {
+  switch (loader) {
+    case 1: return 3.0;    // element loads: 8 (fp16) or 16 (int8) per 16-byte chunk
+    case 2: return 4.5;    // im2col gather: element loads plus the tap arithmetic
+    case 3: return 1.12;   // vectors along the rows, transposed in registers
+  }
+  return 1.0;
+}
+
+static double estimate_seconds(const Problem& pb, int ti, int tj, int split, bool allow_direct = true) {
   const double es = pb.in_dtype == AMOS_I8 ? 1.0 : 2.0;
-  const double rate = (pb.in_dtype == AMOS_I8 ? Gfx950::kOpsPerClkCuI8 : Gfx950::kFlopsPerClkCuF16) *
-                      Gfx950::kClockGhz * 1e9;
-  const int64_t tiles = ((pb.I + ti - 1) / ti) * ((pb.J + tj - 1) / tj) * pb.batch * split;
-  const int per_cu = (int)std::min<int64_t>(Gfx950::kLdsBytes / lds_bytes_of(ti, tj), 2);
-  const int64_t slots = (int64_t)Gfx950::kComputeUnits * per_cu;
-  const int64_t rounds = (tiles + slots - 1) / slots;
-  const double bke = 128.0 / es;
-  const double ksteps = std::ceil(std::ceil((double)pb.K / bke) / split);
-  // LDS bytes read per MFMA flop fall with the wave tile; 0.85 is the ceiling we plan with
-  const double wave_i = ti / 2.0, wave_j = tj / 2.0;
-  const double eff = 0.85 * (wave_i * wave_j) / (wave_i * wave_j + 24.0 * (wave_i + wave_j));
-  const double tile_flop = 2.0 * ti * tj * ksteps * bke;
-  const double t_tile = tile_flop / (rate * eff) * per_cu;  // co-resident blocks share the CU
-  const double t_mfma = rounds * t_tile + 1.5e-6 /* prologue + epilogue */;
-  double bytes = (double)pb.in_bytes + (double)pb.out_bytes * (split > 1 ? 2.0 * split + 1.0 : 1.0);
-  const double t_hbm = bytes / Gfx950::kHbmBytesPerSec;
-  return std::max(t_mfma, t_hbm) + 2e-6;
+  const TileCost* tc = nullptr;
+  for (auto& t : kTileCost)
+    if (t.ti == ti && t.tj == tj) tc = &t;
+  if (!tc) return 1e9;
+  const bool direct = allow_direct && pb.direct_ok && ti == 256 && tj == 256 && split == 1;
+  if (direct) tc = &kDirectCost;
+  const double k_tiles = std::ceil((double)pb.K / (128.0 / es));
+  const int eff_split = (int)std::min<double>(split, k_tiles);
+  const double ksteps = std::ceil(k_tiles / eff_split);
+  const double lf = direct ? 1.0 : loader_factor(pb.row_loader) * loader_factor(pb.col_loader);
+  const double tau = tc->tau_us * lf, alone = tc->alone_us * lf;
+  const int64_t blocks = ((pb.I + ti - 1) / ti) * ((pb.J + tj - 1) / tj) * pb.batch * eff_split;
+  const int64_t per_cu = (blocks + Gfx950::kComputeUnits - 1) / Gfx950::kComputeUnits;
+  const int64_t groups = per_cu / tc->occ, rest = per_cu % tc->occ;
+  double step_us = (double)groups * std::max(alone, tc->occ * tau);
+  if (rest) step_us += std::max(alone, (double)rest * tau);
+  double t = 3e-6 + ksteps * step_us * 1e-6;
+  // output: written once; a split-K launch zero-fills it and accumulates with atomics (measured:
+  // (1 + 2*split) passes over the output at ~3.5 TB/s)
+  if (eff_split > 1) t += (double)pb.out_bytes * (1.0 + 2.0 * eff_split) / 3.5e12;
+  // memory floor; the shorter of the two legs is not hidden completely, which also orders
+  // memory-bound candidates by their compute time
+  const double t_hbm = ((double)pb.in_bytes + (double)pb.out_bytes) / (0.7 * Gfx950::kHbmBytesPerSec) + 3e-6;
+  return std::max(t, t_hbm) + 0.1 * std::min(t, t_hbm);
 }
 
 // Patch-staged convolution: blocks of one per CU; a K step costs its MFMA issue time plus a
 // per-step instruction overhead that does not shrink with the tile; split-K pays for atomic
 // accumulation into the output.  Returns <= 0 where the pipeline does not apply.
 static double conv_patch_estimate(const amos_conv_desc_t& c, int op, const Problem& pb, int ti, int tj,
-                                  int split) {
-  ConvPatchPlan pp = conv_patch_plan(c, op, ti, tj, split, 0);
+                                  int split, int waves = 0, bool allow_w9 = true) {
+  ConvPatchPlan pp = conv_patch_plan(c, op, ti, tj, split, waves, allow_w9);
   if (pp.why) return -1.0;
   const bool two_streams = pp.occ == 2 || pp.waves == 8;   // two waves per SIMD
   const double es = pb.in_dtype == AMOS_I8 ? 1.0 : 2.0;
   const int64_t T = op == AMOS_OP_CONV2D ? 1 : c.T;
   const double steps_all = (double)T * c.R * c.S * std::ceil(c.C * es / 128.0);
+  const double macro_steps = (double)T * std::ceil(c.C * es / 128.0);
+  if (split > macro_steps) split = (int)macro_steps;     // what the launch clamps it to
   const double blocks = std::ceil((double)pb.I / ti) * std::ceil((double)pb.J / tj) * split;
   // two resident workgroups take turns on the matrix cores while their per-step instruction
   // overheads overlap
   const double rounds = std::ceil(blocks / (Gfx950::kComputeUnits * (double)pp.occ));
   const double steps = std::ceil(steps_all / split);
   const double mfma_per_step = (ti / 64.0) * (tj / 64.0) * 4.0 * 32.0;
-  const double cycles = rounds * (steps * (pp.occ * mfma_per_step + (two_streams ? 500.0 : 600.0)) + 4000.0);
+  // measured (profiles/conv_fprop_kernel_trace.md): a 128x64 step takes ~700 cycles with the taps
+  // unrolled, ~760 with two instruction streams per SIMD, ~850 with one; set-up 6000-8000 cycles
+  const double overhead = pp.w9 ? 440.0 : two_streams ? 500.0 : 600.0;
+  const double cycles = rounds * (steps * (pp.occ * mfma_per_step + overhead) + (pp.w9 ? 8000.0 : 6000.0));
   const double relayout = ((double)pb.in_bytes * 2.0) / 2.5e12 + 3e-6;
   return cycles / 2.1e9 + relayout + (split > 1 ? (double)pb.out_bytes * split / 1.2e12 : 0.0);
 }
@@ -345,19 +392,23 @@ int amos_estimate_seconds(int op, const void* desc, const amos_kernel_config_t* 
   if (rc) return rc;
   const int split = cfg->split_k < 1 ? 1 : cfg->split_k;
   if ((op == AMOS_OP_CONV2D || op == AMOS_OP_CONV3D) && cfg->pipeline != AMOS_PIPE_STAGED) {
-    double s = conv_patch_estimate(*(const amos_conv_desc_t*)desc, op, pb, cfg->tile_i, cfg->tile_j, split);
+    const int waves = cfg->pipeline == AMOS_PIPE_PATCH ? 4 : cfg->pipeline == AMOS_PIPE_PATCH8 ? 8 : 0;
+    double s = conv_patch_estimate(*(const amos_conv_desc_t*)desc, op, pb, cfg->tile_i, cfg->tile_j, split,
+                                   waves, !(cfg->reserved[0] & AMOS_FLAG_NO_UNROLLED_TAPS));
     if (s > 0) { *seconds = s; return 0; }
+    if (waves) return set_error(AMOS_ERR_INFEASIBLE, "patch-staged convolution not applicable to this config");
   }
-  *seconds = estimate_seconds(pb, cfg->tile_i, cfg->tile_j, split);
+  *seconds = estimate_seconds(pb, cfg->tile_i, cfg->tile_j, split, cfg->pipeline != AMOS_PIPE_STAGED);
   return 0;
 }
 
-int amos_default_config(int op, const void* desc, amos_kernel_config_t* out) {
+int amos_default_config(int op, const void* desc, amos_kernel_config_t* result) {
   Problem pb;
   int rc = problem_of(op, desc, &pb);
   if (rc) return rc;
-  if (!out) return set_error(AMOS_ERR_BAD_ARG, "null config");
-  memset(out, 0, sizeof(*out));
+  if (!result) return set_error(AMOS_ERR_BAD_ARG, "null config");
+  memset(result, 0, sizeof(*result));
+  amos_kernel_config_t* out = result;
   const double es = pb.in_dtype == AMOS_I8 ? 1.0 : 2.0;
   const int k_tiles = (int)std::ceil((double)pb.K / (128.0 / es));
   double best = 1e30;
@@ -377,20 +428,27 @@ int amos_default_config(int op, const void* desc, amos_kernel_config_t* out) {
         }
       }
     }
-    if (best < 1e30) return 0;
   }
+  // a convolution leaves the patch-staged pipeline only for a clearly better estimate of the
+  // register-staged kernel (whose im2col constants are the less certain ones)
+  const double patch_best = best;
+  amos_kernel_config_t staged = *out;
+  if (patch_best < 1e30) best = patch_best / 1.25;
+  out = &staged;
   for (auto& t : kTiles) {
     for (int split = 1; split <= 16; split *= 2) {
-      if (split > 1 && (split > k_tiles / 4 || pb.batch > 1)) break;
+      if (split > 1 && (split > k_tiles / 2 || pb.batch > 1)) break;
       double s = estimate_seconds(pb, t[0], t[1], split);
       if (s < best * 0.98) {
         best = s;
         out->tile_i = t[0];
         out->tile_j = t[1];
         out->split_k = split;
+        out->pipeline = patch_best < 1e30 ? AMOS_PIPE_STAGED : AMOS_PIPE_AUTO;
       }
     }
   }
+  *result = staged;
   return 0;
 }
 

@@ -27,6 +27,11 @@ struct Problem {
   int64_t I, J, K, batch;
   int in_dtype;
   int64_t in_bytes, out_bytes;  // algorithmic bytes: every input read once, output written once
+  // how the register-staged kernel would load the two operands (leading dimensions assumed
+  // aligned): 0 = 16-byte vectors along K, 1 = element loads, 2 = im2col gather, 3 = vectors
+  // along the rows transposed in registers
+  int row_loader, col_loader;
+  int direct_ok;                // the direct-to-LDS GEMM kernel applies (256x256 tile)
 };
 
 int problem_of(int op, const void* desc, Problem* out);

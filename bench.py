@@ -1,7 +1,7 @@
 """Headline benchmark: fp16 GEMM M=N=K=8192, fp32 accumulate, row-major A, column-major B,
 on one MI355X, next to the CPU restatement of the reference's llvm path timed in the same run.
 
-  python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--report FILE]
+  python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--report FILE] [--model-check FILE]
 
 A step is one launch of the GEMM over device-resident operands.  Prints ONE JSON line.
 `--report FILE` additionally times every configuration of the path (GEMM, batched GEMM,
@@ -151,6 +151,97 @@ def run_all_configs(cpu=True):
     return rows
 
 
+def model_check():
+    """The mapper's analytical model against measurement: for a set of shapes (the benchmark
+    configurations the constants were fitted on, and shapes they were not), every kernel
+    configuration is timed and ranked both ways."""
+    import ctypes
+    import torch
+    from scipy.stats import spearmanr
+    from amos_amd import _lib, ops
+    lib = _lib.load()
+    tiles = [(256, 256), (256, 128), (128, 256), (128, 128), (256, 64), (128, 64), (64, 128), (64, 64), (64, 256)]
+
+    def sweep(name, fitted, op, d, a, b, out, pipes, splits):
+        rows = []
+        for pipe in pipes:
+            for ti, tj in tiles:
+                for sp in splits:
+                    cfg = dict(tile_i=ti, tile_j=tj, split_k=sp, pipeline=pipe)
+                    c = ops.make_config(cfg)
+                    est = ctypes.c_double()
+                    if lib.amos_check_config(op, ctypes.byref(d), ctypes.byref(c), None, None) < 0 or \
+                            lib.amos_kernel_name(op, ctypes.byref(d), ctypes.byref(c)) is None or \
+                            lib.amos_estimate_seconds(op, ctypes.byref(d), ctypes.byref(c), ctypes.byref(est)) != 0:
+                        continue
+                    try:
+                        t = ops.time_op(op, d, a, b, out, config=cfg, number=5, repeat=1, min_repeat_ms=20)[0]
+                    except _lib.AmosError:
+                        continue
+                    rows.append((t, est.value, ops.kernel_name(op, d, cfg), sp))
+        rows.sort(key=lambda r: r[0])
+        by_est = sorted(rows, key=lambda r: r[1])
+        dflt = ops.default_config(op, d)
+        t_default = ops.time_op(op, d, a, b, out, config=dflt, number=5, repeat=1, min_repeat_ms=20)[0]
+        return {"shape": name, "fitted_on": fitted, "configs": len(rows),
+                "spearman": float(spearmanr([r[0] for r in rows], [r[1] for r in rows]).correlation),
+                "best_us": rows[0][0] * 1e6, "best_kernel": "%s split %d" % (rows[0][2], rows[0][3]),
+                "model_first_us": by_est[0][0] * 1e6, "model_first_est_us": by_est[0][1] * 1e6,
+                "model_first_kernel": "%s split %d" % (by_est[0][2], by_est[0][3]),
+                "rank_of_best_in_model_order": [i for i, r in enumerate(by_est) if r is rows[0]][0],
+                "default_config_us": t_default * 1e6,
+                "default_kernel": "%s split %d" % (ops.kernel_name(op, d, dflt), dflt.split_k)}
+
+    out = []
+    GEMM, BGEMM, CONV2D, CONV3D = _lib.AMOS_OP_GEMM, _lib.AMOS_OP_BGEMM, _lib.AMOS_OP_CONV2D, _lib.AMOS_OP_CONV3D
+    f16, i8 = torch.float16, torch.int8
+
+    def gemm_case(M, N, K, ta, tb, dt, fitted):
+        if dt == i8:
+            a = torch.randint(-8, 8, (K, M) if ta else (M, K), device="cuda", dtype=dt)
+            b = torch.randint(-8, 8, (N, K) if tb else (K, N), device="cuda", dtype=dt)
+            c = torch.empty(M, N, device="cuda", dtype=torch.int32)
+        else:
+            a = torch.randn((K, M) if ta else (M, K), device="cuda").to(dt)
+            b = torch.randn((N, K) if tb else (K, N), device="cuda").to(dt)
+            c = torch.empty(M, N, device="cuda")
+        name = "GEMM %dx%dx%d %s%s %s" % (M, N, K, "t" if ta else "n", "t" if tb else "n", str(dt).split(".")[1])
+        out.append(sweep(name, fitted, GEMM, ops.gemm_desc(M, N, K, dt, ta, tb), a, b, c, (0, 1), (1, 2, 4, 8)))
+
+    def conv_case(name, fitted, xs, ws, st, pd, dt=f16, op=CONV2D):
+        if dt == i8:
+            x = torch.randint(-128, 127, xs, device="cuda", dtype=dt)
+            w = torch.randint(-64, 63, ws, device="cuda", dtype=dt)
+        else:
+            x, w = torch.rand(xs, device="cuda").to(dt), (torch.randn(ws, device="cuda") * 0.05).to(dt)
+        xs5 = tuple(xs) if op == CONV3D else (xs[0], xs[1], 1, xs[2], xs[3])
+        ws5 = tuple(ws) if op == CONV3D else (ws[0], ws[1], 1, ws[2], ws[3])
+        d = ops.conv_desc(xs5, ws5, dt, st, pd, (1, 1, 1))
+        oshape = ops.conv_out_shape(xs5, ws5, st, pd, (1, 1, 1))
+        y = torch.empty(oshape if op == CONV3D else (oshape[0], oshape[1], oshape[3], oshape[4]),
+                        device="cuda", dtype=torch.int32 if dt == i8 else torch.float32)
+        out.append(sweep(name, fitted, op, d, x, w, y, (4, 5, 1), (1, 2, 4) if op == CONV2D else (1,)))
+
+    for M, N, K in [(8192, 8192, 8192), (2048, 2048, 2048), (512, 512, 4096), (4096, 256, 1024)]:
+        gemm_case(M, N, K, 0, 1, f16, True)
+    conv_case("C3 conv2d N32 C256 14x14 K256 3x3 f16", True, (32, 256, 14, 14), (256, 256, 3, 3), (1, 1, 1), (0, 1, 1))
+    conv_case("C4 conv2d N64 C128 28x28 K128 3x3 i8", True, (64, 128, 28, 28), (128, 128, 3, 3), (1, 1, 1), (0, 1, 1), i8)
+    conv_case("C5b conv3d N8 C64 D16 56x56 K64 3x3x3 f16", True, (8, 64, 16, 56, 56), (64, 64, 3, 3, 3), (1, 1, 1),
+              (1, 1, 1), f16, CONV3D)
+    for M, N, K, ta, tb, dt in [(3000, 1000, 2000, 0, 1, f16), (1024, 8192, 512, 0, 1, f16), (2048, 2048, 2048, 0, 0, f16),
+                                (6144, 768, 3072, 1, 0, f16), (2048, 2048, 2048, 0, 1, i8), (200, 120, 5000, 0, 1, f16)]:
+        gemm_case(M, N, K, ta, tb, dt, False)
+    a = torch.randn(16, 512, 256, device="cuda").half()
+    b = torch.randn(16, 512, 256, device="cuda").half()
+    c = torch.empty(16, 512, 512, device="cuda")
+    out.append(sweep("bGEMM 16x(512x512x256) nt f16", False, BGEMM, ops.bgemm_desc(16, 512, 512, 256, f16, False, True),
+                     a, b, c, (0, 1), (1,)))
+    conv_case("conv2d N8 C128 28x28 K256 3x3 f16", False, (8, 128, 28, 28), (256, 128, 3, 3), (1, 1, 1), (0, 1, 1))
+    conv_case("conv2d N16 C64 56x56 K64 1x1 f16", False, (16, 64, 56, 56), (64, 64, 1, 1), (1, 1, 1), (0, 0, 0))
+    conv_case("conv2d N4 C48 30x30 K96 5x5 f16", False, (4, 48, 30, 30), (96, 48, 5, 5), (1, 1, 1), (0, 2, 2))
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -158,6 +249,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU-baseline leg")
     ap.add_argument("--report", default=None, help="also time every config, write JSON here")
+    ap.add_argument("--model-check", default=None,
+                    help="also rank every kernel configuration of a set of shapes by the mapper's model "
+                         "and by measurement, write JSON here")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a 256 MiB device copy, the known-size kernel that rocprofv3's "
                          "FETCH_SIZE / WRITE_SIZE readings are scaled by")
@@ -223,6 +317,9 @@ def main():
     if args.report:
         with open(args.report, "w") as f:
             json.dump(run_all_configs(cpu=not args.no_cpu), f, indent=1)
+    if args.model_check:
+        with open(args.model_check, "w") as f:
+            json.dump(model_check(), f, indent=1)
     print(json.dumps(line), flush=True)
 
 
