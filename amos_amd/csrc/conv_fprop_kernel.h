@@ -268,9 +268,10 @@ __device__ __forceinline__ void wait_vmcnt_le(int n) {
 // three stages.  The tap loop is unrolled, so ring stages, patch buffers, patch read addresses
 // per tap, copy slots and wait counts are compile-time or precomputed registers, and a step is
 // about half the instructions of the table-driven one.  The patch buffers are a fixed distance
-// apart (it must fit the 16-bit offset field of ds_read): 56 KB next to 64-row weight tiles, 48 KB
-// next to 128-row ones.
-constexpr unsigned conv_w9_xbuf(int bi) { return bi <= 64 ? 56 * 1024 : 48 * 1024; }
+// apart, a multiple of 8 KB so that a position has the same swizzle in both: 48 KB next to
+// 128-row weight tiles (fits the 16-bit offset field of ds_read), 64 KB next to 64-row ones
+// (512 positions; the second buffer's read addresses cost an addition each).
+constexpr unsigned conv_w9_xbuf(int bi) { return bi <= 64 ? 64 * 1024 : 48 * 1024; }
 template <int N> struct IntC { static constexpr int value = N; };
 
 template <int DT, int BI64, int BJ64, int NW, int PL, int OCC, int W9 = 0>

@@ -226,10 +226,10 @@ static ConvPatchPlan conv_patch_plan_waves(const amos_conv_desc_t& cin, int op, 
                    : "input patch too large to prefetch behind the window's taps";
   };
   // the instance with the nine taps unrolled: 8 waves, three ring stages, patch buffers a fixed
-  // 48 KB (56 KB next to 64-row weight tiles) apart, the next patch fetched on taps 0..6 with at
+  // 48 KB (64 KB next to 64-row weight tiles) apart, the next patch fetched on taps 0..6 with at
   // most two copies per wave and step
   if (allow_w9 && waves == 8 && RS == 9 && BI <= 128 && BJ <= 128 && !(BI == 64 && BJ == 64)) {
-    const int max_pos9 = one_macro ? max_pos : (BI <= 64 ? 448 : 384);
+    const int max_pos9 = one_macro ? max_pos : (BI <= 64 ? 512 : 384);
     const size_t patch9 = (size_t)pp.xbufs * max_pos9 * 128 + (size_t)max_pos9 * 8 + 1024;
     const int pls9 = one_macro ? 0 : (per_wave + 6) / 7;
     if (real_pos <= max_pos9 && 3 * wstage + patch9 <= budget && pls9 <= 2) {
