@@ -53,6 +53,7 @@ class KernelConfig(ctypes.Structure):
 
 
 AMOS_EPI_NONE, AMOS_EPI_ADD = 0, 1
+AMOS_FLAG_NO_UNROLLED_TAPS, AMOS_FLAG_NO_TILE_WALK = 1, 2
 
 
 class Epilogue(ctypes.Structure):

@@ -292,7 +292,7 @@ static int plan_conv(Plan& pl, int op, const amos_conv_desc_t* d, const amos_ker
   const int Wp = (OQ - 1) * c.stride_w + ((int)c.S - 1) * c.dil_w + 1;
   ConvPatchPlan pp = conv_patch_plan(c, op, BI, BJ, pl.cfg.split_k,
                                      pipe == AMOS_PIPE_PATCH ? 4 : pipe == AMOS_PIPE_PATCH8 ? 8 : 0,
-                                     !(pl.cfg.reserved[0] & AMOS_FLAG_NO_UNROLLED_TAPS));
+                                     conv_unroll_level(pl.cfg.reserved[0]));
   const char* why = pp.why;
   if (!why && (!workspace || ws_bytes < (size_t)need_ws || ((uintptr_t)workspace & 255)))
     why = "workspace smaller than amos_workspace_bytes() or not 256-byte aligned";
@@ -330,6 +330,12 @@ static int plan_conv(Plan& pl, int op, const amos_conv_desc_t* d, const amos_ker
   q.sx_off = nsw * BI * 128;
   q.tab_off = q.sx_off + pp.xbufs * max_pos * 128;
   q.dump_off = q.tab_off + max_pos * 8;
+  q.tab1_off = q.tab_off;
+  if (pp.w9) {
+    q.tab_off = q.sx_off + pp.tab_rel;
+    q.tab1_off = q.sx_off + pp.tab1_rel;
+    q.dump_off = q.sx_off + pp.dump_rel;
+  }
   q.c_chunks = (int)(c.C * es / 128);
   q.macro_steps = (int)c.T * q.c_chunks;
   q.total_steps = q.macro_steps * RS;
@@ -431,6 +437,8 @@ static int launch_conv(const Plan& pl, hipStream_t stream) {
   const ConvFpropParams& q = pl.cv;
   launch_conv_prepare(pl.dt == DT_I8 ? 1 : 2, q, stream);
   dim3 grid((unsigned)(q.tiles_i * q.tiles_j), (unsigned)pl.split, 1);
+  // blocks that walk their tiles: one per compute unit, tiles blockIdx.x, + gridDim.x, ...
+  if (pl.conv_w9 == 2 && grid.x > (unsigned)Gfx950::kComputeUnits) grid.x = Gfx950::kComputeUnits;
   hipLaunchKernelGGL(inst->fn, grid, dim3(inst->threads), pl.conv_lds, stream, q);
   HIP_TRY(hipGetLastError());
   return 0;

@@ -55,8 +55,10 @@ inline FastDiv make_fast_div(uint32_t d) {
   f.shift = (uint32_t)(s - 32);
   return f;
 }
+// (branch-free: a branch per division would keep the scalar loads of the kernel arguments from
+// being issued together, and each then costs its full latency)
 __device__ __forceinline__ int fast_div(int n, const FastDiv& f) {
-  return f.one ? n : (int)(__umulhi((unsigned)n, f.magic) >> f.shift);
+  return (int)((__umulhi((unsigned)n, f.magic) + (unsigned)n * f.one) >> f.shift);
 }
 
 #define AMOS_LDS_PTR_FROM(off) ((const __attribute__((address_space(3))) char*)(size_t)(off))
@@ -79,6 +81,7 @@ struct ConvFpropParams {
   int pls;           // patch copy instructions per wave per K step (the instance's PL)
   int xbufs;         // patch buffers: 2, or 1 when a block handles a single (depth tap, channel chunk)
   int sx_off, tab_off, dump_off;   // LDS byte offsets: patch buffers, position table, dump line
+  int tab1_off;      // second position table (blocks that walk several tiles)
   int total_steps;   // macro_steps * R * S
   void* steps;       // [total_steps + 1] step table (workspace), written by the prepare kernel
   int c_chunks;      // C*ES / 128
@@ -300,8 +303,8 @@ __global__ __launch_bounds__(64 * NW, OCC) void amos_conv_fprop(const ConvFpropP
   const int wi = wave / WJ, wj = wave % WJ;
   const int frag_row = lane & 31, frag_half = lane >> 5;
 
-  const int tile_j = blockIdx.x / p.tiles_i, tile_i = blockIdx.x - tile_j * p.tiles_i;
-  const int bi0 = tile_i * BI, bj0 = tile_j * BJ;
+  // W9 = 2: the block walks the tiles blockIdx.x, blockIdx.x + gridDim.x, ...; else one tile
+  constexpr bool PERSIST = W9 == 2;
   const int m_begin = blockIdx.y * p.macro_per_split;
   int m_end = m_begin + p.macro_per_split;
   if (m_end > p.macro_steps) m_end = p.macro_steps;
@@ -313,23 +316,62 @@ __global__ __launch_bounds__(64 * NW, OCC) void amos_conv_fprop(const ConvFpropP
   const unsigned xbuf_bytes = (unsigned)p.max_pos * 128u;
   const unsigned pos_bytes = (unsigned)p.C * ES;
 
+  // ---- what depends on the tile: its origin and image slices (wave-uniform scalars) --------------
+  typedef int seg4_t __attribute__((ext_vector_type(4)));
+  struct TileGeo {
+    int bi0, bj0, j_last, sl_a, nseg, npos;
+    // per slice, as vector values (arrays inside the struct would live in scratch memory)
+    seg4_t seg_pos0, seg_pa, seg_base, seg_d0;
+  };
+  static_assert(kConvMaxSeg == 4, "TileGeo holds four segments");
+  const int halo_rows = (p.R - 1) * p.dh + 1;
+  auto geo_of = [&](int tile_i, int tile_j) {
+    TileGeo q;
+    q.bi0 = tile_i * BI;
+    q.bj0 = tile_j * BJ;
+    q.j_last = (q.bj0 + BJ - 1 < p.J ? q.bj0 + BJ - 1 : p.J - 1);
+    q.sl_a = fast_div(q.bj0, p.fd_opq);
+    const int sl_b = fast_div(q.j_last, p.fd_opq);
+    q.nseg = sl_b - q.sl_a + 1;
+    int pos = 0;
+#pragma unroll
+    for (int g = 0; g < kConvMaxSeg; ++g) {
+      const int sl = q.sl_a + (g < q.nseg ? g : q.nseg - 1);
+      const int lo = q.bj0 > sl * OPQ ? q.bj0 : sl * OPQ;
+      const int hi = q.j_last < (sl + 1) * OPQ - 1 ? q.j_last : (sl + 1) * OPQ - 1;
+      const int pa = fast_div(lo - sl * OPQ, p.fd_oq), pb = fast_div(hi - sl * OPQ, p.fd_oq);
+      const int rows = (pb - pa) * p.sh + halo_rows;
+      const int n = fast_div(sl, p.fd_od);
+      q.seg_pos0[g] = pos;
+      q.seg_pa[g] = pa;
+      q.seg_d0[g] = (sl - n * p.OD) * p.sd - p.pd;
+      q.seg_base[g] = (n * p.D + q.seg_d0[g]) * HW;   // position index of (n, d0, 0, 0)
+      pos += g < q.nseg ? rows * p.Wp : 0;
+    }
+    q.npos = pos;
+    return q;
+  };
   // ---- weight copy slots ---------------------------------------------------------------------
   const unsigned w_row_bytes = (unsigned)(p.T * RS) * pos_bytes;
-  unsigned w_off[WCH];
+  auto weight_rows = [&](int bi0, unsigned (&wo)[WCH]) {
 #pragma unroll
-  for (int u = 0; u < WCH; ++u) {
-    const int q = wave + NW * u;   // 1 KB chunk = 8 rows
-    const int row = q * 8 + (lane >> 3);
-    const int chunk = (lane & 7) ^ ((row ^ (row >> 3)) & 7);
-    const int r = bi0 + row < p.K ? bi0 + row : p.K - 1;
-    w_off[u] = (unsigned)r * w_row_bytes + chunk * 16;
-  }
+    for (int u = 0; u < WCH; ++u) {
+      const int q = wave + NW * u;   // 1 KB chunk = 8 rows
+      const int row = q * 8 + (lane >> 3);
+      const int chunk = (lane & 7) ^ ((row ^ (row >> 3)) & 7);
+      const int r = bi0 + row < p.K ? bi0 + row : p.K - 1;
+      wo[u] = (unsigned)r * w_row_bytes + chunk * 16;
+    }
+  };
+  unsigned w_off[WCH];
+  const int tile_j0 = (int)(blockIdx.x / (unsigned)p.tiles_i), tile_i0 = (int)blockIdx.x - tile_j0 * p.tiles_i;
+  weight_rows(tile_i0 * BI, w_off);
   // weight tile whose K slice starts wk bytes into a packed weight row -> ring stage at stage_off
   // (32-bit offsets from the packed weights: the host keeps them under 4 GiB)
-  auto issue_weights = [&](unsigned wk, unsigned stage_off) {
+  auto issue_weights = [&](const unsigned (&wo)[WCH], unsigned wk, unsigned stage_off) {
 #pragma unroll
     for (int u = 0; u < WCH; ++u)
-      __builtin_amdgcn_global_load_lds(AMOS_GLOBAL_PTR(p.wp + (size_t)(w_off[u] + wk)),
+      __builtin_amdgcn_global_load_lds(AMOS_GLOBAL_PTR(p.wp + (size_t)(wo[u] + wk)),
                                        AMOS_LDS_PTR_RW(stage_off + (unsigned)(wave + NW * u) * 1024), 16, 0, 0);
   };
 
@@ -344,65 +386,49 @@ __global__ __launch_bounds__(64 * NW, OCC) void amos_conv_fprop(const ConvFpropP
     const unsigned last = (unsigned)(p.total_steps - 1);
     for (int u = 0; u < NSW; ++u) {
       const unsigned gu = (unsigned)(g + u) < last ? (unsigned)(g + u) : last;
-      issue_weights((unsigned)tbl[gu][7], (unsigned)u * WSTAGE);
+      issue_weights(w_off, (unsigned)tbl[gu][7], (unsigned)u * WSTAGE);
     }
   }
 
-  // ---- segments of this tile (wave-uniform scalars) -------------------------------------------
-  const int j_last = (bj0 + BJ - 1 < p.J ? bj0 + BJ - 1 : p.J - 1);
-  const int sl_a = fast_div(bj0, p.fd_opq), sl_b = fast_div(j_last, p.fd_opq);
-  const int nseg = sl_b - sl_a + 1;
-  int seg_pos0[kConvMaxSeg + 1], seg_pa[kConvMaxSeg], seg_base[kConvMaxSeg], seg_d0[kConvMaxSeg];
-  {
-    int pos = 0;
-#pragma unroll
-    for (int g = 0; g < kConvMaxSeg; ++g) {
-      const int sl = sl_a + (g < nseg ? g : nseg - 1);
-      const int lo = bj0 > sl * OPQ ? bj0 : sl * OPQ;
-      const int hi = j_last < (sl + 1) * OPQ - 1 ? j_last : (sl + 1) * OPQ - 1;
-      const int pa = fast_div(lo - sl * OPQ, p.fd_oq), pb = fast_div(hi - sl * OPQ, p.fd_oq);
-      const int rows = (pb - pa) * p.sh + (p.R - 1) * p.dh + 1;
-      const int n = fast_div(sl, p.fd_od);
-      seg_pos0[g] = pos;
-      seg_pa[g] = pa;
-      seg_d0[g] = (sl - n * p.OD) * p.sd - p.pd;
-      seg_base[g] = (n * p.D + seg_d0[g]) * HW;   // position index of (n, d0, 0, 0)
-      if (g < nseg) pos += rows * p.Wp;
-    }
-    seg_pos0[kConvMaxSeg] = pos;
-  }
-  const int npos = seg_pos0[kConvMaxSeg];
-  const int npos8 = (npos + 7) & ~7;
+  TileGeo geo = geo_of(tile_i0, tile_j0);
 
-  // position table: {byte offset of the position's channels in NDHWC at depth tap 0 (modulo 2^32;
-  // a depth shift is added before use), d0 + 32768, or 0 when (h, w) lies outside the image}
-  {
-    int2* const sTab = (int2*)(smem + p.tab_off);
+  // position table of a tile: {byte offset of the position's channels in NDHWC at depth tap 0
+  // (modulo 2^32; a depth shift is added before use), d0 + 32768, or 0 when (h, w) lies outside
+  // the image}
+  auto write_table = [&](const TileGeo& q, int tab_off) {
+    const int npos8 = (q.npos + 7) & ~7;
     for (int pos = t; pos < npos8; pos += 64 * NW) {
-      int g_pos0 = 0, g_pa = seg_pa[0], g_base = seg_base[0], g_d0 = seg_d0[0];
+      int g_pos0 = 0, g_pa = q.seg_pa[0], g_base = q.seg_base[0], g_d0 = q.seg_d0[0];
 #pragma unroll
       for (int g = 1; g < kConvMaxSeg; ++g)
-        if (g < nseg && pos >= seg_pos0[g]) { g_pos0 = seg_pos0[g]; g_pa = seg_pa[g]; g_base = seg_base[g]; g_d0 = seg_d0[g]; }
+        if (g < q.nseg && pos >= q.seg_pos0[g]) { g_pos0 = q.seg_pos0[g]; g_pa = q.seg_pa[g]; g_base = q.seg_base[g]; g_d0 = q.seg_d0[g]; }
       const int rel = pos - g_pos0;
       const int hr = fast_div(rel, p.fd_wp);
       const int wc = rel - hr * p.Wp;
       const int h = g_pa * p.sh - p.ph + hr, w = wc - p.pw;
-      const bool ok = pos < npos && (unsigned)h < (unsigned)p.H && (unsigned)w < (unsigned)p.W;
-      sTab[pos] = int2{(int)((unsigned)(g_base + h * p.W + w) * pos_bytes), ok ? g_d0 + 32768 : 0};
+      const bool ok = pos < q.npos && (unsigned)h < (unsigned)p.H && (unsigned)w < (unsigned)p.W;
+      const int2 e = int2{(int)((unsigned)(g_base + h * p.W + w) * pos_bytes), ok ? g_d0 + 32768 : 0};
+      ((int2*)(smem + tab_off))[pos] = e;
     }
-  }
+  };
+  write_table(geo, p.tab_off);
 
   // ---- patch copies: copy v of this wave fills positions [8q, 8q+8), q = wave + NW*v -------------
-  const int n_chunks8 = npos8 >> 3;
-  const int n_pl = n_chunks8 > wave ? (n_chunks8 - wave + NW - 1) / NW : 0;   // copies this wave owns per patch
-  const unsigned tab_lane = (unsigned)p.tab_off + (unsigned)(lane >> 3) * 8;
+  auto copies_of = [&](int npos) {   // copies this wave owns per patch
+    const int n_chunks8 = (npos + 7) >> 3;
+    return n_chunks8 > wave ? (n_chunks8 - wave + NW - 1) / NW : 0;
+  };
+  int n_pl = copies_of(geo.npos);
+  // table and copy count the patch copies read from: those of the tile whose patch is fetched
+  unsigned tab_lane = (unsigned)p.tab_off + (unsigned)(lane >> 3) * 8;
+  int n_pl_rd = n_pl;
   // 16-byte chunk a lane fetches: the swizzle of the LDS position it fills (8 KB-aligned buffers)
   const unsigned lane_c16 = (unsigned)((lane & 7) ^ (lane >> 3)) << 4;
   // The table is read with an explicit ds_read the compiler does not see as a memory access: next
   // to outstanding global -> LDS copies it would otherwise wait for all of them before an LDS
   // load it cannot tell apart from their destinations.  The caller waits (lgkmcnt) before use.
   auto read_tab = [&](int v) {
-    int vq = v < n_pl - 1 ? v : n_pl - 1;
+    int vq = v < n_pl_rd - 1 ? v : n_pl_rd - 1;
     if (vq < 0) vq = 0;
     int2 e;
     asm volatile("ds_read_b64 %0, %1" : "=v"(e) : "v"(tab_lane + (unsigned)(wave + NW * vq) * 64));
@@ -422,18 +448,21 @@ __global__ __launch_bounds__(64 * NW, OCC) void amos_conv_fprop(const ConvFpropP
 
   // ---- this lane's output columns -> patch positions ---------------------------------------------
   unsigned col_byte[TJ];
+  auto column_bytes = [&](const TileGeo& q) {
 #pragma unroll
-  for (int b = 0; b < TJ; ++b) {
-    int j = bj0 + (wj * TJ + b) * 32 + frag_row;
-    if (j > j_last) j = j_last;
-    const int sl = fast_div(j, p.fd_opq), rem = j - sl * OPQ;
-    const int op = fast_div(rem, p.fd_oq), oq = rem - op * p.OQ;
-    int g_pos0 = seg_pos0[0], g_pa = seg_pa[0];
+    for (int b = 0; b < TJ; ++b) {
+      int j = q.bj0 + (wj * TJ + b) * 32 + frag_row;
+      if (j > q.j_last) j = q.j_last;
+      const int sl = fast_div(j, p.fd_opq), rem = j - sl * OPQ;
+      const int op = fast_div(rem, p.fd_oq), oq = rem - op * p.OQ;
+      int g_pos0 = q.seg_pos0[0], g_pa = q.seg_pa[0];
 #pragma unroll
-    for (int g = 1; g < kConvMaxSeg; ++g)
-      if (sl - sl_a == g) { g_pos0 = seg_pos0[g]; g_pa = seg_pa[g]; }
-    col_byte[b] = (unsigned)(g_pos0 + (op - g_pa) * p.sh * p.Wp + oq * p.sw) * 128u;
-  }
+      for (int g = 1; g < kConvMaxSeg; ++g)
+        if (sl - q.sl_a == g) { g_pos0 = q.seg_pos0[g]; g_pa = q.seg_pa[g]; }
+      col_byte[b] = (unsigned)(g_pos0 + (op - g_pa) * p.sh * p.Wp + oq * p.sw) * 128u;
+    }
+  };
+  column_bytes(geo);
   // LDS byte offsets: weights by (parity of the 32-row tile, sub-step), the lane's chunk per sub-step
   unsigned a_off[2][4], kh[4];
 #pragma unroll
@@ -479,6 +508,50 @@ __global__ __launch_bounds__(64 * NW, OCC) void amos_conv_fprop(const ConvFpropP
       for (int a = 0; a < TI; ++a)
 #pragma unroll
         for (int b = 0; b < TJ; ++b) acc[a][b] = MM::run(af[slot][ks][a], bf[slot][ks][b], acc[a][b]);
+  };
+
+  // ---- epilogue: Y[(n*K + i)*ODPQ + (od*OPQ + opq)] ---------------------------------------------
+  auto store_tile = [&](const TileGeo& q) {
+  out_t* const out = (out_t*)p.y;
+  const int ODPQ = p.OD * OPQ;
+  const bool full = q.bi0 + BI <= p.K && q.bj0 + BJ <= p.J && !p.atomic_out;
+#pragma unroll
+  for (int b = 0; b < TJ; ++b) {
+    const int j = q.bj0 + (wj * TJ + b) * 32 + frag_row;
+    const int jc = j < p.J ? j : p.J - 1;
+    const int n = fast_div(jc, p.fd_odpq);
+    const int64_t coff = (int64_t)n * p.K * ODPQ + (jc - n * ODPQ);
+#pragma unroll
+    for (int a = 0; a < TI; ++a) {
+      const int i0 = q.bi0 + (wi * TI + a) * 32 + 4 * frag_half;
+      out_t* const dst0 = out + (int64_t)i0 * ODPQ + coff;
+      if (p.epi.dt != EPI_NONE && blockIdx.y == 0) {   // one K split adds D; all loads first
+        out_t dv[16];
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int i = i0 + 8 * (r >> 2) + (r & 3);
+          dv[r] = epi_value<out_t>(p.epi, (int64_t)(i < p.K ? i : p.K - 1) * ODPQ + coff);
+        }
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[a][b][r] += dv[r];
+      }
+      if (full) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) dst0[(int64_t)(8 * (r >> 2) + (r & 3)) * ODPQ] = acc[a][b][r];
+      } else if (j < p.J) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int di = 8 * (r >> 2) + (r & 3);
+          if (i0 + di < p.K) {
+            if (p.atomic_out)
+              atomicAdd(dst0 + (int64_t)di * ODPQ, acc[a][b][r]);
+            else
+              dst0[(int64_t)di * ODPQ] = acc[a][b][r];
+          }
+        }
+      }
+    }
+  }
   };
 
   int2 pt[PL > 0 ? PL : 1];   // table entries of the patch copies of the coming step
@@ -561,7 +634,7 @@ __global__ __launch_bounds__(64 * NW, OCC) void amos_conv_fprop(const ConvFpropP
                    live ? (unsigned)p.D : 0u);
       }
     }
-    issue_weights((unsigned)e[0], istage);   // tile step+NSW into the stage just freed
+    issue_weights(w_off, (unsigned)e[0], istage);   // tile step+NSW into the stage just freed
     istage = rstage;
     // the next step's table entry, last: it has until the top of the next step to arrive
     __builtin_amdgcn_sched_barrier(0);
@@ -579,7 +652,7 @@ __global__ __launch_bounds__(64 * NW, OCC) void amos_conv_fprop(const ConvFpropP
     // ---- nine unrolled taps per macro step ------------------------------------------------------
     // patch read addresses per tap (buffer 0): position shift and swizzle term folded in
     unsigned baddr[9][TJ][4];
-    {
+    auto tap_addresses = [&]() {
       int tr = 0, ts = 0;
 #pragma unroll
       for (int tap = 0; tap < 9; ++tap) {
@@ -593,8 +666,17 @@ __global__ __launch_bounds__(64 * NW, OCC) void amos_conv_fprop(const ConvFpropP
         }
         if (++ts == p.S) { ts = 0; ++tr; }
       }
-    }
+    };
+    tap_addresses();
     const int n_macro = m_end - m_begin;
+    // blocks that walk several tiles: the weight rows of the next macro step's tile, whether
+    // this macro step is a tile's last with another tile to follow (its last tap then leaves
+    // the next operands to the tile switch), whether it is the first after a switch (the
+    // stores of the finished tile are then still in flight)
+    unsigned w_off_nx[WCH];
+#pragma unroll
+    for (int u = 0; u < WCH; ++u) w_off_nx[u] = w_off[u];
+    bool hand_over = false, after_switch = false;
     auto wk_of_macro = [&](int m) {
       if (m > p.macro_steps - 1) m = p.macro_steps - 1;
       const int tt = fast_div(m, p.fd_cc), cc = m - tt * p.c_chunks;
@@ -610,7 +692,16 @@ __global__ __launch_bounds__(64 * NW, OCC) void amos_conv_fprop(const ConvFpropP
       }
       // the copies of the previous step may still be in flight: WCH of the weight tile, PL of the
       // patch if that step was one of the taps 0..6 that fetch it
-      asm volatile("s_waitcnt vmcnt(%0)" ::"n"(WCH + ((TAP >= 1 && TAP <= 7) ? PL : 0)) : "memory");
+      constexpr int IN_FLIGHT = WCH + ((TAP >= 1 && TAP <= 7) ? PL : 0);
+      if constexpr (PERSIST && TAP <= 1) {
+        // memory instructions complete in issue order: the 16 stores per 32x32 tile of the
+        // finished tile sit between the copies waited for here and the younger ones
+        constexpr int WITH_STORES = IN_FLIGHT + 16 * TI * TJ > 63 ? 63 : IN_FLIGHT + 16 * TI * TJ;
+        if (after_switch) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(WITH_STORES) : "memory");
+        else asm volatile("s_waitcnt vmcnt(%0)" ::"n"(IN_FLIGHT) : "memory");
+      } else {
+        asm volatile("s_waitcnt vmcnt(%0)" ::"n"(IN_FLIGHT) : "memory");
+      }
       if (PL == 2)
         asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" : "+v"(pt[0]), "+v"(pt[PL > 1 ? 1 : 0])::"memory");
       else if (PL == 1)
@@ -620,14 +711,16 @@ __global__ __launch_bounds__(64 * NW, OCC) void amos_conv_fprop(const ConvFpropP
       // operands of the next K step
       // (PL = 0: a block runs one macro step and has one patch buffer; its last read is unused)
       constexpr int TN = TAP == 8 ? 0 : TAP + 1, BN = (TAP == 8 && PL > 0) ? BUF ^ 1 : BUF;
+      if (!(PERSIST && TAP == 8) || !hand_over) {
 #pragma unroll
-      for (int ks = 0; ks < 4; ++ks) {
+        for (int ks = 0; ks < 4; ++ks) {
 #pragma unroll
-        for (int a = 0; a < TI; ++a)
-          af[SLOT ^ 1][ks][a] = *(const v4i*)AMOS_LDS_PTR_FROM(a_off[a & 1][ks] + (unsigned)((TN % 3) * WSTAGE + (a >> 1) * (64 * 128)));
+          for (int a = 0; a < TI; ++a)
+            af[SLOT ^ 1][ks][a] = *(const v4i*)AMOS_LDS_PTR_FROM(a_off[a & 1][ks] + (unsigned)((TN % 3) * WSTAGE + (a >> 1) * (64 * 128)));
 #pragma unroll
-        for (int b = 0; b < TJ; ++b)
-          bf[SLOT ^ 1][ks][b] = *(const v4i*)AMOS_LDS_PTR_FROM(baddr[TN][b][ks] + (unsigned)BN * conv_w9_xbuf(BI));
+          for (int b = 0; b < TJ; ++b)
+            bf[SLOT ^ 1][ks][b] = *(const v4i*)AMOS_LDS_PTR_FROM(baddr[TN][b][ks] + (unsigned)BN * conv_w9_xbuf(BI));
+        }
       }
       mma_step(SLOT);
       // patch of the next macro step, on taps 0..6, before this step's weight tile
@@ -642,16 +735,10 @@ __global__ __launch_bounds__(64 * NW, OCC) void amos_conv_fprop(const ConvFpropP
       }
       // weight tile of the step three ahead, into the stage the previous step read
       constexpr int NT = TAP + 3;
-      issue_weights(NT < 9 ? wk_cur + (unsigned)NT * pos_bytes : wk_nxt + (unsigned)(NT - 9) * pos_bytes,
-                    (unsigned)((TAP % 3) * WSTAGE));
+      if constexpr (NT < 9) issue_weights(w_off, wk_cur + (unsigned)NT * pos_bytes, (unsigned)((TAP % 3) * WSTAGE));
+      else issue_weights(w_off_nx, wk_nxt + (unsigned)(NT - 9) * pos_bytes, (unsigned)((TAP % 3) * WSTAGE));
     };
-    auto macro9 = [&](auto buf_c, int mi) {
-      const int m = m_begin + mi;
-      const unsigned wk_cur = wk_of_macro(m), wk_nxt = wk_of_macro(m + 1);
-      const int n_live = m + 1 < m_end ? n_pl : 0;
-      const int tt1 = fast_div(m + 1, p.fd_cc), cc1 = (m + 1) - tt1 * p.c_chunks;
-      const unsigned po = 256u + (unsigned)(tt1 * p.dd * HW) * pos_bytes + (unsigned)cc1 * 128u;
-      const int pdb = tt1 * p.dd - 32768;
+    auto nine_taps = [&](auto buf_c, unsigned wk_cur, unsigned wk_nxt, int n_live, unsigned po, int pdb) {
       step9(IntC<0>{}, buf_c, wk_cur, wk_nxt, n_live, po, pdb);
       step9(IntC<1>{}, buf_c, wk_cur, wk_nxt, n_live, po, pdb);
       step9(IntC<2>{}, buf_c, wk_cur, wk_nxt, n_live, po, pdb);
@@ -662,53 +749,112 @@ __global__ __launch_bounds__(64 * NW, OCC) void amos_conv_fprop(const ConvFpropP
       step9(IntC<7>{}, buf_c, wk_cur, wk_nxt, n_live, po, pdb);
       step9(IntC<8>{}, buf_c, wk_cur, wk_nxt, n_live, po, pdb);
     };
-    for (int mi = 0; mi < n_macro; mi += 2) {
-      macro9(IntC<0>{}, mi);
-      if (mi + 1 < n_macro) macro9(IntC<1>{}, mi + 1);
+    auto macro9 = [&](auto buf_c, int mi) {
+      const int m = m_begin + mi;
+      const unsigned wk_cur = wk_of_macro(m), wk_nxt = wk_of_macro(m + 1);
+      const int n_live = m + 1 < m_end ? n_pl : 0;
+      const int tt1 = fast_div(m + 1, p.fd_cc), cc1 = (m + 1) - tt1 * p.c_chunks;
+      const unsigned po = 256u + (unsigned)(tt1 * p.dd * HW) * pos_bytes + (unsigned)cc1 * 128u;
+      const int pdb = tt1 * p.dd - 32768;
+      nine_taps(buf_c, wk_cur, wk_nxt, n_live, po, pdb);
+    };
+    if constexpr (!PERSIST) {
+      for (int mi = 0; mi < n_macro; mi += 2) {
+        macro9(IntC<0>{}, mi);
+        if (mi + 1 < n_macro) macro9(IntC<1>{}, mi + 1);
+      }
+    } else {
+      // ---- a block's tiles, one after the other ---------------------------------------------------
+      // The macro steps of all its tiles form one sequence: the last macro step of a tile fetches
+      // the first patch and the first weight tiles of the next tile, so that only the output
+      // stores and the new tile's addresses stand between two tiles.  The position table of the
+      // next tile is written (into the other of two tables) when a tile starts; the step barriers
+      // of the macro steps before its first use publish it.  The host launches such blocks
+      // without split-K and with at least two macro steps per tile.
+      const int total_tiles = p.tiles_i * p.tiles_j;
+      int tile = (int)blockIdx.x;
+      int buf = 0;            // patch buffer of the current macro step
+      int tab_cur = p.tab_off, tab_oth = p.tab1_off;
+      for (;;) {
+        const int next_tile = tile + (int)gridDim.x;
+        const bool has_next = next_tile < total_tiles;
+        TileGeo geo_n = geo;
+        int n_pl_n = n_pl;
+        if (has_next) {
+          const int tj = (int)((unsigned)next_tile / (unsigned)p.tiles_i);
+          geo_n = geo_of(next_tile - tj * p.tiles_i, tj);
+          write_table(geo_n, tab_oth);
+          n_pl_n = copies_of(geo_n.npos);
+        }
+        for (int m = 0; m < n_macro; ++m) {
+          const bool last = m == n_macro - 1;
+          hand_over = last && has_next;
+          unsigned wk_nxt, po;
+          int pdb, n_live;
+          if (!last) {
+            const int tt1 = fast_div(m + 1, p.fd_cc), cc1 = (m + 1) - tt1 * p.c_chunks;
+            wk_nxt = wk_of_macro(m + 1);
+            po = 256u + (unsigned)(tt1 * p.dd * HW) * pos_bytes + (unsigned)cc1 * 128u;
+            pdb = tt1 * p.dd - 32768;
+            n_live = n_pl;
+            n_pl_rd = n_pl;
+            tab_lane = (unsigned)tab_cur + (unsigned)(lane >> 3) * 8;
+          } else {
+            // macro step 0 of the next tile (of this one again, unused, when there is none)
+            wk_nxt = 0;
+            po = 256u;
+            pdb = -32768;
+            n_live = has_next ? n_pl_n : 0;
+            n_pl_rd = n_pl_n;
+            tab_lane = (unsigned)(has_next ? tab_oth : tab_cur) + (unsigned)(lane >> 3) * 8;
+            if (has_next) weight_rows(geo_n.bi0, w_off_nx);
+          }
+          if (buf == 0) nine_taps(IntC<0>{}, wk_of_macro(m), wk_nxt, n_live, po, pdb);
+          else nine_taps(IntC<1>{}, wk_of_macro(m), wk_nxt, n_live, po, pdb);
+          buf ^= 1;
+          after_switch = false;
+        }
+        store_tile(geo);
+        if (!has_next) break;
+        // a ragged tile issues fewer stores than the waits after the switch allow for
+        const bool counted = geo.bi0 + BI <= p.K && geo.bj0 + BJ <= p.J;
+        if (!counted) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        after_switch = counted;
+        geo = geo_n;
+        n_pl = n_pl_n;
+        tile = next_tile;
+        { const int x = tab_cur; tab_cur = tab_oth; tab_oth = x; }
+#pragma unroll
+        for (int u = 0; u < WCH; ++u) w_off[u] = w_off_nx[u];
+        column_bytes(geo);
+        tap_addresses();
+#pragma unroll
+        for (int a = 0; a < TI; ++a)
+#pragma unroll
+          for (int b = 0; b < TJ; ++b)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[a][b][r] = 0;
+        // operands of the new tile's first step: tap 0 in the buffer its patch was fetched to,
+        // into the fragment slot that step computes from (the parity of tap + buffer)
+        auto first_operands = [&](auto buf_c) {
+          constexpr int B = decltype(buf_c)::value;
+#pragma unroll
+          for (int ks = 0; ks < 4; ++ks) {
+#pragma unroll
+            for (int a = 0; a < TI; ++a)
+              af[B][ks][a] = *(const v4i*)AMOS_LDS_PTR_FROM(a_off[a & 1][ks] + (unsigned)((a >> 1) * (64 * 128)));
+#pragma unroll
+            for (int b = 0; b < TJ; ++b)
+              bf[B][ks][b] = *(const v4i*)AMOS_LDS_PTR_FROM(baddr[0][b][ks] + (unsigned)B * conv_w9_xbuf(BI));
+          }
+        };
+        if (buf == 0) first_operands(IntC<0>{});
+        else first_operands(IntC<1>{});
+      }
     }
   }
 
-  // ---- epilogue: Y[(n*K + i)*ODPQ + (od*OPQ + opq)] ---------------------------------------------
-  out_t* const out = (out_t*)p.y;
-  const int ODPQ = p.OD * OPQ;
-  const bool full = bi0 + BI <= p.K && bj0 + BJ <= p.J && !p.atomic_out;
-#pragma unroll
-  for (int b = 0; b < TJ; ++b) {
-    const int j = bj0 + (wj * TJ + b) * 32 + frag_row;
-    const int jc = j < p.J ? j : p.J - 1;
-    const int n = fast_div(jc, p.fd_odpq);
-    const int64_t coff = (int64_t)n * p.K * ODPQ + (jc - n * ODPQ);
-#pragma unroll
-    for (int a = 0; a < TI; ++a) {
-      const int i0 = bi0 + (wi * TI + a) * 32 + 4 * frag_half;
-      out_t* const dst0 = out + (int64_t)i0 * ODPQ + coff;
-      if (p.epi.dt != EPI_NONE && blockIdx.y == 0) {   // one K split adds D; all loads first
-        out_t dv[16];
-#pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          const int i = i0 + 8 * (r >> 2) + (r & 3);
-          dv[r] = epi_value<out_t>(p.epi, (int64_t)(i < p.K ? i : p.K - 1) * ODPQ + coff);
-        }
-#pragma unroll
-        for (int r = 0; r < 16; ++r) acc[a][b][r] += dv[r];
-      }
-      if (full) {
-#pragma unroll
-        for (int r = 0; r < 16; ++r) dst0[(int64_t)(8 * (r >> 2) + (r & 3)) * ODPQ] = acc[a][b][r];
-      } else if (j < p.J) {
-#pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          const int di = 8 * (r >> 2) + (r & 3);
-          if (i0 + di < p.K) {
-            if (p.atomic_out)
-              atomicAdd(dst0 + (int64_t)di * ODPQ, acc[a][b][r]);
-            else
-              dst0[(int64_t)di * ODPQ] = acc[a][b][r];
-          }
-        }
-      }
-    }
-  }
+  if constexpr (!PERSIST) store_tile(geo);
   // the re-fetched tiles of the last steps still target this block's LDS
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 }

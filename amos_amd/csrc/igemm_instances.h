@@ -99,7 +99,7 @@ ConvInstance* conv_instance() {
   static const char* dtn[] = {"f16", "bf16", "i8"};
   static std::string name = std::string("amos_conv_fprop<") + dtn[DT] + "," + std::to_string(64 * TI) +
                             "x" + std::to_string(64 * TJ) + "," + std::to_string(NW) + "w,pl" +
-                            std::to_string(PL) + (OCC == 2 ? ",occ2" : "") + (W9 ? ",9taps>" : ">");
+                            std::to_string(PL) + (OCC == 2 ? ",occ2" : "") + (W9 == 2 ? ",9taps,walk>" : W9 ? ",9taps>" : ">");
   inst.fn = amos_conv_fprop<DT, TI, TJ, NW, PL, OCC, W9>;
   inst.name = name.c_str();
   inst.threads = 64 * NW;
@@ -133,22 +133,31 @@ ConvInstance* pick_conv_tile8(int ti, int tj) {
   if (ti == 128 && tj == 256) return conv_instance<DT, 2, 4, 8, PL, 1>();
   return nullptr;
 }
-template <int DT, int PL>
+template <int DT, int PL, int W9>
 ConvInstance* pick_conv_tile9(int ti, int tj) {
-  if (ti == 128 && tj == 64) return conv_instance<DT, 2, 1, 8, PL, 1, 1>();
-  if (ti == 64 && tj == 128) return conv_instance<DT, 1, 2, 8, PL, 1, 1>();
-  if (ti == 128 && tj == 128) return conv_instance<DT, 2, 2, 8, PL, 1, 1>();
+  if (ti == 128 && tj == 64) return conv_instance<DT, 2, 1, 8, PL, 1, W9>();
+  if (ti == 64 && tj == 128) return conv_instance<DT, 1, 2, 8, PL, 1, W9>();
+  if constexpr (W9 != 2) {   // (walking tiles, a 128x128 block would not fit the register file)
+    if (ti == 128 && tj == 128) return conv_instance<DT, 2, 2, 8, PL, 1, W9>();
+  }
   return nullptr;
 }
 // waves = 4 or 8; pls = patch copies per wave per K step the plan asks for: 0, 2 or 4 with 4
-// waves, 0, 1 or 2 with 8; w9 = the instance with nine unrolled taps
+// waves, 0, 1 or 2 with 8; w9 = 1: the instance with nine unrolled taps, 2: the one whose
+// blocks walk several tiles
 template <int DT>
 ConvInstance* pick_conv_tile(int ti, int tj, int waves, int pls, int occ, int w9) {
+  if (w9 == 2) {
+    if (waves != 8 || occ != 1) return nullptr;
+    if (pls == 1) return pick_conv_tile9<DT, 1, 2>(ti, tj);
+    if (pls == 2) return pick_conv_tile9<DT, 2, 2>(ti, tj);
+    return nullptr;
+  }
   if (w9) {
     if (waves != 8 || occ != 1) return nullptr;
-    if (pls == 0) return pick_conv_tile9<DT, 0>(ti, tj);
-    if (pls == 1) return pick_conv_tile9<DT, 1>(ti, tj);
-    if (pls == 2) return pick_conv_tile9<DT, 2>(ti, tj);
+    if (pls == 0) return pick_conv_tile9<DT, 0, 1>(ti, tj);
+    if (pls == 1) return pick_conv_tile9<DT, 1, 1>(ti, tj);
+    if (pls == 2) return pick_conv_tile9<DT, 2, 1>(ti, tj);
     return nullptr;
   }
   if (waves == 8) {

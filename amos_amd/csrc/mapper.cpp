@@ -137,12 +137,12 @@ int64_t conv_workspace_bytes(const amos_conv_desc_t& c, int op) {
 
 
 static ConvPatchPlan conv_patch_plan_waves(const amos_conv_desc_t& cin, int op, int BI, int BJ, int split_k,
-                                           int waves, bool allow_w9);
+                                           int waves, int allow_w9);
 
 // waves: 4, 8, or 0 = 8 where that applies and four waves would leave a CU with a single workgroup
 // (or where the unrolled 3x3 instance applies, which exists with 8 waves)
 ConvPatchPlan conv_patch_plan(const amos_conv_desc_t& c, int op, int BI, int BJ, int split_k, int waves,
-                              bool allow_w9) {
+                              int allow_w9) {
   if (waves == 4 || waves == 8) return conv_patch_plan_waves(c, op, BI, BJ, split_k, waves, allow_w9);
   ConvPatchPlan p8 = conv_patch_plan_waves(c, op, BI, BJ, split_k, 8, allow_w9);
   if (!p8.why && p8.w9) return p8;
@@ -152,8 +152,8 @@ ConvPatchPlan conv_patch_plan(const amos_conv_desc_t& c, int op, int BI, int BJ,
 }
 
 static ConvPatchPlan conv_patch_plan_waves(const amos_conv_desc_t& cin, int op, int BI, int BJ, int split_k,
-                                           int waves, bool allow_w9) {
-  ConvPatchPlan pp = {nullptr, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+                                           int waves, int allow_w9) {
+  ConvPatchPlan pp = {nullptr, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
   pp.waves = waves;
   amos_conv_desc_t c = cin;
   if (op == AMOS_OP_CONV2D) { c.D = 1; c.T = 1; c.stride_d = 1; c.pad_d = 0; c.dil_d = 1; }
@@ -239,6 +239,31 @@ static ConvPatchPlan conv_patch_plan_waves(const amos_conv_desc_t& cin, int op, 
       pp.max_pos = max_pos9;
       pp.occ = 1;
       pp.lds = 3 * wstage + patch9;
+      pp.tab_rel = pp.xbufs * max_pos9 * 128;
+      pp.dump_rel = pp.tab_rel + max_pos9 * 8;
+      pp.tab1_rel = pp.tab_rel;
+      // Blocks that walk several tiles (more tiles than CUs, no split-K, at least two macro steps
+      // per tile) need a second position table: tables and dump line go behind the used part of
+      // each patch buffer where they fit there, behind the second buffer otherwise
+      const int64_t tiles = ((c.K + BI - 1) / BI) * ((J + BJ - 1) / BJ);
+      if (allow_w9 >= 2 && !one_macro && split == 1 && tiles > Gfx950::kComputeUnits && !(BI == 128 && BJ == 128)) {
+        const int xbuf = BI <= 64 ? 64 * 1024 : 48 * 1024;
+        const int P = real_pos * 128, TB = real_pos * 8;
+        int tab, tab1, dump;
+        size_t total;
+        if (P + TB + 1024 <= xbuf) {
+          tab = P; dump = P + TB; tab1 = xbuf + P;
+          total = 3 * wstage + (size_t)xbuf + P + TB;
+        } else {
+          tab = 2 * xbuf; tab1 = tab + TB; dump = tab1 + TB;
+          total = 3 * wstage + (size_t)dump + 1024;
+        }
+        if (total <= budget) {
+          pp.w9 = 2;
+          pp.tab_rel = tab; pp.tab1_rel = tab1; pp.dump_rel = dump;
+          pp.lds = total;
+        }
+      }
       return pp;
     }
   }
@@ -323,11 +348,15 @@ static double estimate_seconds(const Problem& pb, int ti, int tj, int split, boo
   return std::max(t, t_hbm) + 0.1 * std::min(t, t_hbm);
 }
 
+int conv_unroll_level(int flags) {
+  return (flags & AMOS_FLAG_NO_UNROLLED_TAPS) ? 0 : (flags & AMOS_FLAG_NO_TILE_WALK) ? 1 : 2;
+}
+
 // Patch-staged convolution: blocks of one per CU; a K step costs its MFMA issue time plus a
 // per-step instruction overhead that does not shrink with the tile; split-K pays for atomic
 // accumulation into the output.  Returns <= 0 where the pipeline does not apply.
 static double conv_patch_estimate(const amos_conv_desc_t& c, int op, const Problem& pb, int ti, int tj,
-                                  int split, int waves = 0, bool allow_w9 = true) {
+                                  int split, int waves = 0, int allow_w9 = 2) {
   ConvPatchPlan pp = conv_patch_plan(c, op, ti, tj, split, waves, allow_w9);
   if (pp.why) return -1.0;
   const bool two_streams = pp.occ == 2 || pp.waves == 8;   // two waves per SIMD
@@ -345,7 +374,9 @@ static double conv_patch_estimate(const amos_conv_desc_t& c, int op, const Probl
   // measured (profiles/conv_fprop_kernel_trace.md): a 128x64 step takes ~700 cycles with the taps
   // unrolled, ~760 with two instruction streams per SIMD, ~850 with one; set-up 6000-8000 cycles
   const double overhead = pp.w9 ? 440.0 : two_streams ? 500.0 : 600.0;
-  const double cycles = rounds * (steps * (pp.occ * mfma_per_step + overhead) + (pp.w9 ? 8000.0 : 6000.0));
+  double cycles = rounds * (steps * (pp.occ * mfma_per_step + overhead) + (pp.w9 ? 8000.0 : 6000.0));
+  // blocks that walk their tiles set up once; a tile switch costs the stores and the new addresses
+  if (pp.w9 == 2) cycles = rounds * (steps * (mfma_per_step + overhead) + 1500.0) + 8000.0;
   const double relayout = ((double)pb.in_bytes * 2.0) / 2.5e12 + 3e-6;
   return cycles / 2.1e9 + relayout + (split > 1 ? (double)pb.out_bytes * split / 1.2e12 : 0.0);
 }
@@ -394,7 +425,7 @@ int amos_estimate_seconds(int op, const void* desc, const amos_kernel_config_t* 
   if ((op == AMOS_OP_CONV2D || op == AMOS_OP_CONV3D) && cfg->pipeline != AMOS_PIPE_STAGED) {
     const int waves = cfg->pipeline == AMOS_PIPE_PATCH ? 4 : cfg->pipeline == AMOS_PIPE_PATCH8 ? 8 : 0;
     double s = conv_patch_estimate(*(const amos_conv_desc_t*)desc, op, pb, cfg->tile_i, cfg->tile_j, split,
-                                   waves, !(cfg->reserved[0] & AMOS_FLAG_NO_UNROLLED_TAPS));
+                                   waves, conv_unroll_level(cfg->reserved[0]));
     if (s > 0) { *seconds = s; return 0; }
     if (waves) return set_error(AMOS_ERR_INFEASIBLE, "patch-staged convolution not applicable to this config");
   }

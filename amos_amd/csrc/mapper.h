@@ -47,13 +47,17 @@ struct ConvPatchPlan {
   int xbufs;         // patch buffers (1 when a block runs a single macro step)
   int occ;           // workgroups per CU the instance is built for (2 when LDS and registers allow)
   int waves;         // waves per workgroup: 4 or 8
-  int w9;            // the instance with the nine taps of a 3x3 window unrolled
+  int w9;            // 1: the instance with the nine taps of a 3x3 window unrolled; 2: that
+                     // instance with blocks that walk several tiles
   size_t lds;        // dynamic LDS bytes of the block
+  int tab_rel, tab1_rel, dump_rel;   // w9: position tables and dump line, bytes from the first patch buffer
 };
 int64_t conv_packed_bytes(const amos_conv_desc_t& c, int op);
 int64_t conv_relaid_bytes(const amos_conv_desc_t& c, int op);
 int64_t conv_workspace_bytes(const amos_conv_desc_t& c, int op);
+// allow_w9: 0 = table-driven instances only, 1 = unrolled taps, 2 = unrolled taps and tile walk
 ConvPatchPlan conv_patch_plan(const amos_conv_desc_t& c, int op, int BI, int BJ, int split_k, int waves,
-                              bool allow_w9 = true);
+                              int allow_w9 = 2);
+int conv_unroll_level(int config_flags);
 
 }  // namespace amos

@@ -136,6 +136,9 @@ typedef struct {
 /* conv: do not use the instances whose 3x3 window taps are unrolled (they are preferred where
  * they apply; the flag lets a sweep time the table-driven ones) */
 #define AMOS_FLAG_NO_UNROLLED_TAPS 1
+/* conv: one tile per workgroup also where the unrolled instance would let a workgroup walk
+ * several tiles (more tiles than compute units, no split-K) */
+#define AMOS_FLAG_NO_TILE_WALK 2
 
 /* how tiles travel from HBM to the MFMA operands */
 #define AMOS_PIPE_AUTO 0

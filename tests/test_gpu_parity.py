@@ -295,6 +295,54 @@ def test_conv_patch_pipeline(gpu, dtype, case):
                   "patch conv %s %s tile %s split %d pipeline %d flags %d" % (dtype, case, tile, split, pipe, flags))
 
 
+WALK_CASES = [
+    # more tiles than compute units, 3x3 windows, at least two macro steps per tile
+    ("float16", (16, 128, 1, 41, 41, 72, 1, 3, 3, (1, 1, 1), (0, 1, 1), (1, 1, 1))),    # ragged K-out and J
+    ("int8", (24, 256, 1, 40, 40, 64, 1, 3, 3, (1, 1, 1), (0, 1, 1), (1, 1, 1))),
+    ("float16", (4, 64, 9, 32, 32, 64, 3, 3, 3, (1, 1, 1), (1, 1, 1), (1, 1, 1))),      # three macro steps per tile
+    ("bfloat16", (5, 64, 10, 34, 30, 40, 3, 3, 3, (1, 1, 1), (0, 1, 1), (1, 1, 1))),
+]
+
+
+@pytest.mark.parametrize("dtype,case", WALK_CASES)
+def test_conv_tile_walk(gpu, dtype, case):
+    """workgroups that walk several tiles: against the oracle, and bit for bit against the same
+    kernel with one tile per workgroup (same accumulation order)"""
+    import torch
+    from amos_amd import _lib, ops
+    N, C, D, H, W, K, T, R, S, st, pd, dl = case
+    rng = np.random.default_rng(11)
+    x = make_operand(rng, (N, C, D, H, W), dtype, "normal")
+    w = make_operand(rng, (K, C, T, R, S), dtype, "normal")
+    ref = co.lib_conv3d(x, w, dtype, st, pd, dl, acc="float64")
+    dx, dw = to_device(x, dtype), to_device(w, dtype)
+    is2d = D == 1 and T == 1
+    xs5, ws5 = (N, C, D, H, W), (K, C, T, R, S)
+    op = _lib.AMOS_OP_CONV2D if is2d else _lib.AMOS_OP_CONV3D
+    desc = ops.conv_desc(xs5, ws5, getattr(torch, dtype), st, pd, dl)
+    d_add = torch.randn(ref.shape, device="cuda").to(torch.int32 if dtype == "int8" else torch.float32)
+    walked = 0
+    for tile in [(64, 128), (128, 64)]:
+        outs = {}
+        for flags in (0, _lib.AMOS_FLAG_NO_TILE_WALK):
+            cfg = dict(tile_i=tile[0], tile_j=tile[1], split_k=1, pipeline=_lib.AMOS_PIPE_PATCH8, flags=flags)
+            name = ops.kernel_name(op, desc, cfg)
+            assert name is not None and "9taps" in name and (("walk" in name) == (flags == 0)), name
+            for add in (None, d_add):
+                if is2d:
+                    got = ops.conv2d(dx[:, :, 0], dw[:, :, 0], st[1:], pd[1:], dl[1:], config=cfg,
+                                     add=None if add is None else add[:, :, 0])[:, :, None]
+                else:
+                    got = ops.conv3d(dx, dw, st, pd, dl, config=cfg, add=add)
+                outs[(flags, add is None)] = got
+        walked += 1
+        assert torch.equal(outs[(0, True)], outs[(_lib.AMOS_FLAG_NO_TILE_WALK, True)]), "tile %s" % (tile,)
+        assert torch.equal(outs[(0, False)], outs[(_lib.AMOS_FLAG_NO_TILE_WALK, False)]), "tile %s + D" % (tile,)
+        check(outs[(0, True)].cpu().numpy(), ref, dtype, "walk %s %s tile %s" % (dtype, case, tile))
+        check((outs[(0, False)] - d_add).cpu().numpy(), ref, dtype, "walk + D %s %s tile %s" % (dtype, case, tile))
+    assert walked == 2
+
+
 def test_conv_patch_is_the_default_when_applicable(gpu):
     import torch
     from amos_amd import _lib, ops
