@@ -44,7 +44,7 @@ class ConvDesc(ctypes.Structure):
                 ("stride_d", _i32), ("stride_h", _i32), ("stride_w", _i32),
                 ("pad_d", _i32), ("pad_h", _i32), ("pad_w", _i32),
                 ("dil_d", _i32), ("dil_h", _i32), ("dil_w", _i32),
-                ("in_dtype", _i32), ("out_dtype", _i32), ("groups", _i32), ("reserved", _i32)]
+                ("in_dtype", _i32), ("out_dtype", _i32), ("groups", _i32), ("layout", _i32)]
 
 
 class KernelConfig(ctypes.Structure):
@@ -53,6 +53,8 @@ class KernelConfig(ctypes.Structure):
 
 
 AMOS_EPI_NONE, AMOS_EPI_ADD = 0, 1
+AMOS_LAYOUT_NCHW, AMOS_LAYOUT_NHWC, AMOS_LAYOUT_HWNC = 0, 1, 2
+LAYOUT_CODE = {"nchw": 0, "ncdhw": 0, "nhwc": 1, "ndhwc": 1, "hwnc": 2, "dhwnc": 2}
 AMOS_FLAG_NO_UNROLLED_TAPS, AMOS_FLAG_NO_TILE_WALK = 1, 2
 
 

@@ -260,11 +260,14 @@ def _lower_strided_gemm(main_op, l0, l1):
     return LoweredOp("bgemm", _lib.AMOS_OP_BGEMM, bd, [ra[0], rb[0]], main_op.output(0), attrs)
 
 
-def _pad_stage(tensor):
-    """tensor made by the padding compute -> (source placeholder, pads per spatial dim)"""
+def _pad_stage(tensor, spatial_dims=None):
+    """tensor made by the padding compute -> (source placeholder, pads per spatial dim);
+    spatial_dims: which dimensions may be padded (default: all but the first two)"""
     op = tensor.op
+    if spatial_dims is None:
+        spatial_dims = list(range(2, len(tensor.shape)))
     if isinstance(op, te.PlaceholderOp):
-        return tensor, [0] * (len(tensor.shape) - 2)
+        return tensor, [0] * len(spatial_dims)
     if not isinstance(op, te.ComputeOp) or op.reduce_axis:
         raise NoKernelError("activation operand is neither a placeholder nor a padding stage")
     body = op.body[0]
@@ -278,20 +281,32 @@ def _pad_stage(tensor):
     if not isinstance(src.op, te.PlaceholderOp):
         raise NoKernelError("padding stage does not read a placeholder")
     variables = [iv.var for iv in op.axis]
-    pads = []
+    pads = {}
     for d, idx in enumerate(load.indices):
         form = te.affine_form(idx, variables)
         if form is None or len(form[0]) != 1 or list(form[0].items())[0] != (variables[d], 1):
             raise NoKernelError("padding stage permutes or scales indices")
         pad = -form[1]
-        if d < 2:
+        if d not in spatial_dims:
             if pad != 0:
                 raise NoKernelError("padding on the batch or channel dimension")
         else:
             if pad < 0 or int(op.output(0).shape[d]) != int(src.shape[d]) + 2 * pad:
                 raise NoKernelError("padding stage is not symmetric zero padding")
-            pads.append(pad)
-    return src, pads
+            pads[d] = pad
+    return src, [pads[d] for d in spatial_dims]
+
+
+# where batch / channel / spatial dimensions sit in the three tensors of a convolution
+# (reference: the three layouts of benchmark/amos/mapping_conv2d_tensorcore.py:7-104)
+def _conv_templates(nsp):
+    sp = list(range(nsp))
+    return [
+        # name, x: (n, c, spatial), w: (k, c, window), out: (n, k, spatial)
+        ("nchw", (0, 1, [2 + d for d in sp]), (0, 1, [2 + d for d in sp]), (0, 1, [2 + d for d in sp])),
+        ("nhwc", (0, nsp + 1, [1 + d for d in sp]), (nsp + 1, nsp, sp), (0, nsp + 1, [1 + d for d in sp])),
+        ("hwnc", (nsp, nsp + 1, sp), (nsp + 1, nsp, sp), (nsp, nsp + 1, sp)),
+    ]
 
 
 def _lower_conv(main_op, l0, l1, iters, forms0, forms1):
@@ -299,20 +314,23 @@ def _lower_conv(main_op, l0, l1, iters, forms0, forms1):
     nsp = len(spatial) - 2                     # 1, 2 or 3 spatial output dims
     if nsp not in (1, 2, 3) or len(reduce_) != nsp + 1:
         return None
-    n_iv, k_iv, out_sp = spatial[0], spatial[1], spatial[2:]
-    rc, red_sp = reduce_[0], reduce_[1:]
 
-    def try_roles(lx, fx, lw, fw):
+    def try_roles(template, lx, fx, lw, fw):
+        _, (xn, xc, xsp), (wk, wc, wsp), (on, ok, osp) = template
         if len(fx) != nsp + 2 or len(fw) != nsp + 2:
             return None
+        n_iv, k_iv, out_sp = spatial[on], spatial[ok], [spatial[d] for d in osp]
         wv = [_single_var(f, iters) for f in fw]
-        if wv[0] is not k_iv or wv[1] is not rc or any(a is not b for a, b in zip(wv[2:], red_sp)):
+        rc, red_sp = wv[wc], [wv[d] for d in wsp]
+        if wv[wk] is not k_iv or rc is None or any(r is None for r in red_sp):
             return None
-        if _single_var(fx[0], iters) is not n_iv or _single_var(fx[1], iters) is not rc:
+        if set(id(r) for r in [rc] + red_sp) != set(id(r) for r in reduce_):
+            return None
+        if _single_var(fx[xn], iters) is not n_iv or _single_var(fx[xc], iters) is not rc:
             return None
         strides, dils = [], []
         for d in range(nsp):
-            f = fx[2 + d]
+            f = fx[xsp[d]]
             if f is None:
                 return None
             coef, const = f
@@ -324,20 +342,28 @@ def _lower_conv(main_op, l0, l1, iters, forms0, forms1):
             dils.append(int(coef.get(red_sp[d].var, 1)))
             if strides[-1] < 1 or dils[-1] < 1:
                 return None
-        return strides, dils
+        return strides, dils, rc, red_sp, out_sp
 
-    roles = try_roles(l0, forms0, l1, forms1)
-    lx, lw = l0, l1
-    if roles is None:
-        roles = try_roles(l1, forms1, l0, forms0)
-        lx, lw = l1, l0
-    if roles is None:
+    found = None
+    for template in _conv_templates(nsp):
+        for lx, fx, lw, fw in ((l0, forms0, l1, forms1), (l1, forms1, l0, forms0)):
+            roles = try_roles(template, lx, fx, lw, fw)
+            if roles is not None:
+                found = (template, lx, lw, roles)
+                break
+        if found:
+            break
+    if found is None:
         return None
-    strides, dils = roles
-    src, pads = _pad_stage(lx.tensor)
+    template, lx, lw, (strides, dils, rc, red_sp, out_sp) = found
+    layout, (xn, xc, xsp), (wk, wc, wsp), _ = template
+    src, pads = _pad_stage(lx.tensor, xsp)
     if not isinstance(lw.tensor.op, te.PlaceholderOp):
         raise NoKernelError("convolution weights must be a placeholder")
-    xs, ws = [int(s) for s in src.shape], [int(s) for s in lw.tensor.shape]
+    xs_mem, ws_mem = [int(s) for s in src.shape], [int(s) for s in lw.tensor.shape]
+    # logical extents: N, C, spatial...; K, C, window...
+    xs = [xs_mem[xn], xs_mem[xc]] + [xs_mem[d] for d in xsp]
+    ws = [ws_mem[wk], ws_mem[wc]] + [ws_mem[d] for d in wsp]
     for d in range(nsp):
         if int(red_sp[d].dom.extent) != ws[2 + d]:
             raise NoKernelError("reduce extent %d differs from the kernel window %d"
@@ -364,12 +390,10 @@ def _lower_conv(main_op, l0, l1, iters, forms0, forms1):
     c.pad_d, c.pad_h, c.pad_w = pd
     c.dil_d, c.dil_h, c.dil_w = dl
     c.in_dtype, c.out_dtype = ind, outd
-    out_shape = [int(s) for s in main_op.output(0).shape]
-    J = out_shape[0]
-    for e in out_shape[2:]:
-        J *= e
+    c.layout = _lib.LAYOUT_CODE[layout]
+    J = _numel(main_op.output(0).shape) // ws[0]
     attrs = dict(x_shape=xs, w_shape=ws, stride=strides, pad=pads, dil=dils, dtype=lx.dtype, J=J,
-                 K_out=ws[0], K_red=ws[1] * (ws5[2] * ws5[3] * ws5[4]))
+                 K_out=ws[0], K_red=ws[1] * (ws5[2] * ws5[3] * ws5[4]), layout=layout)
     kind, code = ("conv2d", _lib.AMOS_OP_CONV2D) if nsp <= 2 else ("conv3d", _lib.AMOS_OP_CONV3D)
     return LoweredOp(kind, code, c, [src, lw.tensor], main_op.output(0), attrs)
 

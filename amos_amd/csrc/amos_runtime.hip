@@ -171,6 +171,7 @@ static int plan_gemm(Plan& pl, int op, const void* desc_any, const amos_gemm_des
   p.out = (char*)C;
   p.out_si = d->ldc;
   p.out_sjo = 0;
+  p.out_sj = 1;
   p.out_jmod = 0x7fffffff;
   p.out_batch = sc;
   pl.batch = batch;
@@ -231,6 +232,11 @@ static int plan_conv(Plan& pl, int op, const amos_conv_desc_t* d, const amos_ker
   if (c.C % G || c.K % G)
     return set_error(AMOS_ERR_BAD_ARG, "groups (%lld) must divide C (%lld) and K (%lld)", (long long)G,
                      (long long)c.C, (long long)c.K);
+  const int layout = c.layout;
+  if (layout < AMOS_LAYOUT_NCHW || layout > AMOS_LAYOUT_HWNC)
+    return set_error(AMOS_ERR_BAD_ARG, "unknown tensor layout %d", layout);
+  if (layout != AMOS_LAYOUT_NCHW && G > 1)
+    return set_error(AMOS_ERR_UNSUPPORTED, "grouped convolution exists for the NCHW layout only");
   const int64_t Cg = c.C / G, Kg = c.K / G;
   int OD = conv_out_extent(c.D, c.pad_d, c.dil_d, c.T, c.stride_d);
   int OP = conv_out_extent(c.H, c.pad_h, c.dil_h, c.R, c.stride_h);
@@ -240,7 +246,8 @@ static int plan_conv(Plan& pl, int op, const amos_conv_desc_t* d, const amos_ker
   int64_t J = c.N * OD * (int64_t)OP * OQ;
   int64_t Kred = Cg * c.T * c.R * c.S;
   int64_t per_image = c.C * c.D * c.H * c.W;
-  if (!fits_int(J) || !fits_int(Kred) || !fits_int(per_image) || !fits_int(c.K))
+  if (!fits_int(J) || !fits_int(Kred) || !fits_int(per_image) || !fits_int(c.K) ||
+      (layout == AMOS_LAYOUT_HWNC && !fits_int(per_image * c.N)))
     return set_error(AMOS_ERR_UNSUPPORTED, "conv extents above 2^31");
   if ((c.T - 1) * c.dil_d >= 1024 || (c.R - 1) * c.dil_h >= 1024 || (c.S - 1) * c.dil_w >= 1024)
     return set_error(AMOS_ERR_UNSUPPORTED, "dilated kernel extent above 1023");
@@ -260,7 +267,24 @@ static int plan_conv(Plan& pl, int op, const amos_conv_desc_t* d, const amos_ker
   p.col_base = (const char*)X;
   pl.cl = LD_CONV;
   ConvGeom& g = p.g;
-  g.C = (int)Cg; g.Cimg = (int)c.C; g.D = (int)c.D; g.H = (int)c.H; g.W = (int)c.W;
+  g.C = (int)Cg; g.D = (int)c.D; g.H = (int)c.H; g.W = (int)c.W;
+  const int64_t dhw = c.D * c.H * c.W;
+  if (layout == AMOS_LAYOUT_NCHW) {
+    g.x_sn = c.C * dhw; g.x_sc = (int)dhw; g.x_sd = (int)(c.H * c.W); g.x_sh = (int)c.W; g.x_sw = 1;
+    g.k_order = 0;
+  } else {
+    // channels innermost; weights [T][R][S][C][K]: the reduction runs tap-major, and a weight
+    // row (one output channel) has its K index strided by the number of output channels
+    g.x_sc = 1; g.k_order = 1;
+    if (layout == AMOS_LAYOUT_NHWC) {
+      g.x_sn = dhw * c.C; g.x_sd = (int)(c.H * c.W * c.C); g.x_sh = (int)(c.W * c.C); g.x_sw = (int)c.C;
+    } else {
+      g.x_sn = c.C; g.x_sw = (int)(c.N * c.C); g.x_sh = (int)(c.W * c.N * c.C); g.x_sd = (int)(c.H * c.W * c.N * c.C);
+    }
+    p.row_s_row = 1;
+    p.row_s_k = c.K;
+    pl.rl = LD_STRIDED;
+  }
   g.T = (int)c.T; g.R = (int)c.R; g.S = (int)c.S;
   g.sd = c.stride_d; g.sh = c.stride_h; g.sw = c.stride_w;
   g.pd = c.pad_d; g.ph = c.pad_h; g.pw = c.pad_w;
@@ -271,7 +295,10 @@ static int plan_conv(Plan& pl, int op, const amos_conv_desc_t* d, const amos_ker
   p.out = (char*)Y;
   p.out_si = odpq;
   p.out_sjo = c.K * odpq;
+  p.out_sj = 1;
   p.out_jmod = (int)odpq;
+  if (layout == AMOS_LAYOUT_NHWC) { p.out_si = 1; p.out_sjo = odpq * c.K; p.out_sj = c.K; }
+  if (layout == AMOS_LAYOUT_HWNC) { p.out_si = 1; p.out_sjo = c.K; p.out_sj = c.N * c.K; }
   p.out_batch = Kg * odpq;                        // ... its Kg channels of every output image
   pl.batch = G;
   pl.fill_rows = 1;
@@ -280,6 +307,7 @@ static int plan_conv(Plan& pl, int op, const amos_conv_desc_t* d, const amos_ker
   pl.fill_once = 1;                               // the whole output in one fill, not per group
   rc = plan_finish(pl, op, d, cfg);
   if (rc) return rc;
+  p.out_vec4 = layout != AMOS_LAYOUT_NCHW && c.K % 4 == 0 && aligned16(Y) && !p.atomic_out;
 
   // ---- patch-staged pipeline: channels fill whole 128-byte K steps, the relaid operands fit
   // the workspace, the patch of a tile fits LDS next to a ring of weight tiles
@@ -296,6 +324,8 @@ static int plan_conv(Plan& pl, int op, const amos_conv_desc_t* d, const amos_ker
   const char* why = pp.why;
   if (!why && (!workspace || ws_bytes < (size_t)need_ws || ((uintptr_t)workspace & 255)))
     why = "workspace smaller than amos_workspace_bytes() or not 256-byte aligned";
+  if (!why && layout != AMOS_LAYOUT_NCHW && !aligned16(X))
+    why = "channel-innermost activations not 16-byte aligned";
   const int max_pos = pp.max_pos, nsw = pp.nsw, pls = pp.pls;
   pl.conv_occ = pp.occ;
   pl.conv_waves = pp.waves;
@@ -359,6 +389,10 @@ static int plan_conv(Plan& pl, int op, const amos_conv_desc_t* d, const amos_ker
   q.fd_slab = make_fast_div((uint32_t)(c.C * c.T * c.R * c.S));
   q.prep_w_blocks = (int)((welems + 1023) / 1024 < 2048 ? (welems + 1023) / 1024 : 2048);
   q.prep_x_blocks = (int)(c.N * c.D * (((int64_t)c.H * c.W + 63) / 64) * (c.C * es / 128));
+  if (layout != AMOS_LAYOUT_NCHW) q.prep_x_blocks = (int)((c.N * dhw * (c.C * es / 16) + 1023) / 1024);
+  q.layout = layout;
+  q.y_si = p.out_si; q.y_sn = p.out_sjo; q.y_ss = p.out_sj;
+  q.y_vec4 = layout != AMOS_LAYOUT_NCHW && c.K % 4 == 0 && aligned16(Y);
   q.prep_z_blocks = q.zero_words ? (int)((q.zero_words + 4095) / 4096 < 2048 ? (q.zero_words + 4095) / 4096 : 2048) : 0;
   return 0;
 }

@@ -94,6 +94,11 @@ struct ConvFpropParams {
   int prep_w_blocks, prep_x_blocks, prep_z_blocks;
   int64_t zero_words;
   EpiParams epi;     // fused tail: Y = acc + cast(D), D laid out like Y
+  // tensor layouts (AMOS_LAYOUT_*): 0 = NCDHW / KCTRS / NKDPQ, 1 = NDHWC / TRSCK / NDPQK,
+  // 2 = DHWNC / TRSCK / DPQNK.  Output element (i, j), j = n*ODPQ + s, at i*y_si + n*y_sn + s*y_ss.
+  int layout;
+  int64_t y_si, y_sn, y_ss;
+  int y_vec4;        // y_si == 1, K % 4 == 0, Y (and D) 16-byte aligned: four output channels per store
 };
 
 // ---- launch 1: relayout ---------------------------------------------------------------------
@@ -169,7 +174,7 @@ __global__ __launch_bounds__(256) void amos_conv_prepare(const ConvFpropParams p
         const int k = fast_div((int)oc, p.fd_slab);   // the host keeps the packed weights under 2^31 elements
         const int o = (int)(oc - (int64_t)k * slab);
         const int tap = fast_div(o, p.fd_c), c = o - tap * p.C;
-        v[u] = w[(int64_t)k * slab + c * TRS + tap];
+        v[u] = p.layout == 0 ? w[(int64_t)k * slab + c * TRS + tap] : w[((int64_t)tap * p.C + c) * p.K + k];
       }
 #pragma unroll
       for (int u = 0; u < 4; ++u)
@@ -182,6 +187,34 @@ __global__ __launch_bounds__(256) void amos_conv_prepare(const ConvFpropParams p
     return;
   }
   b -= p.prep_w_blocks;
+  if (b < p.prep_x_blocks && p.layout != 0) {
+    // channels are innermost already: 16-byte chunks, four per thread; DHWNC moves image n's
+    // positions from [s][n] to [n][s]
+    const int cpp = p.C * (int)sizeof(T) / 16;           // chunks per position
+    const int64_t dhw = (int64_t)p.D * p.H * p.W;
+    const int64_t total = (int64_t)p.N * dhw * cpp;
+    const uint4* x = (const uint4*)p.x;
+    uint4* xt = (uint4*)p.xt;
+    uint4 v[4];
+    int64_t of[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      of[u] = (int64_t)b * 1024 + t + 256 * u;
+      const int64_t oc = of[u] < total ? of[u] : total - 1;
+      int64_t src = oc;
+      if (p.layout == 2) {
+        const int64_t pos = oc / cpp;
+        const int ch = (int)(oc - pos * cpp);
+        const int64_t n = pos / dhw, s = pos - n * dhw;
+        src = (s * p.N + n) * cpp + ch;
+      }
+      v[u] = x[src];
+    }
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+      if (of[u] < total) xt[of[u]] = v[u];
+    return;
+  }
   if (b < p.prep_x_blocks) {
     // xt[slice][s][c] = x[n][c][d][s] through an LDS tile of 128 bytes of channels x 64
     // positions, moved 8 bytes per lane on both sides where the rows of x are 8-byte aligned
@@ -515,38 +548,48 @@ __global__ __launch_bounds__(64 * NW, OCC) void amos_conv_fprop(const ConvFpropP
   out_t* const out = (out_t*)p.y;
   const int ODPQ = p.OD * OPQ;
   const bool full = q.bi0 + BI <= p.K && q.bj0 + BJ <= p.J && !p.atomic_out;
+  const int64_t y_si = p.y_si;
 #pragma unroll
   for (int b = 0; b < TJ; ++b) {
     const int j = q.bj0 + (wj * TJ + b) * 32 + frag_row;
     const int jc = j < p.J ? j : p.J - 1;
     const int n = fast_div(jc, p.fd_odpq);
-    const int64_t coff = (int64_t)n * p.K * ODPQ + (jc - n * ODPQ);
+    const int64_t coff = (int64_t)n * p.y_sn + (int64_t)(jc - n * ODPQ) * p.y_ss;
 #pragma unroll
     for (int a = 0; a < TI; ++a) {
       const int i0 = q.bi0 + (wi * TI + a) * 32 + 4 * frag_half;
-      out_t* const dst0 = out + (int64_t)i0 * ODPQ + coff;
+      out_t* const dst0 = out + (int64_t)i0 * y_si + coff;
       if (p.epi.dt != EPI_NONE && blockIdx.y == 0) {   // one K split adds D; all loads first
         out_t dv[16];
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
           const int i = i0 + 8 * (r >> 2) + (r & 3);
-          dv[r] = epi_value<out_t>(p.epi, (int64_t)(i < p.K ? i : p.K - 1) * ODPQ + coff);
+          dv[r] = epi_value<out_t>(p.epi, (int64_t)(i < p.K ? i : p.K - 1) * y_si + coff);
         }
 #pragma unroll
         for (int r = 0; r < 16; ++r) acc[a][b][r] += dv[r];
       }
-      if (full) {
+      if (full && p.y_vec4) {
+        // channels innermost: a lane's four consecutive channels in one store, a position's 32
+        // channels of the tile 128 contiguous bytes
+        typedef out_t out4_t __attribute__((ext_vector_type(4)));
 #pragma unroll
-        for (int r = 0; r < 16; ++r) dst0[(int64_t)(8 * (r >> 2) + (r & 3)) * ODPQ] = acc[a][b][r];
+        for (int g4 = 0; g4 < 4; ++g4) {
+          const out4_t v = {acc[a][b][4 * g4], acc[a][b][4 * g4 + 1], acc[a][b][4 * g4 + 2], acc[a][b][4 * g4 + 3]};
+          *(out4_t*)(dst0 + 8 * g4) = v;
+        }
+      } else if (full) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) dst0[(int64_t)(8 * (r >> 2) + (r & 3)) * y_si] = acc[a][b][r];
       } else if (j < p.J) {
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
           const int di = 8 * (r >> 2) + (r & 3);
           if (i0 + di < p.K) {
             if (p.atomic_out)
-              atomicAdd(dst0 + (int64_t)di * ODPQ, acc[a][b][r]);
+              atomicAdd(dst0 + (int64_t)di * y_si, acc[a][b][r]);
             else
-              dst0[(int64_t)di * ODPQ] = acc[a][b][r];
+              dst0[(int64_t)di * y_si] = acc[a][b][r];
           }
         }
       }
@@ -676,7 +719,8 @@ __global__ __launch_bounds__(64 * NW, OCC) void amos_conv_fprop(const ConvFpropP
     unsigned w_off_nx[WCH];
 #pragma unroll
     for (int u = 0; u < WCH; ++u) w_off_nx[u] = w_off[u];
-    bool hand_over = false, after_switch = false;
+    bool hand_over = false;
+    int after_switch = 0;   // 1: sixteen stores per 32x32 tile in flight, 2: four (vector stores)
     auto wk_of_macro = [&](int m) {
       if (m > p.macro_steps - 1) m = p.macro_steps - 1;
       const int tt = fast_div(m, p.fd_cc), cc = m - tt * p.c_chunks;
@@ -697,7 +741,9 @@ __global__ __launch_bounds__(64 * NW, OCC) void amos_conv_fprop(const ConvFpropP
         // memory instructions complete in issue order: the 16 stores per 32x32 tile of the
         // finished tile sit between the copies waited for here and the younger ones
         constexpr int WITH_STORES = IN_FLIGHT + 16 * TI * TJ > 63 ? 63 : IN_FLIGHT + 16 * TI * TJ;
-        if (after_switch) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(WITH_STORES) : "memory");
+        constexpr int WITH_VSTORES = IN_FLIGHT + 4 * TI * TJ;
+        if (after_switch == 1) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(WITH_STORES) : "memory");
+        else if (after_switch == 2) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(WITH_VSTORES) : "memory");
         else asm volatile("s_waitcnt vmcnt(%0)" ::"n"(IN_FLIGHT) : "memory");
       } else {
         asm volatile("s_waitcnt vmcnt(%0)" ::"n"(IN_FLIGHT) : "memory");
@@ -812,14 +858,14 @@ __global__ __launch_bounds__(64 * NW, OCC) void amos_conv_fprop(const ConvFpropP
           if (buf == 0) nine_taps(IntC<0>{}, wk_of_macro(m), wk_nxt, n_live, po, pdb);
           else nine_taps(IntC<1>{}, wk_of_macro(m), wk_nxt, n_live, po, pdb);
           buf ^= 1;
-          after_switch = false;
+          after_switch = 0;
         }
         store_tile(geo);
         if (!has_next) break;
         // a ragged tile issues fewer stores than the waits after the switch allow for
         const bool counted = geo.bi0 + BI <= p.K && geo.bj0 + BJ <= p.J;
         if (!counted) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-        after_switch = counted;
+        after_switch = counted ? (p.y_vec4 ? 2 : 1) : 0;
         geo = geo_n;
         n_pl = n_pl_n;
         tile = next_tile;

@@ -103,7 +103,9 @@ template <int N> struct NSlots { static constexpr int value = N; };
 
 struct ConvGeom {
   int C, D, H, W;   // C = channels that are reduced over (of one group)
-  int Cimg;         // channels between images in memory (all groups)
+  int64_t x_sn;     // element strides of the activations: image, channel, depth, row, column
+  int x_sc, x_sd, x_sh, x_sw;
+  int k_order;      // reduction index k = c*TRS + tap (0, weights KCTRS) or tap*C + c (1, weights TRSCK)
   int T, R, S;
   int sd, sh, sw;
   int pd, ph, pw;
@@ -126,11 +128,12 @@ struct IgemmParams {
   int64_t col_s_row, col_s_k;
   int64_t col_batch;
   ConvGeom g;                   // LD_CONV only
-  // output: element (i, j) at  i*out_si + (j / out_jmod)*out_sjo + j % out_jmod
+  // output: element (i, j) at  i*out_si + (j / out_jmod)*out_sjo + (j % out_jmod)*out_sj
   char* out;
-  int64_t out_si, out_sjo;
+  int64_t out_si, out_sjo, out_sj;
   int out_jmod;
   int64_t out_batch;
+  int out_vec4;                 // out_si == 1, rows % 4 == 0, 16-byte aligned, no atomics: 4 rows per store
   int atomic_out;               // split-K: accumulate into a zeroed output
   EpiParams epi;                // D is indexed like the output, with its own row stride
 };
@@ -243,8 +246,8 @@ __global__ __launch_bounds__(256) void amos_igemm(const IgemmParams p) {
     cv_d0 = od * p.g.sd - p.g.pd;
     cv_h0 = op * p.g.sh - p.g.ph;
     cv_w0 = oq * p.g.sw - p.g.pw;
-    cv_base = (int64_t)img * p.g.Cimg * p.g.D * p.g.H * p.g.W +
-              ((int64_t)cv_d0 * p.g.H + cv_h0) * p.g.W + cv_w0;
+    cv_base = (int64_t)img * p.g.x_sn + (int64_t)cv_d0 * p.g.x_sd + (int64_t)cv_h0 * p.g.x_sh +
+              (int64_t)cv_w0 * p.g.x_sw;
     if (p.g.use_mask && cv_valid) {
       int tap = 0;
       for (int tt = 0; tt < p.g.T; ++tt)
@@ -265,13 +268,14 @@ __global__ __launch_bounds__(256) void amos_igemm(const IgemmParams p) {
       if (k < p.Kred) {
         int rs = p.g.R * p.g.S;
         int trs = p.g.T * rs;
-        int c = k / trs;
-        int tap = k - c * trs;
+        int c, tap;
+        if (p.g.k_order == 0) { c = k / trs; tap = k - c * trs; }
+        else { tap = k / p.g.C; c = k - tap * p.g.C; }
         int tt = tap / rs;
         int rem = tap - tt * rs;
         int rr = rem / p.g.S;
         int ss = rem - rr * p.g.S;
-        e.x = ((c * p.g.D + tt * p.g.dd) * p.g.H + rr * p.g.dh) * p.g.W + ss * p.g.dw;
+        e.x = c * p.g.x_sc + tt * p.g.dd * p.g.x_sd + rr * p.g.dh * p.g.x_sh + ss * p.g.dw * p.g.x_sw;
         e.y = p.g.use_mask ? tap : ((tt * p.g.dd) << 20 | (rr * p.g.dh) << 10 | (ss * p.g.dw));
       } else {
         e.x = 0;
@@ -468,7 +472,7 @@ __global__ __launch_bounds__(256) void amos_igemm(const IgemmParams p) {
     const int j = bj0 + (wj * TJ + b) * 32 + frag_row;
     if (j >= p.J) continue;
     const int jo = j / p.out_jmod;
-    const int64_t coff = (int64_t)jo * p.out_sjo + (j - jo * p.out_jmod);
+    const int64_t coff = (int64_t)jo * p.out_sjo + (int64_t)(j - jo * p.out_jmod) * p.out_sj;
 #pragma unroll
     for (int a = 0; a < TI; ++a) {
       if (add_d) {   // all sixteen loads of the tile in flight before the first addition
@@ -480,6 +484,16 @@ __global__ __launch_bounds__(256) void amos_igemm(const IgemmParams p) {
         }
 #pragma unroll
         for (int r = 0; r < 16; ++r) acc[a][b][r] += dv[r];
+      }
+      if (p.out_vec4) {   // rows (output channels) innermost
+        typedef out_t out4_t __attribute__((ext_vector_type(4)));
+#pragma unroll
+        for (int g4 = 0; g4 < 4; ++g4) {
+          const int i = bi0 + (wi * TI + a) * 32 + 8 * g4 + 4 * frag_half;
+          const out4_t v = {acc[a][b][4 * g4], acc[a][b][4 * g4 + 1], acc[a][b][4 * g4 + 2], acc[a][b][4 * g4 + 3]};
+          if (i < p.I) *(out4_t*)(out + i + coff) = v;
+        }
+        continue;
       }
 #pragma unroll
       for (int r = 0; r < 16; ++r) {

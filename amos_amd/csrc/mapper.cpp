@@ -78,7 +78,7 @@ int problem_of(int op, const void* desc, Problem* out) {
       out->in_dtype = c->in_dtype;
       out->in_bytes = (c->N * c->C * D * c->H * c->W + c->K * out->K) * esize(c->in_dtype);
       out->out_bytes = c->K * out->J * 4;
-      out->row_loader = (out->K % (16 / esize(c->in_dtype)) == 0) ? 0 : 1;
+      out->row_loader = (c->layout == AMOS_LAYOUT_NCHW && out->K % (16 / esize(c->in_dtype)) == 0) ? 0 : 1;
       out->col_loader = 2;
       return 0;
     }

@@ -83,9 +83,11 @@ def gemm_desc(M, N, K, in_dtype, trans_a=False, trans_b=False, lda=None, ldb=Non
     return d
 
 
-def conv_desc(x_shape, w_shape, in_dtype, stride, pad, dil, groups=1):
-    """x_shape NCDHW, w_shape K,(C/groups),T,R,S; stride / pad / dil are 3-tuples"""
+def conv_desc(x_shape, w_shape, in_dtype, stride, pad, dil, groups=1, layout="nchw"):
+    """x_shape NCDHW, w_shape K,(C/groups),T,R,S (the logical extents, whatever the layout in
+    memory); stride / pad / dil are 3-tuples"""
     d = ConvDesc()
+    d.layout = _lib.LAYOUT_CODE[layout] if isinstance(layout, str) else int(layout)
     d.N, d.C, d.D, d.H, d.W = x_shape
     d.K, cg, d.T, d.R, d.S = w_shape
     if cg * groups != d.C:
@@ -169,20 +171,46 @@ def _workspace(op, desc, cfg, device):
     return ws, ptr, need
 
 
-def conv2d(x, w, stride=1, pad=0, dil=1, out=None, config=None, stream=None, add=None, groups=1):
-    """x NCHW, w K,(C/groups),R,S -> NKPQ (+ add of the output's shape)"""
+def logical_conv_shapes(x_shape, w_shape, layout):
+    """(N,C,D,H,W), (K,C/groups,T,R,S) of operands stored in `layout` (4-d operands: D = T = 1)"""
+    code = _lib.LAYOUT_CODE[layout]
+    x_shape, w_shape = tuple(int(e) for e in x_shape), tuple(int(e) for e in w_shape)
+    if len(x_shape) == 4:
+        x_shape = {0: x_shape[:2] + (1,) + x_shape[2:], 1: x_shape[:1] + (1,) + x_shape[1:],
+                   2: (1,) + x_shape}[code]
+        w_shape = w_shape[:2] + (1,) + w_shape[2:] if code == 0 else (1,) + w_shape
+    if code == 0:
+        return x_shape, w_shape
+    t, r, s, c, k = w_shape
+    if code == 1:
+        n, d, h, w_, cx = x_shape
+    else:
+        d, h, w_, n, cx = x_shape
+    return (n, cx, d, h, w_), (k, c, t, r, s)
+
+
+def stored_conv_out_shape(oshape, layout, ndim):
+    """NKDPQ extents -> the output's shape as stored in `layout` (ndim 4: without the depth)"""
+    code = _lib.LAYOUT_CODE[layout]
+    n, k, od, op, oq = oshape
+    sp = (op, oq) if ndim == 4 else (od, op, oq)
+    return {0: (n, k) + sp, 1: (n,) + sp + (k,), 2: sp + (n, k)}[code]
+
+
+def conv2d(x, w, stride=1, pad=0, dil=1, out=None, config=None, stream=None, add=None, groups=1,
+           layout="nchw"):
+    """layout nchw: x NCHW, w K,(C/groups),R,S -> NKPQ; nhwc: x NHWC, w RSCK -> NPQK; hwnc:
+    x HWNC, w RSCK -> PQNK (+ add of the output's shape)"""
     _need_device(x, w)
     st, pd, dl = (1,) + _tup(stride, 2), (0,) + _tup(pad, 2), (1,) + _tup(dil, 2)
-    xs = (x.shape[0], x.shape[1], 1, x.shape[2], x.shape[3])
-    ws = (w.shape[0], w.shape[1], 1, w.shape[2], w.shape[3])
-    if x.shape[1] != w.shape[1] * groups or x.dtype != w.dtype:
+    xs, ws = logical_conv_shapes(x.shape, w.shape, layout)
+    if xs[1] != ws[1] * groups or x.dtype != w.dtype:
         raise ValueError("operand shapes / dtypes do not agree")
     oshape = conv_out_shape(xs, ws, st, pd, dl)
     if out is None:
-        out = torch.empty((oshape[0], oshape[1], oshape[3], oshape[4]), dtype=_OUT_OF[x.dtype],
-                          device=x.device)
+        out = torch.empty(stored_conv_out_shape(oshape, layout, 4), dtype=_OUT_OF[x.dtype], device=x.device)
     _need_device(out)
-    d = conv_desc(xs, ws, x.dtype, st, pd, dl, groups)
+    d = conv_desc(xs, ws, x.dtype, st, pd, dl, groups, layout)
     cfg = make_config(config)
     ws, ws_ptr, ws_bytes = _workspace(AMOS_OP_CONV2D, d, cfg, x.device)
     epi = make_epilogue(add, tuple(out.shape), out.dtype)
@@ -191,17 +219,20 @@ def conv2d(x, w, stride=1, pad=0, dil=1, out=None, config=None, stream=None, add
     return out
 
 
-def conv3d(x, w, stride=1, pad=0, dil=1, out=None, config=None, stream=None, add=None, groups=1):
-    """x NCDHW, w K,(C/groups),T,R,S -> NKDPQ (+ add of the output's shape)"""
+def conv3d(x, w, stride=1, pad=0, dil=1, out=None, config=None, stream=None, add=None, groups=1,
+           layout="ncdhw"):
+    """layout ncdhw: x NCDHW, w K,(C/groups),T,R,S -> NKDPQ; ndhwc: x NDHWC, w TRSCK -> NDPQK;
+    dhwnc: x DHWNC, w TRSCK -> DPQNK (+ add of the output's shape)"""
     _need_device(x, w)
     st, pd, dl = _tup(stride, 3), _tup(pad, 3), _tup(dil, 3)
-    if x.shape[1] != w.shape[1] * groups or x.dtype != w.dtype:
+    xs, ws = logical_conv_shapes(x.shape, w.shape, layout)
+    if xs[1] != ws[1] * groups or x.dtype != w.dtype:
         raise ValueError("operand shapes / dtypes do not agree")
-    oshape = conv_out_shape(tuple(x.shape), tuple(w.shape), st, pd, dl)
+    oshape = conv_out_shape(xs, ws, st, pd, dl)
     if out is None:
-        out = torch.empty(oshape, dtype=_OUT_OF[x.dtype], device=x.device)
+        out = torch.empty(stored_conv_out_shape(oshape, layout, 5), dtype=_OUT_OF[x.dtype], device=x.device)
     _need_device(out)
-    d = conv_desc(tuple(x.shape), tuple(w.shape), x.dtype, st, pd, dl, groups)
+    d = conv_desc(xs, ws, x.dtype, st, pd, dl, groups, layout)
     cfg = make_config(config)
     ws, ws_ptr, ws_bytes = _workspace(AMOS_OP_CONV3D, d, cfg, x.device)
     epi = make_epilogue(add, tuple(out.shape), out.dtype)

@@ -105,7 +105,12 @@ typedef struct {
  * groups > 1: channel group g of X (C/groups channels) meets output channels
  * [g*K/groups, (g+1)*K/groups) only; Wt is [K][C/groups][T][R][S].  groups = C is the
  * depthwise convolution with K/C outputs per channel.
- * (reference computes: benchmark/amos/mapping_conv2d_tensorcore.py:7-42,
+ * layout: how the three tensors (and a fused tail's D, like Y) are stored:
+ *   AMOS_LAYOUT_NCHW  X [N][C][D][H][W]   Wt [K][C][T][R][S]   Y [N][K][OD][OP][OQ]
+ *   AMOS_LAYOUT_NHWC  X [N][D][H][W][C]   Wt [T][R][S][C][K]   Y [N][OD][OP][OQ][K]
+ *   AMOS_LAYOUT_HWNC  X [D][H][W][N][C]   Wt [T][R][S][C][K]   Y [OD][OP][OQ][N][K]
+ * (groups > 1 exists for AMOS_LAYOUT_NCHW only.)
+ * (reference computes: benchmark/amos/mapping_conv2d_tensorcore.py:7-104 (the three layouts),
  *  benchmark/amos/mapping_conv3d_tensorcore.py:7-55, mapping_groupedconv2d_tensorcore.py:7-60,
  *  mapping_depthwiseconv2d_tensorcore.py:7-48)
  */
@@ -117,8 +122,12 @@ typedef struct {
   int32_t dil_d, dil_h, dil_w;
   int32_t in_dtype, out_dtype;
   int32_t groups;        /* 0 or 1 = ordinary convolution */
-  int32_t reserved;
+  int32_t layout;        /* AMOS_LAYOUT_* */
 } amos_conv_desc_t;
+
+#define AMOS_LAYOUT_NCHW 0
+#define AMOS_LAYOUT_NHWC 1
+#define AMOS_LAYOUT_HWNC 2
 
 /*
  * How the implicit GEMM is tiled on the chip -- the counterpart of the

@@ -9,8 +9,8 @@ import pytest
 import amos_amd.tvm as tvm
 from amos_amd.tvm import auto_tensorize as at
 from oracle import cpu_oracle as co
-from test_mapper import (batched_fc, conv1d, conv2d, depthwise_conv2d, gemm, gemv, grouped_conv2d,
-                         grouped_conv_reference)
+from test_mapper import (batched_fc, conv1d, conv2d, conv2d_layout, depthwise_conv2d, from_nkpq, gemm, gemv,
+                         grouped_conv2d, grouped_conv_reference, to_nchw)
 
 pytestmark = pytest.mark.gpu
 
@@ -195,6 +195,25 @@ def test_conv1d_script_flow(gpu, tmp_path, C):
     assert result.sch_app.lowered.kind == "conv2d"
     ref = co.lib_conv2d(a[:, :, None, :], b[:, :, None, :], "float16", (1, stride), (0, padding), (1, dilation),
                         acc="float64")[:, :, 0, :]
+    mx, mean = co.rel_errors(got, ref)
+    assert got.shape == ref.shape and mx <= 1e-2 and mean <= 1e-3
+
+
+@pytest.mark.parametrize("layout", ["nhwc", "hwnc"])
+@pytest.mark.parametrize("C", [64, 24])    # patch-staged and register-staged kernels
+def test_conv2d_layout_script_flow(gpu, tmp_path, layout, C):
+    """reference computes: benchmark/amos/mapping_conv2d_tensorcore.py:43-104"""
+    N, H, W, K, R, S, stride, padding, dilation = 3, 20, 18, 40, 3, 3, 1, 1, 1
+    A, B, Conv = conv2d_layout(N, C, H, W, K, R, S, stride, padding, dilation, layout)
+    rng = np.random.default_rng(9)
+    a = rng.uniform(-1, 1, [int(e) for e in A.shape]).astype(np.float16)
+    b = rng.uniform(-1, 1, (R, S, C, K)).astype(np.float16)
+    got, result = _run_script_flow([A, B, Conv], {"A": a, "B": b}, tmp_path, "conv2d_" + layout)
+    low = result.sch_app.lowered
+    assert low.kind == "conv2d" and low.attrs["layout"] == layout
+    an, bn = to_nchw(a, b, layout)
+    ref = from_nkpq(co.lib_conv2d(np.ascontiguousarray(an), np.ascontiguousarray(bn), "float16", stride, padding,
+                                  dilation, acc="float64"), layout)
     mx, mean = co.rel_errors(got, ref)
     assert got.shape == ref.shape and mx <= 1e-2 and mean <= 1e-3
 

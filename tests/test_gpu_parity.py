@@ -343,6 +343,93 @@ def test_conv_tile_walk(gpu, dtype, case):
     assert walked == 2
 
 
+@pytest.mark.parametrize("layout", ["nhwc", "hwnc"])
+def test_conv_tile_walk_channel_innermost(gpu, layout):
+    """walking workgroups with vector stores of four output channels"""
+    import torch
+    from amos_amd import _lib, ops
+    N, C, H, W, K, R, S = 16, 128, 41, 41, 72, 3, 3
+    rng = np.random.default_rng(12)
+    x = make_operand(rng, (N, C, 1, H, W), "float16", "normal")
+    w = make_operand(rng, (K, C, 1, R, S), "float16", "normal")
+    ref = co.lib_conv3d(x, w, "float16", (1, 1, 1), (0, 1, 1), (1, 1, 1), acc="float64")[:, :, 0]
+    to_x = (0, 2, 3, 1) if layout == "nhwc" else (2, 3, 0, 1)
+    dx = to_device(np.ascontiguousarray(np.transpose(x[:, :, 0], to_x)), "float16")
+    dw = to_device(np.ascontiguousarray(np.transpose(w[:, :, 0], (2, 3, 1, 0))), "float16")
+    refs = np.transpose(ref, to_x)
+    d_add = torch.randn(refs.shape, device="cuda")
+    desc = ops.conv_desc((N, C, 1, H, W), (K, C, 1, R, S), torch.float16, (1, 1, 1), (0, 1, 1), (1, 1, 1), 1, layout)
+    for tile in [(64, 128), (128, 64)]:
+        outs = {}
+        for flags in (0, _lib.AMOS_FLAG_NO_TILE_WALK):
+            cfg = dict(tile_i=tile[0], tile_j=tile[1], split_k=1, pipeline=_lib.AMOS_PIPE_PATCH8, flags=flags)
+            assert ("walk" in ops.kernel_name(_lib.AMOS_OP_CONV2D, desc, cfg)) == (flags == 0)
+            for add in (None, d_add):
+                outs[(flags, add is None)] = ops.conv2d(dx, dw, 1, 1, 1, config=cfg, add=add, layout=layout)
+        assert torch.equal(outs[(0, True)], outs[(_lib.AMOS_FLAG_NO_TILE_WALK, True)])
+        assert torch.equal(outs[(0, False)], outs[(_lib.AMOS_FLAG_NO_TILE_WALK, False)])
+        check(outs[(0, True)].cpu().numpy(), refs, "float16", "walk %s tile %s" % (layout, tile))
+        check((outs[(0, False)] - d_add).cpu().numpy(), refs, "float16", "walk + D %s tile %s" % (layout, tile))
+
+
+LAYOUT_CASES = [
+    # N, C, D, H, W, K, T, R, S, stride, pad, dil
+    (3, 24, 1, 9, 7, 40, 1, 3, 3, (1, 1, 1), (0, 1, 1), (1, 1, 1)),      # register-staged kernel only
+    (2, 128, 1, 12, 10, 72, 1, 3, 3, (1, 1, 1), (0, 1, 1), (1, 1, 1)),   # patch-staged applies
+    (2, 128, 1, 9, 11, 64, 1, 3, 2, (1, 2, 1), (0, 1, 0), (1, 1, 2)),    # stride, dilation
+    (2, 128, 4, 6, 6, 24, 3, 3, 3, (1, 1, 1), (1, 1, 1), (1, 1, 1)),     # conv3d
+]
+
+
+@pytest.mark.parametrize("layout", ["nhwc", "hwnc"])
+@pytest.mark.parametrize("dtype", ["float16", "int8"])
+@pytest.mark.parametrize("case", LAYOUT_CASES)
+def test_conv_layouts(gpu, layout, dtype, case):
+    """channel-innermost layouts (NHWC / RSCK / NPQK and HWNC / RSCK / PQNK, their 3-d forms):
+    every pipeline against the oracle evaluated on the same tensors in NCDHW order"""
+    import torch
+    from amos_amd import _lib, ops
+    N, C, D, H, W, K, T, R, S, st, pd, dl = case
+    rng = np.random.default_rng(3)
+    x = make_operand(rng, (N, C, D, H, W), dtype, "normal")
+    w = make_operand(rng, (K, C, T, R, S), dtype, "normal")
+    ref = co.lib_conv3d(x, w, dtype, st, pd, dl, acc="float64")            # N K OD OP OQ
+    is2d = D == 1 and T == 1
+    to_x = (0, 2, 3, 4, 1) if layout == "nhwc" else (2, 3, 4, 0, 1)
+    xs = np.ascontiguousarray(np.transpose(x, to_x))
+    ws_ = np.ascontiguousarray(np.transpose(w, (2, 3, 4, 1, 0)))          # T R S C K
+    refs = np.ascontiguousarray(np.transpose(ref, to_x))
+    if is2d:
+        xs, ws_, refs = (xs[:, 0], ws_[0], refs[:, 0]) if layout == "nhwc" else (xs[0], ws_[0], refs[0])
+    dx, dw = to_device(np.ascontiguousarray(xs), dtype), to_device(np.ascontiguousarray(ws_), dtype)
+    d_add = torch.randn(refs.shape, device="cuda").to(torch.int32 if dtype == "int8" else torch.float32)
+    ran = set()
+    for pipe in (None, _lib.AMOS_PIPE_STAGED, _lib.AMOS_PIPE_PATCH, _lib.AMOS_PIPE_PATCH8):
+        for tile, split in [((64, 64), 1), ((128, 64), 2), ((64, 128), 1)]:
+            cfg = None if pipe is None else dict(tile_i=tile[0], tile_j=tile[1], split_k=split, pipeline=pipe)
+            for add in (None, d_add):
+                try:
+                    if is2d:
+                        got = ops.conv2d(dx, dw, st[1:], pd[1:], dl[1:], config=cfg, add=add, layout=layout)
+                    else:
+                        got = ops.conv3d(dx, dw, st, pd, dl, config=cfg, add=add,
+                                         layout="ndhwc" if layout == "nhwc" else "dhwnc")
+                except _lib.AmosError as e:
+                    assert pipe in (_lib.AMOS_PIPE_PATCH, _lib.AMOS_PIPE_PATCH8) and "not applicable" in str(e)
+                    continue
+                ran.add(pipe)
+                assert tuple(got.shape) == refs.shape
+                if add is not None:
+                    got = got - add
+                check(got.cpu().numpy(), refs, dtype, "%s %s %s pipeline %s tile %s split %d add %s"
+                      % (layout, dtype, case, pipe, tile, split, add is not None))
+            if pipe is None:
+                break
+    assert None in ran and _lib.AMOS_PIPE_STAGED in ran
+    if C * (1 if dtype == "int8" else 2) % 128 == 0:
+        assert _lib.AMOS_PIPE_PATCH in ran or _lib.AMOS_PIPE_PATCH8 in ran
+
+
 def test_conv_patch_is_the_default_when_applicable(gpu):
     import torch
     from amos_amd import _lib, ops

@@ -233,6 +233,69 @@ def test_lowered_conv2d_means_what_the_compute_says(case):
     assert np.array_equal(got, want)
 
 
+def conv2d_layout(N, C, H, W, K, R, S, stride, padding, dilation, layout, dtype="float16", out_dtype="float32",
+                  exact_int=False):
+    """the reference's conv2d in its nhwc and hwnc spellings (benchmark/amos/mapping_conv2d_tensorcore.py:43-104)"""
+    kH, kW = (R - 1) * dilation + 1, (S - 1) * dilation + 1
+    pH, pW = H + 2 * padding, W + 2 * padding
+    P, Q = (pH - kH) // stride + 1, (pW - kW) // stride + 1
+    rc = te.reduce_axis([0, C], name="rc")
+    rr = te.reduce_axis([0, R], name="rr")
+    rs = te.reduce_axis([0, S], name="rs")
+    B = te.placeholder([R, S, C, K], dtype=dtype, name="B")
+
+    def mul(a, b):
+        return a.astype(out_dtype) * b.astype(out_dtype) if exact_int else (a * b).astype(out_dtype)
+
+    inside = lambda h, w: tir.all(h >= padding, h - padding < H, w >= padding, w - padding < W)
+    if layout == "nhwc":
+        A = te.placeholder([N, H, W, C], dtype=dtype, name="A")
+        Pad = te.compute([N, pH, pW, C], lambda n, h, w, c: tir.if_then_else(
+            inside(h, w), A[n, h - padding, w - padding, c], tir.const(0.0, A.dtype)), name="Pad")
+        Conv = te.compute([N, P, Q, K], lambda n, p, q, k: te.sum(
+            mul(Pad[n, p * stride + rr * dilation, q * stride + rs * dilation, rc], B[rr, rs, rc, k]),
+            axis=[rr, rs, rc]), name="Conv")
+    else:
+        A = te.placeholder([H, W, N, C], dtype=dtype, name="A")
+        Pad = te.compute([pH, pW, N, C], lambda h, w, n, c: tir.if_then_else(
+            inside(h, w), A[h - padding, w - padding, n, c], tir.const(0.0, A.dtype)), name="Pad")
+        Conv = te.compute([P, Q, N, K], lambda p, q, n, k: te.sum(
+            mul(Pad[p * stride + rr * dilation, q * stride + rs * dilation, n, rc], B[rr, rs, rc, k]),
+            axis=[rr, rs, rc]), name="Conv")
+    return A, B, Conv
+
+
+def to_nchw(a, b, layout):
+    """operands stored in `layout` -> NCHW activations, KCRS weights"""
+    return (np.transpose(a, (0, 3, 1, 2) if layout == "nhwc" else (2, 3, 0, 1)), np.transpose(b, (3, 2, 0, 1)))
+
+
+def from_nkpq(y, layout):
+    return np.transpose(y, (0, 2, 3, 1) if layout == "nhwc" else (2, 3, 0, 1))
+
+
+@pytest.mark.parametrize("layout", ["nhwc", "hwnc"])
+@pytest.mark.parametrize("case", CONV_LOWER_CASES)
+def test_lowered_conv2d_layouts_mean_what_the_compute_says(case, layout):
+    N, C, H, W, K, R, S, st, pd, dl = case
+    A, B, Conv = conv2d_layout(N, C, H, W, K, R, S, st, pd, dl, layout, dtype="int8", out_dtype="int32",
+                               exact_int=True)
+    assert len(at.get_match_results(at.compute_dag_from_tensors([Conv]), "hip")) > 0
+    low = at.lower_main_op(Conv.op)
+    assert low.kind == "conv2d" and low.attrs["layout"] == layout and low.desc.layout == _lib.LAYOUT_CODE[layout]
+    assert low.attrs["stride"] == [st, st] and low.attrs["pad"] == [pd, pd] and low.attrs["dil"] == [dl, dl]
+    assert (low.desc.N, low.desc.C, low.desc.H, low.desc.W, low.desc.K, low.desc.R, low.desc.S) == (N, C, H, W, K, R, S)
+    assert [t.name for t in low.inputs] == ["A", "B"]
+    rng = np.random.default_rng(2)
+    a = rng.integers(-9, 10, [int(e) for e in A.shape]).astype(np.int8)
+    b = rng.integers(-9, 10, (R, S, C, K)).astype(np.int8)
+    want = te_interp.evaluate(Conv, {"A": a, "B": b})
+    an, bn = to_nchw(a, b, layout)
+    got = co.te_literal_conv2d(np.ascontiguousarray(an), np.ascontiguousarray(bn), "int8", low.attrs["stride"],
+                               low.attrs["pad"], low.attrs["dil"], mode="exact")
+    assert np.array_equal(from_nkpq(got, layout), want)
+
+
 def test_no_kernel_for_other_layouts():
     # NHWC activations match the intrinsic but have no kernel
     N, H, W, C, K = 2, 6, 6, 8, 8
