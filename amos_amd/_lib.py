@@ -63,6 +63,11 @@ class Epilogue(ctypes.Structure):
                 ("stride", _i64)]
 
 
+class GatherDesc(ctypes.Structure):
+    _fields_ = [("ndim", _i32), ("elem_bytes", _i32), ("out_shape", _i64 * 5), ("table_offset", _i64 * 5),
+                ("in_elems", _i64)]
+
+
 class ComputeC(ctypes.Structure):
     _fields_ = [("n_tokens", _i32), ("tokens", ctypes.POINTER(_i32)), ("n_iters", _i32),
                 ("iter_kinds", ctypes.POINTER(_i32)), ("iter_extents", ctypes.POINTER(_i64)),
@@ -82,8 +87,8 @@ class AmosError(RuntimeError):
 EXPORTS = [
     "amos_version", "amos_last_error", "amos_device_info", "amos_default_config",
     "amos_check_config", "amos_workspace_bytes", "amos_estimate_seconds", "amos_gemm", "amos_bgemm", "amos_conv2d",
-    "amos_conv3d", "amos_run_fused", "amos_time", "amos_time_fused", "amos_kernel_name", "amos_match",
-    "amos_enumerate_mappings",
+    "amos_conv3d", "amos_run_fused", "amos_time", "amos_time_fused", "amos_gather", "amos_time_gather",
+    "amos_kernel_name", "amos_match", "amos_enumerate_mappings",
 ]
 
 _lib = None
@@ -122,6 +127,9 @@ def load():
     lib.amos_time_fused.argtypes = [ctypes.c_int, vp, ctypes.POINTER(KernelConfig), ctypes.POINTER(Epilogue),
                                     vp, vp, vp, vp, sz, vp, ctypes.c_int, ctypes.c_int, ctypes.c_int,
                                     ctypes.POINTER(ctypes.c_double)]
+    lib.amos_gather.argtypes = [ctypes.POINTER(GatherDesc), vp, vp, vp, vp]
+    lib.amos_time_gather.argtypes = [ctypes.POINTER(GatherDesc), vp, vp, vp, vp, ctypes.c_int, ctypes.c_int,
+                                     ctypes.c_int, ctypes.POINTER(ctypes.c_double)]
     lib.amos_kernel_name.argtypes = [ctypes.c_int, vp, ctypes.POINTER(KernelConfig)]
     lib.amos_kernel_name.restype = ctypes.c_char_p
     lib.amos_match.argtypes = [ctypes.POINTER(ComputeC), ctypes.POINTER(ComputeC),

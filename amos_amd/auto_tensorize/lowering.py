@@ -28,6 +28,9 @@ class LoweredOp(object):
         self.output = output
         self.attrs = attrs
         self.add_input = None    # tensor D of a fused tail  output = main + D.astype(out), else None
+        # {0 or 1: OperandView}: the kernel does not read inputs[k] itself but a tensor gathered
+        # from it (stages in front of the operand that no loader folds in), materialised per call
+        self.gathers = {}
 
     def flops(self):
         a = self.attrs
@@ -54,6 +57,129 @@ def _single_var(form, iters):
         if iv.var is v:
             return iv
     return None
+
+
+class OperandView(object):
+    """a tensor every element of which is one element of a placeholder or zero, the source
+    index of each dimension depending on that dimension's index alone:
+    view[o0, .., on] = src.flat[sum_d tables[d][o_d]] if all tables[d][o_d] >= 0 else 0"""
+
+    def __init__(self, src, shape, tables, dtype):
+        self.src, self.shape, self.tables, self.dtype = src, list(shape), tables, dtype
+
+
+class _NotSeparable(Exception):
+    pass
+
+
+def _eval_int(e, env):
+    if isinstance(e, te.IntImm):
+        return int(e.value)
+    if isinstance(e, te.Var):
+        if id(e) not in env:
+            raise _NotSeparable("free variable %s" % e.name)
+        return env[id(e)]
+    if isinstance(e, te.Cast):
+        return _eval_int(e.value, env)
+    if isinstance(e, te.And):
+        return all(_eval_int(t, env) for t in e.terms)
+    if isinstance(e, te.Cmp):
+        a, b = _eval_int(e.a, env), _eval_int(e.b, env)
+        return {"==": a == b, ">=": a >= b, ">": a > b, "<=": a <= b, "<": a < b, "!=": a != b}[e.op]
+    if isinstance(e, (te.Add, te.Sub, te.Mul, te.FloorDiv, te.FloorMod)):
+        a, b = _eval_int(e.a, env), _eval_int(e.b, env)
+        if isinstance(e, te.Add): return a + b
+        if isinstance(e, te.Sub): return a - b
+        if isinstance(e, te.Mul): return a * b
+        if b == 0:
+            raise _NotSeparable("division by zero")
+        return a // b if isinstance(e, te.FloorDiv) else a % b
+    raise _NotSeparable("expression %r" % (e,))
+
+
+def _vars_in(e, out):
+    if isinstance(e, te.Var):
+        out[id(e)] = e
+    for name in ("a", "b", "value", "cond", "then_value", "else_value"):
+        if hasattr(e, name) and isinstance(getattr(e, name), te.Expr):
+            _vars_in(getattr(e, name), out)
+    for t in getattr(e, "terms", []):
+        _vars_in(t, out)
+    return out
+
+
+def _index_tables(indices, variables, extents, src_shape, cond=None):
+    """for a load `src[indices]` under `cond`, with every index and every term of the condition a
+    function of one variable: {position of the variable: (source dimension, [source index or -1])}"""
+    ids = [id(v) for v in variables]
+    terms = []
+    if cond is not None:
+        terms = list(cond.terms) if isinstance(cond, te.And) else [cond]
+    term_var = []
+    for t in terms:
+        vs = [k for k in _vars_in(t, {}) if k in ids]
+        if len(vs) > 1:
+            raise _NotSeparable("a condition couples two indices")
+        term_var.append(ids.index(vs[0]) if vs else None)
+    if any(tv is None and not _eval_int(t, {}) for t, tv in zip(terms, term_var)):
+        raise _NotSeparable("constant false condition")
+    stage = {}
+    for k, idx in enumerate(indices):
+        vs = [v for v in _vars_in(idx, {}) if v in ids]
+        if len(vs) != 1:
+            raise _NotSeparable("an index of %d variables" % len(vs))
+        d = ids.index(vs[0])
+        if d in stage:
+            raise _NotSeparable("one variable in two indices")
+        table = []
+        for v in range(extents[d]):
+            env = {ids[d]: v}
+            ok = all(_eval_int(t, env) for t, tv in zip(terms, term_var) if tv == d)
+            x = _eval_int(idx, env)
+            table.append(x if ok and 0 <= x < int(src_shape[k]) else -1)
+        stage[d] = (k, table)
+    if len(stage) != len(variables):
+        raise _NotSeparable("an index variable that selects nothing")
+    return stage
+
+
+def _operand_view(tensor, head=None):
+    """OperandView of `tensor` (a chain of index-remapping stages over a placeholder); `head`:
+    an extra outermost stage (shape, variables, indices into `tensor`), e.g. a load with
+    flipped or permuted indices"""
+    try:
+        if head is not None:
+            shape, variables, indices = head
+            stage = _index_tables(indices, variables, shape, tensor.shape)
+            view = [stage[d] for d in range(len(shape))]
+        else:
+            shape = [int(s) for s in tensor.shape]
+            view = [(d, list(range(shape[d]))) for d in range(len(shape))]
+        cur = tensor
+        while not isinstance(cur.op, te.PlaceholderOp):
+            op = cur.op
+            if not isinstance(op, te.ComputeOp) or op.reduce_axis:
+                raise _NotSeparable("stage %s reduces" % op.name)
+            body, cond = op.body[0], None
+            if isinstance(body, te.Select):
+                zero = body.else_value
+                if not isinstance(zero, (te.IntImm, te.FloatImm)) or zero.value != 0:
+                    raise _NotSeparable("a stage fills with something other than zero")
+                body, cond = body.then_value, body.cond
+            if not isinstance(body, te.ProducerLoad) or body.dtype != cur.dtype:
+                raise _NotSeparable("stage %s computes" % op.name)
+            stage = _index_tables(body.indices, [iv.var for iv in op.axis],
+                                  [int(iv.dom.extent) for iv in op.axis], body.tensor.shape, cond)
+            view = [(stage[cd][0], [stage[cd][1][i] if i >= 0 else -1 for i in idxs]) for cd, idxs in view]
+            cur = body.tensor
+        if sorted(cd for cd, _ in view) != list(range(len(cur.shape))):
+            raise _NotSeparable("dimensions of the source are merged or dropped")
+    except _NotSeparable as e:
+        raise NoKernelError("operand %s is not a per-dimension rearrangement of a placeholder: %s"
+                            % (tensor.name, e))
+    strides = _row_major_strides([int(s) for s in cur.shape])
+    tables = [[i * strides[cd] if i >= 0 else -1 for i in idxs] for cd, idxs in view]
+    return OperandView(cur, shape, tables, cur.dtype)
 
 
 def _strip_cast(e):
@@ -320,29 +446,47 @@ def _lower_conv(main_op, l0, l1, iters, forms0, forms1):
         if len(fx) != nsp + 2 or len(fw) != nsp + 2:
             return None
         n_iv, k_iv, out_sp = spatial[on], spatial[ok], [spatial[d] for d in osp]
-        wv = [_single_var(f, iters) for f in fw]
-        rc, red_sp = wv[wc], [wv[d] for d in wsp]
-        if wv[wk] is not k_iv or rc is None or any(r is None for r in red_sp):
+        # the activations say which reduce axis is the channel and which belongs to which
+        # spatial dimension
+        rc = _single_var(fx[xc], iters)
+        if _single_var(fx[xn], iters) is not n_iv or rc is None or all(rc is not r for r in reduce_):
             return None
-        if set(id(r) for r in [rc] + red_sp) != set(id(r) for r in reduce_):
-            return None
-        if _single_var(fx[xn], iters) is not n_iv or _single_var(fx[xc], iters) is not rc:
-            return None
-        strides, dils = [], []
+        strides, dils, red_sp = [], [], []
         for d in range(nsp):
             f = fx[xsp[d]]
             if f is None:
                 return None
             coef, const = f
-            if const != 0 or set(coef.keys()) != {out_sp[d].var, red_sp[d].var}:
-                # a 1-wide window has a reduce axis of extent 1 that may be folded away
-                if const != 0 or set(coef.keys()) - {out_sp[d].var, red_sp[d].var}:
-                    return None
+            rv = [iv for iv in reduce_ if iv.var in coef]
+            if const != 0 or len(rv) > 1 or set(coef.keys()) - {out_sp[d].var} - {iv.var for iv in rv}:
+                return None
+            # (a 1-wide window has a reduce axis of extent 1 that may be folded away)
+            red_sp.append(rv[0] if rv else None)
             strides.append(int(coef.get(out_sp[d].var, 1)))
-            dils.append(int(coef.get(red_sp[d].var, 1)))
+            dils.append(int(coef[rv[0].var]) if rv else 1)
             if strides[-1] < 1 or dils[-1] < 1:
                 return None
-        return strides, dils, rc, red_sp, out_sp
+        # the weights: laid out as the template says, or any per-dimension rearrangement of the
+        # same axes (flipped windows, swapped channel dimensions: gathered into the template's order)
+        wv = [_single_var(f, iters) for f in fw]
+        canonical = wv[wk] is k_iv and wv[wc] is rc and all(
+            wv[wsp[d]] is not None and (red_sp[d] is None or wv[wsp[d]] is red_sp[d]) for d in range(nsp))
+        if canonical:
+            red_sp = [wv[wsp[d]] for d in range(nsp)]
+        else:
+            per_dim = []
+            for idx in lw.indices:
+                vs = [iv for iv in iters if id(iv.var) in _vars_in(idx, {})]
+                if len(vs) != 1:
+                    return None
+                per_dim.append(vs[0])
+            left = [r for r in reduce_ if r is not rc and all(r is not q for q in red_sp)]
+            red_sp = [q if q is not None else left.pop(0) for q in red_sp if q is not None or left]
+            if len(red_sp) != nsp or sorted(id(v) for v in per_dim) != sorted(id(v) for v in [k_iv, rc] + red_sp):
+                return None
+        if sorted(id(r) for r in [rc] + red_sp) != sorted(id(r) for r in reduce_):
+            return None
+        return strides, dils, rc, red_sp, out_sp, k_iv, canonical
 
     found = None
     for template in _conv_templates(nsp):
@@ -355,12 +499,31 @@ def _lower_conv(main_op, l0, l1, iters, forms0, forms1):
             break
     if found is None:
         return None
-    template, lx, lw, (strides, dils, rc, red_sp, out_sp) = found
+    template, lx, lw, (strides, dils, rc, red_sp, out_sp, k_iv, canonical) = found
     layout, (xn, xc, xsp), (wk, wc, wsp), _ = template
-    src, pads = _pad_stage(lx.tensor, xsp)
-    if not isinstance(lw.tensor.op, te.PlaceholderOp):
-        raise NoKernelError("convolution weights must be a placeholder")
-    xs_mem, ws_mem = [int(s) for s in src.shape], [int(s) for s in lw.tensor.shape]
+    gathers = {}
+    try:
+        src, pads = _pad_stage(lx.tensor, xsp)
+        xs_mem = [int(s) for s in src.shape]
+    except NoKernelError:
+        # stages other than one symmetric zero padding (the zero expansion and one-sided padding
+        # of a transposed convolution ...): materialised, the kernel then reads a dense tensor
+        view = _operand_view(lx.tensor)
+        src, pads, xs_mem = view.src, [0] * nsp, list(view.shape)
+        gathers[0] = view
+    if canonical and isinstance(lw.tensor.op, te.PlaceholderOp):
+        wt, ws_mem = lw.tensor, [int(s) for s in lw.tensor.shape]
+    else:
+        head = None
+        if not canonical:
+            order = [None] * (nsp + 2)
+            order[wk], order[wc] = k_iv, rc
+            for d in range(nsp):
+                order[wsp[d]] = red_sp[d]
+            head = ([int(iv.dom.extent) for iv in order], [iv.var for iv in order], lw.indices)
+        view = _operand_view(lw.tensor, head)
+        wt, ws_mem = view.src, list(view.shape)
+        gathers[1] = view
     # logical extents: N, C, spatial...; K, C, window...
     xs = [xs_mem[xn], xs_mem[xc]] + [xs_mem[d] for d in xsp]
     ws = [ws_mem[wk], ws_mem[wc]] + [ws_mem[d] for d in wsp]
@@ -395,7 +558,9 @@ def _lower_conv(main_op, l0, l1, iters, forms0, forms1):
     attrs = dict(x_shape=xs, w_shape=ws, stride=strides, pad=pads, dil=dils, dtype=lx.dtype, J=J,
                  K_out=ws[0], K_red=ws[1] * (ws5[2] * ws5[3] * ws5[4]), layout=layout)
     kind, code = ("conv2d", _lib.AMOS_OP_CONV2D) if nsp <= 2 else ("conv3d", _lib.AMOS_OP_CONV3D)
-    return LoweredOp(kind, code, c, [src, lw.tensor], main_op.output(0), attrs)
+    low = LoweredOp(kind, code, c, [src, wt], main_op.output(0), attrs)
+    low.gathers = gathers
+    return low
 
 
 def _numel(shape):

@@ -73,10 +73,22 @@ def evaluate_params_on_device(lowered, params, measure_opt):
     """milliseconds per launch of one kernel configuration"""
     from .. import ops
     in0, in1, out = random_device_arrays(lowered, measure_opt.dev_id)
-    secs = ops.time_op(lowered.op_code, lowered.desc, in0, in1, out, config=params.to_config(),
+    # stages materialised in front of an operand: the same for every configuration, timed once
+    extra, ins = 0.0, [in0, in1]
+    for pos, view in getattr(lowered, "gathers", {}).items():
+        g = ops.Gather(view.shape, view.tables, _TORCH_DTYPE[view.dtype], ins[pos].numel(), ins[pos].device)
+        src = ins[pos]
+        ins[pos] = g(src)
+        if not hasattr(lowered, "_gather_seconds"):
+            lowered._gather_seconds = {}
+        if pos not in lowered._gather_seconds:
+            t = g.time(src, ins[pos], number=measure_opt.number, repeat=1, min_repeat_ms=measure_opt.min_repeat_ms)
+            lowered._gather_seconds[pos] = t[0]
+        extra += lowered._gather_seconds[pos]
+    secs = ops.time_op(lowered.op_code, lowered.desc, ins[0], ins[1], out, config=params.to_config(),
                        number=measure_opt.number, repeat=max(1, measure_opt.repeat),
                        min_repeat_ms=measure_opt.min_repeat_ms, add=random_add_array(lowered, measure_opt.dev_id))
-    return sum(secs) / len(secs) * 1e3
+    return (sum(secs) / len(secs) + extra) * 1e3
 
 
 def evaluate_params(schedule_app, params, measure_opt, timeout=100, dump=False):

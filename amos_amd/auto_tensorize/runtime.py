@@ -89,6 +89,19 @@ class Module(object):
         except ValueError:
             raise ValueError("build() args must hold the compute's inputs and its output tensor")
         self.imported_modules = [_Source(self)]
+        self._gathers = {}     # operand position -> (ops.Gather, materialised operand), made on first use
+
+    def _kernel_inputs(self, in0, in1):
+        """the operands the kernel reads: the caller's arrays, or what the stages in front of an
+        operand make of them (materialised into a buffer the module keeps)"""
+        ins = [in0, in1]
+        for pos, view in getattr(self.lowered, "gathers", {}).items():
+            if pos not in self._gathers:
+                g = ops.Gather(view.shape, view.tables, _TORCH_DTYPE[view.dtype], ins[pos].numel(), ins[pos].device)
+                self._gathers[pos] = (g, torch.empty(g.out_shape, dtype=g.dtype, device=ins[pos].device))
+            g, buf = self._gathers[pos]
+            ins[pos] = g(ins[pos].contiguous(), buf)
+        return ins
 
     def _pick(self, arrays):
         if len(arrays) <= max(self.arg_index):
@@ -101,7 +114,8 @@ class Module(object):
 
     def _run(self, in0, in1, out, add=None):
         cfg = self.params.to_config() if self.params is not None else None
-        ops.run_desc(self.lowered.op_code, self.lowered.desc, in0, in1, out, config=cfg, add=add)
+        k0, k1 = self._kernel_inputs(in0, in1)
+        ops.run_desc(self.lowered.op_code, self.lowered.desc, k0, k1, out, config=cfg, add=add)
 
     def __call__(self, *arrays):
         self._run(*self._pick(arrays))
@@ -109,11 +123,17 @@ class Module(object):
     def time_evaluator(self, func_name=None, ctx=None, number=10, repeat=1, min_repeat_ms=0):
         def evaluator(*arrays):
             picked = self._pick(arrays)
-            in0, in1, out = picked[:3]
+            out = picked[2]
+            in0, in1 = self._kernel_inputs(picked[0], picked[1])
             cfg = self.params.to_config() if self.params is not None else None
-            return TimeResult(ops.time_op(self.lowered.op_code, self.lowered.desc, in0, in1, out, config=cfg,
-                                          number=number, repeat=repeat, min_repeat_ms=min_repeat_ms,
-                                          add=picked[3] if len(picked) > 3 else None))
+            secs = ops.time_op(self.lowered.op_code, self.lowered.desc, in0, in1, out, config=cfg,
+                               number=number, repeat=repeat, min_repeat_ms=min_repeat_ms,
+                               add=picked[3] if len(picked) > 3 else None)
+            # the stages materialised in front of an operand run on every call: their time counts
+            for pos, (g, buf) in self._gathers.items():
+                extra = g.time(picked[pos].contiguous(), buf, number=number, repeat=repeat, min_repeat_ms=min_repeat_ms)
+                secs = [a + b for a, b in zip(secs, extra)]
+            return TimeResult(secs)
         return evaluator
 
     def get_source(self):

@@ -33,6 +33,36 @@ int set_error(int code, const char* fmt, ...) {
       return set_error(AMOS_ERR_HIP, "%s failed: %s", #expr, hipGetErrorString(e_));    \
   } while (0)
 
+// out[o] = in[sum_d tab_d[o_d]] where all table entries are >= 0 (else 0); five dimensions,
+// the innermost fastest, unused leading ones of extent 1
+struct GatherParams {
+  int shape[5];
+  int use[5];
+  int64_t tab[5];
+  int64_t total, in_elems;
+};
+template <typename T>
+__global__ __launch_bounds__(256) void amos_gather_kernel(const GatherParams g, const T* __restrict__ in,
+                                                         const int* __restrict__ tables, T* __restrict__ out) {
+  for (int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x; idx < g.total; idx += (int64_t)gridDim.x * 256) {
+    int64_t rest = idx, off = 0;
+    bool ok = true;
+#pragma unroll
+    for (int k = 4; k >= 0; --k) {
+      const int64_t q = rest / g.shape[k];
+      const int o = (int)(rest - q * g.shape[k]);
+      rest = q;
+      if (g.use[k]) {
+        const int e = tables[g.tab[k] + o];
+        ok = ok && e >= 0;
+        off += e;
+      }
+    }
+    ok = ok && off < g.in_elems;
+    out[idx] = ok ? in[off] : (T)0;
+  }
+}
+
 template <typename T>
 __global__ void fill_zero_kernel(T* p, int64_t rows, int64_t cols, int64_t ld) {
   int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -557,6 +587,88 @@ static int run_op(int op, const void* desc, const amos_kernel_config_t* cfg, con
 
 using namespace amos;
 
+static int launch_gather(const amos_gather_desc_t* d, const void* in, const int32_t* tables, void* out,
+                         hipStream_t stream) {
+  if (!d || !in || !tables || !out) return set_error(AMOS_ERR_BAD_ARG, "null pointer argument");
+  if (d->ndim < 1 || d->ndim > 5) return set_error(AMOS_ERR_BAD_ARG, "gather of %d dimensions", d->ndim);
+  if (d->elem_bytes != 1 && d->elem_bytes != 2 && d->elem_bytes != 4)
+    return set_error(AMOS_ERR_UNSUPPORTED, "gather of %d-byte elements", d->elem_bytes);
+  GatherParams g;
+  memset(&g, 0, sizeof(g));
+  int64_t total = 1;
+  for (int k = 0; k < 5; ++k) {   // right-aligned: unused leading dimensions have extent 1
+    const int src = k - (5 - d->ndim);
+    g.shape[k] = 1;
+    g.tab[k] = 0;
+    g.use[k] = 0;
+    if (src >= 0) {
+      if (d->out_shape[src] <= 0 || d->out_shape[src] >= (1ll << 31) || d->table_offset[src] < 0)
+        return set_error(AMOS_ERR_BAD_ARG, "gather extent or table offset out of range");
+      g.shape[k] = (int)d->out_shape[src];
+      g.tab[k] = d->table_offset[src];
+      g.use[k] = 1;
+      total *= d->out_shape[src];
+    }
+  }
+  if (total >= (1ll << 40) || d->in_elems <= 0 || d->in_elems >= (1ll << 31))
+    return set_error(AMOS_ERR_UNSUPPORTED, "gather size out of range");
+  g.total = total;
+  g.in_elems = d->in_elems;
+  const int64_t want = (total + 255) / 256;
+  const int blocks = (int)(want < 65536 ? want : 65536);
+  if (d->elem_bytes == 1)
+    hipLaunchKernelGGL(amos_gather_kernel<unsigned char>, dim3(blocks), dim3(256), 0, stream, g,
+                       (const unsigned char*)in, tables, (unsigned char*)out);
+  else if (d->elem_bytes == 2)
+    hipLaunchKernelGGL(amos_gather_kernel<unsigned short>, dim3(blocks), dim3(256), 0, stream, g,
+                       (const unsigned short*)in, tables, (unsigned short*)out);
+  else
+    hipLaunchKernelGGL(amos_gather_kernel<unsigned>, dim3(blocks), dim3(256), 0, stream, g, (const unsigned*)in,
+                       tables, (unsigned*)out);
+  HIP_TRY(hipGetLastError());
+  return 0;
+}
+
+// time_evaluator's loop (src/runtime/rpc/rpc_module.cc:355-388) around a launch
+template <typename Launch>
+static int time_launches(Launch launch_once, hipStream_t stream, int number, int repeat, int min_repeat_ms,
+                         double* out_seconds) {
+  int rc = launch_once();  // warm-up
+  if (rc) return rc;
+  HIP_TRY(hipStreamSynchronize(stream));
+  hipEvent_t e0, e1;
+  HIP_TRY(hipEventCreate(&e0));
+  HIP_TRY(hipEventCreate(&e1));
+  long long n = number;  // like the reference, a grown `number` carries over to later repeats
+  for (int r = 0; r < repeat; ++r) {
+    double ms = 0.0;
+    for (;;) {
+      if (ms > 0.0) {
+        double want = (double)min_repeat_ms / (ms / (double)n) + 1.0;
+        double grown = (double)n * 1.618;
+        double nn = want > grown ? want : grown;
+        if (nn > 1e8) nn = 1e8;
+        n = (long long)nn;
+      }
+      HIP_TRY(hipEventRecord(e0, stream));
+      for (long long i = 0; i < n; ++i) {
+        rc = launch_once();
+        if (rc) return rc;
+      }
+      HIP_TRY(hipEventRecord(e1, stream));
+      HIP_TRY(hipEventSynchronize(e1));
+      float f = 0.f;
+      HIP_TRY(hipEventElapsedTime(&f, e0, e1));
+      ms = f;
+      if (ms >= (double)min_repeat_ms || n >= 100000000LL) break;
+    }
+    out_seconds[r] = ms * 1e-3 / (double)n;
+  }
+  (void)hipEventDestroy(e0);
+  (void)hipEventDestroy(e1);
+  return 0;
+}
+
 extern "C" {
 
 int amos_version(void) { return AMOS_ABI_VERSION; }
@@ -636,6 +748,20 @@ const char* amos_kernel_name(int op, const void* desc, const amos_kernel_config_
   return inst->name;
 }
 
+int amos_gather(const amos_gather_desc_t* desc, const void* in, const int32_t* tables, void* out,
+                void* stream) {
+  return launch_gather(desc, in, tables, out, (hipStream_t)stream);
+}
+
+int amos_time_gather(const amos_gather_desc_t* desc, const void* in, const int32_t* tables, void* out,
+                     void* stream_v, int number, int repeat, int min_repeat_ms, double* out_seconds) {
+  if (!out_seconds || number < 1 || repeat < 1)
+    return set_error(AMOS_ERR_BAD_ARG, "amos_time_gather needs number >= 1, repeat >= 1 and an output array");
+  hipStream_t stream = (hipStream_t)stream_v;
+  return time_launches([&] { return launch_gather(desc, in, tables, out, stream); }, stream, number, repeat,
+                       min_repeat_ms, out_seconds);
+}
+
 int amos_time(int op, const void* desc, const amos_kernel_config_t* cfg, const void* in0,
               const void* in1, void* out, void* workspace, size_t ws_bytes, void* stream_v,
               int number, int repeat, int min_repeat_ms, double* out_seconds) {
@@ -655,40 +781,7 @@ int amos_time_fused(int op, const void* desc, const amos_kernel_config_t* cfg,
   if (rc) return rc;
   rc = plan_epilogue(pl, op, desc, epilogue);
   if (rc) return rc;
-  rc = launch(pl, stream);  // warm-up
-  if (rc) return rc;
-  HIP_TRY(hipStreamSynchronize(stream));
-  hipEvent_t e0, e1;
-  HIP_TRY(hipEventCreate(&e0));
-  HIP_TRY(hipEventCreate(&e1));
-  long long n = number;  // like the reference, a grown `number` carries over to later repeats
-  for (int r = 0; r < repeat; ++r) {
-    double ms = 0.0;
-    for (;;) {
-      if (ms > 0.0) {
-        double want = (double)min_repeat_ms / (ms / (double)n) + 1.0;
-        double grown = (double)n * 1.618;
-        double nn = want > grown ? want : grown;
-        if (nn > 1e8) nn = 1e8;
-        n = (long long)nn;
-      }
-      HIP_TRY(hipEventRecord(e0, stream));
-      for (long long i = 0; i < n; ++i) {
-        rc = launch(pl, stream);
-        if (rc) return rc;
-      }
-      HIP_TRY(hipEventRecord(e1, stream));
-      HIP_TRY(hipEventSynchronize(e1));
-      float f = 0.f;
-      HIP_TRY(hipEventElapsedTime(&f, e0, e1));
-      ms = f;
-      if (ms >= (double)min_repeat_ms || n >= 100000000LL) break;
-    }
-    out_seconds[r] = ms * 1e-3 / (double)n;
-  }
-  (void)hipEventDestroy(e0);
-  (void)hipEventDestroy(e1);
-  return 0;
+  return time_launches([&] { return launch(pl, stream); }, stream, number, repeat, min_repeat_ms, out_seconds);
 }
 
 }  // extern "C"

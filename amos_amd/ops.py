@@ -241,6 +241,49 @@ def conv3d(x, w, stride=1, pad=0, dil=1, out=None, config=None, stream=None, add
     return out
 
 
+class Gather(object):
+    """device side of a dimension-separable gather (amos_gather): `tables[d][o]` = source element
+    offset contributed by index o of output dimension d, or -1 where the result is zero"""
+
+    def __init__(self, out_shape, tables, dtype, in_elems, device):
+        self.out_shape = [int(e) for e in out_shape]
+        self.dtype = dtype
+        if not 1 <= len(self.out_shape) <= 5 or [len(t) for t in tables] != self.out_shape:
+            raise ValueError("gather needs one table per output dimension, at most five")
+        flat, offsets = [], []
+        for t in tables:
+            offsets.append(len(flat))
+            flat.extend(int(e) for e in t)
+        self.tables = torch.tensor(flat, dtype=torch.int32, device=device)
+        d = _lib.GatherDesc()
+        d.ndim, d.elem_bytes, d.in_elems = len(self.out_shape), torch.empty(0, dtype=dtype).element_size(), int(in_elems)
+        for k, (ext, off) in enumerate(zip(self.out_shape, offsets)):
+            d.out_shape[k], d.table_offset[k] = ext, off
+        self.desc = d
+
+    def _check(self, src, out):
+        _need_device(src, out)
+        if src.numel() != self.desc.in_elems or src.dtype != self.dtype or not src.is_contiguous():
+            raise ValueError("gather source must be a dense %s tensor of %d elements" % (self.dtype, self.desc.in_elems))
+        if list(out.shape) != self.out_shape or out.dtype != self.dtype or not out.is_contiguous():
+            raise ValueError("gather output must be a dense %s tensor of shape %s" % (self.dtype, self.out_shape))
+
+    def __call__(self, src, out=None, stream=None):
+        if out is None:
+            out = torch.empty(self.out_shape, dtype=self.dtype, device=src.device)
+        self._check(src, out)
+        check(_lib.load().amos_gather(ctypes.byref(self.desc), src.data_ptr(), self.tables.data_ptr(),
+                                      out.data_ptr(), _stream_ptr(stream)))
+        return out
+
+    def time(self, src, out, number=100, repeat=1, min_repeat_ms=150, stream=None):
+        self._check(src, out)
+        res = (ctypes.c_double * repeat)()
+        check(_lib.load().amos_time_gather(ctypes.byref(self.desc), src.data_ptr(), self.tables.data_ptr(),
+                                           out.data_ptr(), _stream_ptr(stream), number, repeat, min_repeat_ms, res))
+        return list(res)
+
+
 def _epilogue_for(op, desc, add, out):
     """Epilogue for an operand laid out like the output the descriptor describes"""
     if add is None:

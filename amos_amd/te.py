@@ -43,6 +43,9 @@ class Expr(object):
     def __le__(self, o): return Cmp("<=", self, const_like(o, self))
     def __lt__(self, o): return Cmp("<", self, const_like(o, self))
     def equal(self, o): return Cmp("==", self, const_like(o, self))
+    # `a == b` builds the comparison, as in TVM; asked for its truth value (tuple, set and dict
+    # comparisons do) it answers whether both sides are the same object
+    def __eq__(self, o): return _EqCmp(self, const_like(o, self))
 
     def astype(self, dtype):
         return self if dtype == self.dtype else Cast(dtype, self)
@@ -146,6 +149,14 @@ class Cmp(Expr):
         self.dtype = "bool"
 
     def __repr__(self): return "(%r %s %r)" % (self.a, self.op, self.b)
+
+
+class _EqCmp(Cmp):
+    def __init__(self, a, b):
+        Cmp.__init__(self, "==", a, b)
+
+    def __bool__(self):
+        return self.a is self.b
 
 
 class And(Expr):
@@ -358,6 +369,8 @@ class _Tir(object):
 
 
 tir = _Tir()
+if_then_else = tir.if_then_else
+globals()["all"] = tir.all      # te.all(...), as tvm.te.all
 
 
 # ---- affine views of index expressions -------------------------------------------------------

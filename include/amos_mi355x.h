@@ -230,6 +230,31 @@ int amos_time_fused(int op, const void* desc, const amos_kernel_config_t* cfg,
                     void* workspace, size_t ws_bytes, void* stream, int number, int repeat,
                     int min_repeat_ms, double* out_seconds);
 
+/*
+ * Dimension-separable gather:  out[o0, ..., o(n-1)] = in[ sum_d table_d[o_d] ]  where every
+ * table_d[o_d] >= 0, else 0 (out dense, row-major).  It materialises the stages the reference
+ * computes in front of an operand and that are not folded into a kernel's loader -- the zero
+ * expansion and one-sided padding of a transposed convolution's input, its flipped and
+ * transposed weights (benchmark/amos/mapping_transposedconv2d_tensorcore.py:7-102) -- as TVM's
+ * default schedule would, each stage at root.  `tables` is device memory: for dimension d,
+ * out_shape[d] entries from tables[table_offset[d]], each the source element offset that index
+ * contributes (index * stride of the source dimension it maps to) or -1 where the stage's
+ * predicate is false.  Sums that fall outside [0, in_elems) read as 0.
+ */
+typedef struct {
+  int32_t ndim;             /* 1..5 */
+  int32_t elem_bytes;       /* 1, 2 or 4 */
+  int64_t out_shape[5];
+  int64_t table_offset[5];
+  int64_t in_elems;
+} amos_gather_desc_t;
+
+int amos_gather(const amos_gather_desc_t* desc, const void* in, const int32_t* tables, void* out,
+                void* stream);
+/* amos_time's loop around amos_gather */
+int amos_time_gather(const amos_gather_desc_t* desc, const void* in, const int32_t* tables, void* out,
+                     void* stream, int number, int repeat, int min_repeat_ms, double* out_seconds);
+
 /* name of the kernel instance a (desc, cfg) pair dispatches to, e.g.
  * "amos_igemm<f16,vec,vec,256x256>"; replaces func.imported_modules[0].get_source()
  * as the way to see what was chosen (reference: README.md:340). */

@@ -10,7 +10,7 @@ import amos_amd.tvm as tvm
 from amos_amd.tvm import auto_tensorize as at
 from oracle import cpu_oracle as co
 from test_mapper import (batched_fc, conv1d, conv2d, conv2d_layout, depthwise_conv2d, from_nkpq, gemm, gemv,
-                         grouped_conv2d, grouped_conv_reference, to_nchw)
+                         grouped_conv2d, grouped_conv_reference, to_nchw, transposed_conv2d)
 
 pytestmark = pytest.mark.gpu
 
@@ -216,6 +216,60 @@ def test_conv2d_layout_script_flow(gpu, tmp_path, layout, C):
                                   dilation, acc="float64"), layout)
     mx, mean = co.rel_errors(got, ref)
     assert got.shape == ref.shape and mx <= 1e-2 and mean <= 1e-3
+
+
+@pytest.mark.parametrize("dtype", ["float16", "int8", "float32"])
+def test_gather_entry_point(gpu, dtype):
+    """amos_gather against numpy: a padded, zero-expanded, flipped and transposed view"""
+    import torch
+    from amos_amd import ops
+    from amos_amd.auto_tensorize.measure import _TORCH_DTYPE
+    rng = np.random.default_rng(5)
+    src = (rng.integers(-100, 100, (3, 5, 6, 7))).astype(dtype)
+    # out[a, b, c, d] = src[b, a, 5 - (c - 2) / 2, d - 1] where c - 2 is even and in range, 0 <= d - 1 < 7
+    strides = [5 * 6 * 7, 6 * 7, 7, 1]
+    tables = [[i * strides[1] for i in range(5)], [i * strides[0] for i in range(3)],
+              [(5 - (c - 2) // 2) * strides[2] if (c - 2) % 2 == 0 and 0 <= (c - 2) // 2 < 6 else -1 for c in range(15)],
+              [(d - 1) * strides[3] if 0 <= d - 1 < 7 else -1 for d in range(10)]]
+    want = np.zeros((5, 3, 15, 10), dtype=src.dtype)
+    for c in range(15):
+        for d in range(10):
+            if tables[2][c] >= 0 and tables[3][d] >= 0:
+                want[:, :, c, d] = src[:, :, 5 - (c - 2) // 2, d - 1].T
+    g = ops.Gather([5, 3, 15, 10], tables, _TORCH_DTYPE[dtype], src.size, torch.device("cuda", 0))
+    got = g(torch.from_numpy(src).cuda())
+    assert np.array_equal(got.cpu().numpy(), want)
+    secs = g.time(torch.from_numpy(src).cuda(), got, number=3, repeat=2, min_repeat_ms=1)
+    assert len(secs) == 2 and all(0 < t < 1e-2 for t in secs)
+
+
+@pytest.mark.parametrize("case", [(2, 48, 14, 14, 64, 4, 2, 1, 0, 1), (1, 24, 9, 11, 40, 3, 2, 1, 1, 1),
+                                  (3, 64, 8, 8, 64, 3, 1, 1, 0, 2)])
+def test_transposed_conv_script_flow(gpu, tmp_path, case):
+    """reference compute: benchmark/amos/mapping_transposedconv2d_tensorcore.py:55-102; against the
+    scatter definition of a transposed convolution in double precision"""
+    import torch
+    N, C, H, W, K, ks, stride, padding, output_padding, dilation = case
+    A, B, Out = transposed_conv2d(N, C, H, W, K, ks, stride, padding, output_padding, dilation)
+    rng = np.random.default_rng(8)
+    a = rng.uniform(-1, 1, (N, K, H, W)).astype(np.float16)
+    b = rng.uniform(-1, 1, (K, C, ks, ks)).astype(np.float16)
+    got, result = _run_script_flow([A, B, Out], {"A": a, "B": b}, tmp_path, "tconv")
+    low = result.sch_app.lowered
+    assert low.kind == "conv2d" and sorted(low.gathers) == [0, 1]
+    ref = torch.nn.functional.conv_transpose2d(torch.from_numpy(a).double(), torch.from_numpy(b).double(),
+                                               stride=stride, padding=padding, output_padding=output_padding,
+                                               dilation=dilation).numpy()
+    mx, mean = co.rel_errors(got, ref)
+    assert got.shape == ref.shape and mx <= 1e-2 and mean <= 1e-3
+    # the module's timing covers the materialised stages as well
+    sch, args = at.get_schedule(result.sch_app, result.params)
+    func = tvm.build(sch, args, "hip")
+    ctx = tvm.context("hip", 0)
+    arrs = [tvm.nd.array(a, ctx), tvm.nd.array(b, ctx), tvm.nd.array(np.zeros(ref.shape, dtype=np.float32), ctx)]
+    t = func.time_evaluator(func.entry_name, ctx, number=3, min_repeat_ms=2)(*arrs).mean
+    mx2, _ = co.rel_errors(arrs[2].asnumpy(), ref)     # (a split-K configuration sums in any order)
+    assert 0 < t < 1e-2 and mx2 <= 1e-2
 
 
 @pytest.mark.parametrize("kind", ["grouped", "depthwise"])

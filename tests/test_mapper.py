@@ -296,6 +296,83 @@ def test_lowered_conv2d_layouts_mean_what_the_compute_says(case, layout):
     assert np.array_equal(from_nkpq(got, layout), want)
 
 
+def transposed_conv2d(N, C, H, W, K, kernel_size, stride, padding, output_padding, dilation,
+                      in_dtype="float16", out_dtype="float32", exact_int=False):
+    """the reference's transposed convolution: zero expansion, one-sided padding, a stride-1
+    convolution with the window flipped (benchmark/amos/mapping_transposedconv2d_tensorcore.py:7-102)"""
+    A = te.placeholder([N, K, H, W], dtype=in_dtype, name="A")
+    B = te.placeholder([K, C, kernel_size, kernel_size], dtype=in_dtype, name="B")
+    k_h = k_w = kernel_size
+    He, We = (H - 1) * stride + 1, (W - 1) * stride + 1
+    expanded = te.compute([N, K, He, We], lambda b, c, h, w: te.if_then_else(
+        te.all(h % stride == 0, w % stride == 0), A[b, c, h // stride, w // stride], tir.const(0, in_dtype)),
+        name="expanded")
+    kernel_h, kernel_w = (k_h - 1) * dilation + 1, (k_w - 1) * dilation + 1
+    p0, p1 = kernel_h - 1 - padding, kernel_h - 1 - padding + output_padding
+    q0, q1 = kernel_w - 1 - padding, kernel_w - 1 - padding + output_padding
+    padded = te.compute([N, K, He + p0 + p1, We + q0 + q1], lambda b, c, h, w: te.if_then_else(
+        te.all(h >= p0, h < He + p0, w >= q0, w < We + q0), expanded[b, c, h - p0, w - q0], tir.const(0, in_dtype)),
+        name="Padding")
+    out_h = (H - 1) * stride - 2 * padding + kernel_h + output_padding
+    out_w = (W - 1) * stride - 2 * padding + kernel_w + output_padding
+    rc = te.reduce_axis((0, K), name="rc")
+    rh = te.reduce_axis((0, k_h), name="rh")
+    rw = te.reduce_axis((0, k_w), name="rw")
+
+    def body(b, c, h, w):
+        x, wt = padded[b, rc, h + rh * dilation, w + rw * dilation], B[rc, c, k_h - rh - 1, k_w - rw - 1]
+        prod = x.astype(out_dtype) * wt.astype(out_dtype) if exact_int else (x * wt).astype(out_dtype)
+        return te.sum(prod, axis=[rc, rw, rh])
+
+    output = te.compute((N, C, out_h, out_w), body, name="output")
+    return [A, B, output]
+
+
+def apply_view(view, src):
+    """numpy meaning of a lowering.OperandView"""
+    off = np.zeros(view.shape, dtype=np.int64)
+    ok = np.ones(view.shape, dtype=bool)
+    for d, table in enumerate(view.tables):
+        t = np.asarray(table, dtype=np.int64).reshape([-1 if k == d else 1 for k in range(len(view.shape))])
+        ok &= t >= 0
+        off += np.maximum(t, 0)
+    return np.where(ok, src.reshape(-1)[off], 0).astype(src.dtype)
+
+
+TRANSPOSED_CASES = [(2, 3, 5, 4, 6, 3, 2, 1, 1, 1), (1, 4, 6, 6, 2, 4, 2, 1, 0, 1), (1, 2, 4, 5, 3, 3, 1, 0, 0, 2),
+                    (2, 2, 3, 3, 2, 2, 3, 0, 2, 1)]
+
+
+@pytest.mark.parametrize("case", TRANSPOSED_CASES)
+def test_transposed_conv_lowers_to_gathers_and_a_convolution(case):
+    N, C, H, W, K, ks, st, pd, opd, dl = case
+    A, B, Out = transposed_conv2d(N, C, H, W, K, ks, st, pd, opd, dl, "int8", "int32", exact_int=True)
+    assert len(at.get_match_results(at.compute_dag_from_tensors([Out]), "hip")) > 0
+    low = at.lower_main_op(Out.op)
+    assert low.kind == "conv2d" and sorted(low.gathers) == [0, 1] and [t.name for t in low.inputs] == ["A", "B"]
+    assert low.attrs["stride"] == [1, 1] and low.attrs["pad"] == [0, 0] and low.attrs["dil"] == [dl, dl]
+    rng = np.random.default_rng(4)
+    a = rng.integers(-9, 10, (N, K, H, W)).astype(np.int8)
+    b = rng.integers(-9, 10, (K, C, ks, ks)).astype(np.int8)
+    want = te_interp.evaluate(Out, {"A": a, "B": b})
+    x, w = apply_view(low.gathers[0], a), apply_view(low.gathers[1], b)
+    assert w.shape == (C, K, ks, ks) and np.array_equal(w, np.transpose(b, (1, 0, 2, 3))[:, :, ::-1, ::-1])
+    got = co.te_literal_conv2d(x, w, "int8", [1, 1], [0, 0], [dl, dl], mode="exact")
+    assert np.array_equal(got, want)
+    # and the textbook definition: scatter every input element times the window into the output
+    ref = np.zeros(want.shape, dtype=np.int64)
+    for n in range(N):
+        for k in range(K):
+            for h in range(H):
+                for ww in range(W):
+                    for r in range(ks):
+                        for s_ in range(ks):
+                            oh, ow = h * st - pd + r * dl, ww * st - pd + s_ * dl
+                            if 0 <= oh < ref.shape[2] and 0 <= ow < ref.shape[3]:
+                                ref[n, :, oh, ow] += int(a[n, k, h, ww]) * b[k, :, r, s_].astype(np.int64)
+    assert np.array_equal(ref, want)
+
+
 def test_no_kernel_for_other_layouts():
     # NHWC activations match the intrinsic but have no kernel
     N, H, W, C, K = 2, 6, 6, 8, 8
