@@ -31,6 +31,8 @@ class LoweredOp(object):
         # {0 or 1: OperandView}: the kernel does not read inputs[k] itself but a tensor gathered
         # from it (stages in front of the operand that no loader folds in), materialised per call
         self.gathers = {}
+        # {0 or 1: numpy array}: inputs[k] is computed from its indices alone; the module holds it
+        self.constants = {}
 
     def flops(self):
         a = self.attrs
@@ -110,7 +112,9 @@ def _vars_in(e, out):
 
 def _index_tables(indices, variables, extents, src_shape, cond=None):
     """for a load `src[indices]` under `cond`, with every index and every term of the condition a
-    function of one variable: {position of the variable: (source dimension, [source index or -1])}"""
+    function of at most one variable: per variable a list, over its values, of
+    {source dimension: index} (None where the condition fails or an index leaves the source);
+    indices without a variable come back as a second dictionary"""
     ids = [id(v) for v in variables]
     terms = []
     if cond is not None:
@@ -123,24 +127,35 @@ def _index_tables(indices, variables, extents, src_shape, cond=None):
         term_var.append(ids.index(vs[0]) if vs else None)
     if any(tv is None and not _eval_int(t, {}) for t, tv in zip(terms, term_var)):
         raise _NotSeparable("constant false condition")
-    stage = {}
+    index_var, fixed = [], {}
     for k, idx in enumerate(indices):
         vs = [v for v in _vars_in(idx, {}) if v in ids]
-        if len(vs) != 1:
+        if len(vs) > 1:
             raise _NotSeparable("an index of %d variables" % len(vs))
-        d = ids.index(vs[0])
-        if d in stage:
-            raise _NotSeparable("one variable in two indices")
-        table = []
+        index_var.append(ids.index(vs[0]) if vs else None)
+        if not vs:
+            fixed[k] = _eval_int(idx, {})
+            if not 0 <= fixed[k] < int(src_shape[k]):
+                raise _NotSeparable("constant index outside the source")
+    stage = []
+    for d in range(len(variables)):
+        column = []
         for v in range(extents[d]):
             env = {ids[d]: v}
-            ok = all(_eval_int(t, env) for t, tv in zip(terms, term_var) if tv == d)
-            x = _eval_int(idx, env)
-            table.append(x if ok and 0 <= x < int(src_shape[k]) else -1)
-        stage[d] = (k, table)
-    if len(stage) != len(variables):
-        raise _NotSeparable("an index variable that selects nothing")
-    return stage
+            entry = {}
+            if not all(_eval_int(t, env) for t, tv in zip(terms, term_var) if tv == d):
+                entry = None
+            else:
+                for k, idx in enumerate(indices):
+                    if index_var[k] == d:
+                        x = _eval_int(idx, env)
+                        if not 0 <= x < int(src_shape[k]):
+                            entry = None
+                            break
+                        entry[k] = x
+            column.append(entry)
+        stage.append(column)
+    return stage, fixed
 
 
 def _operand_view(tensor, head=None):
@@ -150,11 +165,10 @@ def _operand_view(tensor, head=None):
     try:
         if head is not None:
             shape, variables, indices = head
-            stage = _index_tables(indices, variables, shape, tensor.shape)
-            view = [stage[d] for d in range(len(shape))]
+            view, fixed = _index_tables(indices, variables, shape, tensor.shape)
         else:
             shape = [int(s) for s in tensor.shape]
-            view = [(d, list(range(shape[d]))) for d in range(len(shape))]
+            view, fixed = [[{d: o} for o in range(shape[d])] for d in range(len(shape))], {}
         cur = tensor
         while not isinstance(cur.op, te.PlaceholderOp):
             op = cur.op
@@ -168,18 +182,97 @@ def _operand_view(tensor, head=None):
                 body, cond = body.then_value, body.cond
             if not isinstance(body, te.ProducerLoad) or body.dtype != cur.dtype:
                 raise _NotSeparable("stage %s computes" % op.name)
-            stage = _index_tables(body.indices, [iv.var for iv in op.axis],
-                                  [int(iv.dom.extent) for iv in op.axis], body.tensor.shape, cond)
-            view = [(stage[cd][0], [stage[cd][1][i] if i >= 0 else -1 for i in idxs]) for cd, idxs in view]
+            stage, sfixed = _index_tables(body.indices, [iv.var for iv in op.axis],
+                                          [int(iv.dom.extent) for iv in op.axis], body.tensor.shape, cond)
+
+            def through(entry):
+                """coordinates in `cur` -> coordinates in the tensor the stage reads"""
+                if entry is None:
+                    return None
+                out = {}
+                for cd, i in entry.items():
+                    e = stage[cd][i]
+                    if e is None:
+                        return None
+                    out.update(e)
+                return out
+
+            # (coordinates of `cur` fixed by an outer stage go through this stage as well)
+            passed = through(fixed)
+            if passed is None:
+                raise _NotSeparable("a constant index selects a zero")
+            view = [[through(e) for e in column] for column in view]
+            fixed = dict(sfixed)
+            fixed.update(passed)
             cur = body.tensor
-        if sorted(cd for cd, _ in view) != list(range(len(cur.shape))):
-            raise _NotSeparable("dimensions of the source are merged or dropped")
+        ndim = len(cur.shape)
+        owner = {}
+        for d, column in enumerate(view):
+            for e in column:
+                for k in (e or {}):
+                    if owner.setdefault(k, d) != d:
+                        raise _NotSeparable("a source dimension addressed from two dimensions")
+        if sorted(list(owner) + list(fixed)) != list(range(ndim)):
+            raise _NotSeparable("a source dimension is not addressed")
     except _NotSeparable as e:
         raise NoKernelError("operand %s is not a per-dimension rearrangement of a placeholder: %s"
                             % (tensor.name, e))
     strides = _row_major_strides([int(s) for s in cur.shape])
-    tables = [[i * strides[cd] if i >= 0 else -1 for i in idxs] for cd, idxs in view]
+    base = sum(i * strides[k] for k, i in fixed.items())
+    tables = [[sum(i * strides[k] for k, i in e.items()) if e is not None else -1 for e in column]
+              for column in view]
+    # the constant part of the address rides on the first dimension's entries
+    tables[0] = [t + base if t >= 0 else -1 for t in tables[0]]
     return OperandView(cur, shape, tables, cur.dtype)
+
+
+def _eval_array(e, env):
+    """numpy value of an index-only expression over the index grids in `env`"""
+    import numpy as np
+    if isinstance(e, (te.IntImm, te.FloatImm)):
+        return np.asarray(e.value)
+    if isinstance(e, te.Var):
+        if id(e) not in env:
+            raise _NotSeparable("free variable %s" % e.name)
+        return env[id(e)]
+    if isinstance(e, te.Cast):
+        return _eval_array(e.value, env)
+    if isinstance(e, te.And):
+        out = np.asarray(True)
+        for t in e.terms:
+            out = np.logical_and(out, _eval_array(t, env))
+        return out
+    if isinstance(e, te.Select):
+        return np.where(_eval_array(e.cond, env), _eval_array(e.then_value, env), _eval_array(e.else_value, env))
+    if isinstance(e, te.Cmp):
+        a, b = _eval_array(e.a, env), _eval_array(e.b, env)
+        return {"==": a == b, ">=": a >= b, ">": a > b, "<=": a <= b, "<": a < b, "!=": a != b}[e.op]
+    if isinstance(e, (te.Add, te.Sub, te.Mul, te.FloorDiv, te.FloorMod)):
+        a, b = _eval_array(e.a, env), _eval_array(e.b, env)
+        if isinstance(e, te.Add): return a + b
+        if isinstance(e, te.Sub): return a - b
+        if isinstance(e, te.Mul): return a * b
+        return a // b if isinstance(e, te.FloorDiv) else a % b
+    raise _NotSeparable("expression %r" % (e,))
+
+
+def _constant_operand(tensor):
+    """host array of a tensor computed from its indices alone (the reference's vector of
+    1/n in benchmark/amos/mapping_mean_tensorcore.py:14-16, the triangle of ones in
+    mapping_scan_tensorcore.py:9-15), or None"""
+    import numpy as np
+    op = tensor.op
+    if not isinstance(op, te.ComputeOp) or op.reduce_axis or te.collect_loads(op.body[0]):
+        return None
+    shape = [int(s) for s in tensor.shape]
+    grids = np.meshgrid(*[np.arange(n) for n in shape], indexing="ij") if shape else []
+    try:
+        val = _eval_array(op.body[0], {id(iv.var): g for iv, g in zip(op.axis, grids)})
+    except _NotSeparable:
+        return None
+    if tensor.dtype == "bfloat16":
+        raise NoKernelError("constant bfloat16 operands have no host form")
+    return np.ascontiguousarray(np.broadcast_to(val, shape).astype(tensor.dtype))
 
 
 def _strip_cast(e):
@@ -238,8 +331,18 @@ def _lower_gemm(main_op, l0, l1, iters, forms0, forms1):
         return None
     if not (has(da, k) and has(db, k)):
         return None
-    if not (isinstance(la.tensor.op, te.PlaceholderOp) and isinstance(lb.tensor.op, te.PlaceholderOp)):
-        raise NoKernelError("GEMM operands must be placeholders")
+    # an operand that is computed: a constant (a function of its indices), or a per-dimension
+    # rearrangement of a placeholder that is materialised in front of the kernel
+    sources, gathers, constants = [la.tensor, lb.tensor], {}, {}
+    for pos, ld in enumerate((la, lb)):
+        if isinstance(ld.tensor.op, te.PlaceholderOp):
+            continue
+        const = _constant_operand(ld.tensor)
+        if const is not None:
+            constants[pos] = const
+        else:
+            gathers[pos] = _operand_view(ld.tensor)
+            sources[pos] = gathers[pos].src
     trans_a = 0 if da[0] is x else 1          # [x, k] row-major A, [k, x] transposed
     trans_b = 0 if db[0] is k else 1          # [k, y] row-major B, [y, k] column-major B
     M, N, K = int(x.dom.extent), int(y.dom.extent), int(k.dom.extent)
@@ -249,13 +352,16 @@ def _lower_gemm(main_op, l0, l1, iters, forms0, forms1):
     g.lda, g.ldb, g.ldc = (M if trans_a else K), (K if trans_b else N), N
     attrs = dict(M=M, N=N, K=K, trans_a=trans_a, trans_b=trans_b, dtype=la.dtype)
     if batch is None:
-        return LoweredOp("gemm", _lib.AMOS_OP_GEMM, g, [la.tensor, lb.tensor], main_op.output(0), attrs)
-    b = _lib.BGemmDesc()
-    b.batch = int(batch.dom.extent)
-    b.g = g
-    b.stride_a, b.stride_b, b.stride_c = M * K, K * N, M * N
-    attrs["batch"] = b.batch
-    return LoweredOp("bgemm", _lib.AMOS_OP_BGEMM, b, [la.tensor, lb.tensor], main_op.output(0), attrs)
+        low = LoweredOp("gemm", _lib.AMOS_OP_GEMM, g, sources, main_op.output(0), attrs)
+    else:
+        b = _lib.BGemmDesc()
+        b.batch = int(batch.dom.extent)
+        b.g = g
+        b.stride_a, b.stride_b, b.stride_c = M * K, K * N, M * N
+        attrs["batch"] = b.batch
+        low = LoweredOp("bgemm", _lib.AMOS_OP_BGEMM, b, sources, main_op.output(0), attrs)
+    low.gathers, low.constants = gathers, constants
+    return low
 
 
 def _row_major_strides(shape):

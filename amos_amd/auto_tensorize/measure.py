@@ -51,6 +51,8 @@ def random_device_arrays(lowered, dev_id=0, seed=0):
             arrays.append(torch.randint(-128, 128, shape, dtype=torch.int8, device=dev, generator=gen))
         else:
             arrays.append((torch.rand(shape, device=dev, generator=gen) * 2 - 1).to(_TORCH_DTYPE[t.dtype]))
+    for pos, const in getattr(lowered, "constants", {}).items():
+        arrays[pos] = torch.from_numpy(const).to(dev)
     out = torch.empty([int(s) for s in lowered.output.shape], dtype=_TORCH_DTYPE[lowered.output.dtype], device=dev)
     return arrays[0], arrays[1], out
 

@@ -81,15 +81,18 @@ class Module(object):
         self.params = params
         # positions of (in0, in1, out[, added tensor of a fused tail]) among the caller's arguments
         ids = [id(t) for t in arg_tensors]
+        consts = getattr(lowered, "constants", {})
         try:
-            self.arg_index = [ids.index(id(lowered.inputs[0])), ids.index(id(lowered.inputs[1])),
-                              ids.index(id(lowered.output))]
+            # (an operand computed from its indices alone is held by the module, not passed)
+            self.arg_index = [None if k in consts else ids.index(id(lowered.inputs[k])) for k in (0, 1)]
+            self.arg_index.append(ids.index(id(lowered.output)))
             if getattr(lowered, "add_input", None) is not None:
                 self.arg_index.append(ids.index(id(lowered.add_input)))
         except ValueError:
             raise ValueError("build() args must hold the compute's inputs and its output tensor")
         self.imported_modules = [_Source(self)]
         self._gathers = {}     # operand position -> (ops.Gather, materialised operand), made on first use
+        self._constants = {}   # operand position -> device tensor of a constant operand
 
     def _kernel_inputs(self, in0, in1):
         """the operands the kernel reads: the caller's arrays, or what the stages in front of an
@@ -104,10 +107,18 @@ class Module(object):
         return ins
 
     def _pick(self, arrays):
-        if len(arrays) <= max(self.arg_index):
-            raise ValueError("expected %d arrays (inputs + outputs)" % (max(self.arg_index) + 1))
+        need = max(i for i in self.arg_index if i is not None)
+        if len(arrays) <= need:
+            raise ValueError("expected %d arrays (inputs + outputs)" % (need + 1))
         out = []
-        for i in self.arg_index:
+        for k, i in enumerate(self.arg_index):
+            if i is None:
+                if k not in self._constants:
+                    dev = [a for a in arrays if isinstance(a, (NDArray, torch.Tensor))][0]
+                    dev = (dev.tensor if isinstance(dev, NDArray) else dev).device
+                    self._constants[k] = torch.from_numpy(self.lowered.constants[k]).to(dev)
+                out.append(self._constants[k])
+                continue
             a = arrays[i]
             out.append(a.tensor if isinstance(a, NDArray) else a)
         return out

@@ -10,7 +10,7 @@ import amos_amd.tvm as tvm
 from amos_amd.tvm import auto_tensorize as at
 from oracle import cpu_oracle as co
 from test_mapper import (batched_fc, conv1d, conv2d, conv2d_layout, depthwise_conv2d, from_nkpq, gemm, gemv,
-                         grouped_conv2d, grouped_conv_reference, to_nchw, transposed_conv2d)
+                         grouped_conv2d, grouped_conv_reference, mean, scan, to_nchw, transposed_conv2d)
 
 pytestmark = pytest.mark.gpu
 
@@ -270,6 +270,28 @@ def test_transposed_conv_script_flow(gpu, tmp_path, case):
     t = func.time_evaluator(func.entry_name, ctx, number=3, min_repeat_ms=2)(*arrs).mean
     mx2, _ = co.rel_errors(arrs[2].asnumpy(), ref)     # (a split-K configuration sums in any order)
     assert 0 < t < 1e-2 and mx2 <= 1e-2
+
+
+def test_mean_and_scan_script_flows(gpu, tmp_path):
+    """reference computes: benchmark/amos/mapping_mean_tensorcore.py:7-25 (a GEMM whose left
+    operand is a gathered view and whose right operand is a constant vector; like the GEMV its
+    N = 1 needs transform_strict=False) and mapping_scan_tensorcore.py:7-21 (prefix sums as a
+    GEMM with a constant triangle of ones)"""
+    rng = np.random.default_rng(10)
+    N, C, H, W = 8, 96, 14, 14
+    A, B, E = mean(N, C, H, W)
+    a = rng.uniform(-1, 1, (N, C, H, W)).astype(np.float16)
+    got, result = _run_script_flow([A, B, E], {"A": a}, tmp_path, "mean", transform_strict=False)
+    low = result.sch_app.lowered
+    assert low.kind == "gemm" and list(low.gathers) == [0] and list(low.constants) == [1]
+    ref = (a.astype(np.float64) * float(np.float16(1.0 / (N * H * W)))).sum(axis=(0, 2, 3))
+    assert got.shape == (C,) and np.abs(got - ref).max() <= 1e-2 * np.abs(ref).max() + 1e-4
+    M, Nn, K = 300, 256, 256
+    A, B, Cc = scan(M, Nn, K)
+    a = rng.integers(-3, 4, (M, K)).astype(np.float16)
+    got, result = _run_script_flow([A, B, Cc], {"A": a}, tmp_path, "scan")
+    assert list(result.sch_app.lowered.constants) == [1]
+    assert np.array_equal(got, np.cumsum(a.astype(np.float32), axis=1))     # small integers: exact
 
 
 @pytest.mark.parametrize("kind", ["grouped", "depthwise"])

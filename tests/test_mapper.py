@@ -373,6 +373,55 @@ def test_transposed_conv_lowers_to_gathers_and_a_convolution(case):
     assert np.array_equal(ref, want)
 
 
+def mean(N, C, H, W, in_dtype="float16", out_dtype="float32"):
+    """reference: benchmark/amos/mapping_mean_tensorcore.py:7-25"""
+    A = te.placeholder([N, C, H, W], dtype=in_dtype, name="A")
+    B = te.compute([C, N * H * W], lambda i, j: A[j // (H * W), i, j % (H * W) // W, j % W], name="B")
+    C_ = te.compute([N * H * W, 1], lambda i, j: tir.const(1.0 / (N * H * W), in_dtype), name="C")
+    rk = te.reduce_axis([0, N * H * W], name="k")
+    D = te.compute([C, 1], lambda i, j: te.sum((B[i, rk] * C_[rk, j]).astype(out_dtype), axis=rk), name="D")
+    E = te.compute([C], lambda i: D[i, 0], name="E")
+    return [A, B, E]
+
+
+def scan(M, N, K, in_dtype="float16", out_dtype="float32"):
+    """reference: benchmark/amos/mapping_scan_tensorcore.py:7-21"""
+    A = te.placeholder([M, K], dtype=in_dtype, name="A")
+    B = te.compute([K, N], lambda i, j: tir.if_then_else(i > j, tir.const(0.0, in_dtype), tir.const(1.0, "float16")),
+                   name="B")
+    rk = te.reduce_axis([0, K], name="k")
+    C = te.compute([M, N], lambda i, j: te.sum((A[i, rk] * B[rk, j]).astype(out_dtype), axis=rk), name="C")
+    return [A, B, C]
+
+
+def test_mean_and_scan_lower_to_gemm_with_computed_operands():
+    rng = np.random.default_rng(6)
+    # mean: the [C, N*H*W] view of A is gathered, the vector of 1/n is a constant
+    N, C, H, W = 2, 5, 3, 4
+    A, B, E = mean(N, C, H, W)
+    dag = at.compute_dag_from_tensors([E])
+    low = at.lower_main_op([op for op in dag.op_lst if op.reduce_axis][0], dag)
+    assert low.kind == "gemm" and (low.attrs["M"], low.attrs["N"], low.attrs["K"]) == (C, 1, N * H * W)
+    assert list(low.gathers) == [0] and list(low.constants) == [1] and low.output is E
+    a = rng.uniform(-1, 1, (N, C, H, W)).astype(np.float16)
+    b = apply_view(low.gathers[0], a)
+    assert np.array_equal(b, np.transpose(a, (1, 0, 2, 3)).reshape(C, -1))
+    assert np.array_equal(low.constants[1], np.full((N * H * W, 1), np.float16(1.0 / (N * H * W))))
+    want = te_interp.evaluate(E, {"A": a})
+    got = co.te_literal_gemm(b, low.constants[1], "float16").reshape(-1)
+    # (the loop nest rounds every product to fp16, the interpreter does not)
+    assert np.allclose(got, want, atol=1e-3) and np.allclose(want, a.astype(np.float64).mean(axis=(0, 2, 3)), atol=2e-3)
+    # scan: the triangle of ones is a constant; row i of the result = prefix sums of row i of A
+    M, Nn, K = 6, 7, 7
+    A, B, Cc = scan(M, Nn, K)
+    low = at.lower_main_op(Cc.op)
+    assert low.kind == "gemm" and not low.gathers and list(low.constants) == [1]
+    assert np.array_equal(low.constants[1], np.triu(np.ones((K, Nn), dtype=np.float16)))
+    a = rng.integers(-4, 5, (M, K)).astype(np.float16)
+    want = te_interp.evaluate(Cc, {"A": a})
+    assert np.array_equal(want, np.cumsum(a.astype(np.float32), axis=1))
+
+
 def test_no_kernel_for_other_layouts():
     # NHWC activations match the intrinsic but have no kernel
     N, H, W, C, K = 2, 6, 6, 8, 8
