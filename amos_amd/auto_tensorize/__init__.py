@@ -14,3 +14,5 @@ from .target import MI355X, get_device_arch  # noqa: F401
 from .runtime import build, array, context, Module, NDArray  # noqa: F401
 from .auto_tensorize import (AutoTensorizeResult, auto_tensorize, auto_tensorize_compute,  # noqa: F401
                              auto_tensorize_schedule, auto_tensorize_v4, get_schedule)
+from .network import (AutoScheduleMultiGraphDispatch, AutoTensorizeContext, SubGraph, evaluate_graph,  # noqa: F401
+                      resnet18)
