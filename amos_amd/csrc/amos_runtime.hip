@@ -218,12 +218,14 @@ static int plan_gemm(Plan& pl, int op, const void* desc_any, const amos_gemm_des
                      256 * d->ldb * es + 128 < ((int64_t)1 << 32);
   const int pipe = pl.cfg.pipeline;
   if (pipe == AMOS_PIPE_DIRECT4 || pipe == AMOS_PIPE_DIRECT8) {
-    if (!tn_ok || pl.cfg.tile_i != 256 || pl.cfg.tile_j != 256)
+    const int waves = pipe == AMOS_PIPE_DIRECT4 ? 4 : 8;
+    if (!tn_ok || !pick_gemm_tn(pl.dt, pl.cfg.tile_i, pl.cfg.tile_j, waves))
       return set_error(AMOS_ERR_INFEASIBLE,
                        "direct-to-LDS pipeline needs K-contiguous 16-byte aligned operands, "
-                       "K %% %d == 0, tile 256x256 and split_k 1", bke);
-    pl.tn_waves = pipe == AMOS_PIPE_DIRECT4 ? 4 : 8;
-  } else if (pipe == AMOS_PIPE_AUTO && tn_ok && pl.cfg.tile_i == 256 && pl.cfg.tile_j == 256) {
+                       "K %% %d == 0, split_k 1 and a tile of 256x256 (4 or 8 waves), 128x128, "
+                       "128x256 or 256x128 (8 waves)", bke);
+    pl.tn_waves = waves;
+  } else if (pipe == AMOS_PIPE_AUTO && tn_ok && pick_gemm_tn(pl.dt, pl.cfg.tile_i, pl.cfg.tile_j, 8)) {
     pl.tn_waves = 8;  // measured a few percent ahead of 4 waves on the 8192^3 fp16 GEMM
   }
   if (pl.tn_waves) {
@@ -459,7 +461,7 @@ static int resolve(const Plan& pl, Instance** out) {
 }
 
 static int launch_tn(const Plan& pl, hipStream_t stream) {
-  TnInstance* inst = pick_gemm_tn(pl.dt, pl.tn_waves);
+  TnInstance* inst = pick_gemm_tn(pl.dt, pl.cfg.tile_i, pl.cfg.tile_j, pl.tn_waves);
   if (!inst) return set_error(AMOS_ERR_INFEASIBLE, "no direct-to-LDS instance");
   hipError_t attr_err = hipSuccess;
   std::call_once(inst->once, [&] {
@@ -740,7 +742,7 @@ const char* amos_kernel_name(int op, const void* desc, const amos_kernel_config_
     return ci ? ci->name : nullptr;
   }
   if (pl.tn_waves) {
-    TnInstance* tn = pick_gemm_tn(pl.dt, pl.tn_waves);
+    TnInstance* tn = pick_gemm_tn(pl.dt, pl.cfg.tile_i, pl.cfg.tile_j, pl.tn_waves);
     return tn ? tn->name : nullptr;
   }
   Instance* inst;

@@ -1,16 +1,20 @@
 // GEMM / batched GEMM with both operands K-contiguous ("ntn": A[M,K], B stored [N,K]),
 // the layout v_mfma wants: every lane's operand fragment is 16 contiguous bytes of K.
 //
-// Block tile 256x256, K step 128 bytes per row (64 halves / 128 int8), two LDS
-// stages of 64 KB.  Differences to the generic implicit-GEMM kernel:
+// Block tile BI x BJ (256x256 for large problems; 128x128, 128x256, 256x128 where those fill
+// the chip better), K step 128 bytes per row (64 halves / 128 int8), NS LDS stages of
+// (BI + BJ) * 128 bytes (two for 256x256; the smaller tiles, whose workgroups are often alone on
+// a CU, keep three or four tiles in flight).  Differences to the generic implicit-GEMM kernel:
 //   * global -> LDS copies are direct (global_load_lds_dwordx4): no staging
 //     registers, no ds_write; the XOR swizzle of the LDS layout is applied on the
 //     global-address side (a wave instruction fills 1 KB of LDS linearly, lane l
 //     fetches the 16-byte chunk that belongs at that position);
 //   * operand fragments are double buffered in registers: the ds_reads of K
 //     sub-step s+1 are in flight while the MFMAs of sub-step s issue;
-//   * one barrier per K step; the copies for step kt+2 are issued right after it and
-//     have a whole step to land.
+//   * one barrier per K step; the copies for step kt+NS are issued right after it and
+//     have NS-1 steps to land.  Every step issues a tile (steps past the end fetch the last
+//     one again), so that the number of copies in flight behind the tile a step waits for
+//     is the same at every step.
 // Rows beyond M / N are clamped to the last valid row on load (their products only
 // reach outputs that are never stored); K must be a multiple of the K step.
 //
@@ -40,7 +44,7 @@ struct GemmTnParams {
 #define AMOS_GLOBAL_PTR(p) ((const __attribute__((address_space(1))) void*)(p))
 #define AMOS_LDS_PTR(p) ((__attribute__((address_space(3))) void*)(p))
 
-template <int DT, int WI, int WJ>
+template <int DT, int WI, int WJ, int BI = 256, int BJ = 256, int NS = 2>
 __global__ __launch_bounds__(64 * WI * WJ) void amos_gemm_tn(const GemmTnParams p) {
   typedef Mfma<DT> MM;
   typedef typename MM::acc_t acc_t;
@@ -48,10 +52,13 @@ __global__ __launch_bounds__(64 * WI * WJ) void amos_gemm_tn(const GemmTnParams 
   constexpr int ES = MM::ES;
   constexpr int BKE = 128 / ES;
   constexpr int NW = WI * WJ;
-  constexpr int TI = 256 / (32 * WI), TJ = 256 / (32 * WJ);
-  constexpr int OPER = 256 * 128;      // bytes of one operand tile
-  constexpr int STAGE = 2 * OPER;      // A tile then B tile
-  constexpr int CH = 64 / NW;          // 1 KB copy chunks per wave per K step
+  constexpr int TI = BI / (32 * WI), TJ = BJ / (32 * WJ);
+  static_assert(TI >= 1 && TJ >= 1 && TI * WI * 32 == BI && TJ * WJ * 32 == BJ, "wave tile");
+  constexpr int OPER = BI * 128;       // bytes of the A tile; the B tile follows it
+  constexpr int STAGE = (BI + BJ) * 128;
+  constexpr int QA = BI / 8;           // 1 KB copy chunks (8 rows) of the A tile
+  constexpr int CH = (BI + BJ) / 8 / NW;   // copy chunks per wave per K step
+  static_assert(CH >= 1 && CH * NW * 8 == BI + BJ, "copy chunks");
 
   extern __shared__ __attribute__((aligned(16))) char smem[];
 
@@ -62,20 +69,20 @@ __global__ __launch_bounds__(64 * WI * WJ) void amos_gemm_tn(const GemmTnParams 
 
   int tile_i, tile_j;
   block_to_tile(blockIdx.x, gridDim.x, p.tiles_i, p.tiles_j, tile_i, tile_j);
-  const int bi0 = tile_i * 256, bj0 = tile_j * 256;
+  const int bi0 = tile_i * BI, bj0 = tile_j * BJ;
   const int64_t batch = blockIdx.z;
   const char* const abase = p.a + (batch * p.batch_a + (int64_t)bi0 * p.lda) * ES;
   const char* const bbase = p.b + (batch * p.batch_b + (int64_t)bj0 * p.ldb) * ES;
 
-  // ---- copy slots: chunk q of this wave covers tile rows [8*qq, 8*qq+8) of A (q < 32) or B
+  // ---- copy slots: chunk q of this wave covers tile rows [8*qq, 8*qq+8) of A (q < BI/8) or B
   unsigned g_off[CH];   // byte offset from the operand's tile base, K step 0
 #pragma unroll
   for (int u = 0; u < CH; ++u) {
-    const int q = wave + NW * u;       // 0..63, uniform per wave
-    const int qq = q & 31;
+    const int q = wave + NW * u;       // uniform per wave
+    const int qq = q < QA ? q : q - QA;
     const int row = qq * 8 + (lane >> 3);
     const int chunk = (lane & 7) ^ ((row ^ (row >> 3)) & 7);
-    if (q < 32) {
+    if (q < QA) {
       int r = bi0 + row < p.I ? row : p.I - 1 - bi0;
       g_off[u] = (unsigned)r * (unsigned)(p.lda * ES) + chunk * 16;
     } else {
@@ -91,7 +98,7 @@ __global__ __launch_bounds__(64 * WI * WJ) void amos_gemm_tn(const GemmTnParams 
 #pragma unroll
     for (int u = 0; u < CH; ++u) {
       const int q = wave + NW * u;
-      const char* src = (q < 32 ? ak : bk) + g_off[u];
+      const char* src = (q < QA ? ak : bk) + g_off[u];
       __builtin_amdgcn_global_load_lds(AMOS_GLOBAL_PTR(src), AMOS_LDS_PTR(s + q * 1024), 16, 0, 0);
     }
   };
@@ -133,15 +140,16 @@ __global__ __launch_bounds__(64 * WI * WJ) void amos_gemm_tn(const GemmTnParams 
   };
 
   const int KT = p.K / BKE;
-  issue_copies(0, 0);
-  if (KT > 1) issue_copies(1, 1);
-  // stage 0 must have landed; stage 1 may still be in flight, but a counter wait cannot
-  // tell them apart cheaply here, so wait for both once
-  asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");
+  static_assert(NS >= 2 && (NS - 1) * CH <= 63, "stages");
+#pragma unroll
+  for (int s = 0; s < NS; ++s) issue_copies(s < KT ? s : KT - 1, s);
+  // tile 0 has landed once at most the NS-1 younger tiles are in flight (copies complete in order)
+  asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"((NS - 1) * CH) : "memory");
   read_frags(0, 0, 0);
 
+  int st = 0;   // stage of tile kt
   for (int kt = 0; kt < KT; ++kt) {
-    const int st = kt & 1;
+    const int st_next = st + 1 == NS ? 0 : st + 1;
     read_frags(st, 1, 1);
     mma(0);
     read_frags(st, 2, 0);
@@ -149,12 +157,14 @@ __global__ __launch_bounds__(64 * WI * WJ) void amos_gemm_tn(const GemmTnParams 
     read_frags(st, 3, 1);
     mma(0);
     // every ds_read of this stage has been issued; once they and this wave's copies of the
-    // other stage are complete, meet the other waves: after the barrier the other stage
-    // is fully written and this stage is free to be overwritten
-    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
-    if (kt + 2 < KT) issue_copies(kt + 2, st);
-    if (kt + 1 < KT) read_frags(st ^ 1, 0, 0);
+    // next tile are complete (the NS-2 tiles behind it may still be in flight), meet the other
+    // waves: after the barrier the next stage is fully written and this stage is free to be
+    // overwritten
+    asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"((NS - 2) * CH) : "memory");
+    issue_copies(kt + NS < KT ? kt + NS : KT - 1, st);
+    if (kt + 1 < KT) read_frags(st_next, 0, 0);
     mma(1);
+    st = st_next;
   }
 
   // ---- epilogue ---------------------------------------------------------------------
@@ -182,6 +192,8 @@ __global__ __launch_bounds__(64 * WI * WJ) void amos_gemm_tn(const GemmTnParams 
       }
     }
   }
+  // the tiles fetched again by the last steps still target this block's LDS
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 }
 
 }  // namespace amos

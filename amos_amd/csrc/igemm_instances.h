@@ -74,8 +74,9 @@ struct TnInstance {
   const char* name;
   std::once_flag once;
 };
-// direct-to-LDS GEMM (defined in inst_gemm_tn.hip); waves = 4 or 8
-TnInstance* pick_gemm_tn(int dt, int waves);
+// direct-to-LDS GEMM (defined in inst_gemm_tn.hip); 256x256 with 4 or 8 waves, 128x128 / 128x256 /
+// 256x128 with 8
+TnInstance* pick_gemm_tn(int dt, int ti, int tj, int waves);
 
 // patch-staged convolution (defined in inst_conv_*.hip)
 struct ConvFpropParams;

@@ -309,7 +309,9 @@ static const TileCost kTileCost[] = {
     {256, 256, 1, 2.45, 2.75}, {256, 128, 1, 1.38, 1.55}, {128, 256, 1, 1.46, 1.65},
     {128, 128, 2, 0.654, 1.03}, {256, 64, 1, 1.09, 1.17}, {128, 64, 3, 0.394, 0.69},
     {64, 128, 3, 0.403, 0.69},  {64, 64, 4, 0.24, 0.50},  {64, 256, 1, 1.26, 1.22}};
-static const TileCost kDirectCost = {256, 256, 1, 1.95, 1.65};   // amos_gemm_tn, 8 waves
+// amos_gemm_tn (direct-to-LDS copies, 8 waves)
+static const TileCost kDirectCost[] = {
+    {256, 256, 1, 1.85, 1.65}, {128, 256, 1, 1.06, 0.95}, {256, 128, 1, 1.05, 0.92}, {128, 128, 2, 0.56, 0.70}};
 
 static double loader_factor(int loader) {
   switch (loader) {
@@ -326,8 +328,10 @@ static double estimate_seconds(const Problem& pb, int ti, int tj, int split, boo
   for (auto& t : kTileCost)
     if (t.ti == ti && t.tj == tj) tc = &t;
   if (!tc) return 1e9;
-  const bool direct = allow_direct && pb.direct_ok && ti == 256 && tj == 256 && split == 1;
-  if (direct) tc = &kDirectCost;
+  bool direct = false;
+  if (allow_direct && pb.direct_ok && split == 1)
+    for (auto& t : kDirectCost)
+      if (t.ti == ti && t.tj == tj) { tc = &t; direct = true; }
   const double k_tiles = std::ceil((double)pb.K / (128.0 / es));
   const int eff_split = (int)std::min<double>(split, k_tiles);
   const double ksteps = std::ceil(k_tiles / eff_split);
@@ -451,7 +455,7 @@ int amos_default_config(int op, const void* desc, amos_kernel_config_t* result) 
     for (auto& t : kTiles) {
       for (int split = 1; split <= 4; split *= 2) {
         const double s = conv_patch_estimate(c, op, pb, t[0], t[1], split);
-        if (s > 0 && s < best * 0.98) {
+        if (s > 0 && s < best * 0.995) {
           best = s;
           out->tile_i = t[0];
           out->tile_j = t[1];
@@ -470,7 +474,7 @@ int amos_default_config(int op, const void* desc, amos_kernel_config_t* result) 
     for (int split = 1; split <= 16; split *= 2) {
       if (split > 1 && (split > k_tiles / 2 || pb.batch > 1)) break;
       double s = estimate_seconds(pb, t[0], t[1], split);
-      if (s < best * 0.98) {
+      if (s < best * 0.995) {
         best = s;
         out->tile_i = t[0];
         out->tile_j = t[1];

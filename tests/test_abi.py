@@ -92,8 +92,15 @@ def test_default_config_is_a_compiled_instance():
 def test_kernel_name_reflects_layout():
     lib = _lib.load()
     cfg = _lib.KernelConfig(128, 128, 1)
+    # aligned K-contiguous operands: the direct-to-LDS kernel where it has the tile, else (or on
+    # request) the register-staged one
     assert lib.amos_kernel_name(0, ctypes.byref(gemm_desc(256, 256, 256, tb=1)), ctypes.byref(cfg)) == \
+        b"amos_gemm_tn<f16,128x128,8w>"
+    staged = _lib.KernelConfig(128, 128, 1, _lib.AMOS_PIPE_STAGED)
+    assert lib.amos_kernel_name(0, ctypes.byref(gemm_desc(256, 256, 256, tb=1)), ctypes.byref(staged)) == \
         b"amos_igemm<f16,vec,vec,128x128>"
+    assert lib.amos_kernel_name(0, ctypes.byref(gemm_desc(256, 256, 256, tb=1)),
+                                ctypes.byref(_lib.KernelConfig(128, 64, 1))) == b"amos_igemm<f16,vec,vec,128x64>"
     # row-major B: rows (n) contiguous, vector loads transposed in registers ...
     assert lib.amos_kernel_name(0, ctypes.byref(gemm_desc(256, 256, 256)), ctypes.byref(cfg)) == \
         b"amos_igemm<f16,vec,tvec,128x128>"

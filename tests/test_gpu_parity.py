@@ -86,20 +86,23 @@ def test_gemm_every_tile(gpu, dtype, tile, split):
 
 
 @pytest.mark.parametrize("dtype", ["float16", "bfloat16", "int8"])
-@pytest.mark.parametrize("pipeline", [2, 3])   # direct-to-LDS copies, 4 and 8 waves
+# direct-to-LDS copies: 256x256 with 4 and 8 waves, the smaller tiles (two and three LDS stages) with 8
+@pytest.mark.parametrize("pipeline,tile", [(2, (256, 256)), (3, (256, 256)), (3, (128, 128)), (3, (128, 256)),
+                                           (3, (256, 128)), (0, (128, 128))])
 @pytest.mark.parametrize("shape", [(256, 256, 128), (512, 768, 1024), (300, 520, 384), (1, 257, 128)])
-def test_gemm_direct_pipeline(gpu, dtype, pipeline, shape):
+def test_gemm_direct_pipeline(gpu, dtype, pipeline, tile, shape):
     from amos_amd import _lib, ops
     M, N, K = shape
     rng = np.random.default_rng(M * 7 + N * 3 + K)
     a = make_operand(rng, (M, K), dtype)
     b = make_operand(rng, (N, K), dtype)
-    cfg = dict(tile_i=256, tile_j=256, split_k=1, pipeline=pipeline)
+    cfg = dict(tile_i=tile[0], tile_j=tile[1], split_k=1, pipeline=pipeline)
     d = ops.gemm_desc(M, N, K, to_device(a, dtype).dtype, False, True)
-    assert "amos_gemm_tn" in ops.kernel_name(_lib.AMOS_OP_GEMM, d, cfg)
+    assert "amos_gemm_tn<%s,%dx%d" % ({"float16": "f16", "bfloat16": "bf16", "int8": "i8"}[dtype], tile[0], tile[1]) \
+        in ops.kernel_name(_lib.AMOS_OP_GEMM, d, cfg)
     got = ops.gemm(to_device(a, dtype), to_device(b, dtype), False, True, config=cfg).cpu().numpy()
     check(got, co.lib_gemm(a, b, dtype, False, True, acc="float64"), dtype,
-          "direct gemm %s pipe %d %s" % (dtype, pipeline, shape))
+          "direct gemm %s pipe %d tile %s %s" % (dtype, pipeline, tile, shape))
     # batched through the same kernel
     ab = make_operand(rng, (3, M, K), dtype)
     bb = make_operand(rng, (3, N, K), dtype)
