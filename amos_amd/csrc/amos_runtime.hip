@@ -283,6 +283,32 @@ static int plan_conv(Plan& pl, int op, const amos_conv_desc_t* d, const amos_ker
     return set_error(AMOS_ERR_UNSUPPORTED, "conv extents above 2^31");
   if ((c.T - 1) * c.dil_d >= 1024 || (c.R - 1) * c.dil_h >= 1024 || (c.S - 1) * c.dil_w >= 1024)
     return set_error(AMOS_ERR_UNSUPPORTED, "dilated kernel extent above 1023");
+  // A 1x1(x1) window with unit stride and no padding is a matrix product as it stands:
+  // per image Y[K][DHW] = Wt[K][C] X[C][DHW] (NCDHW), or Y[NDHW][K] = X[NDHW][C] Wt[C][K]
+  // (channels innermost).  It runs on the GEMM kernels, vector loaders included, unless the
+  // patch-staged pipeline is asked for.
+  if (c.T == 1 && c.R == 1 && c.S == 1 && c.stride_d == 1 && c.stride_h == 1 && c.stride_w == 1 &&
+      c.pad_d == 0 && c.pad_h == 0 && c.pad_w == 0 && G == 1 &&
+      (!cfg || (cfg->pipeline != AMOS_PIPE_PATCH && cfg->pipeline != AMOS_PIPE_PATCH8))) {
+    const int64_t dhw = c.D * c.H * c.W;
+    amos_bgemm_desc_t b;
+    memset(&b, 0, sizeof(b));
+    b.g.in_dtype = c.in_dtype;
+    b.g.out_dtype = c.out_dtype;
+    b.g.K = c.C;
+    if (layout == AMOS_LAYOUT_NCHW) {
+      b.batch = c.N;
+      b.g.M = c.K; b.g.N = dhw;
+      b.g.lda = c.C; b.g.ldb = dhw; b.g.ldc = dhw;
+      b.stride_a = 0; b.stride_b = c.C * dhw; b.stride_c = c.K * dhw;
+      return plan_gemm(pl, AMOS_OP_BGEMM, &b, &b.g, b.batch, b.stride_a, b.stride_b, b.stride_c, cfg, Wt, X, Y);
+    }
+    b.batch = 1;
+    b.g.M = c.N * dhw; b.g.N = c.K;
+    b.g.lda = c.C; b.g.ldb = c.K; b.g.ldc = c.K;
+    b.stride_a = b.g.M * c.C; b.stride_b = c.C * c.K; b.stride_c = b.g.M * c.K;
+    return plan_gemm(pl, AMOS_OP_BGEMM, &b, &b.g, 1, b.stride_a, b.stride_b, b.stride_c, cfg, X, Wt, Y);
+  }
   const int es = pl.dt == DT_I8 ? 1 : 2;
   const int ce = 16 / es;
   IgemmParams& p = pl.p;

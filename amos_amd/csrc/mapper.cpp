@@ -80,6 +80,20 @@ int problem_of(int op, const void* desc, Problem* out) {
       out->out_bytes = c->K * out->J * 4;
       out->row_loader = (c->layout == AMOS_LAYOUT_NCHW && out->K % (16 / esize(c->in_dtype)) == 0) ? 0 : 1;
       out->col_loader = 2;
+      // a pointwise convolution runs as a (batched) matrix product: the activations' rows are the
+      // contiguous direction (NCDHW), or both operands go through vector loaders
+      if (T == 1 && c->R == 1 && c->S == 1 && c->stride_h == 1 && c->stride_w == 1 && c->pad_h == 0 &&
+          c->pad_w == 0 && (op == AMOS_OP_CONV2D || (c->stride_d == 1 && c->pad_d == 0)) && G == 1) {
+        const bool wide = esize(c->in_dtype) == 2;
+        if (c->layout == AMOS_LAYOUT_NCHW) {
+          out->col_loader = (wide && (D * c->H * c->W) % 8 == 0 && out->row_loader == 0) ? 3 : 1;
+          if (out->col_loader == 1) out->row_loader = 1;
+        } else {
+          const bool vec = c->C % (16 / esize(c->in_dtype)) == 0;
+          out->row_loader = (wide && c->K % 8 == 0 && vec) ? 3 : 1;
+          out->col_loader = (vec && out->row_loader == 3) ? 0 : 1;
+        }
+      }
       return 0;
     }
   }
@@ -304,14 +318,18 @@ static int64_t acc_regs_of(int ti, int tj) { return (int64_t)(ti / 2) * (tj / 2)
 //     the busiest CU has ceil(workgroups / CUs) of them, at most occ(tile) at a time;
 //   * operands that are not loaded as 16-byte vectors along K slow both constants down;
 //   * split-K adds the zero fill and the atomic read-modify-writes of the output.
-struct TileCost { int ti, tj, occ; double tau_us, alone_us; };
+//   * a round of workgroups has a fixed cost (prologue, the stores of the accumulators), large for
+//     the 256x256 tile of the register-staged kernel (256 scattered stores per lane from four
+//     waves per CU: 83 us for a 256 x 50176 x 64 product against 16 us with 128x64 tiles);
+struct TileCost { int ti, tj, occ; double tau_us, alone_us, fixed_us; };
 static const TileCost kTileCost[] = {
-    {256, 256, 1, 2.45, 2.75}, {256, 128, 1, 1.38, 1.55}, {128, 256, 1, 1.46, 1.65},
-    {128, 128, 2, 0.654, 1.03}, {256, 64, 1, 1.09, 1.17}, {128, 64, 3, 0.394, 0.69},
-    {64, 128, 3, 0.403, 0.69},  {64, 64, 4, 0.24, 0.50},  {64, 256, 1, 1.26, 1.22}};
+    {256, 256, 1, 2.45, 2.75, 70.0}, {256, 128, 1, 1.38, 1.55, 8.0}, {128, 256, 1, 1.46, 1.65, 8.0},
+    {128, 128, 2, 0.654, 1.03, 2.0}, {256, 64, 1, 1.09, 1.17, 4.0}, {128, 64, 3, 0.394, 0.69, 1.0},
+    {64, 128, 3, 0.403, 0.69, 1.0},  {64, 64, 4, 0.24, 0.50, 0.5},  {64, 256, 1, 1.26, 1.22, 4.0}};
 // amos_gemm_tn (direct-to-LDS copies, 8 waves)
 static const TileCost kDirectCost[] = {
-    {256, 256, 1, 1.85, 1.65}, {128, 256, 1, 1.06, 0.95}, {256, 128, 1, 1.05, 0.92}, {128, 128, 2, 0.56, 0.70}};
+    {256, 256, 1, 1.85, 1.65, 4.0}, {128, 256, 1, 1.06, 0.95, 2.0}, {256, 128, 1, 1.05, 0.92, 2.0},
+    {128, 128, 2, 0.56, 0.70, 1.0}};
 
 static double loader_factor(int loader) {
   switch (loader) {
@@ -342,7 +360,8 @@ static double estimate_seconds(const Problem& pb, int ti, int tj, int split, boo
   const int64_t groups = per_cu / tc->occ, rest = per_cu % tc->occ;
   double step_us = (double)groups * std::max(alone, tc->occ * tau);
   if (rest) step_us += std::max(alone, (double)rest * tau);
-  double t = 3e-6 + ksteps * step_us * 1e-6;
+  const double rounds = (double)groups + (rest ? 1.0 : 0.0);
+  double t = 3e-6 + (ksteps * step_us + rounds * tc->fixed_us) * 1e-6;
   // output: written once; a split-K launch zero-fills it and accumulates with atomics (measured:
   // (1 + 2*split) passes over the output at ~3.5 TB/s)
   if (eff_split > 1) t += (double)pb.out_bytes * (1.0 + 2.0 * eff_split) / 3.5e12;

@@ -375,6 +375,37 @@ def test_conv_tile_walk_channel_innermost(gpu, layout):
         check((outs[(0, False)] - d_add).cpu().numpy(), refs, "float16", "walk + D %s tile %s" % (layout, tile))
 
 
+@pytest.mark.parametrize("layout", ["nchw", "nhwc", "hwnc"])
+@pytest.mark.parametrize("dtype", ["float16", "int8"])
+@pytest.mark.parametrize("case", [(3, 64, 1, 9, 8, 40), (2, 24, 1, 7, 5, 33), (2, 128, 3, 6, 4, 72)])
+def test_pointwise_conv_runs_as_gemm(gpu, layout, dtype, case):
+    """1x1(x1) windows, unit stride, no padding: the (batched) GEMM kernels, no im2col gather"""
+    import torch
+    from amos_amd import _lib, ops
+    N, C, D, H, W, K = case
+    rng = np.random.default_rng(21)
+    x = make_operand(rng, (N, C, D, H, W), dtype, "normal")
+    w = make_operand(rng, (K, C, 1, 1, 1), dtype, "normal")
+    ref = co.lib_conv3d(x, w, dtype, (1, 1, 1), (0, 0, 0), (1, 1, 1), acc="float64")
+    to_x = {"nchw": (0, 1, 2, 3, 4), "nhwc": (0, 2, 3, 4, 1), "hwnc": (2, 3, 4, 0, 1)}[layout]
+    xs = np.ascontiguousarray(np.transpose(x, to_x))
+    ws_ = np.ascontiguousarray(w if layout == "nchw" else np.transpose(w, (2, 3, 4, 1, 0)))
+    refs = np.ascontiguousarray(np.transpose(ref, to_x))
+    lay3 = {"nchw": "ncdhw", "nhwc": "ndhwc", "hwnc": "dhwnc"}[layout]
+    desc = ops.conv_desc((N, C, D, H, W), (K, C, 1, 1, 1), to_device(xs, dtype).dtype, (1, 1, 1), (0, 0, 0), (1, 1, 1),
+                         1, lay3)
+    name = ops.kernel_name(_lib.AMOS_OP_CONV3D, desc, None)
+    assert "im2col" not in name and "conv_fprop" not in name, name
+    d_add = torch.randn(refs.shape, device="cuda").to(torch.int32 if dtype == "int8" else torch.float32)
+    dx, dw = to_device(xs, dtype), to_device(ws_, dtype)
+    for cfg in (None, dict(tile_i=64, tile_j=64, split_k=2), dict(tile_i=128, tile_j=128, split_k=1)):
+        for add in (None, d_add):
+            got = ops.conv3d(dx, dw, 1, 0, 1, config=cfg, add=add, layout=lay3)
+            assert tuple(got.shape) == refs.shape
+            check((got if add is None else got - add).cpu().numpy(), refs, dtype,
+                  "pointwise %s %s %s cfg %s add %s" % (layout, dtype, case, cfg, add is not None))
+
+
 LAYOUT_CASES = [
     # N, C, D, H, W, K, T, R, S, stride, pad, dil
     (3, 24, 1, 9, 7, 40, 1, 3, 3, (1, 1, 1), (0, 1, 1), (1, 1, 1)),      # register-staged kernel only
