@@ -63,6 +63,60 @@ __global__ __launch_bounds__(256) void amos_gather_kernel(const GatherParams g, 
   }
 }
 
+// dst[b][c][r] = src[b][r][c] for r < rows, c < cols (src rows ld_src apart, dst dense): an
+// operand whose rows are the contiguous direction becomes K-contiguous.  64 x 64 tiles through
+// LDS, 8 bytes per lane on both sides where alignment allows.
+struct TransposeJob {
+  const char* src;
+  char* dst;
+  int rows, cols;
+  int64_t ld_src, batch_src, batch_dst;
+  int batch;
+};
+template <typename T>
+__global__ __launch_bounds__(256) void amos_transpose_kernel(const TransposeJob j) {
+  constexpr int VE = 8 / (int)sizeof(T);      // elements per 8-byte access
+  constexpr int PITCH = 64 + VE;              // LDS row in elements (keeps 8-byte alignment)
+  __shared__ __attribute__((aligned(16))) T tile[64 * PITCH];
+  const int t = threadIdx.x;
+  const int c0 = blockIdx.x * 64, r0 = blockIdx.y * 64;
+  const T* src = (const T*)j.src + (int64_t)blockIdx.z * j.batch_src;
+  T* dst = (T*)j.dst + (int64_t)blockIdx.z * j.batch_dst;
+  constexpr int LT = 64 / VE;                 // threads per 64-element row
+  constexpr int RPP = 256 / LT;               // rows per pass
+  const bool vec_in = (((uintptr_t)src | (uintptr_t)(j.ld_src * sizeof(T))) & 7) == 0;
+  const int lc = (t % LT) * VE, lr = t / LT;
+#pragma unroll
+  for (int pass = 0; pass < 64 / RPP; ++pass) {
+    const int r = lr + pass * RPP;
+    const int gr = r0 + r, gc = c0 + lc;
+    T v[VE];
+    if (gr < j.rows && vec_in && gc + VE <= j.cols) {
+      *(uint2*)v = *(const uint2*)(src + (int64_t)gr * j.ld_src + gc);
+    } else {
+#pragma unroll
+      for (int e = 0; e < VE; ++e) v[e] = (gr < j.rows && gc + e < j.cols) ? src[(int64_t)gr * j.ld_src + gc + e] : (T)0;
+    }
+#pragma unroll
+    for (int e = 0; e < VE; ++e) tile[(lc + e) * PITCH + r] = v[e];     // transposed into LDS
+  }
+  __syncthreads();
+  const bool vec_out = (((uintptr_t)dst | (uintptr_t)((int64_t)j.rows * sizeof(T))) & 7) == 0;
+#pragma unroll
+  for (int pass = 0; pass < 64 / RPP; ++pass) {
+    const int c = lr + pass * RPP;           // a column of the source = a row of the result
+    const int gc = c0 + c, gr = r0 + lc;
+    if (gc >= j.cols) continue;
+    if (vec_out && gr + VE <= j.rows) {
+      *(uint2*)(dst + (int64_t)gc * j.rows + gr) = *(const uint2*)(tile + c * PITCH + lc);
+    } else {
+#pragma unroll
+      for (int e = 0; e < VE; ++e)
+        if (gr + e < j.rows) dst[(int64_t)gc * j.rows + gr + e] = tile[c * PITCH + lc + e];
+    }
+  }
+}
+
 template <typename T>
 __global__ void fill_zero_kernel(T* p, int64_t rows, int64_t cols, int64_t ld) {
   int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -108,6 +162,9 @@ struct Plan {
   int conv_occ;
   int conv_waves;
   int conv_w9;
+  // GEMM operands copied K-contiguous into the workspace in front of the kernel
+  int n_transposes;
+  TransposeJob tr[2];
 };
 
 static int dtype_pair(int in_dtype, int out_dtype, int* dt) {
@@ -156,8 +213,73 @@ static int plan_finish(Plan& pl, int op, const void* desc, const amos_kernel_con
 
 static int plan_gemm(Plan& pl, int op, const void* desc_any, const amos_gemm_desc_t* d,
                      int64_t batch, int64_t sa, int64_t sb, int64_t sc,
-                     const amos_kernel_config_t* cfg, const void* A, const void* B, void* C) {
+                     const amos_kernel_config_t* cfg, const void* A, const void* B, void* C,
+                     void* workspace = nullptr, size_t ws_bytes = 0);
+
+// workspace that lets a GEMM with row-contiguous operands (a transposed A, a row-major B) run on
+// the K-contiguous kernels: room for the transposed copies
+static int64_t gemm_transpose_bytes(const amos_gemm_desc_t& g, int64_t batch) {
+  const int es = g.in_dtype == AMOS_I8 ? 1 : 2;
+  if (g.K % (128 / es) != 0 || g.M <= 0 || g.N <= 0) return 0;
+  // below ~8 GFLOP the copies cost what the faster kernel gains; ~1 GFLOP where the register-staged
+  // kernel would have to load the operand element by element (8-bit types, rows not a multiple of 8)
+  const bool vectors = es == 2 && (!g.trans_a || g.M % 8 == 0) && (g.trans_b || g.N % 8 == 0);
+  if (2.0 * (double)g.M * (double)g.N * (double)g.K * (double)batch < (vectors ? 8e9 : 1e9)) return 0;
+  int64_t need = 0;
+  if (g.trans_a) need += (batch * g.M * g.K * es + 255) / 256 * 256;
+  if (!g.trans_b) need += (batch * g.N * g.K * es + 255) / 256 * 256;
+  return need;
+}
+
+// plan a GEMM whose row-contiguous operands are first copied K-contiguous into the workspace
+static int plan_gemm_transposed(Plan& pl, int op, const amos_gemm_desc_t* d, int64_t batch, int64_t sa,
+                                int64_t sb, int64_t sc, const amos_kernel_config_t* cfg, const void* A,
+                                const void* B, void* C, void* workspace) {
+  const int es = d->in_dtype == AMOS_I8 ? 1 : 2;
+  amos_bgemm_desc_t e;
+  memset(&e, 0, sizeof(e));
+  e.g = *d;
+  e.batch = batch;
+  e.stride_a = sa; e.stride_b = sb; e.stride_c = sc;
+  TransposeJob jobs[2];
+  int n = 0;
+  char* ws = (char*)workspace;
+  const void *A2 = A, *B2 = B;
+  if (d->trans_a) {   // stored [K][M] -> [M][K]
+    jobs[n++] = TransposeJob{(const char*)A, ws, (int)d->K, (int)d->M, d->lda, sa, d->M * d->K, (int)batch};
+    A2 = ws;
+    ws += (batch * d->M * d->K * es + 255) / 256 * 256;
+    e.g.trans_a = 0; e.g.lda = d->K; e.stride_a = d->M * d->K;
+  }
+  if (!d->trans_b) {  // stored [K][N] -> [N][K]
+    jobs[n++] = TransposeJob{(const char*)B, ws, (int)d->K, (int)d->N, d->ldb, sb, d->N * d->K, (int)batch};
+    B2 = ws;
+    e.g.trans_b = 1; e.g.ldb = d->K; e.stride_b = d->N * d->K;
+  }
+  int rc = plan_gemm(pl, batch > 1 || op == AMOS_OP_BGEMM ? AMOS_OP_BGEMM : AMOS_OP_GEMM,
+                     batch > 1 || op == AMOS_OP_BGEMM ? (const void*)&e : (const void*)&e.g, &e.g, batch,
+                     e.stride_a, e.stride_b, e.stride_c, cfg, A2, B2, C);
+  if (rc) return rc;
+  pl.n_transposes = n;
+  for (int k = 0; k < n; ++k) pl.tr[k] = jobs[k];
+  return 0;
+}
+
+static int plan_gemm(Plan& pl, int op, const void* desc_any, const amos_gemm_desc_t* d,
+                     int64_t batch, int64_t sa, int64_t sb, int64_t sc,
+                     const amos_kernel_config_t* cfg, const void* A, const void* B, void* C,
+                     void* workspace, size_t ws_bytes) {
   if (!d || !A || !B || !C) return set_error(AMOS_ERR_BAD_ARG, "null pointer argument");
+  pl.n_transposes = 0;
+  if (workspace && (d->trans_a || !d->trans_b) && batch > 0 && batch < 65536 &&
+      (!cfg || cfg->pipeline != AMOS_PIPE_STAGED) && ((uintptr_t)workspace & 255) == 0) {
+    const int64_t need = gemm_transpose_bytes(*d, batch);
+    const int es = d->in_dtype == AMOS_I8 ? 1 : 2;
+    if (need > 0 && ws_bytes >= (size_t)need && fits_int(d->M) && fits_int(d->N) && fits_int(d->K) &&
+        d->lda >= (d->trans_a ? d->M : d->K) && d->ldb >= (d->trans_b ? d->K : d->N) &&
+        (d->K * es) % 16 == 0)
+      return plan_gemm_transposed(pl, op, d, batch, sa, sb, sc, cfg, A, B, C, workspace);
+  }
   if (!fits_int(d->M) || !fits_int(d->N) || !fits_int(d->K) || batch <= 0)
     return set_error(AMOS_ERR_BAD_ARG, "extents must be in [1, 2^31): M=%lld N=%lld K=%lld batch=%lld",
                      (long long)d->M, (long long)d->N, (long long)d->K, (long long)batch);
@@ -301,13 +423,15 @@ static int plan_conv(Plan& pl, int op, const amos_conv_desc_t* d, const amos_ker
       b.g.M = c.K; b.g.N = dhw;
       b.g.lda = c.C; b.g.ldb = dhw; b.g.ldc = dhw;
       b.stride_a = 0; b.stride_b = c.C * dhw; b.stride_c = c.K * dhw;
-      return plan_gemm(pl, AMOS_OP_BGEMM, &b, &b.g, b.batch, b.stride_a, b.stride_b, b.stride_c, cfg, Wt, X, Y);
+      return plan_gemm(pl, AMOS_OP_BGEMM, &b, &b.g, b.batch, b.stride_a, b.stride_b, b.stride_c, cfg, Wt, X, Y,
+                       workspace, ws_bytes);
     }
     b.batch = 1;
     b.g.M = c.N * dhw; b.g.N = c.K;
     b.g.lda = c.C; b.g.ldb = c.K; b.g.ldc = c.K;
     b.stride_a = b.g.M * c.C; b.stride_b = c.C * c.K; b.stride_c = b.g.M * c.K;
-    return plan_gemm(pl, AMOS_OP_BGEMM, &b, &b.g, 1, b.stride_a, b.stride_b, b.stride_c, cfg, X, Wt, Y);
+    return plan_gemm(pl, AMOS_OP_BGEMM, &b, &b.g, 1, b.stride_a, b.stride_b, b.stride_c, cfg, X, Wt, Y,
+                     workspace, ws_bytes);
   }
   const int es = pl.dt == DT_I8 ? 1 : 2;
   const int ce = 16 / es;
@@ -461,14 +585,16 @@ static int make_plan(Plan& pl, int op, const void* desc, const amos_kernel_confi
   pl.tn_waves = 0;
   pl.conv_ups = 0;
   pl.fill_once = 0;
+  pl.n_transposes = 0;
   switch (op) {
     case AMOS_OP_GEMM:
-      return plan_gemm(pl, op, desc, (const amos_gemm_desc_t*)desc, 1, 0, 0, 0, cfg, in0, in1, out);
+      return plan_gemm(pl, op, desc, (const amos_gemm_desc_t*)desc, 1, 0, 0, 0, cfg, in0, in1, out, workspace,
+                       ws_bytes);
     case AMOS_OP_BGEMM: {
       const amos_bgemm_desc_t* b = (const amos_bgemm_desc_t*)desc;
       if (!b) return set_error(AMOS_ERR_BAD_ARG, "null descriptor");
       return plan_gemm(pl, op, desc, &b->g, b->batch, b->stride_a, b->stride_b, b->stride_c, cfg,
-                       in0, in1, out);
+                       in0, in1, out, workspace, ws_bytes);
     }
     case AMOS_OP_CONV2D:
     case AMOS_OP_CONV3D:
@@ -537,6 +663,14 @@ static int launch_conv(const Plan& pl, hipStream_t stream) {
 }
 
 static int launch(const Plan& pl, hipStream_t stream) {
+  for (int k = 0; k < pl.n_transposes; ++k) {
+    const TransposeJob& j = pl.tr[k];
+    dim3 grid((unsigned)((j.cols + 63) / 64), (unsigned)((j.rows + 63) / 64), (unsigned)j.batch);
+    if (pl.dt == DT_I8)
+      hipLaunchKernelGGL(amos_transpose_kernel<unsigned char>, grid, dim3(256), 0, stream, j);
+    else
+      hipLaunchKernelGGL(amos_transpose_kernel<unsigned short>, grid, dim3(256), 0, stream, j);
+  }
   if (pl.tn_waves) return launch_tn(pl, stream);
   if (pl.conv_ups) return launch_conv(pl, stream);
   Instance* inst;
@@ -748,11 +882,37 @@ int amos_run_fused(int op, const void* desc, const amos_kernel_config_t* cfg,
 }
 
 size_t amos_workspace_bytes(int op, const void* desc, const amos_kernel_config_t* cfg) {
-  // GEMM: none (split-K accumulates straight into the zero-filled output).
+  // GEMM: room for K-contiguous copies of row-contiguous operands (a transposed A, a row-major B)
+  // where the problem is large enough for the copies to pay; none otherwise (split-K accumulates
+  // straight into the zero-filled output).
   // conv: room for the weights repacked to K,(TRS),C when the patch-staged pipeline applies.
-  (void)cfg;
-  if (!desc || (op != AMOS_OP_CONV2D && op != AMOS_OP_CONV3D)) return 0;
-  return (size_t)conv_workspace_bytes(*(const amos_conv_desc_t*)desc, op);
+  if (!desc) return 0;
+  if (cfg && cfg->pipeline == AMOS_PIPE_STAGED && (op == AMOS_OP_GEMM || op == AMOS_OP_BGEMM)) return 0;
+  if (op == AMOS_OP_GEMM) return (size_t)gemm_transpose_bytes(*(const amos_gemm_desc_t*)desc, 1);
+  if (op == AMOS_OP_BGEMM) {
+    const amos_bgemm_desc_t* b = (const amos_bgemm_desc_t*)desc;
+    return b->batch > 0 && b->batch < 65536 ? (size_t)gemm_transpose_bytes(b->g, b->batch) : 0;
+  }
+  if (op != AMOS_OP_CONV2D && op != AMOS_OP_CONV3D) return 0;
+  const amos_conv_desc_t& c = *(const amos_conv_desc_t*)desc;
+  int64_t need = conv_workspace_bytes(c, op);
+  // a pointwise convolution runs as a matrix product; its row-contiguous operand (NCDHW
+  // activations, [C][K] weights) may want a K-contiguous copy
+  const bool is2d = op == AMOS_OP_CONV2D;
+  if ((is2d || c.T == 1) && c.R == 1 && c.S == 1 && c.stride_h == 1 && c.stride_w == 1 && c.pad_h == 0 &&
+      c.pad_w == 0 && (is2d || (c.stride_d == 1 && c.pad_d == 0)) && c.groups <= 1 && c.N > 0 && c.N < 65536) {
+    const int64_t dhw = (is2d ? 1 : c.D) * c.H * c.W;
+    amos_gemm_desc_t g;
+    memset(&g, 0, sizeof(g));
+    g.in_dtype = c.in_dtype;
+    g.K = c.C;
+    g.trans_a = 0; g.trans_b = 0;
+    int64_t t;
+    if (c.layout == AMOS_LAYOUT_NCHW) { g.M = c.K; g.N = dhw; t = gemm_transpose_bytes(g, c.N); }
+    else { g.M = c.N * dhw; g.N = c.K; t = gemm_transpose_bytes(g, 1); }
+    if (t > need) need = t;
+  }
+  return (size_t)need;
 }
 
 const char* amos_kernel_name(int op, const void* desc, const amos_kernel_config_t* cfg) {

@@ -129,8 +129,9 @@ def gemm(a, b, trans_a=False, trans_b=False, out=None, config=None, stream=None,
     d = gemm_desc(M, N, K, a.dtype, trans_a, trans_b)
     cfg = make_config(config)
     epi = make_epilogue(add, (M, N), out.dtype)
+    ws, ws_ptr, ws_bytes = _workspace(AMOS_OP_GEMM, d, cfg, a.device)
     check(_lib.load().amos_run_fused(AMOS_OP_GEMM, ctypes.byref(d), _cfg_ref(cfg), _epi_ref(epi), a.data_ptr(),
-                                     b.data_ptr(), out.data_ptr(), None, 0, _stream_ptr(stream)))
+                                     b.data_ptr(), out.data_ptr(), ws_ptr, ws_bytes, _stream_ptr(stream)))
     return out
 
 
@@ -156,9 +157,15 @@ def bgemm(a, b, trans_a=False, trans_b=False, out=None, config=None, stream=None
     d = bgemm_desc(B, M, N, K, a.dtype, trans_a, trans_b)
     cfg = make_config(config)
     epi = make_epilogue(add, (B, M, N), out.dtype)
+    ws, ws_ptr, ws_bytes = _workspace(AMOS_OP_BGEMM, d, cfg, a.device)
     check(_lib.load().amos_run_fused(AMOS_OP_BGEMM, ctypes.byref(d), _cfg_ref(cfg), _epi_ref(epi), a.data_ptr(),
-                                     b.data_ptr(), out.data_ptr(), None, 0, _stream_ptr(stream)))
+                                     b.data_ptr(), out.data_ptr(), ws_ptr, ws_bytes, _stream_ptr(stream)))
     return out
+
+
+def workspace_bytes(op, desc, config=None):
+    cfg = make_config(config)
+    return int(_lib.load().amos_workspace_bytes(op, ctypes.byref(desc), _cfg_ref(cfg)))
 
 
 def _workspace(op, desc, cfg, device):

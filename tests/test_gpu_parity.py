@@ -10,6 +10,8 @@ fp16 (reference: README.md:334), atol=rtol=1e-1 for bf16 (reference:
 tests/python/auto_tensorize/manual_mapping_conv2d_fp16fp32_tensorcore.py:114), both scaled
 by max(1, rms) of the output, and mean-rel-err <= 1e-3 for fp16 on the config-sized cases.
 """
+import ctypes
+
 import numpy as np
 import pytest
 
@@ -137,6 +139,48 @@ def test_gemm_row_contiguous_operands(gpu, dtype, trans, tile):
         bb = make_operand(rng, (3, N, K) if tb else (3, K, N), dtype)
         gb = ops.bgemm(to_device(ab, dtype), to_device(bb, dtype), ta, tb, config=cfg).cpu().numpy()
         check(gb, co.lib_gemm(ab, bb, dtype, ta, tb, acc="float64"), dtype, "batched %s" % name)
+
+
+@pytest.mark.parametrize("dtype", ["float16", "int8"])
+@pytest.mark.parametrize("trans", [(0, 0), (1, 1), (1, 0)])
+def test_gemm_row_contiguous_operands_through_transposed_copies(gpu, dtype, trans):
+    """large GEMMs with a transposed A / a row-major B and a workspace: the operands are copied
+    K-contiguous and the direct-to-LDS kernel runs; without workspace (or with the register-staged
+    pipeline asked for) the register-staged kernel does, and both agree with the oracle"""
+    import torch
+    from amos_amd import _lib, ops
+    ta, tb = trans
+    M, N, K = 2056, 1992, 1024      # ragged M and N, whole K steps
+    rng = np.random.default_rng(31)
+    a = make_operand(rng, (K, M) if ta else (M, K), dtype)
+    b = make_operand(rng, (N, K) if tb else (K, N), dtype)
+    da, db = to_device(a, dtype), to_device(b, dtype)
+    d = ops.gemm_desc(M, N, K, da.dtype, ta, tb)
+    assert ops.workspace_bytes(_lib.AMOS_OP_GEMM, d) > 0
+    assert "amos_gemm_tn" in ops.kernel_name(_lib.AMOS_OP_GEMM, d, None)
+    assert "amos_igemm" in ops.kernel_name(_lib.AMOS_OP_GEMM, d, dict(tile_i=128, tile_j=128, split_k=1,
+                                                                      pipeline=_lib.AMOS_PIPE_STAGED))
+    ref = co.lib_gemm(a, b, dtype, bool(ta), bool(tb), acc="float64")
+    got = ops.gemm(da, db, bool(ta), bool(tb))
+    check(got.cpu().numpy(), ref, dtype, "transposed-copy gemm %s %s" % (dtype, trans))
+    staged = ops.gemm(da, db, bool(ta), bool(tb), config=dict(tile_i=128, tile_j=128, split_k=1,
+                                                              pipeline=_lib.AMOS_PIPE_STAGED))
+    check(staged.cpu().numpy(), ref, dtype, "staged gemm %s %s" % (dtype, trans))
+    # no workspace: the same call still works (register-staged kernel)
+    out = torch.empty_like(got)
+    _lib.check(_lib.load().amos_gemm(ctypes.byref(d), None, da.data_ptr(), db.data_ptr(), out.data_ptr(), None, 0, None))
+    torch.cuda.synchronize()
+    check(out.cpu().numpy(), ref, dtype, "gemm without workspace %s %s" % (dtype, trans))
+    # batched, with the fused tail
+    Bn, m, n, k = 5, 1000, 1096, 1024
+    ab = make_operand(rng, (Bn, k, m) if ta else (Bn, m, k), dtype)
+    bb = make_operand(rng, (Bn, n, k) if tb else (Bn, k, n), dtype)
+    dd = torch.randn((Bn, m, n), device="cuda").to(torch.int32 if dtype == "int8" else torch.float32)
+    bd = ops.bgemm_desc(Bn, m, n, k, da.dtype, ta, tb)
+    assert "amos_gemm_tn" in ops.kernel_name(_lib.AMOS_OP_BGEMM, bd, None)
+    gb = ops.bgemm(to_device(ab, dtype), to_device(bb, dtype), bool(ta), bool(tb), add=dd)
+    check((gb - dd).cpu().numpy(), co.lib_gemm(ab, bb, dtype, bool(ta), bool(tb), acc="float64"), dtype,
+          "transposed-copy bgemm %s %s" % (dtype, trans))
 
 
 def test_gemm_direct_pipeline_rejects_ragged_k(gpu):
