@@ -69,9 +69,11 @@ __global__ __launch_bounds__(256) void amos_gather_kernel(const GatherParams g, 
 struct TransposeJob {
   const char* src;
   char* dst;
-  int rows, cols;
+  int rows, cols;          // of the source: rows = the reduction index K of a row-contiguous operand
   int64_t ld_src, batch_src, batch_dst;
   int batch;
+  int ld_dst;              // >= rows; the result's rows are zero-filled from `rows` up to it
+  int copy;                // 1: no transposition, dst[r][k] = src[r][k] (k < cols), zero up to ld_dst
 };
 template <typename T>
 __global__ __launch_bounds__(256) void amos_transpose_kernel(const TransposeJob j) {
@@ -101,19 +103,42 @@ __global__ __launch_bounds__(256) void amos_transpose_kernel(const TransposeJob 
     for (int e = 0; e < VE; ++e) tile[(lc + e) * PITCH + r] = v[e];     // transposed into LDS
   }
   __syncthreads();
-  const bool vec_out = (((uintptr_t)dst | (uintptr_t)((int64_t)j.rows * sizeof(T))) & 7) == 0;
+  const bool vec_out = (((uintptr_t)dst | (uintptr_t)((int64_t)j.ld_dst * sizeof(T))) & 7) == 0;
 #pragma unroll
   for (int pass = 0; pass < 64 / RPP; ++pass) {
     const int c = lr + pass * RPP;           // a column of the source = a row of the result
     const int gc = c0 + c, gr = r0 + lc;
     if (gc >= j.cols) continue;
-    if (vec_out && gr + VE <= j.rows) {
-      *(uint2*)(dst + (int64_t)gc * j.rows + gr) = *(const uint2*)(tile + c * PITCH + lc);
+    if (vec_out && gr + VE <= j.ld_dst) {    // (rows of the source past `rows` were read as zeros)
+      *(uint2*)(dst + (int64_t)gc * j.ld_dst + gr) = *(const uint2*)(tile + c * PITCH + lc);
     } else {
 #pragma unroll
       for (int e = 0; e < VE; ++e)
-        if (gr + e < j.rows) dst[(int64_t)gc * j.rows + gr + e] = tile[c * PITCH + lc + e];
+        if (gr + e < j.ld_dst) dst[(int64_t)gc * j.ld_dst + gr + e] = tile[c * PITCH + lc + e];
     }
+  }
+}
+
+// dst[b][r][k] = src[b][r][k] for k < cols, 0 for cols <= k < ld_dst (rows of a K-contiguous
+// operand copied to whole, aligned K steps)
+template <typename T>
+__global__ __launch_bounds__(256) void amos_padcopy_kernel(const TransposeJob j) {
+  constexpr int VE = 8 / (int)sizeof(T);
+  const T* src = (const T*)j.src + (int64_t)blockIdx.z * j.batch_src;
+  T* dst = (T*)j.dst + (int64_t)blockIdx.z * j.batch_dst;
+  const int per_row = j.ld_dst / VE;          // ld_dst is a multiple of a K step
+  const bool vec_in = (((uintptr_t)src | (uintptr_t)(j.ld_src * sizeof(T))) & 7) == 0;
+  const int64_t total = (int64_t)j.rows * per_row;
+  for (int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x; idx < total; idx += (int64_t)gridDim.x * 256) {
+    const int r = (int)(idx / per_row), k = (int)(idx - (int64_t)r * per_row) * VE;
+    T v[VE];
+    if (vec_in && k + VE <= j.cols) {
+      *(uint2*)v = *(const uint2*)(src + (int64_t)r * j.ld_src + k);
+    } else {
+#pragma unroll
+      for (int e = 0; e < VE; ++e) v[e] = k + e < j.cols ? src[(int64_t)r * j.ld_src + k + e] : (T)0;
+    }
+    *(uint2*)(dst + (int64_t)r * j.ld_dst + k) = *(const uint2*)v;
   }
 }
 
@@ -216,49 +241,93 @@ static int plan_gemm(Plan& pl, int op, const void* desc_any, const amos_gemm_des
                      const amos_kernel_config_t* cfg, const void* A, const void* B, void* C,
                      void* workspace = nullptr, size_t ws_bytes = 0);
 
-// workspace that lets a GEMM with row-contiguous operands (a transposed A, a row-major B) run on
-// the K-contiguous kernels: room for the transposed copies
-static int64_t gemm_transpose_bytes(const amos_gemm_desc_t& g, int64_t batch) {
+// Which operands of a GEMM are copied into the workspace so that the direct-to-LDS kernel can run:
+// row-contiguous ones (a transposed A, a row-major B) are transposed, K-contiguous ones whose rows
+// are not whole, 16-byte aligned K steps are copied with the K steps zero-filled (a ragged K
+// concerns both operands: garbage times the other side's zeros could be a NaN).
+struct GemmRepack {
+  bool copy_a, copy_b;
+  int64_t Kp;              // K rounded up to whole K steps
+  int64_t bytes_a, bytes_b;
+  int64_t total() const { return bytes_a + bytes_b; }
+};
+static GemmRepack gemm_repack(const amos_gemm_desc_t& g, int64_t batch, bool a_unaligned, bool b_unaligned) {
+  GemmRepack r = {false, false, 0, 0, 0};
   const int es = g.in_dtype == AMOS_I8 ? 1 : 2;
-  if (g.K % (128 / es) != 0 || g.M <= 0 || g.N <= 0) return 0;
+  const int bke = 128 / es;
+  if (g.M <= 0 || g.N <= 0 || g.K <= 0 || batch <= 0 || batch >= 65536) return r;
+  const bool ragged = g.K % bke != 0;
+  const bool a_bad = !g.trans_a && ((g.lda * es) % 16 != 0 || a_unaligned);
+  const bool b_bad = g.trans_b && ((g.ldb * es) % 16 != 0 || b_unaligned);
+  const bool copy_a = g.trans_a || ragged || a_bad, copy_b = !g.trans_b || ragged || b_bad;
+  if (!copy_a && !copy_b) return r;
   // below ~8 GFLOP the copies cost what the faster kernel gains; ~1 GFLOP where the register-staged
-  // kernel would have to load the operand element by element (8-bit types, rows not a multiple of 8)
-  const bool vectors = es == 2 && (!g.trans_a || g.M % 8 == 0) && (g.trans_b || g.N % 8 == 0);
-  if (2.0 * (double)g.M * (double)g.N * (double)g.K * (double)batch < (vectors ? 8e9 : 1e9)) return 0;
-  int64_t need = 0;
-  if (g.trans_a) need += (batch * g.M * g.K * es + 255) / 256 * 256;
-  if (!g.trans_b) need += (batch * g.N * g.K * es + 255) / 256 * 256;
-  return need;
+  // kernel would have to load an operand element by element
+  const bool vectors = es == 2 && !a_bad && !b_bad && g.K % 8 == 0 &&
+                       (!g.trans_a || g.M % 8 == 0) && (g.trans_b || g.N % 8 == 0);
+  if (2.0 * (double)g.M * (double)g.N * (double)g.K * (double)batch < (vectors ? 8e9 : 1e9)) return r;
+  r.Kp = (g.K + bke - 1) / bke * bke;
+  r.copy_a = copy_a;
+  r.copy_b = copy_b;
+  if (copy_a) r.bytes_a = (batch * g.M * r.Kp * es + 255) / 256 * 256;
+  if (copy_b) r.bytes_b = (batch * g.N * r.Kp * es + 255) / 256 * 256;
+  return r;
 }
 
-// plan a GEMM whose row-contiguous operands are first copied K-contiguous into the workspace
-static int plan_gemm_transposed(Plan& pl, int op, const amos_gemm_desc_t* d, int64_t batch, int64_t sa,
-                                int64_t sb, int64_t sc, const amos_kernel_config_t* cfg, const void* A,
-                                const void* B, void* C, void* workspace) {
-  const int es = d->in_dtype == AMOS_I8 ? 1 : 2;
+// plan a GEMM on copies of its operands (see gemm_repack)
+static int plan_gemm_repacked(Plan& pl, int op, const amos_gemm_desc_t* d, const GemmRepack& rp, int64_t batch,
+                              int64_t sa, int64_t sb, int64_t sc, const amos_kernel_config_t* cfg,
+                              const void* A, const void* B, void* C, void* workspace) {
   amos_bgemm_desc_t e;
   memset(&e, 0, sizeof(e));
   e.g = *d;
+  e.g.K = rp.Kp;
   e.batch = batch;
   e.stride_a = sa; e.stride_b = sb; e.stride_c = sc;
   TransposeJob jobs[2];
   int n = 0;
   char* ws = (char*)workspace;
   const void *A2 = A, *B2 = B;
-  if (d->trans_a) {   // stored [K][M] -> [M][K]
-    jobs[n++] = TransposeJob{(const char*)A, ws, (int)d->K, (int)d->M, d->lda, sa, d->M * d->K, (int)batch};
+  if (rp.copy_a) {
+    if (d->trans_a)   // stored [K][M] -> [M][Kp]
+      jobs[n++] = TransposeJob{(const char*)A, ws, (int)d->K, (int)d->M, d->lda, sa, d->M * rp.Kp, (int)batch, (int)rp.Kp, 0};
+    else              // stored [M][K] -> [M][Kp]
+      jobs[n++] = TransposeJob{(const char*)A, ws, (int)d->M, (int)d->K, d->lda, sa, d->M * rp.Kp, (int)batch, (int)rp.Kp, 1};
     A2 = ws;
-    ws += (batch * d->M * d->K * es + 255) / 256 * 256;
-    e.g.trans_a = 0; e.g.lda = d->K; e.stride_a = d->M * d->K;
+    ws += rp.bytes_a;
+    e.g.trans_a = 0; e.g.lda = rp.Kp; e.stride_a = d->M * rp.Kp;
   }
-  if (!d->trans_b) {  // stored [K][N] -> [N][K]
-    jobs[n++] = TransposeJob{(const char*)B, ws, (int)d->K, (int)d->N, d->ldb, sb, d->N * d->K, (int)batch};
+  if (rp.copy_b) {
+    if (!d->trans_b)  // stored [K][N] -> [N][Kp]
+      jobs[n++] = TransposeJob{(const char*)B, ws, (int)d->K, (int)d->N, d->ldb, sb, d->N * rp.Kp, (int)batch, (int)rp.Kp, 0};
+    else
+      jobs[n++] = TransposeJob{(const char*)B, ws, (int)d->N, (int)d->K, d->ldb, sb, d->N * rp.Kp, (int)batch, (int)rp.Kp, 1};
     B2 = ws;
-    e.g.trans_b = 1; e.g.ldb = d->K; e.stride_b = d->N * d->K;
+    e.g.trans_b = 1; e.g.ldb = rp.Kp; e.stride_b = d->N * rp.Kp;
   }
-  int rc = plan_gemm(pl, batch > 1 || op == AMOS_OP_BGEMM ? AMOS_OP_BGEMM : AMOS_OP_GEMM,
-                     batch > 1 || op == AMOS_OP_BGEMM ? (const void*)&e : (const void*)&e.g, &e.g, batch,
-                     e.stride_a, e.stride_b, e.stride_c, cfg, A2, B2, C);
+  const bool batched = batch > 1 || op == AMOS_OP_BGEMM;
+  // the copies are made for the direct-to-LDS kernel: without a tile from the caller, take the
+  // best of its tiles by the mapper's model
+  amos_kernel_config_t direct;
+  if (!cfg || cfg->tile_i <= 0 || cfg->tile_j <= 0) {
+    static const int tiles[4][2] = {{256, 256}, {128, 128}, {128, 256}, {256, 128}};
+    double best = 1e30;
+    memset(&direct, 0, sizeof(direct));
+    for (auto& t : tiles) {
+      amos_kernel_config_t c2;
+      memset(&c2, 0, sizeof(c2));
+      c2.tile_i = t[0]; c2.tile_j = t[1]; c2.split_k = 1; c2.pipeline = AMOS_PIPE_DIRECT8;
+      double sec = 0.0;
+      if (amos_estimate_seconds(batched ? AMOS_OP_BGEMM : AMOS_OP_GEMM,
+                                batched ? (const void*)&e : (const void*)&e.g, &c2, &sec) == 0 && sec < best) {
+        best = sec;
+        direct = c2;
+      }
+    }
+    if (best < 1e30) cfg = &direct;
+  }
+  int rc = plan_gemm(pl, batched ? AMOS_OP_BGEMM : AMOS_OP_GEMM, batched ? (const void*)&e : (const void*)&e.g,
+                     &e.g, batch, e.stride_a, e.stride_b, e.stride_c, cfg, A2, B2, C);
   if (rc) return rc;
   pl.n_transposes = n;
   for (int k = 0; k < n; ++k) pl.tr[k] = jobs[k];
@@ -271,14 +340,13 @@ static int plan_gemm(Plan& pl, int op, const void* desc_any, const amos_gemm_des
                      void* workspace, size_t ws_bytes) {
   if (!d || !A || !B || !C) return set_error(AMOS_ERR_BAD_ARG, "null pointer argument");
   pl.n_transposes = 0;
-  if (workspace && (d->trans_a || !d->trans_b) && batch > 0 && batch < 65536 &&
-      (!cfg || cfg->pipeline != AMOS_PIPE_STAGED) && ((uintptr_t)workspace & 255) == 0) {
-    const int64_t need = gemm_transpose_bytes(*d, batch);
-    const int es = d->in_dtype == AMOS_I8 ? 1 : 2;
-    if (need > 0 && ws_bytes >= (size_t)need && fits_int(d->M) && fits_int(d->N) && fits_int(d->K) &&
-        d->lda >= (d->trans_a ? d->M : d->K) && d->ldb >= (d->trans_b ? d->K : d->N) &&
-        (d->K * es) % 16 == 0)
-      return plan_gemm_transposed(pl, op, d, batch, sa, sb, sc, cfg, A, B, C, workspace);
+  if (workspace && (!cfg || cfg->pipeline != AMOS_PIPE_STAGED) && ((uintptr_t)workspace & 255) == 0 &&
+      fits_int(d->M) && fits_int(d->N) && fits_int(d->K) && d->K < (1 << 30) &&
+      d->lda >= (d->trans_a ? d->M : d->K) && d->ldb >= (d->trans_b ? d->K : d->N) &&
+      (d->in_dtype == AMOS_F16 || d->in_dtype == AMOS_BF16 || d->in_dtype == AMOS_I8)) {
+    const GemmRepack rp = gemm_repack(*d, batch, !aligned16(A), !aligned16(B));
+    if (rp.total() > 0 && ws_bytes >= (size_t)rp.total())
+      return plan_gemm_repacked(pl, op, d, rp, batch, sa, sb, sc, cfg, A, B, C, workspace);
   }
   if (!fits_int(d->M) || !fits_int(d->N) || !fits_int(d->K) || batch <= 0)
     return set_error(AMOS_ERR_BAD_ARG, "extents must be in [1, 2^31): M=%lld N=%lld K=%lld batch=%lld",
@@ -665,7 +733,18 @@ static int launch_conv(const Plan& pl, hipStream_t stream) {
 static int launch(const Plan& pl, hipStream_t stream) {
   for (int k = 0; k < pl.n_transposes; ++k) {
     const TransposeJob& j = pl.tr[k];
-    dim3 grid((unsigned)((j.cols + 63) / 64), (unsigned)((j.rows + 63) / 64), (unsigned)j.batch);
+    if (j.copy) {
+      const int ve = pl.dt == DT_I8 ? 8 : 4;
+      const int64_t want = ((int64_t)j.rows * (j.ld_dst / ve) + 255) / 256;
+      dim3 grid((unsigned)(want < 16384 ? want : 16384), 1, (unsigned)j.batch);
+      if (pl.dt == DT_I8)
+        hipLaunchKernelGGL(amos_padcopy_kernel<unsigned char>, grid, dim3(256), 0, stream, j);
+      else
+        hipLaunchKernelGGL(amos_padcopy_kernel<unsigned short>, grid, dim3(256), 0, stream, j);
+      continue;
+    }
+    // (the tiles over the result's zero-filled K steps read past the source's rows as zeros)
+    dim3 grid((unsigned)((j.cols + 63) / 64), (unsigned)((j.ld_dst + 63) / 64), (unsigned)j.batch);
     if (pl.dt == DT_I8)
       hipLaunchKernelGGL(amos_transpose_kernel<unsigned char>, grid, dim3(256), 0, stream, j);
     else
@@ -888,10 +967,10 @@ size_t amos_workspace_bytes(int op, const void* desc, const amos_kernel_config_t
   // conv: room for the weights repacked to K,(TRS),C when the patch-staged pipeline applies.
   if (!desc) return 0;
   if (cfg && cfg->pipeline == AMOS_PIPE_STAGED && (op == AMOS_OP_GEMM || op == AMOS_OP_BGEMM)) return 0;
-  if (op == AMOS_OP_GEMM) return (size_t)gemm_transpose_bytes(*(const amos_gemm_desc_t*)desc, 1);
+  if (op == AMOS_OP_GEMM) return (size_t)gemm_repack(*(const amos_gemm_desc_t*)desc, 1, false, false).total();
   if (op == AMOS_OP_BGEMM) {
     const amos_bgemm_desc_t* b = (const amos_bgemm_desc_t*)desc;
-    return b->batch > 0 && b->batch < 65536 ? (size_t)gemm_transpose_bytes(b->g, b->batch) : 0;
+    return (size_t)gemm_repack(b->g, b->batch, false, false).total();
   }
   if (op != AMOS_OP_CONV2D && op != AMOS_OP_CONV3D) return 0;
   const amos_conv_desc_t& c = *(const amos_conv_desc_t*)desc;
@@ -907,9 +986,10 @@ size_t amos_workspace_bytes(int op, const void* desc, const amos_kernel_config_t
     g.in_dtype = c.in_dtype;
     g.K = c.C;
     g.trans_a = 0; g.trans_b = 0;
+    g.lda = c.C;
     int64_t t;
-    if (c.layout == AMOS_LAYOUT_NCHW) { g.M = c.K; g.N = dhw; t = gemm_transpose_bytes(g, c.N); }
-    else { g.M = c.N * dhw; g.N = c.K; t = gemm_transpose_bytes(g, 1); }
+    if (c.layout == AMOS_LAYOUT_NCHW) { g.M = c.K; g.N = dhw; g.ldb = dhw; t = gemm_repack(g, c.N, false, false).total(); }
+    else { g.M = c.N * dhw; g.N = c.K; g.ldb = c.K; t = gemm_repack(g, 1, false, false).total(); }
     if (t > need) need = t;
   }
   return (size_t)need;

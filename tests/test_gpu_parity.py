@@ -183,6 +183,36 @@ def test_gemm_row_contiguous_operands_through_transposed_copies(gpu, dtype, tran
           "transposed-copy bgemm %s %s" % (dtype, trans))
 
 
+@pytest.mark.parametrize("dtype", ["float16", "int8"])
+@pytest.mark.parametrize("trans", [(0, 1), (0, 0), (1, 1), (1, 0)])
+@pytest.mark.parametrize("K", [1000, 1027])
+def test_gemm_ragged_k_through_padded_copies(gpu, dtype, trans, K):
+    """K that is not a whole number of K steps (or not even of 16-byte vectors): with a workspace
+    both operands are copied with zero-filled K steps and the direct-to-LDS kernel runs"""
+    import torch
+    from amos_amd import _lib, ops
+    ta, tb = trans
+    M, N = 1032, 1544
+    rng = np.random.default_rng(41 + K)
+    a = make_operand(rng, (K, M) if ta else (M, K), dtype)
+    b = make_operand(rng, (N, K) if tb else (K, N), dtype)
+    da, db = to_device(a, dtype), to_device(b, dtype)
+    d = ops.gemm_desc(M, N, K, da.dtype, ta, tb)
+    es = 1 if dtype == "int8" else 2
+    kp = -(-K // (128 // es)) * (128 // es)
+    # (fp16 with K a multiple of 8 keeps its vector loaders in the register-staged kernel: copies
+    # only pay for larger problems than this one)
+    copies = dtype == "int8" or K % 8 != 0
+    assert (ops.workspace_bytes(_lib.AMOS_OP_GEMM, d) >= (M + N) * kp * es) == copies
+    assert ("amos_gemm_tn" in ops.kernel_name(_lib.AMOS_OP_GEMM, d, None)) == copies
+    ref = co.lib_gemm(a, b, dtype, bool(ta), bool(tb), acc="float64")
+    got = ops.gemm(da, db, bool(ta), bool(tb))
+    check(got.cpu().numpy(), ref, dtype, "padded-copy gemm %s %s K=%d" % (dtype, trans, K))
+    staged = ops.gemm(da, db, bool(ta), bool(tb), config=dict(tile_i=64, tile_j=64, split_k=1,
+                                                              pipeline=_lib.AMOS_PIPE_STAGED))
+    check(staged.cpu().numpy(), ref, dtype, "staged gemm %s %s K=%d" % (dtype, trans, K))
+
+
 def test_gemm_direct_pipeline_rejects_ragged_k(gpu):
     import torch
     from amos_amd import _lib, ops
