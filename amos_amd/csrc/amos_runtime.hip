@@ -595,7 +595,8 @@ static int plan_conv(Plan& pl, int op, const amos_conv_desc_t* d, const amos_ker
   q.zeros = (char*)workspace + packed;
   q.xt = (char*)workspace + packed + 256;
   q.steps = (char*)workspace + packed + 256 + conv_relaid_bytes(c, op);
-  q.N = (int)c.N; q.C = (int)c.C; q.D = (int)c.D; q.H = (int)c.H; q.W = (int)c.W; q.K = (int)c.K;
+  const int64_t Cp = conv_padded_channels(c);   // whole K steps; the relayout zero-fills [C, Cp)
+  q.N = (int)c.N; q.C = (int)Cp; q.Csrc = (int)c.C; q.D = (int)c.D; q.H = (int)c.H; q.W = (int)c.W; q.K = (int)c.K;
   q.T = (int)c.T; q.R = (int)c.R; q.S = (int)c.S;
   q.sd = c.stride_d; q.sh = c.stride_h; q.sw = c.stride_w;
   q.pd = c.pad_d; q.ph = c.pad_h; q.pw = c.pad_w;
@@ -616,7 +617,7 @@ static int plan_conv(Plan& pl, int op, const amos_conv_desc_t* d, const amos_ker
     q.tab1_off = q.sx_off + pp.tab1_rel;
     q.dump_off = q.sx_off + pp.dump_rel;
   }
-  q.c_chunks = (int)(c.C * es / 128);
+  q.c_chunks = (int)(Cp * es / 128);
   q.macro_steps = (int)c.T * q.c_chunks;
   q.total_steps = q.macro_steps * RS;
   int split = pl.cfg.split_k < 1 ? 1 : pl.cfg.split_k;
@@ -634,12 +635,12 @@ static int plan_conv(Plan& pl, int op, const amos_conv_desc_t* d, const amos_ker
   q.fd_wp = make_fast_div((uint32_t)Wp);
   q.fd_odpq = make_fast_div((uint32_t)odpq);
   q.fd_cc = make_fast_div((uint32_t)q.c_chunks);
-  q.fd_c = make_fast_div((uint32_t)c.C);
-  const int64_t welems = c.K * c.T * c.R * c.S * c.C;
-  q.fd_slab = make_fast_div((uint32_t)(c.C * c.T * c.R * c.S));
+  q.fd_c = make_fast_div((uint32_t)Cp);
+  const int64_t welems = c.K * c.T * c.R * c.S * Cp;
+  q.fd_slab = make_fast_div((uint32_t)(Cp * c.T * c.R * c.S));
   q.prep_w_blocks = (int)((welems + 1023) / 1024 < 2048 ? (welems + 1023) / 1024 : 2048);
-  q.prep_x_blocks = (int)(c.N * c.D * (((int64_t)c.H * c.W + 63) / 64) * (c.C * es / 128));
-  if (layout != AMOS_LAYOUT_NCHW) q.prep_x_blocks = (int)((c.N * dhw * (c.C * es / 16) + 1023) / 1024);
+  q.prep_x_blocks = (int)(c.N * c.D * (((int64_t)c.H * c.W + 63) / 64) * (Cp * es / 128));
+  if (layout != AMOS_LAYOUT_NCHW) q.prep_x_blocks = (int)((c.N * dhw * (Cp * es / 16) + 1023) / 1024);
   q.layout = layout;
   q.y_si = p.out_si; q.y_sn = p.out_sjo; q.y_ss = p.out_sj;
   q.y_vec4 = layout != AMOS_LAYOUT_NCHW && c.K % 4 == 0 && aligned16(Y);

@@ -71,7 +71,8 @@ struct ConvFpropParams {
   char* wp;          // packed weights [K][T*R*S][C] (workspace)
   char* zeros;       // 128 zero bytes (workspace)
   char* y;           // NKDPQ, fp32 / int32
-  int N, C, D, H, W, K, T, R, S;
+  int N, C, D, H, W, K, T, R, S;   // C: channels of the relaid operands (whole 128-byte K steps)
+  int Csrc;          // channels of the caller's tensors (<= C; the rest is zero-filled by the relayout)
   int sd, sh, sw, pd, ph, pw, dd, dh, dw;
   int OD, OP, OQ;
   int J;             // N*OD*OP*OQ
@@ -162,7 +163,7 @@ __global__ __launch_bounds__(256) void amos_conv_prepare(const ConvFpropParams p
     // thread so that the loads overlap
     const T* w = (const T*)p.w;
     T* wp = (T*)p.wp;
-    const int slab = p.C * TRS;
+    const int slab = p.C * TRS, slab_src = p.Csrc * TRS;
     const int64_t total = (int64_t)p.K * slab;
     for (int64_t base = (int64_t)b * 1024; base < total; base += (int64_t)p.prep_w_blocks * 1024) {
       T v[4];
@@ -174,7 +175,9 @@ __global__ __launch_bounds__(256) void amos_conv_prepare(const ConvFpropParams p
         const int k = fast_div((int)oc, p.fd_slab);   // the host keeps the packed weights under 2^31 elements
         const int o = (int)(oc - (int64_t)k * slab);
         const int tap = fast_div(o, p.fd_c), c = o - tap * p.C;
-        v[u] = p.layout == 0 ? w[(int64_t)k * slab + c * TRS + tap] : w[((int64_t)tap * p.C + c) * p.K + k];
+        v[u] = c >= p.Csrc ? (T)0
+                           : p.layout == 0 ? w[(int64_t)k * slab_src + c * TRS + tap]
+                                           : w[((int64_t)tap * p.Csrc + c) * p.K + k];
       }
 #pragma unroll
       for (int u = 0; u < 4; ++u)
@@ -191,6 +194,7 @@ __global__ __launch_bounds__(256) void amos_conv_prepare(const ConvFpropParams p
     // channels are innermost already: 16-byte chunks, four per thread; DHWNC moves image n's
     // positions from [s][n] to [n][s]
     const int cpp = p.C * (int)sizeof(T) / 16;           // chunks per position
+    const int cpp_src = p.Csrc * (int)sizeof(T) / 16;    // (the host pads channels only in whole chunks here)
     const int64_t dhw = (int64_t)p.D * p.H * p.W;
     const int64_t total = (int64_t)p.N * dhw * cpp;
     const uint4* x = (const uint4*)p.x;
@@ -201,14 +205,14 @@ __global__ __launch_bounds__(256) void amos_conv_prepare(const ConvFpropParams p
     for (int u = 0; u < 4; ++u) {
       of[u] = (int64_t)b * 1024 + t + 256 * u;
       const int64_t oc = of[u] < total ? of[u] : total - 1;
-      int64_t src = oc;
+      const int64_t pos = oc / cpp;
+      const int ch = (int)(oc - pos * cpp);
+      int64_t spos = pos;
       if (p.layout == 2) {
-        const int64_t pos = oc / cpp;
-        const int ch = (int)(oc - pos * cpp);
         const int64_t n = pos / dhw, s = pos - n * dhw;
-        src = (s * p.N + n) * cpp + ch;
+        spos = s * p.N + n;
       }
-      v[u] = x[src];
+      v[u] = ch < cpp_src ? x[spos * cpp_src + ch] : uint4{0, 0, 0, 0};
     }
 #pragma unroll
     for (int u = 0; u < 4; ++u)
@@ -241,9 +245,13 @@ __global__ __launch_bounds__(256) void amos_conv_prepare(const ConvFpropParams p
     for (int r = 0; r < CT / LROWS; ++r) {
       const int cl = lc + LROWS * r;
       const int sg = st * 64 + ls;
-      const T* src = x + ((((int64_t)n * p.C + ct * CT + cl) * p.D + d) * HW + sg);
+      const int ch = ct * CT + cl;
+      const T* src = x + ((((int64_t)n * p.Csrc + (ch < p.Csrc ? ch : 0)) * p.D + d) * HW + sg);
       T v[VE];
-      if (vec && sg + VE <= HW) {
+      if (ch >= p.Csrc) {
+#pragma unroll
+        for (int e = 0; e < VE; ++e) v[e] = (T)0;
+      } else if (vec && sg + VE <= HW) {
         *(uint2*)v = *(const uint2*)src;
       } else {
 #pragma unroll

@@ -129,23 +129,37 @@ static void conv_patch_extent(int64_t J, int OPQ, int OQ, int BJ, int sh, int R,
 
 // workspace of the patch-staged pipeline:
 // [packed weights | 256 zero bytes | NDHWC activations | step table, 32 bytes per K step + 1]
+// channels of the relaid operands: C rounded up to whole 128-byte K steps, zero-filled by the
+// relayout launch, where that at most doubles the work (0: the patch-staged pipeline does not apply);
+// channel-innermost layouts want whole 16-byte chunks of real channels
+int64_t conv_padded_channels(const amos_conv_desc_t& c) {
+  const int es = c.in_dtype == AMOS_I8 ? 1 : 2;
+  const int64_t step = 128 / es;
+  if (c.C <= 0) return 0;
+  const int64_t cp = (c.C + step - 1) / step * step;
+  if (cp == c.C) return cp;
+  if (cp > 2 * c.C) return 0;
+  if (c.layout != AMOS_LAYOUT_NCHW && (c.C * es) % 16 != 0) return 0;
+  return cp;
+}
 int64_t conv_packed_bytes(const amos_conv_desc_t& c, int op) {
   int64_t T = op == AMOS_OP_CONV2D ? 1 : c.T;
   int es = c.in_dtype == AMOS_I8 ? 1 : 2;
-  if (c.C <= 0 || (c.C * es) % 128 != 0) return 0;
-  return (c.K * T * c.R * c.S * c.C * es + 255) / 256 * 256;
+  const int64_t cp = conv_padded_channels(c);
+  if (cp == 0) return 0;
+  return (c.K * T * c.R * c.S * cp * es + 255) / 256 * 256;
 }
 int64_t conv_relaid_bytes(const amos_conv_desc_t& c, int op) {
   int64_t D = op == AMOS_OP_CONV2D ? 1 : c.D;
   int es = c.in_dtype == AMOS_I8 ? 1 : 2;
-  return (c.N * c.C * D * c.H * c.W * es + 255) / 256 * 256;
+  return (c.N * conv_padded_channels(c) * D * c.H * c.W * es + 255) / 256 * 256;
 }
 int64_t conv_workspace_bytes(const amos_conv_desc_t& c, int op) {
   int64_t packed = conv_packed_bytes(c, op);
   if (packed == 0 || c.groups > 1) return 0;
   int64_t T = op == AMOS_OP_CONV2D ? 1 : c.T;
   int es = c.in_dtype == AMOS_I8 ? 1 : 2;
-  int64_t steps = T * c.R * c.S * (c.C * es / 128);
+  int64_t steps = T * c.R * c.S * (conv_padded_channels(c) * es / 128);
   return packed + 256 + conv_relaid_bytes(c, op) + (steps + 1) * 32;
 }
 
@@ -186,7 +200,7 @@ static ConvPatchPlan conv_patch_plan_waves(const amos_conv_desc_t& cin, int op, 
                                      (BI == 256 && (BJ == 64 || BJ == 128)));
   if (OD <= 0 || OP <= 0 || OQ <= 0) { pp.why = "empty output"; return pp; }
   if (c.groups > 1) { pp.why = "grouped convolution runs on the register-staged kernel"; return pp; }
-  if (packed == 0) { pp.why = "C * element size is not a multiple of 128 bytes"; return pp; }
+  if (packed == 0) { pp.why = "channels fill less than half of the 128-byte K steps they would be padded to"; return pp; }
   if (packed >= ((int64_t)1 << 31)) { pp.why = "packed weights above 2 GiB"; return pp; }
   if (conv_relaid_bytes(c, op) + 256 >= ((int64_t)1 << 32)) { pp.why = "activations above 4 GiB"; return pp; }
   if (c.N * c.D * c.H * c.W >= ((int64_t)1 << 31) || J >= ((int64_t)1 << 31) - 512) {
@@ -202,7 +216,7 @@ static ConvPatchPlan conv_patch_plan_waves(const amos_conv_desc_t& cin, int op, 
   // taken from its address
   const int max_pos = (real_pos + 63) & ~63;
   const size_t budget = (size_t)160 * 1024 - 512;
-  const int64_t macro_steps = c.T * (c.C * es / 128);
+  const int64_t macro_steps = c.T * (conv_padded_channels(c) * es / 128);
   const int split = split_k < 1 ? 1 : split_k;
   const bool one_macro = (macro_steps + split - 1) / split <= 1;   // no next patch at all
   pp.xbufs = one_macro ? 1 : 2;

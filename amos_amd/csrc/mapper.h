@@ -52,6 +52,7 @@ struct ConvPatchPlan {
   size_t lds;        // dynamic LDS bytes of the block
   int tab_rel, tab1_rel, dump_rel;   // w9: position tables and dump line, bytes from the first patch buffer
 };
+int64_t conv_padded_channels(const amos_conv_desc_t& c);
 int64_t conv_packed_bytes(const amos_conv_desc_t& c, int op);
 int64_t conv_relaid_bytes(const amos_conv_desc_t& c, int op);
 int64_t conv_workspace_bytes(const amos_conv_desc_t& c, int op);

@@ -480,6 +480,40 @@ def test_pointwise_conv_runs_as_gemm(gpu, layout, dtype, case):
                   "pointwise %s %s %s cfg %s add %s" % (layout, dtype, case, cfg, add is not None))
 
 
+# (channel-innermost operands are padded in whole 16-byte chunks only: no int8 C=104 in nhwc)
+@pytest.mark.parametrize("dtype,C,layout", [(d, c, l) for d, c in [("float16", 96), ("float16", 40), ("bfloat16", 72),
+                                                                    ("int8", 64), ("int8", 104)]
+                                            for l in ("nchw", "nhwc") if not (l == "nhwc" and c == 104)])
+def test_conv_padded_channels(gpu, dtype, C, layout):
+    """channel counts that do not fill whole 128-byte K steps: the relayout launch zero-fills the
+    rest, the patch-staged kernels run on the padded operands"""
+    import torch
+    from amos_amd import _lib, ops
+    N, H, W, K, R, S = 3, 13, 11, 72, 3, 3
+    rng = np.random.default_rng(51 + C)
+    x = make_operand(rng, (N, C, 1, H, W), dtype, "normal")
+    w = make_operand(rng, (K, C, 1, R, S), dtype, "normal")
+    ref = co.lib_conv3d(x, w, dtype, (1, 1, 1), (0, 1, 1), (1, 1, 1), acc="float64")[:, :, 0]
+    if layout == "nhwc":
+        xs, ws_, refs = np.transpose(x[:, :, 0], (0, 2, 3, 1)), np.transpose(w[:, :, 0], (2, 3, 1, 0)), np.transpose(ref, (0, 2, 3, 1))
+    else:
+        xs, ws_, refs = x[:, :, 0], w[:, :, 0], ref
+    dx, dw = to_device(np.ascontiguousarray(xs), dtype), to_device(np.ascontiguousarray(ws_), dtype)
+    desc = ops.conv_desc((N, C, 1, H, W), (K, C, 1, R, S), dx.dtype, (1, 1, 1), (0, 1, 1), (1, 1, 1), 1, layout)
+    assert "amos_conv_fprop" in ops.kernel_name(_lib.AMOS_OP_CONV2D, desc, None)
+    ran = 0
+    for pipe in (None, _lib.AMOS_PIPE_PATCH, _lib.AMOS_PIPE_PATCH8, _lib.AMOS_PIPE_STAGED):
+        for tile, split in [((128, 128), 1), ((128, 64), 1), ((64, 128), 2)]:
+            cfg = None if pipe is None else dict(tile_i=tile[0], tile_j=tile[1], split_k=split, pipeline=pipe)
+            got = ops.conv2d(dx, dw, 1, 1, 1, config=cfg, layout=layout)
+            check(got.cpu().numpy(), np.ascontiguousarray(refs), dtype,
+                  "padded channels %s C=%d %s pipeline %s tile %s split %d" % (dtype, C, layout, pipe, tile, split))
+            ran += 1
+            if pipe is None:
+                break
+    assert ran == 10
+
+
 LAYOUT_CASES = [
     # N, C, D, H, W, K, T, R, S, stride, pad, dil
     (3, 24, 1, 9, 7, 40, 1, 3, 3, (1, 1, 1), (0, 1, 1), (1, 1, 1)),      # register-staged kernel only
