@@ -735,7 +735,7 @@ def _fuse_tail(low, main_op, target_dag):
         res = _flat_address_of_compute(_strip_cast(body), main_op, variables)
         want = dict(zip(variables, _row_major_strides(tail.output(0).shape)))
         want = {v: c for v, c in want.items() if int([iv for iv in tail.axis if iv.var is v][0].dom.extent) > 1}
-        if res is not None and res[1] == 0 and {v: c for v, c in res[0].items()} == want and \
+        if res is not None and res[1] == 0 and {v: c for v, c in res[0].items() if v in want} == want and \
                 _numel(tail.output(0).shape) == _numel(main_op.output(0).shape) and _dense_output(low):
             low.output = tail.output(0)
             return low

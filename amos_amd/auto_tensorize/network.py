@@ -85,7 +85,109 @@ def resnet18(batch=1, in_dtype="float16", out_dtype="float32", num_classes=1000)
         ("layer4 3x3 512->512 @7", conv2d_nchw(b, 512, 7, 7, 512, 3, 3, 1, 1, in_dtype, out_dtype), 3),
         ("fc 512->%d" % num_classes, dense(b, num_classes, 512, in_dtype, out_dtype), 1),
     ]
-    return [SubGraph("resnet18:subgraph%d" % i, ts, cnt, note) for i, (note, ts, cnt) in enumerate(layers)]
+    return _subgraphs("resnet18", layers)
+
+
+def batched_matmul(B, M, N, K, trans_b, in_dtype="float16", out_dtype="float32"):
+    """B independent products A[b] (M x K) times B[b] (stored N x K if trans_b, else K x N)"""
+    A = te.placeholder([B, M, K], dtype=in_dtype, name="A")
+    Bt = te.placeholder([B, N, K] if trans_b else [B, K, N], dtype=in_dtype, name="B")
+    rk = te.reduce_axis([0, K], name="k")
+    C = te.compute([B, M, N], lambda b, i, j: te.sum(
+        (A[b, i, rk] * (Bt[b, j, rk] if trans_b else Bt[b, rk, j])).astype(out_dtype), axis=rk), name="C")
+    return [A, Bt, C]
+
+
+def depthwise_conv2d_nchw(N, C, H, W, R, S, stride, padding, in_dtype="float16", out_dtype="float32"):
+    """one 3x3 filter per channel (benchmark/amos/mapping_depthwiseconv2d_tensorcore.py:7-48, K = C)"""
+    pH, pW = H + 2 * padding, W + 2 * padding
+    A = te.placeholder([N, C, H, W], dtype=in_dtype, name="A")
+    B = te.placeholder([C, R, S], dtype=in_dtype, name="B")
+    Pad = te.compute([N, C, pH, pW], lambda n, c, h, w: tir.if_then_else(
+        tir.all(h >= padding, h - padding < H, w >= padding, w - padding < W),
+        A[n, c, h - padding, w - padding], tir.const(0.0, A.dtype)), name="Pad")
+    B_reshaped = te.compute([C, 1, R, S], lambda k_o, k_i, r, s: B[k_o + k_i, r, s])
+    rr = te.reduce_axis([0, R], name="rr")
+    rs = te.reduce_axis([0, S], name="rs")
+    P, Q = (pH - R) // stride + 1, (pW - S) // stride + 1
+    Conv = te.compute([N, C, 1, P, Q], lambda n, k_o, k_i, p, q: te.sum(
+        (Pad[n, k_o, p * stride + rr, q * stride + rs] * B_reshaped[k_o, k_i, rr, rs]).astype(out_dtype),
+        axis=[rr, rs]), name="Conv")
+    Reshaped = te.compute([N, C, P, Q], lambda n, k, p, q: Conv[n, k, 0, p, q], name="Reshaped")
+    return [A, B, Reshaped]
+
+
+def _subgraphs(net, layers):
+    return [SubGraph("%s:subgraph%d" % (net, i), ts, cnt, note) for i, (note, ts, cnt) in enumerate(layers)]
+
+
+def resnet50(batch=1, in_dtype="float16", out_dtype="float32", num_classes=1000):
+    """the convolutions and the classifier of ResNet-50 at 224x224 (the stride of a down-sampling
+    bottleneck on its 3x3, python/tvm/tensor_graph/testing/models/resnet.py:60-215), equal shapes merged"""
+    b, d = batch, (in_dtype, out_dtype)
+    layers = [("conv1 7x7/2 3->64 @224", conv2d_nchw(b, 3, 224, 224, 64, 7, 7, 2, 3, *d), 1)]
+    cin, hw = 64, 56
+    for stage, (mid, blocks) in enumerate([(64, 3), (128, 4), (256, 6), (512, 3)]):
+        cout, stride = 4 * mid, (1 if stage == 0 else 2)
+        layers += [
+            ("stage%d 1x1 %d->%d @%d" % (stage + 1, cin, mid, hw), conv2d_nchw(b, cin, hw, hw, mid, 1, 1, 1, 0, *d), 1),
+            ("stage%d 3x3/%d %d->%d @%d" % (stage + 1, stride, mid, mid, hw), conv2d_nchw(b, mid, hw, hw, mid, 3, 3, stride, 1, *d), 1),
+            ("stage%d 1x1/%d %d->%d @%d (shortcut)" % (stage + 1, stride, cin, cout, hw), conv2d_nchw(b, cin, hw, hw, cout, 1, 1, stride, 0, *d), 1),
+        ]
+        hw //= stride
+        layers += [
+            ("stage%d 1x1 %d->%d @%d" % (stage + 1, mid, cout, hw), conv2d_nchw(b, mid, hw, hw, cout, 1, 1, 1, 0, *d), blocks),
+            ("stage%d 1x1 %d->%d @%d" % (stage + 1, cout, mid, hw), conv2d_nchw(b, cout, hw, hw, mid, 1, 1, 1, 0, *d), blocks - 1),
+            ("stage%d 3x3 %d->%d @%d" % (stage + 1, mid, mid, hw), conv2d_nchw(b, mid, hw, hw, mid, 3, 3, 1, 1, *d), blocks - 1),
+        ]
+        cin = cout
+    layers.append(("fc 2048->%d" % num_classes, dense(b, num_classes, 2048, *d), 1))
+    return _subgraphs("resnet50", layers)
+
+
+def mobilenet_v1(batch=1, in_dtype="float16", out_dtype="float32", num_classes=1000):
+    """MobileNet-V1 at 224x224 (python/tvm/tensor_graph/testing/models/mobilenet_v1.py): the first
+    convolution, thirteen depthwise 3x3 + pointwise 1x1 pairs, the classifier"""
+    b, d = batch, (in_dtype, out_dtype)
+    layers = [("conv 3x3/2 3->32 @224", conv2d_nchw(b, 3, 224, 224, 32, 3, 3, 2, 1, *d), 1)]
+    cfg = [(32, 64, 1), (64, 128, 2), (128, 128, 1), (128, 256, 2), (256, 256, 1), (256, 512, 2)] + \
+          [(512, 512, 1)] * 5 + [(512, 1024, 2), (1024, 1024, 1)]
+    hw, seen = 112, {}
+    for cin, cout, stride in cfg:
+        key = (cin, cout, stride, hw)
+        if key in seen:
+            for i in seen[key]:
+                layers[i] = (layers[i][0], layers[i][1], layers[i][2] + 1)
+        else:
+            seen[key] = [len(layers), len(layers) + 1]
+            layers.append(("depthwise 3x3/%d %d @%d" % (stride, cin, hw),
+                           depthwise_conv2d_nchw(b, cin, hw, hw, 3, 3, stride, 1, *d), 1))
+            layers.append(("pointwise %d->%d @%d" % (cin, cout, hw // stride),
+                           conv2d_nchw(b, cin, hw // stride, hw // stride, cout, 1, 1, 1, 0, *d), 1))
+        hw //= stride
+    layers.append(("fc 1024->%d" % num_classes, dense(b, num_classes, 1024, *d), 1))
+    return _subgraphs("mobilenet_v1", layers)
+
+
+def bert_base(batch=1, seq=512, in_dtype="float16", out_dtype="float32", blocks=12, heads=12, d_model=768, d_ff=3072):
+    """the matrix products of BERT-base (benchmark/amos/mapping_bertbase_tensorcore.py:19-46;
+    python/tvm/tensor_graph/testing/models/transformer.py:290-303): per block four d_model x d_model
+    projections, the attention scores and context (batched over batch x heads), two feed-forward
+    layers"""
+    rows, d = batch * seq, (in_dtype, out_dtype)
+    layers = [
+        ("projection %d->%d (Q, K, V, O)" % (d_model, d_model), dense(rows, d_model, d_model, *d), 4 * blocks),
+        ("scores Q K^T, %d x (%d x %d x %d)" % (batch * heads, seq, seq, d_model // heads),
+         batched_matmul(batch * heads, seq, seq, d_model // heads, True, *d), blocks),
+        ("context P V, %d x (%d x %d x %d)" % (batch * heads, seq, d_model // heads, seq),
+         batched_matmul(batch * heads, seq, d_model // heads, seq, False, *d), blocks),
+        ("feed-forward %d->%d" % (d_model, d_ff), dense(rows, d_ff, d_model, *d), blocks),
+        ("feed-forward %d->%d" % (d_ff, d_model), dense(rows, d_model, d_ff, *d), blocks),
+    ]
+    return _subgraphs("bertbase", layers)
+
+
+NETWORKS = {"resnet18": None, "resnet50": resnet50, "mobilenet_v1": mobilenet_v1, "bertbase": bert_base}
 
 
 SKIPPED_RESNET18 = ("batch norm x20, ReLU x17, max pool, global average pool, residual additions x8: "
@@ -209,3 +311,6 @@ def evaluate_graph(multi_graph, sch_tensors, target="hip", dev_id=0, number=100,
             print("%s (%s) x%d: %.4f ms, %s" % (sg.name, sg.note, sg.count, ms, rows[-1][-1]), flush=True)
     evaluate_graph.last_rows = rows
     return total
+
+
+NETWORKS["resnet18"] = resnet18

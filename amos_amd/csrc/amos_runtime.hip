@@ -10,6 +10,7 @@
 
 #include "amos_mi355x.h"
 #include "conv_fprop_kernel.h"
+#include "depthwise_kernel.h"
 #include "gemm_tn_kernel.h"
 #include "igemm_instances.h"
 #include "mapper.h"
@@ -190,6 +191,9 @@ struct Plan {
   // GEMM operands copied K-contiguous into the workspace in front of the kernel
   int n_transposes;
   TransposeJob tr[2];
+  // depthwise convolution on the vector ALUs (0 = not used, else 1 + DW_* kind)
+  int dw;
+  DepthwiseParams dwp;
 };
 
 static int dtype_pair(int in_dtype, int out_dtype, int* dt) {
@@ -240,39 +244,6 @@ static int plan_gemm(Plan& pl, int op, const void* desc_any, const amos_gemm_des
                      int64_t batch, int64_t sa, int64_t sb, int64_t sc,
                      const amos_kernel_config_t* cfg, const void* A, const void* B, void* C,
                      void* workspace = nullptr, size_t ws_bytes = 0);
-
-// Which operands of a GEMM are copied into the workspace so that the direct-to-LDS kernel can run:
-// row-contiguous ones (a transposed A, a row-major B) are transposed, K-contiguous ones whose rows
-// are not whole, 16-byte aligned K steps are copied with the K steps zero-filled (a ragged K
-// concerns both operands: garbage times the other side's zeros could be a NaN).
-struct GemmRepack {
-  bool copy_a, copy_b;
-  int64_t Kp;              // K rounded up to whole K steps
-  int64_t bytes_a, bytes_b;
-  int64_t total() const { return bytes_a + bytes_b; }
-};
-static GemmRepack gemm_repack(const amos_gemm_desc_t& g, int64_t batch, bool a_unaligned, bool b_unaligned) {
-  GemmRepack r = {false, false, 0, 0, 0};
-  const int es = g.in_dtype == AMOS_I8 ? 1 : 2;
-  const int bke = 128 / es;
-  if (g.M <= 0 || g.N <= 0 || g.K <= 0 || batch <= 0 || batch >= 65536) return r;
-  const bool ragged = g.K % bke != 0;
-  const bool a_bad = !g.trans_a && ((g.lda * es) % 16 != 0 || a_unaligned);
-  const bool b_bad = g.trans_b && ((g.ldb * es) % 16 != 0 || b_unaligned);
-  const bool copy_a = g.trans_a || ragged || a_bad, copy_b = !g.trans_b || ragged || b_bad;
-  if (!copy_a && !copy_b) return r;
-  // below ~8 GFLOP the copies cost what the faster kernel gains; ~1 GFLOP where the register-staged
-  // kernel would have to load an operand element by element
-  const bool vectors = es == 2 && !a_bad && !b_bad && g.K % 8 == 0 &&
-                       (!g.trans_a || g.M % 8 == 0) && (g.trans_b || g.N % 8 == 0);
-  if (2.0 * (double)g.M * (double)g.N * (double)g.K * (double)batch < (vectors ? 8e9 : 1e9)) return r;
-  r.Kp = (g.K + bke - 1) / bke * bke;
-  r.copy_a = copy_a;
-  r.copy_b = copy_b;
-  if (copy_a) r.bytes_a = (batch * g.M * r.Kp * es + 255) / 256 * 256;
-  if (copy_b) r.bytes_b = (batch * g.N * r.Kp * es + 255) / 256 * 256;
-  return r;
-}
 
 // plan a GEMM on copies of its operands (see gemm_repack)
 static int plan_gemm_repacked(Plan& pl, int op, const amos_gemm_desc_t* d, const GemmRepack& rp, int64_t batch,
@@ -473,33 +444,52 @@ static int plan_conv(Plan& pl, int op, const amos_conv_desc_t* d, const amos_ker
     return set_error(AMOS_ERR_UNSUPPORTED, "conv extents above 2^31");
   if ((c.T - 1) * c.dil_d >= 1024 || (c.R - 1) * c.dil_h >= 1024 || (c.S - 1) * c.dil_w >= 1024)
     return set_error(AMOS_ERR_UNSUPPORTED, "dilated kernel extent above 1023");
-  // A 1x1(x1) window with unit stride and no padding is a matrix product as it stands:
-  // per image Y[K][DHW] = Wt[K][C] X[C][DHW] (NCDHW), or Y[NDHW][K] = X[NDHW][C] Wt[C][K]
-  // (channels innermost).  It runs on the GEMM kernels, vector loaders included, unless the
-  // patch-staged pipeline is asked for.
-  if (c.T == 1 && c.R == 1 && c.S == 1 && c.stride_d == 1 && c.stride_h == 1 && c.stride_w == 1 &&
-      c.pad_d == 0 && c.pad_h == 0 && c.pad_w == 0 && G == 1 &&
-      (!cfg || (cfg->pipeline != AMOS_PIPE_PATCH && cfg->pipeline != AMOS_PIPE_PATCH8))) {
-    const int64_t dhw = c.D * c.H * c.W;
-    amos_bgemm_desc_t b;
-    memset(&b, 0, sizeof(b));
-    b.g.in_dtype = c.in_dtype;
+  // A pointwise convolution runs on the GEMM kernels, vector loaders and operand copies
+  // included, unless the patch-staged pipeline is asked for.
+  amos_bgemm_desc_t b;
+  if ((!cfg || (cfg->pipeline != AMOS_PIPE_PATCH && cfg->pipeline != AMOS_PIPE_PATCH8)) && conv_as_gemm(c, op, &b)) {
     b.g.out_dtype = c.out_dtype;
-    b.g.K = c.C;
-    if (layout == AMOS_LAYOUT_NCHW) {
-      b.batch = c.N;
-      b.g.M = c.K; b.g.N = dhw;
-      b.g.lda = c.C; b.g.ldb = dhw; b.g.ldc = dhw;
-      b.stride_a = 0; b.stride_b = c.C * dhw; b.stride_c = c.K * dhw;
-      return plan_gemm(pl, AMOS_OP_BGEMM, &b, &b.g, b.batch, b.stride_a, b.stride_b, b.stride_c, cfg, Wt, X, Y,
-                       workspace, ws_bytes);
+    const bool w_first = layout == AMOS_LAYOUT_NCHW;
+    return plan_gemm(pl, AMOS_OP_BGEMM, &b, &b.g, b.batch, b.stride_a, b.stride_b, b.stride_c, cfg,
+                     w_first ? Wt : X, w_first ? X : Wt, Y, workspace, ws_bytes);
+  }
+  // Depthwise (one input channel per group): no reduction but over the window, so it runs on the
+  // vector ALUs as the byte mover it is, unless a matrix-core pipeline is asked for by name.
+  if (conv_is_depthwise(c) && (!cfg || cfg->pipeline == AMOS_PIPE_AUTO)) {
+    // (the 3x3 kinds assume one stride for rows and columns)
+    const bool win3 = c.R == 3 && c.S == 3 && c.dil_h == 1 && c.dil_w == 1 && c.stride_h == c.stride_w;
+    const int kind = win3 && c.stride_w == 1 ? DW_3x3_S1 : win3 && c.stride_w == 2 ? DW_3x3_S2 : DW_GENERIC;
+    const int64_t qgroups = (OQ + 3) / 4;
+    const int64_t pgroups = (OP + dw_rows_per_lane(kind) - 1) / dw_rows_per_lane(kind);
+    const int64_t items = c.N * c.K * OD * pgroups * qgroups;
+    if (fits_int(items) && fits_int(c.D * c.H * c.W) && fits_int(c.T * c.R * c.S) && fits_int(c.N) && fits_int(c.K)) {
+      DepthwiseParams& q = pl.dwp;
+      memset(&q, 0, sizeof(q));
+      q.x = (const char*)X; q.w = (const char*)Wt; q.y = (char*)Y;
+      q.N = (int)c.N; q.C = (int)c.C; q.D = (int)c.D; q.H = (int)c.H; q.W = (int)c.W;
+      q.K = (int)c.K; q.mult = (int)Kg;
+      q.T = (int)c.T; q.R = (int)c.R; q.S = (int)c.S;
+      q.OD = OD; q.OP = OP; q.OQ = OQ;
+      q.sd = c.stride_d; q.sh = c.stride_h; q.sw = c.stride_w;
+      q.pd = c.pad_d; q.ph = c.pad_h; q.pw = c.pad_w;
+      q.dd = c.dil_d; q.dh = c.dil_h; q.dw = c.dil_w;
+      q.qgroups = (int)qgroups;
+      q.pgroups = (int)pgroups;
+      q.items = (unsigned)items;
+      q.vec_store = OQ % 4 == 0 && aligned16(Y);
+      q.fd_qg = make_fast_div((uint32_t)qgroups);
+      q.fd_pg = make_fast_div((uint32_t)pgroups);
+      q.fd_od = make_fast_div((uint32_t)OD);
+      q.fd_k = make_fast_div((uint32_t)c.K);
+      q.fd_mult = make_fast_div((uint32_t)Kg);
+      pl.dw = 1 + kind;
+      memset(&pl.cfg, 0, sizeof(pl.cfg));
+      if (cfg) pl.cfg = *cfg;
+      memset(&pl.p, 0, sizeof(pl.p));
+      pl.batch = 1;
+      pl.split = 1;
+      return 0;
     }
-    b.batch = 1;
-    b.g.M = c.N * dhw; b.g.N = c.K;
-    b.g.lda = c.C; b.g.ldb = c.K; b.g.ldc = c.K;
-    b.stride_a = b.g.M * c.C; b.stride_b = c.C * c.K; b.stride_c = b.g.M * c.K;
-    return plan_gemm(pl, AMOS_OP_BGEMM, &b, &b.g, 1, b.stride_a, b.stride_b, b.stride_c, cfg, X, Wt, Y,
-                     workspace, ws_bytes);
   }
   const int es = pl.dt == DT_I8 ? 1 : 2;
   const int ce = 16 / es;
@@ -655,6 +645,7 @@ static int make_plan(Plan& pl, int op, const void* desc, const amos_kernel_confi
   pl.conv_ups = 0;
   pl.fill_once = 0;
   pl.n_transposes = 0;
+  pl.dw = 0;
   switch (op) {
     case AMOS_OP_GEMM:
       return plan_gemm(pl, op, desc, (const amos_gemm_desc_t*)desc, 1, 0, 0, 0, cfg, in0, in1, out, workspace,
@@ -751,6 +742,11 @@ static int launch(const Plan& pl, hipStream_t stream) {
     else
       hipLaunchKernelGGL(amos_transpose_kernel<unsigned short>, grid, dim3(256), 0, stream, j);
   }
+  if (pl.dw) {
+    launch_depthwise(pl.dt, pl.dw - 1, pl.dwp, stream);
+    HIP_TRY(hipGetLastError());
+    return 0;
+  }
   if (pl.tn_waves) return launch_tn(pl, stream);
   if (pl.conv_ups) return launch_conv(pl, stream);
   Instance* inst;
@@ -811,6 +807,7 @@ static int plan_epilogue(Plan& pl, int op, const void* desc, const amos_epilogue
   pl.p.epi = ep;
   pl.tn.epi = ep;
   pl.cv.epi = ep;
+  pl.dwp.epi = ep;
   return 0;
 }
 
@@ -978,19 +975,9 @@ size_t amos_workspace_bytes(int op, const void* desc, const amos_kernel_config_t
   int64_t need = conv_workspace_bytes(c, op);
   // a pointwise convolution runs as a matrix product; its row-contiguous operand (NCDHW
   // activations, [C][K] weights) may want a K-contiguous copy
-  const bool is2d = op == AMOS_OP_CONV2D;
-  if ((is2d || c.T == 1) && c.R == 1 && c.S == 1 && c.stride_h == 1 && c.stride_w == 1 && c.pad_h == 0 &&
-      c.pad_w == 0 && (is2d || (c.stride_d == 1 && c.pad_d == 0)) && c.groups <= 1 && c.N > 0 && c.N < 65536) {
-    const int64_t dhw = (is2d ? 1 : c.D) * c.H * c.W;
-    amos_gemm_desc_t g;
-    memset(&g, 0, sizeof(g));
-    g.in_dtype = c.in_dtype;
-    g.K = c.C;
-    g.trans_a = 0; g.trans_b = 0;
-    g.lda = c.C;
-    int64_t t;
-    if (c.layout == AMOS_LAYOUT_NCHW) { g.M = c.K; g.N = dhw; g.ldb = dhw; t = gemm_repack(g, c.N, false, false).total(); }
-    else { g.M = c.N * dhw; g.N = c.K; g.ldb = c.K; t = gemm_repack(g, 1, false, false).total(); }
+  amos_bgemm_desc_t b;
+  if (conv_as_gemm(c, op, &b) && b.batch < 65536) {
+    const int64_t t = gemm_repack(b.g, b.batch, false, false).total();
     if (t > need) need = t;
   }
   return (size_t)need;
@@ -1004,6 +991,7 @@ const char* amos_kernel_name(int op, const void* desc, const amos_kernel_config_
   // amos_workspace_bytes() gets
   static char dummy_ws[256] __attribute__((aligned(256)));
   if (make_plan(pl, op, desc, cfg, dummy, dummy, dummy, dummy_ws, (size_t)-1)) return nullptr;
+  if (pl.dw) return depthwise_name(pl.dt, pl.dw - 1);
   if (pl.conv_ups) {
     ConvInstance* ci = pick_conv(pl.dt, pl.cfg.tile_i, pl.cfg.tile_j, pl.conv_waves, pl.cv.pls, pl.conv_occ, pl.conv_w9);
     return ci ? ci->name : nullptr;

@@ -19,6 +19,70 @@ static int64_t conv_out(int64_t in, int pad, int dil, int64_t k, int stride) {
   return (in + 2 * (int64_t)pad - eff) / stride + 1;
 }
 
+GemmRepack gemm_repack(const amos_gemm_desc_t& g, int64_t batch, bool a_unaligned, bool b_unaligned) {
+  GemmRepack r = {false, false, 0, 0, 0};
+  const int es = g.in_dtype == AMOS_I8 ? 1 : 2;
+  const int bke = 128 / es;
+  if (g.M <= 0 || g.N <= 0 || g.K <= 0 || batch <= 0 || batch >= 65536) return r;
+  const bool ragged = g.K % bke != 0;
+  const bool a_bad = !g.trans_a && ((g.lda * es) % 16 != 0 || a_unaligned);
+  const bool b_bad = g.trans_b && ((g.ldb * es) % 16 != 0 || b_unaligned);
+  const bool copy_a = g.trans_a || ragged || a_bad, copy_b = !g.trans_b || ragged || b_bad;
+  if (!copy_a && !copy_b) return r;
+  // below ~8 GFLOP the copies cost what the faster kernel gains; ~1 GFLOP where the register-staged
+  // kernel would have to load an operand element by element
+  const bool vectors = es == 2 && !a_bad && !b_bad && g.K % 8 == 0 &&
+                       (!g.trans_a || g.M % 8 == 0) && (g.trans_b || g.N % 8 == 0);
+  if (2.0 * (double)g.M * (double)g.N * (double)g.K * (double)batch < (vectors ? 8e9 : 1e9)) return r;
+  r.Kp = (g.K + bke - 1) / bke * bke;
+  r.copy_a = copy_a;
+  r.copy_b = copy_b;
+  if (copy_a) r.bytes_a = (batch * g.M * r.Kp * es + 255) / 256 * 256;
+  if (copy_b) r.bytes_b = (batch * g.N * r.Kp * es + 255) / 256 * 256;
+  return r;
+}
+
+
+bool conv_is_depthwise(const amos_conv_desc_t& c) {
+  return c.groups > 1 && c.groups == c.C && c.layout == AMOS_LAYOUT_NCHW;
+}
+
+bool conv_as_gemm(const amos_conv_desc_t& c, int op, amos_bgemm_desc_t* out) {
+  const bool is2d = op == AMOS_OP_CONV2D;
+  const int64_t G = c.groups > 1 ? c.groups : 1;
+  if (!(is2d || (c.T == 1 && c.stride_d == 1 && c.pad_d == 0)) || c.R != 1 || c.S != 1 || c.stride_h != 1 ||
+      c.stride_w != 1 || c.pad_h != 0 || c.pad_w != 0 || G != 1 || c.N <= 0)
+    return false;
+  const int64_t dhw = (is2d ? 1 : c.D) * c.H * c.W;
+  amos_bgemm_desc_t& b = *out;
+  memset(&b, 0, sizeof(b));
+  b.g.in_dtype = c.in_dtype;
+  b.g.out_dtype = c.out_dtype;
+  b.g.K = c.C;
+  if (c.layout == AMOS_LAYOUT_NCHW) {
+    b.batch = c.N;
+    b.g.M = c.K; b.g.N = dhw;
+    b.g.lda = c.C; b.g.ldb = dhw; b.g.ldc = dhw;
+    b.stride_a = 0; b.stride_b = c.C * dhw; b.stride_c = c.K * dhw;
+    return true;
+  }
+  b.batch = 1;
+  b.g.M = c.N * dhw; b.g.N = c.K;
+  b.g.lda = c.C; b.g.ldb = c.K; b.g.ldc = c.K;
+  b.stride_a = b.g.M * c.C; b.stride_b = c.C * c.K; b.stride_c = b.g.M * c.K;
+  return true;
+}
+
+// what the copies of gemm_repack cost: each reads and writes its operand once at about a third of
+// the HBM rate (64x64 blocks through LDS), plus a launch
+static void note_repack(Problem* pb, const amos_gemm_desc_t& g, int64_t batch) {
+  const GemmRepack rp = gemm_repack(g, batch, false, false);
+  if (rp.total() <= 0) return;
+  pb->repack = 1;
+  pb->Kp = rp.Kp;
+  pb->repack_seconds = 2.0 * (double)rp.total() / 2.5e12 + 2.5e-6 * ((rp.copy_a ? 1 : 0) + (rp.copy_b ? 1 : 0));
+}
+
 int problem_of(int op, const void* desc, Problem* out) {
   if (!desc || !out) return set_error(AMOS_ERR_BAD_ARG, "null descriptor");
   memset(out, 0, sizeof(*out));
@@ -53,6 +117,7 @@ int problem_of(int op, const void* desc, Problem* out) {
       }
       out->in_bytes = batch * (g->M * g->K + g->K * g->N) * esize(g->in_dtype);
       out->out_bytes = batch * g->M * g->N * 4;
+      note_repack(out, *g, batch);
       return 0;
     }
     case AMOS_OP_CONV2D:
@@ -93,6 +158,8 @@ int problem_of(int op, const void* desc, Problem* out) {
           out->row_loader = (wide && c->K % 8 == 0 && vec) ? 3 : 1;
           out->col_loader = (vec && out->row_loader == 3) ? 0 : 1;
         }
+        amos_bgemm_desc_t b;
+        if (conv_as_gemm(*c, op, &b)) note_repack(out, b.g, b.batch);
       }
       return 0;
     }
@@ -345,6 +412,9 @@ static const TileCost kDirectCost[] = {
     {256, 256, 1, 1.85, 1.65, 4.0}, {128, 256, 1, 1.06, 0.95, 2.0}, {256, 128, 1, 1.05, 0.92, 2.0},
     {128, 128, 2, 0.56, 0.70, 1.0}};
 
+// the direct kernel's tiles in the order plan_gemm_repacked() tries them
+static const int kRepackTiles[4][2] = {{256, 256}, {128, 128}, {128, 256}, {256, 128}};
+
 static double loader_factor(int loader) {
   switch (loader) {
     case 1: return 3.0;    // element loads: 8 (fp16) or 16 (int8) per 16-byte chunk
@@ -361,13 +431,14 @@ static double estimate_seconds(const Problem& pb, int ti, int tj, int split, boo
     if (t.ti == ti && t.tj == tj) tc = &t;
   if (!tc) return 1e9;
   bool direct = false;
-  if (allow_direct && pb.direct_ok && split == 1)
+  const bool repacked = allow_direct && pb.repack;    // the kernel runs on K-contiguous copies
+  if (allow_direct && (pb.direct_ok || repacked) && split == 1)
     for (auto& t : kDirectCost)
       if (t.ti == ti && t.tj == tj) { tc = &t; direct = true; }
-  const double k_tiles = std::ceil((double)pb.K / (128.0 / es));
+  const double k_tiles = std::ceil((double)(repacked ? pb.Kp : pb.K) / (128.0 / es));
   const int eff_split = (int)std::min<double>(split, k_tiles);
   const double ksteps = std::ceil(k_tiles / eff_split);
-  const double lf = direct ? 1.0 : loader_factor(pb.row_loader) * loader_factor(pb.col_loader);
+  const double lf = (direct || repacked) ? 1.0 : loader_factor(pb.row_loader) * loader_factor(pb.col_loader);
   const double tau = tc->tau_us * lf, alone = tc->alone_us * lf;
   const int64_t blocks = ((pb.I + ti - 1) / ti) * ((pb.J + tj - 1) / tj) * pb.batch * eff_split;
   const int64_t per_cu = (blocks + Gfx950::kComputeUnits - 1) / Gfx950::kComputeUnits;
@@ -375,7 +446,7 @@ static double estimate_seconds(const Problem& pb, int ti, int tj, int split, boo
   double step_us = (double)groups * std::max(alone, tc->occ * tau);
   if (rest) step_us += std::max(alone, (double)rest * tau);
   const double rounds = (double)groups + (rest ? 1.0 : 0.0);
-  double t = 3e-6 + (ksteps * step_us + rounds * tc->fixed_us) * 1e-6;
+  double t = 3e-6 + (ksteps * step_us + rounds * tc->fixed_us) * 1e-6 + (repacked ? pb.repack_seconds : 0.0);
   // output: written once; a split-K launch zero-fills it and accumulates with atomics (measured:
   // (1 + 2*split) passes over the output at ~3.5 TB/s)
   if (eff_split > 1) t += (double)pb.out_bytes * (1.0 + 2.0 * eff_split) / 3.5e12;
@@ -459,6 +530,16 @@ int amos_estimate_seconds(int op, const void* desc, const amos_kernel_config_t* 
   rc = amos_check_config(op, desc, cfg, nullptr, nullptr);
   if (rc) return rc;
   const int split = cfg->split_k < 1 ? 1 : cfg->split_k;
+  if ((op == AMOS_OP_CONV2D || op == AMOS_OP_CONV3D) && cfg->pipeline == AMOS_PIPE_AUTO &&
+      conv_is_depthwise(*(const amos_conv_desc_t*)desc)) {
+    // bytes in and out at about a third of the HBM rate (element loads), plus a launch
+    *seconds = ((double)pb.in_bytes + (double)pb.out_bytes) / (0.35 * Gfx950::kHbmBytesPerSec) + 3e-6;
+    return 0;
+  }
+  amos_bgemm_desc_t as_gemm;
+  if ((op == AMOS_OP_CONV2D || op == AMOS_OP_CONV3D) && cfg->pipeline != AMOS_PIPE_PATCH &&
+      cfg->pipeline != AMOS_PIPE_PATCH8 && conv_as_gemm(*(const amos_conv_desc_t*)desc, op, &as_gemm))
+    return amos_estimate_seconds(AMOS_OP_BGEMM, &as_gemm, cfg, seconds);   // what the launch runs
   if ((op == AMOS_OP_CONV2D || op == AMOS_OP_CONV3D) && cfg->pipeline != AMOS_PIPE_STAGED) {
     const int waves = cfg->pipeline == AMOS_PIPE_PATCH ? 4 : cfg->pipeline == AMOS_PIPE_PATCH8 ? 8 : 0;
     double s = conv_patch_estimate(*(const amos_conv_desc_t*)desc, op, pb, cfg->tile_i, cfg->tile_j, split,
@@ -475,6 +556,16 @@ int amos_default_config(int op, const void* desc, amos_kernel_config_t* result) 
   int rc = problem_of(op, desc, &pb);
   if (rc) return rc;
   if (!result) return set_error(AMOS_ERR_BAD_ARG, "null config");
+  // a depthwise convolution runs on the vector ALUs, whatever the tile
+  if ((op == AMOS_OP_CONV2D || op == AMOS_OP_CONV3D) && conv_is_depthwise(*(const amos_conv_desc_t*)desc)) {
+    memset(result, 0, sizeof(*result));
+    result->tile_i = 64; result->tile_j = 64; result->split_k = 1; result->pipeline = AMOS_PIPE_AUTO;
+    return 0;
+  }
+  // a pointwise convolution runs as a batched matrix product: that product's configuration
+  amos_bgemm_desc_t as_gemm;
+  if ((op == AMOS_OP_CONV2D || op == AMOS_OP_CONV3D) && conv_as_gemm(*(const amos_conv_desc_t*)desc, op, &as_gemm))
+    return amos_default_config(AMOS_OP_BGEMM, &as_gemm, result);
   memset(result, 0, sizeof(*result));
   amos_kernel_config_t* out = result;
   const double es = pb.in_dtype == AMOS_I8 ? 1.0 : 2.0;
@@ -517,6 +608,20 @@ int amos_default_config(int op, const void* desc, amos_kernel_config_t* result) 
     }
   }
   *result = staged;
+  // operands that get copied for the direct-to-LDS kernel: the best of its tiles, as a launch
+  // without a config takes it
+  if (pb.repack && result->pipeline == AMOS_PIPE_AUTO) {
+    double best_direct = 1e30;
+    for (auto& t : kRepackTiles) {
+      const double s = estimate_seconds(pb, t[0], t[1], 1);
+      if (s < best_direct) {
+        best_direct = s;
+        result->tile_i = t[0];
+        result->tile_j = t[1];
+        result->split_k = 1;
+      }
+    }
+  }
   return 0;
 }
 

@@ -32,7 +32,31 @@ struct Problem {
   // along the rows transposed in registers
   int row_loader, col_loader;
   int direct_ok;                // the direct-to-LDS GEMM kernel applies (256x256 tile)
+  // the runtime copies operands into the caller's workspace first (see gemm_repack) unless the
+  // register-staged pipeline is asked for: K as the kernel then sees it, what the copies cost
+  int repack;
+  int64_t Kp;
+  double repack_seconds;
 };
+
+// Which operands of a GEMM are copied into the workspace so that the direct-to-LDS kernel can run:
+// row-contiguous ones (a transposed A, a row-major B) are transposed, K-contiguous ones whose rows
+// are not whole, 16-byte aligned K steps are copied with the K steps zero-filled (a ragged K
+// concerns both operands: garbage times the other side's zeros could be a NaN).
+struct GemmRepack {
+  bool copy_a, copy_b;
+  int64_t Kp;              // K rounded up to whole K steps
+  int64_t bytes_a, bytes_b;
+  int64_t total() const { return bytes_a + bytes_b; }
+};
+GemmRepack gemm_repack(const amos_gemm_desc_t& g, int64_t batch, bool a_unaligned, bool b_unaligned);
+// A 1x1(x1) window with unit stride, no padding and one group is a matrix product as it stands:
+// per image Y[K][DHW] = Wt[K][C] X[C][DHW] (NCDHW, batch = N, the weights shared), or
+// Y[NDHW][K] = X[NDHW][C] Wt[C][K] (channels innermost).  Fills *out and returns true for such a
+// convolution (out->g is the product with A = the weights resp. the activations).
+bool conv_as_gemm(const amos_conv_desc_t& c, int op, amos_bgemm_desc_t* out);
+// groups == input channels (NCDHW): runs on the vector ALUs unless a matrix-core pipeline is named
+bool conv_is_depthwise(const amos_conv_desc_t& c);
 
 int problem_of(int op, const void* desc, Problem* out);
 

@@ -242,32 +242,35 @@ def model_check():
     return out
 
 
-def network_report(trials=200):
-    """ResNet-18's convolutions and classifier through the network dispatcher (the flow of the
-    reference's benchmark/amos/mapping_resnet18_tensorcore.py): per layer the tuned kernel and its
-    time, and the sum over the network's 21 tensorisable layers"""
+def network_report(trials=200, networks=("resnet18", "resnet50", "mobilenet_v1", "bertbase"), batches=(1, 16)):
+    """The tensorisable layers of whole networks through the network dispatcher (the flow of the
+    reference's benchmark/amos/mapping_{resnet18,resnet50,mobilenetv1,bertbase}_tensorcore.py): per
+    distinct layer the tuned kernel and its time, and the sum over the network's layers"""
     import contextlib
     import io
     import tempfile
     from amos_amd import auto_tensorize as at
     out = []
-    for batch in (1, 16):
-        multi_graph = at.resnet18(batch=batch)
-        opt = at.MeasureOptions(target="hip", timeout=100, number=5, min_repeat_ms=10)
-        with tempfile.TemporaryDirectory() as log_dir:
-            dispatch = at.AutoScheduleMultiGraphDispatch
-            with contextlib.redirect_stdout(io.StringIO()):
-                tid = dispatch.add_graph_task("resnet18", multi_graph, opt, trials=trials, log_dir=log_dir,
-                                              transform_strict=False)
-                dispatch.auto_schedule(tid)
-                sch_tensors = dispatch.get_schedules(tid)
-                total = at.evaluate_graph(multi_graph, sch_tensors, "hip", 0, 20, False, min_repeat_ms=50)
-            rows = at.evaluate_graph.last_rows
-        flop = sum(r[4] * r[2] for r in rows)
-        out.append({"network": "resnet18", "batch": batch, "layers_ms": total, "flop": flop,
-                    "tflops": flop / (total * 1e-3) / 1e12,
-                    "layers": [{"name": r[0], "layer": r[1], "count": r[2], "ms": r[3], "flop": r[4], "kernel": r[5]}
-                               for r in rows]})
+    for name in networks:
+        for batch in batches:
+            multi_graph = at.NETWORKS[name](batch)
+            opt = at.MeasureOptions(target="hip", timeout=100, number=5, min_repeat_ms=10)
+            with tempfile.TemporaryDirectory() as log_dir:
+                dispatch = at.AutoScheduleMultiGraphDispatch
+                with contextlib.redirect_stdout(io.StringIO()):
+                    tid = dispatch.add_graph_task(name, multi_graph, opt, trials=trials, log_dir=log_dir,
+                                                  transform_strict=False)
+                    dispatch.auto_schedule(tid)
+                    sch_tensors = dispatch.get_schedules(tid)
+                    total = at.evaluate_graph(multi_graph, sch_tensors, "hip", 0, 20, False, min_repeat_ms=50)
+                rows = at.evaluate_graph.last_rows
+            flop = sum(r[4] * r[2] for r in rows)
+            out.append({"network": name, "batch": batch, "layers_ms": total, "flop": flop,
+                        "tflops": flop / (total * 1e-3) / 1e12,
+                        "layers": [{"name": r[0], "layer": r[1], "count": r[2], "ms": r[3], "flop": r[4],
+                                    "kernel": r[5]} for r in rows]})
+            print("network %s batch %d: %.3f ms over %d layers" % (name, batch, total, sum(r[2] for r in rows)),
+                  file=sys.stderr, flush=True)
     return out
 
 
@@ -282,8 +285,10 @@ def main():
                     help="also rank every kernel configuration of a set of shapes by the mapper's model "
                          "and by measurement, write JSON here")
     ap.add_argument("--network", default=None,
-                    help="also tune and time ResNet-18's tensorisable layers at batch 1 and 16 through the "
-                         "network dispatcher, write JSON here")
+                    help="also tune and time the tensorisable layers of ResNet-18, ResNet-50, MobileNet-V1 and "
+                         "BERT-base at batch 1 and 16 through the network dispatcher, write JSON here")
+    ap.add_argument("--networks", default="resnet18,resnet50,mobilenet_v1,bertbase",
+                    help="the networks --network covers, comma-separated")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a 256 MiB device copy, the known-size kernel that rocprofv3's "
                          "FETCH_SIZE / WRITE_SIZE readings are scaled by")
@@ -354,7 +359,7 @@ def main():
             json.dump(model_check(), f, indent=1)
     if args.network:
         with open(args.network, "w") as f:
-            json.dump(network_report(), f, indent=1)
+            json.dump(network_report(networks=tuple(args.networks.split(","))), f, indent=1)
     print(json.dumps(line), flush=True)
 
 

@@ -151,7 +151,9 @@ def test_grouped_conv(gpu, dtype, case):
                                         np.ascontiguousarray(w[g * kg:(g + 1) * kg]), dtype, st, pd, dl,
                                         acc="float64") for g in range(G)], axis=1)
     dx, dw = to_device(x, dtype), to_device(w, dtype)
-    for cfg in (None, dict(tile_i=64, tile_j=64, split_k=2)):
+    # (pipeline 1, the register-staged implicit GEMM, also for the depthwise cases, whose default is
+    # the vector-ALU kernel)
+    for cfg in (None, dict(tile_i=64, tile_j=64, split_k=2, pipeline=1)):
         if D == 1 and T == 1:
             got = ops.conv2d(dx[:, :, 0], dw[:, :, 0], st[1:], pd[1:], dl[1:], config=cfg, groups=G)[:, :, None]
         else:

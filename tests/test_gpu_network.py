@@ -57,3 +57,57 @@ def test_resnet18_dispatch(gpu, tmp_path, capsys):
             ref = co.lib_conv2d(feeds[0], feeds[1], "float16", stride, 1, 1, acc="float64")
         mx, mean = co.rel_errors(out.asnumpy(), ref)
         assert mx <= 1e-2 and mean <= 1e-3, (sg.name, mx, mean)
+
+
+def _by_note(multi_graph, text):
+    found = [sg for sg in multi_graph if text in sg.note]
+    assert found, text
+    return found[0]
+
+
+def test_other_networks_dispatch(gpu, tmp_path, capsys):
+    """layers of ResNet-50, MobileNet-V1 and BERT-base that ResNet-18 has no like of, through the
+    dispatcher: the 7x7 stem, a strided pointwise shortcut, depthwise 3x3 with and without a
+    stride, the attention products"""
+    r50, mb, bert = at.resnet50(2), at.mobilenet_v1(2), at.bert_base(1, seq=128)
+    picked = [_by_note(r50, "conv1 7x7/2"), _by_note(r50, "stage2 1x1/2 256->512 @56 (shortcut)"),
+              _by_note(r50, "stage4 1x1 2048->512 @7"),
+              _by_note(mb, "depthwise 3x3/2 64 @112"), _by_note(mb, "depthwise 3x3/1 512 @14"),
+              _by_note(mb, "pointwise 512->1024 @7"),
+              _by_note(bert, "scores"), _by_note(bert, "context"), _by_note(bert, "feed-forward 3072->768")]
+    opt = at.MeasureOptions(target="hip", timeout=100, number=3, min_repeat_ms=2)
+    dispatch = at.AutoScheduleMultiGraphDispatch
+    tid = dispatch.add_graph_task("mixed", picked, opt, trials=2, log_dir=str(tmp_path), transform_strict=False)
+    dispatch.auto_schedule(tid)
+    assert dispatch.ready(tid)
+    sch_tensors = dispatch.get_schedules(tid)
+    capsys.readouterr()
+    rng = np.random.default_rng(29)
+    ctx = tvm.context("hip", 0)
+    for sg in picked:
+        sch, args, _ = sch_tensors[sg.name]
+        func = tvm.build(sch, args, "hip")
+        feeds = [rng.uniform(-1, 1, [int(e) for e in t.shape]).astype(np.float16) for t in args[:-1]]
+        out = tvm.nd.array(np.zeros([int(e) for e in args[-1].shape], dtype=np.float32), ctx)
+        func(*[tvm.nd.array(f, ctx) for f in feeds], out)
+        ctx.sync()
+        a, b = [f.astype(np.float64) for f in feeds]
+        if "depthwise" in sg.note:
+            stride = 2 if "/2" in sg.note else 1
+            ap = np.pad(a, ((0, 0), (0, 0), (1, 1), (1, 1)))
+            p, q = out.shape[2], out.shape[3]
+            ref = sum(ap[:, :, r:r + stride * (p - 1) + 1:stride, s:s + stride * (q - 1) + 1:stride] *
+                      b[None, :, r, s, None, None] for r in range(3) for s in range(3))
+        elif "scores" in sg.note:
+            ref = np.einsum("bik,bjk->bij", a, b)
+        elif "context" in sg.note:
+            ref = np.einsum("bik,bkj->bij", a, b)
+        elif "feed-forward" in sg.note:
+            ref = a @ b.T
+        else:
+            stride = 2 if "/2" in sg.note else 1
+            ref = co.lib_conv2d(feeds[0], feeds[1], "float16", stride, 3 if "7x7" in sg.note else 0, 1, acc="float64")
+        mx, mean = co.rel_errors(out.asnumpy(), ref)
+        assert mx <= 1e-2 and mean <= 1e-3, (sg.note, mx, mean)
+    cost = at.evaluate_graph(picked, sch_tensors, "hip", 0, 5, False, min_repeat_ms=2)
+    assert len(at.evaluate_graph.last_rows) == len(picked) and 0 < cost < 50

@@ -649,6 +649,59 @@ def test_conv3d_config5b(gpu):
     check_float(full[5:6].cpu().numpy(), ref0, "C5b image 5 vs fp32 (64x128)")
 
 
+DEPTHWISE_CASES = [
+    # N, C, D, H, W, mult, T, R, S, stride, pad, dil, kernel-name suffix
+    (2, 32, 1, 28, 28, 1, 1, 3, 3, (1, 1, 1), (0, 1, 1), (1, 1, 1), ",3x3>"),       # MobileNet's 3x3
+    (3, 24, 1, 29, 31, 1, 1, 3, 3, (1, 2, 2), (0, 1, 1), (1, 1, 1), ",3x3/2>"),     # strided, ragged rows
+    (1, 16, 1, 7, 7, 2, 1, 3, 3, (1, 1, 1), (0, 1, 1), (1, 1, 1), ",3x3>"),         # two outputs per channel
+    (2, 8, 1, 20, 18, 1, 1, 5, 5, (1, 2, 1), (0, 2, 2), (1, 1, 1), ">"),            # 5x5
+    (2, 8, 1, 17, 19, 3, 1, 3, 3, (1, 1, 1), (0, 2, 2), (1, 2, 2), ">"),            # dilated
+    (2, 6, 5, 9, 12, 1, 3, 3, 3, (1, 1, 1), (1, 1, 1), (1, 1, 1), ",3x3>"),         # 3-D
+    (1, 5, 4, 6, 10, 2, 2, 2, 3, (2, 1, 2), (1, 0, 1), (1, 2, 1), ">"),             # 3-D, uneven everything
+    (1, 4, 1, 1, 3, 1, 1, 3, 3, (1, 1, 1), (0, 1, 1), (1, 1, 1), ",3x3>"),          # one output row of 3
+]
+
+
+@pytest.mark.parametrize("dtype", ["float16", "bfloat16", "int8"])
+@pytest.mark.parametrize("case", DEPTHWISE_CASES)
+def test_depthwise_conv(gpu, dtype, case):
+    """depthwise convolution (reference compute: benchmark/amos/mapping_depthwiseconv2d_tensorcore.py:7-48)
+    on the vector-ALU kernel: against the oracle run once per channel, and against the
+    register-staged implicit GEMM of the same op (bit for bit for int8)"""
+    from amos_amd import _lib, ops
+    N, C, D, H, W, mult, T, R, S, st, pd, dl, suffix = case
+    K = C * mult
+    rng = np.random.default_rng(hash(case[:-1]) % 2**32)
+    x = make_operand(rng, (N, C, D, H, W), dtype, "normal")
+    w = make_operand(rng, (K, 1, T, R, S), dtype, "normal")
+    ref = np.concatenate([co.lib_conv3d(np.ascontiguousarray(x[:, c:c + 1]),
+                                        np.ascontiguousarray(w[c * mult:(c + 1) * mult]), dtype, st, pd, dl,
+                                        acc="float64") for c in range(C)], axis=1)
+    dx, dw = to_device(x, dtype), to_device(w, dtype)
+    desc = ops.conv_desc((N, C, D, H, W), (K, 1, T, R, S), dx.dtype, st, pd, dl, C)
+    name = ops.kernel_name(_lib.AMOS_OP_CONV3D, desc, None)
+    assert name.startswith("amos_depthwise_conv<") and name.endswith(suffix), name
+    got = ops.conv3d(dx, dw, st, pd, dl, groups=C).cpu().numpy()
+    check(got, ref, dtype, "depthwise %s %s" % (dtype, case))
+    staged = dict(tile_i=64, tile_j=64, split_k=1, pipeline=1)
+    assert ops.kernel_name(_lib.AMOS_OP_CONV3D, desc, staged).startswith("amos_igemm<")
+    other = ops.conv3d(dx, dw, st, pd, dl, groups=C, config=staged).cpu().numpy()
+    if dtype == "int8":
+        assert np.array_equal(got, other)
+    else:
+        check_float(got, other, "depthwise vs implicit GEMM %s %s" % (dtype, case))
+    # the default configuration named explicitly is the same launch
+    cfg = ops.default_config(_lib.AMOS_OP_CONV3D, desc)
+    assert cfg.pipeline == 0 and ops.kernel_name(_lib.AMOS_OP_CONV3D, desc, cfg) == name
+    # a misaligned output takes element stores
+    flat = np.zeros(got.size + 1, dtype=got.dtype)
+    import torch
+    buf = torch.from_numpy(flat).cuda()
+    out = buf[1:].view(got.shape)
+    ops.conv3d(dx, dw, st, pd, dl, groups=C, out=out)
+    assert np.array_equal(out.cpu().numpy(), got) and int(buf[0]) == 0
+
+
 def test_errors(gpu):
     import torch
     from amos_amd import _lib, ops

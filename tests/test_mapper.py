@@ -750,3 +750,26 @@ def test_grouped_and_depthwise_conv_lowering(build, groups):
                                                    b.shape[-2], b.shape[-1])
     got = grouped_conv_reference(a, b, (c.stride_h, c.stride_w), (c.pad_h, c.pad_w), groups)
     assert np.array_equal(got, want)
+
+
+def test_other_networks_layer_lists():
+    """layer counts and multiply-accumulate totals of the other networks the reference maps
+    (benchmark/amos/mapping_{resnet50,mobilenetv1,bertbase}_tensorcore.py) against the published
+    figures of the architectures: ResNet-50 4.09 G, MobileNet-V1 0.57 G multiply-accumulates at
+    224x224; BERT-base at 512 tokens 12 x (4 x 512 x 768^2 + 2 x 512 x 768 x 3072 + 2 x 12 x 512^2 x 64)"""
+    from amos_amd import auto_tensorize as _at
+
+    def macs(mg):
+        total = 0
+        for sg in mg:
+            main = [op for op in sg.dag.op_lst if op.reduce_axis][0]
+            total += _at.lower_main_op(main, sg.dag).flops() // 2 * sg.count
+        return total
+    r50 = _at.resnet50(1)
+    assert sum(sg.count for sg in r50) == 54 and abs(macs(r50) / 4.09e9 - 1) < 0.01    # 53 convolutions + fc
+    mb = _at.mobilenet_v1(1)
+    assert sum(sg.count for sg in mb) == 28 and abs(macs(mb) / 0.569e9 - 1) < 0.01    # 1 + 13 x 2 + fc
+    bert = _at.bert_base(1)
+    assert sum(sg.count for sg in bert) == 96
+    assert macs(bert) == 12 * (4 * 512 * 768 ** 2 + 2 * 512 * 768 * 3072 + 2 * 12 * 512 ** 2 * 64)
+    assert set(_at.NETWORKS) == {"resnet18", "resnet50", "mobilenet_v1", "bertbase"}
