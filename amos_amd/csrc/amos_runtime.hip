@@ -75,6 +75,11 @@ struct TransposeJob {
   int batch;
   int ld_dst;              // >= rows; the result's rows are zero-filled from `rows` up to it
   int copy;                // 1: no transposition, dst[r][k] = src[r][k] (k < cols), zero up to ld_dst
+  // col_w > 0: column c of the source is the element (c / col_w) * col_so + (c % col_w) * col_si
+  // of its row (every stride-th pixel of an image plane); 0: the element c
+  int col_w, col_si;
+  int64_t col_so;
+  FastDiv fd_col_w;
 };
 template <typename T>
 __global__ __launch_bounds__(256) void amos_transpose_kernel(const TransposeJob j) {
@@ -87,8 +92,13 @@ __global__ __launch_bounds__(256) void amos_transpose_kernel(const TransposeJob 
   T* dst = (T*)j.dst + (int64_t)blockIdx.z * j.batch_dst;
   constexpr int LT = 64 / VE;                 // threads per 64-element row
   constexpr int RPP = 256 / LT;               // rows per pass
-  const bool vec_in = (((uintptr_t)src | (uintptr_t)(j.ld_src * sizeof(T))) & 7) == 0;
+  const bool vec_in = (((uintptr_t)src | (uintptr_t)(j.ld_src * sizeof(T))) & 7) == 0 && j.col_w == 0;
   const int lc = (t % LT) * VE, lr = t / LT;
+  auto col_at = [&](int c) -> int64_t {
+    if (j.col_w == 0) return c;
+    const int outer = fast_div(c, j.fd_col_w);
+    return outer * j.col_so + (int64_t)(c - outer * j.col_w) * j.col_si;
+  };
 #pragma unroll
   for (int pass = 0; pass < 64 / RPP; ++pass) {
     const int r = lr + pass * RPP;
@@ -98,7 +108,8 @@ __global__ __launch_bounds__(256) void amos_transpose_kernel(const TransposeJob 
       *(uint2*)v = *(const uint2*)(src + (int64_t)gr * j.ld_src + gc);
     } else {
 #pragma unroll
-      for (int e = 0; e < VE; ++e) v[e] = (gr < j.rows && gc + e < j.cols) ? src[(int64_t)gr * j.ld_src + gc + e] : (T)0;
+      for (int e = 0; e < VE; ++e)
+        v[e] = (gr < j.rows && gc + e < j.cols) ? src[(int64_t)gr * j.ld_src + col_at(gc + e)] : (T)0;
     }
 #pragma unroll
     for (int e = 0; e < VE; ++e) tile[(lc + e) * PITCH + r] = v[e];     // transposed into LDS
@@ -248,7 +259,8 @@ static int plan_gemm(Plan& pl, int op, const void* desc_any, const amos_gemm_des
 // plan a GEMM on copies of its operands (see gemm_repack)
 static int plan_gemm_repacked(Plan& pl, int op, const amos_gemm_desc_t* d, const GemmRepack& rp, int64_t batch,
                               int64_t sa, int64_t sb, int64_t sc, const amos_kernel_config_t* cfg,
-                              const void* A, const void* B, void* C, void* workspace) {
+                              const void* A, const void* B, void* C, void* workspace,
+                              const ConvSubsample* sub = nullptr) {
   amos_bgemm_desc_t e;
   memset(&e, 0, sizeof(e));
   e.g = *d;
@@ -269,9 +281,15 @@ static int plan_gemm_repacked(Plan& pl, int op, const amos_gemm_desc_t* d, const
     e.g.trans_a = 0; e.g.lda = rp.Kp; e.stride_a = d->M * rp.Kp;
   }
   if (rp.copy_b) {
-    if (!d->trans_b)  // stored [K][N] -> [N][Kp]
+    if (!d->trans_b) {  // stored [K][N] -> [N][Kp]
       jobs[n++] = TransposeJob{(const char*)B, ws, (int)d->K, (int)d->N, d->ldb, sb, d->N * rp.Kp, (int)batch, (int)rp.Kp, 0};
-    else
+      if (sub) {        // the logical row is gathered from an image plane
+        TransposeJob& j = jobs[n - 1];
+        j.ld_src = sub->chan_step;
+        j.col_w = sub->out_w; j.col_si = sub->col_step; j.col_so = sub->row_step;
+        j.fd_col_w = make_fast_div((uint32_t)sub->out_w);
+      }
+    } else
       jobs[n++] = TransposeJob{(const char*)B, ws, (int)d->N, (int)d->K, d->ldb, sb, d->N * rp.Kp, (int)batch, (int)rp.Kp, 1};
     B2 = ws;
     e.g.trans_b = 1; e.g.ldb = rp.Kp; e.stride_b = d->N * rp.Kp;
@@ -452,6 +470,18 @@ static int plan_conv(Plan& pl, int op, const amos_conv_desc_t* d, const amos_ker
     const bool w_first = layout == AMOS_LAYOUT_NCHW;
     return plan_gemm(pl, AMOS_OP_BGEMM, &b, &b.g, b.batch, b.stride_a, b.stride_b, b.stride_c, cfg,
                      w_first ? Wt : X, w_first ? X : Wt, Y, workspace, ws_bytes);
+  }
+  // ... and with a stride where the copy that makes the activations K-contiguous pays: it picks
+  // every stride-th pixel on its way
+  ConvSubsample sub;
+  if ((!cfg || conv_subsample_pipeline(cfg->pipeline)) && workspace && ((uintptr_t)workspace & 255) == 0 &&
+      conv_as_subsampled_gemm(c, op, &b, &sub)) {
+    const GemmRepack rp = gemm_repack(b.g, b.batch, !aligned16(Wt), false, true);
+    if (ws_bytes >= (size_t)rp.total()) {
+      b.g.out_dtype = c.out_dtype;
+      return plan_gemm_repacked(pl, AMOS_OP_BGEMM, &b.g, rp, b.batch, b.stride_a, b.stride_b, b.stride_c, cfg,
+                                Wt, X, Y, workspace, &sub);
+    }
   }
   // Depthwise (one input channel per group): no reduction but over the window, so it runs on the
   // vector ALUs as the byte mover it is, unless a matrix-core pipeline is asked for by name.
@@ -978,6 +1008,9 @@ size_t amos_workspace_bytes(int op, const void* desc, const amos_kernel_config_t
   amos_bgemm_desc_t b;
   if (conv_as_gemm(c, op, &b) && b.batch < 65536) {
     const int64_t t = gemm_repack(b.g, b.batch, false, false).total();
+    if (t > need) need = t;
+  } else if ((!cfg || conv_subsample_pipeline(cfg->pipeline)) && conv_as_subsampled_gemm(c, op, &b, nullptr)) {
+    const int64_t t = gemm_repack(b.g, b.batch, false, false, true).total();
     if (t > need) need = t;
   }
   return (size_t)need;

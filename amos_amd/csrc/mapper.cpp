@@ -19,7 +19,8 @@ static int64_t conv_out(int64_t in, int pad, int dil, int64_t k, int stride) {
   return (in + 2 * (int64_t)pad - eff) / stride + 1;
 }
 
-GemmRepack gemm_repack(const amos_gemm_desc_t& g, int64_t batch, bool a_unaligned, bool b_unaligned) {
+GemmRepack gemm_repack(const amos_gemm_desc_t& g, int64_t batch, bool a_unaligned, bool b_unaligned,
+                       bool b_gathered) {
   GemmRepack r = {false, false, 0, 0, 0};
   const int es = g.in_dtype == AMOS_I8 ? 1 : 2;
   const int bke = 128 / es;
@@ -27,11 +28,11 @@ GemmRepack gemm_repack(const amos_gemm_desc_t& g, int64_t batch, bool a_unaligne
   const bool ragged = g.K % bke != 0;
   const bool a_bad = !g.trans_a && ((g.lda * es) % 16 != 0 || a_unaligned);
   const bool b_bad = g.trans_b && ((g.ldb * es) % 16 != 0 || b_unaligned);
-  const bool copy_a = g.trans_a || ragged || a_bad, copy_b = !g.trans_b || ragged || b_bad;
+  const bool copy_a = g.trans_a || ragged || a_bad, copy_b = !g.trans_b || ragged || b_bad || b_gathered;
   if (!copy_a && !copy_b) return r;
   // below ~8 GFLOP the copies cost what the faster kernel gains; ~1 GFLOP where the register-staged
   // kernel would have to load an operand element by element
-  const bool vectors = es == 2 && !a_bad && !b_bad && g.K % 8 == 0 &&
+  const bool vectors = es == 2 && !a_bad && !b_bad && !b_gathered && g.K % 8 == 0 &&
                        (!g.trans_a || g.M % 8 == 0) && (g.trans_b || g.N % 8 == 0);
   if (2.0 * (double)g.M * (double)g.N * (double)g.K * (double)batch < (vectors ? 8e9 : 1e9)) return r;
   r.Kp = (g.K + bke - 1) / bke * bke;
@@ -42,6 +43,10 @@ GemmRepack gemm_repack(const amos_gemm_desc_t& g, int64_t batch, bool a_unaligne
   return r;
 }
 
+
+bool conv_subsample_pipeline(int pipeline) {
+  return pipeline == AMOS_PIPE_AUTO || pipeline == AMOS_PIPE_DIRECT4 || pipeline == AMOS_PIPE_DIRECT8;
+}
 
 bool conv_is_depthwise(const amos_conv_desc_t& c) {
   return c.groups > 1 && c.groups == c.C && c.layout == AMOS_LAYOUT_NCHW;
@@ -73,10 +78,37 @@ bool conv_as_gemm(const amos_conv_desc_t& c, int op, amos_bgemm_desc_t* out) {
   return true;
 }
 
+bool conv_as_subsampled_gemm(const amos_conv_desc_t& c, int op, amos_bgemm_desc_t* out, ConvSubsample* sub) {
+  const bool flat = op == AMOS_OP_CONV2D || (c.D == 1 && c.T == 1 && c.pad_d == 0);
+  const int64_t G = c.groups > 1 ? c.groups : 1;
+  if (!flat || c.R != 1 || c.S != 1 || c.pad_h != 0 || c.pad_w != 0 || G != 1 || c.N <= 0 ||
+      c.layout != AMOS_LAYOUT_NCHW || c.stride_h < 1 || c.stride_w < 1 || (c.stride_h == 1 && c.stride_w == 1) ||
+      c.H <= 0 || c.W <= 0)
+    return false;
+  const int64_t OP = (c.H - 1) / c.stride_h + 1, OQ = (c.W - 1) / c.stride_w + 1;
+  if (OP * OQ >= (1ll << 31) || c.H * c.W >= (1ll << 31)) return false;
+  amos_bgemm_desc_t& b = *out;
+  memset(&b, 0, sizeof(b));
+  b.g.in_dtype = c.in_dtype;
+  b.g.out_dtype = c.out_dtype;
+  b.batch = c.N;
+  b.g.M = c.K; b.g.N = OP * OQ; b.g.K = c.C;
+  b.g.lda = c.C; b.g.ldb = OP * OQ; b.g.ldc = OP * OQ;
+  b.stride_a = 0; b.stride_b = c.C * c.H * c.W; b.stride_c = c.K * OP * OQ;
+  if (gemm_repack(b.g, b.batch, false, false, true).total() <= 0) return false;
+  if (sub) {
+    sub->out_w = (int)OQ;
+    sub->row_step = (int64_t)c.stride_h * c.W;
+    sub->col_step = c.stride_w;
+    sub->chan_step = c.H * c.W;
+  }
+  return true;
+}
+
 // what the copies of gemm_repack cost: each reads and writes its operand once at about a third of
 // the HBM rate (64x64 blocks through LDS), plus a launch
-static void note_repack(Problem* pb, const amos_gemm_desc_t& g, int64_t batch) {
-  const GemmRepack rp = gemm_repack(g, batch, false, false);
+static void note_repack(Problem* pb, const amos_gemm_desc_t& g, int64_t batch, bool b_gathered = false) {
+  const GemmRepack rp = gemm_repack(g, batch, false, false, b_gathered);
   if (rp.total() <= 0) return;
   pb->repack = 1;
   pb->Kp = rp.Kp;
@@ -540,6 +572,15 @@ int amos_estimate_seconds(int op, const void* desc, const amos_kernel_config_t* 
   if ((op == AMOS_OP_CONV2D || op == AMOS_OP_CONV3D) && cfg->pipeline != AMOS_PIPE_PATCH &&
       cfg->pipeline != AMOS_PIPE_PATCH8 && conv_as_gemm(*(const amos_conv_desc_t*)desc, op, &as_gemm))
     return amos_estimate_seconds(AMOS_OP_BGEMM, &as_gemm, cfg, seconds);   // what the launch runs
+  if ((op == AMOS_OP_CONV2D || op == AMOS_OP_CONV3D) && conv_subsample_pipeline(cfg->pipeline) &&
+      conv_as_subsampled_gemm(*(const amos_conv_desc_t*)desc, op, &as_gemm, nullptr)) {
+    Problem pg;
+    rc = problem_of(AMOS_OP_BGEMM, &as_gemm, &pg);
+    if (rc) return rc;
+    note_repack(&pg, as_gemm.g, as_gemm.batch, true);
+    *seconds = estimate_seconds(pg, cfg->tile_i, cfg->tile_j, cfg->split_k < 1 ? 1 : cfg->split_k);
+    return 0;
+  }
   if ((op == AMOS_OP_CONV2D || op == AMOS_OP_CONV3D) && cfg->pipeline != AMOS_PIPE_STAGED) {
     const int waves = cfg->pipeline == AMOS_PIPE_PATCH ? 4 : cfg->pipeline == AMOS_PIPE_PATCH8 ? 8 : 0;
     double s = conv_patch_estimate(*(const amos_conv_desc_t*)desc, op, pb, cfg->tile_i, cfg->tile_j, split,
@@ -566,6 +607,27 @@ int amos_default_config(int op, const void* desc, amos_kernel_config_t* result) 
   amos_bgemm_desc_t as_gemm;
   if ((op == AMOS_OP_CONV2D || op == AMOS_OP_CONV3D) && conv_as_gemm(*(const amos_conv_desc_t*)desc, op, &as_gemm))
     return amos_default_config(AMOS_OP_BGEMM, &as_gemm, result);
+  // ... a strided one after its pixels are picked by the operand copy: the best direct tile
+  if ((op == AMOS_OP_CONV2D || op == AMOS_OP_CONV3D) &&
+      conv_as_subsampled_gemm(*(const amos_conv_desc_t*)desc, op, &as_gemm, nullptr)) {
+    Problem pg;
+    rc = problem_of(AMOS_OP_BGEMM, &as_gemm, &pg);
+    if (rc) return rc;
+    note_repack(&pg, as_gemm.g, as_gemm.batch, true);
+    memset(result, 0, sizeof(*result));
+    result->pipeline = AMOS_PIPE_AUTO;
+    double best_direct = 1e30;
+    for (auto& t : kRepackTiles) {
+      const double s = estimate_seconds(pg, t[0], t[1], 1);
+      if (s < best_direct) {
+        best_direct = s;
+        result->tile_i = t[0];
+        result->tile_j = t[1];
+        result->split_k = 1;
+      }
+    }
+    return 0;
+  }
   memset(result, 0, sizeof(*result));
   amos_kernel_config_t* out = result;
   const double es = pb.in_dtype == AMOS_I8 ? 1.0 : 2.0;

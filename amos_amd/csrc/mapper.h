@@ -49,12 +49,28 @@ struct GemmRepack {
   int64_t bytes_a, bytes_b;
   int64_t total() const { return bytes_a + bytes_b; }
 };
-GemmRepack gemm_repack(const amos_gemm_desc_t& g, int64_t batch, bool a_unaligned, bool b_unaligned);
+// b_gathered: B is not stored as the descriptor says but gathered by the copy (see
+// conv_as_subsampled_gemm): it is always copied
+GemmRepack gemm_repack(const amos_gemm_desc_t& g, int64_t batch, bool a_unaligned, bool b_unaligned,
+                       bool b_gathered = false);
 // A 1x1(x1) window with unit stride, no padding and one group is a matrix product as it stands:
 // per image Y[K][DHW] = Wt[K][C] X[C][DHW] (NCDHW, batch = N, the weights shared), or
 // Y[NDHW][K] = X[NDHW][C] Wt[C][K] (channels innermost).  Fills *out and returns true for such a
 // convolution (out->g is the product with A = the weights resp. the activations).
 bool conv_as_gemm(const amos_conv_desc_t& c, int op, amos_bgemm_desc_t* out);
+// A 2-D 1x1 window with a stride (no padding, one group, NCHW) is the same product over every
+// stride-th pixel: X'[C][OP*OQ] with X'[c][p*OQ + q] = X[c][p*sh][q*sw].  The copy that makes the
+// activations K-contiguous for the direct-to-LDS kernel picks those pixels on its way, so the
+// route exists where that copy pays (gemm_repack's bar for element-wise loaded operands) and the
+// caller provides the workspace.  Fills *out like conv_as_gemm (ldb = OP*OQ, the logical row).
+struct ConvSubsample {
+  int out_w;           // OQ: logical column j = p * OQ + q
+  int64_t row_step;    // elements between source rows p: sh * W
+  int col_step;        // elements between source columns q: sw
+  int64_t chan_step;   // elements between channels (the source's leading dimension): H * W
+};
+bool conv_subsample_pipeline(int pipeline);   // the pipelines of a config that take this route
+bool conv_as_subsampled_gemm(const amos_conv_desc_t& c, int op, amos_bgemm_desc_t* out, ConvSubsample* sub);
 // groups == input channels (NCDHW): runs on the vector ALUs unless a matrix-core pipeline is named
 bool conv_is_depthwise(const amos_conv_desc_t& c);
 

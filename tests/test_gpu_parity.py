@@ -649,6 +649,41 @@ def test_conv3d_config5b(gpu):
     check_float(full[5:6].cpu().numpy(), ref0, "C5b image 5 vs fp32 (64x128)")
 
 
+@pytest.mark.parametrize("dtype", ["float16", "int8"])
+@pytest.mark.parametrize("case", [(20, 256, 30, 30, 512, (2, 2)), (24, 200, 41, 37, 520, (2, 3)), (24, 512, 14, 27, 256, (1, 2))])
+def test_strided_pointwise_conv_runs_as_gemm(gpu, dtype, case):
+    """a 1x1 window with a stride (ResNet's down-sampling shortcuts): the copy that makes the
+    activations K-contiguous picks every stride-th pixel, the direct-to-LDS GEMM does the rest;
+    against the oracle, against the implicit GEMM of the same op (bit for bit for int8), and
+    without a workspace (the implicit GEMM again)"""
+    import torch
+    from amos_amd import _lib, ops
+    N, C, H, W, K, st = case
+    rng = np.random.default_rng(hash(case) % 2**32)
+    x = make_operand(rng, (N, C, H, W), dtype)
+    w = make_operand(rng, (K, C, 1, 1), dtype)
+    dx, dw = to_device(x, dtype), to_device(w, dtype)
+    desc = ops.conv_desc((N, C, 1, H, W), (K, C, 1, 1, 1), dx.dtype, (1,) + st, (0, 0, 0), (1, 1, 1))
+    assert ops.kernel_name(_lib.AMOS_OP_CONV2D, desc, None).startswith("amos_gemm_tn<")
+    assert ops.workspace_bytes(_lib.AMOS_OP_CONV2D, desc) > 0
+    cfg = ops.default_config(_lib.AMOS_OP_CONV2D, desc)
+    assert ops.kernel_name(_lib.AMOS_OP_CONV2D, desc, cfg) == ops.kernel_name(_lib.AMOS_OP_CONV2D, desc, None)
+    got = ops.conv2d(dx, dw, st, 0, 1).cpu().numpy()
+    ref = co.lib_conv2d(x, w, dtype, st, 0, 1, acc="float64")
+    check(got, ref, dtype, "strided pointwise %s %s" % (dtype, case))
+    staged = dict(tile_i=64, tile_j=64, split_k=1, pipeline=1)
+    assert ops.kernel_name(_lib.AMOS_OP_CONV2D, desc, staged).startswith("amos_igemm<")
+    other = ops.conv2d(dx, dw, st, 0, 1, config=staged).cpu().numpy()
+    check(other, ref, dtype, "strided pointwise, implicit GEMM %s %s" % (dtype, case))
+    if dtype == "int8":
+        assert np.array_equal(got, other)
+    # no workspace: the same call through the C ABI falls back to the implicit GEMM
+    out = torch.empty(got.shape, dtype=torch.from_numpy(got).dtype, device="cuda")
+    rc = _lib.load().amos_conv2d(ctypes.byref(desc), None, dx.data_ptr(), dw.data_ptr(), out.data_ptr(), None, 0, None)
+    assert rc == 0
+    check(out.cpu().numpy(), ref, dtype, "strided pointwise, no workspace %s %s" % (dtype, case))
+
+
 DEPTHWISE_CASES = [
     # N, C, D, H, W, mult, T, R, S, stride, pad, dil, kernel-name suffix
     (2, 32, 1, 28, 28, 1, 1, 3, 3, (1, 1, 1), (0, 1, 1), (1, 1, 1), ",3x3>"),       # MobileNet's 3x3
