@@ -34,7 +34,8 @@ GemmRepack gemm_repack(const amos_gemm_desc_t& g, int64_t batch, bool a_unaligne
   // kernel would have to load an operand element by element
   const bool vectors = es == 2 && !a_bad && !b_bad && !b_gathered && g.K % 8 == 0 &&
                        (!g.trans_a || g.M % 8 == 0) && (g.trans_b || g.N % 8 == 0);
-  if (2.0 * (double)g.M * (double)g.N * (double)g.K * (double)batch < (vectors ? 8e9 : 1e9)) return r;
+  // (0.2 GFLOP where the copy also spares an im2col gather)
+  if (2.0 * (double)g.M * (double)g.N * (double)g.K * (double)batch < (vectors ? 8e9 : b_gathered ? 2e8 : 1e9)) return r;
   r.Kp = (g.K + bke - 1) / bke * bke;
   r.copy_a = copy_a;
   r.copy_b = copy_b;

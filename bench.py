@@ -60,7 +60,7 @@ def _timed(fn):
     return time.perf_counter() - t0
 
 
-def run_all_configs(cpu=True):
+def run_all_configs(cpu=True, only=None):
     """Every configuration of the path: GPU ms, TFLOP/s (TOP/s), % of the MFMA peak, % of the
     HBM roof for the algorithmic bytes, which roof binds, and the te_literal CPU loop nest
     (1 thread and all cores) on a slab of the same workload, linearly scaled."""
@@ -79,6 +79,8 @@ def run_all_configs(cpu=True):
         return min(t), cfg
 
     def add(name, op, desc, hin, dtype, flop, nbytes, out_shape, cpu_fn, frac, fused_tail=False):
+        if only and only not in name:
+            return
         tin = [torch.from_numpy(h).cuda() for h in hin]
         out = torch.empty(out_shape, dtype=torch.int32 if dtype == "int8" else torch.float32,
                           device="cuda")
@@ -148,6 +150,13 @@ def run_all_configs(cpu=True):
         [x3, w3], "float16", 2.0 * 401408 * 64 * 1728, 154361856, (8, 64, 16, 56, 56),
         lambda th, big: co.te_literal_conv3d(x3s, w3, "float16", 1, 1, 1, threads=th),
         (1 / 32, 1 / 32))
+    # beyond the headline configurations: MobileNet-V1's first depthwise layer at batch 16 (the
+    # reference's benchmark/amos/mapping_depthwiseconv2d_tensorcore.py op), a byte mover
+    xd, wd = f16(rng.standard_normal((16, 32, 112, 112))), f16(rng.standard_normal((32, 1, 3, 3)))
+    add("depthwise fp16 conv2d N16 C32 112x112 3x3 (groups 32)", _lib.AMOS_OP_CONV2D,
+        ops.conv_desc((16, 32, 1, 112, 112), (32, 1, 1, 3, 3), torch.float16, (1, 1, 1), (0, 1, 1), (1, 1, 1), 32),
+        [xd, wd], "float16", 2.0 * 16 * 32 * 112 * 112 * 9, 16 * 32 * 112 * 112 * 6 + 32 * 9 * 2,
+        (16, 32, 112, 112), None, None)
     return rows
 
 
@@ -281,6 +290,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU-baseline leg")
     ap.add_argument("--report", default=None, help="also time every config, write JSON here")
+    ap.add_argument("--report-only", default=None,
+                    help="restrict --report to the configurations whose name contains this text")
     ap.add_argument("--model-check", default=None,
                     help="also rank every kernel configuration of a set of shapes by the mapper's model "
                          "and by measurement, write JSON here")
@@ -353,7 +364,7 @@ def main():
         line["cpu_baseline"] = cpu_baseline_gemm(a, b)
     if args.report:
         with open(args.report, "w") as f:
-            json.dump(run_all_configs(cpu=not args.no_cpu), f, indent=1)
+            json.dump(run_all_configs(cpu=not args.no_cpu, only=args.report_only), f, indent=1)
     if args.model_check:
         with open(args.model_check, "w") as f:
             json.dump(model_check(), f, indent=1)
