@@ -150,7 +150,8 @@ typedef struct {
 #define AMOS_FLAG_NO_TILE_WALK 2
 
 /* how tiles travel from HBM to the MFMA operands */
-#define AMOS_PIPE_AUTO 0
+#define AMOS_PIPE_AUTO 0      /* the mapper's choice; a depthwise convolution (groups == C,  */
+                              /* NCDHW) runs on the vector-ALU kernel under this value only   */
 #define AMOS_PIPE_STAGED 1    /* global -> registers -> LDS, any layout, ragged K             */
 #define AMOS_PIPE_DIRECT4 2   /* global -> LDS direct copies, 256x256 tile, 4 waves           */
 #define AMOS_PIPE_DIRECT8 3   /* same with 8 waves (two per SIMD)                             */
@@ -172,8 +173,9 @@ int amos_default_config(int op, const void* desc, amos_kernel_config_t* out);
  * returns AMOS_ERR_INFEASIBLE when over budget */
 int amos_check_config(int op, const void* desc, const amos_kernel_config_t* cfg,
                       int64_t* lds_bytes, int64_t* acc_regs);
-/* bytes of device scratch the op's fastest pipeline wants (conv: repacked weights); calls
- * that get less fall back to the register-staged pipeline, which needs none */
+/* bytes of device scratch the op's fastest pipeline wants (conv: repacked weights and
+ * activations; GEMM and 1x1 convolutions: K-contiguous copies of operands); calls that get less
+ * fall back to the register-staged pipeline, which needs none */
 size_t amos_workspace_bytes(int op, const void* desc, const amos_kernel_config_t* cfg);
 /* the mapper's analytical estimate (seconds per launch) for a config: wave quantisation of the
  * grid over the CUs against MFMA issue time, HBM time for the algorithmic bytes, a launch floor
