@@ -180,6 +180,61 @@ static Instance* pick(int dt, int rl, int cl, int ti, int tj) {
 }
 
 // ---- descriptor -> launch plan --------------------------------------------------------
+// Col[n][od,op,oq][k] = X[n][c][od*sd - pd + t*dd][op*sh - ph + r*dh][oq*sw - pw + s*dw] for
+// k = ((c*T + t)*R + r)*S + s < Kred, zero where the window hangs over the edge and for
+// Kred <= k < Kp.  One thread per 16 bytes of the result; loads at clamped addresses, masked.
+struct Im2colParams {
+  const char* x;
+  char* dst;
+  int C, D, H, W, T, R, S, OD, OP, OQ;
+  int sd, sh, sw, pd, ph, pw, dd, dh, dw;
+  int Kred, chunks;        // chunks = Kp / elements per 16 bytes
+  unsigned total;          // N * OD * OP * OQ * chunks, below 2^31
+  int64_t x_image;         // elements per image
+  FastDiv fd_chunks, fd_oq, fd_op, fd_od, fd_trs, fd_rs, fd_s;
+};
+template <typename T>
+__global__ __launch_bounds__(256) void amos_im2col_kernel(const Im2colParams p) {
+  constexpr int VE = 16 / (int)sizeof(T);
+  const T* __restrict__ x = (const T*)p.x;
+  const unsigned step = gridDim.x * 256u;
+  for (unsigned idx = blockIdx.x * 256u + threadIdx.x; idx < p.total; idx += step) {
+    const int row = fast_div((int)idx, p.fd_chunks);
+    const int k0 = ((int)idx - row * p.chunks) * VE;
+    int rest = fast_div(row, p.fd_oq);
+    const int oq = row - rest * p.OQ;
+    int nx = fast_div(rest, p.fd_op);
+    const int op = rest - nx * p.OP;
+    const int n = fast_div(nx, p.fd_od);
+    const int od = nx - n * p.OD;
+    int c = fast_div(k0, p.fd_trs);
+    rest = k0 - c * (p.T * p.R * p.S);
+    int t = fast_div(rest, p.fd_rs);
+    rest -= t * (p.R * p.S);
+    int r = fast_div(rest, p.fd_s);
+    int s = rest - r * p.S;
+    const T* img = x + (int64_t)n * p.x_image;
+    const int d0 = od * p.sd - p.pd, h0 = op * p.sh - p.ph, w0 = oq * p.sw - p.pw;
+    T v[VE];
+#pragma unroll
+    for (int e = 0; e < VE; ++e) {
+      const int id = d0 + t * p.dd, ih = h0 + r * p.dh, iw = w0 + s * p.dw;
+      const bool ok = k0 + e < p.Kred && (unsigned)id < (unsigned)p.D && (unsigned)ih < (unsigned)p.H &&
+                      (unsigned)iw < (unsigned)p.W;
+      unsigned m = ok ? 0xffffffffu : 0u;
+      asm("" : "+v"(m));       // (a select of "loaded or zero" would become a branch around the load)
+      const int cc = c < p.C ? c : p.C - 1;
+      const int dc = id < 0 ? 0 : id >= p.D ? p.D - 1 : id;
+      const int hc = ih < 0 ? 0 : ih >= p.H ? p.H - 1 : ih;
+      const int wc = iw < 0 ? 0 : iw >= p.W ? p.W - 1 : iw;
+      const unsigned raw = (unsigned)img[((cc * p.D + dc) * p.H + hc) * p.W + wc];
+      v[e] = (T)(raw & m);
+      if (++s == p.S) { s = 0; if (++r == p.R) { r = 0; if (++t == p.T) { t = 0; ++c; } } }
+    }
+    *(uint4*)(p.dst + (int64_t)idx * 16) = *(const uint4*)v;
+  }
+}
+
 struct Plan {
   IgemmParams p;
   int dt, rl, cl;
@@ -205,6 +260,9 @@ struct Plan {
   // depthwise convolution on the vector ALUs (0 = not used, else 1 + DW_* kind)
   int dw;
   DepthwiseParams dwp;
+  // im2col copy of a convolution's activations in front of the GEMM (0 = not used)
+  int im2col;
+  Im2colParams icp;
 };
 
 static int dtype_pair(int in_dtype, int out_dtype, int* dt) {
@@ -483,6 +541,51 @@ static int plan_conv(Plan& pl, int op, const amos_conv_desc_t* d, const amos_ker
                                 Wt, X, Y, workspace, &sub);
     }
   }
+  // Few channels (no whole 128-byte chunk of them for the patch-staged pipeline): an im2col copy
+  // of the activations and zero-padded weights in the workspace, then the direct-to-LDS GEMM
+  ConvIm2col ic;
+  if ((!cfg || conv_subsample_pipeline(cfg->pipeline)) && workspace && ((uintptr_t)workspace & 255) == 0 &&
+      conv_as_im2col_gemm(c, op, &b, &ic) && ws_bytes >= (size_t)(ic.bytes_w + ic.bytes_x)) {
+    char* wpad = (char*)workspace;
+    char* col = wpad + ic.bytes_w;
+    b.g.out_dtype = c.out_dtype;
+    // without a tile from the caller: the convolution's own default (the best direct tile)
+    amos_kernel_config_t own;
+    if (!cfg || cfg->tile_i <= 0 || cfg->tile_j <= 0) {
+      rc = amos_default_config(op, &c, &own);
+      if (rc) return rc;
+      if (cfg && cfg->split_k > 0) own.split_k = cfg->split_k;
+      cfg = &own;
+    }
+    rc = plan_gemm(pl, AMOS_OP_BGEMM, &b, &b.g, b.batch, b.stride_a, b.stride_b, b.stride_c, cfg, wpad, col, Y);
+    if (rc) return rc;
+    // weights [K][Kred] -> [K][Kp], zero-filled
+    pl.n_transposes = 1;
+    pl.tr[0] = TransposeJob{(const char*)Wt, wpad, (int)c.K, (int)ic.Kred, ic.Kred, 0, 0, 1, (int)ic.Kp, 1};
+    const int es2 = pl.dt == DT_I8 ? 1 : 2;
+    Im2colParams& q = pl.icp;
+    memset(&q, 0, sizeof(q));
+    q.x = (const char*)X; q.dst = col;
+    q.C = (int)c.C; q.D = (int)c.D; q.H = (int)c.H; q.W = (int)c.W;
+    q.T = (int)c.T; q.R = (int)c.R; q.S = (int)c.S;
+    q.OD = ic.OD; q.OP = ic.OP; q.OQ = ic.OQ;
+    q.sd = c.stride_d; q.sh = c.stride_h; q.sw = c.stride_w;
+    q.pd = c.pad_d; q.ph = c.pad_h; q.pw = c.pad_w;
+    q.dd = c.dil_d; q.dh = c.dil_h; q.dw = c.dil_w;
+    q.Kred = (int)ic.Kred;
+    q.chunks = (int)(ic.Kp / (16 / es2));
+    q.total = (unsigned)(c.N * ic.OD * (int64_t)ic.OP * ic.OQ * q.chunks);
+    q.x_image = c.C * c.D * c.H * c.W;
+    q.fd_chunks = make_fast_div((uint32_t)q.chunks);
+    q.fd_oq = make_fast_div((uint32_t)ic.OQ);
+    q.fd_op = make_fast_div((uint32_t)ic.OP);
+    q.fd_od = make_fast_div((uint32_t)ic.OD);
+    q.fd_trs = make_fast_div((uint32_t)(c.T * c.R * c.S));
+    q.fd_rs = make_fast_div((uint32_t)(c.R * c.S));
+    q.fd_s = make_fast_div((uint32_t)c.S);
+    pl.im2col = 1;
+    return 0;
+  }
   // Depthwise (one input channel per group): no reduction but over the window, so it runs on the
   // vector ALUs as the byte mover it is, unless a matrix-core pipeline is asked for by name.
   if (conv_is_depthwise(c) && (!cfg || cfg->pipeline == AMOS_PIPE_AUTO)) {
@@ -676,6 +779,7 @@ static int make_plan(Plan& pl, int op, const void* desc, const amos_kernel_confi
   pl.fill_once = 0;
   pl.n_transposes = 0;
   pl.dw = 0;
+  pl.im2col = 0;
   switch (op) {
     case AMOS_OP_GEMM:
       return plan_gemm(pl, op, desc, (const amos_gemm_desc_t*)desc, 1, 0, 0, 0, cfg, in0, in1, out, workspace,
@@ -753,6 +857,14 @@ static int launch_conv(const Plan& pl, hipStream_t stream) {
 }
 
 static int launch(const Plan& pl, hipStream_t stream) {
+  if (pl.im2col) {
+    const unsigned want = (pl.icp.total + 255u) / 256u;
+    dim3 grid(want < (1u << 20) ? want : (1u << 20));
+    if (pl.dt == DT_I8)
+      hipLaunchKernelGGL(amos_im2col_kernel<unsigned char>, grid, dim3(256), 0, stream, pl.icp);
+    else
+      hipLaunchKernelGGL(amos_im2col_kernel<unsigned short>, grid, dim3(256), 0, stream, pl.icp);
+  }
   for (int k = 0; k < pl.n_transposes; ++k) {
     const TransposeJob& j = pl.tr[k];
     if (j.copy) {
@@ -1012,6 +1124,11 @@ size_t amos_workspace_bytes(int op, const void* desc, const amos_kernel_config_t
   } else if ((!cfg || conv_subsample_pipeline(cfg->pipeline)) && conv_as_subsampled_gemm(c, op, &b, nullptr)) {
     const int64_t t = gemm_repack(b.g, b.batch, false, false, true).total();
     if (t > need) need = t;
+  } else {
+    ConvIm2col ic;
+    if ((!cfg || conv_subsample_pipeline(cfg->pipeline)) && conv_as_im2col_gemm(c, op, &b, &ic) &&
+        ic.bytes_w + ic.bytes_x > need)
+      need = ic.bytes_w + ic.bytes_x;
   }
   return (size_t)need;
 }

@@ -106,6 +106,47 @@ bool conv_as_subsampled_gemm(const amos_conv_desc_t& c, int op, amos_bgemm_desc_
   return true;
 }
 
+bool conv_as_im2col_gemm(const amos_conv_desc_t& cin, int op, amos_bgemm_desc_t* out, ConvIm2col* info) {
+  amos_conv_desc_t c = cin;
+  if (op == AMOS_OP_CONV2D) { c.D = 1; c.T = 1; c.stride_d = 1; c.pad_d = 0; c.dil_d = 1; }
+  const int64_t G = c.groups > 1 ? c.groups : 1;
+  if (G != 1 || c.layout != AMOS_LAYOUT_NCHW || c.N <= 0 || c.N >= 65536 || c.C <= 0 || c.K <= 0) return false;
+  if (conv_padded_channels(c) != 0) return false;            // the patch-staged pipeline applies
+  // the copy is made once, the on-the-fly gather once per 64 output channels: measured ahead from
+  // 256 output channels on (N16 3->256 7x7/2 @224: 111 us against 231 us), behind at 64-128
+  if (c.K < 256) return false;
+  if (c.T * c.R * c.S == 1) return false;                    // pointwise: a product as it stands
+  const int es = c.in_dtype == AMOS_I8 ? 1 : 2;
+  const int64_t bke = 128 / es;
+  const int64_t Kred = c.C * c.T * c.R * c.S;
+  if (Kred > 4096) return false;
+  const int64_t OD = conv_out(c.D, c.pad_d, c.dil_d, c.T, c.stride_d);
+  const int64_t OP = conv_out(c.H, c.pad_h, c.dil_h, c.R, c.stride_h);
+  const int64_t OQ = conv_out(c.W, c.pad_w, c.dil_w, c.S, c.stride_w);
+  if (OD <= 0 || OP <= 0 || OQ <= 0) return false;
+  const int64_t J = OD * OP * OQ, Kp = (Kred + bke - 1) / bke * bke;
+  if (2.0 * (double)c.N * (double)J * (double)c.K * (double)Kred < 2e8) return false;
+  const int64_t bytes_x = (c.N * J * Kp * es + 255) / 256 * 256;
+  if (bytes_x > (1ll << 30) || c.N * J * (Kp / (16 / es)) >= (1ll << 31) || c.C * c.D * c.H * c.W >= (1ll << 31))
+    return false;
+  amos_bgemm_desc_t& b = *out;
+  memset(&b, 0, sizeof(b));
+  b.g.in_dtype = c.in_dtype;
+  b.g.out_dtype = c.out_dtype;
+  b.batch = c.N;
+  b.g.M = c.K; b.g.N = J; b.g.K = Kp;
+  b.g.trans_a = 0; b.g.trans_b = 1;
+  b.g.lda = Kp; b.g.ldb = Kp; b.g.ldc = J;
+  b.stride_a = 0; b.stride_b = J * Kp; b.stride_c = c.K * J;
+  if (info) {
+    info->Kred = Kred; info->Kp = Kp;
+    info->bytes_w = (c.K * Kp * es + 255) / 256 * 256;
+    info->bytes_x = bytes_x;
+    info->OD = (int)OD; info->OP = (int)OP; info->OQ = (int)OQ;
+  }
+  return true;
+}
+
 // what the copies of gemm_repack cost: each reads and writes its operand once at about a third of
 // the HBM rate (64x64 blocks through LDS), plus a launch
 static void note_repack(Problem* pb, const amos_gemm_desc_t& g, int64_t batch, bool b_gathered = false) {
@@ -448,6 +489,30 @@ static const TileCost kDirectCost[] = {
 // the direct kernel's tiles in the order plan_gemm_repacked() tries them
 static const int kRepackTiles[4][2] = {{256, 256}, {128, 128}, {128, 256}, {256, 128}};
 
+// A convolution that runs as a batched matrix product on a copy of its activations (every
+// stride-th pixel of a 1x1 window, or an im2col matrix for few channels): that product, with
+// the copy's time, as the mapper's problem.
+static bool conv_copied_gemm_problem(const amos_conv_desc_t& c, int op, Problem* pg) {
+  amos_bgemm_desc_t g;
+  if (conv_as_subsampled_gemm(c, op, &g, nullptr)) {
+    if (problem_of(AMOS_OP_BGEMM, &g, pg)) return false;
+    note_repack(pg, g.g, g.batch, true);
+    return true;
+  }
+  ConvIm2col ic;
+  if (conv_as_im2col_gemm(c, op, &g, &ic)) {
+    if (problem_of(AMOS_OP_BGEMM, &g, pg)) return false;
+    pg->repack = 1;
+    pg->Kp = ic.Kp;
+    // the copy writes the im2col matrix at about a quarter of the HBM rate (8 element loads and
+    // their index arithmetic per 16 bytes) and pads the weights in a second launch
+    pg->repack_seconds = (double)ic.bytes_x / 2.0e12 + 6e-6;
+    pg->direct_ok = 1;
+    return true;
+  }
+  return false;
+}
+
 static double loader_factor(int loader) {
   switch (loader) {
     case 1: return 3.0;    // element loads: 8 (fp16) or 16 (int8) per 16-byte chunk
@@ -573,14 +638,12 @@ int amos_estimate_seconds(int op, const void* desc, const amos_kernel_config_t* 
   if ((op == AMOS_OP_CONV2D || op == AMOS_OP_CONV3D) && cfg->pipeline != AMOS_PIPE_PATCH &&
       cfg->pipeline != AMOS_PIPE_PATCH8 && conv_as_gemm(*(const amos_conv_desc_t*)desc, op, &as_gemm))
     return amos_estimate_seconds(AMOS_OP_BGEMM, &as_gemm, cfg, seconds);   // what the launch runs
-  if ((op == AMOS_OP_CONV2D || op == AMOS_OP_CONV3D) && conv_subsample_pipeline(cfg->pipeline) &&
-      conv_as_subsampled_gemm(*(const amos_conv_desc_t*)desc, op, &as_gemm, nullptr)) {
+  if ((op == AMOS_OP_CONV2D || op == AMOS_OP_CONV3D) && conv_subsample_pipeline(cfg->pipeline)) {
     Problem pg;
-    rc = problem_of(AMOS_OP_BGEMM, &as_gemm, &pg);
-    if (rc) return rc;
-    note_repack(&pg, as_gemm.g, as_gemm.batch, true);
-    *seconds = estimate_seconds(pg, cfg->tile_i, cfg->tile_j, cfg->split_k < 1 ? 1 : cfg->split_k);
-    return 0;
+    if (conv_copied_gemm_problem(*(const amos_conv_desc_t*)desc, op, &pg)) {
+      *seconds = estimate_seconds(pg, cfg->tile_i, cfg->tile_j, cfg->split_k < 1 ? 1 : cfg->split_k);
+      return 0;
+    }
   }
   if ((op == AMOS_OP_CONV2D || op == AMOS_OP_CONV3D) && cfg->pipeline != AMOS_PIPE_STAGED) {
     const int waves = cfg->pipeline == AMOS_PIPE_PATCH ? 4 : cfg->pipeline == AMOS_PIPE_PATCH8 ? 8 : 0;
@@ -609,12 +672,9 @@ int amos_default_config(int op, const void* desc, amos_kernel_config_t* result) 
   if ((op == AMOS_OP_CONV2D || op == AMOS_OP_CONV3D) && conv_as_gemm(*(const amos_conv_desc_t*)desc, op, &as_gemm))
     return amos_default_config(AMOS_OP_BGEMM, &as_gemm, result);
   // ... a strided one after its pixels are picked by the operand copy: the best direct tile
+  Problem pg;
   if ((op == AMOS_OP_CONV2D || op == AMOS_OP_CONV3D) &&
-      conv_as_subsampled_gemm(*(const amos_conv_desc_t*)desc, op, &as_gemm, nullptr)) {
-    Problem pg;
-    rc = problem_of(AMOS_OP_BGEMM, &as_gemm, &pg);
-    if (rc) return rc;
-    note_repack(&pg, as_gemm.g, as_gemm.batch, true);
+      conv_copied_gemm_problem(*(const amos_conv_desc_t*)desc, op, &pg)) {
     memset(result, 0, sizeof(*result));
     result->pipeline = AMOS_PIPE_AUTO;
     double best_direct = 1e30;

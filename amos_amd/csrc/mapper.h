@@ -71,6 +71,18 @@ struct ConvSubsample {
 };
 bool conv_subsample_pipeline(int pipeline);   // the pipelines of a config that take this route
 bool conv_as_subsampled_gemm(const amos_conv_desc_t& c, int op, amos_bgemm_desc_t* out, ConvSubsample* sub);
+// A convolution on few channels (the patch-staged pipeline wants whole 128-byte chunks of
+// channels; a 7x7 stem on RGB has 6 bytes) as a batched matrix product over an im2col copy of
+// the activations: per image Y[K][ODPQ] = Wt'[K][Kp] Col[ODPQ][Kp]^T with Kp = C*T*R*S rounded up
+// to whole K steps, both operands K-contiguous and zero-filled, so the direct-to-LDS kernel runs.
+// NCDHW, one group, where the copy pays (0.2 GFLOP, 256 output channels or more) and stays under
+// 1 GiB; needs the workspace.
+struct ConvIm2col {
+  int64_t Kred, Kp;
+  int64_t bytes_w, bytes_x;     // workspace: padded weights, then the im2col matrix
+  int OD, OP, OQ;
+};
+bool conv_as_im2col_gemm(const amos_conv_desc_t& c, int op, amos_bgemm_desc_t* out, ConvIm2col* info);
 // groups == input channels (NCDHW): runs on the vector ALUs unless a matrix-core pipeline is named
 bool conv_is_depthwise(const amos_conv_desc_t& c);
 

@@ -684,6 +684,52 @@ def test_strided_pointwise_conv_runs_as_gemm(gpu, dtype, case):
     check(out.cpu().numpy(), ref, dtype, "strided pointwise, no workspace %s %s" % (dtype, case))
 
 
+IM2COL_CASES = [
+    # N, C, D, H, W, K, T, R, S, stride, pad, dil
+    (3, 3, 1, 64, 60, 256, 1, 7, 7, (1, 2, 2), (0, 3, 3), (1, 1, 1)),     # a wide 7x7 stem on RGB
+    (7, 3, 1, 113, 97, 264, 1, 3, 3, (1, 2, 2), (0, 1, 1), (1, 1, 1)),    # 3x3 on RGB, ragged everything
+    (4, 20, 1, 30, 31, 300, 1, 5, 3, (1, 1, 2), (0, 2, 0), (1, 2, 1)),    # 20 channels, dilated, uneven
+    (4, 5, 6, 20, 18, 256, 3, 3, 3, (1, 2, 1), (1, 0, 1), (1, 1, 1)),     # 3-D
+]
+
+
+@pytest.mark.parametrize("dtype", ["float16", "bfloat16", "int8"])
+@pytest.mark.parametrize("case", IM2COL_CASES)
+def test_conv_few_channels_through_im2col_copy(gpu, dtype, case):
+    """a convolution on few channels: im2col copy + zero-padded weights in the workspace, then the
+    GEMM kernels; against the oracle, against the on-the-fly im2col of the same op (bit for bit
+    for int8), and without a workspace"""
+    import torch
+    from amos_amd import _lib, ops
+    N, C, D, H, W, K, T, R, S, st, pd, dl = case
+    rng = np.random.default_rng(hash(case) % 2**32)
+    x = make_operand(rng, (N, C, D, H, W), dtype)
+    w = make_operand(rng, (K, C, T, R, S), dtype)
+    dx, dw = to_device(x, dtype), to_device(w, dtype)
+    desc = ops.conv_desc((N, C, D, H, W), (K, C, T, R, S), dx.dtype, st, pd, dl)
+    assert ops.workspace_bytes(_lib.AMOS_OP_CONV3D, desc) > 0
+    name = ops.kernel_name(_lib.AMOS_OP_CONV3D, desc, None)
+    assert name.startswith("amos_gemm_tn<") or ",vec,vec," in name, name
+    cfg = ops.default_config(_lib.AMOS_OP_CONV3D, desc)
+    assert ops.kernel_name(_lib.AMOS_OP_CONV3D, desc, cfg) == name
+    ref = co.lib_conv3d(x, w, dtype, st, pd, dl, acc="float64")
+    got = ops.conv3d(dx, dw, st, pd, dl).cpu().numpy()
+    check(got, ref, dtype, "im2col copy %s %s" % (dtype, case))
+    # a staged tile on the copies, split-K
+    got2 = ops.conv3d(dx, dw, st, pd, dl, config=dict(tile_i=64, tile_j=64, split_k=2, pipeline=0)).cpu().numpy()
+    check(got2, ref, dtype, "im2col copy, 64x64 split 2 %s %s" % (dtype, case))
+    staged = dict(tile_i=64, tile_j=64, split_k=1, pipeline=1)
+    assert ",im2col," in ops.kernel_name(_lib.AMOS_OP_CONV3D, desc, staged)
+    other = ops.conv3d(dx, dw, st, pd, dl, config=staged).cpu().numpy()
+    check(other, ref, dtype, "on-the-fly im2col %s %s" % (dtype, case))
+    if dtype == "int8":
+        assert np.array_equal(got, other) and np.array_equal(got2, other)
+    out = torch.empty(got.shape, dtype=torch.from_numpy(got).dtype, device="cuda")
+    rc = _lib.load().amos_conv3d(ctypes.byref(desc), None, dx.data_ptr(), dw.data_ptr(), out.data_ptr(), None, 0, None)
+    assert rc == 0
+    check(out.cpu().numpy(), ref, dtype, "few channels, no workspace %s %s" % (dtype, case))
+
+
 DEPTHWISE_CASES = [
     # N, C, D, H, W, mult, T, R, S, stride, pad, dil, kernel-name suffix
     (2, 32, 1, 28, 28, 1, 1, 3, 3, (1, 1, 1), (0, 1, 1), (1, 1, 1), ",3x3>"),       # MobileNet's 3x3
