@@ -591,8 +591,12 @@ static int plan_conv(Plan& pl, int op, const amos_conv_desc_t* d, const amos_ker
   if (conv_is_depthwise(c) && (!cfg || cfg->pipeline == AMOS_PIPE_AUTO)) {
     // (the 3x3 kinds assume one stride for rows and columns)
     const bool win3 = c.R == 3 && c.S == 3 && c.dil_h == 1 && c.dil_w == 1 && c.stride_h == c.stride_w;
-    const int kind = win3 && c.stride_w == 1 ? DW_3x3_S1 : win3 && c.stride_w == 2 ? DW_3x3_S2 : DW_GENERIC;
+    int kind = win3 && c.stride_w == 1 ? DW_3x3_S1 : win3 && c.stride_w == 2 ? DW_3x3_S2 : DW_GENERIC;
     const int64_t qgroups = (OQ + 3) / 4;
+    // four output rows per lane only where that leaves 4096 waves or more (four per SIMD): below,
+    // one generation of waves is all there is and its latency the whole kernel (measured: N16
+    // C512 14x14 9.2 -> 8.6 us, C1024 7x7 6.7 -> 5.8 us with two rows)
+    if (kind == DW_3x3_S1 && c.N * c.K * OD * ((OP + 3) / 4) * qgroups < 4096 * 64) kind = DW_3x3_S1_SMALL;
     const int64_t pgroups = (OP + dw_rows_per_lane(kind) - 1) / dw_rows_per_lane(kind);
     const int64_t items = c.N * c.K * OD * pgroups * qgroups;
     if (fits_int(items) && fits_int(c.D * c.H * c.W) && fits_int(c.T * c.R * c.S) && fits_int(c.N) && fits_int(c.K)) {

@@ -32,9 +32,12 @@ struct DepthwiseParams {
   EpiParams epi;
 };
 
-enum { DW_GENERIC = 0, DW_3x3_S1 = 1, DW_3x3_S2 = 2 };
-// output rows per lane: the 3x3 kinds keep the input rows two output rows share in registers
-constexpr int dw_rows_per_lane(int kind) { return kind == DW_3x3_S1 ? 4 : kind == DW_3x3_S2 ? 2 : 1; }
+enum { DW_GENERIC = 0, DW_3x3_S1 = 1, DW_3x3_S2 = 2, DW_3x3_S1_SMALL = 3 };
+// output rows per lane: the 3x3 kinds keep the input rows that output rows share in registers;
+// four rows where that still leaves every SIMD several waves, two for smaller problems
+constexpr int dw_rows_per_lane(int kind) {
+  return kind == DW_3x3_S1 ? 4 : (kind == DW_3x3_S2 || kind == DW_3x3_S1_SMALL) ? 2 : 1;
+}
 
 template <int DT> struct DwTypes { typedef unsigned short in_t; typedef float acc_t; };
 template <> struct DwTypes<DT_I8> { typedef signed char in_t; typedef int acc_t; };
@@ -96,7 +99,7 @@ __global__ __launch_bounds__(256) void amos_depthwise_conv(const DepthwiseParams
       const int d = d0 + t * p.dd;
       if ((unsigned)d >= (unsigned)p.D) continue;
       if constexpr (KIND != DW_GENERIC) {
-        constexpr int ST = KIND == DW_3x3_S1 ? 1 : 2;
+        constexpr int ST = KIND == DW_3x3_S2 ? 2 : 1;
         constexpr int NV = 3 * ST + 3;            // input columns under four outputs
         constexpr int NH = (PR - 1) * ST + 3;     // input rows under PR output rows
         acc_t wv[9];
