@@ -10,6 +10,7 @@
 
 #include "amos_mi355x.h"
 #include "conv_fprop_kernel.h"
+#include "conv_fewc_kernel.h"
 #include "depthwise_kernel.h"
 #include "gemm_tn_kernel.h"
 #include "igemm_instances.h"
@@ -263,6 +264,10 @@ struct Plan {
   // im2col copy of a convolution's activations in front of the GEMM (0 = not used)
   int im2col;
   Im2colParams icp;
+  // convolution on few input channels (0 = not used)
+  int fewc;
+  ConvFewcParams fcp;
+  size_t fewc_lds;
 };
 
 static int dtype_pair(int in_dtype, int out_dtype, int* dt) {
@@ -541,6 +546,38 @@ static int plan_conv(Plan& pl, int op, const amos_conv_desc_t* d, const amos_ker
                                 Wt, X, Y, workspace, &sub);
     }
   }
+  // Input channels that fit one 16-byte pixel: the kernel whose reduction unit is the pixel
+  ConvFewcPlan fw;
+  if ((!cfg || cfg->pipeline == AMOS_PIPE_AUTO) && workspace && ((uintptr_t)workspace & 255) == 0 &&
+      conv_fewc_plan(c, op, &fw) && ws_bytes >= (size_t)(fw.bytes_x + fw.bytes_w)) {
+    ConvFewcParams& q = pl.fcp;
+    memset(&q, 0, sizeof(q));
+    q.x = (const char*)X; q.w = (const char*)Wt; q.y = (char*)Y;
+    q.xt = (char*)workspace; q.wp = (char*)workspace + fw.bytes_x;
+    q.N = (int)c.N; q.C = (int)c.C; q.H = (int)c.H; q.W = (int)c.W; q.K = (int)c.K; q.R = (int)c.R; q.S = (int)c.S;
+    q.OP = fw.OP; q.OQ = fw.OQ;
+    q.sh = c.stride_h; q.sw = c.stride_w; q.ph = c.pad_h; q.pw = c.pad_w; q.dh = c.dil_h; q.dw = c.dil_w;
+    q.taps = fw.taps; q.taps_p = fw.taps_p; q.Wp = fw.Wp; q.rows_max = fw.rows_max;
+    q.tiles_j = fw.tiles_j; q.k_tiles = fw.k_tiles;
+    q.prep_x_blocks = (int)((c.N * c.H * c.W + 255) / 256);
+    q.prep_w_blocks = (int)(((int64_t)fw.k_tiles * 64 * fw.taps_p + 255) / 256);
+    q.patch_off = fw.patch_off; q.zero_off = fw.zero_off; q.tab_off = fw.tab_off;
+    q.patch_bytes = fw.patch_bytes; q.nbuf = fw.nbuf; q.grid_x = fw.grid_x;
+    q.fd_tiles_j = make_fast_div((uint32_t)fw.tiles_j);
+    q.fd_oq = make_fast_div((uint32_t)fw.OQ);
+    q.fd_wp = make_fast_div((uint32_t)fw.Wp);
+    q.fd_hw = make_fast_div((uint32_t)(c.H * c.W));
+    q.fd_taps_p = make_fast_div((uint32_t)fw.taps_p);
+    q.fd_s = make_fast_div((uint32_t)c.S);
+    pl.fewc = 1;
+    pl.fewc_lds = fw.lds;
+    memset(&pl.cfg, 0, sizeof(pl.cfg));
+    if (cfg) pl.cfg = *cfg;
+    memset(&pl.p, 0, sizeof(pl.p));
+    pl.batch = 1;
+    pl.split = 1;
+    return 0;
+  }
   // Few channels (no whole 128-byte chunk of them for the patch-staged pipeline): an im2col copy
   // of the activations and zero-padded weights in the workspace, then the direct-to-LDS GEMM
   ConvIm2col ic;
@@ -784,6 +821,7 @@ static int make_plan(Plan& pl, int op, const void* desc, const amos_kernel_confi
   pl.n_transposes = 0;
   pl.dw = 0;
   pl.im2col = 0;
+  pl.fewc = 0;
   switch (op) {
     case AMOS_OP_GEMM:
       return plan_gemm(pl, op, desc, (const amos_gemm_desc_t*)desc, 1, 0, 0, 0, cfg, in0, in1, out, workspace,
@@ -888,6 +926,10 @@ static int launch(const Plan& pl, hipStream_t stream) {
     else
       hipLaunchKernelGGL(amos_transpose_kernel<unsigned short>, grid, dim3(256), 0, stream, j);
   }
+  if (pl.fewc) {
+    HIP_TRY(launch_conv_fewc(pl.dt, pl.fcp, pl.fewc_lds, stream));
+    return 0;
+  }
   if (pl.dw) {
     launch_depthwise(pl.dt, pl.dw - 1, pl.dwp, stream);
     HIP_TRY(hipGetLastError());
@@ -954,6 +996,7 @@ static int plan_epilogue(Plan& pl, int op, const void* desc, const amos_epilogue
   pl.tn.epi = ep;
   pl.cv.epi = ep;
   pl.dwp.epi = ep;
+  pl.fcp.epi = ep;
   return 0;
 }
 
@@ -1130,9 +1173,13 @@ size_t amos_workspace_bytes(int op, const void* desc, const amos_kernel_config_t
     if (t > need) need = t;
   } else {
     ConvIm2col ic;
-    if ((!cfg || conv_subsample_pipeline(cfg->pipeline)) && conv_as_im2col_gemm(c, op, &b, &ic) &&
-        ic.bytes_w + ic.bytes_x > need)
+    ConvFewcPlan fw;
+    if ((!cfg || cfg->pipeline == AMOS_PIPE_AUTO) && conv_fewc_plan(c, op, &fw)) {
+      if (fw.bytes_x + fw.bytes_w > need) need = fw.bytes_x + fw.bytes_w;
+    } else if ((!cfg || conv_subsample_pipeline(cfg->pipeline)) && conv_as_im2col_gemm(c, op, &b, &ic) &&
+               ic.bytes_w + ic.bytes_x > need) {
       need = ic.bytes_w + ic.bytes_x;
+    }
   }
   return (size_t)need;
 }
@@ -1146,6 +1193,7 @@ const char* amos_kernel_name(int op, const void* desc, const amos_kernel_config_
   static char dummy_ws[256] __attribute__((aligned(256)));
   if (make_plan(pl, op, desc, cfg, dummy, dummy, dummy, dummy_ws, (size_t)-1)) return nullptr;
   if (pl.dw) return depthwise_name(pl.dt, pl.dw - 1);
+  if (pl.fewc) return conv_fewc_name(pl.dt);
   if (pl.conv_ups) {
     ConvInstance* ci = pick_conv(pl.dt, pl.cfg.tile_i, pl.cfg.tile_j, pl.conv_waves, pl.cv.pls, pl.conv_occ, pl.conv_w9);
     return ci ? ci->name : nullptr;

@@ -106,6 +106,54 @@ bool conv_as_subsampled_gemm(const amos_conv_desc_t& c, int op, amos_bgemm_desc_
   return true;
 }
 
+bool conv_fewc_plan(const amos_conv_desc_t& c, int op, ConvFewcPlan* out) {
+  const bool flat = op == AMOS_OP_CONV2D || (c.D == 1 && c.T == 1 && c.pad_d == 0);
+  const int64_t G = c.groups > 1 ? c.groups : 1;
+  const int es = c.in_dtype == AMOS_I8 ? 1 : 2;
+  if (!flat || G != 1 || c.layout != AMOS_LAYOUT_NCHW || c.C <= 0 || c.C * es > 16 || c.K <= 0 || c.N <= 0 ||
+      c.N > 65535 || c.H <= 0 || c.W <= 0 || c.R <= 0 || c.S <= 0 || c.N * c.H * c.W >= (1ll << 31))
+    return false;
+  const int64_t OP = conv_out(c.H, c.pad_h, c.dil_h, c.R, c.stride_h);
+  const int64_t OQ = conv_out(c.W, c.pad_w, c.dil_w, c.S, c.stride_w);
+  if (OP <= 0 || OQ <= 0 || OP * OQ >= (1ll << 30) || c.K * OP * OQ >= (1ll << 40)) return false;
+  const int64_t taps = c.R * c.S, taps_p = (taps + 1) / 2 * 2;
+  if (taps < 2 || taps_p > 512) return false;   // (a 1x1 window is a matrix product as it stands)
+  if (2.0 * (double)c.N * (double)(OP * OQ) * (double)c.K * (double)(c.C * taps) < 1e8) return false;
+  const int64_t k_tiles = (c.K + 63) / 64, tiles_j = (OP * OQ + 255) / 256;
+  if (k_tiles > 65535 || tiles_j >= (1ll << 31)) return false;
+  const int64_t Wp = c.W + 2 * (int64_t)c.pad_w;
+  // the most patch rows a tile of 256 consecutive output pixels touches
+  int64_t rows_max = 0;
+  for (int64_t tile = 0; tile < tiles_j; ++tile) {
+    const int64_t j0 = tile * 256, j1 = std::min<int64_t>(j0 + 255, OP * OQ - 1);
+    const int64_t rows = (j1 / OQ - j0 / OQ) * c.stride_h + (c.R - 1) * c.dil_h + 1;
+    rows_max = std::max(rows_max, rows);
+    if (tile > 4096) { rows_max = std::max<int64_t>(rows_max, (255 / OQ + 1) * c.stride_h + (c.R - 1) * c.dil_h + 1); break; }
+  }
+  // (the patch is filled in 1 KB chunks)
+  const int64_t w_bytes = 64 * taps_p * 16, patch_bytes = (rows_max * Wp * 16 + 1023) / 1024 * 1024;
+  // two patch buffers where they fit: the next tile's patch travels while this one is computed
+  int64_t lds = w_bytes + 2 * patch_bytes + 16 + taps_p * 4;
+  int nbuf = 2;
+  if (lds > 160 * 1024) { lds -= patch_bytes; nbuf = 1; }
+  if (lds > 160 * 1024) return false;
+  if (tiles_j * c.N >= (1ll << 31)) return false;
+  // one workgroup per CU, shared between the tiles of output channels
+  const int64_t per_ktile = std::max<int64_t>(1, Gfx950::kComputeUnits / k_tiles);
+  const int64_t grid_x = std::min<int64_t>(tiles_j * c.N, per_ktile);
+  if (out) {
+    out->taps = (int)taps; out->taps_p = (int)taps_p; out->Wp = (int)Wp; out->rows_max = (int)rows_max;
+    out->tiles_j = (int)tiles_j; out->k_tiles = (int)k_tiles; out->OP = (int)OP; out->OQ = (int)OQ;
+    out->patch_off = (int)w_bytes; out->zero_off = (int)(w_bytes + nbuf * patch_bytes);
+    out->tab_off = (int)(w_bytes + nbuf * patch_bytes + 16);
+    out->patch_bytes = (int)patch_bytes; out->nbuf = nbuf; out->grid_x = (int)grid_x;
+    out->lds = (size_t)lds;
+    out->bytes_x = (c.N * c.H * c.W * 16 + 16 + 255) / 256 * 256;   // + the zero pixel
+    out->bytes_w = (k_tiles * 64 * taps_p * 16 + 255) / 256 * 256;
+  }
+  return true;
+}
+
 bool conv_as_im2col_gemm(const amos_conv_desc_t& cin, int op, amos_bgemm_desc_t* out, ConvIm2col* info) {
   amos_conv_desc_t c = cin;
   if (op == AMOS_OP_CONV2D) { c.D = 1; c.T = 1; c.stride_d = 1; c.pad_d = 0; c.dil_d = 1; }
@@ -116,6 +164,7 @@ bool conv_as_im2col_gemm(const amos_conv_desc_t& cin, int op, amos_bgemm_desc_t*
   // 256 output channels on (N16 3->256 7x7/2 @224: 111 us against 231 us), behind at 64-128
   if (c.K < 256) return false;
   if (c.T * c.R * c.S == 1) return false;                    // pointwise: a product as it stands
+  if (conv_fewc_plan(c, op, nullptr)) return false;          // the few-channel kernel applies
   const int es = c.in_dtype == AMOS_I8 ? 1 : 2;
   const int64_t bke = 128 / es;
   const int64_t Kred = c.C * c.T * c.R * c.S;
@@ -634,6 +683,18 @@ int amos_estimate_seconds(int op, const void* desc, const amos_kernel_config_t* 
     *seconds = ((double)pb.in_bytes + (double)pb.out_bytes) / (0.35 * Gfx950::kHbmBytesPerSec) + 3e-6;
     return 0;
   }
+  ConvFewcPlan fp;
+  if ((op == AMOS_OP_CONV2D || op == AMOS_OP_CONV3D) && cfg->pipeline == AMOS_PIPE_AUTO &&
+      conv_fewc_plan(*(const amos_conv_desc_t*)desc, op, &fp)) {
+    // the relayout launch, then rounds of workgroups that each load ~100 KB, compute for ~1 us and
+    // store 64 KB; floored by the bytes
+    const amos_conv_desc_t& c = *(const amos_conv_desc_t*)desc;
+    const double rounds = std::ceil((double)fp.tiles_j * c.N / fp.grid_x);
+    const double t_conv = 6e-6 + rounds * 4.5e-6;
+    const double t_mem = ((double)pb.in_bytes * 2 + (double)fp.bytes_x * 2 + (double)pb.out_bytes) / (0.5 * Gfx950::kHbmBytesPerSec);
+    *seconds = 4e-6 + (double)fp.bytes_x / 2.5e12 + std::max(t_conv, t_mem);
+    return 0;
+  }
   amos_bgemm_desc_t as_gemm;
   if ((op == AMOS_OP_CONV2D || op == AMOS_OP_CONV3D) && cfg->pipeline != AMOS_PIPE_PATCH &&
       cfg->pipeline != AMOS_PIPE_PATCH8 && conv_as_gemm(*(const amos_conv_desc_t*)desc, op, &as_gemm))
@@ -665,6 +726,12 @@ int amos_default_config(int op, const void* desc, amos_kernel_config_t* result) 
   if ((op == AMOS_OP_CONV2D || op == AMOS_OP_CONV3D) && conv_is_depthwise(*(const amos_conv_desc_t*)desc)) {
     memset(result, 0, sizeof(*result));
     result->tile_i = 64; result->tile_j = 64; result->split_k = 1; result->pipeline = AMOS_PIPE_AUTO;
+    return 0;
+  }
+  // few input channels: one kernel, one tile
+  if ((op == AMOS_OP_CONV2D || op == AMOS_OP_CONV3D) && conv_fewc_plan(*(const amos_conv_desc_t*)desc, op, nullptr)) {
+    memset(result, 0, sizeof(*result));
+    result->tile_i = 64; result->tile_j = 256; result->split_k = 1; result->pipeline = AMOS_PIPE_AUTO;
     return 0;
   }
   // a pointwise convolution runs as a batched matrix product: that product's configuration

@@ -83,6 +83,16 @@ struct ConvIm2col {
   int OD, OP, OQ;
 };
 bool conv_as_im2col_gemm(const amos_conv_desc_t& c, int op, amos_bgemm_desc_t* out, ConvIm2col* info);
+// A 2-D convolution whose input channels fit 16 bytes (an RGB stem) on the kernel that treats a
+// pixel as the 16-byte unit of the reduction (conv_fewc_kernel.h): NCHW, one group, from 0.1 GFLOP
+// on, where a workgroup's weights and input patch fit LDS; needs the workspace.
+struct ConvFewcPlan {
+  int taps, taps_p, Wp, rows_max, tiles_j, k_tiles, OP, OQ;
+  int patch_off, zero_off, tab_off, patch_bytes, nbuf, grid_x;
+  size_t lds;
+  int64_t bytes_x, bytes_w;    // workspace: pixel-major activations, then the packed weights
+};
+bool conv_fewc_plan(const amos_conv_desc_t& c, int op, ConvFewcPlan* out);
 // groups == input channels (NCDHW): runs on the vector ALUs unless a matrix-core pipeline is named
 bool conv_is_depthwise(const amos_conv_desc_t& c);
 

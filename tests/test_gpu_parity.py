@@ -686,8 +686,8 @@ def test_strided_pointwise_conv_runs_as_gemm(gpu, dtype, case):
 
 IM2COL_CASES = [
     # N, C, D, H, W, K, T, R, S, stride, pad, dil
-    (3, 3, 1, 64, 60, 256, 1, 7, 7, (1, 2, 2), (0, 3, 3), (1, 1, 1)),     # a wide 7x7 stem on RGB
-    (7, 3, 1, 113, 97, 264, 1, 3, 3, (1, 2, 2), (0, 1, 1), (1, 1, 1)),    # 3x3 on RGB, ragged everything
+    (2, 17, 1, 64, 60, 256, 1, 7, 7, (1, 2, 2), (0, 3, 3), (1, 1, 1)),    # a wide 7x7 on 17 channels
+    (3, 24, 1, 113, 97, 264, 1, 3, 3, (1, 2, 2), (0, 1, 1), (1, 1, 1)),   # 3x3 on 24 channels, ragged everything
     (4, 20, 1, 30, 31, 300, 1, 5, 3, (1, 1, 2), (0, 2, 0), (1, 2, 1)),    # 20 channels, dilated, uneven
     (4, 5, 6, 20, 18, 256, 3, 3, 3, (1, 2, 1), (1, 0, 1), (1, 1, 1)),     # 3-D
 ]
@@ -695,7 +695,7 @@ IM2COL_CASES = [
 
 @pytest.mark.parametrize("dtype", ["float16", "bfloat16", "int8"])
 @pytest.mark.parametrize("case", IM2COL_CASES)
-def test_conv_few_channels_through_im2col_copy(gpu, dtype, case):
+def test_conv_through_im2col_copy(gpu, dtype, case):
     """a convolution on few channels: im2col copy + zero-padded weights in the workspace, then the
     GEMM kernels; against the oracle, against the on-the-fly im2col of the same op (bit for bit
     for int8), and without a workspace"""
@@ -726,6 +726,57 @@ def test_conv_few_channels_through_im2col_copy(gpu, dtype, case):
         assert np.array_equal(got, other) and np.array_equal(got2, other)
     out = torch.empty(got.shape, dtype=torch.from_numpy(got).dtype, device="cuda")
     rc = _lib.load().amos_conv3d(ctypes.byref(desc), None, dx.data_ptr(), dw.data_ptr(), out.data_ptr(), None, 0, None)
+    assert rc == 0
+    check(out.cpu().numpy(), ref, dtype, "few channels, no workspace %s %s" % (dtype, case))
+
+
+FEW_CHANNEL_CASES = [
+    # N, C, H, W, K, R, S, stride, pad, dil
+    (6, 3, 64, 60, 64, 7, 7, (2, 2), (3, 3), (1, 1)),       # ResNet's stem, small
+    (8, 3, 113, 97, 100, 3, 3, (2, 2), (1, 1), (1, 1)),     # MobileNet's, ragged output channels
+    (16, 8, 30, 31, 72, 5, 3, (1, 2), (2, 0), (2, 1)),      # a full pixel of channels, dilated, uneven
+    (3, 1, 50, 300, 130, 3, 3, (1, 1), (1, 1), (1, 1)),     # one channel, wide rows
+    (60, 4, 40, 37, 65, 2, 4, (3, 1), (0, 2), (1, 2)),      # even taps, 65 output channels
+]
+
+
+@pytest.mark.parametrize("dtype", ["float16", "bfloat16", "int8"])
+@pytest.mark.parametrize("case", FEW_CHANNEL_CASES)
+def test_conv_few_channels(gpu, dtype, case):
+    """convolutions whose input channels fit one 16-byte pixel (the networks' stems) on
+    amos_conv_few_channels: against the oracle, against the implicit GEMM of the same op (bit for
+    bit for int8), with a fused addition, and without a workspace"""
+    import torch
+    from amos_amd import _lib, ops
+    N, C, H, W, K, R, S, st, pd, dl = case
+    if dtype == "int8":
+        C = C * 2          # sixteen int8 channels fill a pixel
+    rng = np.random.default_rng(hash(case) % 2**32)
+    x = make_operand(rng, (N, C, H, W), dtype)
+    w = make_operand(rng, (K, C, R, S), dtype)
+    dx, dw = to_device(x, dtype), to_device(w, dtype)
+    desc = ops.conv_desc((N, C, 1, H, W), (K, C, 1, R, S), dx.dtype, (1,) + st, (0,) + pd, (1,) + dl)
+    name = ops.kernel_name(_lib.AMOS_OP_CONV2D, desc, None)
+    assert name.startswith("amos_conv_few_channels<"), name
+    cfg = ops.default_config(_lib.AMOS_OP_CONV2D, desc)
+    assert ops.kernel_name(_lib.AMOS_OP_CONV2D, desc, cfg) == name and ops.workspace_bytes(_lib.AMOS_OP_CONV2D, desc) > 0
+    ref = co.lib_conv2d(x, w, dtype, st, pd, dl, acc="float64")
+    got = ops.conv2d(dx, dw, st, pd, dl).cpu().numpy()
+    check(got, ref, dtype, "few channels %s %s" % (dtype, case))
+    staged = dict(tile_i=64, tile_j=64, split_k=1, pipeline=1)
+    assert ops.kernel_name(_lib.AMOS_OP_CONV2D, desc, staged).startswith("amos_igemm<")
+    other = ops.conv2d(dx, dw, st, pd, dl, config=staged).cpu().numpy()
+    if dtype == "int8":
+        assert np.array_equal(got, other)
+    else:
+        check_float(got, other, "few channels vs implicit GEMM %s %s" % (dtype, case))
+    # fused addition of a tensor of the output's shape
+    d_host = rng.integers(-1000, 1000, got.shape).astype(got.dtype)
+    with_d = ops.conv2d(dx, dw, st, pd, dl, add=torch.from_numpy(d_host).cuda()).cpu().numpy()
+    want = (ref.astype(np.int64) + d_host).astype(np.int32) if dtype == "int8" else ref + d_host
+    check(with_d, want, dtype, "few channels + D %s %s" % (dtype, case))
+    out = torch.empty(got.shape, dtype=torch.from_numpy(got).dtype, device="cuda")
+    rc = _lib.load().amos_conv2d(ctypes.byref(desc), None, dx.data_ptr(), dw.data_ptr(), out.data_ptr(), None, 0, None)
     assert rc == 0
     check(out.cpu().numpy(), ref, dtype, "few channels, no workspace %s %s" % (dtype, case))
 
