@@ -559,7 +559,7 @@ static int plan_conv(Plan& pl, int op, const amos_conv_desc_t* d, const amos_ker
     q.sh = c.stride_h; q.sw = c.stride_w; q.ph = c.pad_h; q.pw = c.pad_w; q.dh = c.dil_h; q.dw = c.dil_w;
     q.taps = fw.taps; q.taps_p = fw.taps_p; q.Wp = fw.Wp; q.rows_max = fw.rows_max;
     q.tiles_j = fw.tiles_j; q.k_tiles = fw.k_tiles;
-    q.prep_x_blocks = (int)((c.N * c.H * c.W + 255) / 256);
+    q.prep_x_blocks = (int)((c.N * c.H * c.W + 1023) / 1024);
     q.prep_w_blocks = (int)(((int64_t)fw.k_tiles * 64 * fw.taps_p + 255) / 256);
     q.patch_off = fw.patch_off; q.zero_off = fw.zero_off; q.tab_off = fw.tab_off;
     q.patch_bytes = fw.patch_bytes; q.nbuf = fw.nbuf; q.grid_x = fw.grid_x;

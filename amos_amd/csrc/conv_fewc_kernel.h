@@ -51,18 +51,23 @@ __global__ __launch_bounds__(256) void amos_conv_fewc_prepare(const ConvFewcPara
   const int t = threadIdx.x;
   int b = blockIdx.x;
   const int HW = p.H * p.W;
-  if (b < p.prep_x_blocks) {
+  if (b < p.prep_x_blocks) {   // four pixels per thread, 256 apart: their loads overlap
     const int64_t total = (int64_t)p.N * HW;
-    const int64_t idx = (int64_t)b * 256 + t;
-    if (idx == 0) *(uint4*)(p.xt + total * 16) = uint4{0, 0, 0, 0};   // the zero pixel behind the last image
-    if (idx >= total) return;
-    const int n = fast_div((int)idx, p.fd_hw);
-    const int hw = (int)idx - n * HW;
-    const T* src = (const T*)p.x + (int64_t)n * p.C * HW + hw;
-    T v[CE];
+    if (b == 0 && t == 0) *(uint4*)(p.xt + total * 16) = uint4{0, 0, 0, 0};   // the zero pixel behind the last image
+    T v[4][CE];
+    int64_t idx[4];
 #pragma unroll
-    for (int c = 0; c < CE; ++c) v[c] = c < p.C ? src[(int64_t)c * HW] : (T)0;
-    *(uint4*)(p.xt + idx * 16) = *(const uint4*)v;
+    for (int u = 0; u < 4; ++u) {
+      idx[u] = (int64_t)b * 1024 + t + 256 * u;
+      const int ic = (int)(idx[u] < total ? idx[u] : total - 1);
+      const int n = fast_div(ic, p.fd_hw);
+      const T* src = (const T*)p.x + (int64_t)n * p.C * HW + (ic - n * HW);
+#pragma unroll
+      for (int c = 0; c < CE; ++c) v[u][c] = c < p.C ? src[(int64_t)c * HW] : (T)0;   // (uniform)
+    }
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+      if (idx[u] < total) *(uint4*)(p.xt + idx[u] * 16) = *(const uint4*)v[u];
     return;
   }
   b -= p.prep_x_blocks;
@@ -138,11 +143,15 @@ __global__ __launch_bounds__(512) void amos_conv_fewc(const ConvFewcParams p) {
   const int a_row = col * p.taps_p, a_row1 = (32 + col) * p.taps_p;
   out_t* const out = (out_t*)p.y;
   int buf = 0;
+  bool counted = false;   // the previous tile ended with exactly 32 store instructions per wave
   for (; item < items; item += gridDim.x) {
-    // this wave's copies (and the previous tile's stores) are done; then everybody's are, and
-    // everybody is past the previous tile's reads of the other buffer
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    __syncthreads();
+    // This wave's copies are done; then everybody's are, and everybody is past the previous
+    // tile's reads of the other buffer.  Memory operations complete in order and the previous
+    // tile's stores were issued after this tile's copies: where their number is known they may
+    // stay in flight and drain under this tile's MFMAs.
+    // (the barrier as an instruction: __syncthreads() is also a fence that drains every store)
+    if (counted) asm volatile("s_waitcnt vmcnt(32) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+    else asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
     const int next = item + gridDim.x;
     if (p.nbuf == 2 && next < items) issue_patch(next, buf ^ 1);
 
@@ -203,7 +212,15 @@ __global__ __launch_bounds__(512) void amos_conv_fewc(const ConvFewcParams p) {
     }
 
     // ---- store: register r of a 32x32 tile is row 8*(r/4) + 4*half + r%4, column col
-    if (j < OPQ) {
+    // (uniform) every pixel and output channel of the tile exists, nothing to add: 32 plain stores
+    const bool full = j0 + 255 < OPQ && k0 + 64 <= p.K && p.epi.dt == EPI_NONE && p.nbuf == 2;
+    if (full) {
+      out_t* const o = out + (int64_t)n * p.K * OPQ + (int64_t)(k0 + 4 * half) * OPQ + j;
+#pragma unroll
+      for (int a = 0; a < 2; ++a)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) o[(int64_t)(a * 32 + 8 * (r >> 2) + (r & 3)) * OPQ] = acc[a][r];
+    } else if (j < OPQ) {
 #pragma unroll
       for (int a = 0; a < 2; ++a) {
         const int i0 = k0 + a * 32 + 4 * half;
@@ -226,6 +243,7 @@ __global__ __launch_bounds__(512) void amos_conv_fewc(const ConvFewcParams p) {
         }
       }
     }
+    counted = full;
     if (p.nbuf == 2) {
       buf ^= 1;
     } else if (next < items) {   // one buffer: refill it once everybody has read it
