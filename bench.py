@@ -157,6 +157,12 @@ def run_all_configs(cpu=True, only=None):
         ops.conv_desc((16, 32, 1, 112, 112), (32, 1, 1, 3, 3), torch.float16, (1, 1, 1), (0, 1, 1), (1, 1, 1), 32),
         [xd, wd], "float16", 2.0 * 16 * 32 * 112 * 112 * 9, 16 * 32 * 112 * 112 * 6 + 32 * 9 * 2,
         (16, 32, 112, 112), None, None)
+    # ResNet's stem at batch 16 (three input channels: the kernel whose reduction unit is the pixel)
+    xs, ws = f16(rng.standard_normal((16, 3, 224, 224))), f16(rng.standard_normal((64, 3, 7, 7)) * 0.1)
+    add("stem fp16 conv2d N16 C3 224x224 K64 7x7/2", _lib.AMOS_OP_CONV2D,
+        ops.conv_desc((16, 3, 1, 224, 224), (64, 3, 1, 7, 7), torch.float16, (1, 2, 2), (0, 3, 3), (1, 1, 1)),
+        [xs, ws], "float16", 2.0 * 16 * 112 * 112 * 64 * 147, 16 * 3 * 224 * 224 * 2 + 64 * 147 * 2 + 16 * 64 * 112 * 112 * 4,
+        (16, 64, 112, 112), None, None)
     return rows
 
 
