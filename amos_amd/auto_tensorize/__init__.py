@@ -15,4 +15,4 @@ from .runtime import build, array, context, Module, NDArray  # noqa: F401
 from .auto_tensorize import (AutoTensorizeResult, auto_tensorize, auto_tensorize_compute,  # noqa: F401
                              auto_tensorize_schedule, auto_tensorize_v4, get_schedule)
 from .network import (AutoScheduleMultiGraphDispatch, AutoTensorizeContext, SubGraph, evaluate_graph,  # noqa: F401
-                      NETWORKS, bert_base, mobilenet_v1, resnet18, resnet50)
+                      NETWORKS, bert_base, mi_lstm, mobilenet_v1, resnet18, resnet50, shufflenet)

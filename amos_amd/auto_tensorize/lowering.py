@@ -888,6 +888,73 @@ def _lower_grouped_conv(main_op, l0, l1):
     return LoweredOp(kind, code, c, [src, wt], main_op.output(0), attrs)
 
 
+def _lower_batch_conv(main_op, l0, l1):
+    """Convolution with a filter bank per image (benchmark/amos/mapping_batchconv2d_tensorcore.py:7-40:
+    Conv[n,k,p,q] = sum Pad[n,rc,...] * B[n,k,rc,rr,rs]): the image index reaches both operands, so it
+    is a batch of independent products -- exactly a grouped convolution of ONE image whose
+    channels are the N*C channels of all images and whose groups are the images.  The memory of
+    A [N][C][...], B [N][K][C][...] and the output [N][K][...] is already that convolution's."""
+    spatial, reduce_ = list(main_op.axis), list(main_op.reduce_axis)
+    nsp = len(spatial) - 2
+    if nsp not in (1, 2, 3) or len(reduce_) != nsp + 1:
+        return None
+    n_iv, k_iv, out_sp = spatial[0], spatial[1], spatial[2:]
+    rc, red_sp = reduce_[0], reduce_[1:]
+    variables = [iv.var for iv in spatial + reduce_]
+
+    def try_roles(lx, lw):
+        if not isinstance(lw.tensor.op, te.PlaceholderOp) or len(lw.indices) != nsp + 3:
+            return None
+        if any(i is not v for i, v in zip(lw.indices, [n_iv.var, k_iv.var, rc.var] + [r.var for r in red_sp])):
+            return None
+        rx = _resolve_dims(lx, variables)
+        if rx is None:
+            return None
+        xt, fx = rx
+        if len(fx) != nsp + 2 or fx[0] != ({n_iv.var: 1}, 0) or fx[1] != ({rc.var: 1}, 0):
+            return None
+        strides, dils = [], []
+        for d in range(nsp):
+            coef, const = fx[2 + d]
+            if const != 0 or set(coef) - {out_sp[d].var, red_sp[d].var}:
+                return None
+            strides.append(int(coef.get(out_sp[d].var, 1)))
+            dils.append(int(coef.get(red_sp[d].var, 1)))
+        return xt, strides, dils
+
+    roles, lx, lw = try_roles(l0, l1), l0, l1
+    if roles is None:
+        roles, lx, lw = try_roles(l1, l0), l1, l0
+    if roles is None:
+        return None
+    xt, strides, dils = roles
+    src, pads = _pad_stage(xt)
+    xs, ws = [int(e) for e in src.shape], [int(e) for e in lw.tensor.shape]
+    N, C, K, win = xs[0], xs[1], ws[1], ws[3:]
+    if ws[0] != N or ws[2] != C or int(rc.dom.extent) != C or [int(r.dom.extent) for r in red_sp] != win:
+        raise NoKernelError("per-image filters %s do not go with activations %s" % (ws, xs))
+    for d in range(nsp):
+        want = (xs[2 + d] + 2 * pads[d] - ((win[d] - 1) * dils[d] + 1)) // strides[d] + 1
+        if int(out_sp[d].dom.extent) != want:
+            raise NoKernelError("output extent %d is not what stride / padding / dilation give (%d)"
+                                % (int(out_sp[d].dom.extent), want))
+    ind, outd = _dtype_pair(lx, lw, main_op.output(0))
+    c = _lib.ConvDesc()
+    lead = 3 - nsp
+    c.N, c.C, c.D, c.H, c.W = [1, N * C] + [1] * lead + xs[2:]
+    c.K, _, c.T, c.R, c.S = [N * K, C] + [1] * lead + win
+    c.stride_d, c.stride_h, c.stride_w = [1] * lead + strides
+    c.pad_d, c.pad_h, c.pad_w = [0] * lead + pads
+    c.dil_d, c.dil_h, c.dil_w = [1] * lead + dils
+    c.in_dtype, c.out_dtype = ind, outd
+    c.groups = N
+    J = _numel([iv.dom.extent for iv in out_sp])
+    attrs = dict(x_shape=[1, N * C] + xs[2:], w_shape=[N * K, C] + win, stride=strides, pad=pads, dil=dils,
+                 dtype=lx.dtype, J=J, K_out=N * K, K_red=C * _numel(win), groups=N)
+    kind, code = ("conv2d", _lib.AMOS_OP_CONV2D) if nsp <= 2 else ("conv3d", _lib.AMOS_OP_CONV3D)
+    return LoweredOp(kind, code, c, [src, lw.tensor], main_op.output(0), attrs)
+
+
 def lower_main_op(main_op, target_dag=None):
     """ComputeOp that matched a GEMM-like intrinsic -> LoweredOp; with the compute DAG it
     belongs to, an element-wise addition behind it is fused into the kernel"""
@@ -901,7 +968,7 @@ def _lower_main_op(main_op):
     variables = [iv.var for iv in iters]
     forms0 = [te.affine_form(i, variables) for i in l0.indices]
     forms1 = [te.affine_form(i, variables) for i in l1.indices]
-    for fn in (_lower_strided_gemm, _lower_grouped_conv):
+    for fn in (_lower_strided_gemm, _lower_grouped_conv, _lower_batch_conv):
         low = fn(main_op, l0, l1)
         if low is not None:
             return low

@@ -117,6 +117,28 @@ def depthwise_conv2d_nchw(N, C, H, W, R, S, stride, padding, in_dtype="float16",
     return [A, B, Reshaped]
 
 
+def grouped_conv2d_nchw(N, C, H, W, K, R, S, stride, padding, groups, in_dtype="float16", out_dtype="float32"):
+    """convolution in channel groups (benchmark/amos/mapping_groupedconv2d_tensorcore.py:7-60)"""
+    pH, pW = H + 2 * padding, W + 2 * padding
+    cg, kg = C // groups, K // groups
+    A = te.placeholder([N, C, H, W], dtype=in_dtype, name="A")
+    B = te.placeholder([K, cg, R, S], dtype=in_dtype, name="B")
+    Pad = te.compute([N, C, pH, pW], lambda n, c, h, w: tir.if_then_else(
+        tir.all(h >= padding, h - padding < H, w >= padding, w - padding < W),
+        A[n, c, h - padding, w - padding], tir.const(0.0, A.dtype)), name="Pad")
+    A_reshaped = te.compute([N, groups, cg, pH, pW], lambda n, c_o, c_i, r, s: Pad[n, c_o * cg + c_i, r, s])
+    B_reshaped = te.compute([groups, kg, cg, R, S], lambda k_o, k_i, c, r, s: B[k_o * kg + k_i, c, r, s])
+    rc = te.reduce_axis([0, cg], name="rc")
+    rr = te.reduce_axis([0, R], name="rr")
+    rs = te.reduce_axis([0, S], name="rs")
+    P, Q = (pH - R) // stride + 1, (pW - S) // stride + 1
+    Conv = te.compute([N, groups, kg, P, Q], lambda n, k_o, k_i, p, q: te.sum(
+        (A_reshaped[n, k_o, rc, p * stride + rr, q * stride + rs] * B_reshaped[k_o, k_i, rc, rr, rs]).astype(out_dtype),
+        axis=[rc, rr, rs]), name="Conv")
+    Reshaped = te.compute([N, K, P, Q], lambda n, k, p, q: Conv[n, k // kg, k % kg, p, q], name="Reshaped")
+    return [A, B, Reshaped]
+
+
 def _subgraphs(net, layers):
     return [SubGraph("%s:subgraph%d" % (net, i), ts, cnt, note) for i, (note, ts, cnt) in enumerate(layers)]
 
@@ -187,7 +209,49 @@ def bert_base(batch=1, seq=512, in_dtype="float16", out_dtype="float32", blocks=
     return _subgraphs("bertbase", layers)
 
 
-NETWORKS = {"resnet18": None, "resnet50": resnet50, "mobilenet_v1": mobilenet_v1, "bertbase": bert_base}
+def shufflenet(batch=1, in_dtype="float16", out_dtype="float32", num_classes=1000, groups=3):
+    """ShuffleNet (groups = 3) at 224x224 (python/tvm/tensor_graph/testing/models/shufflenet.py:68-185):
+    the first convolution; per unit a grouped 1x1, a depthwise 3x3 (strided in the first unit of a
+    stage, whose output channels are the stage's minus its input's: the rest is a pooled copy) and
+    a grouped 1x1; the classifier.  Channel shuffles, pooling and concatenation have no reduction."""
+    b, d = batch, (in_dtype, out_dtype)
+    layers = [("conv 3x3/2 3->24 @224", conv2d_nchw(b, 3, 224, 224, 24, 3, 3, 2, 1, *d), 1)]
+    cin, hw = 24, 56
+    for stage, (cout, repeats) in enumerate([(240, 3), (480, 7), (960, 3)]):
+        tag = "stage%d" % (stage + 2)
+        grown, mid = cout - cin, (cout - cin) // 4
+        layers += [
+            ("%s grouped 1x1 %d->%d @%d" % (tag, cin, mid, hw), grouped_conv2d_nchw(b, cin, hw, hw, mid, 1, 1, 1, 0, groups, *d), 1),
+            ("%s depthwise 3x3/2 %d @%d" % (tag, mid, hw), depthwise_conv2d_nchw(b, mid, hw, hw, 3, 3, 2, 1, *d), 1),
+            ("%s grouped 1x1 %d->%d @%d" % (tag, mid, grown, hw // 2), grouped_conv2d_nchw(b, mid, hw // 2, hw // 2, grown, 1, 1, 1, 0, groups, *d), 1),
+        ]
+        hw //= 2
+        mid = cout // 4
+        layers += [
+            ("%s grouped 1x1 %d->%d @%d" % (tag, cout, mid, hw), grouped_conv2d_nchw(b, cout, hw, hw, mid, 1, 1, 1, 0, groups, *d), repeats),
+            ("%s depthwise 3x3 %d @%d" % (tag, mid, hw), depthwise_conv2d_nchw(b, mid, hw, hw, 3, 3, 1, 1, *d), repeats),
+            ("%s grouped 1x1 %d->%d @%d" % (tag, mid, cout, hw), grouped_conv2d_nchw(b, mid, hw, hw, cout, 1, 1, 1, 0, groups, *d), repeats),
+        ]
+        cin = cout
+    layers.append(("fc 960->%d" % num_classes, dense(b, num_classes, 960, *d), 1))
+    return _subgraphs("shufflenet", layers)
+
+
+def mi_lstm(batch=1, in_dtype="float16", out_dtype="float32", input_size=512, hidden=1024):
+    """one step of the MI-LSTM cell (python/tvm/tensor_graph/testing/models/MI_LSTM.py:71-124;
+    benchmark/amos/mapping_milstm_tensorcore.py:19-26): four gate projections of the hidden state,
+    four of the input, the classifier; the gates' element-wise arithmetic has no reduction"""
+    d = (in_dtype, out_dtype)
+    layers = [
+        ("gate projection of h %d->%d (f, i, z, o)" % (hidden, hidden), dense(batch, hidden, hidden, *d), 4),
+        ("gate projection of x %d->%d (f, i, z, o)" % (input_size, hidden), dense(batch, hidden, input_size, *d), 4),
+        ("classifier %d->10" % hidden, dense(batch, 10, hidden, *d), 1),
+    ]
+    return _subgraphs("milstm", layers)
+
+
+NETWORKS = {"resnet18": None, "resnet50": resnet50, "mobilenet_v1": mobilenet_v1, "bertbase": bert_base,
+            "shufflenet": shufflenet, "milstm": mi_lstm}
 
 
 SKIPPED_RESNET18 = ("batch norm x20, ReLU x17, max pool, global average pool, residual additions x8: "

@@ -257,9 +257,10 @@ def model_check():
     return out
 
 
-def network_report(trials=200, networks=("resnet18", "resnet50", "mobilenet_v1", "bertbase"), batches=(1, 16)):
+def network_report(trials=200, networks=("resnet18", "resnet50", "mobilenet_v1", "bertbase", "shufflenet", "milstm"),
+                   batches=(1, 16)):
     """The tensorisable layers of whole networks through the network dispatcher (the flow of the
-    reference's benchmark/amos/mapping_{resnet18,resnet50,mobilenetv1,bertbase}_tensorcore.py): per
+    reference's benchmark/amos/mapping_{resnet18,resnet50,mobilenetv1,bertbase,shufflenet,milstm}_tensorcore.py): per
     distinct layer the tuned kernel and its time, and the sum over the network's layers"""
     import contextlib
     import io
@@ -302,9 +303,10 @@ def main():
                     help="also rank every kernel configuration of a set of shapes by the mapper's model "
                          "and by measurement, write JSON here")
     ap.add_argument("--network", default=None,
-                    help="also tune and time the tensorisable layers of ResNet-18, ResNet-50, MobileNet-V1 and "
-                         "BERT-base at batch 1 and 16 through the network dispatcher, write JSON here")
-    ap.add_argument("--networks", default="resnet18,resnet50,mobilenet_v1,bertbase",
+                    help="also tune and time the tensorisable layers of ResNet-18, ResNet-50, MobileNet-V1, "
+                         "BERT-base, ShuffleNet and an MI-LSTM cell at batch 1 and 16 through the network "
+                         "dispatcher, write JSON here")
+    ap.add_argument("--networks", default="resnet18,resnet50,mobilenet_v1,bertbase,shufflenet,milstm",
                     help="the networks --network covers, comma-separated")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a 256 MiB device copy, the known-size kernel that rocprofv3's "

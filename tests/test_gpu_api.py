@@ -9,7 +9,7 @@ import pytest
 import amos_amd.tvm as tvm
 from amos_amd.tvm import auto_tensorize as at
 from oracle import cpu_oracle as co
-from test_mapper import (batched_fc, conv1d, conv2d, conv2d_layout, depthwise_conv2d, from_nkpq, gemm, gemv,
+from test_mapper import (batch_conv2d, batched_fc, conv1d, conv2d, conv2d_layout, depthwise_conv2d, from_nkpq, gemm, gemv,
                          grouped_conv2d, grouped_conv_reference, mean, scan, to_nchw, transposed_conv2d)
 
 pytestmark = pytest.mark.gpu
@@ -294,10 +294,25 @@ def test_mean_and_scan_script_flows(gpu, tmp_path):
     assert np.array_equal(got, np.cumsum(a.astype(np.float32), axis=1))     # small integers: exact
 
 
-@pytest.mark.parametrize("kind", ["grouped", "depthwise"])
+@pytest.mark.parametrize("kind", ["grouped", "depthwise", "batch"])
 def test_grouped_conv_script_flow(gpu, tmp_path, kind):
     """reference computes: benchmark/amos/mapping_groupedconv2d_tensorcore.py:7-60,
-    mapping_depthwiseconv2d_tensorcore.py:7-48"""
+    mapping_depthwiseconv2d_tensorcore.py:7-48, mapping_batchconv2d_tensorcore.py:7-40 (a filter
+    bank per image: the images are the groups of a one-image convolution)"""
+    if kind == "batch":
+        N, C, H, W, K, R, S, stride, padding = 6, 32, 14, 14, 48, 3, 3, 1, 1
+        A, B, Out = batch_conv2d(N, C, H, W, K, R, S, stride, padding)
+        rng = np.random.default_rng(10)
+        a = rng.uniform(-1, 1, (N, C, H, W)).astype(np.float16)
+        b = rng.uniform(-1, 1, (N, K, C, R, S)).astype(np.float16)
+        got, result = _run_script_flow([A, B, Out], {"A": a, "B": b}, tmp_path, kind, transform_strict=False)
+        low = result.sch_app.lowered
+        assert low.kind == "conv2d" and low.desc.groups == N and low.desc.N == 1
+        ref = np.stack([co.lib_conv2d(a[n:n + 1], b[n], "float16", stride, padding, 1, acc="float64")[0]
+                        for n in range(N)])
+        mx, mean = co.rel_errors(got, ref)
+        assert got.shape == ref.shape and mx <= 1e-2 and mean <= 1e-3
+        return
     if kind == "grouped":
         N, C, H, W, K, R, S, stride, padding, groups = 4, 64, 14, 14, 128, 3, 3, 1, 1, 4
         A, B, Out = grouped_conv2d(N, C, H, W, K, R, S, stride, padding, groups)

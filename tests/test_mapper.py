@@ -772,4 +772,57 @@ def test_other_networks_layer_lists():
     bert = _at.bert_base(1)
     assert sum(sg.count for sg in bert) == 96
     assert macs(bert) == 12 * (4 * 512 * 768 ** 2 + 2 * 512 * 768 * 3072 + 2 * 12 * 512 ** 2 * 64)
-    assert set(_at.NETWORKS) == {"resnet18", "resnet50", "mobilenet_v1", "bertbase"}
+    assert set(_at.NETWORKS) == {"resnet18", "resnet50", "mobilenet_v1", "bertbase", "shufflenet", "milstm"}
+    # ShuffleNet (groups 3) as the reference's model builds it: 1 + 3 x (3 + 3 x repeats) + 1 layers;
+    # multiply-accumulates from its channel arithmetic (shufflenet.py:68-185)
+    sh = _at.shufflenet(1)
+    assert sum(sg.count for sg in sh) == 1 + 3 * 3 + 3 * (3 + 7 + 3) + 1
+    want, cin, hw = 112 * 112 * 24 * 27, 24, 56
+    for cout, rep in ((240, 3), (480, 7), (960, 3)):
+        mid = (cout - cin) // 4
+        want += hw * hw * mid * cin // 3 + (hw // 2) ** 2 * mid * 9 + (hw // 2) ** 2 * (cout - cin) * mid // 3
+        hw //= 2
+        mid = cout // 4
+        want += rep * (hw * hw * mid * cout // 3 + hw * hw * mid * 9 + hw * hw * cout * mid // 3)
+        cin = cout
+    assert macs(sh) == want + 960 * 1000
+    lstm = _at.mi_lstm(8)
+    assert sum(sg.count for sg in lstm) == 9 and macs(lstm) == 8 * (4 * 1024 * 1024 + 4 * 512 * 1024 + 10 * 1024)
+
+
+def batch_conv2d(N, C, H, W, K, R, S, stride, padding, in_dtype="float16", out_dtype="float32"):
+    """reference: benchmark/amos/mapping_batchconv2d_tensorcore.py:7-40 (a filter bank per image)"""
+    pH, pW = H + 2 * padding, W + 2 * padding
+    A = te.placeholder([N, C, H, W], dtype=in_dtype, name="A")
+    B = te.placeholder([N, K, C, R, S], dtype=in_dtype, name="B")
+    Pad = te.compute([N, C, pH, pW], lambda n, c, h, w: tir.if_then_else(
+        tir.all(h >= padding, h - padding < H, w >= padding, w - padding < W),
+        A[n, c, h - padding, w - padding], tir.const(0.0, A.dtype)), name="Pad")
+    rc = te.reduce_axis([0, C], name="rc")
+    rr = te.reduce_axis([0, R], name="rr")
+    rs = te.reduce_axis([0, S], name="rs")
+    P, Q = (pH - R) // stride + 1, (pW - S) // stride + 1
+    Conv = te.compute([N, K, P, Q], lambda n, k, p, q: te.sum(
+        (Pad[n, rc, p * stride + rr, q * stride + rs] * B[n, k, rc, rr, rs]).astype(out_dtype),
+        axis=[rc, rr, rs]), name="Conv")
+    return A, B, Conv
+
+
+def test_batch_conv_lowering():
+    """per-image filters lower to a grouped convolution of one image with the images as groups;
+    checked against the brute-force evaluation of the compute as written"""
+    from amos_amd.auto_tensorize.lowering import lower_main_op
+    A, B, Out = batch_conv2d(3, 4, 6, 5, 6, 3, 2, 2, 1)
+    dag = at.compute_dag_from_tensors([Out])
+    main = [op for op in dag.op_lst if op.reduce_axis][0]
+    assert at.get_match_results(dag, "hip")
+    low = lower_main_op(main, dag)
+    c = low.desc
+    assert low.kind == "conv2d" and (c.N, c.C, c.K, c.groups, c.R, c.S) == (1, 12, 18, 3, 3, 2)
+    assert (c.stride_h, c.stride_w, c.pad_h, c.pad_w) == (2, 2, 1, 1) and [t.name for t in low.inputs] == ["A", "B"]
+    rng = np.random.default_rng(21)
+    a = rng.integers(-3, 4, (3, 4, 6, 5)).astype(np.float64)
+    b = rng.integers(-3, 4, (3, 6, 4, 3, 2)).astype(np.float64)
+    want = te_interp.evaluate(Out, {"A": a, "B": b})
+    got = grouped_conv_reference(a.reshape(1, 12, 6, 5), b.reshape(18, 4, 3, 2), (2, 2), (1, 1), 3)
+    assert np.array_equal(got.reshape(want.shape), want)
