@@ -781,6 +781,73 @@ def test_conv_few_channels(gpu, dtype, case):
     check(out.cpu().numpy(), ref, dtype, "few channels, no workspace %s %s" % (dtype, case))
 
 
+def _random_route_cases():
+    """seeded random int8 convolutions aimed at the routes beside the patch-staged and the
+    register-staged kernels: few input channels, strided 1x1, depthwise, im2col copy"""
+    rng = np.random.default_rng(20240607)
+    cases = []
+    for _ in range(10):     # few channels
+        R, S = int(rng.integers(1, 8)), int(rng.integers(2, 8))
+        cases.append(("few", int(rng.integers(3, 12)), int(rng.integers(1, 17)), int(rng.integers(24, 90)),
+                      int(rng.integers(24, 130)), int(rng.integers(33, 140)), R, S,
+                      (int(rng.integers(1, 4)), int(rng.integers(1, 4))), (int(rng.integers(0, R)), int(rng.integers(0, S))),
+                      (int(rng.integers(1, 3)), int(rng.integers(1, 3))), 1))
+    for _ in range(8):      # strided 1x1
+        cases.append(("sub", int(rng.integers(6, 20)), int(rng.integers(40, 300)), int(rng.integers(14, 40)),
+                      int(rng.integers(14, 40)), int(rng.integers(100, 400)), 1, 1,
+                      (int(rng.integers(1, 4)), int(rng.integers(2, 4))), (0, 0), (1, 1), 1))
+    for _ in range(10):     # depthwise, with and without a channel multiplier
+        C = int(rng.integers(3, 70))
+        R, S = int(rng.integers(1, 6)), int(rng.integers(1, 6))
+        cases.append(("dw", int(rng.integers(1, 5)), C, int(rng.integers(5, 60)), int(rng.integers(5, 60)),
+                      C * int(rng.integers(1, 4)), R, S, (int(rng.integers(1, 4)), int(rng.integers(1, 4))),
+                      (int(rng.integers(0, R + 1)), int(rng.integers(0, S + 1))),
+                      (int(rng.integers(1, 3)), int(rng.integers(1, 3))), C))
+    for _ in range(6):      # more than a pixel of channels, no 128-byte chunk, wide output
+        cases.append(("col", int(rng.integers(2, 6)), int(rng.integers(17, 60)), int(rng.integers(12, 40)),
+                      int(rng.integers(12, 40)), int(rng.integers(256, 400)), int(rng.integers(1, 5)), int(rng.integers(2, 5)),
+                      (int(rng.integers(1, 3)), int(rng.integers(1, 3))), (int(rng.integers(0, 2)), int(rng.integers(0, 2))),
+                      (1, 1), 1))
+    return cases
+
+
+@pytest.mark.parametrize("case", _random_route_cases())
+def test_conv_routes_random_int8(gpu, case):
+    """whatever kernel the default picks against the register-staged implicit GEMM of the same
+    convolution: int8, so the two must agree bit for bit; a quarter of the cases also against the
+    oracle"""
+    from amos_amd import _lib, ops
+    kind, N, C, H, W, K, R, S, st, pd, dl, G = case
+    if (H + 2 * pd[0] - ((R - 1) * dl[0] + 1)) < 0 or (W + 2 * pd[1] - ((S - 1) * dl[1] + 1)) < 0:
+        pytest.skip("window larger than the padded input")
+    rng = np.random.default_rng(hash(case) % 2**32)
+    x = make_operand(rng, (N, C, H, W), "int8")
+    w = make_operand(rng, (K, C // G, R, S), "int8")
+    dx, dw = to_device(x, "int8"), to_device(w, "int8")
+    got = ops.conv2d(dx, dw, st, pd, dl, groups=G).cpu().numpy()
+    other = ops.conv2d(dx, dw, st, pd, dl, groups=G, config=dict(tile_i=64, tile_j=64, split_k=1, pipeline=1)).cpu().numpy()
+    desc = ops.conv_desc((N, C, 1, H, W), (K, C // G, 1, R, S), dx.dtype, (1,) + st, (0,) + pd, (1,) + dl, G)
+    name = ops.kernel_name(_lib.AMOS_OP_CONV2D, desc, None)
+    assert np.array_equal(got, other), (name, case)
+    if hash(case) % 4 == 0 and G == 1:
+        assert np.array_equal(got, co.lib_conv2d(x, w, "int8", st, pd, dl)), (name, case)
+
+
+def test_conv_few_channels_single_patch_buffer(gpu):
+    """rows so wide that two patch buffers do not fit LDS: the kernel refills its one buffer
+    between tiles"""
+    from amos_amd import _lib, ops
+    N, C, H, W, K = 2, 3, 20, 1198, 64
+    rng = np.random.default_rng(5)
+    x = make_operand(rng, (N, C, H, W), "int8")
+    w = make_operand(rng, (K, C, 3, 3), "int8")
+    dx, dw = to_device(x, "int8"), to_device(w, "int8")
+    desc = ops.conv_desc((N, C, 1, H, W), (K, C, 1, 3, 3), dx.dtype, (1, 1, 1), (0, 1, 1), (1, 1, 1))
+    assert ops.kernel_name(_lib.AMOS_OP_CONV2D, desc, None) == "amos_conv_few_channels<i8>"
+    got = ops.conv2d(dx, dw, 1, 1, 1).cpu().numpy()
+    assert np.array_equal(got, co.lib_conv2d(x, w, "int8", 1, 1, 1))
+
+
 DEPTHWISE_CASES = [
     # N, C, D, H, W, mult, T, R, S, stride, pad, dil, kernel-name suffix
     (2, 32, 1, 28, 28, 1, 1, 3, 3, (1, 1, 1), (0, 1, 1), (1, 1, 1), ",3x3>"),       # MobileNet's 3x3
