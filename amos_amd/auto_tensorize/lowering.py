@@ -33,6 +33,9 @@ class LoweredOp(object):
         self.gathers = {}
         # {0 or 1: numpy array}: inputs[k] is computed from its indices alone; the module holds it
         self.constants = {}
+        # OperandView (src None) or None: the kernel writes a tensor of the same size in another
+        # order and `output` is gathered from it (a stage behind the main op that no epilogue folds in)
+        self.out_view = None
 
     def flops(self):
         a = self.attrs
@@ -955,6 +958,97 @@ def _lower_batch_conv(main_op, l0, l1):
     return LoweredOp(kind, code, c, [src, lw.tensor], main_op.output(0), attrs)
 
 
+def _lower_capsule_conv(main_op, l0, l1):
+    """Convolution whose filters carry a trailing capsule axis
+    (benchmark/amos/mapping_capsuleconv2d_tensorcore.py:33-72:
+    Out[b,k,h,w,s] = sum padded[b,rc,h*st+rh*dil,w*st+rw*dil] * B[k,rc,rh,rw,s]): (k, s) together are
+    the output channels of an ordinary convolution with K * caps filters.  The filters are
+    gathered to [K*caps][C][window] in front of the kernel and the result [N][K*caps][spatial] to
+    the compute's [N][K][spatial][caps] behind it."""
+    spatial, reduce_ = list(main_op.axis), list(main_op.reduce_axis)
+    nsp = len(spatial) - 3
+    if nsp not in (1, 2, 3) or len(reduce_) != nsp + 1:
+        return None
+    n_iv, k_iv, out_sp, s_iv = spatial[0], spatial[1], spatial[2:-1], spatial[-1]
+    variables = [iv.var for iv in spatial + reduce_]
+
+    def try_roles(lx, lw):
+        if not isinstance(lw.tensor.op, te.PlaceholderOp) or len(lw.indices) != nsp + 3:
+            return None
+        rx = _resolve_dims(lx, variables)
+        if rx is None:
+            return None
+        xt, fx = rx
+        if len(fx) != nsp + 2 or fx[0] != ({n_iv.var: 1}, 0):
+            return None
+        rc = [r for r in reduce_ if fx[1] == ({r.var: 1}, 0)]
+        if len(rc) != 1:
+            return None
+        rc = rc[0]
+        strides, dils, red_sp = [], [], []
+        for d in range(nsp):
+            coef, const = fx[2 + d]
+            rv = [r for r in reduce_ if r.var in coef and r is not rc]
+            if const != 0 or len(rv) != 1 or set(coef) - {out_sp[d].var, rv[0].var}:
+                return None
+            red_sp.append(rv[0])
+            strides.append(int(coef.get(out_sp[d].var, 1)))
+            dils.append(int(coef[rv[0].var]))
+        want = [k_iv.var, rc.var] + [r.var for r in red_sp] + [s_iv.var]
+        if any(i is not v for i, v in zip(lw.indices, want)):
+            return None
+        return xt, rc, red_sp, strides, dils
+
+    roles, lx, lw = try_roles(l0, l1), l0, l1
+    if roles is None:
+        roles, lx, lw = try_roles(l1, l0), l1, l0
+    if roles is None:
+        return None
+    xt, rc, red_sp, strides, dils = roles
+    src, pads = _pad_stage(xt)
+    xs, ws = [int(e) for e in src.shape], [int(e) for e in lw.tensor.shape]
+    N, C = xs[0], xs[1]
+    K, win, caps = ws[0], ws[2:-1], ws[-1]
+    if ws[1] != C or int(rc.dom.extent) != C or [int(r.dom.extent) for r in red_sp] != win or \
+            int(s_iv.dom.extent) != caps or int(k_iv.dom.extent) != K:
+        raise NoKernelError("capsule filters %s do not go with activations %s" % (ws, xs))
+    osp = [int(iv.dom.extent) for iv in out_sp]
+    for d in range(nsp):
+        want = (xs[2 + d] + 2 * pads[d] - ((win[d] - 1) * dils[d] + 1)) // strides[d] + 1
+        if osp[d] != want:
+            raise NoKernelError("output extent %d is not what stride / padding / dilation give (%d)" % (osp[d], want))
+    ind, outd = _dtype_pair(lx, lw, main_op.output(0))
+    Kc, trs, pq = K * caps, _numel(win), _numel(osp)
+    c = _lib.ConvDesc()
+    lead = 3 - nsp
+    c.N, c.C, c.D, c.H, c.W = [N, C] + [1] * lead + xs[2:]
+    c.K, _, c.T, c.R, c.S = [Kc, C] + [1] * lead + win
+    c.stride_d, c.stride_h, c.stride_w = [1] * lead + strides
+    c.pad_d, c.pad_h, c.pad_w = [0] * lead + pads
+    c.dil_d, c.dil_h, c.dil_w = [1] * lead + dils
+    c.in_dtype, c.out_dtype = ind, outd
+    attrs = dict(x_shape=xs, w_shape=[Kc, C] + win, stride=strides, pad=pads, dil=dils, dtype=lx.dtype,
+                 J=N * pq, K_out=Kc, K_red=C * trs)
+    kind, code = ("conv2d", _lib.AMOS_OP_CONV2D) if nsp <= 2 else ("conv3d", _lib.AMOS_OP_CONV3D)
+    low = LoweredOp(kind, code, c, [src, lw.tensor], main_op.output(0), attrs)
+    # filters: element (k*caps + s, c, window...) of the kernel's operand is B[k][c][window...][s]
+    w_tabs = [[(i // caps) * (C * trs * caps) + i % caps for i in range(Kc)], [cc * trs * caps for cc in range(C)]]
+    stride = trs
+    for e in win:
+        stride //= e
+        w_tabs.append([i * stride * caps for i in range(e)])
+    low.gathers[1] = OperandView(lw.tensor, [Kc, C] + win, w_tabs, lw.tensor.dtype)
+    # result: Out[n][k][spatial...][s] is element (n, k*caps + s, spatial...) of what the kernel writes
+    o_tabs = [[n * Kc * pq for n in range(N)], [k * caps * pq for k in range(K)]]
+    stride = pq
+    for e in osp:
+        stride //= e
+        o_tabs.append([i * stride for i in range(e)])
+    o_tabs.append([sx * pq for sx in range(caps)])
+    low.out_view = OperandView(None, [N, K] + osp + [caps], o_tabs, main_op.output(0).dtype)
+    return low
+
+
 def lower_main_op(main_op, target_dag=None):
     """ComputeOp that matched a GEMM-like intrinsic -> LoweredOp; with the compute DAG it
     belongs to, an element-wise addition behind it is fused into the kernel"""
@@ -968,7 +1062,7 @@ def _lower_main_op(main_op):
     variables = [iv.var for iv in iters]
     forms0 = [te.affine_form(i, variables) for i in l0.indices]
     forms1 = [te.affine_form(i, variables) for i in l1.indices]
-    for fn in (_lower_strided_gemm, _lower_grouped_conv, _lower_batch_conv):
+    for fn in (_lower_strided_gemm, _lower_grouped_conv, _lower_batch_conv, _lower_capsule_conv):
         low = fn(main_op, l0, l1)
         if low is not None:
             return low

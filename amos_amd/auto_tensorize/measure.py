@@ -87,6 +87,13 @@ def evaluate_params_on_device(lowered, params, measure_opt):
             t = g.time(src, ins[pos], number=measure_opt.number, repeat=1, min_repeat_ms=measure_opt.min_repeat_ms)
             lowered._gather_seconds[pos] = t[0]
         extra += lowered._gather_seconds[pos]
+    view = getattr(lowered, "out_view", None)
+    if view is not None:   # the result is reordered behind the kernel: the same for every configuration
+        if not hasattr(lowered, "_out_gather_seconds"):
+            g = ops.Gather(view.shape, view.tables, _TORCH_DTYPE[view.dtype], out.numel(), out.device)
+            lowered._out_gather_seconds = g.time(out.reshape(-1).clone(), out, number=measure_opt.number, repeat=1,
+                                                 min_repeat_ms=measure_opt.min_repeat_ms)[0]
+        extra += lowered._out_gather_seconds
     secs = ops.time_op(lowered.op_code, lowered.desc, ins[0], ins[1], out, config=params.to_config(),
                        number=measure_opt.number, repeat=max(1, measure_opt.repeat),
                        min_repeat_ms=measure_opt.min_repeat_ms, add=random_add_array(lowered, measure_opt.dev_id))

@@ -93,6 +93,7 @@ class Module(object):
         self.imported_modules = [_Source(self)]
         self._gathers = {}     # operand position -> (ops.Gather, materialised operand), made on first use
         self._constants = {}   # operand position -> device tensor of a constant operand
+        self._out_gather = None   # (ops.Gather, the kernel's own output buffer) where the result is reordered
 
     def _kernel_inputs(self, in0, in1):
         """the operands the kernel reads: the caller's arrays, or what the stages in front of an
@@ -123,10 +124,24 @@ class Module(object):
             out.append(a.tensor if isinstance(a, NDArray) else a)
         return out
 
+    def _kernel_output(self, out):
+        """where the kernel writes: the caller's array, or a buffer of the module's from which
+        the caller's array is gathered afterwards"""
+        view = getattr(self.lowered, "out_view", None)
+        if view is None:
+            return out, None
+        if self._out_gather is None:
+            g = ops.Gather(view.shape, view.tables, _TORCH_DTYPE[view.dtype], out.numel(), out.device)
+            self._out_gather = (g, torch.empty(out.numel(), dtype=g.dtype, device=out.device))
+        return self._out_gather[1], self._out_gather[0]
+
     def _run(self, in0, in1, out, add=None):
         cfg = self.params.to_config() if self.params is not None else None
         k0, k1 = self._kernel_inputs(in0, in1)
-        ops.run_desc(self.lowered.op_code, self.lowered.desc, k0, k1, out, config=cfg, add=add)
+        kout, g = self._kernel_output(out)
+        ops.run_desc(self.lowered.op_code, self.lowered.desc, k0, k1, kout, config=cfg, add=add)
+        if g is not None:
+            g(kout, out)
 
     def __call__(self, *arrays):
         self._run(*self._pick(arrays))
@@ -137,9 +152,13 @@ class Module(object):
             out = picked[2]
             in0, in1 = self._kernel_inputs(picked[0], picked[1])
             cfg = self.params.to_config() if self.params is not None else None
-            secs = ops.time_op(self.lowered.op_code, self.lowered.desc, in0, in1, out, config=cfg,
+            kout, og = self._kernel_output(out)
+            secs = ops.time_op(self.lowered.op_code, self.lowered.desc, in0, in1, kout, config=cfg,
                                number=number, repeat=repeat, min_repeat_ms=min_repeat_ms,
                                add=picked[3] if len(picked) > 3 else None)
+            if og is not None:   # the reordering of the result runs on every call too
+                extra = og.time(kout, out, number=number, repeat=repeat, min_repeat_ms=min_repeat_ms)
+                secs = [a + b for a, b in zip(secs, extra)]
             # the stages materialised in front of an operand run on every call: their time counts
             for pos, (g, buf) in self._gathers.items():
                 extra = g.time(picked[pos].contiguous(), buf, number=number, repeat=repeat, min_repeat_ms=min_repeat_ms)

@@ -9,7 +9,7 @@ import pytest
 import amos_amd.tvm as tvm
 from amos_amd.tvm import auto_tensorize as at
 from oracle import cpu_oracle as co
-from test_mapper import (batch_conv2d, batched_fc, conv1d, conv2d, conv2d_layout, depthwise_conv2d, from_nkpq, gemm, gemv,
+from test_mapper import (batch_conv2d, batched_fc, capsule_conv2d, conv1d, conv2d, conv2d_layout, depthwise_conv2d, from_nkpq, gemm, gemv,
                          grouped_conv2d, grouped_conv_reference, mean, scan, to_nchw, transposed_conv2d)
 
 pytestmark = pytest.mark.gpu
@@ -329,3 +329,35 @@ def test_grouped_conv_script_flow(gpu, tmp_path, kind):
     ref = grouped_conv_reference(a, b, stride, padding, groups)
     mx, mean = co.rel_errors(got, ref)
     assert got.shape == ref.shape and mx <= 1e-2 and mean <= 1e-3
+
+
+def test_capsule_conv_script_flow(gpu, tmp_path):
+    """reference compute: benchmark/amos/mapping_capsuleconv2d_tensorcore.py:7-72 (filters with a
+    trailing capsule axis: gathered in front of an ordinary convolution, the result reordered
+    behind it); the module's time_evaluator counts both gathers"""
+    N, C, H, W, K, R, S, caps, stride, padding, dilation = 4, 32, 14, 14, 16, 3, 3, 8, 1, 1, 1
+    A, B, Out = capsule_conv2d(N, C, H, W, K, R, S, caps, stride, padding, dilation)
+    rng = np.random.default_rng(12)
+    a = rng.uniform(-1, 1, (N, C, H, W)).astype(np.float16)
+    b = rng.uniform(-1, 1, (K, C, R, S, caps)).astype(np.float16)
+    got, result = _run_script_flow([A, B, Out], {"A": a, "B": b}, tmp_path, "capsule", transform_strict=False)
+    low = result.sch_app.lowered
+    assert low.kind == "conv2d" and low.desc.K == K * caps and low.out_view is not None and list(low.gathers) == [1]
+    wk = np.ascontiguousarray(b.transpose(0, 4, 1, 2, 3).reshape(K * caps, C, R, S))
+    ref = co.lib_conv2d(a, wk, "float16", stride, padding, dilation, acc="float64")
+    ref = ref.reshape(N, K, caps, H, W).transpose(0, 1, 3, 4, 2)
+    mx, mean = co.rel_errors(got, ref)
+    assert got.shape == ref.shape == (N, K, H, W, caps) and mx <= 1e-2 and mean <= 1e-3
+    # a second call reuses the module's buffers; timing includes the two gathers
+    sch, args = at.get_schedule(result.sch_app, result.params)
+    func = tvm.build(sch, args, "hip")
+    ctx = tvm.context("hip", 0)
+    arrays = [tvm.nd.array(x, ctx) for x in (a, b)] + [tvm.nd.array(np.zeros(got.shape, dtype=np.float32), ctx)]
+    func(*arrays)
+    func(*arrays)
+    ctx.sync()
+    # (a tuned split-K config accumulates with atomics: equal up to the order of additions)
+    assert np.allclose(arrays[-1].asnumpy(), got, rtol=1e-5, atol=1e-5)
+    t = func.time_evaluator(func.entry_name, ctx, number=5, min_repeat_ms=5)(*arrays).mean
+    assert 0 < t < 1e-3
+

@@ -826,3 +826,54 @@ def test_batch_conv_lowering():
     want = te_interp.evaluate(Out, {"A": a, "B": b})
     got = grouped_conv_reference(a.reshape(1, 12, 6, 5), b.reshape(18, 4, 3, 2), (2, 2), (1, 1), 3)
     assert np.array_equal(got.reshape(want.shape), want)
+
+
+def capsule_conv2d(N, C, H, W, K, R, S, caps, stride, padding, dilation, in_dtype="float16", out_dtype="float32"):
+    """reference: benchmark/amos/mapping_capsuleconv2d_tensorcore.py:7-72"""
+    A = te.placeholder([N, C, H, W], dtype=in_dtype, name="A")
+    B = te.placeholder([K, C, R, S, caps], dtype=in_dtype, name="B")
+    P = (H + 2 * padding - dilation * (R - 1) - 1) // stride + 1
+    Q = (W + 2 * padding - dilation * (S - 1) - 1) // stride + 1
+    padded = te.compute([N, C, H + 2 * padding, W + 2 * padding], lambda b, c, h, w: tir.if_then_else(
+        tir.all(h >= padding, h < H + padding, w >= padding, w < W + padding),
+        A[b, c, h - padding, w - padding], tir.const(0, A.dtype)), name="Padding")
+    rc = te.reduce_axis((0, C), name="rc")
+    rw = te.reduce_axis((0, S), name="rw")
+    rh = te.reduce_axis((0, R), name="rh")
+    Out = te.compute((N, K, P, Q, caps), lambda b, k, h, w, s: te.sum(
+        (padded[b, rc, h * stride + rh * dilation, w * stride + rw * dilation] * B[k, rc, rh, rw, s]).astype(out_dtype),
+        axis=[rc, rw, rh]), name="conv2d_capsule")
+    return A, B, Out
+
+
+def apply_out_view(view, flat):
+    """what the module gathers from the kernel's output buffer"""
+    out = np.zeros(view.shape, dtype=flat.dtype)
+    for idx in np.ndindex(*view.shape):
+        out[idx] = flat[sum(view.tables[d][i] for d, i in enumerate(idx))]
+    return out
+
+
+def test_capsule_conv_lowering():
+    """a capsule axis on the filters: an ordinary convolution with K * caps filters between a
+    gather of the filters and one of the result; checked against the compute as written"""
+    from amos_amd.auto_tensorize.lowering import lower_main_op
+    N, C, H, W, K, R, S, caps, stride, padding, dilation = 2, 3, 7, 6, 4, 3, 2, 5, 2, 1, 1
+    A, B, Out = capsule_conv2d(N, C, H, W, K, R, S, caps, stride, padding, dilation)
+    dag = at.compute_dag_from_tensors([Out])
+    main = [op for op in dag.op_lst if op.reduce_axis][0]
+    assert at.get_match_results(dag, "hip")
+    low = lower_main_op(main, dag)
+    c = low.desc
+    assert low.kind == "conv2d" and (c.N, c.C, c.K, c.R, c.S, c.groups) == (N, C, K * caps, R, S, 0)
+    assert (c.stride_h, c.pad_h, c.dil_w) == (stride, padding, dilation) and list(low.gathers) == [1]
+    rng = np.random.default_rng(33)
+    a = rng.integers(-3, 4, (N, C, H, W)).astype(np.float64)
+    b = rng.integers(-3, 4, (K, C, R, S, caps)).astype(np.float64)
+    want = te_interp.evaluate(Out, {"A": a, "B": b})
+    w_kernel = apply_view(low.gathers[1], b)
+    assert w_kernel.shape == (K * caps, C, R, S) and np.array_equal(w_kernel, b.transpose(0, 4, 1, 2, 3).reshape(K * caps, C, R, S))
+    y_kernel = co.lib_conv2d(a.astype(np.int8), w_kernel.astype(np.int8), "int8", stride, padding, dilation).astype(np.float64)
+    got = apply_out_view(low.out_view, y_kernel.reshape(-1))
+    assert got.shape == want.shape and np.array_equal(got, want)
+
