@@ -68,6 +68,14 @@ class GatherDesc(ctypes.Structure):
                 ("in_elems", _i64)]
 
 
+AMOS_ELT_LOAD, AMOS_ELT_CONST, AMOS_ELT_ADD, AMOS_ELT_SUB, AMOS_ELT_MUL = 1, 2, 3, 4, 5
+
+
+class EltwiseDesc(ctypes.Structure):
+    _fields_ = [("dtype", _i32), ("n_inputs", _i32), ("n_ops", _i32), ("reserved", _i32), ("elems", _i64),
+                ("program", _i32 * 16), ("consts", ctypes.c_float * 4)]
+
+
 class ComputeC(ctypes.Structure):
     _fields_ = [("n_tokens", _i32), ("tokens", ctypes.POINTER(_i32)), ("n_iters", _i32),
                 ("iter_kinds", ctypes.POINTER(_i32)), ("iter_extents", ctypes.POINTER(_i64)),
@@ -88,7 +96,7 @@ EXPORTS = [
     "amos_version", "amos_last_error", "amos_device_info", "amos_default_config",
     "amos_check_config", "amos_workspace_bytes", "amos_estimate_seconds", "amos_gemm", "amos_bgemm", "amos_conv2d",
     "amos_conv3d", "amos_run_fused", "amos_time", "amos_time_fused", "amos_gather", "amos_time_gather",
-    "amos_kernel_name", "amos_match", "amos_enumerate_mappings",
+    "amos_eltwise", "amos_time_eltwise", "amos_kernel_name", "amos_match", "amos_enumerate_mappings",
 ]
 
 _lib = None
@@ -128,6 +136,11 @@ def load():
                                     vp, vp, vp, vp, sz, vp, ctypes.c_int, ctypes.c_int, ctypes.c_int,
                                     ctypes.POINTER(ctypes.c_double)]
     lib.amos_gather.argtypes = [ctypes.POINTER(GatherDesc), vp, vp, vp, vp]
+    lib.amos_eltwise.argtypes = [ctypes.POINTER(EltwiseDesc), ctypes.POINTER(vp), vp, vp]
+    lib.amos_eltwise.restype = ctypes.c_int
+    lib.amos_time_eltwise.argtypes = [ctypes.POINTER(EltwiseDesc), ctypes.POINTER(vp), vp, vp, ctypes.c_int,
+                                      ctypes.c_int, ctypes.c_int, ctypes.POINTER(ctypes.c_double)]
+    lib.amos_time_eltwise.restype = ctypes.c_int
     lib.amos_time_gather.argtypes = [ctypes.POINTER(GatherDesc), vp, vp, vp, vp, ctypes.c_int, ctypes.c_int,
                                      ctypes.c_int, ctypes.POINTER(ctypes.c_double)]
     lib.amos_kernel_name.argtypes = [ctypes.c_int, vp, ctypes.POINTER(KernelConfig)]

@@ -33,6 +33,9 @@ class LoweredOp(object):
         self.gathers = {}
         # {0 or 1: numpy array}: inputs[k] is computed from its indices alone; the module holds it
         self.constants = {}
+        # {0 or 1: EltwiseStage}: inputs[k] is not a placeholder but an element-wise function of
+        # placeholders (computed per call by amos_eltwise; a gather may sit on top of it)
+        self.computed = {}
         # OperandView (src None) or None: the kernel writes a tensor of the same size in another
         # order and `output` is gathered from it (a stage behind the main op that no epilogue folds in)
         self.out_view = None
@@ -161,10 +164,66 @@ def _index_tables(indices, variables, extents, src_shape, cond=None):
     return stage, fixed
 
 
-def _operand_view(tensor, head=None):
+class EltwiseStage(object):
+    """tensor = f(placeholders at the same index): `inputs` the placeholders, `program` postfix
+    steps ("load", k) / ("const", value) / "add" / "sub" / "mul" (ops.Eltwise)"""
+
+    def __init__(self, tensor, inputs, program):
+        self.tensor, self.inputs, self.program = tensor, inputs, program
+
+
+def _eltwise_stage(tensor):
+    """EltwiseStage if `tensor` is a compute without reduction whose body is +, -, * over constants
+    and loads of placeholders of its own shape and type at exactly its own indices
+    (benchmark/amos/mapping_variance_tensorcore.py:12-16), else None"""
+    op = tensor.op
+    if not isinstance(op, te.ComputeOp) or op.reduce_axis:
+        return None
+    variables = [iv.var for iv in op.axis]
+    shape = [int(e) for e in tensor.shape]
+    inputs, program = [], []
+
+    def walk(e):
+        if isinstance(e, te.ProducerLoad):
+            t = e.tensor
+            if not isinstance(t.op, te.PlaceholderOp) or t.dtype != tensor.dtype or \
+                    [int(x) for x in t.shape] != shape or len(e.indices) != len(variables) or \
+                    any(i is not v for i, v in zip(e.indices, variables)):
+                return False
+            if all(t is not u for u in inputs):
+                inputs.append(t)
+            program.append(("load", [k for k, u in enumerate(inputs) if u is t][0]))
+            return True
+        if isinstance(e, (te.IntImm, te.FloatImm)):
+            program.append(("const", float(e.value)))
+            return True
+        if isinstance(e, te.Cast) and e.dtype == tensor.dtype:
+            return walk(e.value)
+        if isinstance(e, (te.Add, te.Sub, te.Mul)):
+            if not (walk(e.a) and walk(e.b)):
+                return False
+            program.append({te.Add: "add", te.Sub: "sub", te.Mul: "mul"}[type(e)])
+            return True
+        return False
+
+    if not walk(op.body[0]) or not inputs or len(inputs) > 4 or len(program) > 16 or \
+            sum(1 for p in program if isinstance(p, tuple) and p[0] == "const") > 4:
+        return None
+    # the register stack of the kernel is four deep
+    depth = peak = 0
+    for p in program:
+        depth += 1 if isinstance(p, tuple) else -1
+        peak = max(peak, depth)
+    if peak > 4 or tensor.dtype not in ("float16", "bfloat16", "int8"):
+        return None
+    return EltwiseStage(tensor, inputs, program)
+
+
+def _operand_view(tensor, head=None, computed_source=False):
     """OperandView of `tensor` (a chain of index-remapping stages over a placeholder); `head`:
     an extra outermost stage (shape, variables, indices into `tensor`), e.g. a load with
-    flipped or permuted indices"""
+    flipped or permuted indices.  With `computed_source` the chain may also end at an element-wise
+    function of placeholders (see _eltwise_stage), which then is the view's source."""
     try:
         if head is not None:
             shape, variables, indices = head
@@ -175,6 +234,9 @@ def _operand_view(tensor, head=None):
         cur = tensor
         while not isinstance(cur.op, te.PlaceholderOp):
             op = cur.op
+            if computed_source and _eltwise_stage(cur) is not None and not (
+                    isinstance(op.body[0], te.ProducerLoad) or isinstance(op.body[0], te.Select)):
+                break      # an element-wise function of placeholders: the view's source is computed per call
             if not isinstance(op, te.ComputeOp) or op.reduce_axis:
                 raise _NotSeparable("stage %s reduces" % op.name)
             body, cond = op.body[0], None
@@ -336,7 +398,7 @@ def _lower_gemm(main_op, l0, l1, iters, forms0, forms1):
         return None
     # an operand that is computed: a constant (a function of its indices), or a per-dimension
     # rearrangement of a placeholder that is materialised in front of the kernel
-    sources, gathers, constants = [la.tensor, lb.tensor], {}, {}
+    sources, gathers, constants, computed = [la.tensor, lb.tensor], {}, {}, {}
     for pos, ld in enumerate((la, lb)):
         if isinstance(ld.tensor.op, te.PlaceholderOp):
             continue
@@ -344,8 +406,10 @@ def _lower_gemm(main_op, l0, l1, iters, forms0, forms1):
         if const is not None:
             constants[pos] = const
         else:
-            gathers[pos] = _operand_view(ld.tensor)
+            gathers[pos] = _operand_view(ld.tensor, computed_source=True)
             sources[pos] = gathers[pos].src
+            if not isinstance(sources[pos].op, te.PlaceholderOp):
+                computed[pos] = _eltwise_stage(sources[pos])
     trans_a = 0 if da[0] is x else 1          # [x, k] row-major A, [k, x] transposed
     trans_b = 0 if db[0] is k else 1          # [k, y] row-major B, [y, k] column-major B
     M, N, K = int(x.dom.extent), int(y.dom.extent), int(k.dom.extent)
@@ -363,7 +427,7 @@ def _lower_gemm(main_op, l0, l1, iters, forms0, forms1):
         b.stride_a, b.stride_b, b.stride_c = M * K, K * N, M * N
         attrs["batch"] = b.batch
         low = LoweredOp("bgemm", _lib.AMOS_OP_BGEMM, b, sources, main_op.output(0), attrs)
-    low.gathers, low.constants = gathers, constants
+    low.gathers, low.constants, low.computed = gathers, constants, computed
     return low
 
 

@@ -87,6 +87,19 @@ def evaluate_params_on_device(lowered, params, measure_opt):
             t = g.time(src, ins[pos], number=measure_opt.number, repeat=1, min_repeat_ms=measure_opt.min_repeat_ms)
             lowered._gather_seconds[pos] = t[0]
         extra += lowered._gather_seconds[pos]
+    for pos, stage in getattr(lowered, "computed", {}).items():
+        # an element-wise stage in front of an operand: the same for every configuration, timed once
+        # on arrays of the right size (ins[pos] stands for its result in the kernel's timing)
+        if not hasattr(lowered, "_eltwise_seconds"):
+            lowered._eltwise_seconds = {}
+        if pos not in lowered._eltwise_seconds:
+            src = torch.empty([int(e) for e in stage.tensor.shape], dtype=_TORCH_DTYPE[stage.tensor.dtype],
+                              device=out.device).zero_()
+            e = ops.Eltwise(stage.program, len(stage.inputs), src.dtype, src.numel())
+            lowered._eltwise_seconds[pos] = e.time([src] * len(stage.inputs), torch.empty_like(src),
+                                                   number=measure_opt.number, repeat=1,
+                                                   min_repeat_ms=measure_opt.min_repeat_ms)[0]
+        extra += lowered._eltwise_seconds[pos]
     view = getattr(lowered, "out_view", None)
     if view is not None:   # the result is reordered behind the kernel: the same for every configuration
         if not hasattr(lowered, "_out_gather_seconds"):

@@ -82,9 +82,13 @@ class Module(object):
         # positions of (in0, in1, out[, added tensor of a fused tail]) among the caller's arguments
         ids = [id(t) for t in arg_tensors]
         consts = getattr(lowered, "constants", {})
+        computed = getattr(lowered, "computed", {})
         try:
-            # (an operand computed from its indices alone is held by the module, not passed)
-            self.arg_index = [None if k in consts else ids.index(id(lowered.inputs[k])) for k in (0, 1)]
+            # (an operand computed from its indices alone is held by the module, not passed; one
+            # computed element-wise from placeholders is made per call from those)
+            self.arg_index = [None if (k in consts or k in computed) else ids.index(id(lowered.inputs[k]))
+                              for k in (0, 1)]
+            self._computed_args = {k: [ids.index(id(t)) for t in st.inputs] for k, st in computed.items()}
             self.arg_index.append(ids.index(id(lowered.output)))
             if getattr(lowered, "add_input", None) is not None:
                 self.arg_index.append(ids.index(id(lowered.add_input)))
@@ -94,6 +98,7 @@ class Module(object):
         self._gathers = {}     # operand position -> (ops.Gather, materialised operand), made on first use
         self._constants = {}   # operand position -> device tensor of a constant operand
         self._out_gather = None   # (ops.Gather, the kernel's own output buffer) where the result is reordered
+        self._eltwise = {}        # operand position -> (ops.Eltwise, its result buffer)
 
     def _kernel_inputs(self, in0, in1):
         """the operands the kernel reads: the caller's arrays, or what the stages in front of an
@@ -107,12 +112,30 @@ class Module(object):
             ins[pos] = g(ins[pos].contiguous(), buf)
         return ins
 
+    def _computed_operand(self, k, arrays):
+        """(stage, its input tensors, its result buffer) of an operand that is an element-wise
+        function of the caller's arrays"""
+        stage = self.lowered.computed[k]
+        ins = []
+        for i in self._computed_args[k]:
+            a = arrays[i]
+            ins.append((a.tensor if isinstance(a, NDArray) else a).contiguous())
+        if k not in self._eltwise:
+            e = ops.Eltwise(stage.program, len(ins), ins[0].dtype, ins[0].numel())
+            self._eltwise[k] = (e, torch.empty_like(ins[0]))
+        e, buf = self._eltwise[k]
+        return e, ins, buf
+
     def _pick(self, arrays):
-        need = max(i for i in self.arg_index if i is not None)
+        need = max([i for i in self.arg_index if i is not None] + [i for v in self._computed_args.values() for i in v])
         if len(arrays) <= need:
             raise ValueError("expected %d arrays (inputs + outputs)" % (need + 1))
         out = []
         for k, i in enumerate(self.arg_index):
+            if i is None and k in self._computed_args:
+                e, ins, buf = self._computed_operand(k, arrays)
+                out.append(e(ins, buf))
+                continue
             if i is None:
                 if k not in self._constants:
                     dev = [a for a in arrays if isinstance(a, (NDArray, torch.Tensor))][0]
@@ -156,6 +179,10 @@ class Module(object):
             secs = ops.time_op(self.lowered.op_code, self.lowered.desc, in0, in1, kout, config=cfg,
                                number=number, repeat=repeat, min_repeat_ms=min_repeat_ms,
                                add=picked[3] if len(picked) > 3 else None)
+            for k in self._computed_args:   # element-wise stages in front of an operand run on every call
+                e, ins, buf = self._computed_operand(k, arrays)
+                extra = e.time(ins, buf, number=number, repeat=repeat, min_repeat_ms=min_repeat_ms)
+                secs = [a + b for a, b in zip(secs, extra)]
             if og is not None:   # the reordering of the result runs on every call too
                 extra = og.time(kout, out, number=number, repeat=repeat, min_repeat_ms=min_repeat_ms)
                 secs = [a + b for a, b in zip(secs, extra)]

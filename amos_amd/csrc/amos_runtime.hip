@@ -65,6 +65,61 @@ __global__ __launch_bounds__(256) void amos_gather_kernel(const GatherParams g, 
   }
 }
 
+// out[e] = program(in_0[e], ...): a postfix program on a four-deep register stack; every value is
+// rounded to the element type (fp16 / bf16 round-to-nearest-even, int8 wraps) as soon as it exists
+struct EltwiseParams {
+  const void* in[4];
+  void* out;
+  int64_t elems;
+  int n_ops;
+  int program[16];
+  float consts[4];
+};
+template <int DT> struct EltType { typedef unsigned short raw_t; };
+template <> struct EltType<DT_I8> { typedef signed char raw_t; };
+template <int DT>
+__device__ __forceinline__ float elt_round(float v) {
+  if constexpr (DT == DT_F16) {
+    return (float)(_Float16)v;
+  } else if constexpr (DT == DT_BF16) {
+    unsigned u = __builtin_bit_cast(unsigned, v);
+    if ((u & 0x7f800000u) != 0x7f800000u) u += 0x7fffu + ((u >> 16) & 1u);   // (NaN / Inf keep their bits)
+    return __builtin_bit_cast(float, u & 0xffff0000u);
+  } else {
+    return (float)(signed char)(int)v;      // |v| < 2^17 here: exact in float, wraps like int8
+  }
+}
+template <int DT>
+__device__ __forceinline__ float elt_load(const void* p, int64_t e) {
+  typedef typename EltType<DT>::raw_t raw_t;
+  const raw_t r = ((const raw_t*)p)[e];
+  if constexpr (DT == DT_F16) return (float)__builtin_bit_cast(_Float16, r);
+  else if constexpr (DT == DT_BF16) return __builtin_bit_cast(float, (unsigned)r << 16);
+  else return (float)r;
+}
+template <int DT>
+__global__ __launch_bounds__(256) void amos_eltwise_kernel(const EltwiseParams p) {
+  typedef typename EltType<DT>::raw_t raw_t;
+  for (int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x; e < p.elems; e += (int64_t)gridDim.x * 256) {
+    float s0 = 0, s1 = 0, s2 = 0, s3 = 0;     // s0 = top of the stack
+    for (int k = 0; k < p.n_ops; ++k) {       // (uniform control flow: the program is a kernel argument)
+      const int op = p.program[k] & 255, arg = p.program[k] >> 8;
+      if (op == AMOS_ELT_LOAD || op == AMOS_ELT_CONST) {
+        const float v = op == AMOS_ELT_LOAD ? elt_load<DT>(p.in[arg], e) : elt_round<DT>(p.consts[arg]);
+        s3 = s2; s2 = s1; s1 = s0; s0 = v;
+      } else {
+        const float r = op == AMOS_ELT_ADD ? s1 + s0 : op == AMOS_ELT_SUB ? s1 - s0 : s1 * s0;
+        s0 = elt_round<DT>(r); s1 = s2; s2 = s3;
+      }
+    }
+    raw_t o;
+    if constexpr (DT == DT_F16) o = __builtin_bit_cast(unsigned short, (_Float16)s0);
+    else if constexpr (DT == DT_BF16) o = (unsigned short)(__builtin_bit_cast(unsigned, s0) >> 16);
+    else o = (signed char)(int)s0;
+    ((raw_t*)p.out)[e] = o;
+  }
+}
+
 // dst[b][c][r] = src[b][r][c] for r < rows, c < cols (src rows ld_src apart, dst dense): an
 // operand whose rows are the contiguous direction becomes K-contiguous.  64 x 64 tiles through
 // LDS, 8 bytes per lane on both sides where alignment allows.
@@ -1015,6 +1070,46 @@ static int run_op(int op, const void* desc, const amos_kernel_config_t* cfg, con
 
 using namespace amos;
 
+static int launch_eltwise(const amos_eltwise_desc_t* d, const void* const* inputs, void* out, hipStream_t stream) {
+  if (!d || !inputs || !out) return set_error(AMOS_ERR_BAD_ARG, "null pointer argument");
+  if (d->n_inputs < 1 || d->n_inputs > 4 || d->n_ops < 1 || d->n_ops > 16 || d->elems < 0)
+    return set_error(AMOS_ERR_BAD_ARG, "element-wise stage with %d inputs, %d operations", d->n_inputs, d->n_ops);
+  if (d->dtype != AMOS_F16 && d->dtype != AMOS_BF16 && d->dtype != AMOS_I8)
+    return set_error(AMOS_ERR_UNSUPPORTED, "element-wise stage on dtype %d", d->dtype);
+  EltwiseParams p;
+  memset(&p, 0, sizeof(p));
+  int depth = 0;
+  for (int k = 0; k < d->n_ops; ++k) {     // the program must keep its stack within 1..4 and read what exists
+    const int op = d->program[k] & 255, arg = d->program[k] >> 8;
+    if (op == AMOS_ELT_LOAD || op == AMOS_ELT_CONST) {
+      if (arg < 0 || arg >= (op == AMOS_ELT_LOAD ? d->n_inputs : 4) || ++depth > 4)
+        return set_error(AMOS_ERR_BAD_ARG, "element-wise program: bad operand or stack deeper than 4 at %d", k);
+    } else if (op == AMOS_ELT_ADD || op == AMOS_ELT_SUB || op == AMOS_ELT_MUL) {
+      if (--depth < 1) return set_error(AMOS_ERR_BAD_ARG, "element-wise program: stack underflow at %d", k);
+    } else {
+      return set_error(AMOS_ERR_BAD_ARG, "element-wise program: unknown opcode %d at %d", op, k);
+    }
+    p.program[k] = d->program[k];
+  }
+  if (depth != 1) return set_error(AMOS_ERR_BAD_ARG, "element-wise program leaves %d values", depth);
+  for (int k = 0; k < d->n_inputs; ++k) {
+    if (!inputs[k]) return set_error(AMOS_ERR_BAD_ARG, "element-wise stage: input %d is null", k);
+    p.in[k] = inputs[k];
+  }
+  for (int k = 0; k < 4; ++k) p.consts[k] = d->consts[k];
+  p.out = out;
+  p.elems = d->elems;
+  p.n_ops = d->n_ops;
+  if (d->elems == 0) return 0;
+  const int64_t want = (d->elems + 255) / 256;
+  dim3 grid((unsigned)(want < 65536 ? want : 65536));
+  if (d->dtype == AMOS_F16) hipLaunchKernelGGL(amos_eltwise_kernel<DT_F16>, grid, dim3(256), 0, stream, p);
+  else if (d->dtype == AMOS_BF16) hipLaunchKernelGGL(amos_eltwise_kernel<DT_BF16>, grid, dim3(256), 0, stream, p);
+  else hipLaunchKernelGGL(amos_eltwise_kernel<DT_I8>, grid, dim3(256), 0, stream, p);
+  HIP_TRY(hipGetLastError());
+  return 0;
+}
+
 static int launch_gather(const amos_gather_desc_t* d, const void* in, const int32_t* tables, void* out,
                          hipStream_t stream) {
   if (!d || !in || !tables || !out) return set_error(AMOS_ERR_BAD_ARG, "null pointer argument");
@@ -1218,6 +1313,19 @@ int amos_time_gather(const amos_gather_desc_t* desc, const void* in, const int32
     return set_error(AMOS_ERR_BAD_ARG, "amos_time_gather needs number >= 1, repeat >= 1 and an output array");
   hipStream_t stream = (hipStream_t)stream_v;
   return time_launches([&] { return launch_gather(desc, in, tables, out, stream); }, stream, number, repeat,
+                       min_repeat_ms, out_seconds);
+}
+
+int amos_eltwise(const amos_eltwise_desc_t* desc, const void* const* inputs, void* out, void* stream) {
+  return launch_eltwise(desc, inputs, out, (hipStream_t)stream);
+}
+
+int amos_time_eltwise(const amos_eltwise_desc_t* desc, const void* const* inputs, void* out, void* stream_v,
+                      int number, int repeat, int min_repeat_ms, double* out_seconds) {
+  if (!out_seconds || number < 1 || repeat < 1)
+    return set_error(AMOS_ERR_BAD_ARG, "amos_time_eltwise needs number >= 1, repeat >= 1 and an output array");
+  hipStream_t stream = (hipStream_t)stream_v;
+  return time_launches([&] { return launch_eltwise(desc, inputs, out, stream); }, stream, number, repeat,
                        min_repeat_ms, out_seconds);
 }
 

@@ -291,6 +291,57 @@ class Gather(object):
         return list(res)
 
 
+class Eltwise(object):
+    """device side of an element-wise stage in front of an operand (amos_eltwise): `program` is a
+    list of ("load", k) / ("const", value) / "add" / "sub" / "mul" in postfix order"""
+
+    _DT = {torch.float16: _lib.AMOS_F16, torch.bfloat16: _lib.AMOS_BF16, torch.int8: _lib.AMOS_I8}
+
+    def __init__(self, program, n_inputs, dtype, elems):
+        d = _lib.EltwiseDesc()
+        d.dtype, d.n_inputs, d.elems = self._DT[dtype], int(n_inputs), int(elems)
+        consts = []
+        code = {"add": _lib.AMOS_ELT_ADD, "sub": _lib.AMOS_ELT_SUB, "mul": _lib.AMOS_ELT_MUL}
+        if len(program) > 16:
+            raise ValueError("element-wise stage of %d operations (16 at most)" % len(program))
+        for k, step in enumerate(program):
+            if isinstance(step, tuple) and step[0] == "load":
+                d.program[k] = _lib.AMOS_ELT_LOAD | (int(step[1]) << 8)
+            elif isinstance(step, tuple) and step[0] == "const":
+                if len(consts) == 4:
+                    raise ValueError("element-wise stage with more than four constants")
+                d.program[k] = _lib.AMOS_ELT_CONST | (len(consts) << 8)
+                consts.append(float(step[1]))
+            else:
+                d.program[k] = code[step]
+        d.n_ops = len(program)
+        for k, c in enumerate(consts):
+            d.consts[k] = c
+        self.desc, self.dtype, self.n_inputs = d, dtype, int(n_inputs)
+
+    def _args(self, inputs, out):
+        _need_device(out, *inputs)
+        if len(inputs) != self.n_inputs or any(t.numel() != self.desc.elems or t.dtype != self.dtype or
+                                               not t.is_contiguous() for t in list(inputs) + [out]):
+            raise ValueError("element-wise stage wants %d dense %s tensors of %d elements" %
+                             (self.n_inputs, self.dtype, self.desc.elems))
+        return (ctypes.c_void_p * self.n_inputs)(*[t.data_ptr() for t in inputs])
+
+    def __call__(self, inputs, out=None, stream=None):
+        if out is None:
+            out = torch.empty_like(inputs[0])
+        ptrs = self._args(inputs, out)
+        check(_lib.load().amos_eltwise(ctypes.byref(self.desc), ptrs, out.data_ptr(), _stream_ptr(stream)))
+        return out
+
+    def time(self, inputs, out, number=100, repeat=1, min_repeat_ms=150, stream=None):
+        ptrs = self._args(inputs, out)
+        res = (ctypes.c_double * repeat)()
+        check(_lib.load().amos_time_eltwise(ctypes.byref(self.desc), ptrs, out.data_ptr(), _stream_ptr(stream),
+                                            number, repeat, min_repeat_ms, res))
+        return list(res)
+
+
 def _epilogue_for(op, desc, add, out):
     """Epilogue for an operand laid out like the output the descriptor describes"""
     if add is None:

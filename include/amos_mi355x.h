@@ -257,6 +257,34 @@ int amos_gather(const amos_gather_desc_t* desc, const void* in, const int32_t* t
 int amos_time_gather(const amos_gather_desc_t* desc, const void* in, const int32_t* tables, void* out,
                      void* stream, int number, int repeat, int min_repeat_ms, double* out_seconds);
 
+/* An element-wise stage in front of an operand: out[e] = f(in_0[e], ..., in_{n-1}[e]) for tensors
+ * of one shape and element type, f a short postfix program over +, -, * and constants.  The
+ * reference's default schedule computes such stages at root like any other TE stage (the
+ * squared differences of benchmark/amos/mapping_variance_tensorcore.py:12-16); every operation
+ * rounds to the element type as the compute's own arithmetic does (int8 wraps).
+ *   program[k] = opcode | (argument << 8):  AMOS_ELT_LOAD  pushes in_argument[e],
+ *   AMOS_ELT_CONST pushes consts[argument], AMOS_ELT_ADD / _SUB / _MUL replace the two topmost
+ *   values (below OP top); at most four values on the stack, one left at the end */
+#define AMOS_ELT_LOAD 1
+#define AMOS_ELT_CONST 2
+#define AMOS_ELT_ADD 3
+#define AMOS_ELT_SUB 4
+#define AMOS_ELT_MUL 5
+typedef struct {
+  int32_t dtype;      /* AMOS_F16 / AMOS_BF16 / AMOS_I8: inputs and output */
+  int32_t n_inputs;   /* 1..4 */
+  int32_t n_ops;      /* 1..16 */
+  int32_t reserved;
+  int64_t elems;
+  int32_t program[16];
+  float consts[4];
+} amos_eltwise_desc_t;
+
+int amos_eltwise(const amos_eltwise_desc_t* desc, const void* const* inputs, void* out, void* stream);
+/* amos_time's loop around amos_eltwise */
+int amos_time_eltwise(const amos_eltwise_desc_t* desc, const void* const* inputs, void* out, void* stream,
+                      int number, int repeat, int min_repeat_ms, double* out_seconds);
+
 /* name of the kernel instance a (desc, cfg) pair dispatches to, e.g.
  * "amos_igemm<f16,vec,vec,256x256>"; replaces func.imported_modules[0].get_source()
  * as the way to see what was chosen (reference: README.md:340). */

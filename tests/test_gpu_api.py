@@ -10,7 +10,7 @@ import amos_amd.tvm as tvm
 from amos_amd.tvm import auto_tensorize as at
 from oracle import cpu_oracle as co
 from test_mapper import (batch_conv2d, batched_fc, capsule_conv2d, conv1d, conv2d, conv2d_layout, depthwise_conv2d, from_nkpq, gemm, gemv,
-                         grouped_conv2d, grouped_conv_reference, mean, scan, to_nchw, transposed_conv2d)
+                         grouped_conv2d, grouped_conv_reference, mean, scan, to_nchw, transposed_conv2d, variance)
 
 pytestmark = pytest.mark.gpu
 
@@ -360,4 +360,52 @@ def test_capsule_conv_script_flow(gpu, tmp_path):
     assert np.allclose(arrays[-1].asnumpy(), got, rtol=1e-5, atol=1e-5)
     t = func.time_evaluator(func.entry_name, ctx, number=5, min_repeat_ms=5)(*arrays).mean
     assert 0 < t < 1e-3
+
+
+def test_variance_script_flow(gpu, tmp_path):
+    """reference compute: benchmark/amos/mapping_variance_tensorcore.py:7-31 (squared differences
+    computed element-wise in front of the mean's GEMM)"""
+    N, C, H, W = 8, 96, 14, 14
+    A, Mean, E = variance(N, C, H, W)
+    rng = np.random.default_rng(14)
+    a = rng.uniform(-1, 1, (N, C, H, W)).astype(np.float16)
+    m = rng.uniform(-0.2, 0.2, (N, C, H, W)).astype(np.float16)
+    got, result = _run_script_flow([A, Mean, E], {"A": a, "Mean": m}, tmp_path, "variance", transform_strict=False)
+    low = result.sch_app.lowered
+    assert low.kind == "gemm" and list(low.computed) == [0]
+    # as the compute's own fp16 arithmetic rounds: difference, then square, both to fp16
+    diff = (a - m).astype(np.float16)
+    sq = (diff * diff).astype(np.float16).astype(np.float64)
+    ref = sq.transpose(1, 0, 2, 3).reshape(C, -1).sum(axis=1) * float(np.float16(1.0 / (N * H * W)))
+    assert got.shape == (C,) and np.allclose(got, ref, rtol=2e-3, atol=1e-4)
+
+
+@pytest.mark.parametrize("dtype", ["float16", "bfloat16", "int8"])
+def test_eltwise_entry_point(gpu, dtype):
+    """amos_eltwise: every operation rounds to the element type (int8 wraps)"""
+    import torch
+    from amos_amd import ops
+    rng = np.random.default_rng(15)
+    n = 100003
+    if dtype == "int8":
+        x = rng.integers(-128, 128, n).astype(np.int8)
+        y = rng.integers(-128, 128, n).astype(np.int8)
+        tx, ty = torch.from_numpy(x).cuda(), torch.from_numpy(y).cuda()
+        d = (x - y).astype(np.int8)                     # numpy wraps like the compute's int8 arithmetic
+        want = ((d * d).astype(np.int8) + np.int8(3)).astype(np.int8)
+    else:
+        tdt = torch.float16 if dtype == "float16" else torch.bfloat16
+        tx = torch.from_numpy(rng.uniform(-4, 4, n).astype(np.float32)).cuda().to(tdt)
+        ty = torch.from_numpy(rng.uniform(-4, 4, n).astype(np.float32)).cuda().to(tdt)
+        d = (tx.float() - ty.float()).to(tdt)
+        want = ((d.float() * d.float()).to(tdt).float() + 3.0).to(tdt)
+    prog = [("load", 0), ("load", 1), "sub", ("load", 0), ("load", 1), "sub", "mul", ("const", 3.0), "add"]
+    e = ops.Eltwise(prog, 2, tx.dtype, n)
+    got = e([tx, ty])
+    if dtype == "int8":
+        assert np.array_equal(got.cpu().numpy(), want)
+    else:
+        assert torch.equal(got, want)
+    with pytest.raises(Exception, match="stack|program"):
+        ops.Eltwise(["add"], 1, tx.dtype, n)([tx])
 

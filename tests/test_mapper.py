@@ -877,3 +877,48 @@ def test_capsule_conv_lowering():
     got = apply_out_view(low.out_view, y_kernel.reshape(-1))
     assert got.shape == want.shape and np.array_equal(got, want)
 
+
+def variance(N, C, H, W, in_dtype="float16", out_dtype="float32"):
+    """reference: benchmark/amos/mapping_variance_tensorcore.py:7-31"""
+    A = te.placeholder([N, C, H, W], dtype=in_dtype, name="A")
+    Mean = te.placeholder([N, C, H, W], dtype=in_dtype, name="Mean")
+    Diff = te.compute([N, C, H, W], lambda n, c, h, w: (A[n, c, h, w] - Mean[n, c, h, w]) * (A[n, c, h, w] - Mean[n, c, h, w]),
+                      name="Diff")
+    B = te.compute([C, N * H * W], lambda i, j: Diff[j // (H * W), i, j % (H * W) // W, j % W], name="B")
+    C_ = te.compute([N * H * W, 1], lambda i, j: tir.const(1.0 / (N * H * W), in_dtype), name="C")
+    rk = te.reduce_axis([0, N * H * W], name="k")
+    D = te.compute([C, 1], lambda i, j: te.sum((B[i, rk] * C_[rk, j]).astype(out_dtype), axis=rk), name="D")
+    E = te.compute([C], lambda i: D[i, 0], name="E")
+    return A, Mean, E
+
+
+def test_variance_lowering():
+    """squared differences in front of the mean's GEMM: an element-wise stage (computed per call),
+    a gather on top of it, a constant second operand; checked against the compute as written"""
+    from amos_amd.auto_tensorize.lowering import lower_main_op
+    N, C, H, W = 2, 5, 3, 4
+    A, Mean, E = variance(N, C, H, W)
+    dag = at.compute_dag_from_tensors([E])
+    main = [op for op in dag.op_lst if op.reduce_axis][0]
+    assert at.get_match_results(dag, "hip")
+    low = lower_main_op(main, dag)
+    assert low.kind == "gemm" and list(low.computed) == [0] and list(low.gathers) == [0] and list(low.constants) == [1]
+    stage = low.computed[0]
+    assert [t.name for t in stage.inputs] == ["A", "Mean"]
+    assert stage.program == [("load", 0), ("load", 1), "sub", ("load", 0), ("load", 1), "sub", "mul"]
+    rng = np.random.default_rng(41)
+    a = rng.integers(-3, 4, (N, C, H, W)).astype(np.float64)
+    m = rng.integers(-2, 3, (N, C, H, W)).astype(np.float64)
+    want = te_interp.evaluate(E, {"A": a, "Mean": m})
+    # the program on numpy arrays, then the gather, then the product with the constant
+    stack = []
+    for step in stage.program:
+        if isinstance(step, tuple):
+            stack.append((a, m)[step[1]] if step[0] == "load" else step[1])
+        else:
+            y, x = stack.pop(), stack.pop()
+            stack.append({"add": x + y, "sub": x - y, "mul": x * y}[step])
+    lhs = apply_view(low.gathers[0], stack[0])
+    got = (lhs @ low.constants[1].astype(np.float64)).reshape(-1)
+    assert lhs.shape == (C, N * H * W) and np.allclose(got, want, rtol=1e-3)
+
