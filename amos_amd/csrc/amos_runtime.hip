@@ -413,26 +413,9 @@ static int plan_gemm_repacked(Plan& pl, int op, const amos_gemm_desc_t* d, const
     e.g.trans_b = 1; e.g.ldb = rp.Kp; e.stride_b = d->N * rp.Kp;
   }
   const bool batched = batch > 1 || op == AMOS_OP_BGEMM;
-  // the copies are made for the direct-to-LDS kernel: without a tile from the caller, take the
-  // best of its tiles by the mapper's model
-  amos_kernel_config_t direct;
-  if (!cfg || cfg->tile_i <= 0 || cfg->tile_j <= 0) {
-    static const int tiles[4][2] = {{256, 256}, {128, 128}, {128, 256}, {256, 128}};
-    double best = 1e30;
-    memset(&direct, 0, sizeof(direct));
-    for (auto& t : tiles) {
-      amos_kernel_config_t c2;
-      memset(&c2, 0, sizeof(c2));
-      c2.tile_i = t[0]; c2.tile_j = t[1]; c2.split_k = 1; c2.pipeline = AMOS_PIPE_DIRECT8;
-      double sec = 0.0;
-      if (amos_estimate_seconds(batched ? AMOS_OP_BGEMM : AMOS_OP_GEMM,
-                                batched ? (const void*)&e : (const void*)&e.g, &c2, &sec) == 0 && sec < best) {
-        best = sec;
-        direct = c2;
-      }
-    }
-    if (best < 1e30) cfg = &direct;
-  }
+  // without a tile from the caller: the mapper's choice for the product on the copies (the same
+  // one amos_default_config makes for the original problem, whose estimate differs by the copies'
+  // constant time)
   int rc = plan_gemm(pl, batched ? AMOS_OP_BGEMM : AMOS_OP_GEMM, batched ? (const void*)&e : (const void*)&e.g,
                      &e.g, batch, e.stride_a, e.stride_b, e.stride_c, cfg, A2, B2, C);
   if (rc) return rc;

@@ -593,14 +593,17 @@ static double estimate_seconds(const Problem& pb, int ti, int tj, int split, boo
   double step_us = (double)groups * std::max(alone, tc->occ * tau);
   if (rest) step_us += std::max(alone, (double)rest * tau);
   const double rounds = (double)groups + (rest ? 1.0 : 0.0);
-  double t = 3e-6 + (ksteps * step_us + rounds * tc->fixed_us) * 1e-6 + (repacked ? pb.repack_seconds : 0.0);
+  double t = 3e-6 + (ksteps * step_us + rounds * tc->fixed_us) * 1e-6;
   // output: written once; a split-K launch zero-fills it and accumulates with atomics (measured:
   // (1 + 2*split) passes over the output at ~3.5 TB/s)
   if (eff_split > 1) t += (double)pb.out_bytes * (1.0 + 2.0 * eff_split) / 3.5e12;
   // memory floor; the shorter of the two legs is not hidden completely, which also orders
   // memory-bound candidates by their compute time
-  const double t_hbm = ((double)pb.in_bytes + (double)pb.out_bytes) / (0.7 * Gfx950::kHbmBytesPerSec) + 3e-6;
-  return std::max(t, t_hbm) + 0.1 * std::min(t, t_hbm);
+  // (on copies the kernel reads the padded operands; the copies' own time is the same for every
+  // configuration and stays outside the comparison of the two legs)
+  const double in_bytes = repacked ? (double)pb.batch * (double)(pb.I + pb.J) * (double)pb.Kp * es : (double)pb.in_bytes;
+  const double t_hbm = (in_bytes + (double)pb.out_bytes) / (0.7 * Gfx950::kHbmBytesPerSec) + 3e-6;
+  return std::max(t, t_hbm) + 0.1 * std::min(t, t_hbm) + (repacked ? pb.repack_seconds : 0.0);
 }
 
 int conv_unroll_level(int flags) {
@@ -738,24 +741,12 @@ int amos_default_config(int op, const void* desc, amos_kernel_config_t* result) 
   amos_bgemm_desc_t as_gemm;
   if ((op == AMOS_OP_CONV2D || op == AMOS_OP_CONV3D) && conv_as_gemm(*(const amos_conv_desc_t*)desc, op, &as_gemm))
     return amos_default_config(AMOS_OP_BGEMM, &as_gemm, result);
-  // ... a strided one after its pixels are picked by the operand copy: the best direct tile
+  // ... a strided one, or one on few channels, after a copy of its activations: the product on
+  // the copies
   Problem pg;
-  if ((op == AMOS_OP_CONV2D || op == AMOS_OP_CONV3D) &&
-      conv_copied_gemm_problem(*(const amos_conv_desc_t*)desc, op, &pg)) {
-    memset(result, 0, sizeof(*result));
-    result->pipeline = AMOS_PIPE_AUTO;
-    double best_direct = 1e30;
-    for (auto& t : kRepackTiles) {
-      const double s = estimate_seconds(pg, t[0], t[1], 1);
-      if (s < best_direct) {
-        best_direct = s;
-        result->tile_i = t[0];
-        result->tile_j = t[1];
-        result->split_k = 1;
-      }
-    }
-    return 0;
-  }
+  const bool copied = (op == AMOS_OP_CONV2D || op == AMOS_OP_CONV3D) &&
+                      conv_copied_gemm_problem(*(const amos_conv_desc_t*)desc, op, &pg);
+  if (copied) { pb = pg; op = AMOS_OP_BGEMM; }
   memset(result, 0, sizeof(*result));
   amos_kernel_config_t* out = result;
   const double es = pb.in_dtype == AMOS_I8 ? 1.0 : 2.0;
@@ -798,20 +789,6 @@ int amos_default_config(int op, const void* desc, amos_kernel_config_t* result) 
     }
   }
   *result = staged;
-  // operands that get copied for the direct-to-LDS kernel: the best of its tiles, as a launch
-  // without a config takes it
-  if (pb.repack && result->pipeline == AMOS_PIPE_AUTO) {
-    double best_direct = 1e30;
-    for (auto& t : kRepackTiles) {
-      const double s = estimate_seconds(pb, t[0], t[1], 1);
-      if (s < best_direct) {
-        best_direct = s;
-        result->tile_i = t[0];
-        result->tile_j = t[1];
-        result->split_k = 1;
-      }
-    }
-  }
   return 0;
 }
 
