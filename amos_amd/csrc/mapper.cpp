@@ -535,9 +535,6 @@ static const TileCost kDirectCost[] = {
     {256, 256, 1, 1.85, 1.65, 4.0}, {128, 256, 1, 1.06, 0.95, 2.0}, {256, 128, 1, 1.05, 0.92, 2.0},
     {128, 128, 2, 0.56, 0.70, 1.0}};
 
-// the direct kernel's tiles in the order plan_gemm_repacked() tries them
-static const int kRepackTiles[4][2] = {{256, 256}, {128, 128}, {128, 256}, {256, 128}};
-
 // A convolution that runs as a batched matrix product on a copy of its activations (every
 // stride-th pixel of a 1x1 window, or an im2col matrix for few channels): that product, with
 // the copy's time, as the mapper's problem.
