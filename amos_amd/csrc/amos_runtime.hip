@@ -15,6 +15,7 @@
 #include "gemm_tn_kernel.h"
 #include "igemm_instances.h"
 #include "mapper.h"
+#include "skinny_gemm_kernel.h"
 
 namespace amos {
 
@@ -319,6 +320,10 @@ struct Plan {
   // im2col copy of a convolution's activations in front of the GEMM (0 = not used)
   int im2col;
   Im2colParams icp;
+  // GEMM with at most 16 rows on one side, on the vector ALUs (0 = not used)
+  int skinny;
+  int skinny_big_is_a;
+  SkinnyParams sk;
   // convolution on few input channels (0 = not used)
   int fewc;
   ConvFewcParams fcp;
@@ -429,6 +434,9 @@ static int plan_gemm(Plan& pl, int op, const void* desc_any, const amos_gemm_des
                      const amos_kernel_config_t* cfg, const void* A, const void* B, void* C,
                      void* workspace, size_t ws_bytes) {
   if (!d || !A || !B || !C) return set_error(AMOS_ERR_BAD_ARG, "null pointer argument");
+  // (a one-column row-major B or a one-row transposed A is K-contiguous memory: say so)
+  const amos_gemm_desc_t norm = batch == 1 ? gemm_normalized(*d) : *d;
+  d = &norm;
   pl.n_transposes = 0;
   if (workspace && (!cfg || cfg->pipeline != AMOS_PIPE_STAGED) && ((uintptr_t)workspace & 255) == 0 &&
       fits_int(d->M) && fits_int(d->N) && fits_int(d->K) && d->K < (1 << 30) &&
@@ -507,6 +515,27 @@ static int plan_gemm(Plan& pl, int op, const void* desc_any, const amos_gemm_des
     pl.tn_waves = waves;
   } else if (pipe == AMOS_PIPE_AUTO && tn_ok && pick_gemm_tn(pl.dt, pl.cfg.tile_i, pl.cfg.tile_j, 8)) {
     pl.tn_waves = 8;  // measured a few percent ahead of 4 waves on the 8192^3 fp16 GEMM
+  }
+  // One side of a few rows: a byte mover on the vector ALUs, under the mapper's own pipeline
+  if (pipe == AMOS_PIPE_AUTO && gemm_is_skinny(*d, batch) && pl.rl == LD_VEC && pl.cl == LD_VEC) {
+    pl.tn_waves = 0;
+    pl.skinny = 1;
+    pl.skinny_big_is_a = d->N <= kSkinnyMaxRows && (d->M > kSkinnyMaxRows || d->N <= d->M);
+    SkinnyParams& q = pl.sk;
+    memset(&q, 0, sizeof(q));
+    q.out = (char*)C;
+    q.K = (int)d->K;
+    if (pl.skinny_big_is_a) {
+      q.big = (const char*)A; q.small = (const char*)B;
+      q.NB = (int)d->M; q.MS = (int)d->N; q.ld_big = d->lda; q.ld_small = d->ldb;
+      q.out_s_big = d->ldc; q.out_s_small = 1;
+    } else {
+      q.big = (const char*)B; q.small = (const char*)A;
+      q.NB = (int)d->N; q.MS = (int)d->M; q.ld_big = d->ldb; q.ld_small = d->lda;
+      q.out_s_big = 1; q.out_s_small = d->ldc;
+    }
+    pl.split = 1;
+    return 0;
   }
   if (pl.tn_waves) {
     GemmTnParams& q = pl.tn;
@@ -860,6 +889,7 @@ static int make_plan(Plan& pl, int op, const void* desc, const amos_kernel_confi
   pl.dw = 0;
   pl.im2col = 0;
   pl.fewc = 0;
+  pl.skinny = 0;
   switch (op) {
     case AMOS_OP_GEMM:
       return plan_gemm(pl, op, desc, (const amos_gemm_desc_t*)desc, 1, 0, 0, 0, cfg, in0, in1, out, workspace,
@@ -968,6 +998,10 @@ static int launch(const Plan& pl, hipStream_t stream) {
     HIP_TRY(launch_conv_fewc(pl.dt, pl.fcp, pl.fewc_lds, stream));
     return 0;
   }
+  if (pl.skinny) {
+    HIP_TRY(launch_skinny_gemm(pl.dt, pl.sk, stream));
+    return 0;
+  }
   if (pl.dw) {
     launch_depthwise(pl.dt, pl.dw - 1, pl.dwp, stream);
     HIP_TRY(hipGetLastError());
@@ -1035,6 +1069,9 @@ static int plan_epilogue(Plan& pl, int op, const void* desc, const amos_epilogue
   pl.cv.epi = ep;
   pl.dwp.epi = ep;
   pl.fcp.epi = ep;
+  pl.sk.epi = ep;
+  pl.sk.epi_s_big = pl.skinny_big_is_a ? ep.si : 1;
+  pl.sk.epi_s_small = pl.skinny_big_is_a ? 1 : ep.si;
   return 0;
 }
 
@@ -1272,6 +1309,7 @@ const char* amos_kernel_name(int op, const void* desc, const amos_kernel_config_
   if (make_plan(pl, op, desc, cfg, dummy, dummy, dummy, dummy_ws, (size_t)-1)) return nullptr;
   if (pl.dw) return depthwise_name(pl.dt, pl.dw - 1);
   if (pl.fewc) return conv_fewc_name(pl.dt);
+  if (pl.skinny) return skinny_gemm_name(pl.dt);
   if (pl.conv_ups) {
     ConvInstance* ci = pick_conv(pl.dt, pl.cfg.tile_i, pl.cfg.tile_j, pl.conv_waves, pl.cv.pls, pl.conv_occ, pl.conv_w9);
     return ci ? ci->name : nullptr;

@@ -45,6 +45,26 @@ GemmRepack gemm_repack(const amos_gemm_desc_t& g, int64_t batch, bool a_unaligne
 }
 
 
+amos_gemm_desc_t gemm_normalized(const amos_gemm_desc_t& gin) {
+  amos_gemm_desc_t g = gin;
+  if (g.N == 1 && !g.trans_b && g.ldb == 1) { g.trans_b = 1; g.ldb = g.K; }
+  if (g.M == 1 && g.trans_a && g.lda == 1) { g.trans_a = 0; g.lda = g.K; }
+  return g;
+}
+
+bool gemm_is_skinny(const amos_gemm_desc_t& gin, int64_t batch) {
+  const amos_gemm_desc_t g = gemm_normalized(gin);
+  const int es = g.in_dtype == AMOS_I8 ? 1 : 2;
+  const int ce = 16 / es;
+  if (batch != 1 || g.trans_a || !g.trans_b || g.M <= 0 || g.N <= 0 || g.K <= 0) return false;
+  if (g.K % ce || g.lda % ce || g.ldb % ce || g.K >= (1 << 30) || g.M >= (1ll << 31) || g.N >= (1ll << 31)) return false;
+  const int64_t small = std::min(g.M, g.N);
+  if (small > kSkinnyMaxRows) return false;
+  int msp = 1;
+  while (msp < small) msp <<= 1;
+  return (int64_t)msp * g.K * es <= kSkinnyMaxLds;
+}
+
 bool conv_subsample_pipeline(int pipeline) {
   return pipeline == AMOS_PIPE_AUTO || pipeline == AMOS_PIPE_DIRECT4 || pipeline == AMOS_PIPE_DIRECT8;
 }
@@ -224,6 +244,8 @@ int problem_of(int op, const void* desc, Problem* out) {
       }
       if (g->M <= 0 || g->N <= 0 || g->K <= 0 || batch <= 0)
         return set_error(AMOS_ERR_BAD_ARG, "non-positive GEMM extent");
+      const amos_gemm_desc_t norm = gemm_normalized(*g);
+      if (batch == 1) g = &norm;
       out->I = g->M; out->J = g->N; out->K = g->K; out->batch = batch;
       out->in_dtype = g->in_dtype;
       {
@@ -683,6 +705,13 @@ int amos_estimate_seconds(int op, const void* desc, const amos_kernel_config_t* 
     *seconds = ((double)pb.in_bytes + (double)pb.out_bytes) / (0.35 * Gfx950::kHbmBytesPerSec) + 3e-6;
     return 0;
   }
+  if ((op == AMOS_OP_GEMM || op == AMOS_OP_BGEMM) && cfg->pipeline == AMOS_PIPE_AUTO &&
+      gemm_is_skinny(op == AMOS_OP_GEMM ? *(const amos_gemm_desc_t*)desc : ((const amos_bgemm_desc_t*)desc)->g,
+                     op == AMOS_OP_GEMM ? 1 : ((const amos_bgemm_desc_t*)desc)->batch)) {
+    // one pass over the operands at about half the HBM rate, plus a launch
+    *seconds = ((double)pb.in_bytes + (double)pb.out_bytes) / (0.5 * Gfx950::kHbmBytesPerSec) + 3.5e-6;
+    return 0;
+  }
   ConvFewcPlan fp;
   if ((op == AMOS_OP_CONV2D || op == AMOS_OP_CONV3D) && cfg->pipeline == AMOS_PIPE_AUTO &&
       conv_fewc_plan(*(const amos_conv_desc_t*)desc, op, &fp)) {
@@ -722,6 +751,14 @@ int amos_default_config(int op, const void* desc, amos_kernel_config_t* result) 
   int rc = problem_of(op, desc, &pb);
   if (rc) return rc;
   if (!result) return set_error(AMOS_ERR_BAD_ARG, "null config");
+  // so does a GEMM with one skinny side
+  if ((op == AMOS_OP_GEMM || op == AMOS_OP_BGEMM) &&
+      gemm_is_skinny(op == AMOS_OP_GEMM ? *(const amos_gemm_desc_t*)desc : ((const amos_bgemm_desc_t*)desc)->g,
+                     op == AMOS_OP_GEMM ? 1 : ((const amos_bgemm_desc_t*)desc)->batch)) {
+    memset(result, 0, sizeof(*result));
+    result->tile_i = 64; result->tile_j = 64; result->split_k = 1; result->pipeline = AMOS_PIPE_AUTO;
+    return 0;
+  }
   // a depthwise convolution runs on the vector ALUs, whatever the tile
   if ((op == AMOS_OP_CONV2D || op == AMOS_OP_CONV3D) && conv_is_depthwise(*(const amos_conv_desc_t*)desc)) {
     memset(result, 0, sizeof(*result));

@@ -93,6 +93,19 @@ struct ConvFewcPlan {
   int64_t bytes_x, bytes_w;    // workspace: pixel-major activations, then the packed weights
 };
 bool conv_fewc_plan(const amos_conv_desc_t& c, int op, ConvFewcPlan* out);
+// A single GEMM with at most 8 rows on one side, both operands K-contiguous in whole 16-byte
+// chunks, the skinny side (rows rounded up to a power of two) within 16 KB of LDS: runs on the
+// vector ALUs (skinny_gemm_kernel.h) unless a matrix-core pipeline is named.  The limits are where
+// it stopped winning against the split-K matrix-core kernel when timed: every row of the skinny
+// side costs a pass of LDS reads and packed dot products over the big operand's chunk (at 16
+// rows that rate is below the matrix cores'), and past 16 KB too few workgroups fit on a CU to
+// hide the loads' latency.
+constexpr int kSkinnyMaxRows = 8;
+constexpr int64_t kSkinnyMaxLds = 16 * 1024;
+bool gemm_is_skinny(const amos_gemm_desc_t& g, int64_t batch);
+// a one-column row-major B ([K][1], ldb 1) is the same memory as a one-row column-major one
+// ([1][K]); likewise a one-row transposed A: the descriptor with those spelled K-contiguous
+amos_gemm_desc_t gemm_normalized(const amos_gemm_desc_t& g);
 // groups == input channels (NCDHW): runs on the vector ALUs unless a matrix-core pipeline is named
 bool conv_is_depthwise(const amos_conv_desc_t& c);
 

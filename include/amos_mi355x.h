@@ -151,7 +151,9 @@ typedef struct {
 
 /* how tiles travel from HBM to the MFMA operands */
 #define AMOS_PIPE_AUTO 0      /* the mapper's choice; a depthwise convolution (groups == C,  */
-                              /* NCDHW) runs on the vector-ALU kernel under this value only   */
+                              /* NCDHW) and a GEMM with at most 8 rows on one side (K-       */
+                              /* contiguous operands, that side within 16 KB) run on the     */
+                              /* vector-ALU kernels under this value only                    */
 #define AMOS_PIPE_STAGED 1    /* global -> registers -> LDS, any layout, ragged K             */
 #define AMOS_PIPE_DIRECT4 2   /* global -> LDS direct copies, 256x256 tile, 4 waves           */
 #define AMOS_PIPE_DIRECT8 3   /* same with 8 waves (two per SIMD)                             */

@@ -100,8 +100,11 @@ def test_gemm_direct_pipeline(gpu, dtype, pipeline, tile, shape):
     b = make_operand(rng, (N, K), dtype)
     cfg = dict(tile_i=tile[0], tile_j=tile[1], split_k=1, pipeline=pipeline)
     d = ops.gemm_desc(M, N, K, to_device(a, dtype).dtype, False, True)
-    assert "amos_gemm_tn<%s,%dx%d" % ({"float16": "f16", "bfloat16": "bf16", "int8": "i8"}[dtype], tile[0], tile[1]) \
-        in ops.kernel_name(_lib.AMOS_OP_GEMM, d, cfg)
+    name = ops.kernel_name(_lib.AMOS_OP_GEMM, d, cfg)
+    if pipeline == 0 and M == 1:     # one row under the mapper's own pipeline: the vector-ALU kernel
+        assert name.startswith("amos_skinny_gemm<")
+    else:
+        assert "amos_gemm_tn<%s,%dx%d" % ({"float16": "f16", "bfloat16": "bf16", "int8": "i8"}[dtype], tile[0], tile[1]) in name
     got = ops.gemm(to_device(a, dtype), to_device(b, dtype), False, True, config=cfg).cpu().numpy()
     check(got, co.lib_gemm(a, b, dtype, False, True, acc="float64"), dtype,
           "direct gemm %s pipe %d tile %s %s" % (dtype, pipeline, tile, shape))
@@ -219,6 +222,63 @@ def test_gemm_ragged_k_through_padded_copies(gpu, dtype, trans, K):
     staged = ops.gemm(da, db, bool(ta), bool(tb), config=dict(tile_i=64, tile_j=64, split_k=1,
                                                               pipeline=_lib.AMOS_PIPE_STAGED))
     check(staged.cpu().numpy(), ref, dtype, "staged gemm %s %s K=%d" % (dtype, trans, K))
+
+
+SKINNY_CASES = [
+    # M, N, K, trans_a, trans_b
+    (1, 1000, 2048, 0, 1), (8, 1031, 1000, 0, 1), (5, 333, 1000, 0, 1), (3000, 1, 520, 0, 0), (777, 8, 264, 0, 1),
+    (7, 7, 72, 0, 1), (1, 4099, 8192, 0, 1), (2050, 3, 16, 0, 1),
+]
+
+
+@pytest.mark.parametrize("dtype", ["float16", "bfloat16", "int8"])
+@pytest.mark.parametrize("case", SKINNY_CASES)
+def test_gemm_skinny(gpu, dtype, case):
+    """GEMV and dense layers on a small batch (at most 8 rows on one side within 16 KB, K-contiguous
+    operands) on the vector-ALU kernel: against the oracle, bit for bit in int8 against the register-staged
+    kernel, with the fused addition"""
+    import torch
+    from amos_amd import _lib, ops
+    M, N, K, ta, tb = case
+    if dtype == "int8" and K % 16:
+        K += 16 - K % 16           # whole 16-byte chunks of int8
+    rng = np.random.default_rng(hash(case) % 2**32)
+    a = make_operand(rng, (K, M) if ta else (M, K), dtype)
+    b = make_operand(rng, (N, K) if tb else (K, N), dtype)
+    da, db = to_device(a, dtype), to_device(b, dtype)
+    d = ops.gemm_desc(M, N, K, da.dtype, ta, tb)
+    assert ops.kernel_name(_lib.AMOS_OP_GEMM, d, None).startswith("amos_skinny_gemm<")
+    cfg = ops.default_config(_lib.AMOS_OP_GEMM, d)
+    assert ops.kernel_name(_lib.AMOS_OP_GEMM, d, cfg).startswith("amos_skinny_gemm<")
+    ref = co.lib_gemm(a, b, dtype, bool(ta), bool(tb), acc="float64")
+    got = ops.gemm(da, db, bool(ta), bool(tb)).cpu().numpy()
+    check(got, ref, dtype, "skinny gemm %s %s" % (dtype, case))
+    staged = dict(tile_i=64, tile_j=64, split_k=1, pipeline=_lib.AMOS_PIPE_STAGED)
+    assert ops.kernel_name(_lib.AMOS_OP_GEMM, d, staged).startswith("amos_igemm<")
+    other = ops.gemm(da, db, bool(ta), bool(tb), config=staged).cpu().numpy()
+    if dtype == "int8":
+        assert np.array_equal(got, other)
+    d_host = rng.integers(-1000, 1000, got.shape).astype(got.dtype)
+    with_d = ops.gemm(da, db, bool(ta), bool(tb), add=torch.from_numpy(d_host).cuda()).cpu().numpy()
+    want = (ref.astype(np.int64) + d_host).astype(np.int32) if dtype == "int8" else ref + d_host
+    check(with_d, want, dtype, "skinny gemm + D %s %s" % (dtype, case))
+
+
+def test_gemm_skinny_limits(gpu):
+    """past the limits of the vector-ALU kernel (rows, LDS bytes, K-contiguous operands, a single
+    GEMM) the matrix-core kernels run, with the same results"""
+    import torch
+    from amos_amd import _lib, ops
+    rng = np.random.default_rng(5)
+    for (M, N, K, ta, tb) in ((9, 500, 512, 0, 1), (4, 500, 4096, 0, 1), (4, 504, 512, 0, 0), (4, 500, 516, 0, 1)):
+        a = make_operand(rng, (K, M) if ta else (M, K), "float16")
+        b = make_operand(rng, (N, K) if tb else (K, N), "float16")
+        d = ops.gemm_desc(M, N, K, torch.float16, ta, tb)
+        assert ops.kernel_name(_lib.AMOS_OP_GEMM, d, None).startswith("amos_igemm<"), (M, N, K)
+        got = ops.gemm(to_device(a, "float16"), to_device(b, "float16"), bool(ta), bool(tb)).cpu().numpy()
+        check(got, co.lib_gemm(a, b, "float16", bool(ta), bool(tb), acc="float64"), "float16", "gemm %s" % ((M, N, K),))
+    bd = ops.bgemm_desc(3, 4, 500, 512, torch.float16, False, True)
+    assert not ops.kernel_name(_lib.AMOS_OP_BGEMM, bd, None).startswith("amos_skinny")
 
 
 def test_gemm_direct_pipeline_rejects_ragged_k(gpu):
