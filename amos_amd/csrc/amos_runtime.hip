@@ -505,13 +505,19 @@ static int plan_gemm(Plan& pl, int op, const void* desc_any, const amos_gemm_des
                      256 * d->lda * es + 128 < ((int64_t)1 << 32) &&
                      256 * d->ldb * es + 128 < ((int64_t)1 << 32);
   const int pipe = pl.cfg.pipeline;
-  if (pipe == AMOS_PIPE_DIRECT4 || pipe == AMOS_PIPE_DIRECT8) {
-    const int waves = pipe == AMOS_PIPE_DIRECT4 ? 4 : 8;
+  // The four-wave instance of the direct-to-LDS kernel is withdrawn: its 128x128 wave tile made the
+  // compiler spill over a kilobyte of registers per lane, it measured behind the eight-wave one at
+  // every size, and a launch of it at 8192^3 ended in a memory fault whose cause is not found.
+  if (pipe == AMOS_PIPE_DIRECT4)
+    return set_error(AMOS_ERR_INFEASIBLE, "AMOS_PIPE_DIRECT4 is withdrawn (the four-wave direct-to-LDS instance "
+                     "spilled registers and was slower than AMOS_PIPE_DIRECT8 everywhere): use AMOS_PIPE_DIRECT8 "
+                     "or AMOS_PIPE_AUTO");
+  if (pipe == AMOS_PIPE_DIRECT8) {
+    const int waves = 8;
     if (!tn_ok || !pick_gemm_tn(pl.dt, pl.cfg.tile_i, pl.cfg.tile_j, waves))
       return set_error(AMOS_ERR_INFEASIBLE,
                        "direct-to-LDS pipeline needs K-contiguous 16-byte aligned operands, "
-                       "K %% %d == 0, split_k 1 and a tile of 256x256 (4 or 8 waves), 128x128, "
-                       "128x256 or 256x128 (8 waves)", bke);
+                       "K %% %d == 0, split_k 1 and a tile of 256x256, 128x128, 128x256 or 256x128", bke);
     pl.tn_waves = waves;
   } else if (pipe == AMOS_PIPE_AUTO && tn_ok && pick_gemm_tn(pl.dt, pl.cfg.tile_i, pl.cfg.tile_j, 8)) {
     pl.tn_waves = 8;  // measured a few percent ahead of 4 waves on the 8192^3 fp16 GEMM

@@ -155,7 +155,8 @@ typedef struct {
                               /* contiguous operands, that side within 16 KB) run on the     */
                               /* vector-ALU kernels under this value only                    */
 #define AMOS_PIPE_STAGED 1    /* global -> registers -> LDS, any layout, ragged K             */
-#define AMOS_PIPE_DIRECT4 2   /* global -> LDS direct copies, 256x256 tile, 4 waves           */
+#define AMOS_PIPE_DIRECT4 2   /* withdrawn (was: direct copies, 256x256 tile, 4 waves - it   */
+                              /* spilled registers and was slower): AMOS_ERR_INFEASIBLE       */
 #define AMOS_PIPE_DIRECT8 3   /* same with 8 waves (two per SIMD)                             */
 #define AMOS_PIPE_PATCH 4     /* conv: input patch staged once per channel chunk, weights     */
                               /* repacked into the workspace; needs amos_workspace_bytes();   */

@@ -37,7 +37,7 @@ def d_types(dtype):
     (200, 136, 72, 0, 0, None),                                           # register-staged kernel, ragged
     (130, 264, 520, 1, 1, dict(tile_i=64, tile_j=128, split_k=3)),        # split-K: D is added once
     (512, 768, 256, 0, 1, dict(tile_i=256, tile_j=256, split_k=1, pipeline=3)),   # direct-to-LDS kernel
-    (300, 520, 384, 0, 1, dict(tile_i=256, tile_j=256, split_k=1, pipeline=2)),
+    (300, 520, 384, 0, 1, dict(tile_i=128, tile_j=128, split_k=1, pipeline=3)),
 ])
 def test_gemm_add(gpu, dtype, case):
     from amos_amd import ops

@@ -88,8 +88,8 @@ def test_gemm_every_tile(gpu, dtype, tile, split):
 
 
 @pytest.mark.parametrize("dtype", ["float16", "bfloat16", "int8"])
-# direct-to-LDS copies: 256x256 with 4 and 8 waves, the smaller tiles (two and three LDS stages) with 8
-@pytest.mark.parametrize("pipeline,tile", [(2, (256, 256)), (3, (256, 256)), (3, (128, 128)), (3, (128, 256)),
+# direct-to-LDS copies: 256x256 and the smaller tiles (two and three LDS stages), eight waves
+@pytest.mark.parametrize("pipeline,tile", [(3, (256, 256)), (3, (128, 128)), (3, (128, 256)),
                                            (3, (256, 128)), (0, (128, 128))])
 @pytest.mark.parametrize("shape", [(256, 256, 128), (512, 768, 1024), (300, 520, 384), (1, 257, 128)])
 def test_gemm_direct_pipeline(gpu, dtype, pipeline, tile, shape):
@@ -286,8 +286,30 @@ def test_gemm_direct_pipeline_rejects_ragged_k(gpu):
     from amos_amd import _lib, ops
     a = torch.zeros((256, 72), dtype=torch.float16, device="cuda")
     with pytest.raises(_lib.AmosError) as e:
-        ops.gemm(a, a, False, True, config=dict(tile_i=256, tile_j=256, split_k=1, pipeline=2))
+        ops.gemm(a, a, False, True, config=dict(tile_i=256, tile_j=256, split_k=1, pipeline=3))
     assert e.value.code == _lib.AMOS_ERR_INFEASIBLE
+
+
+def test_gemm_four_wave_pipeline_withdrawn(gpu):
+    """AMOS_PIPE_DIRECT4 (the four-wave direct-to-LDS instance) is refused: nothing is launched"""
+    import torch
+    from amos_amd import _lib, ops
+    a = torch.zeros((256, 128), dtype=torch.float16, device="cuda")
+    with pytest.raises(_lib.AmosError) as e:
+        ops.gemm(a, a, False, True, config=dict(tile_i=256, tile_j=256, split_k=1, pipeline=_lib.AMOS_PIPE_DIRECT4))
+    assert e.value.code == _lib.AMOS_ERR_INFEASIBLE and "withdrawn" in str(e.value)
+
+
+@pytest.mark.skip(reason="the four-wave direct-to-LDS instance is withdrawn: a launch of it at 8192^3 ended in a "
+                         "GPU memory fault whose cause is not found; the library refuses AMOS_PIPE_DIRECT4")
+def test_gemm_four_wave_pipeline(gpu):
+    from amos_amd import ops
+    rng = np.random.default_rng(3)
+    a = make_operand(rng, (300, 384), "float16")
+    b = make_operand(rng, (520, 384), "float16")
+    cfg = dict(tile_i=256, tile_j=256, split_k=1, pipeline=2)
+    got = ops.gemm(to_device(a, "float16"), to_device(b, "float16"), False, True, config=cfg).cpu().numpy()
+    check(got, co.lib_gemm(a, b, "float16", False, True, acc="float64"), "float16", "four-wave direct gemm")
 
 
 def test_gemm_config1_512(gpu):
