@@ -9,8 +9,8 @@
 //     registers, no ds_write; the XOR swizzle of the LDS layout is applied on the
 //     global-address side (a wave instruction fills 1 KB of LDS linearly, lane l
 //     fetches the 16-byte chunk that belongs at that position);
-//   * operand fragments are double buffered in registers: the ds_reads of K
-//     sub-step s+1 are in flight while the MFMAs of sub-step s issue;
+//   * operand fragments are double buffered in registers: the ds_reads of the next half
+//     sub-step are in flight while the MFMAs (16x16x32, int8 16x16x64) of this one issue;
 //   * one barrier per K step; the copies for step kt+NS are issued right after it and
 //     have NS-1 steps to land.  Every step issues a tile (steps past the end fetch the last
 //     one again), so that the number of copies in flight behind the tile a step waits for
@@ -44,162 +44,10 @@ struct GemmTnParams {
 #define AMOS_GLOBAL_PTR(p) ((const __attribute__((address_space(1))) void*)(p))
 #define AMOS_LDS_PTR(p) ((__attribute__((address_space(3))) void*)(p))
 
-template <int DT, int WI, int WJ, int BI, int BJ, int NS>
-__device__ __forceinline__ void gemm_tn_body32(const GemmTnParams p) {
-  typedef Mfma<DT> MM;
-  typedef typename MM::acc_t acc_t;
-  typedef typename MM::out_t out_t;
-  constexpr int ES = MM::ES;
-  constexpr int BKE = 128 / ES;
-  constexpr int NW = WI * WJ;
-  constexpr int TI = BI / (32 * WI), TJ = BJ / (32 * WJ);
-  static_assert(TI >= 1 && TJ >= 1 && TI * WI * 32 == BI && TJ * WJ * 32 == BJ, "wave tile");
-  constexpr int OPER = BI * 128;       // bytes of the A tile; the B tile follows it
-  constexpr int STAGE = (BI + BJ) * 128;
-  constexpr int QA = BI / 8;           // 1 KB copy chunks (8 rows) of the A tile
-  constexpr int CH = (BI + BJ) / 8 / NW;   // copy chunks per wave per K step
-  static_assert(CH >= 1 && CH * NW * 8 == BI + BJ, "copy chunks");
-
-  extern __shared__ __attribute__((aligned(16))) char smem[];
-
-  const int t = threadIdx.x;
-  const int lane = t & 63;
-  const int wave = __builtin_amdgcn_readfirstlane(t >> 6);
-  const int wi = wave / WJ, wj = wave % WJ;
-
-  int tile_i, tile_j;
-  block_to_tile(blockIdx.x, gridDim.x, p.tiles_i, p.tiles_j, tile_i, tile_j);
-  const int bi0 = tile_i * BI, bj0 = tile_j * BJ;
-  const int64_t batch = blockIdx.z;
-  const char* const abase = p.a + (batch * p.batch_a + (int64_t)bi0 * p.lda) * ES;
-  const char* const bbase = p.b + (batch * p.batch_b + (int64_t)bj0 * p.ldb) * ES;
-
-  // ---- copy slots: chunk q of this wave covers tile rows [8*qq, 8*qq+8) of A (q < BI/8) or B
-  unsigned g_off[CH];   // byte offset from the operand's tile base, K step 0
-#pragma unroll
-  for (int u = 0; u < CH; ++u) {
-    const int q = wave + NW * u;       // uniform per wave
-    const int qq = q < QA ? q : q - QA;
-    const int row = qq * 8 + (lane >> 3);
-    const int chunk = (lane & 7) ^ ((row ^ (row >> 3)) & 7);
-    if (q < QA) {
-      int r = bi0 + row < p.I ? row : p.I - 1 - bi0;
-      g_off[u] = (unsigned)r * (unsigned)(p.lda * ES) + chunk * 16;
-    } else {
-      int r = bj0 + row < p.J ? row : p.J - 1 - bj0;
-      g_off[u] = (unsigned)r * (unsigned)(p.ldb * ES) + chunk * 16;
-    }
-  }
-
-  auto issue_copies = [&](int kt, int stage) {
-    const char* ak = abase + (int64_t)kt * 128;
-    const char* bk = bbase + (int64_t)kt * 128;
-    char* s = smem + stage * STAGE;
-#pragma unroll
-    for (int u = 0; u < CH; ++u) {
-      const int q = wave + NW * u;
-      const char* src = (q < QA ? ak : bk) + g_off[u];
-      __builtin_amdgcn_global_load_lds(AMOS_GLOBAL_PTR(src), AMOS_LDS_PTR(s + q * 1024), 16, 0, 0);
-    }
-  };
-
-  // ---- fragment read offsets: row = tile_row0 + a*32 + lane%32, chunk = 2*ks + lane/32
-  const int frag_row = lane & 31, frag_half = lane >> 5;
-  int a_off[2][4], b_off[2][4];   // [a & 1][ks]: the swizzle term flips with the parity of a
-#pragma unroll
-  for (int par = 0; par < 2; ++par)
-#pragma unroll
-    for (int ks = 0; ks < 4; ++ks) {
-      a_off[par][ks] = lds_chunk_offset(wi * TI * 32 + par * 32 + frag_row, ks * 2 + frag_half);
-      b_off[par][ks] = OPER + lds_chunk_offset(wj * TJ * 32 + par * 32 + frag_row, ks * 2 + frag_half);
-    }
-
-  acc_t acc[TI][TJ];
-#pragma unroll
-  for (int a = 0; a < TI; ++a)
-#pragma unroll
-    for (int b = 0; b < TJ; ++b)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) acc[a][b][r] = 0;
-
-  v4i af[2][TI], bf[2][TJ];
-  auto read_frags = [&](int stage, int ks, int slot) {
-    const char* s = smem + stage * STAGE;
-#pragma unroll
-    for (int a = 0; a < TI; ++a)
-      af[slot][a] = *(const v4i*)(s + a_off[a & 1][ks] + (a >> 1) * (64 * 128));
-#pragma unroll
-    for (int b = 0; b < TJ; ++b)
-      bf[slot][b] = *(const v4i*)(s + b_off[b & 1][ks] + (b >> 1) * (64 * 128));
-  };
-  auto mma = [&](int slot) {
-#pragma unroll
-    for (int a = 0; a < TI; ++a)
-#pragma unroll
-      for (int b = 0; b < TJ; ++b) acc[a][b] = MM::run(af[slot][a], bf[slot][b], acc[a][b]);
-  };
-
-  const int KT = p.K / BKE;
-  static_assert(NS >= 2 && (NS - 1) * CH <= 63, "stages");
-#pragma unroll
-  for (int s = 0; s < NS; ++s) issue_copies(s < KT ? s : KT - 1, s);
-  // tile 0 has landed once at most the NS-1 younger tiles are in flight (copies complete in order)
-  asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"((NS - 1) * CH) : "memory");
-  read_frags(0, 0, 0);
-
-  int st = 0;   // stage of tile kt
-  for (int kt = 0; kt < KT; ++kt) {
-    const int st_next = st + 1 == NS ? 0 : st + 1;
-    read_frags(st, 1, 1);
-    mma(0);
-    read_frags(st, 2, 0);
-    mma(1);
-    read_frags(st, 3, 1);
-    mma(0);
-    // every ds_read of this stage has been issued; once they and this wave's copies of the
-    // next tile are complete (the NS-2 tiles behind it may still be in flight), meet the other
-    // waves: after the barrier the next stage is fully written and this stage is free to be
-    // overwritten
-    asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"((NS - 2) * CH) : "memory");
-    issue_copies(kt + NS < KT ? kt + NS : KT - 1, st);
-    if (kt + 1 < KT) read_frags(st_next, 0, 0);
-    mma(1);
-    st = st_next;
-  }
-
-  // ---- epilogue ---------------------------------------------------------------------
-  out_t* const out = (out_t*)p.c + batch * p.batch_c;
-#pragma unroll
-  for (int b = 0; b < TJ; ++b) {
-    const int j = bj0 + (wj * TJ + b) * 32 + frag_row;
-    if (j >= p.J) continue;
-#pragma unroll
-    for (int a = 0; a < TI; ++a) {
-      if (p.epi.dt != EPI_NONE) {   // all sixteen loads of the tile in flight before the first addition
-        out_t dv[16];
-#pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          const int i = bi0 + (wi * TI + a) * 32 + 8 * (r >> 2) + 4 * frag_half + (r & 3);
-          dv[r] = epi_value<out_t>(p.epi, batch * p.epi.batch + (int64_t)(i < p.I ? i : p.I - 1) * p.epi.si + j);
-        }
-#pragma unroll
-        for (int r = 0; r < 16; ++r) acc[a][b][r] += dv[r];
-      }
-#pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const int i = bi0 + (wi * TI + a) * 32 + 8 * (r >> 2) + 4 * frag_half + (r & 3);
-        if (i < p.I) out[(int64_t)i * p.ldc + j] = acc[a][b][r];
-      }
-    }
-  }
-  // the tiles fetched again by the last steps still target this block's LDS
-  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-}
-
 // The 16x16 matrix-core shapes (v_mfma_f32_16x16x32_f16 / _bf16, v_mfma_i32_16x16x64_i8): the same
-// flops per LDS byte as 32x32x16 on the same wave tile, and measured 4-6 % faster on the 8192^3
-// fp16 product (on random operands the chip sustains a higher clock under them).  An operand
-// fragment is row = lane % 16, 16-byte chunk = lane / 16 of a 64-byte K sub-step.
+// flops per LDS byte as 32x32x16 on the same wave tile, and measured 3-8 % faster at every tile here
+// (on random operands the chip sustains a higher clock under them).  An operand fragment is
+// row = lane % 16 and one 16-byte chunk of a 64-byte K sub-step per lane group lane / 16.
 template <int DT>
 struct Mfma16;
 template <>
@@ -224,11 +72,11 @@ struct Mfma16<DT_I8> {
   }
 };
 
-// Same tiles, copies, LDS layout and barriers as gemm_tn_body32.  A K step (128 bytes per row) is
-// two sub-steps of 64 bytes; each is issued in two halves over the wave tile's rows, so that the
-// fragment registers in flight stay at two half-sets of A and two sets of B.
-template <int DT, int WI, int WJ, int BI, int BJ, int NS>
-__device__ __forceinline__ void gemm_tn_body16(const GemmTnParams p) {
+// A K step (128 bytes per row) is two sub-steps of 64 bytes; each is issued in two halves over the
+// wave tile's rows, so that the fragment registers in flight stay at two half-sets of A and two
+// sets of B while the reads of the next half are in flight behind the MFMAs of this one.
+template <int DT, int WI, int WJ, int BI = 256, int BJ = 256, int NS = 2>
+__global__ __launch_bounds__(64 * WI * WJ) void amos_gemm_tn(const GemmTnParams p) {
   typedef Mfma16<DT> MM;
   typedef typename MM::acc_t acc_t;
   typedef typename Mfma<DT>::out_t out_t;
@@ -290,15 +138,23 @@ __device__ __forceinline__ void gemm_tn_body16(const GemmTnParams p) {
     }
   };
 
+  // Lane group q = lane / 16 feeds the matrix core's K positions [8q, 8q + 8) of a sub-step; which
+  // 16-byte chunk of the tile it takes them from is free as long as both operands agree (a dot
+  // product does not care about the order of K).  A 16-byte LDS read serves lanes l and l + 32 in
+  // the same cycle, so groups q and q + 2 take chunks that differ in the lowest bit, which the
+  // swizzle maps to different banks: chunks 0, 2, 1, 3 for q = 0..3.  (With chunk = q the
+  // conflict counter read half of all LDS cycles.)
   const int frag_row = lane & 15, frag_q = lane >> 4;
+  const int frag_chunk = (frag_q >> 1) | ((frag_q & 1) << 1);
   int a_off[AO][2], b_off[BO][2];
 #pragma unroll
   for (int ks = 0; ks < 2; ++ks) {
 #pragma unroll
-    for (int a = 0; a < AO; ++a) a_off[a][ks] = lds_chunk_offset(wi * TI * 16 + a * 16 + frag_row, ks * 4 + frag_q);
+    for (int a = 0; a < AO; ++a)
+      a_off[a][ks] = lds_chunk_offset(wi * TI * 16 + a * 16 + frag_row, ks * 4 + frag_chunk);
 #pragma unroll
     for (int b = 0; b < BO; ++b)
-      b_off[b][ks] = OPER + lds_chunk_offset(wj * TJ * 16 + b * 16 + frag_row, ks * 4 + frag_q);
+      b_off[b][ks] = OPER + lds_chunk_offset(wj * TJ * 16 + b * 16 + frag_row, ks * 4 + frag_chunk);
   }
 
   acc_t acc[TI][TJ];
@@ -348,7 +204,10 @@ __device__ __forceinline__ void gemm_tn_body16(const GemmTnParams p) {
     mma(1, 1, 0);
     read_a(st, 1, 1, 1);
     mma(0, 0, 1);
-    // (as in gemm_tn_body32: reads of this stage issued, the next tile's copies complete)
+    // every ds_read of this stage has been issued; once they and this wave's copies of the
+    // next tile are complete (the NS-2 tiles behind it may still be in flight), meet the other
+    // waves: after the barrier the next stage is fully written and this stage is free to be
+    // overwritten
     asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"((NS - 2) * CH) : "memory");
     issue_copies(kt + NS < KT ? kt + NS : KT - 1, st);
     if (kt + 1 < KT) {
@@ -392,15 +251,6 @@ __device__ __forceinline__ void gemm_tn_body16(const GemmTnParams p) {
     }
   }
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-}
-
-// MF = rows of the matrix-core shape: 32 (32x32x16 / 32x32x32 int8) or 16 (16x16x32 / 16x16x64)
-template <int DT, int WI, int WJ, int BI = 256, int BJ = 256, int NS = 2, int MF = 32>
-__global__ __launch_bounds__(64 * WI * WJ) void amos_gemm_tn(const GemmTnParams p) {
-  if constexpr (MF == 16)
-    gemm_tn_body16<DT, WI, WJ, BI, BJ, NS>(p);
-  else
-    gemm_tn_body32<DT, WI, WJ, BI, BJ, NS>(p);
 }
 
 }  // namespace amos

@@ -1,13 +1,13 @@
 #include "gemm_tn_kernel.h"
 #include "igemm_instances.h"
 namespace amos {
-template <int DT, int WI, int WJ, int BI, int BJ, int NS, int MF = 32>
+template <int DT, int WI, int WJ, int BI, int BJ, int NS>
 static TnInstance* tn_instance() {
   static TnInstance inst;
   static const char* dtn[] = {"f16", "bf16", "i8"};
   static std::string name = std::string("amos_gemm_tn<") + dtn[DT] + "," + std::to_string(BI) + "x" +
                             std::to_string(BJ) + "," + std::to_string(WI * WJ) + "w>";
-  inst.fn = amos_gemm_tn<DT, WI, WJ, BI, BJ, NS, MF>;
+  inst.fn = amos_gemm_tn<DT, WI, WJ, BI, BJ, NS>;
   inst.lds = NS * (BI + BJ) * 128;
   inst.threads = 64 * WI * WJ;
   inst.name = name.c_str();
@@ -15,14 +15,9 @@ static TnInstance* tn_instance() {
 }
 template <int DT>
 static TnInstance* pick_tn(int ti, int tj, int waves) {
-  // The 16x16 matrix-core shapes where they measured ahead of 32x32: the 256x256 tile with eight
-  // waves (8192^3: fp16 931 -> 903 us, bf16 881 -> 862, int8 488 -> 475; 4096^3 fp16 122 -> 115.5) and
-  // the 128x128 tile in fp16 / bf16 (2048^3 25.4 -> 24.5 us; int8 14.4 -> 15.3, so not there); the
-  // 128x256 / 256x128 tiles were level or behind with them.
   if (waves != 8) return nullptr;   // (a four-wave 256x256 instance existed: spills, slower, withdrawn)
-  if (ti == 256 && tj == 256) return tn_instance<DT, 2, 4, 256, 256, 2, 16>();
-  if (ti == 128 && tj == 128)
-    return DT == DT_I8 ? tn_instance<DT, 2, 4, 128, 128, 2>() : tn_instance<DT, 2, 4, 128, 128, 2, 16>();
+  if (ti == 256 && tj == 256) return tn_instance<DT, 2, 4, 256, 256, 2>();
+  if (ti == 128 && tj == 128) return tn_instance<DT, 2, 4, 128, 128, 2>();
   if (ti == 128 && tj == 256) return tn_instance<DT, 2, 4, 128, 256, 3>();
   if (ti == 256 && tj == 128) return tn_instance<DT, 4, 2, 256, 128, 3>();
   return nullptr;

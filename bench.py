@@ -23,7 +23,7 @@ PEAK_I8_TOPS = 5000.0      # published dense int8 peak
 PEAK_HBM_GBS = 8000.0      # published HBM3E bandwidth
 # bytes beyond L2 per launch, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this command,
 # each scaled by the same counter's reading for a 256 MiB device copy (x2.0 and x1.0)
-MEASURED_TRAFFIC = {"amos_gemm_tn<f16,256x256,8w>": 870610 * 1024 * 2.0 + 262140 * 1024 * 1.0}
+MEASURED_TRAFFIC = {"amos_gemm_tn<f16,256x256,8w>": 793010 * 1024 * 2.0 + 305010 * 1024 * 1.0}
 
 
 def cpu_baseline_gemm(a, b, seconds_budget=12.0):
