@@ -179,11 +179,11 @@ __global__ __launch_bounds__(64 * WI * WJ) void amos_gemm_tn(const GemmTnParams 
 #pragma unroll
     for (int b = 0; b < TJ; ++b) bf[slot][b] = *(const v4i*)(s + b_off[b & 3][ks] + (b >> 2) * (64 * 128));
   };
-  auto mma = [&](int h, int sa, int sb) {
+  auto mma = [&](int h, int sa, int sb) {   // (B fragment outermost: measured 1 % ahead of A outermost)
 #pragma unroll
-    for (int a = 0; a < HA; ++a)
+    for (int b = 0; b < TJ; ++b)
 #pragma unroll
-      for (int b = 0; b < TJ; ++b) acc[h * HA + a][b] = MM::run(af[sa][a], bf[sb][b], acc[h * HA + a][b]);
+      for (int a = 0; a < HA; ++a) acc[h * HA + a][b] = MM::run(af[sa][a], bf[sb][b], acc[h * HA + a][b]);
   };
 
   const int KT = p.K / BKE;
