@@ -163,6 +163,13 @@ def run_all_configs(cpu=True, only=None):
         ops.conv_desc((16, 3, 1, 224, 224), (64, 3, 1, 7, 7), torch.float16, (1, 2, 2), (0, 3, 3), (1, 1, 1)),
         [xs, ws], "float16", 2.0 * 16 * 112 * 112 * 64 * 147, 16 * 3 * 224 * 224 * 2 + 64 * 147 * 2 + 16 * 64 * 112 * 112 * 4,
         (16, 64, 112, 112), None, None)
+    # a GEMV as benchmark/amos/mapping_gemv_tensorcore.py spells it (A [M, K], B [K, 1]), at a size
+    # where it is the pass over A that is timed (the reference's own shapes, up to 1024 x 1024, are
+    # launch-bound): one pass over 268 MB on the vector-ALU kernel
+    mv, kv = 16384, 8192
+    av, bv = f16(rng.uniform(-1, 1, (mv, kv))), f16(rng.uniform(-1, 1, (kv, 1)))
+    add("GEMV fp16 M=16384 K=8192 (B [K, 1])", _lib.AMOS_OP_GEMM, ops.gemm_desc(mv, 1, kv, torch.float16, False, False),
+        [av, bv], "float16", 2.0 * mv * kv, mv * kv * 2 + kv * 2 + mv * 4, (mv, 1), None, None)
     return rows
 
 
