@@ -81,7 +81,7 @@ def run_all_configs(cpu=True, only=None):
     def add(name, op, desc, hin, dtype, flop, nbytes, out_shape, cpu_fn, frac, fused_tail=False):
         if only and only not in name:
             return
-        tin = [torch.from_numpy(h).cuda() for h in hin]
+        tin = [(torch.from_numpy(h) if isinstance(h, np.ndarray) else h).cuda() for h in hin]
         out = torch.empty(out_shape, dtype=torch.int32 if dtype == "int8" else torch.float32,
                           device="cuda")
         # fused tail out = acc + D: D has the output's shape and type, read once more
@@ -163,6 +163,13 @@ def run_all_configs(cpu=True, only=None):
         ops.conv_desc((16, 3, 1, 224, 224), (64, 3, 1, 7, 7), torch.float16, (1, 2, 2), (0, 3, 3), (1, 1, 1)),
         [xs, ws], "float16", 2.0 * 16 * 112 * 112 * 64 * 147, 16 * 3 * 224 * 224 * 2 + 64 * 147 * 2 + 16 * 64 * 112 * 112 * 4,
         (16, 64, 112, 112), None, None)
+    # the 8192^3 product in the path's other two operand types (bf16 -> fp32, int8 -> int32)
+    add("GEMM bf16 8192^3 (ntn)", _lib.AMOS_OP_GEMM, ops.gemm_desc(n, n, n, torch.bfloat16, False, True),
+        [torch.from_numpy(a.astype(np.float32)).to(torch.bfloat16), torch.from_numpy(b.astype(np.float32)).to(torch.bfloat16)],
+        "bfloat16", 2.0 * n ** 3, 2 * n * n * 2 + n * n * 4, (n, n), None, None)
+    a8, b8 = rng.integers(-128, 128, (n, n), dtype=np.int8), rng.integers(-128, 128, (n, n), dtype=np.int8)
+    add("GEMM int8 8192^3 (ntn)", _lib.AMOS_OP_GEMM, ops.gemm_desc(n, n, n, torch.int8, False, True),
+        [a8, b8], "int8", 2.0 * n ** 3, 2 * n * n + n * n * 4, (n, n), None, None)
     # a GEMV as benchmark/amos/mapping_gemv_tensorcore.py spells it (A [M, K], B [K, 1]), at a size
     # where it is the pass over A that is timed (the reference's own shapes, up to 1024 x 1024, are
     # launch-bound): one pass over 268 MB on the vector-ALU kernel
