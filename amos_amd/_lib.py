@@ -15,6 +15,7 @@ AMOS_ERR_UNSUPPORTED = -2
 AMOS_ERR_INFEASIBLE = -3
 AMOS_ERR_HIP = -4
 AMOS_ERR_WORKSPACE = -5
+AMOS_NOALLOC_SCRATCH_BYTES = 8 << 20
 
 DTYPE_CODE = {"float16": AMOS_F16, "bfloat16": AMOS_BF16, "int8": AMOS_I8, "float32": AMOS_F32,
               "int32": AMOS_I32}
@@ -95,7 +96,7 @@ class AmosError(RuntimeError):
 EXPORTS = [
     "amos_version", "amos_last_error", "amos_device_info", "amos_default_config",
     "amos_check_config", "amos_workspace_bytes", "amos_estimate_seconds", "amos_gemm", "amos_bgemm", "amos_conv2d",
-    "amos_conv3d", "amos_run_fused", "amos_time", "amos_time_fused", "amos_gather", "amos_time_gather",
+    "amos_conv3d", "amos_conv2d_noalloc", "amos_run_fused", "amos_time", "amos_time_fused", "amos_gather", "amos_time_gather",
     "amos_eltwise", "amos_time_eltwise", "amos_kernel_name", "amos_match", "amos_enumerate_mappings",
 ]
 
@@ -127,6 +128,8 @@ def load():
         fn = getattr(lib, name)
         fn.argtypes = [ctypes.POINTER(desc), ctypes.POINTER(KernelConfig), vp, vp, vp, vp, sz, vp]
         fn.restype = ctypes.c_int
+    lib.amos_conv2d_noalloc.argtypes = [ctypes.POINTER(ConvDesc), ctypes.POINTER(KernelConfig), vp, vp, vp, vp]
+    lib.amos_conv2d_noalloc.restype = ctypes.c_int
     lib.amos_time.argtypes = [ctypes.c_int, vp, ctypes.POINTER(KernelConfig), vp, vp, vp, vp, sz, vp,
                               ctypes.c_int, ctypes.c_int, ctypes.c_int,
                               ctypes.POINTER(ctypes.c_double)]

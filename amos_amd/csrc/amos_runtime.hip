@@ -1178,6 +1178,31 @@ static int launch_gather(const amos_gather_desc_t* d, const void* in, const int3
   return 0;
 }
 
+// ---- scratch memory for the entry point that allocates nothing ---------------------------------
+// One array per GPU, held from the moment the code object is loaded there until the process ends.
+// In host code the array's name is only a stand-in: the address a kernel may use is the one
+// hipGetSymbolAddress returns with that device current, looked up once per device and kept.
+static __device__ __align__(256) unsigned char scratch[AMOS_NOALLOC_SCRATCH_BYTES];
+constexpr int kScratchMaxDevices = 64;
+static void* g_scratch_ptr[kScratchMaxDevices];
+static std::mutex g_scratch_mutex;
+
+static int scratch_of_current_device(void** out) {
+  int dev = 0;
+  HIP_TRY(hipGetDevice(&dev));
+  if (dev < 0 || dev >= kScratchMaxDevices)
+    return set_error(AMOS_ERR_UNSUPPORTED, "device ordinal %d above %d", dev, kScratchMaxDevices - 1);
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (!g_scratch_ptr[dev]) {
+    void* ptr = nullptr;
+    HIP_TRY(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)));
+    if (!ptr) return set_error(AMOS_ERR_HIP, "hipGetSymbolAddress returned a null address for the scratch array");
+    g_scratch_ptr[dev] = ptr;
+  }
+  *out = g_scratch_ptr[dev];
+  return 0;
+}
+
 // time_evaluator's loop (src/runtime/rpc/rpc_module.cc:355-388) around a launch
 template <typename Launch>
 static int time_launches(Launch launch_once, hipStream_t stream, int number, int repeat, int min_repeat_ms,
@@ -1258,6 +1283,22 @@ int amos_conv2d(const amos_conv_desc_t* desc, const amos_kernel_config_t* cfg, c
 int amos_conv3d(const amos_conv_desc_t* desc, const amos_kernel_config_t* cfg, const void* X,
                 const void* Wt, void* Y, void* workspace, size_t ws_bytes, void* stream) {
   return run_op(AMOS_OP_CONV3D, desc, cfg, nullptr, X, Wt, Y, workspace, ws_bytes, stream);
+}
+
+int amos_conv2d_noalloc(const amos_conv_desc_t* desc, const amos_kernel_config_t* cfg, const void* X,
+                        const void* Wt, void* Y, void* stream) {
+  if (!desc) return set_error(AMOS_ERR_BAD_ARG, "null descriptor");
+  const size_t need = amos_workspace_bytes(AMOS_OP_CONV2D, desc, cfg);
+  if (need > (size_t)AMOS_NOALLOC_SCRATCH_BYTES)
+    return set_error(AMOS_ERR_WORKSPACE, "this convolution wants %zu bytes of scratch memory, the library's own "
+                     "array holds %zu (amos_conv2d with a caller-owned workspace has no such limit)",
+                     need, (size_t)AMOS_NOALLOC_SCRATCH_BYTES);
+  void* ptr = nullptr;
+  int rc = scratch_of_current_device(&ptr);
+  if (rc) return rc;
+  // every launch below is handed `ptr`; what a kernel needs cleared in it (the zero block, the step
+  // table) is rewritten by the relayout launch of this very call
+  return run_op(AMOS_OP_CONV2D, desc, cfg, nullptr, X, Wt, Y, ptr, (size_t)AMOS_NOALLOC_SCRATCH_BYTES, stream);
 }
 
 int amos_run_fused(int op, const void* desc, const amos_kernel_config_t* cfg,

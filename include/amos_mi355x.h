@@ -198,6 +198,21 @@ int amos_conv2d(const amos_conv_desc_t* desc, const amos_kernel_config_t* cfg, c
 int amos_conv3d(const amos_conv_desc_t* desc, const amos_kernel_config_t* cfg, const void* X,
                 const void* Wt, void* Y, void* workspace, size_t ws_bytes, void* stream);
 
+/*
+ * amos_conv2d without a workspace argument and without any allocation: the scratch memory the
+ * patch-staged pipeline wants (relaid weights and activations, the step table, split-K partial
+ * sums) is an array of AMOS_NOALLOC_SCRATCH_BYTES that the library keeps on every GPU it has run
+ * on, from the first call there until the process ends.  This entry point has no counterpart in
+ * the reference; it is for callers that cannot allocate device memory: code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc.  It calls no hipMalloc / hipFree
+ * and no allocating library routine.  A convolution whose amos_workspace_bytes() exceeds the
+ * array is refused with AMOS_ERR_WORKSPACE.  All calls on one GPU share that GPU's array: calls
+ * that overlap in time on one GPU (two streams, two threads) race; serialise them.
+ */
+#define AMOS_NOALLOC_SCRATCH_BYTES (8u << 20)
+int amos_conv2d_noalloc(const amos_conv_desc_t* desc, const amos_kernel_config_t* cfg, const void* X,
+                        const void* Wt, void* Y, void* stream);
+
 /* A tail operation fused into the store of the accumulators.  AMOS_EPI_ADD: out = acc + cast(D),
  * D an operand with the output's shape: GEMM / batched GEMM [M][ld] (ld 0 = N) with `stride`
  * elements between batches (0 = M*ld); convolution NKDPQ, contiguous.  D is fp32, fp16 or bf16
