@@ -138,8 +138,9 @@ def mfma_fragment_layout(shape_key):
       a(lane, e) -> (i, k)   e-th element of the lane's A fragment
       b(lane, e) -> (k, j)
       d(lane, r) -> (i, j)   r-th accumulator register of the lane
-    The 32x32 layouts are the ones the shipped kernels use and are checked on hardware by
-    the parity tests; the 16x16 entries document the other shape key.
+    Both are checked on hardware by the parity tests: the direct-to-LDS GEMM kernels issue the
+    16x16 shapes (16x16x32 fp16 / bf16, 16x16x64 int8), the register-staged implicit GEMM and
+    the patch-staged convolution the 32x32 ones (32x32x16, int8 32x32x32).
     """
     m, n, k = (int(x) for x in shape_key.split("x"))
     per_lane = k * m // 64          # K elements a lane holds (8 halves or 16 int8)

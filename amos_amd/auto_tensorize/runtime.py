@@ -145,7 +145,32 @@ class Module(object):
                 continue
             a = arrays[i]
             out.append(a.tensor if isinstance(a, NDArray) else a)
+        passed = [(k, t) for k, (t, i) in enumerate(zip(out, self.arg_index)) if i is not None]
+        for k, t in passed:     # extents and element types of every array first, then where they live
+            self._check_array(k, t, placement=False)
+        for k, t in passed:
+            self._check_array(k, t, placement=True)
         return out
+
+    def _check_array(self, k, t, placement):
+        """The kernels take raw pointers: an array that is not the tensor the compute declares
+        (its extents, its element type, on a device, dense) is refused before any launch, as the
+        reference's argument binder does at call time."""
+        lw = self.lowered
+        decl = lw.inputs[k] if k < 2 else lw.output if k == 2 else lw.add_input
+        what = ("first operand", "second operand", "output", "added operand")[k]
+        if not isinstance(t, torch.Tensor):
+            raise ValueError("%s %s must be a device array, got %s" % (what, decl.name, type(t).__name__))
+        shape = tuple(int(e) for e in decl.shape)
+        if tuple(t.shape) != shape or t.dtype != _TORCH_DTYPE[decl.dtype]:
+            raise ValueError("%s %s is declared %s %s, the array passed is %s %s"
+                             % (what, decl.name, decl.dtype, shape, str(t.dtype).replace("torch.", ""), tuple(t.shape)))
+        if not placement:
+            return
+        if not t.is_cuda:
+            raise ValueError("%s %s must be a device array, got one on %s" % (what, decl.name, t.device))
+        if not t.is_contiguous():
+            raise ValueError("%s %s must be a dense (contiguous) array" % (what, decl.name))
 
     def _kernel_output(self, out):
         """where the kernel writes: the caller's array, or a buffer of the module's from which

@@ -3,6 +3,12 @@ per-architecture limits of `CUDA(arch)`)."""
 
 supported_target = ["hip", "rocm"]
 
+# MI355X's published dense peaks: the one place they are written down (bench.py and the reports
+# divide by these; the figure a device's own clock and CU count give is amos_device_info's)
+PEAK_F16_TFLOPS = 2500.0    # fp16 / bf16 MFMA, dense
+PEAK_I8_TOPS = 5000.0       # int8 MFMA, dense
+PEAK_HBM_GBS = 8000.0       # HBM3E
+
 
 class AcceleratorTarget(object):
     pass
@@ -19,9 +25,16 @@ class MI355X(AcceleratorTarget):
     def get_register_bytes_per_thread(self): return 512 * 4
     def max_threads(self): return 1024
     def max_blocks(self): return 2 ** 31 - 1
-    def compute_units(self): return 256
-    def peak_tflops(self, dtype): return 5033.2 if dtype == "int8" else 2516.6
-    def hbm_bytes_per_second(self): return 8e12
+    def compute_units(self):
+        """of the device when one is visible (a partitioned or binned part has fewer), else the full part's 256"""
+        import torch
+        if torch.cuda.is_available():
+            from .. import ops
+            return int(ops.device_info().compute_units)
+        return 256
+
+    def peak_tflops(self, dtype): return PEAK_I8_TOPS if dtype == "int8" else PEAK_F16_TFLOPS
+    def hbm_bytes_per_second(self): return PEAK_HBM_GBS * 1e9
 
 
 def get_device_arch(dev_id=0):

@@ -929,10 +929,19 @@ static int launch_tn(const Plan& pl, hipStream_t stream) {
   std::call_once(inst->once, [&] {
     attr_err = hipFuncSetAttribute((const void*)inst->fn, hipFuncAttributeMaxDynamicSharedMemorySize,
                                    (int)inst->lds);
+    // The kernel decides that a direct-to-LDS tile has landed by counting its own outstanding
+    // vector-memory operations (s_waitcnt vmcnt(n)); register spills are vector-memory operations
+    // too, so an instance the compiler gave scratch memory would wait on the wrong ones.
+    hipFuncAttributes fa;
+    if (attr_err == hipSuccess) attr_err = hipFuncGetAttributes(&fa, (const void*)inst->fn);
+    if (attr_err == hipSuccess) inst->scratch_bytes = (int)fa.localSizeBytes;
   });
   if (attr_err != hipSuccess)
     return set_error(AMOS_ERR_HIP, "hipFuncSetAttribute(%s): %s", inst->name,
                      hipGetErrorString(attr_err));
+  if (inst->scratch_bytes)
+    return set_error(AMOS_ERR_INFEASIBLE, "%s was built with %d bytes of scratch memory per lane (register "
+                     "spills), which its wait counts do not allow for", inst->name, inst->scratch_bytes);
   dim3 grid((unsigned)(pl.tn.tiles_i * pl.tn.tiles_j), 1, (unsigned)pl.batch);
   hipLaunchKernelGGL(inst->fn, grid, dim3(inst->threads), inst->lds, stream, pl.tn);
   HIP_TRY(hipGetLastError());
@@ -966,7 +975,7 @@ static int launch_conv(const Plan& pl, hipStream_t stream) {
   launch_conv_prepare(pl.dt == DT_I8 ? 1 : 2, q, stream);
   dim3 grid((unsigned)(q.tiles_i * q.tiles_j), (unsigned)pl.split, 1);
   // blocks that walk their tiles: one per compute unit, tiles blockIdx.x, + gridDim.x, ...
-  if (pl.conv_w9 == 2 && grid.x > (unsigned)Gfx950::kComputeUnits) grid.x = Gfx950::kComputeUnits;
+  if (pl.conv_w9 == 2 && grid.x > (unsigned)device_compute_units()) grid.x = (unsigned)device_compute_units();
   hipLaunchKernelGGL(inst->fn, grid, dim3(inst->threads), pl.conv_lds, stream, q);
   HIP_TRY(hipGetLastError());
   return 0;

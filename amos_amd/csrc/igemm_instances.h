@@ -73,6 +73,7 @@ struct TnInstance {
   int threads;
   const char* name;
   std::once_flag once;
+  int scratch_bytes = 0;   // per-lane scratch memory of the built kernel, read before its first launch
 };
 // direct-to-LDS GEMM (defined in inst_gemm_tn.hip); 256x256 with 4 or 8 waves, 128x128 / 128x256 /
 // 256x128 with 8

@@ -7,11 +7,35 @@
 // shapes.
 #include "mapper.h"
 
+#include <hip/hip_runtime_api.h>
+
 #include <algorithm>
+#include <atomic>
 #include <cmath>
 #include <cstring>
 
 namespace amos {
+
+int device_compute_units() {
+  constexpr int kMaxDevices = 64;
+  static std::atomic<int> cached[kMaxDevices];   // 0 = not read yet
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) {
+    (void)hipGetLastError();                     // no device: the host-only uses of the mapper
+    return 256;
+  }
+  int cu = cached[dev].load(std::memory_order_relaxed);
+  if (cu == 0) {
+    int v = 0;
+    if (hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || v <= 0) {
+      (void)hipGetLastError();
+      v = 256;
+    }
+    cached[dev].store(v, std::memory_order_relaxed);
+    cu = v;
+  }
+  return cu;
+}
 
 static int64_t conv_out(int64_t in, int pad, int dil, int64_t k, int stride) {
   int64_t eff = (k - 1) * dil + 1;
@@ -164,7 +188,7 @@ bool conv_fewc_plan(const amos_conv_desc_t& c, int op, ConvFewcPlan* out) {
   if (lds > 160 * 1024) return false;
   if (tiles_j * c.N >= (1ll << 31)) return false;
   // one workgroup per CU, shared between the tiles of output channels
-  const int64_t per_ktile = std::max<int64_t>(1, Gfx950::kComputeUnits / k_tiles);
+  const int64_t per_ktile = std::max<int64_t>(1, device_compute_units() / k_tiles);
   const int64_t grid_x = std::min<int64_t>(tiles_j * c.N, per_ktile);
   if (out) {
     out->taps = (int)taps; out->taps_p = (int)taps_p; out->Wp = (int)Wp; out->rows_max = (int)rows_max;
@@ -491,7 +515,7 @@ static ConvPatchPlan conv_patch_plan_waves(const amos_conv_desc_t& cin, int op, 
       // per tile) need a second position table: tables and dump line go behind the used part of
       // each patch buffer where they fit there, behind the second buffer otherwise
       const int64_t tiles = ((c.K + BI - 1) / BI) * ((J + BJ - 1) / BJ);
-      if (allow_w9 >= 2 && !one_macro && split == 1 && tiles > Gfx950::kComputeUnits && !(BI == 128 && BJ == 128)) {
+      if (allow_w9 >= 2 && !one_macro && split == 1 && tiles > device_compute_units() && !(BI == 128 && BJ == 128)) {
         const int xbuf = BI <= 64 ? 64 * 1024 : 48 * 1024;
         const int P = real_pos * 128, TB = real_pos * 8;
         int tab, tab1, dump;
@@ -520,7 +544,7 @@ static ConvPatchPlan conv_patch_plan_waves(const amos_conv_desc_t& cin, int op, 
   // fragments within 256 registers (tiles up to 128x128); pointless when every block already has
   // a CU to itself
   const int64_t blocks = ((c.K + BI - 1) / BI) * ((J + BJ - 1) / BJ) * split;
-  if (waves == 4 && BI <= 128 && BJ <= 128 && blocks > Gfx950::kComputeUnits) {
+  if (waves == 4 && BI <= 128 && BJ <= 128 && blocks > device_compute_units()) {
     int nsw2 = 0, pls2 = 0;
     if (!fit((size_t)79 * 1024, &nsw2, &pls2)) {
       pp.occ = 2;
@@ -612,7 +636,7 @@ static double estimate_seconds(const Problem& pb, int ti, int tj, int split, boo
   const double lf = (direct || repacked) ? 1.0 : loader_factor(pb.row_loader) * loader_factor(pb.col_loader);
   const double tau = tc->tau_us * lf, alone = tc->alone_us * lf;
   const int64_t blocks = ((pb.I + ti - 1) / ti) * ((pb.J + tj - 1) / tj) * pb.batch * eff_split;
-  const int64_t per_cu = (blocks + Gfx950::kComputeUnits - 1) / Gfx950::kComputeUnits;
+  const int64_t per_cu = (blocks + device_compute_units() - 1) / device_compute_units();
   const int64_t groups = per_cu / tc->occ, rest = per_cu % tc->occ;
   double step_us = (double)groups * std::max(alone, tc->occ * tau);
   if (rest) step_us += std::max(alone, (double)rest * tau);
@@ -650,7 +674,7 @@ static double conv_patch_estimate(const amos_conv_desc_t& c, int op, const Probl
   const double blocks = std::ceil((double)pb.I / ti) * std::ceil((double)pb.J / tj) * split;
   // two resident workgroups take turns on the matrix cores while their per-step instruction
   // overheads overlap
-  const double rounds = std::ceil(blocks / (Gfx950::kComputeUnits * (double)pp.occ));
+  const double rounds = std::ceil(blocks / (device_compute_units() * (double)pp.occ));
   const double steps = std::ceil(steps_all / split);
   const double mfma_per_step = (ti / 64.0) * (tj / 64.0) * 4.0 * 32.0;
   // measured (profiles/conv_fprop_kernel_trace.md): a 128x64 step takes ~700 cycles with the taps

@@ -9,9 +9,12 @@ namespace amos {
 
 int set_error(int code, const char* fmt, ...);
 
+// Compute units of the current device (hipGetDeviceProperties, read once per device and kept); with
+// no device visible -- the mapper also runs on hosts without a GPU -- the full MI355X's 256.
+int device_compute_units();
+
 // gfx950 limits the mapper plans against (one workgroup of 4 waves per CU slot)
 struct Gfx950 {
-  static constexpr int kComputeUnits = 256;
   static constexpr int kXcds = 8;
   static constexpr int kLdsBytes = 160 * 1024;      // per CU and per workgroup
   static constexpr int kVgprsPerLane = 512;         // unified VGPR+AGPR file, one wave per SIMD

@@ -32,6 +32,58 @@ def _stream_ptr(stream):
     return ctypes.c_void_p(stream.cuda_stream)
 
 
+_CODE_DTYPE = {_lib.AMOS_F16: torch.float16, _lib.AMOS_BF16: torch.bfloat16, _lib.AMOS_I8: torch.int8,
+               _lib.AMOS_F32: torch.float32, _lib.AMOS_I32: torch.int32}
+
+
+def _gemm_spans(g, batch=1, sa=0, sb=0, sc=0):
+    """elements the three operands of a (batched) GEMM descriptor reach"""
+    a = (g.K - 1) * g.lda + g.M if g.trans_a else (g.M - 1) * g.lda + g.K
+    b = (g.N - 1) * g.ldb + g.K if g.trans_b else (g.K - 1) * g.ldb + g.N
+    c = (g.M - 1) * g.ldc + g.N
+    return (batch - 1) * sa + a, (batch - 1) * sb + b, (batch - 1) * sc + c
+
+
+def operand_spans(op, desc):
+    """(elements of in0, in1, out the kernels may touch, input dtype, output dtype) of a descriptor"""
+    if op == AMOS_OP_GEMM:
+        g, spans = desc, _gemm_spans(desc)
+    elif op == AMOS_OP_BGEMM:
+        g, spans = desc.g, _gemm_spans(desc.g, desc.batch, desc.stride_a, desc.stride_b, desc.stride_c)
+    else:
+        g = desc
+        groups = max(1, desc.groups)
+        xs = (desc.N, desc.C, desc.D, desc.H, desc.W)
+        ws = (desc.K, desc.C // groups, desc.T, desc.R, desc.S)
+        o = conv_out_shape(xs, ws, (desc.stride_d, desc.stride_h, desc.stride_w),
+                           (desc.pad_d, desc.pad_h, desc.pad_w), (desc.dil_d, desc.dil_h, desc.dil_w))
+        prod = lambda t: int(torch.Size(t).numel())
+        spans = (prod(xs), prod(ws), prod(o))
+    return spans, _CODE_DTYPE.get(g.in_dtype), _CODE_DTYPE.get(g.out_dtype)
+
+
+def check_operands(op, desc, in0, in1, out):
+    """Refuse, before any launch, arrays that do not hold what the descriptor says: the kernels
+    take raw pointers, so a short or wrongly typed array would be read or written out of bounds.
+    (The reference's argument binder asserts shape and dtype at call time the same way.)"""
+    (n0, n1, nout), in_dt, out_dt = operand_spans(op, desc)
+    for what, t, need, dt in (("first input", in0, n0, in_dt), ("second input", in1, n1, in_dt),
+                              ("output", out, nout, out_dt)):
+        if t.dtype != dt:
+            raise ValueError("%s is %s, the descriptor says %s" % (what, t.dtype, dt))
+        if t.numel() < need:
+            raise ValueError("%s holds %d elements, the descriptor reaches %d" % (what, t.numel(), need))
+        if t.device != in0.device:
+            raise ValueError("%s is on %s, the first input on %s" % (what, t.device, in0.device))
+
+
+def _check_out(out, shape, dtype, like):
+    """a caller-supplied output: exactly the result's shape and type, on the operands' device"""
+    if tuple(out.shape) != tuple(shape) or out.dtype != dtype or out.device != like.device:
+        raise ValueError("out must be a %s tensor of shape %s on %s: got %s %s on %s"
+                         % (dtype, tuple(shape), like.device, out.dtype, tuple(out.shape), out.device))
+
+
 def make_config(config):
     """None | KernelConfig | dict(tile_i=, tile_j=, split_k=) -> KernelConfig or None"""
     if config is None or isinstance(config, KernelConfig):
@@ -126,10 +178,11 @@ def gemm(a, b, trans_a=False, trans_b=False, out=None, config=None, stream=None,
     if out is None:
         out = torch.empty((M, N), dtype=_OUT_OF[a.dtype], device=a.device)
     _need_device(out)
+    _check_out(out, (M, N), _OUT_OF[a.dtype], a)
     d = gemm_desc(M, N, K, a.dtype, trans_a, trans_b)
     cfg = make_config(config)
     epi = make_epilogue(add, (M, N), out.dtype)
-    ws, ws_ptr, ws_bytes = _workspace(AMOS_OP_GEMM, d, cfg, a.device)
+    ws, ws_ptr, ws_bytes = _workspace(AMOS_OP_GEMM, d, cfg, a.device, stream)
     check(_lib.load().amos_run_fused(AMOS_OP_GEMM, ctypes.byref(d), _cfg_ref(cfg), _epi_ref(epi), a.data_ptr(),
                                      b.data_ptr(), out.data_ptr(), ws_ptr, ws_bytes, _stream_ptr(stream)))
     return out
@@ -154,10 +207,11 @@ def bgemm(a, b, trans_a=False, trans_b=False, out=None, config=None, stream=None
     if out is None:
         out = torch.empty((B, M, N), dtype=_OUT_OF[a.dtype], device=a.device)
     _need_device(out)
+    _check_out(out, (B, M, N), _OUT_OF[a.dtype], a)
     d = bgemm_desc(B, M, N, K, a.dtype, trans_a, trans_b)
     cfg = make_config(config)
     epi = make_epilogue(add, (B, M, N), out.dtype)
-    ws, ws_ptr, ws_bytes = _workspace(AMOS_OP_BGEMM, d, cfg, a.device)
+    ws, ws_ptr, ws_bytes = _workspace(AMOS_OP_BGEMM, d, cfg, a.device, stream)
     check(_lib.load().amos_run_fused(AMOS_OP_BGEMM, ctypes.byref(d), _cfg_ref(cfg), _epi_ref(epi), a.data_ptr(),
                                      b.data_ptr(), out.data_ptr(), ws_ptr, ws_bytes, _stream_ptr(stream)))
     return out
@@ -168,12 +222,19 @@ def workspace_bytes(op, desc, config=None):
     return int(_lib.load().amos_workspace_bytes(op, ctypes.byref(desc), _cfg_ref(cfg)))
 
 
-def _workspace(op, desc, cfg, device):
-    """device scratch of amos_workspace_bytes() (conv: repacked weights); (tensor, ptr, bytes)"""
+def _workspace(op, desc, cfg, device, stream=None):
+    """device scratch of amos_workspace_bytes() (conv: repacked weights); (tensor, ptr, bytes).
+    The tensor is dropped as soon as the asynchronous launch returns, so it is allocated on the
+    launch stream: the caching allocator then hands the block to later work of that stream only,
+    which runs behind the kernel that still reads it."""
     need = _lib.load().amos_workspace_bytes(op, ctypes.byref(desc), _cfg_ref(cfg))
     if need == 0:
         return None, None, 0
-    ws = torch.empty(need + 256, dtype=torch.uint8, device=device)
+    if stream is None:
+        ws = torch.empty(need + 256, dtype=torch.uint8, device=device)
+    else:
+        with torch.cuda.stream(stream):
+            ws = torch.empty(need + 256, dtype=torch.uint8, device=device)
     ptr = (ws.data_ptr() + 255) // 256 * 256
     return ws, ptr, need
 
@@ -217,9 +278,10 @@ def conv2d(x, w, stride=1, pad=0, dil=1, out=None, config=None, stream=None, add
     if out is None:
         out = torch.empty(stored_conv_out_shape(oshape, layout, 4), dtype=_OUT_OF[x.dtype], device=x.device)
     _need_device(out)
+    _check_out(out, stored_conv_out_shape(oshape, layout, 4), _OUT_OF[x.dtype], x)
     d = conv_desc(xs, ws, x.dtype, st, pd, dl, groups, layout)
     cfg = make_config(config)
-    ws, ws_ptr, ws_bytes = _workspace(AMOS_OP_CONV2D, d, cfg, x.device)
+    ws, ws_ptr, ws_bytes = _workspace(AMOS_OP_CONV2D, d, cfg, x.device, stream)
     epi = make_epilogue(add, tuple(out.shape), out.dtype)
     check(_lib.load().amos_run_fused(AMOS_OP_CONV2D, ctypes.byref(d), _cfg_ref(cfg), _epi_ref(epi), x.data_ptr(),
                                      w.data_ptr(), out.data_ptr(), ws_ptr, ws_bytes, _stream_ptr(stream)))
@@ -239,9 +301,10 @@ def conv3d(x, w, stride=1, pad=0, dil=1, out=None, config=None, stream=None, add
     if out is None:
         out = torch.empty(stored_conv_out_shape(oshape, layout, 5), dtype=_OUT_OF[x.dtype], device=x.device)
     _need_device(out)
+    _check_out(out, stored_conv_out_shape(oshape, layout, 5), _OUT_OF[x.dtype], x)
     d = conv_desc(xs, ws, x.dtype, st, pd, dl, groups, layout)
     cfg = make_config(config)
-    ws, ws_ptr, ws_bytes = _workspace(AMOS_OP_CONV3D, d, cfg, x.device)
+    ws, ws_ptr, ws_bytes = _workspace(AMOS_OP_CONV3D, d, cfg, x.device, stream)
     epi = make_epilogue(add, tuple(out.shape), out.dtype)
     check(_lib.load().amos_run_fused(AMOS_OP_CONV3D, ctypes.byref(d), _cfg_ref(cfg), _epi_ref(epi), x.data_ptr(),
                                      w.data_ptr(), out.data_ptr(), ws_ptr, ws_bytes, _stream_ptr(stream)))
@@ -360,8 +423,9 @@ def run_desc(op, desc, in0, in1, out, config=None, stream=None, add=None):
     """launch an op from its C descriptor (leading dimensions and batch strides as the descriptor
     says; the tensors only supply the device memory)"""
     _need_device(in0, in1, out)
+    check_operands(op, desc, in0, in1, out)
     cfg = make_config(config)
-    ws, ws_ptr, ws_bytes = _workspace(op, desc, cfg, in0.device)
+    ws, ws_ptr, ws_bytes = _workspace(op, desc, cfg, in0.device, stream)
     epi = _epilogue_for(op, desc, add, out)
     check(_lib.load().amos_run_fused(op, ctypes.byref(desc), _cfg_ref(cfg), _epi_ref(epi), in0.data_ptr(),
                                      in1.data_ptr(), out.data_ptr(), ws_ptr, ws_bytes, _stream_ptr(stream)))
@@ -372,9 +436,10 @@ def time_op(op, desc, in0, in1, out, config=None, number=100, repeat=1, min_repe
             add=None):
     """mean seconds per launch, `repeat` values (time_evaluator semantics)"""
     _need_device(in0, in1, out)
+    check_operands(op, desc, in0, in1, out)
     cfg = make_config(config)
     res = (ctypes.c_double * repeat)()
-    ws, ws_ptr, ws_bytes = _workspace(op, desc, cfg, in0.device)
+    ws, ws_ptr, ws_bytes = _workspace(op, desc, cfg, in0.device, stream)
     epi = _epilogue_for(op, desc, add, out)
     check(_lib.load().amos_time_fused(op, ctypes.byref(desc), _cfg_ref(cfg), _epi_ref(epi), in0.data_ptr(),
                                       in1.data_ptr(), out.data_ptr(), ws_ptr, ws_bytes, _stream_ptr(stream),

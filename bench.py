@@ -3,7 +3,9 @@ on one MI355X, next to the CPU restatement of the reference's llvm path timed in
 
   python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--report FILE] [--model-check FILE]
 
-A step is one launch of the GEMM over device-resident operands.  Prints ONE JSON line.
+A step is one launch of the GEMM over device-resident operands.  Prints ONE JSON line; its
+`config.per_op` holds the other configurations of the path (fp16 / int8 conv2d, batched GEMM,
+conv3d), each timed in the same run next to the CPU loop nest on a slab of the same workload.
 `--report FILE` additionally times every configuration of the path (GEMM, batched GEMM,
 conv2d fp16 / int8, conv3d) and writes a per-config table as JSON to FILE.
 """
@@ -18,12 +20,43 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 METRIC = "TFLOP/s + % of MFMA peak per op (fp16 conv2d/GEMM, int8 TOP/s), 1 MI355X"
-PEAK_F16_TFLOPS = 2500.0   # published dense fp16 MFMA peak of MI355X
-PEAK_I8_TOPS = 5000.0      # published dense int8 peak
-PEAK_HBM_GBS = 8000.0      # published HBM3E bandwidth
-# bytes beyond L2 per launch, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this command,
-# each scaled by the same counter's reading for a 256 MiB device copy (x2.0 and x1.0)
-MEASURED_TRAFFIC = {"amos_gemm_tn<f16,256x256,8w>": 793010 * 1024 * 2.0 + 305010 * 1024 * 1.0}
+# MI355X's published dense fp16 / int8 MFMA peaks and HBM3E bandwidth
+from amos_amd.auto_tensorize.target import PEAK_F16_TFLOPS, PEAK_HBM_GBS, PEAK_I8_TOPS  # noqa: E402
+
+
+def kernel_source_hash(files):
+    """first 12 hex digits of the sha256 over the named kernel sources (relative to the repository)"""
+    import hashlib
+    h = hashlib.sha256()
+    for f in files:
+        with open(os.path.join(ROOT, f), "rb") as fh:
+            h.update(fh.read())
+    return h.hexdigest()[:12]
+
+
+def measured_traffic(kernel_name):
+    """HBM bytes per launch of `kernel_name` from the counter summaries under profiles/: a summary
+    carries a line `traffic_json: {...}` with the kernel's name, the two counter readings (KiB per
+    dispatch), the factors a plain copy of known size gave for them, and the hash of the kernel's
+    sources at the time of the run.  Returns None when no summary names this kernel or its sources
+    have changed since (the figure would describe a kernel that no longer ships)."""
+    pdir = os.path.join(ROOT, "profiles")
+    if not os.path.isdir(pdir):
+        return None
+    for fn in sorted(os.listdir(pdir)):
+        if not fn.endswith(".md"):
+            continue
+        for line in open(os.path.join(pdir, fn)):
+            if not line.startswith("traffic_json:"):
+                continue
+            try:
+                rec = json.loads(line[len("traffic_json:"):])
+                if rec["kernel"] != kernel_name or rec["source_hash"] != kernel_source_hash(rec["sources"]):
+                    continue
+                return (rec["fetch_kib"] * rec["fetch_scale"] + rec["write_kib"] * rec["write_scale"]) * 1024.0
+            except (ValueError, KeyError, OSError):
+                continue
+    return None
 
 
 def cpu_baseline_gemm(a, b, seconds_budget=12.0):
@@ -79,7 +112,7 @@ def run_all_configs(cpu=True, only=None):
         return min(t), cfg
 
     def add(name, op, desc, hin, dtype, flop, nbytes, out_shape, cpu_fn, frac, fused_tail=False):
-        if only and only not in name:
+        if only and not any(o in name for o in ([only] if isinstance(only, str) else only)):
             return
         tin = [(torch.from_numpy(h) if isinstance(h, np.ndarray) else h).cuda() for h in hin]
         out = torch.empty(out_shape, dtype=torch.int32 if dtype == "int8" else torch.float32,
@@ -310,6 +343,8 @@ def main():
     ap.add_argument("--steps", type=int, default=100)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU-baseline leg")
+    ap.add_argument("--no-per-op", action="store_true",
+                    help="skip the per-configuration table (conv2d fp16 / int8, batched GEMM, conv3d)")
     ap.add_argument("--report", default=None, help="also time every config, write JSON here")
     ap.add_argument("--report-only", default=None,
                     help="restrict --report to the configurations whose name contains this text")
@@ -379,11 +414,36 @@ def main():
                    "pct_of_mfma_peak": 100.0 * value / PEAK_F16_TFLOPS},
         "roofline": {"bound": "mfma", "achieved": achieved, "peak": PEAK_F16_TFLOPS,
                      "unit": "TFLOP/s", "frac": achieved / PEAK_F16_TFLOPS,
-                     "traffic": MEASURED_TRAFFIC.get(ops.kernel_name(_lib.AMOS_OP_GEMM, desc, cfg)),
+                     "traffic": measured_traffic(ops.kernel_name(_lib.AMOS_OP_GEMM, desc, cfg)),
                      "kernel_us": per_launch * 1e6},
     }
     if not args.no_cpu:
         line["cpu_baseline"] = cpu_baseline_gemm(a, b)
+    if not args.no_per_op:
+        # every configuration of the path in the same run, each next to the CPU loop nest on a slab
+        # of the same workload: the 8192^3 product from the measurement above, the others timed here
+        del da, db, dc
+        torch.cuda.empty_cache()
+        per_op = [{"config": "C2 fp16 GEMM 8192^3 (ntn)", "kernel": line["config"]["kernel"],
+                   "gpu_us": per_launch * 1e6, "tflops": achieved,
+                   "pct_mfma_peak": 100 * achieved / PEAK_F16_TFLOPS,
+                   "pct_hbm_roof": 100 * (2 * n * n * 2 + n * n * 4) / (PEAK_HBM_GBS * 1e9) / per_launch,
+                   "bound": "mfma"}]
+        if "cpu_baseline" in line:
+            cb = line["cpu_baseline"]
+            per_op[0]["cpu"] = {"threads1_tflops": cb["value"], "threadsN_tflops": cb["all_cores"]["value"],
+                                "cores": cb["all_cores"]["cores"], "extrapolated_from": cb["sample"].split("=")[-1]}
+        for r in run_all_configs(cpu=not args.no_cpu, only=("C3 fp16", "C4 int8", "C5a fp16", "C5b fp16")):
+            row = {k: r[k] for k in ("config", "kernel", "split_k", "gpu_us", "tflops", "pct_mfma_peak",
+                                     "pct_hbm_roof", "bound")}
+            if "cpu" in r:
+                row["cpu"] = {k: r["cpu"][k] for k in ("threads1_tflops", "threadsN_tflops", "cores",
+                                                       "extrapolated_from")}
+            per_op.append(row)
+        line["config"]["per_op"] = per_op
+        line["config"]["per_op_note"] = ("gpu_us: mean seconds per call by HIP events (time_evaluator loop), every "
+                                         "launch of a call included; tflops: TFLOP/s (int8: TOP/s); cpu: the "
+                                         "te_literal loop nest (gcc -O3) on a slab, scaled linearly")
     if args.report:
         with open(args.report, "w") as f:
             json.dump(run_all_configs(cpu=not args.no_cpu, only=args.report_only), f, indent=1)

@@ -122,3 +122,59 @@ def test_kernel_name_reflects_layout():
     assert lib.amos_kernel_name(2, ctypes.byref(c), ctypes.byref(cfg)) == b"amos_igemm<i8,vec,im2col,128x128>"
     c.R = 20   # window larger than the padded input
     assert lib.amos_kernel_name(2, ctypes.byref(c), ctypes.byref(cfg)) is None
+
+
+def test_wrong_arrays_are_refused_before_any_launch():
+    """The kernels take raw pointers; an `out` (or an input) of the wrong extent or element type
+    must never reach them.  These checks run on host tensors: nothing is launched."""
+    import torch
+    from amos_amd import ops
+    like = torch.empty(4, 8, dtype=torch.float16)
+    ops._check_out(torch.empty(4, 6), (4, 6), torch.float32, like)
+    with pytest.raises(ValueError, match="shape"):
+        ops._check_out(torch.empty(4, 5), (4, 6), torch.float32, like)
+    with pytest.raises(ValueError, match="float32"):
+        ops._check_out(torch.empty(4, 6, dtype=torch.float16), (4, 6), torch.float32, like)
+    d = ops.gemm_desc(4, 6, 8, torch.float16, False, True)
+    a, b = torch.empty(4, 8, dtype=torch.float16), torch.empty(6, 8, dtype=torch.float16)
+    ops.check_operands(_lib.AMOS_OP_GEMM, d, a, b, torch.empty(4, 6))
+    with pytest.raises(ValueError, match="output holds 20 elements"):
+        ops.check_operands(_lib.AMOS_OP_GEMM, d, a, b, torch.empty(4, 5))
+    with pytest.raises(ValueError, match="output is torch.float16"):
+        ops.check_operands(_lib.AMOS_OP_GEMM, d, a, b, torch.empty(4, 6, dtype=torch.float16))
+    with pytest.raises(ValueError, match="second input holds"):
+        ops.check_operands(_lib.AMOS_OP_GEMM, d, a, b[:5], torch.empty(4, 6))
+    # leading dimensions and batch strides count
+    bd = ops.bgemm_desc(3, 4, 6, 8, torch.float16, False, True)
+    bd.stride_c = 100
+    assert ops.operand_spans(_lib.AMOS_OP_BGEMM, bd)[0] == (3 * 32, 3 * 48, 2 * 100 + 24)
+    cd = ops.conv_desc((2, 8, 1, 5, 5), (4, 8, 1, 3, 3), torch.int8, (1, 1, 1), (0, 1, 1), (1, 1, 1))
+    spans, in_dt, out_dt = ops.operand_spans(_lib.AMOS_OP_CONV2D, cd)
+    assert spans == (2 * 8 * 25, 4 * 8 * 9, 2 * 4 * 25) and in_dt == torch.int8 and out_dt == torch.int32
+    with pytest.raises(ValueError, match="output is torch.float32"):
+        ops.check_operands(_lib.AMOS_OP_CONV2D, cd, torch.empty(400, dtype=torch.int8),
+                           torch.empty(288, dtype=torch.int8), torch.empty(200))
+
+
+def test_module_refuses_arrays_that_are_not_the_declared_tensors():
+    import torch
+    from amos_amd import te
+    from amos_amd.auto_tensorize import runtime
+    from amos_amd.auto_tensorize.hw_abstraction import compute_dag_from_tensors
+    from amos_amd.auto_tensorize.lowering import lower_main_op
+    A = te.placeholder([32, 64], dtype="float16", name="A")
+    B = te.placeholder([64, 48], dtype="float16", name="B")
+    k = te.reduce_axis([0, 64], name="k")
+    C = te.compute([32, 48], lambda i, j: te.sum((A[i, k] * B[k, j]).astype("float32"), axis=k), name="C")
+    dag = compute_dag_from_tensors([C])
+    lowered = lower_main_op([op for op in dag.op_lst if op.reduce_axis][0], dag)
+    mod = runtime.Module(lowered, None, [A, B, C])
+    a, b = torch.empty(32, 64, dtype=torch.float16), torch.empty(64, 48, dtype=torch.float16)
+    with pytest.raises(ValueError, match="declared float32"):
+        mod(a, b, torch.empty(32, 40))                              # short output
+    with pytest.raises(ValueError, match="declared float32"):
+        mod(a, b, torch.empty(32, 48, dtype=torch.float16))        # fp16 output
+    with pytest.raises(ValueError, match="declared float16"):
+        mod(a.float(), b, torch.empty(32, 48))                      # float32 input wrapped by array()
+    with pytest.raises(ValueError, match="device array"):
+        mod(a, b, torch.empty(32, 48))                              # right shapes, but host memory

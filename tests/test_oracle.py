@@ -82,6 +82,87 @@ def test_gemm_loop_nest_bit_exact_vs_brute_force(dtype, ta, tb):
         assert np.array_equal(got, brute_gemm(a, b, dtype, ta, tb, literal)), (mode, ta, tb)
 
 
+def _bf16_round(x):
+    """float32 -> nearest bfloat16 (ties to even), returned as float32: torch-CPU's conversion"""
+    import torch
+    return torch.tensor([float(x)], dtype=torch.float32).to(torch.bfloat16).float().numpy()[0]
+
+
+@pytest.mark.parametrize("ta,tb", list(itertools.product([0, 1], [0, 1])))
+def test_bf16_gemm_loop_nest_bit_exact_vs_brute_force(ta, tb):
+    """te_literal mode multiplies in bf16 (the product rounded to bf16 by torch-CPU here), widens,
+    accumulates sequentially in fp32; exact mode keeps the fp32 product"""
+    rng = np.random.default_rng(31)
+    M, N, K = 4, 5, 9
+    a = make_operand(rng, (K, M) if ta else (M, K), "bfloat16")
+    b = make_operand(rng, (N, K) if tb else (K, N), "bfloat16")
+    fa, fb = co.bf16_bits_to_float(a), co.bf16_bits_to_float(b)
+    rounded_somewhere = False
+    for mode in ("te_literal", "exact"):
+        want = np.zeros((M, N), dtype=np.float32)
+        for m in range(M):
+            for n in range(N):
+                acc = np.float32(0)
+                for k in range(K):
+                    x = fa[k, m] if ta else fa[m, k]
+                    y = fb[n, k] if tb else fb[k, n]
+                    p = np.float32(x) * np.float32(y)          # exact in fp32: 8-bit significands
+                    if mode == "te_literal":
+                        rounded_somewhere |= bool(_bf16_round(p) != p)
+                        p = np.float32(_bf16_round(p))
+                    acc = np.float32(acc + p)
+                want[m, n] = acc
+        assert np.array_equal(co.te_literal_gemm(a, b, "bfloat16", ta, tb, mode=mode), want), (mode, ta, tb)
+    assert rounded_somewhere   # the two modes were told apart by this data
+
+
+def brute_conv(x, w, dtype, stride, pad, dil, literal):
+    """pure-Python statement of the conv loop nest: padded tensor materialised first, reduction
+    rc outermost then rd, rr, rs, product in the input type (te_literal) or exact"""
+    N, C, D, H, W = x.shape
+    K, _, T, R, S = w.shape
+    (sd, sh, sw), (pd, ph, pw), (dd, dh, dw) = stride, pad, dil
+    if dtype == "bfloat16":
+        x, w = co.bf16_bits_to_float(x), co.bf16_bits_to_float(w)
+    xp = np.zeros((N, C, D + 2 * pd, H + 2 * ph, W + 2 * pw), dtype=x.dtype)
+    xp[:, :, pd:pd + D, ph:ph + H, pw:pw + W] = x
+    OD = (D + 2 * pd - (T - 1) * dd - 1) // sd + 1
+    OP = (H + 2 * ph - (R - 1) * dh - 1) // sh + 1
+    OQ = (W + 2 * pw - (S - 1) * dw - 1) // sw + 1
+    out = np.zeros((N, K, OD, OP, OQ), dtype=np.int32 if dtype == "int8" else np.float32)
+    for n, k, od, op, oq in itertools.product(range(N), range(K), range(OD), range(OP), range(OQ)):
+        acc = np.int32(0) if dtype == "int8" else np.float32(0)
+        for c, t, r, s_ in itertools.product(range(C), range(T), range(R), range(S)):
+            a = xp[n, c, od * sd + t * dd, op * sh + r * dh, oq * sw + s_ * dw]
+            b = w[k, c, t, r, s_]
+            if dtype == "int8":
+                p = np.int32(np.int8((int(a) * int(b) + 128) % 256 - 128)) if literal else np.int32(int(a) * int(b))
+            elif dtype == "float16":
+                p = np.float32(np.float16(np.float32(a) * np.float32(b))) if literal else np.float32(a) * np.float32(b)
+            else:
+                p = np.float32(a) * np.float32(b)
+                p = np.float32(_bf16_round(p)) if literal else p
+            acc = acc + p if dtype == "int8" else np.float32(acc + p)
+        out[n, k, od, op, oq] = acc
+    return out
+
+
+@pytest.mark.parametrize("dtype", ["float16", "bfloat16", "int8"])
+@pytest.mark.parametrize("case", [((1, 2, 1, 4, 5), (2, 2, 1, 3, 3), (1, 1, 1), (0, 1, 1), (1, 1, 1)),
+                                  ((1, 2, 3, 4, 4), (2, 2, 2, 3, 2), (1, 2, 1), (1, 1, 0), (1, 1, 2))])
+def test_conv_loop_nest_bit_exact_vs_brute_force_in_both_modes(dtype, case):
+    """the conv oracle in te_literal mode (and in exact mode) against a Python loop nest on shapes
+    small enough for one: the same padding, the same reduce order, the same rounding of products"""
+    xs, ws, stride, pad, dil = case
+    rng = np.random.default_rng(32)
+    x, w = make_operand(rng, xs, dtype), make_operand(rng, ws, dtype)
+    lit = co.te_literal_conv3d(x, w, dtype, stride, pad, dil, mode="te_literal")
+    exact = co.te_literal_conv3d(x, w, dtype, stride, pad, dil, mode="exact")
+    assert np.array_equal(lit, brute_conv(x, w, dtype, stride, pad, dil, True))
+    assert np.array_equal(exact, brute_conv(x, w, dtype, stride, pad, dil, False))
+    assert not np.array_equal(lit, exact)   # the data tells the two modes apart
+
+
 def test_int8_wraparound_mode_differs_and_matches_closed_form():
     """(a*b).astype(int32) on int8 wraps before widening in the reference's llvm build"""
     a = np.array([[127, -128, 100, 3]], dtype=np.int8)
