@@ -8,7 +8,7 @@ LIB_PATH = os.path.join(_HERE, "libamos_mi355x.so")
 AMOS_F16, AMOS_BF16, AMOS_I8, AMOS_F32, AMOS_I32 = range(5)
 AMOS_OP_GEMM, AMOS_OP_BGEMM, AMOS_OP_CONV2D, AMOS_OP_CONV3D = range(4)
 
-AMOS_PIPE_AUTO, AMOS_PIPE_STAGED, AMOS_PIPE_DIRECT4, AMOS_PIPE_DIRECT8, AMOS_PIPE_PATCH, AMOS_PIPE_PATCH8 = range(6)
+AMOS_PIPE_AUTO, AMOS_PIPE_STAGED, AMOS_PIPE_DIRECT4, AMOS_PIPE_DIRECT8, AMOS_PIPE_PATCH, AMOS_PIPE_PATCH8, AMOS_PIPE_NCHW = range(7)
 
 AMOS_ERR_BAD_ARG = -1
 AMOS_ERR_UNSUPPORTED = -2

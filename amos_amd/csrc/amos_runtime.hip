@@ -11,6 +11,7 @@
 #include "amos_mi355x.h"
 #include "conv_fprop_kernel.h"
 #include "conv_fewc_kernel.h"
+#include "conv_nchw_kernel.h"
 #include "depthwise_kernel.h"
 #include "gemm_tn_kernel.h"
 #include "igemm_instances.h"
@@ -328,6 +329,11 @@ struct Plan {
   int fewc;
   ConvFewcParams fcp;
   size_t fewc_lds;
+  // convolution read straight from NCDHW / KCTRS (0 = not used)
+  int nchw;
+  int nchw_t1;
+  ConvNchwParams nc;
+  size_t nchw_lds;
 };
 
 static int dtype_pair(int in_dtype, int out_dtype, int* dt) {
@@ -738,6 +744,42 @@ static int plan_conv(Plan& pl, int op, const amos_conv_desc_t* d, const amos_ker
       return 0;
     }
   }
+  // Named explicitly: the kernel that reads NCDHW / KCTRS as they are (one launch, no workspace)
+  if (cfg && cfg->pipeline == AMOS_PIPE_NCHW) {
+    const int BI = cfg->tile_i > 0 ? cfg->tile_i : 64;
+    const int BJ = cfg->tile_j > 0 ? cfg->tile_j : 128;
+    ConvNchwPlan np = conv_nchw_plan(c, op, BI, BJ);
+    const char* why = np.why;
+    if (!why && ((uintptr_t)X & 7)) why = "activations not 8-byte aligned";
+    if (!why && cfg->split_k > 1) why = "no split-K in this pipeline";
+    if (why) return set_error(AMOS_ERR_INFEASIBLE, "NCDHW-direct convolution not applicable: %s", why);
+    ConvNchwParams& q = pl.nc;
+    memset(&q, 0, sizeof(q));
+    q.x = (const char*)X; q.w = (const char*)Wt; q.y = (char*)Y;
+    conv_nchw_shape(c, op, &q.s);
+    const int es1 = pl.dt == DT_I8 ? 1 : 2;
+    q.c_chunks = (int)(c.C * es1 / 64);
+    q.macro_steps = q.s.T * q.c_chunks;
+    q.macro_per_split = q.macro_steps;
+    q.tiles_i = (int)((c.K + BI - 1) / BI);
+    q.tiles_j = (int)((J + BJ - 1) / BJ);
+    q.max_pos = np.max_pos;
+    q.split_stride = 0;
+    q.div_cc = nchw_make_div((uint32_t)q.c_chunks);
+    q.div_odpq = nchw_make_div((uint32_t)(OD * OP * OQ));
+    pl.nchw = 1;
+    pl.nchw_t1 = np.t1 && aligned16(Wt);
+    pl.nchw_lds = np.lds;
+    memset(&pl.cfg, 0, sizeof(pl.cfg));
+    pl.cfg = *cfg;
+    pl.cfg.tile_i = BI; pl.cfg.tile_j = BJ; pl.cfg.split_k = 1;
+    memset(&pl.p, 0, sizeof(pl.p));
+    pl.p.out_si = (int64_t)OD * OP * OQ;     // (the fused tail's operand is laid out like the output)
+    pl.p.out_batch = 0;
+    pl.batch = 1;
+    pl.split = 1;
+    return 0;
+  }
   const int es = pl.dt == DT_I8 ? 1 : 2;
   const int ce = 16 / es;
   IgemmParams& p = pl.p;
@@ -896,6 +938,7 @@ static int make_plan(Plan& pl, int op, const void* desc, const amos_kernel_confi
   pl.im2col = 0;
   pl.fewc = 0;
   pl.skinny = 0;
+  pl.nchw = 0;
   switch (op) {
     case AMOS_OP_GEMM:
       return plan_gemm(pl, op, desc, (const amos_gemm_desc_t*)desc, 1, 0, 0, 0, cfg, in0, in1, out, workspace,
@@ -981,7 +1024,39 @@ static int launch_conv(const Plan& pl, hipStream_t stream) {
   return 0;
 }
 
+static ConvNchwInstance* pick_conv_nchw(int dt, int ti, int tj, int t1) {
+  if (dt == DT_F16) return pick_conv_nchw_f16(ti, tj, t1);
+  if (dt == DT_BF16) return pick_conv_nchw_bf16(ti, tj, t1);
+  return pick_conv_nchw_i8(ti, tj, t1);
+}
+
+static int launch_conv_nchw(const Plan& pl, hipStream_t stream) {
+  ConvNchwInstance* inst = pick_conv_nchw(pl.dt, pl.cfg.tile_i, pl.cfg.tile_j, pl.nchw_t1);
+  if (!inst) return set_error(AMOS_ERR_INFEASIBLE, "no NCDHW-direct convolution instance");
+  hipError_t attr_err = hipSuccess;
+  std::call_once(inst->once, [&] {
+    attr_err = hipFuncSetAttribute((const void*)inst->fn, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                   160 * 1024 - 1024);
+    hipFuncAttributes fa;
+    if (attr_err == hipSuccess) attr_err = hipFuncGetAttributes(&fa, (const void*)inst->fn);
+    if (attr_err == hipSuccess) inst->scratch_bytes = (int)fa.localSizeBytes;
+  });
+  if (attr_err != hipSuccess)
+    return set_error(AMOS_ERR_HIP, "hipFuncSetAttribute(%s): %s", inst->name, hipGetErrorString(attr_err));
+  const ConvNchwParams& q = pl.nc;
+  // what the kernel assumes of its launch: the tile of the instance, whole 64-byte chunks of
+  // channels, a patch that fits the LDS asked for
+  if (inst->bi != pl.cfg.tile_i || inst->bj != pl.cfg.tile_j || q.c_chunks < 1 || q.max_pos < 4 ||
+      pl.nchw_lds != (size_t)2 * 9 * inst->bi * 64 + (size_t)2 * q.max_pos * kNchwPosBytes)
+    return set_error(AMOS_ERR_BAD_ARG, "inconsistent plan for %s", inst->name);
+  dim3 grid((unsigned)(q.tiles_i * q.tiles_j), (unsigned)pl.split, 1);
+  hipLaunchKernelGGL(inst->fn, grid, dim3(inst->threads), pl.nchw_lds, stream, q);
+  HIP_TRY(hipGetLastError());
+  return 0;
+}
+
 static int launch(const Plan& pl, hipStream_t stream) {
+  if (pl.nchw) return launch_conv_nchw(pl, stream);
   if (pl.im2col) {
     const unsigned want = (pl.icp.total + 255u) / 256u;
     dim3 grid(want < (1u << 20) ? want : (1u << 20));
@@ -1084,6 +1159,7 @@ static int plan_epilogue(Plan& pl, int op, const void* desc, const amos_epilogue
   pl.cv.epi = ep;
   pl.dwp.epi = ep;
   pl.fcp.epi = ep;
+  pl.nc.epi = ep;
   pl.sk.epi = ep;
   pl.sk.epi_s_big = pl.skinny_big_is_a ? ep.si : 1;
   pl.sk.epi_s_small = pl.skinny_big_is_a ? 1 : ep.si;
@@ -1331,6 +1407,7 @@ size_t amos_workspace_bytes(int op, const void* desc, const amos_kernel_config_t
     return (size_t)gemm_repack(b->g, b->batch, false, false).total();
   }
   if (op != AMOS_OP_CONV2D && op != AMOS_OP_CONV3D) return 0;
+  if (cfg && cfg->pipeline == AMOS_PIPE_NCHW) return 0;   // reads the caller's tensors as they are
   const amos_conv_desc_t& c = *(const amos_conv_desc_t*)desc;
   int64_t need = conv_workspace_bytes(c, op);
   // a pointwise convolution runs as a matrix product; its row-contiguous operand (NCDHW
@@ -1363,6 +1440,10 @@ const char* amos_kernel_name(int op, const void* desc, const amos_kernel_config_
   // amos_workspace_bytes() gets
   static char dummy_ws[256] __attribute__((aligned(256)));
   if (make_plan(pl, op, desc, cfg, dummy, dummy, dummy, dummy_ws, (size_t)-1)) return nullptr;
+  if (pl.nchw) {
+    ConvNchwInstance* ni = pick_conv_nchw(pl.dt, pl.cfg.tile_i, pl.cfg.tile_j, pl.nchw_t1);
+    return ni ? ni->name : nullptr;
+  }
   if (pl.dw) return depthwise_name(pl.dt, pl.dw - 1);
   if (pl.fewc) return conv_fewc_name(pl.dt);
   if (pl.skinny) return skinny_gemm_name(pl.dt);

@@ -1,0 +1,205 @@
+// Geometry of the convolution kernel that reads NCDHW activations and KCTRS weights as they are
+// (conv_nchw_kernel.h): which input positions a tile of output positions touches, where each of
+// them sits in the LDS patch, which thread fetches it, and where a lane finds the operand of an
+// output position at a window tap.  Plain integer functions shared by the kernel, the host-side
+// planner (LDS and task budgets) and a CPU check that every reader address meets the element a
+// writer put there.
+//
+// A tile is BJ consecutive output positions j = ((n * OD + od) * OP + op) * OQ + oq and may touch
+// up to kNchwMaxSeg (image, output depth) slices.  Per slice the patch is a zero-padded window
+// [rows][Wp] of input positions, 64 bytes of channels each (32 halves / 64 int8: one matrix-core
+// K sub-step).  A window tap (r, s) only shifts the position a lane reads: by r * dil_h rows and
+// s * dil_w columns.
+//
+// Bank conflicts: a 64-byte position holds four 16-byte chunks; chunk c of position P is stored at
+// chunk c ^ ((key(P) >> 2) & 3), key(P) = P with the row pitch Wp replaced by key_pitch.  With unit
+// strides key_pitch = OQ, so the sixteen consecutive output positions of a fragment read have
+// sixteen consecutive keys also where they wrap into the next patch row, and, Wp - OQ being a
+// multiple of 4, hit sixteen different 16-byte bank groups at any tap.
+#pragma once
+#include <stdint.h>
+
+#if defined(__HIPCC__) || defined(__CUDACC__)
+#define AMOS_HD __host__ __device__ __forceinline__
+#else
+#define AMOS_HD inline
+#endif
+
+namespace amos {
+
+constexpr int kNchwMaxSeg = 4;
+constexpr int kNchwPosBytes = 64;   // bytes of channels per patch position and macro step
+
+// n / d for 0 <= n < 2^31 by a multiplication with a host-built constant (the extents are known
+// when the kernel is launched; a hardware-less integer division costs dozens of instructions)
+struct NchwDiv {
+  uint32_t magic, shift, one, d;
+};
+inline NchwDiv nchw_make_div(uint32_t d) {
+  NchwDiv f = {0, 0, 0, d};
+  if (d <= 1) { f.one = 1; return f; }
+  uint32_t l = 0;
+  while ((1ull << l) < d) ++l;
+  const uint64_t sft = 31 + l;
+  f.magic = (uint32_t)(((1ull << sft) + d - 1) / d);
+  f.shift = (uint32_t)(sft - 32);
+  return f;
+}
+AMOS_HD int nchw_div(int n, const NchwDiv& f) {
+  const uint32_t hi = (uint32_t)(((uint64_t)(uint32_t)n * f.magic) >> 32);
+  return (int)((hi + (uint32_t)n * f.one) >> f.shift);
+}
+
+struct NchwShape {
+  int N, C, D, H, W, K, T, R, S;
+  int sd, sh, sw, pd, ph, pw, dd, dh, dw;
+  int OD, OP, OQ;
+  int J;           // N * OD * OP * OQ
+  int Wp;          // patch row pitch in positions
+  int key_pitch;   // row pitch of the swizzle key
+  int pg_shift;    // log2 of the input positions per 8-byte load: 2 (16-bit types) or 3 (int8)
+  NchwDiv div_opq, div_oq, div_w, div_od;
+};
+
+// patch row pitch: the columns a row of outputs touches, rounded so that Wp - OQ is a multiple of 4
+// where the key compaction applies
+AMOS_HD int nchw_patch_pitch(int OQ, int S, int sw, int dw, int sh) {
+  int wp = (OQ - 1) * sw + (S - 1) * dw + 1;
+  if (sw == 1 && sh == 1) wp += (4 - ((wp - OQ) & 3)) & 3;
+  return wp;
+}
+AMOS_HD int nchw_key_pitch(int OQ, int Wp, int sw, int sh) { return (sw == 1 && sh == 1) ? OQ : Wp; }
+
+struct NchwSeg {
+  int pos0;      // first LDS position of the slice's window (multiple of 4)
+  int pa;        // first output row of the tile in this slice
+  int h_first;   // input row of window row 0 (may be negative: padding)
+  int n, d0;     // image, input depth of depth tap 0 (may be out of range: padding)
+  int flo, fhi;  // flat in-plane range [flo, fhi) of the input positions that exist (h * W + w)
+  int glo;       // first load group: flo / pg
+  int grp0;      // groups of the slices before this one
+  int rows;      // window rows
+};
+
+// per-slice fields as 4-element vectors: a lane-dependent slice index then becomes a chain of
+// selects (an array inside the struct would put the whole tile into scratch memory on the GPU)
+typedef int nchw_i4 __attribute__((vector_size(16)));
+struct NchwTile {
+  int bj0, j_last, sl_a, nseg;
+  int npos;      // LDS positions used
+  int ngroups;   // load groups of all slices
+  nchw_i4 pos0, pa, h_first, n, d0, flo, fhi, glo, grp0, rows;   // NchwSeg's fields, one element per slice
+};
+static_assert(kNchwMaxSeg == 4, "NchwTile holds four slices");
+
+// nseg > kNchwMaxSeg is reported as it is; only the first kNchwMaxSeg slices are filled
+AMOS_HD NchwTile nchw_tile(const NchwShape& s, int bj0, int BJ) {
+  NchwTile t;
+  const int OPQ = s.OP * s.OQ;
+  const int pg = 1 << s.pg_shift;
+  t.bj0 = bj0;
+  t.j_last = bj0 + BJ - 1 < s.J ? bj0 + BJ - 1 : s.J - 1;
+  t.sl_a = nchw_div(bj0, s.div_opq);
+  const int sl_b = nchw_div(t.j_last, s.div_opq);
+  t.nseg = sl_b - t.sl_a + 1;
+  int pos = 0, grp = 0;
+#pragma unroll
+  for (int g = 0; g < kNchwMaxSeg; ++g) {
+    const bool live = g < t.nseg;
+    const int sl = t.sl_a + (live ? g : t.nseg - 1);
+    const int lo = bj0 > sl * OPQ ? bj0 : sl * OPQ;
+    const int hi = t.j_last < (sl + 1) * OPQ - 1 ? t.j_last : (sl + 1) * OPQ - 1;
+    const int pa = nchw_div(lo - sl * OPQ, s.div_oq), pb = nchw_div(hi - sl * OPQ, s.div_oq);
+    const int rows = (pb - pa) * s.sh + (s.R - 1) * s.dh + 1;
+    const int h_first = pa * s.sh - s.ph;
+    const int hlo = h_first > 0 ? h_first : 0;
+    const int hhi = h_first + rows - 1 < s.H - 1 ? h_first + rows - 1 : s.H - 1;
+    const int flo = hlo * s.W;
+    const int fhi = hhi >= hlo ? (hhi + 1) * s.W : flo;
+    const int glo = flo >> s.pg_shift;
+    const int ghi = (fhi + pg - 1) >> s.pg_shift;
+    const int n = nchw_div(sl, s.div_od);
+    t.pa[g] = pa;
+    t.rows[g] = rows;
+    t.h_first[g] = h_first;
+    t.flo[g] = flo;
+    t.fhi[g] = fhi;
+    t.glo[g] = glo;
+    t.n[g] = n;
+    t.d0[g] = (sl - n * s.OD) * s.sd - s.pd;
+    t.pos0[g] = pos;
+    t.grp0[g] = grp;
+    if (live) {
+      pos += (rows * s.Wp + 3) & ~3;
+      grp += fhi > flo ? ghi - glo : 0;
+    }
+  }
+  t.npos = pos;
+  t.ngroups = grp;
+  return t;
+}
+
+// LDS byte offset (inside a patch buffer) of 16-byte chunk `chunk` of the position in window row
+// hr, window column wc of slice `q`
+AMOS_HD int nchw_lds_offset(const NchwShape& s, const NchwSeg& q, int hr, int wc, int chunk) {
+  const int P = q.pos0 + hr * s.Wp + wc;
+  const int key = q.pos0 + hr * s.key_pitch + wc;
+  return P * kNchwPosBytes + (((chunk ^ (key >> 2)) & 3) << 4);
+}
+
+// slice `idx` (0 .. kNchwMaxSeg - 1) of a tile, picked by selects on constant element numbers
+#define AMOS_NCHW_PICK(field) (idx == 1 ? t.field[1] : idx == 2 ? t.field[2] : idx == 3 ? t.field[3] : t.field[0])
+AMOS_HD NchwSeg nchw_pick_seg(const NchwTile& t, int idx) {
+  NchwSeg q;
+  q.pos0 = AMOS_NCHW_PICK(pos0); q.pa = AMOS_NCHW_PICK(pa); q.h_first = AMOS_NCHW_PICK(h_first);
+  q.n = AMOS_NCHW_PICK(n); q.d0 = AMOS_NCHW_PICK(d0); q.flo = AMOS_NCHW_PICK(flo); q.fhi = AMOS_NCHW_PICK(fhi);
+  q.glo = AMOS_NCHW_PICK(glo); q.grp0 = AMOS_NCHW_PICK(grp0); q.rows = AMOS_NCHW_PICK(rows);
+  return q;
+}
+#undef AMOS_NCHW_PICK
+
+// A load group: `pg` consecutive in-plane input positions of one slice, fetched (for one chunk of
+// channels) by one thread with one 8-byte load per channel.  Returns the slice and sets f, the
+// group's first in-plane position (a multiple of the group size).
+AMOS_HD NchwSeg nchw_group(const NchwShape& s, const NchwTile& t, int grp, int* f) {
+  int idx = 0;
+#pragma unroll
+  for (int g = 1; g < kNchwMaxSeg; ++g)
+    if (g < t.nseg && grp >= t.grp0[g]) idx = g;
+  const NchwSeg q = nchw_pick_seg(t, idx);
+  *f = (q.glo + grp - q.grp0) << s.pg_shift;
+  return q;
+}
+// LDS byte offset where chunk `chunk` of in-plane position f of slice q goes, or -1 when the
+// position is not part of the slice's window (outside [flo, fhi), or a column no output reads)
+AMOS_HD int nchw_writer_offset(const NchwShape& s, const NchwSeg& q, int f, int chunk) {
+  if (f < q.flo || f >= q.fhi) return -1;
+  const int h = nchw_div(f, s.div_w), w = f - h * s.W;
+  if (w + s.pw >= s.Wp) return -1;   // image columns right of what the last output column reads
+  return nchw_lds_offset(s, q, h - q.h_first, w + s.pw, chunk);
+}
+
+// where the lanes of a fragment read find output position j (clamped into the tile by the caller)
+// at tap (0, 0): LDS position and key; a tap adds (tr * dh * Wp + ts * dw) to the position and
+// (tr * dh * key_pitch + ts * dw) to the key
+struct NchwColumn {
+  int P, key;
+};
+AMOS_HD NchwColumn nchw_column(const NchwShape& s, const NchwTile& t, int j) {
+  const int OPQ = s.OP * s.OQ;
+  const int sl = nchw_div(j, s.div_opq), rem = j - sl * OPQ;
+  const int op = nchw_div(rem, s.div_oq), oq = rem - op * s.OQ;
+  const NchwSeg q = nchw_pick_seg(t, (sl - t.sl_a) & (kNchwMaxSeg - 1));
+  NchwColumn c;
+  const int hr = (op - q.pa) * s.sh, wc = oq * s.sw;
+  c.P = q.pos0 + hr * s.Wp + wc;
+  c.key = q.pos0 + hr * s.key_pitch + wc;
+  return c;
+}
+AMOS_HD int nchw_reader_offset(const NchwShape& s, const NchwColumn& c, int tr, int ts, int chunk) {
+  const int P = c.P + tr * s.dh * s.Wp + ts * s.dw;
+  const int key = c.key + tr * s.dh * s.key_pitch + ts * s.dw;
+  return P * kNchwPosBytes + (((chunk ^ (key >> 2)) & 3) << 4);
+}
+
+}  // namespace amos

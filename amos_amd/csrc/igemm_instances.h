@@ -176,6 +176,48 @@ ConvInstance* pick_conv_tile(int ti, int tj, int waves, int pls, int occ, int w9
 }
 #endif
 
+// convolution straight from NCDHW / KCTRS (defined in inst_conv_nchw_*.hip): 3x3 windows, block
+// tiles 64 x 128 and 64 x 256, eight waves; t1 = the weights of a chunk of channels are one
+// contiguous aligned run (conv2d)
+struct ConvNchwParams;
+typedef void (*conv_nchw_fn)(const ConvNchwParams);
+struct ConvNchwInstance {
+  conv_nchw_fn fn;
+  const char* name;
+  int threads;
+  int bi, bj;
+  int groups_per_thread;   // load groups of the patch a thread may own (x 4 chunks of channels)
+  std::once_flag once;
+  int scratch_bytes = 0;   // per-lane scratch memory of the built kernel (register spills)
+};
+ConvNchwInstance* pick_conv_nchw_f16(int ti, int tj, int t1);
+ConvNchwInstance* pick_conv_nchw_bf16(int ti, int tj, int t1);
+ConvNchwInstance* pick_conv_nchw_i8(int ti, int tj, int t1);
+
+#ifdef AMOS_CONV_NCHW_KERNEL_INCLUDED
+template <int DT, int BI, int BJ, int WI, int WJ, int PT, bool T1>
+ConvNchwInstance* conv_nchw_instance() {
+  static ConvNchwInstance inst;
+  static const char* dtn[] = {"f16", "bf16", "i8"};
+  static std::string name = std::string("amos_conv_nchw<") + dtn[DT] + "," + std::to_string(BI) + "x" +
+                            std::to_string(BJ) + "," + std::to_string(WI * WJ) + "w" + (T1 ? ",2d>" : ",3d>");
+  inst.fn = amos_conv_nchw<DT, BI, BJ, WI, WJ, PT, T1>;
+  inst.name = name.c_str();
+  inst.threads = 64 * WI * WJ;
+  inst.bi = BI;
+  inst.bj = BJ;
+  inst.groups_per_thread = PT;
+  return &inst;
+}
+template <int DT>
+ConvNchwInstance* pick_conv_nchw_tile(int ti, int tj, int t1) {
+  constexpr int PT = DT == DT_I8 ? 1 : 2;
+  if (ti == 64 && tj == 128) return t1 ? conv_nchw_instance<DT, 64, 128, 2, 4, PT, true>() : conv_nchw_instance<DT, 64, 128, 2, 4, PT, false>();
+  if (ti == 64 && tj == 256) return t1 ? conv_nchw_instance<DT, 64, 256, 2, 4, PT, true>() : conv_nchw_instance<DT, 64, 256, 2, 4, PT, false>();
+  return nullptr;
+}
+#endif
+
 Instance* pick_f16_tvec(int cl, int ti, int tj);
 Instance* pick_bf16_tvec(int cl, int ti, int tj);
 Instance* pick_f16_vec(int cl, int ti, int tj);

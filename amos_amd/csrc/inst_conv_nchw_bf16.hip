@@ -1,0 +1,5 @@
+#include "conv_nchw_kernel.h"
+#include "igemm_instances.h"
+namespace amos {
+ConvNchwInstance* pick_conv_nchw_bf16(int ti, int tj, int t1) { return pick_conv_nchw_tile<DT_BF16>(ti, tj, t1); }
+}  // namespace amos

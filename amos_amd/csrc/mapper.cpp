@@ -13,6 +13,10 @@
 #include <atomic>
 #include <cmath>
 #include <cstring>
+#include <mutex>
+#include <vector>
+
+#include "conv_nchw_geom.h"
 
 namespace amos {
 
@@ -652,6 +656,82 @@ static double estimate_seconds(const Problem& pb, int ti, int tj, int split, boo
   const double in_bytes = repacked ? (double)pb.batch * (double)(pb.I + pb.J) * (double)pb.Kp * es : (double)pb.in_bytes;
   const double t_hbm = (in_bytes + (double)pb.out_bytes) / (0.7 * Gfx950::kHbmBytesPerSec) + 3e-6;
   return std::max(t, t_hbm) + 0.1 * std::min(t, t_hbm) + (repacked ? pb.repack_seconds : 0.0);
+}
+
+void conv_nchw_shape(const amos_conv_desc_t& c, int op, NchwShape* out) {
+  NchwShape& s = *out;
+  const bool two_d = op == AMOS_OP_CONV2D;
+  s.N = (int)c.N; s.C = (int)c.C; s.D = two_d ? 1 : (int)c.D; s.H = (int)c.H; s.W = (int)c.W; s.K = (int)c.K;
+  s.T = two_d ? 1 : (int)c.T; s.R = (int)c.R; s.S = (int)c.S;
+  s.sd = two_d ? 1 : c.stride_d; s.sh = c.stride_h; s.sw = c.stride_w;
+  s.pd = two_d ? 0 : c.pad_d; s.ph = c.pad_h; s.pw = c.pad_w;
+  s.dd = two_d ? 1 : c.dil_d; s.dh = c.dil_h; s.dw = c.dil_w;
+  auto ext = [](int64_t in, int pad, int dil, int64_t k, int stride) {
+    const int64_t eff = (k - 1) * dil + 1;
+    return in + 2 * (int64_t)pad < eff ? 0 : (int)((in + 2 * (int64_t)pad - eff) / stride + 1);
+  };
+  s.OD = ext(s.D, s.pd, s.dd, s.T, s.sd);
+  s.OP = ext(s.H, s.ph, s.dh, s.R, s.sh);
+  s.OQ = ext(s.W, s.pw, s.dw, s.S, s.sw);
+  s.J = s.N * s.OD * s.OP * s.OQ;
+  s.Wp = nchw_patch_pitch(s.OQ, s.S, s.sw, s.dw, s.sh);
+  s.key_pitch = nchw_key_pitch(s.OQ, s.Wp, s.sw, s.sh);
+  s.pg_shift = c.in_dtype == AMOS_I8 ? 3 : 2;
+  s.div_opq = nchw_make_div((uint32_t)(s.OP * s.OQ));
+  s.div_oq = nchw_make_div((uint32_t)s.OQ);
+  s.div_w = nchw_make_div((uint32_t)s.W);
+  s.div_od = nchw_make_div((uint32_t)s.OD);
+}
+
+ConvNchwPlan conv_nchw_plan(const amos_conv_desc_t& c, int op, int BI, int BJ) {
+  ConvNchwPlan r;
+  memset(&r, 0, sizeof(r));
+  const int es = c.in_dtype == AMOS_I8 ? 1 : 2;
+  const int64_t T = op == AMOS_OP_CONV2D ? 1 : c.T, D = op == AMOS_OP_CONV2D ? 1 : c.D;
+  if (c.layout != AMOS_LAYOUT_NCHW) { r.why = "tensors not in the NCDHW / KCTRS layout"; return r; }
+  if (c.groups > 1) { r.why = "grouped convolution"; return r; }
+  if (c.R != 3 || c.S != 3) { r.why = "window not 3x3"; return r; }
+  if ((c.C * es) % 64) { r.why = "channels do not fill whole 64-byte chunks"; return r; }
+  if ((c.H * c.W) % (8 / es)) { r.why = "a channel plane is not a whole number of 8-byte loads"; return r; }
+  if (BI != 64 || (BJ != 128 && BJ != 256)) { r.why = "block tile not 64x128 or 64x256"; return r; }
+  if (c.N * c.C * D * c.H * c.W >= ((int64_t)1 << 40) || c.K * c.C * T * 9 >= ((int64_t)1 << 40)) { r.why = "tensor too large"; return r; }
+  NchwShape s;
+  conv_nchw_shape(c, op, &s);
+  if (s.OD <= 0 || s.OP <= 0 || s.OQ <= 0) { r.why = "window larger than the padded input"; return r; }
+  // the largest tile: every tile's geometry, kept per shape (a launch plans again on every call)
+  struct Key { int v[24]; };
+  struct Entry { Key k; int max_pos, max_groups, max_seg; };
+  static std::mutex mu;
+  static std::vector<Entry> cache;
+  Key key = {{s.N, s.D, s.H, s.W, s.T, s.sd, s.sh, s.sw, s.pd, s.ph, s.pw, s.dd, s.dh, s.dw, s.OD, s.OP, s.OQ, s.pg_shift, BJ, 0, 0, 0, 0, 0}};
+  int max_pos = -1, max_groups = 0, max_seg = 0;
+  {
+    std::lock_guard<std::mutex> lock(mu);
+    for (const Entry& e : cache)
+      if (!memcmp(&e.k, &key, sizeof(key))) { max_pos = e.max_pos; max_groups = e.max_groups; max_seg = e.max_seg; }
+  }
+  if (max_pos < 0) {
+    max_pos = 0;
+    for (int64_t bj0 = 0; bj0 < s.J; bj0 += BJ) {
+      const NchwTile t = nchw_tile(s, (int)bj0, BJ);
+      max_seg = std::max(max_seg, t.nseg);
+      if (t.nseg > kNchwMaxSeg) break;
+      max_pos = std::max(max_pos, t.npos);
+      max_groups = std::max(max_groups, t.ngroups);
+    }
+    std::lock_guard<std::mutex> lock(mu);
+    if (cache.size() >= 64) cache.erase(cache.begin());
+    cache.push_back(Entry{key, max_pos, max_groups, max_seg});
+  }
+  if (max_seg > kNchwMaxSeg) { r.why = "a tile of output positions touches more than four images"; return r; }
+  r.max_pos = (max_pos + 3) & ~3;
+  r.max_groups = max_groups;
+  r.groups_per_thread = es == 1 ? 1 : 2;
+  if ((int64_t)max_groups * 4 > (int64_t)r.groups_per_thread * 512) { r.why = "input patch of a tile above the threads' load budget"; return r; }
+  r.lds = (size_t)2 * 9 * BI * 64 + (size_t)2 * r.max_pos * kNchwPosBytes;
+  if (r.lds > (size_t)Gfx950::kLdsBytes - 1024) { r.why = "input patch of a tile does not fit LDS"; return r; }
+  r.t1 = T == 1;
+  return r;
 }
 
 int conv_unroll_level(int flags) {

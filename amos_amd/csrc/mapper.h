@@ -139,4 +139,20 @@ ConvPatchPlan conv_patch_plan(const amos_conv_desc_t& c, int op, int BI, int BJ,
                               int allow_w9 = 2);
 int conv_unroll_level(int config_flags);
 
+// ---- convolution read straight from NCDHW / KCTRS (conv_nchw_kernel.h): one launch, no workspace ----
+// 3x3 windows, one group, NCDHW, channels in whole 64-byte chunks, channel planes (H*W elements) in
+// whole 8-byte loads; block tile 64 output channels x 128 or 256 output positions.
+struct ConvNchwPlan {
+  const char* why;      // nullptr = applicable, else the reason it is not
+  int max_pos;          // LDS positions of a patch buffer (the largest tile's, multiple of 4)
+  int max_groups;       // load groups of the largest tile
+  int groups_per_thread;
+  int t1;               // conv2d: a chunk's weights are one contiguous run (needs 16-byte aligned weights)
+  size_t lds;           // dynamic LDS bytes of a workgroup
+};
+ConvNchwPlan conv_nchw_plan(const amos_conv_desc_t& c, int op, int BI, int BJ);
+// the kernel's geometry descriptor of a convolution (extents, patch pitch, dividers)
+struct NchwShape;
+void conv_nchw_shape(const amos_conv_desc_t& c, int op, NchwShape* out);
+
 }  // namespace amos

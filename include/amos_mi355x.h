@@ -163,6 +163,10 @@ typedef struct {
                               /* 4 waves per workgroup                                        */
 #define AMOS_PIPE_PATCH8 5    /* same with 8 waves (two per SIMD)                             */
 
+#define AMOS_PIPE_NCHW 6      /* conv, 3x3 windows, NCDHW: activations and weights read as they   */
+                              /* are and transposed in registers on their way to LDS; one        */
+                              /* launch, no workspace; tiles 64x128 and 64x256                    */
+
 int amos_version(void);
 const char* amos_last_error(void);
 
