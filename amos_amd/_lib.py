@@ -56,7 +56,7 @@ class KernelConfig(ctypes.Structure):
 AMOS_EPI_NONE, AMOS_EPI_ADD = 0, 1
 AMOS_LAYOUT_NCHW, AMOS_LAYOUT_NHWC, AMOS_LAYOUT_HWNC = 0, 1, 2
 LAYOUT_CODE = {"nchw": 0, "ncdhw": 0, "nhwc": 1, "ndhwc": 1, "hwnc": 2, "dhwnc": 2}
-AMOS_FLAG_NO_UNROLLED_TAPS, AMOS_FLAG_NO_TILE_WALK = 1, 2
+AMOS_FLAG_NO_UNROLLED_TAPS, AMOS_FLAG_NO_TILE_WALK, AMOS_FLAG_WEIGHTS_PACKED = 1, 2, 4
 
 
 class Epilogue(ctypes.Structure):
@@ -96,7 +96,7 @@ class AmosError(RuntimeError):
 EXPORTS = [
     "amos_version", "amos_last_error", "amos_device_info", "amos_default_config",
     "amos_check_config", "amos_workspace_bytes", "amos_estimate_seconds", "amos_gemm", "amos_bgemm", "amos_conv2d",
-    "amos_conv3d", "amos_conv2d_noalloc", "amos_run_fused", "amos_time", "amos_time_fused", "amos_gather", "amos_time_gather",
+    "amos_conv3d", "amos_conv2d_noalloc", "amos_conv_packed_weights_bytes", "amos_conv_pack_weights", "amos_run_fused", "amos_time", "amos_time_fused", "amos_gather", "amos_time_gather",
     "amos_eltwise", "amos_time_eltwise", "amos_kernel_name", "amos_match", "amos_enumerate_mappings",
 ]
 
@@ -128,6 +128,10 @@ def load():
         fn = getattr(lib, name)
         fn.argtypes = [ctypes.POINTER(desc), ctypes.POINTER(KernelConfig), vp, vp, vp, vp, sz, vp]
         fn.restype = ctypes.c_int
+    lib.amos_conv_packed_weights_bytes.argtypes = [ctypes.c_int, ctypes.POINTER(ConvDesc)]
+    lib.amos_conv_packed_weights_bytes.restype = sz
+    lib.amos_conv_pack_weights.argtypes = [ctypes.c_int, ctypes.POINTER(ConvDesc), vp, vp, vp]
+    lib.amos_conv_pack_weights.restype = ctypes.c_int
     lib.amos_conv2d_noalloc.argtypes = [ctypes.POINTER(ConvDesc), ctypes.POINTER(KernelConfig), vp, vp, vp, vp]
     lib.amos_conv2d_noalloc.restype = ctypes.c_int
     lib.amos_time.argtypes = [ctypes.c_int, vp, ctypes.POINTER(KernelConfig), vp, vp, vp, vp, sz, vp,

@@ -331,7 +331,9 @@ struct Plan {
   size_t fewc_lds;
   // convolution read straight from NCDHW / KCTRS (0 = not used)
   int nchw;
-  int nchw_t1;
+  int nchw_wmode, nchw_pt;
+  int nchw_pack;            // 1: the weights are packed into the workspace in front of the kernel
+  const void* nchw_w_src;   // ... from here
   ConvNchwParams nc;
   size_t nchw_lds;
 };
@@ -756,7 +758,22 @@ static int plan_conv(Plan& pl, int op, const amos_conv_desc_t* d, const amos_ker
     ConvNchwParams& q = pl.nc;
     memset(&q, 0, sizeof(q));
     q.x = (const char*)X; q.w = (const char*)Wt; q.y = (char*)Y;
-    conv_nchw_shape(c, op, &q.s);
+    conv_nchw_shape(c, op, np.Wp, &q.s);
+    // Weights: already packed by the caller (AMOS_FLAG_WEIGHTS_PACKED), packed into the workspace by
+    // this call, or -- without a workspace -- transposed by every workgroup on its way to LDS
+    const size_t packed_bytes = (size_t)(c.K * c.C * q.s.T * 9) * (pl.dt == DT_I8 ? 1 : 2);
+    pl.nchw_pack = 0;
+    pl.nchw_w_src = Wt;
+    if (cfg->reserved[0] & AMOS_FLAG_WEIGHTS_PACKED) {
+      if (!aligned16(Wt)) return set_error(AMOS_ERR_BAD_ARG, "packed weights must be 16-byte aligned");
+      pl.nchw_wmode = NCHW_W_PACKED;
+    } else if (workspace && ws_bytes >= packed_bytes && ((uintptr_t)workspace & 255) == 0) {
+      pl.nchw_wmode = NCHW_W_PACKED;
+      pl.nchw_pack = 1;
+      q.w = (const char*)workspace;
+    } else {
+      pl.nchw_wmode = (np.t1 && aligned16(Wt)) ? NCHW_W_KCRS : NCHW_W_KCTRS;
+    }
     const int es1 = pl.dt == DT_I8 ? 1 : 2;
     q.c_chunks = (int)(c.C * es1 / 64);
     q.macro_steps = q.s.T * q.c_chunks;
@@ -767,8 +784,10 @@ static int plan_conv(Plan& pl, int op, const amos_conv_desc_t* d, const amos_ker
     q.split_stride = 0;
     q.div_cc = nchw_make_div((uint32_t)q.c_chunks);
     q.div_odpq = nchw_make_div((uint32_t)(OD * OP * OQ));
+    q.dbg = getenv("AMOS_NCHW_DBG") ? (long long*)strtoull(getenv("AMOS_NCHW_DBG"), nullptr, 0) : nullptr;
+    q.dbg_flags = getenv("AMOS_NCHW_DBG_FLAGS") ? atoi(getenv("AMOS_NCHW_DBG_FLAGS")) : 0;
     pl.nchw = 1;
-    pl.nchw_t1 = np.t1 && aligned16(Wt);
+    pl.nchw_pt = np.groups_per_thread;
     pl.nchw_lds = np.lds;
     memset(&pl.cfg, 0, sizeof(pl.cfg));
     pl.cfg = *cfg;
@@ -1024,14 +1043,14 @@ static int launch_conv(const Plan& pl, hipStream_t stream) {
   return 0;
 }
 
-static ConvNchwInstance* pick_conv_nchw(int dt, int ti, int tj, int t1) {
-  if (dt == DT_F16) return pick_conv_nchw_f16(ti, tj, t1);
-  if (dt == DT_BF16) return pick_conv_nchw_bf16(ti, tj, t1);
-  return pick_conv_nchw_i8(ti, tj, t1);
+static ConvNchwInstance* pick_conv_nchw(int dt, int ti, int tj, int wmode, int pt) {
+  if (dt == DT_F16) return pick_conv_nchw_f16(ti, tj, wmode, pt);
+  if (dt == DT_BF16) return pick_conv_nchw_bf16(ti, tj, wmode, pt);
+  return pick_conv_nchw_i8(ti, tj, wmode, pt);
 }
 
 static int launch_conv_nchw(const Plan& pl, hipStream_t stream) {
-  ConvNchwInstance* inst = pick_conv_nchw(pl.dt, pl.cfg.tile_i, pl.cfg.tile_j, pl.nchw_t1);
+  ConvNchwInstance* inst = pick_conv_nchw(pl.dt, pl.cfg.tile_i, pl.cfg.tile_j, pl.nchw_wmode, pl.nchw_pt);
   if (!inst) return set_error(AMOS_ERR_INFEASIBLE, "no NCDHW-direct convolution instance");
   hipError_t attr_err = hipSuccess;
   std::call_once(inst->once, [&] {
@@ -1039,16 +1058,22 @@ static int launch_conv_nchw(const Plan& pl, hipStream_t stream) {
                                    160 * 1024 - 1024);
     hipFuncAttributes fa;
     if (attr_err == hipSuccess) attr_err = hipFuncGetAttributes(&fa, (const void*)inst->fn);
-    if (attr_err == hipSuccess) inst->scratch_bytes = (int)fa.localSizeBytes;
+    if (attr_err == hipSuccess) { inst->scratch_bytes = (int)fa.localSizeBytes; inst->static_lds = (int)fa.sharedSizeBytes; }
   });
   if (attr_err != hipSuccess)
     return set_error(AMOS_ERR_HIP, "hipFuncSetAttribute(%s): %s", inst->name, hipGetErrorString(attr_err));
+  if (inst->static_lds)   // the kernel addresses its dynamic LDS from byte 0
+    return set_error(AMOS_ERR_HIP, "%s was built with %d bytes of static LDS", inst->name, inst->static_lds);
   const ConvNchwParams& q = pl.nc;
   // what the kernel assumes of its launch: the tile of the instance, whole 64-byte chunks of
   // channels, a patch that fits the LDS asked for
   if (inst->bi != pl.cfg.tile_i || inst->bj != pl.cfg.tile_j || q.c_chunks < 1 || q.max_pos < 4 ||
-      pl.nchw_lds != (size_t)2 * 9 * inst->bi * 64 + (size_t)2 * q.max_pos * kNchwPosBytes)
+      q.max_pos > nchw_max_positions(inst->bj) ||
+      pl.nchw_lds != (size_t)2 * 9 * inst->bi * 64 + (size_t)2 * nchw_patch_buffer_bytes(inst->bj) ||
+      inst->threads != inst->bi * 8)
     return set_error(AMOS_ERR_BAD_ARG, "inconsistent plan for %s", inst->name);
+  if (pl.nchw_pack)
+    launch_conv_pack_weights(pl.dt == DT_I8 ? 1 : 2, pl.nchw_w_src, (void*)q.w, q.s.K, q.s.C, q.s.T * 9, stream);
   dim3 grid((unsigned)(q.tiles_i * q.tiles_j), (unsigned)pl.split, 1);
   hipLaunchKernelGGL(inst->fn, grid, dim3(inst->threads), pl.nchw_lds, stream, q);
   HIP_TRY(hipGetLastError());
@@ -1386,6 +1411,30 @@ int amos_conv2d_noalloc(const amos_conv_desc_t* desc, const amos_kernel_config_t
   return run_op(AMOS_OP_CONV2D, desc, cfg, nullptr, X, Wt, Y, ptr, (size_t)AMOS_NOALLOC_SCRATCH_BYTES, stream);
 }
 
+size_t amos_conv_packed_weights_bytes(int op, const amos_conv_desc_t* desc) {
+  if (!desc || (op != AMOS_OP_CONV2D && op != AMOS_OP_CONV3D) || desc->K <= 0 || desc->C <= 0 || desc->R != 3 ||
+      desc->S != 3 || desc->groups > 1 || desc->layout != AMOS_LAYOUT_NCHW)
+    return 0;
+  const int64_t T = op == AMOS_OP_CONV2D ? 1 : desc->T;
+  const int es = desc->in_dtype == AMOS_I8 ? 1 : 2;
+  if (T <= 0 || (desc->C * es) % 16) return 0;
+  return (size_t)(desc->K * desc->C * T * 9 * es);
+}
+
+int amos_conv_pack_weights(int op, const amos_conv_desc_t* desc, const void* Wt, void* packed, void* stream) {
+  if (!desc || !Wt || !packed) return set_error(AMOS_ERR_BAD_ARG, "null pointer argument");
+  const size_t bytes = amos_conv_packed_weights_bytes(op, desc);
+  if (!bytes) return set_error(AMOS_ERR_UNSUPPORTED, "packed weights exist for 3x3 windows, one group, KCTRS weights "
+                                                     "with channels in whole 16-byte chunks");
+  if (bytes >= ((size_t)1 << 32)) return set_error(AMOS_ERR_UNSUPPORTED, "weights of 4 GiB or more");
+  if ((uintptr_t)packed & 15) return set_error(AMOS_ERR_BAD_ARG, "packed weights must be 16-byte aligned");
+  const int es = desc->in_dtype == AMOS_I8 ? 1 : 2;
+  launch_conv_pack_weights(es, Wt, packed, (int)desc->K, (int)desc->C, (int)((op == AMOS_OP_CONV2D ? 1 : desc->T) * 9),
+                           (hipStream_t)stream);
+  HIP_TRY(hipGetLastError());
+  return 0;
+}
+
 int amos_run_fused(int op, const void* desc, const amos_kernel_config_t* cfg,
                    const amos_epilogue_t* epilogue, const void* in0, const void* in1, void* out,
                    void* workspace, size_t ws_bytes, void* stream) {
@@ -1407,7 +1456,13 @@ size_t amos_workspace_bytes(int op, const void* desc, const amos_kernel_config_t
     return (size_t)gemm_repack(b->g, b->batch, false, false).total();
   }
   if (op != AMOS_OP_CONV2D && op != AMOS_OP_CONV3D) return 0;
-  if (cfg && cfg->pipeline == AMOS_PIPE_NCHW) return 0;   // reads the caller's tensors as they are
+  if (cfg && cfg->pipeline == AMOS_PIPE_NCHW) {
+    // the activations are read as they are; the weights are packed into the workspace by every
+    // call unless the caller has packed them already (without a workspace every workgroup
+    // transposes its own share)
+    if (cfg->reserved[0] & AMOS_FLAG_WEIGHTS_PACKED) return 0;
+    return amos_conv_packed_weights_bytes(op, (const amos_conv_desc_t*)desc);
+  }
   const amos_conv_desc_t& c = *(const amos_conv_desc_t*)desc;
   int64_t need = conv_workspace_bytes(c, op);
   // a pointwise convolution runs as a matrix product; its row-contiguous operand (NCDHW
@@ -1441,7 +1496,7 @@ const char* amos_kernel_name(int op, const void* desc, const amos_kernel_config_
   static char dummy_ws[256] __attribute__((aligned(256)));
   if (make_plan(pl, op, desc, cfg, dummy, dummy, dummy, dummy_ws, (size_t)-1)) return nullptr;
   if (pl.nchw) {
-    ConvNchwInstance* ni = pick_conv_nchw(pl.dt, pl.cfg.tile_i, pl.cfg.tile_j, pl.nchw_t1);
+    ConvNchwInstance* ni = pick_conv_nchw(pl.dt, pl.cfg.tile_i, pl.cfg.tile_j, pl.nchw_wmode, pl.nchw_pt);
     return ni ? ni->name : nullptr;
   }
   if (pl.dw) return depthwise_name(pl.dt, pl.dw - 1);

@@ -11,11 +11,22 @@
 // K sub-step).  A window tap (r, s) only shifts the position a lane reads: by r * dil_h rows and
 // s * dil_w columns.
 //
-// Bank conflicts: a 64-byte position holds four 16-byte chunks; chunk c of position P is stored at
-// chunk c ^ ((key(P) >> 2) & 3), key(P) = P with the row pitch Wp replaced by key_pitch.  With unit
-// strides key_pitch = OQ, so the sixteen consecutive output positions of a fragment read have
-// sixteen consecutive keys also where they wrap into the next patch row, and, Wp - OQ being a
-// multiple of 4, hit sixteen different 16-byte bank groups at any tap.
+// Bank conflicts (measured on gfx950 with a microbenchmark: 16-byte accesses of one wave, lane l on
+// a chosen 16-byte slot of the 256-byte bank space).  A 16-byte read of a wave is served in four
+// cycles, two per half of the wave, when no slot is used by more than two lanes of a half (248
+// bytes per clock and CU); sixteen consecutive lanes on sixteen slots, or any other split of a
+// half's 32 lanes into two conflict-free sixteens, all run at that rate, four lanes per slot at
+// half of it.  16-byte writes reach a third of the read rate whatever the slots.
+// Layout: eight consecutive positions form a 512-byte block of two 256-byte lines -- chunks 0 and
+// 1 in the first, 2 and 3 in the second -- chunk c of position P in slot
+// ((P & 7) * 2 + (c & 1)) ^ ((c >> 1) * 4) of its line.
+//   * A fragment read: the lower half of a wave holds sixteen consecutive positions x chunks 0 and
+//     1, the upper half chunks 2 and 3 (lane group q = lane / 16 reads chunk q): every slot twice
+//     per half, whatever position the sixteen start at, so also at every window tap.
+//   * Consecutive outputs are consecutive positions except where they wrap into the next patch
+//     row; with a row pitch that differs from the outputs per row by a multiple of 8 the slots
+//     continue across the wrap.
+//   * The weight tiles use the same formula with the row in the place of the position.
 #pragma once
 #include <stdint.h>
 
@@ -56,22 +67,20 @@ struct NchwShape {
   int OD, OP, OQ;
   int J;           // N * OD * OP * OQ
   int Wp;          // patch row pitch in positions
-  int key_pitch;   // row pitch of the swizzle key
   int pg_shift;    // log2 of the input positions per 8-byte load: 2 (16-bit types) or 3 (int8)
   NchwDiv div_opq, div_oq, div_w, div_od;
 };
 
-// patch row pitch: the columns a row of outputs touches, rounded so that Wp - OQ is a multiple of 4
-// where the key compaction applies
-AMOS_HD int nchw_patch_pitch(int OQ, int S, int sw, int dw, int sh) {
+// patch row pitch: the columns a row of outputs touches, rounded up so that the pitch differs from
+// the outputs per row by a multiple of `align` (16: conflict-free across row wraps; 1: smallest)
+AMOS_HD int nchw_patch_pitch(int OQ, int S, int sw, int dw, int sh, int align) {
   int wp = (OQ - 1) * sw + (S - 1) * dw + 1;
-  if (sw == 1 && sh == 1) wp += (4 - ((wp - OQ) & 3)) & 3;
+  if (sw == 1 && sh == 1 && align > 1) wp += (align - ((wp - OQ) % align)) % align;
   return wp;
 }
-AMOS_HD int nchw_key_pitch(int OQ, int Wp, int sw, int sh) { return (sw == 1 && sh == 1) ? OQ : Wp; }
 
 struct NchwSeg {
-  int pos0;      // first LDS position of the slice's window (multiple of 4)
+  int pos0;      // first LDS position of the slice's window (multiple of 8)
   int pa;        // first output row of the tile in this slice
   int h_first;   // input row of window row 0 (may be negative: padding)
   int n, d0;     // image, input depth of depth tap 0 (may be out of range: padding)
@@ -130,7 +139,7 @@ AMOS_HD NchwTile nchw_tile(const NchwShape& s, int bj0, int BJ) {
     t.pos0[g] = pos;
     t.grp0[g] = grp;
     if (live) {
-      pos += (rows * s.Wp + 3) & ~3;
+      pos += (rows * s.Wp + 7) & ~7;   // whole 8-position blocks
       grp += fhi > flo ? ghi - glo : 0;
     }
   }
@@ -139,12 +148,19 @@ AMOS_HD NchwTile nchw_tile(const NchwShape& s, int bj0, int BJ) {
   return t;
 }
 
-// LDS byte offset (inside a patch buffer) of 16-byte chunk `chunk` of the position in window row
-// hr, window column wc of slice `q`
+// LDS byte offset (inside a patch buffer / a weight tile) of 16-byte chunk `chunk` of position
+// (row) P
+AMOS_HD int nchw_position_offset(int P, int chunk) {
+  return ((P >> 3) << 9) + ((chunk >> 1) << 8) + (((((P & 7) << 1) | (chunk & 1)) ^ ((chunk >> 1) << 2)) << 4);
+}
+// the chunk lane group q (lane / 16) of a fragment read takes
+AMOS_HD int nchw_frag_chunk(int q) { return q; }
+// the row (of sixteen) that the lanes 4x .. 4x+3 of a wave fill when a wave writes sixteen rows
+// of a weight tile with one store
+AMOS_HD int nchw_row_of_slot(int x) { return (x & 3) | ((x & 4) << 1) | ((x & 8) >> 1); }
+// ... of the position in window row hr, window column wc of slice `q`
 AMOS_HD int nchw_lds_offset(const NchwShape& s, const NchwSeg& q, int hr, int wc, int chunk) {
-  const int P = q.pos0 + hr * s.Wp + wc;
-  const int key = q.pos0 + hr * s.key_pitch + wc;
-  return P * kNchwPosBytes + (((chunk ^ (key >> 2)) & 3) << 4);
+  return nchw_position_offset(q.pos0 + hr * s.Wp + wc, chunk);
 }
 
 // slice `idx` (0 .. kNchwMaxSeg - 1) of a tile, picked by selects on constant element numbers
@@ -180,26 +196,16 @@ AMOS_HD int nchw_writer_offset(const NchwShape& s, const NchwSeg& q, int f, int 
 }
 
 // where the lanes of a fragment read find output position j (clamped into the tile by the caller)
-// at tap (0, 0): LDS position and key; a tap adds (tr * dh * Wp + ts * dw) to the position and
-// (tr * dh * key_pitch + ts * dw) to the key
-struct NchwColumn {
-  int P, key;
-};
-AMOS_HD NchwColumn nchw_column(const NchwShape& s, const NchwTile& t, int j) {
+// at tap (0, 0): its LDS position; a tap adds (tr * dh * Wp + ts * dw)
+AMOS_HD int nchw_column(const NchwShape& s, const NchwTile& t, int j) {
   const int OPQ = s.OP * s.OQ;
   const int sl = nchw_div(j, s.div_opq), rem = j - sl * OPQ;
   const int op = nchw_div(rem, s.div_oq), oq = rem - op * s.OQ;
   const NchwSeg q = nchw_pick_seg(t, (sl - t.sl_a) & (kNchwMaxSeg - 1));
-  NchwColumn c;
-  const int hr = (op - q.pa) * s.sh, wc = oq * s.sw;
-  c.P = q.pos0 + hr * s.Wp + wc;
-  c.key = q.pos0 + hr * s.key_pitch + wc;
-  return c;
+  return q.pos0 + (op - q.pa) * s.sh * s.Wp + oq * s.sw;
 }
-AMOS_HD int nchw_reader_offset(const NchwShape& s, const NchwColumn& c, int tr, int ts, int chunk) {
-  const int P = c.P + tr * s.dh * s.Wp + ts * s.dw;
-  const int key = c.key + tr * s.dh * s.key_pitch + ts * s.dw;
-  return P * kNchwPosBytes + (((chunk ^ (key >> 2)) & 3) << 4);
+AMOS_HD int nchw_reader_offset(const NchwShape& s, int column, int tr, int ts, int chunk) {
+  return nchw_position_offset(column + tr * s.dh * s.Wp + ts * s.dw, chunk);
 }
 
 }  // namespace amos

@@ -658,7 +658,8 @@ static double estimate_seconds(const Problem& pb, int ti, int tj, int split, boo
   return std::max(t, t_hbm) + 0.1 * std::min(t, t_hbm) + (repacked ? pb.repack_seconds : 0.0);
 }
 
-void conv_nchw_shape(const amos_conv_desc_t& c, int op, NchwShape* out) {
+// patch_pitch 0: the smallest row pitch
+void conv_nchw_shape(const amos_conv_desc_t& c, int op, int patch_pitch, NchwShape* out) {
   NchwShape& s = *out;
   const bool two_d = op == AMOS_OP_CONV2D;
   s.N = (int)c.N; s.C = (int)c.C; s.D = two_d ? 1 : (int)c.D; s.H = (int)c.H; s.W = (int)c.W; s.K = (int)c.K;
@@ -674,8 +675,7 @@ void conv_nchw_shape(const amos_conv_desc_t& c, int op, NchwShape* out) {
   s.OP = ext(s.H, s.ph, s.dh, s.R, s.sh);
   s.OQ = ext(s.W, s.pw, s.dw, s.S, s.sw);
   s.J = s.N * s.OD * s.OP * s.OQ;
-  s.Wp = nchw_patch_pitch(s.OQ, s.S, s.sw, s.dw, s.sh);
-  s.key_pitch = nchw_key_pitch(s.OQ, s.Wp, s.sw, s.sh);
+  s.Wp = patch_pitch > 0 ? patch_pitch : nchw_patch_pitch(s.OQ, s.S, s.sw, s.dw, s.sh, 1);
   s.pg_shift = c.in_dtype == AMOS_I8 ? 3 : 2;
   s.div_opq = nchw_make_div((uint32_t)(s.OP * s.OQ));
   s.div_oq = nchw_make_div((uint32_t)s.OQ);
@@ -693,43 +693,60 @@ ConvNchwPlan conv_nchw_plan(const amos_conv_desc_t& c, int op, int BI, int BJ) {
   if (c.R != 3 || c.S != 3) { r.why = "window not 3x3"; return r; }
   if ((c.C * es) % 64) { r.why = "channels do not fill whole 64-byte chunks"; return r; }
   if ((c.H * c.W) % (8 / es)) { r.why = "a channel plane is not a whole number of 8-byte loads"; return r; }
-  if (BI != 64 || (BJ != 128 && BJ != 256)) { r.why = "block tile not 64x128 or 64x256"; return r; }
-  if (c.N * c.C * D * c.H * c.W >= ((int64_t)1 << 40) || c.K * c.C * T * 9 >= ((int64_t)1 << 40)) { r.why = "tensor too large"; return r; }
+  if ((BI != 64 && BI != 32) || (BJ != 128 && BJ != 256)) { r.why = "block tile not 32 or 64 by 128 or 256"; return r; }
+  // (lanes address both tensors by 32-bit byte offsets)
+  if (c.N * c.C * D * c.H * c.W * es >= ((int64_t)1 << 32) || c.K * c.C * T * 9 * es >= ((int64_t)1 << 32)) { r.why = "a tensor of 4 GiB or more"; return r; }
   NchwShape s;
-  conv_nchw_shape(c, op, &s);
+  conv_nchw_shape(c, op, 0, &s);
   if (s.OD <= 0 || s.OP <= 0 || s.OQ <= 0) { r.why = "window larger than the padded input"; return r; }
-  // the largest tile: every tile's geometry, kept per shape (a launch plans again on every call)
+  // nine weight tiles and a patch buffer of the tile's fixed size (its last 1 KB a dump line), both twice
+  const int pbuf = BJ <= 128 ? 32 * 1024 : 40 * 1024;
+  const int pos_limit = pbuf / kNchwPosBytes - 16;
+  // The largest tile: every tile's geometry, kept per shape (a launch plans again on every call).
+  // The row pitch of the patch: pitch - outputs per row a multiple of 8 (fragment reads free of bank
+  // conflicts also where they wrap into the next row) where the largest patch then fits the
+  // buffer, else the smallest.
   struct Key { int v[24]; };
   struct Entry { Key k; int max_pos, max_groups, max_seg; };
   static std::mutex mu;
   static std::vector<Entry> cache;
-  Key key = {{s.N, s.D, s.H, s.W, s.T, s.sd, s.sh, s.sw, s.pd, s.ph, s.pw, s.dd, s.dh, s.dw, s.OD, s.OP, s.OQ, s.pg_shift, BJ, 0, 0, 0, 0, 0}};
   int max_pos = -1, max_groups = 0, max_seg = 0;
-  {
-    std::lock_guard<std::mutex> lock(mu);
-    for (const Entry& e : cache)
-      if (!memcmp(&e.k, &key, sizeof(key))) { max_pos = e.max_pos; max_groups = e.max_groups; max_seg = e.max_seg; }
-  }
-  if (max_pos < 0) {
-    max_pos = 0;
-    for (int64_t bj0 = 0; bj0 < s.J; bj0 += BJ) {
-      const NchwTile t = nchw_tile(s, (int)bj0, BJ);
-      max_seg = std::max(max_seg, t.nseg);
-      if (t.nseg > kNchwMaxSeg) break;
-      max_pos = std::max(max_pos, t.npos);
-      max_groups = std::max(max_groups, t.ngroups);
+  for (int align : {8, 1}) {
+    s.Wp = nchw_patch_pitch(s.OQ, s.S, s.sw, s.dw, s.sh, align);
+    Key key = {{s.N, s.D, s.H, s.W, s.T, s.sd, s.sh, s.sw, s.pd, s.ph, s.pw, s.dd, s.dh, s.dw, s.OD, s.OP, s.OQ, s.pg_shift, BJ, s.Wp, 0, 0, 0, 0}};
+    max_pos = -1; max_groups = 0; max_seg = 0;
+    {
+      std::lock_guard<std::mutex> lock(mu);
+      for (const Entry& e : cache)
+        if (!memcmp(&e.k, &key, sizeof(key))) { max_pos = e.max_pos; max_groups = e.max_groups; max_seg = e.max_seg; }
     }
-    std::lock_guard<std::mutex> lock(mu);
-    if (cache.size() >= 64) cache.erase(cache.begin());
-    cache.push_back(Entry{key, max_pos, max_groups, max_seg});
+    if (max_pos < 0) {
+      max_pos = 0;
+      for (int64_t bj0 = 0; bj0 < s.J; bj0 += BJ) {
+        const NchwTile t = nchw_tile(s, (int)bj0, BJ);
+        max_seg = std::max(max_seg, t.nseg);
+        if (t.nseg > kNchwMaxSeg) break;
+        max_pos = std::max(max_pos, t.npos);
+        max_groups = std::max(max_groups, t.ngroups);
+      }
+      std::lock_guard<std::mutex> lock(mu);
+      if (cache.size() >= 64) cache.erase(cache.begin());
+      cache.push_back(Entry{key, max_pos, max_groups, max_seg});
+    }
+    if (max_seg > kNchwMaxSeg || max_pos <= pos_limit) break;
   }
   if (max_seg > kNchwMaxSeg) { r.why = "a tile of output positions touches more than four images"; return r; }
-  r.max_pos = (max_pos + 3) & ~3;
+  r.max_pos = max_pos;   // (whole 8-position blocks)
+  r.Wp = s.Wp;
   r.max_groups = max_groups;
-  r.groups_per_thread = es == 1 ? 1 : 2;
-  if ((int64_t)max_groups * 4 > (int64_t)r.groups_per_thread * 512) { r.why = "input patch of a tile above the threads' load budget"; return r; }
-  r.lds = (size_t)2 * 9 * BI * 64 + (size_t)2 * r.max_pos * kNchwPosBytes;
-  if (r.lds > (size_t)Gfx950::kLdsBytes - 1024) { r.why = "input patch of a tile does not fit LDS"; return r; }
+  const int threads = BI * 8;   // 64-row tiles run eight waves, 32-row tiles four
+  r.groups_per_thread = (int64_t)max_groups * 4 <= threads ? 1 : 2;
+  if (r.groups_per_thread == 2 && (es == 1 || BJ != 128 || (int64_t)max_groups * 4 > 2 * threads)) {
+    r.why = "input patch of a tile above the threads' load budget";
+    return r;
+  }
+  if (r.max_pos > pos_limit) { r.why = "input patch of a tile does not fit its LDS buffer"; return r; }
+  r.lds = (size_t)2 * 9 * BI * 64 + (size_t)2 * pbuf;
   r.t1 = T == 1;
   return r;
 }

@@ -145,6 +145,7 @@ int conv_unroll_level(int config_flags);
 struct ConvNchwPlan {
   const char* why;      // nullptr = applicable, else the reason it is not
   int max_pos;          // LDS positions of a patch buffer (the largest tile's, multiple of 4)
+  int Wp;               // row pitch of the patch in positions
   int max_groups;       // load groups of the largest tile
   int groups_per_thread;
   int t1;               // conv2d: a chunk's weights are one contiguous run (needs 16-byte aligned weights)
@@ -153,6 +154,6 @@ struct ConvNchwPlan {
 ConvNchwPlan conv_nchw_plan(const amos_conv_desc_t& c, int op, int BI, int BJ);
 // the kernel's geometry descriptor of a convolution (extents, patch pitch, dividers)
 struct NchwShape;
-void conv_nchw_shape(const amos_conv_desc_t& c, int op, NchwShape* out);
+void conv_nchw_shape(const amos_conv_desc_t& c, int op, int patch_pitch, NchwShape* out);
 
 }  // namespace amos

@@ -148,6 +148,9 @@ typedef struct {
 /* conv: one tile per workgroup also where the unrolled instance would let a workgroup walk
  * several tiles (more tiles than compute units, no split-K) */
 #define AMOS_FLAG_NO_TILE_WALK 2
+/* conv, AMOS_PIPE_NCHW: `Wt` points at weights that amos_conv_pack_weights has written (their owner
+ * packs them once instead of every call packing them into its workspace) */
+#define AMOS_FLAG_WEIGHTS_PACKED 4
 
 /* how tiles travel from HBM to the MFMA operands */
 #define AMOS_PIPE_AUTO 0      /* the mapper's choice; a depthwise convolution (groups == C,  */
@@ -163,9 +166,13 @@ typedef struct {
                               /* 4 waves per workgroup                                        */
 #define AMOS_PIPE_PATCH8 5    /* same with 8 waves (two per SIMD)                             */
 
-#define AMOS_PIPE_NCHW 6      /* conv, 3x3 windows, NCDHW: activations and weights read as they   */
-                              /* are and transposed in registers on their way to LDS; one        */
-                              /* launch, no workspace; tiles 64x128 and 64x256                    */
+#define AMOS_PIPE_NCHW 6      /* conv, 3x3 windows, NCDHW: the activations are read as they are   */
+                              /* and transposed in registers on their way to LDS; the weights   */
+                              /* are packed to [K][T*9][C] -- into the workspace by the call     */
+                              /* (amos_workspace_bytes), or once by their owner                  */
+                              /* (amos_conv_pack_weights, AMOS_FLAG_WEIGHTS_PACKED) -- or,       */
+                              /* without a workspace, transposed in registers as well; tiles    */
+                              /* 32 or 64 output channels x 128 or 256 output positions          */
 
 int amos_version(void);
 const char* amos_last_error(void);
@@ -216,6 +223,18 @@ int amos_conv3d(const amos_conv_desc_t* desc, const amos_kernel_config_t* cfg, c
 #define AMOS_NOALLOC_SCRATCH_BYTES (8u << 20)
 int amos_conv2d_noalloc(const amos_conv_desc_t* desc, const amos_kernel_config_t* cfg, const void* X,
                         const void* Wt, void* Y, void* stream);
+
+/*
+ * Weights KCTRS -> [K][T*R*S][C] for AMOS_PIPE_NCHW (3x3 windows, one group, channels in whole
+ * 16-byte chunks): amos_conv_packed_weights_bytes() bytes at `packed` (16-byte aligned; 0 = no
+ * packed form for this descriptor).  A convolution called with AMOS_FLAG_WEIGHTS_PACKED takes the
+ * packed weights as its `Wt`.  In the reference the reordered weight operand is a stage of its own
+ * in front of the main kernel, recomputed on every call
+ * (src/auto_tensorize/compute_transform.cc:181-293); a caller whose weights do not change between
+ * calls can do it once here.
+ */
+size_t amos_conv_packed_weights_bytes(int op, const amos_conv_desc_t* desc);
+int amos_conv_pack_weights(int op, const amos_conv_desc_t* desc, const void* Wt, void* packed, void* stream);
 
 /* A tail operation fused into the store of the accumulators.  AMOS_EPI_ADD: out = acc + cast(D),
  * D an operand with the output's shape: GEMM / batched GEMM [M][ld] (ld 0 = N) with `stride`

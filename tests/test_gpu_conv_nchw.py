@@ -24,8 +24,23 @@ def _check(got, ref, dtype, what):
         assert mx <= MAX_REL and mean <= MEAN_REL, "%s: max_rel=%.3e mean_rel=%.3e" % (what, mx, mean)
 
 
-def _cfg(_lib, tj):
-    return dict(tile_i=64, tile_j=tj, split_k=1, pipeline=_lib.AMOS_PIPE_NCHW)
+def _cfg(_lib, tj, ti=64):
+    return dict(tile_i=ti, tile_j=tj, split_k=1, pipeline=_lib.AMOS_PIPE_NCHW)
+
+
+TILES = [(64, 128), (64, 256), (32, 128), (32, 256)]
+
+
+def _run(fn, *args, **kw):
+    """the call, or a skip where the planner says that this tile does not suit the shape (a tile
+    whose input patch is more than its threads load in one round, or more than LDS holds)"""
+    from amos_amd import _lib
+    try:
+        return fn(*args, **kw)
+    except _lib.AmosError as e:
+        if e.code == _lib.AMOS_ERR_INFEASIBLE and ("load budget" in str(e) or "fit LDS" in str(e)):
+            pytest.skip(str(e))
+        raise
 
 
 # N, C, H, W, K, stride, pad, dil
@@ -42,26 +57,27 @@ CASES_2D = [
 
 
 @pytest.mark.parametrize("dtype", ["float16", "bfloat16", "int8"])
-@pytest.mark.parametrize("tj", [128, 256])
+@pytest.mark.parametrize("tile", TILES)
 @pytest.mark.parametrize("case", CASES_2D)
-def test_conv2d_nchw_direct(gpu, dtype, tj, case):
+def test_conv2d_nchw_direct(gpu, dtype, tile, case):
     from amos_amd import _lib, ops
+    ti, tj = tile
     N, C, H, W, K, st, pd, dl = case
     if dtype == "int8" and (H * W) % 8:
         pytest.skip("int8 needs channel planes of whole 8-byte loads")
     rng = np.random.default_rng(N * 1000 + C + H * 7 + K)
     x, w = make_operand(rng, (N, C, H, W), dtype), make_operand(rng, (K, C, 3, 3), dtype)
-    print("conv2d nchw", dtype, tj, case, flush=True)
+    print("conv2d nchw", dtype, tile, case, flush=True)
     oshape = ops.conv_out_shape((N, C, 1, H, W), (K, C, 1, 3, 3), (1,) + ops._tup(st, 2), (0,) + ops._tup(pd, 2), (1,) + ops._tup(dl, 2))
     opq, J = oshape[3] * oshape[4], N * oshape[3] * oshape[4]
     if max((min(j0 + tj, J) - 1) // opq - j0 // opq + 1 for j0 in range(0, J, tj)) > 4:
         # a tile would touch more than four images: the pipeline says so instead of running
         with pytest.raises(_lib.AmosError, match="more than four images"):
-            ops.conv2d(to_device(x, dtype), to_device(w, dtype), st, pd, dl, config=_cfg(_lib, tj))
+            ops.conv2d(to_device(x, dtype), to_device(w, dtype), st, pd, dl, config=_cfg(_lib, tj, ti))
         return
-    got = ops.conv2d(to_device(x, dtype), to_device(w, dtype), st, pd, dl, config=_cfg(_lib, tj)).cpu().numpy()
+    got = _run(ops.conv2d, to_device(x, dtype), to_device(w, dtype), st, pd, dl, config=_cfg(_lib, tj, ti)).cpu().numpy()
     ref = co.lib_conv2d(x, w, dtype, st, pd, dl, acc="float64") if dtype != "int8" else co.lib_conv2d(x, w, dtype, st, pd, dl)
-    _check(got, ref, dtype, "conv2d %s tile 64x%d %s" % (dtype, tj, case))
+    _check(got, ref, dtype, "conv2d %s tile %dx%d %s" % (dtype, ti, tj, case))
 
 
 # N, C, D, H, W, K, stride, pad, dil
@@ -73,19 +89,20 @@ CASES_3D = [
 
 
 @pytest.mark.parametrize("dtype", ["float16", "int8"])
-@pytest.mark.parametrize("tj", [128, 256])
+@pytest.mark.parametrize("tile", TILES)
 @pytest.mark.parametrize("case", CASES_3D)
-def test_conv3d_nchw_direct(gpu, dtype, tj, case):
+def test_conv3d_nchw_direct(gpu, dtype, tile, case):
     from amos_amd import _lib, ops
+    ti, tj = tile
     N, C, D, H, W, K, st, pd, dl = case
     if dtype == "int8" and (H * W) % 8:
         pytest.skip("int8 needs channel planes of whole 8-byte loads")
     rng = np.random.default_rng(N * 1000 + C + D * 31 + H * 7 + K)
     x, w = make_operand(rng, (N, C, D, H, W), dtype), make_operand(rng, (K, C, 3, 3, 3), dtype)
-    print("conv3d nchw", dtype, tj, case, flush=True)
-    got = ops.conv3d(to_device(x, dtype), to_device(w, dtype), st, pd, dl, config=_cfg(_lib, tj)).cpu().numpy()
+    print("conv3d nchw", dtype, tile, case, flush=True)
+    got = _run(ops.conv3d, to_device(x, dtype), to_device(w, dtype), st, pd, dl, config=_cfg(_lib, tj, ti)).cpu().numpy()
     ref = co.lib_conv3d(x, w, dtype, st, pd, dl, acc="float64") if dtype != "int8" else co.lib_conv3d(x, w, dtype, st, pd, dl)
-    _check(got, ref, dtype, "conv3d %s tile 64x%d %s" % (dtype, tj, case))
+    _check(got, ref, dtype, "conv3d %s tile %dx%d %s" % (dtype, ti, tj, case))
 
 
 def test_conv2d_nchw_unaligned_weights_and_fused_tail(gpu):
@@ -110,6 +127,61 @@ def test_conv2d_nchw_unaligned_weights_and_fused_tail(gpu):
     add = torch.randn((2, 48, 10, 10), device="cuda")
     got = ops.conv2d(dx, to_device(w, "float16"), 1, 1, 1, config=_cfg(_lib, 128), add=add)
     _check((got - add).cpu().numpy(), ref, "float16", "fused tail")
+
+
+@pytest.mark.parametrize("dtype", ["float16", "int8"])
+@pytest.mark.parametrize("tile", TILES)
+def test_conv_nchw_weight_modes_agree(gpu, dtype, tile):
+    """the three ways the weights reach LDS -- packed into the workspace by the call, packed once by
+    their owner (AMOS_FLAG_WEIGHTS_PACKED), transposed by every workgroup (no workspace) -- give the
+    same bits (the accumulation order does not depend on them), 2-d and 3-d"""
+    import torch
+    from amos_amd import _lib, ops
+    lib = _lib.load()
+    ti, tj = tile
+    for xs, ws, op in (((2, 128, 1, 12, 12), (72, 128, 1, 3, 3), _lib.AMOS_OP_CONV2D),
+                       ((1, 64, 3, 8, 8), (40, 64, 3, 3, 3), _lib.AMOS_OP_CONV3D)):
+        rng = np.random.default_rng(ti + tj + len(dtype))
+        x, w = make_operand(rng, xs, dtype), make_operand(rng, ws, dtype)
+        dx, dw = to_device(x, dtype), to_device(w, dtype)
+        pad = (0, 1, 1) if op == _lib.AMOS_OP_CONV2D else (1, 1, 1)
+        d = ops.conv_desc(xs, ws, dx.dtype, (1, 1, 1), pad, (1, 1, 1))
+        oshape = ops.conv_out_shape(xs, ws, (1, 1, 1), pad, (1, 1, 1))
+        fn = lib.amos_conv2d if op == _lib.AMOS_OP_CONV2D else lib.amos_conv3d
+        outs = []
+        cfg = ops.make_config(_cfg(_lib, tj, ti))
+        need = ops.workspace_bytes(op, d, cfg)
+        assert need == x.itemsize * w.size == lib.amos_conv_packed_weights_bytes(op, ctypes.byref(d))
+        wsb = torch.empty(need + 256, dtype=torch.uint8, device="cuda")
+        ws_ptr = (wsb.data_ptr() + 255) // 256 * 256
+        for mode in ("workspace", "none", "owner"):
+            out = torch.full(oshape, -3, dtype=torch.int32 if dtype == "int8" else torch.float32, device="cuda")
+            c = ops.make_config(_cfg(_lib, tj, ti))
+            if mode == "workspace":
+                rc = fn(ctypes.byref(d), ctypes.byref(c), dx.data_ptr(), dw.data_ptr(), out.data_ptr(), ws_ptr, need, None)
+            elif mode == "none":
+                rc = fn(ctypes.byref(d), ctypes.byref(c), dx.data_ptr(), dw.data_ptr(), out.data_ptr(), None, 0, None)
+            else:
+                packed = torch.empty(need, dtype=torch.uint8, device="cuda")
+                _lib.check(lib.amos_conv_pack_weights(op, ctypes.byref(d), dw.data_ptr(), packed.data_ptr(), None))
+                # [K][T*9][C]: the caller can check the layout itself
+                want = dw.reshape(ws[0], ws[1], -1).permute(0, 2, 1).contiguous()
+                assert torch.equal(packed.view(dw.dtype).view(want.shape), want)
+                c.reserved[0] = _lib.AMOS_FLAG_WEIGHTS_PACKED
+                assert ops.workspace_bytes(op, d, c) == 0
+                rc = fn(ctypes.byref(d), ctypes.byref(c), dx.data_ptr(), packed.data_ptr(), out.data_ptr(), None, 0, None)
+            if rc == _lib.AMOS_ERR_INFEASIBLE and b"load budget" in lib.amos_last_error():
+                pytest.skip(lib.amos_last_error().decode())
+            _lib.check(rc)
+            torch.cuda.synchronize()
+            assert mode != "workspace" or "packed" in ops.kernel_name(op, d, c)
+            outs.append(out)
+        assert torch.equal(outs[0], outs[1]) and torch.equal(outs[0], outs[2])
+        ref = (co.lib_conv2d if op == _lib.AMOS_OP_CONV2D else co.lib_conv3d)(
+            x if op == _lib.AMOS_OP_CONV3D else x[:, :, 0], w if op == _lib.AMOS_OP_CONV3D else w[:, :, 0], dtype, 1,
+            1, 1, **({} if dtype == "int8" else {"acc": "float64"}))
+        got = outs[0].cpu().numpy()
+        _check(got if op == _lib.AMOS_OP_CONV3D else got[:, :, 0], ref, dtype, "weight modes %s %s" % (dtype, tile))
 
 
 def test_conv_nchw_refusals(gpu):
@@ -137,16 +209,16 @@ def test_conv_nchw_benchmark_shapes(gpu):
     rng = np.random.default_rng(0)
     x = rng.uniform(0, 1, (32, 256, 14, 14)).astype(np.float32).astype(np.float16)
     w = (rng.standard_normal((256, 256, 3, 3)) * 0.05).astype(np.float32).astype(np.float16)
-    for tj in (128, 256):
-        got = ops.conv2d(to_device(x, "float16"), to_device(w, "float16"), 1, 1, 1, config=_cfg(_lib, tj)).cpu().numpy()
-        _check(got, co.lib_conv2d(x, w, "float16", 1, 1, 1, acc="float32"), "float16", "fp16 conv2d 64x%d" % tj)
+    for ti, tj in [(64, 128), (64, 256), (32, 128)]:   # (32 x 256: the patch of a tile is above 256 threads' load budget)
+        got = ops.conv2d(to_device(x, "float16"), to_device(w, "float16"), 1, 1, 1, config=_cfg(_lib, tj, ti)).cpu().numpy()
+        _check(got, co.lib_conv2d(x, w, "float16", 1, 1, 1, acc="float32"), "float16", "fp16 conv2d %dx%d" % (ti, tj))
     xi = rng.integers(-128, 128, (64, 128, 28, 28)).astype(np.int8)
     wi = rng.integers(-64, 64, (128, 128, 3, 3)).astype(np.int8)
-    for tj in (128, 256):
-        got = ops.conv2d(to_device(xi, "int8"), to_device(wi, "int8"), 1, 1, 1, config=_cfg(_lib, tj)).cpu().numpy()
-        _check(got, co.lib_conv2d(xi, wi, "int8", 1, 1, 1), "int8", "int8 conv2d 64x%d" % tj)
+    for ti, tj in TILES:
+        got = ops.conv2d(to_device(xi, "int8"), to_device(wi, "int8"), 1, 1, 1, config=_cfg(_lib, tj, ti)).cpu().numpy()
+        _check(got, co.lib_conv2d(xi, wi, "int8", 1, 1, 1), "int8", "int8 conv2d %dx%d" % (ti, tj))
     x3 = rng.standard_normal((2, 64, 16, 56, 56)).astype(np.float32).astype(np.float16)
     w3 = rng.standard_normal((64, 64, 3, 3, 3)).astype(np.float32).astype(np.float16)
-    for tj in (128, 256):
-        got = ops.conv3d(to_device(x3, "float16"), to_device(w3, "float16"), 1, 1, 1, config=_cfg(_lib, tj)).cpu().numpy()
-        _check(got, co.lib_conv3d(x3, w3, "float16", 1, 1, 1, acc="float32"), "float16", "conv3d 64x%d" % tj)
+    for ti, tj in [(64, 128), (64, 256), (32, 128)]:   # (32 x 256: the patch of a tile is above 256 threads' load budget)
+        got = ops.conv3d(to_device(x3, "float16"), to_device(w3, "float16"), 1, 1, 1, config=_cfg(_lib, tj, ti)).cpu().numpy()
+        _check(got, co.lib_conv3d(x3, w3, "float16", 1, 1, 1, acc="float32"), "float16", "conv3d %dx%d" % (ti, tj))
