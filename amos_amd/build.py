@@ -32,14 +32,20 @@ def build(verbose=True, jobs=8):
         cmd = [hipcc] + HIP_FLAGS + inc + ["-c", src, "-o", obj]
         if verbose:
             print(" ".join(cmd), flush=True)
-        procs.append((src, subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT)))
-        while sum(p.poll() is None for _, p in procs) >= jobs:
-            for _, p in procs:
+        # (the compiler's output goes to a file: a pipe that nobody reads while we wait for the
+        # process fills up after 64 KB of diagnostics and the compiler then blocks for good)
+        log = open(obj + ".log", "w+b")
+        procs.append((src, subprocess.Popen(cmd, stdout=log, stderr=subprocess.STDOUT), log))
+        while sum(p.poll() is None for _, p, _ in procs) >= jobs:
+            for _, p, _ in procs:
                 if p.poll() is None:
                     p.wait()
                     break
-    for src, p in procs:
-        out, _ = p.communicate()
+    for src, p, log in procs:
+        p.wait()
+        log.seek(0)
+        out = log.read()
+        log.close()
         text = "\n".join(l for l in out.decode().splitlines() if "packed-fp32-ops" not in l)
         if p.returncode != 0:
             raise RuntimeError("hipcc failed on %s:\n%s" % (src, text))

@@ -331,7 +331,7 @@ struct Plan {
   size_t fewc_lds;
   // convolution read straight from NCDHW / KCTRS (0 = not used)
   int nchw;
-  int nchw_wmode, nchw_pt;
+  int nchw_wmode, nchw_pt, nchw_groups, nchw_nwl;
   int nchw_pack;            // 1: the weights are packed into the workspace in front of the kernel
   const void* nchw_w_src;   // ... from here
   ConvNchwParams nc;
@@ -784,10 +784,16 @@ static int plan_conv(Plan& pl, int op, const amos_conv_desc_t* d, const amos_ker
     q.split_stride = 0;
     q.div_cc = nchw_make_div((uint32_t)q.c_chunks);
     q.div_odpq = nchw_make_div((uint32_t)(OD * OP * OQ));
-    q.dbg = getenv("AMOS_NCHW_DBG") ? (long long*)strtoull(getenv("AMOS_NCHW_DBG"), nullptr, 0) : nullptr;
-    q.dbg_flags = getenv("AMOS_NCHW_DBG_FLAGS") ? atoi(getenv("AMOS_NCHW_DBG_FLAGS")) : 0;
     pl.nchw = 1;
-    pl.nchw_pt = np.groups_per_thread;
+    // rounds of the loader waves over the patch's load groups: one with packed weights, else two
+    // at most (int8, with sixteen channels per chunk and twice the staging registers per group: one)
+    const bool packed = pl.nchw_wmode == NCHW_W_PACKED;
+    pl.nchw_nwl = nchw_loader_waves(packed, np.max_groups);
+    const int per_round = 16 * pl.nchw_nwl;
+    pl.nchw_pt = std::max(1, (np.max_groups + per_round - 1) / per_round);
+    pl.nchw_groups = np.max_groups;
+    if (pl.nchw_pt > (packed || pl.dt == DT_I8 ? 1 : 2))
+      return set_error(AMOS_ERR_INFEASIBLE, "NCDHW-direct convolution not applicable: input patch of a tile above the threads' load budget");
     pl.nchw_lds = np.lds;
     memset(&pl.cfg, 0, sizeof(pl.cfg));
     pl.cfg = *cfg;
@@ -1043,14 +1049,14 @@ static int launch_conv(const Plan& pl, hipStream_t stream) {
   return 0;
 }
 
-static ConvNchwInstance* pick_conv_nchw(int dt, int ti, int tj, int wmode, int pt) {
-  if (dt == DT_F16) return pick_conv_nchw_f16(ti, tj, wmode, pt);
-  if (dt == DT_BF16) return pick_conv_nchw_bf16(ti, tj, wmode, pt);
-  return pick_conv_nchw_i8(ti, tj, wmode, pt);
+static ConvNchwInstance* pick_conv_nchw(int dt, int ti, int tj, int wmode, int pt, int nwl) {
+  if (dt == DT_F16) return pick_conv_nchw_f16(ti, tj, wmode, pt, nwl);
+  if (dt == DT_BF16) return pick_conv_nchw_bf16(ti, tj, wmode, pt, nwl);
+  return pick_conv_nchw_i8(ti, tj, wmode, pt, nwl);
 }
 
 static int launch_conv_nchw(const Plan& pl, hipStream_t stream) {
-  ConvNchwInstance* inst = pick_conv_nchw(pl.dt, pl.cfg.tile_i, pl.cfg.tile_j, pl.nchw_wmode, pl.nchw_pt);
+  ConvNchwInstance* inst = pick_conv_nchw(pl.dt, pl.cfg.tile_i, pl.cfg.tile_j, pl.nchw_wmode, pl.nchw_pt, pl.nchw_nwl);
   if (!inst) return set_error(AMOS_ERR_INFEASIBLE, "no NCDHW-direct convolution instance");
   hipError_t attr_err = hipSuccess;
   std::call_once(inst->once, [&] {
@@ -1070,7 +1076,8 @@ static int launch_conv_nchw(const Plan& pl, hipStream_t stream) {
   if (inst->bi != pl.cfg.tile_i || inst->bj != pl.cfg.tile_j || q.c_chunks < 1 || q.max_pos < 4 ||
       q.max_pos > nchw_max_positions(inst->bj) ||
       pl.nchw_lds != (size_t)2 * 9 * inst->bi * 64 + (size_t)2 * nchw_patch_buffer_bytes(inst->bj) ||
-      inst->threads != inst->bi * 8)
+      inst->threads != inst->bi * 8 + 64 * pl.nchw_nwl || inst->loader_waves != pl.nchw_nwl ||
+      inst->groups_per_thread != pl.nchw_pt || pl.nchw_pt * 16 * pl.nchw_nwl < pl.nchw_groups)
     return set_error(AMOS_ERR_BAD_ARG, "inconsistent plan for %s", inst->name);
   if (pl.nchw_pack)
     launch_conv_pack_weights(pl.dt == DT_I8 ? 1 : 2, pl.nchw_w_src, (void*)q.w, q.s.K, q.s.C, q.s.T * 9, stream);
@@ -1496,7 +1503,7 @@ const char* amos_kernel_name(int op, const void* desc, const amos_kernel_config_
   static char dummy_ws[256] __attribute__((aligned(256)));
   if (make_plan(pl, op, desc, cfg, dummy, dummy, dummy, dummy_ws, (size_t)-1)) return nullptr;
   if (pl.nchw) {
-    ConvNchwInstance* ni = pick_conv_nchw(pl.dt, pl.cfg.tile_i, pl.cfg.tile_j, pl.nchw_wmode, pl.nchw_pt);
+    ConvNchwInstance* ni = pick_conv_nchw(pl.dt, pl.cfg.tile_i, pl.cfg.tile_j, pl.nchw_wmode, pl.nchw_pt, pl.nchw_nwl);
     return ni ? ni->name : nullptr;
   }
   if (pl.dw) return depthwise_name(pl.dt, pl.dw - 1);

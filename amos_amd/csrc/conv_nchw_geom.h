@@ -43,6 +43,13 @@ constexpr int kNchwPosBytes = 64;   // bytes of channels per patch position and 
 
 // n / d for 0 <= n < 2^31 by a multiplication with a host-built constant (the extents are known
 // when the kernel is launched; a hardware-less integer division costs dozens of instructions)
+// Loader waves of a workgroup (beside its matrix-core waves): they fetch and transpose the patch,
+// 16 load groups (x four chunks of channels) per wave and round.  Four of them; eight for a patch
+// of more than 64 load groups where the weights are packed (copied without registers: the kernel
+// then fits the 128 registers that 16 waves per CU leave each) -- one round of eight waves keeps
+// twice as many loads in flight as two rounds of four.
+constexpr int nchw_loader_waves(bool packed, int groups) { return packed && groups > 64 ? 8 : 4; }
+
 struct NchwDiv {
   uint32_t magic, shift, one, d;
 };
@@ -158,6 +165,14 @@ AMOS_HD int nchw_frag_chunk(int q) { return q; }
 // the row (of sixteen) that the lanes 4x .. 4x+3 of a wave fill when a wave writes sixteen rows
 // of a weight tile with one store
 AMOS_HD int nchw_row_of_slot(int x) { return (x & 3) | ((x & 4) << 1) | ((x & 8) >> 1); }
+// the inverse of nchw_position_offset inside a 1 KB block of 16 rows: which (row, chunk) lives in
+// 16-byte slot x = 0..63 (a direct global -> LDS copy puts lane x's bytes there)
+AMOS_HD void nchw_unit_of_slot(int x, int* row, int* chunk) {
+  const int hi = (x >> 4) & 1;
+  const int y = (x & 15) ^ (hi << 2);
+  *row = (x >> 5) * 8 + (y >> 1);
+  *chunk = hi * 2 + (y & 1);
+}
 // ... of the position in window row hr, window column wc of slice `q`
 AMOS_HD int nchw_lds_offset(const NchwShape& s, const NchwSeg& q, int hr, int wc, int chunk) {
   return nchw_position_offset(q.pos0 + hr * s.Wp + wc, chunk);

@@ -1,22 +1,26 @@
-// Implicit-GEMM forward convolution (3x3 windows, conv2d / conv3d) that reads the tensors as the
-// caller holds them -- NCDHW activations, KCTRS weights -- in ONE launch and without a workspace:
+// Implicit-GEMM forward convolution (3x3 windows, conv2d / conv3d) that reads the activations as
+// the caller holds them (NCDHW) in ONE launch:
 //
 //   Out(i = output channel, j = (image, od, op, oq)) = sum_k W(i, k) * Col(j, k),  k = (t, c, r, s)
 //
 // The matrix core wants, per lane, 16 contiguous bytes of K of one row / column.  Neither tensor
-// offers that (in NCDHW the positions are contiguous, in KCTRS the window taps), so both operands
-// are transposed in registers on their way from global memory to LDS:
-//   * activations: a thread fetches, for one 16-byte chunk of channels, one 8-byte run of input
-//     positions per channel (coalesced: 16 lanes cover 128 contiguous bytes of a channel plane),
-//     turns them with byte permutes into one 16-byte vector of channels per position and stores
-//     those into the zero-padded patch [position][64 bytes of channels] of the tile;
-//   * weights: a thread fetches the nine taps of a chunk of channels of one output channel (144
-//     contiguous bytes in 2-d; per channel an unaligned 18 / 9 byte run in 3-d), and writes one
+// offers that (in NCDHW the positions are contiguous, in KCTRS the window taps):
+//   * activations are transposed in registers on their way to LDS: a loader thread fetches, for
+//     one 16-byte chunk of channels, one 8-byte run of input positions per channel (16 lanes cover
+//     128 contiguous bytes of a channel plane), turns them with byte permutes into one 16-byte
+//     vector of channels per position and stores those into the zero-padded patch
+//     [position][64 bytes of channels] of the tile;
+//   * weights come packed as [K][T*9][C] (amos_conv_pack_weights: by the same call into the
+//     workspace, or once by their owner) and are copied into LDS as they are, 16 bytes a lane,
+//     without passing through registers; or, with no workspace, from the caller's KCTRS tensor:
+//     a loader thread fetches the nine taps of a chunk of channels of one output channel (144
+//     contiguous bytes in 2-d; per channel an unaligned 18 / 9 byte run in 3-d) and writes one
 //     16-byte vector of channels per tap into that tap's weight tile [row][64 bytes].
 // A macro step is (depth tap, 64 bytes of channels): its patch serves all nine taps (a tap only
 // shifts the position a lane reads) and its nine weight tiles are resident together, both double
-// buffered, so a workgroup meets at ONE barrier per macro step = per nine K steps; the loads of
-// macro step m+2 and the transposition of m+1 run under the matrix-core work of m.
+// buffered, so a workgroup meets at ONE barrier per macro step = per nine K steps.  Loader waves
+// bring in macro step m+1 (their loads two macro steps ahead of the use) while the matrix-core
+// waves compute macro step m.
 //
 // What the reference does here: separate kernels write the padded tensor, the im2col matrix and
 // the reordered weights to memory before its "kernel2" (README.md:344-424,
@@ -47,12 +51,17 @@ struct ConvNchwParams {
   int64_t split_stride;  // elements between the partial outputs of the split-K blocks
   NchwDiv div_cc, div_odpq;
   EpiParams epi;         // fused tail: Y = acc + cast(D), D laid out like Y
-  long long* dbg;        // DEBUG: per-workgroup timestamps
-  int dbg_flags;         // DEBUG: 1 = no staging stores, 2 = no global loads after the prologue
 };
 
 #define AMOS_LDS_ADDR(off) ((__attribute__((address_space(3))) char*)(size_t)(off))
 enum { NCHW_W_KCTRS = 0, NCHW_W_KCRS = 1, NCHW_W_PACKED = 2 };
+// a pointer that is the same in every lane, as a scalar register pair (what an "s" operand of an
+// assembly statement needs; the compiler does not always see the uniformity by itself)
+__device__ __forceinline__ const char* nchw_uniform(const char* ptr) {
+  const uint64_t a = (uint64_t)ptr;
+  const unsigned lo = __builtin_amdgcn_readfirstlane((unsigned)a), hi = __builtin_amdgcn_readfirstlane((unsigned)(a >> 32));
+  return (const char*)(((uint64_t)hi << 32) | lo);
+}
 template <int N> struct NchwSet { static constexpr int value = N; };
 // f(NchwSet<B>{}), ..., f(NchwSet<E - 1>{}): a loop whose counter is a constant in every iteration
 template <int B, int E, typename F>
@@ -107,22 +116,29 @@ __global__ __launch_bounds__(256) void amos_conv_pack_weights_kernel(const T* __
 constexpr int nchw_patch_buffer_bytes(int bj) { return bj <= 128 ? 32 * 1024 : 40 * 1024; }
 constexpr int nchw_max_positions(int bj) { return nchw_patch_buffer_bytes(bj) / kNchwPosBytes - 16; }
 
-// BI x BJ: output channels x output positions of a workgroup; WI x WJ: its wave grid; PT: load
-// groups a thread may own per macro step; WMODE: where the weights come from -- NCHW_W_KCTRS: the
-// caller's tensor, per channel an unaligned run of nine taps; NCHW_W_KCRS: the same where a chunk
-// of channels is one contiguous, 16-byte aligned run (conv2d with aligned weights);
-// NCHW_W_PACKED: [K][T*9][C], written by amos_conv_pack_weights (into the workspace by the same
-// call, or once by the owner of the weights): 16-byte loads that four lanes per row make
-// contiguous, no transposition; DEPTH: macro steps a global load
-// has to land (1 or 2 sets of staging registers); OCC: waves per SIMD the compiler leaves room for
-// (the register budget of a wave is 512 / OCC)
-template <int DT, int BI, int BJ, int WI, int WJ, int PT, int WMODE, int DEPTH, int OCC>
-__global__ __launch_bounds__(64 * WI * WJ, OCC) void amos_conv_nchw(const ConvNchwParams p) {
+
+// BI x BJ: output channels x output positions of a workgroup; WI x WJ: the grid of its
+// matrix-core waves; NWL: its loader waves; PTL: load groups of the patch per loader thread (the
+// loaders take 16 * NWL * PTL groups); WMODE: where the weights come from -- NCHW_W_KCTRS: the caller's tensor, per channel
+// an unaligned run of nine taps; NCHW_W_KCRS: the same where a chunk of channels is one
+// contiguous, 16-byte aligned run (conv2d with aligned weights); NCHW_W_PACKED: [K][T*9][C],
+// written by amos_conv_pack_weights (into the workspace by the same call, or once by the owner of
+// the weights): copied into LDS as they are, 16 bytes a lane, without passing through registers.
+//
+// Two kinds of waves.  A memory instruction of 64 lanes occupies the CU's address unit for 10-25
+// cycles, and a wave that cannot issue it stalls with everything behind it, matrix-core
+// instructions included: with loads and matrix-core work in the same waves a macro step took twice
+// its matrix-core time however the loads were spread.  So four loader waves fetch, transpose and
+// store the operands of macro step m + 1 (their loads two macro steps ahead of their use) while
+// the WI x WJ matrix-core waves do nothing but read fragments of macro step m and multiply; the
+// two kinds meet at the one barrier per macro step.
+template <int DT, int BI, int BJ, int WI, int WJ, int PTL, int WMODE, int NWL>
+__global__ __launch_bounds__(64 * (WI * WJ + NWL)) void amos_conv_nchw(const ConvNchwParams p) {
   typedef Mfma16<DT> MM;
   typedef typename MM::acc_t acc_t;
   typedef typename Mfma<DT>::out_t out_t;
   constexpr int ES = Mfma<DT>::ES;
-  constexpr int NW = WI * WJ, NT = 64 * NW;
+  constexpr int NWM = WI * WJ, NTM = 64 * NWM, NTL = 64 * NWL, NTA = NTM + NTL;
   constexpr int TI = BI / (16 * WI), TJ = BJ / (16 * WJ);
   static_assert(TI >= 1 && TJ >= 1 && TI * WI * 16 == BI && TJ * WJ * 16 == BJ, "wave tile");
   constexpr int PG = 8 / ES;      // input positions per 8-byte load
@@ -132,17 +148,15 @@ __global__ __launch_bounds__(64 * WI * WJ, OCC) void amos_conv_nchw(const ConvNc
   constexpr int WTILE = BI * 64;  // one tap's weight tile
   constexpr int WBUF = RS * WTILE;
   constexpr int PBUF = nchw_patch_buffer_bytes(BJ);
-  constexpr int UNITS = BI * 4;   // (row, chunk of channels) pairs of a macro step's weights
-  constexpr int WU = (UNITS + NT - 1) / NT;
   constexpr bool T1 = WMODE == NCHW_W_KCRS, PACKED = WMODE == NCHW_W_PACKED;
   constexpr int CHW = T1 ? 0 : (ES == 2 ? 5 : 3);       // dwords of one channel's taps (3-d path)
   constexpr int WRAW = T1 ? 36 : CG * CHW;              // dwords of a unit's raw weights
-  // packed weights: a thread copies one 16-byte chunk of one row of one tap per item; the taps of
-  // a macro step are 9 * BI * 4 items = 4.5 per thread (taps 2v and 2v + 1 for the lower / upper
-  // half of the threads)
-  static_assert(BI * 8 == NT, "a tap's weight tile is half a round of the threads' chunks");
-  constexpr int WITEMS = 5;
-  static_assert(DEPTH == 1 || DEPTH == 2, "one or two sets of staging registers");
+  constexpr int UNITS = BI * 4;   // (row, chunk of channels) pairs of a macro step's weights
+  static_assert(UNITS <= NTL, "one weight unit per loader thread at most");
+  // packed weights: copied in 1 KB blocks (16 rows x 64 bytes); a tap's tile is NB of them
+  constexpr int NB = BI / 16;
+  constexpr int NPL = PTL * CG;   // patch loads per thread and macro step
+  static_assert(2 * NPL <= 63, "the counter of loads in flight has six bits");
   // LDS, by byte offset from 0 (the kernel has no static LDS; the host checks that):
   //   [2][9][BI * 64] weight tiles | [2][PBUF] patches, the last 1 KB of each a dump line
   constexpr unsigned PBASE = 2 * WBUF;
@@ -150,13 +164,8 @@ __global__ __launch_bounds__(64 * WI * WJ, OCC) void amos_conv_nchw(const ConvNc
 
   const NchwShape& s = p.s;
   const int t = threadIdx.x;
-  int dbg_k = 0;
-  auto stamp = [&]() __attribute__((always_inline)) { if (p.dbg && t == 0 && dbg_k < 16) p.dbg[blockIdx.x * 16 + dbg_k++] = clock64(); };
-  stamp();
   const int lane = t & 63;
   const int wave = __builtin_amdgcn_readfirstlane(t >> 6);
-  const int wi = wave / WJ, wj = wave % WJ;
-  const int frag_row = lane & 15, frag_q = lane >> 4;
 
   // Workgroups are dealt round-robin to the 8 XCDs: give each XCD a contiguous run of tiles, the
   // tiles of one patch (tile_i fastest) next to each other, so that an XCD's L2 sees a patch once
@@ -170,62 +179,62 @@ __global__ __launch_bounds__(64 * WI * WJ, OCC) void amos_conv_nchw(const ConvNc
   const int bi0 = tile_i * BI, bj0 = tile_j * BJ;
   const int HW = s.H * s.W;
   const int64_t DHW = (int64_t)s.D * HW;
-  // ---- this thread's share of the weights ----------------------------------------------------------
-  unsigned w_src[WU];   // byte offset of (row, first channel of the chunk): below 4 GiB
-  unsigned w_dst[WU];   // LDS address inside a tap's tile of the first buffer
-  bool w_on[WU];
   const int TRS = s.T * RS;
-  const int upper = __builtin_amdgcn_readfirstlane(t >= NT / 2 ? 1 : 0);   // packed: which of a pair of taps
-#pragma unroll
-  for (int v = 0; v < WU; ++v) {
-    // (with fewer units than threads they go to the last waves: the first ones own the patch's
-    // load groups, and a macro step waits for the wave with the most staging work)
-    const int u = PACKED ? (t & (NT / 2 - 1)) : UNITS < NT ? t - (NT - UNITS) : t + NT * v;
-    // (lanes 4x .. 4x+3 of a wave take row nchw_row_of_slot(x) of their sixteen: no bank conflicts)
-    const int cq = u & 3, row = ((u >> 6) * 16 + nchw_row_of_slot((u >> 2) & 15)) & (BI - 1);
-    w_on[v] = u >= 0 && u < UNITS;
-    const int k = bi0 + row < s.K ? bi0 + row : s.K - 1;
-    if (PACKED) {
-      w_src[v] = (unsigned)(((int64_t)k * TRS * s.C) * ES + cq * 16);
-      w_dst[v] = (unsigned)(nchw_position_offset(row, cq) + upper * WTILE);
-    } else {
-      w_src[v] = (unsigned)((((int64_t)k * s.C + cq * CG) * TRS) * ES);
-      w_dst[v] = (unsigned)nchw_position_offset(row, cq);
-    }
-  }
   const int m_begin = blockIdx.y * p.macro_per_split;
   int m_end = m_begin + p.macro_per_split;
   if (m_end > p.macro_steps) m_end = p.macro_steps;
 
-  unsigned wraw[DEPTH][WU][PACKED ? WITEMS * 4 : WRAW];
-  unsigned praw[DEPTH][PT][CG][2];
-
-  auto load_weights = [&](auto set_c, int m) __attribute__((always_inline)) {
-    constexpr int SET = decltype(set_c)::value;
-    const int tt = nchw_div(m, p.div_cc), cc = m - tt * p.c_chunks;
-    // (a wave-uniform base plus a 32-bit lane offset: one address register per load, not two)
-    if constexpr (PACKED) {
-      // tap 2v + upper of this macro step: row k's 64 bytes of the chunk at [k][tt * 9 + tap][cc * CK]
-      const char* const wm = p.w + (((int64_t)tt * RS + upper) * s.C + (int64_t)cc * CK) * ES;
-#pragma unroll
-      for (int v = 0; v < WITEMS; ++v) {
-        if (2 * v + upper < RS) {
-          const v4i x = *(const v4i*)(wm + (int64_t)(2 * v) * s.C * ES + w_src[0]);
-          wraw[SET][0][4 * v] = x.x; wraw[SET][0][4 * v + 1] = x.y; wraw[SET][0][4 * v + 2] = x.z; wraw[SET][0][4 * v + 3] = x.w;
-        }
-      }
-      return;
+  // both kinds of waves: clear the patch buffers (padding positions are never written), meet
+  auto clear_patches = [&]() __attribute__((always_inline)) {
+    for (int i = t; i < p.max_pos * 4; i += NTA) {
+      *(v4i*)AMOS_LDS_ADDR(PBASE + i * 16) = v4i{0, 0, 0, 0};
+      *(v4i*)AMOS_LDS_ADDR(PBASE + PBUF + i * 16) = v4i{0, 0, 0, 0};
     }
-    const char* const wm = p.w + ((int64_t)cc * CK * TRS + tt * RS) * ES;
-#pragma unroll
-    for (int v = 0; v < WU; ++v) {
-      if (!w_on[v]) continue;
-      const char* src = wm + w_src[v];
+  };
+  auto meet = [&]() __attribute__((always_inline)) { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); };
+
+  if (wave >= NWM) {
+    // ==================================== loader waves ==============================================
+    // The loaders' memory instructions are all loads into registers: "at most N loads in flight"
+    // says which loads have landed only while loads complete in the order of their issue, and a
+    // direct copy into LDS and a load into registers do not keep that order between them
+    // (measured: with both in one wave a counted wait let through loads that were still on their
+    // way).  The direct copies of packed weights are therefore issued by the matrix-core waves.
+    const int tl = t - NTM;
+    constexpr int NTP = NTL;
+    const bool patch_wave = true;
+    const int tlp = tl;
+    // ---- this thread's share of the weights ----------------------------------------------------
+    unsigned w_src[1] = {0};   // byte offset of (row, first channel of the chunk): below 4 GiB
+    unsigned w_dst = 0;        // LDS address inside a tap's tile of the first buffer
+    bool w_on = !PACKED;
+    if (!PACKED) {
+      // (with fewer units than loader threads they go to the last waves)
+      const int u = tl - (NTL - UNITS);
+      // (lanes 4x .. 4x+3 of a wave take row nchw_row_of_slot(x) of their sixteen: no bank conflicts)
+      const int cq = u & 3, row = ((u >> 6) * 16 + nchw_row_of_slot((u >> 2) & 15)) & (BI - 1);
+      w_on = u >= 0;
+      const int k = bi0 + row < s.K ? bi0 + row : s.K - 1;
+      w_src[0] = (unsigned)((((int64_t)k * s.C + cq * CG) * TRS) * ES);
+      w_dst = (unsigned)nchw_position_offset(row, cq);
+    }
+    unsigned wraw[PACKED ? 1 : WRAW];
+    typedef unsigned nchw_u2 __attribute__((ext_vector_type(2)));
+    // (two staging sets with packed weights: the patch loads run two macro steps ahead; one set
+    // where the weights pass through registers too and every wait is for all loads anyway)
+    constexpr int SETS = PACKED ? 2 : 1;
+    nchw_u2 praw[SETS][PTL][CG] = {};
+
+    // weights that pass through registers: the raw taps of this thread's unit
+    auto load_weights = [&](int m) __attribute__((always_inline)) {
+      if (!w_on) return;
+      const int tt = nchw_div(m, p.div_cc), cc = m - tt * p.c_chunks;
+      const char* const src = p.w + ((int64_t)cc * CK * TRS + tt * RS) * ES + w_src[0];
       if (T1) {
 #pragma unroll
         for (int i = 0; i < 9; ++i) {
           const v4i x = *(const v4i*)(src + i * 16);
-          wraw[SET][v][4 * i] = x.x; wraw[SET][v][4 * i + 1] = x.y; wraw[SET][v][4 * i + 2] = x.z; wraw[SET][v][4 * i + 3] = x.w;
+          wraw[4 * i] = x.x; wraw[4 * i + 1] = x.y; wraw[4 * i + 2] = x.z; wraw[4 * i + 3] = x.w;
         }
       } else {
 #pragma unroll
@@ -233,53 +242,236 @@ __global__ __launch_bounds__(64 * WI * WJ, OCC) void amos_conv_nchw(const ConvNc
           const char* sc = src + (int64_t)ci * TRS * ES;
           if (ES == 2) {
             const v4i x = ((const NchwUnaligned16*)sc)->v;
-            wraw[SET][v][ci * CHW] = x.x; wraw[SET][v][ci * CHW + 1] = x.y; wraw[SET][v][ci * CHW + 2] = x.z; wraw[SET][v][ci * CHW + 3] = x.w;
-            wraw[SET][v][ci * CHW + 4] = *(const unsigned short*)(sc + 16);
+            wraw[ci * CHW] = x.x; wraw[ci * CHW + 1] = x.y; wraw[ci * CHW + 2] = x.z; wraw[ci * CHW + 3] = x.w;
+            wraw[ci * CHW + 4] = *(const unsigned short*)(sc + 16);
           } else {
             const uint2 x = ((const NchwUnaligned8*)sc)->v;
-            wraw[SET][v][ci * CHW] = x.x; wraw[SET][v][ci * CHW + 1] = x.y;
-            wraw[SET][v][ci * CHW + 2] = *(const unsigned char*)(sc + 8);
+            wraw[ci * CHW] = x.x; wraw[ci * CHW + 1] = x.y;
+            wraw[ci * CHW + 2] = *(const unsigned char*)(sc + 8);
           }
         }
       }
+    };
+    // raw byte index of byte bb of channel ci at tap tap
+    auto wbyte = [](int ci, int tap, int bb) __attribute__((always_inline)) {
+      return T1 ? (ci * 9 + tap) * ES + bb : ci * CHW * 4 + tap * ES + bb;
+    };
+    // ... transposed: per tap one 16-byte vector of channels into that tap's tile
+    auto store_weights = [&](auto buf_c) __attribute__((always_inline)) {
+      if (!w_on) return;
+#pragma unroll
+      for (int tap = 0; tap < RS; ++tap) {
+        v4i o;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          if (ES == 2)
+            o[j] = (int)nchw_gather<ES>(wraw, wbyte(2 * j, tap, 0), wbyte(2 * j, tap, 1), wbyte(2 * j + 1, tap, 0),
+                                        wbyte(2 * j + 1, tap, 1));
+          else
+            o[j] = (int)nchw_gather<ES>(wraw, wbyte(4 * j, tap, 0), wbyte(4 * j + 1, tap, 0), wbyte(4 * j + 2, tap, 0),
+                                        wbyte(4 * j + 3, tap, 0));
+        }
+        *(v4i*)AMOS_LDS_ADDR(w_dst + decltype(buf_c)::value * WBUF + tap * WTILE) = o;
+      }
+    };
+    // the first weights go out before the tile's geometry is worked out
+    if (m_begin < m_end) {
+      if constexpr (!PACKED) load_weights(m_begin);
+    }
+
+    const NchwTile tile = nchw_tile(s, bj0, BJ);
+    // ---- this thread's load groups of the patch ------------------------------------------------
+    unsigned p_src[PTL];      // byte offset of (image, first channel of the chunk, depth 0, group): below 4 GiB
+    int p_d0[PTL];            // input depth at depth tap 0
+    unsigned p_dst[PTL][PG];  // LDS addresses (first buffer) of the group's positions; the dump line
+                              // for positions that are not part of the window
+#pragma unroll
+    for (int v = 0; v < PTL; ++v) {
+      const int q = tlp + NTP * v;
+      const int cg = q & 3, grp = q >> 2;
+      const bool on = patch_wave && grp < tile.ngroups;
+      int f = 0;
+      const NchwSeg seg = nchw_group(s, tile, on ? grp : 0, &f);
+      p_src[v] = (unsigned)((((int64_t)seg.n * s.C + cg * CG) * DHW + f) * ES);
+      p_d0[v] = seg.d0;
+#pragma unroll
+      for (int i = 0; i < PG; ++i) {
+        // (the upper half of a wave stores its positions in the order 1, 0, 3, 2, ...: see the bank
+        // conflict notes of the geometry header)
+        const int off = on ? nchw_writer_offset(s, seg, f + (i ^ (lane >> 5)), cg) : -1;
+        p_dst[v][i] = PBASE + (off >= 0 ? (unsigned)off : DUMP + (unsigned)lane * 16);
+      }
+    }
+    // byte selectors that pick position i (lower half of the wave) or i ^ 1 (upper half) out of a
+    // staging dword: 16-bit types hold two positions per dword, int8 four
+    unsigned p_sel[ES == 2 ? 2 : 4];
+#pragma unroll
+    for (int i = 0; i < (ES == 2 ? 2 : 4); ++i) {
+      const int pos = i ^ (lane >> 5);
+      p_sel[i] = ES == 2 ? (pos ? 0x07060302u : 0x05040100u) : ((unsigned)pos | ((unsigned)(4 + pos) << 8));
+    }
+    // the patch loads of macro step m into staging set SET.  Every lane loads, from a depth
+    // clamped into the tensor: a load that some lanes skip needs its registers preset, and the
+    // compiler waits for ALL loads in flight before it writes a register that an earlier load may
+    // still own; a depth in the padding is zeroed when the vector is stored, lanes without a
+    // group store into the dump line.  As assembly, and waited for by landed<N>(): the
+    // compiler's own bookkeeping of loads in flight around the loop ends in "wait for all of
+    // them" in front of the first use, which is the wait the second staging set is there to avoid.
+    auto load_patch = [&](auto set_c, int m) __attribute__((always_inline)) {
+      constexpr int SET = decltype(set_c)::value % SETS;
+      const int tt = nchw_div(m, p.div_cc), cc = m - tt * p.c_chunks;
+      const char* const xm0 = p.x + (int64_t)cc * CK * DHW * ES;
+#pragma unroll
+      for (int v = 0; v < PTL; ++v) {
+        int d = p_d0[v] + tt * s.dd;
+        d = d < 0 ? 0 : d >= s.D ? s.D - 1 : d;
+        // (the depth is the lane's own: its offset stays below 4 GiB like the rest of the tensor)
+        const unsigned off = p_src[v] + (unsigned)d * (unsigned)(HW * ES);
+#pragma unroll
+        for (int ci = 0; ci < CG; ++ci) {
+          const char* const plane = nchw_uniform(xm0 + (int64_t)ci * DHW * ES);
+          nchw_u2 x;
+          asm volatile("s_nop 4\n\tglobal_load_dwordx2 %0, %1, %2" : "=v"(x) : "v"(off), "s"(plane) : "memory");
+          praw[SET][v][ci] = x;
+        }
+      }
+    };
+    // at most N of this wave's loads are still in flight (they land in the order of their
+    // issue); staging set SET is read only behind this point
+    auto landed = [&](auto n_c, auto set_c) __attribute__((always_inline)) {
+      constexpr int SET = decltype(set_c)::value % SETS;
+      asm volatile("s_waitcnt vmcnt(%0)" ::"n"(decltype(n_c)::value) : "memory");
+#pragma unroll
+      for (int v = 0; v < PTL; ++v)
+#pragma unroll
+        for (int ci = 0; ci < CG; ++ci) {
+          nchw_u2 x = praw[SET][v][ci];
+          asm volatile("" : "+v"(x));
+          praw[SET][v][ci] = x;
+        }
+    };
+    // the patch of macro step m out of staging set SET into patch buffer BUF: per position one
+    // 16-byte vector of channels
+    auto store_patch = [&](auto set_c, auto buf_c, int m) __attribute__((always_inline)) {
+      constexpr int SET = decltype(set_c)::value % SETS;
+      const int tt = nchw_div(m, p.div_cc);
+#pragma unroll
+      for (int v = 0; v < PTL; ++v) {
+        const bool ok = (unsigned)(p_d0[v] + tt * s.dd) < (unsigned)s.D;
+#pragma unroll
+        for (int i = 0; i < PG; ++i) {
+          v4i o;
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            if constexpr (ES == 2) {
+              o[j] = (int)__builtin_amdgcn_perm(praw[SET][v][2 * j + 1][i >> 1], praw[SET][v][2 * j][i >> 1], p_sel[i & 1]);
+            } else {
+              const unsigned sel = p_sel[i & 3];
+              const unsigned lo = __builtin_amdgcn_perm(praw[SET][v][4 * j + 1][i >> 2], praw[SET][v][4 * j][i >> 2], sel);
+              const unsigned hi = __builtin_amdgcn_perm(praw[SET][v][4 * j + 3][i >> 2], praw[SET][v][4 * j + 2][i >> 2], sel);
+              o[j] = (int)__builtin_amdgcn_perm(hi, lo, 0x05040100u);
+            }
+          }
+          if (!ok) o = v4i{0, 0, 0, 0};
+          *(v4i*)AMOS_LDS_ADDR(p_dst[v][i] + decltype(buf_c)::value * PBUF) = o;
+        }
+      }
+    };
+
+    // ---- prologue: macro step m_begin into the first buffers, the loads of the next one out ------
+    if (patch_wave) {
+      if (m_begin < m_end) load_patch(NchwSet<0>{}, m_begin);
+      if (PACKED && m_begin + 1 < m_end) load_patch(NchwSet<1>{}, m_begin + 1);
+    }
+    clear_patches();
+    meet();
+    if (m_begin < m_end) {
+      if (patch_wave) {
+        if (PACKED && m_begin + 1 < m_end) landed(NchwSet<NPL>{}, NchwSet<0>{});
+        else landed(NchwSet<0>{}, NchwSet<0>{});
+        store_patch(NchwSet<0>{}, NchwSet<0>{}, m_begin);
+        if (!PACKED && m_begin + 1 < m_end) load_patch(NchwSet<0>{}, m_begin + 1);
+      }
+      if constexpr (!PACKED) store_weights(NchwSet<0>{});
+    }
+    meet();
+    // ---- under macro step m of the matrix-core waves: macro step m + 1 into the other buffers
+    // (last read a macro step ago), the patch out of staging set SET while the loads of m + 2 fill
+    // the other set
+    auto under = [&](auto set_c, auto buf_c, int m) __attribute__((always_inline)) {
+      constexpr int SET = decltype(set_c)::value;
+      const bool next = m + 1 < m_end, more = m + 2 < m_end;
+      if constexpr (PACKED) {
+        if (more) load_patch(NchwSet<SET ^ 1>{}, m + 2);
+        if (next) {
+          if (more) landed(NchwSet<NPL>{}, set_c);
+          else landed(NchwSet<0>{}, set_c);
+          store_patch(set_c, buf_c, m + 1);
+        }
+      } else {
+        // (the compiler's loads of the weights and the patch loads share the wave: wait for all)
+        if (next) load_weights(m + 1);
+        if (patch_wave && next) {
+          landed(NchwSet<0>{}, set_c);
+          store_patch(set_c, buf_c, m + 1);
+        }
+        if (patch_wave && more) load_patch(NchwSet<SET ^ 1>{}, m + 2);
+        if (next) store_weights(buf_c);
+      }
+      meet();
+    };
+    // macro step m_begin + r is computed from buffers r & 1; the loaders fill buffers (r + 1) & 1
+    // from staging set (r + 1) & 1
+    for (int m = m_begin; m < m_end; m += 2) {
+      under(NchwSet<1>{}, NchwSet<1>{}, m);
+      if (m + 1 < m_end) under(NchwSet<0>{}, NchwSet<0>{}, m + 1);
+    }
+    return;
+  }
+
+  // ==================================== matrix-core waves ===========================================
+  // Packed weights are copied straight into LDS (global_load_lds, 16 bytes a lane, no registers)
+  // in 1 KB blocks of 16 rows x 64 bytes: wave w takes block w % NB of the taps w / NB + 2 * i.
+  // Lane l's bytes land at l * 16 of the block, so the lane fetches the (row, chunk) that lives
+  // in that slot.  A copy costs the wave some 30 cycles of issue; the copies of macro step m + 1
+  // go out at the start of macro step m and are waited for at its end.
+  //   As assembly: after the builtin the compiler makes every later LDS instruction wait until
+  //   the copy has landed (it cannot tell which LDS bytes the copy writes).  The wait states are
+  //   the ones the compiler would insert, and cannot inside an assembly statement: five between
+  //   a v_readfirstlane that may have produced the address registers and the memory instruction
+  //   that reads them, one between the write of M0 and the copy that takes its LDS address from
+  //   there; without them the copy can run with stale registers.
+  static_assert(NWM == 2 * NB, "two taps per round of the matrix-core waves' copies");
+  constexpr int NWC = (RS + 1) / 2;
+  const int wblock = wave % NB, wtap0 = wave / NB;
+  unsigned w_lane = 0;
+  if (PACKED) {
+    int row16, cq;
+    nchw_unit_of_slot(lane, &row16, &cq);
+    const int row = wblock * 16 + row16;
+    const int k = bi0 + row < s.K ? bi0 + row : s.K - 1;
+    w_lane = (unsigned)(((int64_t)k * TRS * s.C) * ES + cq * 16);
+  }
+  auto copy_weights = [&](auto buf_c, int m) __attribute__((always_inline)) {
+    const int tt = nchw_div(m, p.div_cc), cc = m - tt * p.c_chunks;
+    const char* const wm = p.w + ((int64_t)tt * RS * s.C + (int64_t)cc * CK) * ES;
+    const unsigned lane_off = w_lane;
+#pragma unroll
+    for (int i = 0; i < NWC; ++i) {
+      const int tap = wtap0 + 2 * i;
+      if (tap < RS) {
+        const char* const src = nchw_uniform(wm + (int64_t)tap * s.C * ES);
+        const unsigned dst = decltype(buf_c)::value * WBUF + tap * WTILE + wblock * 1024;
+        asm volatile("s_nop 4\n\ts_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(dst), "v"(lane_off), "s"(src)
+                     : "memory");
+      }
     }
   };
-  // the first weights go out before the tile's geometry is worked out
-  if (m_begin < m_end) load_weights(NchwSet<0>{}, m_begin);
-
+  // the first weights go out before anything else
+  if (PACKED && m_begin < m_end) copy_weights(NchwSet<0>{}, m_begin);
+  const int wi = wave / WJ, wj = wave % WJ;
+  const int frag_row = lane & 15, frag_q = lane >> 4;
   const NchwTile tile = nchw_tile(s, bj0, BJ);
-
-  // ---- this thread's load groups of the patch ------------------------------------------------
-  unsigned p_src[PT];      // byte offset of (image, first channel of the chunk, depth 0, group): below 4 GiB
-  int p_d0[PT];            // input depth at depth tap 0
-  bool p_on[PT];
-  unsigned p_dst[PT][PG];  // LDS addresses (first buffer) of the group's positions; the dump line
-                           // for positions that are not part of the window
-#pragma unroll
-  for (int v = 0; v < PT; ++v) {
-    const int q = t + NT * v;
-    const int cg = q & 3, grp = q >> 2;
-    p_on[v] = grp < tile.ngroups;
-    int f = 0;
-    const NchwSeg seg = nchw_group(s, tile, p_on[v] ? grp : 0, &f);
-    p_src[v] = (unsigned)((((int64_t)seg.n * s.C + cg * CG) * DHW + f) * ES);
-    p_d0[v] = seg.d0;
-#pragma unroll
-    for (int i = 0; i < PG; ++i) {
-      // (the upper half of a wave stores its positions in the order 1, 0, 3, 2, ...: see the bank
-      // conflict notes of the geometry header)
-      const int off = p_on[v] ? nchw_writer_offset(s, seg, f + (i ^ (lane >> 5)), cg) : -1;
-      p_dst[v][i] = PBASE + (off >= 0 ? (unsigned)off : DUMP + (unsigned)lane * 16);
-    }
-  }
-  // byte selectors that pick position i (lower half of the wave) or i ^ 1 (upper half) out of a
-  // staging dword: 16-bit types hold two positions per dword, int8 four
-  unsigned p_sel[ES == 2 ? 2 : 4];
-#pragma unroll
-  for (int i = 0; i < (ES == 2 ? 2 : 4); ++i) {
-    const int pos = i ^ (lane >> 5);
-    p_sel[i] = ES == 2 ? (pos ? 0x07060302u : 0x05040100u) : ((unsigned)pos | ((unsigned)(4 + pos) << 8));
-  }
   // ---- fragment addresses: all of them are computed here, the loop only adds immediates ----------
   // weights: [buffer][16-row block]; patch: [tap][16-position block], first buffer
   unsigned a_addr[2][TI];
@@ -299,97 +491,6 @@ __global__ __launch_bounds__(64 * WI * WJ, OCC) void amos_conv_nchw(const ConvNc
     for (int tap = 0; tap < RS; ++tap)
       b_addr[tap][b] = PBASE + (unsigned)nchw_reader_offset(s, column, tap / 3, tap % 3, nchw_frag_chunk(frag_q));
   }
-
-  auto load_patch = [&](auto set_c, int m) __attribute__((always_inline)) {
-    constexpr int SET = decltype(set_c)::value;
-    const int tt = nchw_div(m, p.div_cc), cc = m - tt * p.c_chunks;
-#pragma unroll
-    for (int v = 0; v < PT; ++v) {
-      const int d = p_d0[v] + tt * s.dd;
-      if (p_on[v] && (unsigned)d < (unsigned)s.D) {
-        // (the depth is the lane's own: its offset stays below 4 GiB like the rest of the tensor)
-        const unsigned off = p_src[v] + (unsigned)d * (unsigned)(HW * ES);
-#pragma unroll
-        for (int ci = 0; ci < CG; ++ci) {
-          const char* const xm = p.x + ((int64_t)cc * CK + ci) * DHW * ES;
-          const uint2 x = *(const uint2*)(xm + off);
-          praw[SET][v][ci][0] = x.x; praw[SET][v][ci][1] = x.y;
-        }
-      } else {
-#pragma unroll
-        for (int ci = 0; ci < CG; ++ci) { praw[SET][v][ci][0] = 0; praw[SET][v][ci][1] = 0; }
-      }
-    }
-  };
-  auto load_both = [&](auto set_c, int m) __attribute__((always_inline)) {
-    if (m < m_end) {
-      load_weights(set_c, m);
-      load_patch(set_c, m);
-    }
-  };
-  // raw byte index of byte bb of channel ci at tap tap
-  auto wbyte = [](int ci, int tap, int bb) __attribute__((always_inline)) {
-    return T1 ? (ci * 9 + tap) * ES + bb : ci * CHW * 4 + tap * ES + bb;
-  };
-  // tap `tap` of this thread's weight units of the next macro step: one 16-byte vector of channels
-  auto stage_weights_tap = [&](auto set_c, auto buf_c, auto tap_c) __attribute__((always_inline)) {
-    constexpr int SET = decltype(set_c)::value;
-    constexpr int tap = decltype(tap_c)::value;
-    constexpr unsigned OFF = decltype(buf_c)::value * WBUF + tap * WTILE;
-    if constexpr (PACKED) {
-      // item `tap` (of five) is the chunk of tap 2 * tap + upper: stored as it came
-      if constexpr (tap < WITEMS) {
-        if (2 * tap + upper < RS) {
-          const v4i o = {(int)wraw[SET][0][4 * tap], (int)wraw[SET][0][4 * tap + 1], (int)wraw[SET][0][4 * tap + 2],
-                         (int)wraw[SET][0][4 * tap + 3]};
-          *(v4i*)AMOS_LDS_ADDR(w_dst[0] + decltype(buf_c)::value * WBUF + 2 * tap * WTILE) = o;
-        }
-      }
-      return;
-    }
-#pragma unroll
-    for (int v = 0; v < WU; ++v) {
-      if (!w_on[v]) continue;
-      v4i o;
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        if (ES == 2)
-          o[j] = (int)nchw_gather<ES>(wraw[SET][v], wbyte(2 * j, tap, 0), wbyte(2 * j, tap, 1), wbyte(2 * j + 1, tap, 0),
-                                      wbyte(2 * j + 1, tap, 1));
-        else
-          o[j] = (int)nchw_gather<ES>(wraw[SET][v], wbyte(4 * j, tap, 0), wbyte(4 * j + 1, tap, 0), wbyte(4 * j + 2, tap, 0),
-                                      wbyte(4 * j + 3, tap, 0));
-      }
-      *(v4i*)AMOS_LDS_ADDR(w_dst[v] + OFF) = o;
-    }
-  };
-  // position i of load group v of the next macro step's patch: one 16-byte vector of channels
-  auto stage_patch_pos = [&](auto set_c, auto buf_c, auto e_c) __attribute__((always_inline)) {
-    constexpr int SET = decltype(set_c)::value;
-    constexpr int v = decltype(e_c)::value / PG, i = decltype(e_c)::value % PG;
-    v4i o;
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      if constexpr (ES == 2) {
-        o[j] = (int)__builtin_amdgcn_perm(praw[SET][v][2 * j + 1][i >> 1], praw[SET][v][2 * j][i >> 1], p_sel[i & 1]);
-      } else {
-        const unsigned sel = p_sel[i & 3];
-        const unsigned lo = __builtin_amdgcn_perm(praw[SET][v][4 * j + 1][i >> 2], praw[SET][v][4 * j][i >> 2], sel);
-        const unsigned hi = __builtin_amdgcn_perm(praw[SET][v][4 * j + 3][i >> 2], praw[SET][v][4 * j + 2][i >> 2], sel);
-        o[j] = (int)__builtin_amdgcn_perm(hi, lo, 0x05040100u);
-      }
-    }
-    *(v4i*)AMOS_LDS_ADDR(p_dst[v][i] + decltype(buf_c)::value * PBUF) = o;
-  };
-  // the staging work of a macro step in RS slices, one per tap of the macro step it runs under
-  constexpr int PVEC = PT * PG;                       // patch vectors per thread
-  constexpr int PPER = (PVEC + RS - 1) / RS;          // ... per slice
-  auto stage_slice = [&](auto set_c, auto buf_c, auto tap_c) __attribute__((always_inline)) {
-    constexpr int tap = decltype(tap_c)::value;
-    stage_weights_tap(set_c, buf_c, tap_c);
-    constexpr int E0 = tap * PPER < PVEC ? tap * PPER : PVEC, E1 = (tap + 1) * PPER < PVEC ? (tap + 1) * PPER : PVEC;
-    nchw_static_for<E0, E1>([&](auto e_c) { stage_patch_pos(set_c, buf_c, e_c); });
-  };
 
   acc_t acc[TI][TJ];
 #pragma unroll
@@ -417,59 +518,33 @@ __global__ __launch_bounds__(64 * WI * WJ, OCC) void amos_conv_nchw(const ConvNc
       for (int a = 0; a < TI; ++a) acc[a][b] = MM::run(af[slot][a], bf[slot][b], acc[a][b]);
   };
 
-  stamp();
-  // ---- prologue -------------------------------------------------------------------------------------
-  // the first loads go out before anything else; the patch buffers are cleared under their latency
-  // (padding positions are never written, so both buffers start as zeros)
-  if (m_begin < m_end) load_patch(NchwSet<0>{}, m_begin);
-  if (DEPTH == 2) load_both(NchwSet<DEPTH - 1>{}, m_begin + 1);
-  for (int i = t; i < p.max_pos * 4; i += NT) {
-    *(v4i*)AMOS_LDS_ADDR(PBASE + i * 16) = v4i{0, 0, 0, 0};
-    *(v4i*)AMOS_LDS_ADDR(PBASE + PBUF + i * 16) = v4i{0, 0, 0, 0};
-  }
-  asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
-  if (m_begin < m_end) {
-    nchw_static_for<0, RS>([&](auto tap_c) { stage_slice(NchwSet<0>{}, NchwSet<0>{}, tap_c); });
-    load_both(NchwSet<0>{}, m_begin + DEPTH);
-  }
-  asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
-
-  stamp();
-  // One macro step: nine taps out of buffer BUF; under them the next macro step is transposed
-  // from staging set SET into the other buffer (last read a macro step ago) and the set refilled
-  // with the loads of the macro step DEPTH further on.
-  auto macro_body = [&](auto set_c, auto next_c, auto buf_c, int m) __attribute__((always_inline)) {
-    constexpr bool NEXT = decltype(next_c)::value != 0;
+  clear_patches();
+  meet();
+  if (PACKED) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // the first macro step's weights
+  meet();
+  // One macro step: nine taps out of buffers BUF, then the barrier behind which the loaders have
+  // the other buffers ready and may overwrite these
+  auto macro_step = [&](auto buf_c, int m) __attribute__((always_inline)) {
     constexpr int BUF = decltype(buf_c)::value;
+    if (PACKED && m + 1 < m_end) copy_weights(NchwSet<BUF ^ 1>{}, m + 1);
     read_frags(buf_c, NchwSet<0>{});
     if (NF > 2) read_frags(buf_c, NchwSet<1>{});
     __builtin_amdgcn_sched_barrier(0);
     nchw_static_for<0, RS>([&](auto tap_c) {
       constexpr int tap = decltype(tap_c)::value;
-      // (the order below is pinned: left to itself the scheduler moves a tap's fragment reads next
-      // to its matrix-core instructions, and every tap then waits for LDS)
+      // (the order is pinned: left to itself the scheduler moves a tap's fragment reads next to
+      // its matrix-core instructions, and every tap then waits for LDS)
       if constexpr (tap + NF - 1 < RS) read_frags(buf_c, NchwSet<tap + NF - 1>{});
       __builtin_amdgcn_sched_barrier(0);
       mma(tap % NF);
       __builtin_amdgcn_sched_barrier(0);
-      if (NEXT) {
-        if (!(p.dbg_flags & 1)) stage_slice(set_c, NchwSet<BUF ^ 1>{}, tap_c);
-        if (tap == RS - 1 && !(p.dbg_flags & 2)) load_both(set_c, m + 1 + DEPTH);
-        __builtin_amdgcn_sched_barrier(0);
-      }
     });
-    // own LDS writes done, every wave through with this macro step's buffers
-    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
-    stamp();
-  };
-  auto macro_step = [&](auto set_c, auto buf_c, int m) __attribute__((always_inline)) {
-    if (m + 1 < m_end) macro_body(set_c, NchwSet<1>{}, buf_c, m);
-    else macro_body(set_c, NchwSet<0>{}, buf_c, m);
-  };
-  // macro step m_begin + r computes from buffer r & 1 and stages m + 1 from set (r + 1) % DEPTH
+    if (PACKED) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // this wave's copies have landed
+    meet();
+    };
   for (int m = m_begin; m < m_end; m += 2) {
-    macro_step(NchwSet<DEPTH == 2 ? 1 : 0>{}, NchwSet<0>{}, m);
-    if (m + 1 < m_end) macro_step(NchwSet<0>{}, NchwSet<1>{}, m + 1);
+    macro_step(NchwSet<0>{}, m);
+    if (m + 1 < m_end) macro_step(NchwSet<1>{}, m + 1);
   }
 
   // ---- epilogue: Y[(n * K + i) * ODPQ + s], a lane holds column j of rows 4 * frag_q + r ----------
@@ -497,8 +572,6 @@ __global__ __launch_bounds__(64 * WI * WJ, OCC) void amos_conv_nchw(const ConvNc
         if (i0 + r < s.K && j < s.J) out[coff + (int64_t)(i0 + r) * ODPQ] = acc[a][b][r];
     }
   }
-  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-  stamp();
 }
 
 }  // namespace amos

@@ -186,62 +186,62 @@ struct ConvNchwInstance {
   const char* name;
   int threads;
   int bi, bj;
-  int groups_per_thread;   // load groups of the patch a thread may own (x 4 chunks of channels)
+  int groups_per_thread;   // load groups of the patch a loader thread may own (x 4 chunks of channels)
+  int loader_waves;
   std::once_flag once;
   int scratch_bytes = 0;   // per-lane scratch memory of the built kernel (register spills)
   int static_lds = 0;      // must stay 0: the kernel addresses dynamic LDS from byte 0
 };
 // wmode: NCHW_W_KCTRS (0), NCHW_W_KCRS (1), NCHW_W_PACKED (2)
-ConvNchwInstance* pick_conv_nchw_f16(int ti, int tj, int wmode, int pt);
-ConvNchwInstance* pick_conv_nchw_bf16(int ti, int tj, int wmode, int pt);
-ConvNchwInstance* pick_conv_nchw_i8(int ti, int tj, int wmode, int pt);
+ConvNchwInstance* pick_conv_nchw_f16(int ti, int tj, int wmode, int pt, int nwl);
+ConvNchwInstance* pick_conv_nchw_bf16(int ti, int tj, int wmode, int pt, int nwl);
+ConvNchwInstance* pick_conv_nchw_i8(int ti, int tj, int wmode, int pt, int nwl);
 void launch_conv_pack_weights(int es, const void* w, void* out, int K, int C, int TRS, hipStream_t stream);
 
 #ifdef AMOS_CONV_NCHW_KERNEL_INCLUDED
-template <int DT, int BI, int BJ, int WI, int WJ, int PT, int WMODE, int DEPTH, int OCC>
+template <int DT, int BI, int BJ, int WI, int WJ, int PTL, int WMODE, int NWL>
 ConvNchwInstance* conv_nchw_instance() {
   static ConvNchwInstance inst;
   static const char* dtn[] = {"f16", "bf16", "i8"};
   static const char* wmn[] = {",kctrs", ",kcrs", ",packed"};
   static std::string name = std::string("amos_conv_nchw<") + dtn[DT] + "," + std::to_string(BI) + "x" +
-                            std::to_string(BJ) + "," + std::to_string(WI * WJ) + "w" + wmn[WMODE] +
-                            (PT == 2 ? ",pt2>" : ">");
-  inst.fn = amos_conv_nchw<DT, BI, BJ, WI, WJ, PT, WMODE, DEPTH, OCC>;
+                            std::to_string(BJ) + "," + std::to_string(WI * WJ) + "+" + std::to_string(NWL) + "w" +
+                            wmn[WMODE] + (PTL > 1 ? ",pt" + std::to_string(PTL) + ">" : std::string(">"));
+  inst.fn = amos_conv_nchw<DT, BI, BJ, WI, WJ, PTL, WMODE, NWL>;
   inst.name = name.c_str();
-  inst.threads = 64 * WI * WJ;
+  inst.threads = 64 * (WI * WJ + NWL);
   inst.bi = BI;
   inst.bj = BJ;
-  inst.groups_per_thread = PT;
+  inst.groups_per_thread = PTL;
+  inst.loader_waves = NWL;
   return &inst;
 }
-// 64-row tiles: eight waves, one workgroup per CU; 32-row tiles: four waves, two workgroups per CU
-// that cover each other's set-up, stores and load latencies.  pt = load groups of the patch per
-// thread (1 or 2; 2 exists for the 16-bit types at 128 positions).  Two sets of staging registers
-// (loads two macro steps ahead) where the register file has room for them: 128-position tiles
-// with one load group per thread, except the per-channel weight loader and int8 (sixteen channels
-// per chunk: twice the staging registers of a load group).
+// 64-row tiles: eight matrix-core waves, 32-row tiles: four; beside them nwl loader waves, which
+// take 16 * nwl load groups of the patch per round (pt = rounds)
+template <int DT, int WMODE, int PTL, int NWL>
+ConvNchwInstance* pick_conv_nchw_p(int ti, int tj) {
+  if (ti == 64 && tj == 128) return conv_nchw_instance<DT, 64, 128, 2, 4, PTL, WMODE, NWL>();
+  if (ti == 64 && tj == 256) return conv_nchw_instance<DT, 64, 256, 1, 8, PTL, WMODE, NWL>();
+  if (ti == 32 && tj == 128) return conv_nchw_instance<DT, 32, 128, 1, 4, PTL, WMODE, NWL>();
+  if (ti == 32 && tj == 256) return conv_nchw_instance<DT, 32, 256, 1, 4, PTL, WMODE, NWL>();
+  return nullptr;
+}
 template <int DT, int WMODE>
-ConvNchwInstance* pick_conv_nchw_t(int ti, int tj, int pt) {
-  constexpr int D2 = (DT != DT_I8 && WMODE != NCHW_W_KCTRS) ? 2 : 1;
-  if (pt == 1) {
-    if (ti == 64 && tj == 128) return conv_nchw_instance<DT, 64, 128, 2, 4, 1, WMODE, D2, 1>();
-    if (ti == 64 && tj == 256) return conv_nchw_instance<DT, 64, 256, 1, 8, 1, WMODE, 1, 1>();
-    if (ti == 32 && tj == 128) return conv_nchw_instance<DT, 32, 128, 1, 4, 1, WMODE, D2, 2>();
-    if (ti == 32 && tj == 256) return conv_nchw_instance<DT, 32, 256, 1, 4, 1, WMODE, 1, 2>();
-  }
-  if constexpr (DT != DT_I8) {
-    if (pt == 2) {
-      if (ti == 64 && tj == 128) return conv_nchw_instance<DT, 64, 128, 2, 4, 2, WMODE, 1, 1>();
-      if (ti == 32 && tj == 128) return conv_nchw_instance<DT, 32, 128, 1, 4, 2, WMODE, 1, 2>();
-    }
+ConvNchwInstance* pick_conv_nchw_t(int ti, int tj, int pt, int nwl) {
+  if (pt == 1 && nwl == 4) return pick_conv_nchw_p<DT, WMODE, 1, 4>(ti, tj);
+  if constexpr (WMODE == NCHW_W_PACKED) {
+    if (pt == 1 && nwl == 8) return pick_conv_nchw_p<DT, WMODE, 1, 8>(ti, tj);
+  } else if constexpr (DT != DT_I8) {
+    // (int8: sixteen channels per chunk, twice the staging registers of a load group: one round only)
+    if (pt == 2 && nwl == 4) return pick_conv_nchw_p<DT, WMODE, 2, 4>(ti, tj);
   }
   return nullptr;
 }
 template <int DT>
-ConvNchwInstance* pick_conv_nchw_tile(int ti, int tj, int wmode, int pt) {
-  return wmode == NCHW_W_PACKED ? pick_conv_nchw_t<DT, NCHW_W_PACKED>(ti, tj, pt)
-         : wmode == NCHW_W_KCRS ? pick_conv_nchw_t<DT, NCHW_W_KCRS>(ti, tj, pt)
-                                : pick_conv_nchw_t<DT, NCHW_W_KCTRS>(ti, tj, pt);
+ConvNchwInstance* pick_conv_nchw_tile(int ti, int tj, int wmode, int pt, int nwl) {
+  return wmode == NCHW_W_PACKED ? pick_conv_nchw_t<DT, NCHW_W_PACKED>(ti, tj, pt, nwl)
+         : wmode == NCHW_W_KCRS ? pick_conv_nchw_t<DT, NCHW_W_KCRS>(ti, tj, pt, nwl)
+                                : pick_conv_nchw_t<DT, NCHW_W_KCTRS>(ti, tj, pt, nwl);
 }
 #endif
 

@@ -739,12 +739,9 @@ ConvNchwPlan conv_nchw_plan(const amos_conv_desc_t& c, int op, int BI, int BJ) {
   r.max_pos = max_pos;   // (whole 8-position blocks)
   r.Wp = s.Wp;
   r.max_groups = max_groups;
-  const int threads = BI * 8;   // 64-row tiles run eight waves, 32-row tiles four
-  r.groups_per_thread = (int64_t)max_groups * 4 <= threads ? 1 : 2;
-  if (r.groups_per_thread == 2 && (es == 1 || BJ != 128 || (int64_t)max_groups * 4 > 2 * threads)) {
-    r.why = "input patch of a tile above the threads' load budget";
-    return r;
-  }
+  // (how many rounds of the loader waves that is depends on where the weights come from: the
+  // launch plan decides and refuses what is above the loaders' budget)
+  r.groups_per_thread = 0;
   if (r.max_pos > pos_limit) { r.why = "input patch of a tile does not fit its LDS buffer"; return r; }
   r.lds = (size_t)2 * 9 * BI * 64 + (size_t)2 * pbuf;
   r.t1 = T == 1;

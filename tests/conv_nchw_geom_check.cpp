@@ -188,6 +188,14 @@ int main() {
         seen |= bit;
       }
     }
+    // a direct copy of a block of 16 rows: slot x holds the unit nchw_unit_of_slot names
+    for (int x = 0; x < 64; ++x) {
+      int row = -1, ch = -1;
+      nchw_unit_of_slot(x, &row, &ch);
+      REQUIRE(row >= 0 && row < 16 && ch >= 0 && ch < 4 && nchw_position_offset(row, ch) == x * 16,
+              "slot %d is not where unit (%d, %d) lives", x, row, ch);
+      REQUIRE(nchw_position_offset(32 + row, ch) == 2048 + x * 16, "blocks of 16 rows are not 1 KB apart (slot %d)", x);
+    }
     unsigned rows = 0;
     for (int x = 0; x < 16; ++x) rows |= 1u << nchw_row_of_slot(x);
     REQUIRE(rows == 0xffffu, "nchw_row_of_slot is not a permutation");
