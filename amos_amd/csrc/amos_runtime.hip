@@ -746,7 +746,16 @@ static int plan_conv(Plan& pl, int op, const amos_conv_desc_t* d, const amos_ker
       return 0;
     }
   }
-  // Named explicitly: the kernel that reads NCDHW / KCTRS as they are (one launch, no workspace)
+  // The kernel that reads the activations as they are: named by the caller, or the default's
+  // choice where the caller names no tile and brings the workspace for the packed weights (the
+  // default's estimate is for packed weights)
+  amos_kernel_config_t nchw_default;
+  if ((!cfg || (cfg->pipeline == AMOS_PIPE_AUTO && (cfg->tile_i <= 0 || cfg->tile_j <= 0) && cfg->split_k <= 1)) &&
+      workspace && ((uintptr_t)workspace & 255) == 0 && ws_bytes >= amos_conv_packed_weights_bytes(op, &c) &&
+      amos_default_config(op, &c, &nchw_default) == 0 && nchw_default.pipeline == AMOS_PIPE_NCHW) {
+    if (cfg) nchw_default.reserved[0] = cfg->reserved[0];
+    cfg = &nchw_default;
+  }
   if (cfg && cfg->pipeline == AMOS_PIPE_NCHW) {
     const int BI = cfg->tile_i > 0 ? cfg->tile_i : 64;
     const int BJ = cfg->tile_j > 0 ? cfg->tile_j : 128;
@@ -1472,6 +1481,8 @@ size_t amos_workspace_bytes(int op, const void* desc, const amos_kernel_config_t
   }
   const amos_conv_desc_t& c = *(const amos_conv_desc_t*)desc;
   int64_t need = conv_workspace_bytes(c, op);
+  // (no pipeline named: the default may be the kernel above)
+  if (!cfg || cfg->pipeline == AMOS_PIPE_AUTO) need = std::max<int64_t>(need, (int64_t)amos_conv_packed_weights_bytes(op, &c));
   // a pointwise convolution runs as a matrix product; its row-contiguous operand (NCDHW
   // activations, [C][K] weights) may want a K-contiguous copy
   amos_bgemm_desc_t b;

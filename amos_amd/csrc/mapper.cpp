@@ -781,6 +781,36 @@ static double conv_patch_estimate(const amos_conv_desc_t& c, int op, const Probl
   return cycles / 2.1e9 + relayout + (split > 1 ? (double)pb.out_bytes * split / 1.2e12 : 0.0);
 }
 
+// NCDHW-direct convolution (conv_nchw_kernel.h), weights packed by the call: one workgroup per CU
+// at a time; a tile pays its set-up, the latency of its first loads and its stores (~9000 cycles
+// at the 2.4 GHz of the cycle counter, measured), then per macro step (nine taps x 64 bytes of
+// channels) the longer of the matrix-core waves' time (the tile's flops at 72-85 % of the CU's
+// rate, measured with the loaders switched off) and the loader waves' time (a fixed ~1800 cycles
+// of latency that their two-step lookahead does not cover, plus ~45 per load instruction of a
+// wave, measured on 14x14 and 56x56 planes; int8 loads twice the channels per group).
+// Returns <= 0 where the kernel does not apply.
+double conv_nchw_estimate(const amos_conv_desc_t& c, int op, const Problem& pb, int ti, int tj) {
+  if ((ti != 64 && ti != 32) || (tj != 128 && tj != 256)) return -1.0;
+  const ConvNchwPlan np = conv_nchw_plan(c, op, ti, tj);
+  if (np.why) return -1.0;
+  const bool i8 = pb.in_dtype == AMOS_I8;
+  const double es = i8 ? 1.0 : 2.0;
+  const int nwl = nchw_loader_waves(true, np.max_groups);
+  if (np.max_groups > 16 * nwl) return -1.0;
+  const int64_t T = op == AMOS_OP_CONV2D ? 1 : c.T;
+  const double macro_steps = (double)T * (c.C * es / 64.0);
+  const double tiles = std::ceil((double)pb.I / ti) * std::ceil((double)pb.J / tj);
+  const double rounds = std::ceil(tiles / device_compute_units());
+  const double flop_per_cycle = (i8 ? 2.0 : 1.0) * 3850.0 * (ti * tj >= 64 * 256 ? 0.85 : ti * tj >= 64 * 128 ? 0.72 : 0.6);
+  const double mma = 2.0 * ti * tj * 9.0 * (64.0 / es) / flop_per_cycle;
+  const double load_instr = std::ceil(np.max_groups * 4.0 / 64.0) * (16.0 / es) * (i8 ? 2.0 : 1.0);
+  const double loaders = 1800.0 + 45.0 * load_instr;
+  const double prologue = 7000.0 + 40.0 * load_instr;
+  const double cycles = rounds * (prologue + macro_steps * std::max(mma, loaders));
+  const double pack = (double)(c.K * c.C * T * 9) * es * 2.0 / 2.5e12 + 3.5e-6;
+  return cycles / 2.4e9 + 2.5e-6 + pack;
+}
+
 }  // namespace amos
 
 using namespace amos;
@@ -845,6 +875,12 @@ int amos_estimate_seconds(int op, const void* desc, const amos_kernel_config_t* 
     const double t_conv = 6e-6 + rounds * 4.5e-6;
     const double t_mem = ((double)pb.in_bytes * 2 + (double)fp.bytes_x * 2 + (double)pb.out_bytes) / (0.5 * Gfx950::kHbmBytesPerSec);
     *seconds = 4e-6 + (double)fp.bytes_x / 2.5e12 + std::max(t_conv, t_mem);
+    return 0;
+  }
+  if ((op == AMOS_OP_CONV2D || op == AMOS_OP_CONV3D) && cfg->pipeline == AMOS_PIPE_NCHW) {
+    const double s = conv_nchw_estimate(*(const amos_conv_desc_t*)desc, op, pb, cfg->tile_i, cfg->tile_j);
+    if (s <= 0) return set_error(AMOS_ERR_INFEASIBLE, "NCDHW-direct convolution not applicable to this config");
+    *seconds = s;
     return 0;
   }
   amos_bgemm_desc_t as_gemm;
@@ -931,6 +967,7 @@ int amos_default_config(int op, const void* desc, amos_kernel_config_t* result) 
   const double patch_best = best;
   amos_kernel_config_t staged = *out;
   if (patch_best < 1e30) best = patch_best / 1.25;
+  const double staged_bar = best;
   out = &staged;
   for (auto& t : kTiles) {
     for (int split = 1; split <= 16; split *= 2) {
@@ -946,6 +983,20 @@ int amos_default_config(int op, const void* desc, amos_kernel_config_t* result) 
     }
   }
   *result = staged;
+  // the kernel that reads the activations as they are, where it applies and its estimate is lower
+  if (op == AMOS_OP_CONV2D || op == AMOS_OP_CONV3D) {
+    const amos_conv_desc_t& c = *(const amos_conv_desc_t*)desc;
+    if (patch_best < 1e30 && best >= staged_bar) best = patch_best;   // (the estimate of what was chosen)
+    for (int ti : {64, 32})
+      for (int tj : {128, 256}) {
+        const double s = conv_nchw_estimate(c, op, pb, ti, tj);
+        if (s > 0 && s < best * 0.97) {
+          best = s;
+          memset(result, 0, sizeof(*result));
+          result->tile_i = ti; result->tile_j = tj; result->split_k = 1; result->pipeline = AMOS_PIPE_NCHW;
+        }
+      }
+  }
   return 0;
 }
 

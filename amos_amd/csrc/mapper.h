@@ -147,11 +147,13 @@ struct ConvNchwPlan {
   int max_pos;          // LDS positions of a patch buffer (the largest tile's, multiple of 4)
   int Wp;               // row pitch of the patch in positions
   int max_groups;       // load groups of the largest tile
-  int groups_per_thread;
+  int groups_per_thread;   // (set by the launch plan: it depends on where the weights come from)
   int t1;               // conv2d: a chunk's weights are one contiguous run (needs 16-byte aligned weights)
   size_t lds;           // dynamic LDS bytes of a workgroup
 };
 ConvNchwPlan conv_nchw_plan(const amos_conv_desc_t& c, int op, int BI, int BJ);
+// estimated seconds of a call that packs the weights into its workspace; <= 0 where the kernel does not apply
+double conv_nchw_estimate(const amos_conv_desc_t& c, int op, const Problem& pb, int ti, int tj);
 // the kernel's geometry descriptor of a convolution (extents, patch pitch, dividers)
 struct NchwShape;
 void conv_nchw_shape(const amos_conv_desc_t& c, int op, int patch_pitch, NchwShape* out);

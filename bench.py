@@ -128,6 +128,20 @@ def run_all_configs(cpu=True, only=None):
                "gpu_us": sec * 1e6, "tflops": flop / sec / 1e12,
                "pct_mfma_peak": 100 * t_mfma / sec, "pct_hbm_roof": 100 * t_hbm / sec,
                "bound": "mfma" if t_mfma >= t_hbm else "hbm", "flop": flop, "bytes": nbytes}
+        if cfg.pipeline == _lib.AMOS_PIPE_NCHW and not fused_tail:
+            # the same convolution where the owner of the weights has packed them once
+            # (amos_conv_pack_weights + AMOS_FLAG_WEIGHTS_PACKED): no packing launch in the call
+            lib = _lib.load()
+            packed = torch.empty(lib.amos_conv_packed_weights_bytes(op, ctypes.byref(desc)), dtype=torch.uint8,
+                                 device="cuda")
+            _lib.check(lib.amos_conv_pack_weights(op, ctypes.byref(desc), tin[1].data_ptr(), packed.data_ptr(), None))
+            c2 = _lib.KernelConfig.from_buffer_copy(cfg)
+            c2.reserved[0] |= _lib.AMOS_FLAG_WEIGHTS_PACKED
+            res = (ctypes.c_double * 3)()
+            _lib.check(lib.amos_time(op, ctypes.byref(desc), ctypes.byref(c2), tin[0].data_ptr(), packed.data_ptr(),
+                                     out.data_ptr(), None, 0, None, 20, 3, 100, res))
+            row["gpu_us_weights_packed_once"] = min(res) * 1e6
+            del packed
         if cpu and cpu_fn is not None:
             t1 = _timed(lambda: cpu_fn(1, False))
             tn = _timed(lambda: cpu_fn(cores, True))
