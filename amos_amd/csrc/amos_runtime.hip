@@ -219,6 +219,20 @@ __global__ void fill_zero_kernel(T* p, int64_t rows, int64_t cols, int64_t ld) {
   for (; idx < n; idx += (int64_t)gridDim.x * blockDim.x) p[(idx / cols) * ld + idx % cols] = 0;
 }
 
+// out[r][c] = part[0][r][c] + part[1][r][c] + ... in that order (split-K partial sums)
+template <typename T>
+__global__ void reduce_splits_kernel(T* out, const T* part, int64_t rows, int64_t cols, int64_t ld, int nsplit,
+                                     int64_t stride) {
+  int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const int64_t n = rows * cols;
+  for (; idx < n; idx += (int64_t)gridDim.x * blockDim.x) {
+    const int64_t off = (idx / cols) * ld + idx % cols;
+    T acc = part[off];
+    for (int s = 1; s < nsplit; ++s) acc += part[(int64_t)s * stride + off];
+    out[off] = acc;
+  }
+}
+
 // ---- kernel instance table (defined in inst_*.hip) -------------------------------------
 static Instance* pick(int dt, int rl, int cl, int ti, int tj) {
   if (rl == LD_TVEC) {
@@ -299,9 +313,17 @@ struct Plan {
   amos_kernel_config_t cfg;
   int64_t batch;
   int split;
-  // zero fill of the output before a split-K launch
+  // zero fill of the output before a split-K launch that accumulates with atomics
   int64_t fill_rows, fill_cols, fill_ld;
   int fill_once;
+  // split-K with partial sums in the workspace (behind what the pipeline itself keeps there): every
+  // split stores its tile into its own slice, a second launch adds the slices in the order of the
+  // splits -- the same bits on every run, and the output is written after every read of the call
+  char* ws_base;
+  size_t ws_bytes, ws_own;     // the caller's workspace; the pipeline's own share of it
+  char* part;                  // the slices (nullptr: none)
+  int64_t part_stride;         // elements between them
+  char* part_out;              // the output that the reduction writes
   // direct-to-LDS GEMM pipeline (0 = not used, else waves per block)
   int tn_waves;
   GemmTnParams tn;
@@ -350,6 +372,17 @@ static int dtype_pair(int in_dtype, int out_dtype, int* dt) {
 static bool aligned16(const void* p) { return ((uintptr_t)p & 15) == 0; }
 
 static int fits_int(int64_t v) { return v > 0 && v < (int64_t)1 << 31; }
+
+// elements from the first to the last element of the planned output, rounded up to 64
+static int64_t plan_out_footprint(const Plan& pl) {
+  const int64_t n = (pl.fill_once ? 0 : (pl.batch - 1) * pl.p.out_batch) + (pl.fill_rows - 1) * pl.fill_ld + pl.fill_cols;
+  return (n + 63) & ~(int64_t)63;
+}
+// whether the caller's workspace has room for `split` slices of partial sums behind the pipeline's own share
+static bool split_partials_fit(const Plan& pl, int split) {
+  if (!pl.ws_base || ((uintptr_t)pl.ws_base & 255) || split < 2) return false;
+  return pl.ws_bytes >= pl.ws_own + (size_t)split * (size_t)plan_out_footprint(pl) * 4;
+}
 
 static int plan_finish(Plan& pl, int op, const void* desc, const amos_kernel_config_t* cfg) {
   amos_kernel_config_t c;
@@ -509,7 +542,8 @@ static int plan_gemm(Plan& pl, int op, const void* desc_any, const amos_gemm_des
   // direct-to-LDS pipeline: both operands K-contiguous and 16-byte aligned, whole K steps,
   // 32-bit byte offsets inside a 256-row tile
   const int bke = 128 / es;
-  const bool tn_ok = pl.rl == LD_VEC && pl.cl == LD_VEC && d->K % bke == 0 && pl.split == 1 &&
+  const bool tn_ok = pl.rl == LD_VEC && pl.cl == LD_VEC && d->K % bke == 0 &&
+                     (pl.split == 1 || split_partials_fit(pl, pl.split)) &&
                      256 * d->lda * es + 128 < ((int64_t)1 << 32) &&
                      256 * d->ldb * es + 128 < ((int64_t)1 << 32);
   const int pipe = pl.cfg.pipeline;
@@ -525,7 +559,8 @@ static int plan_gemm(Plan& pl, int op, const void* desc_any, const amos_gemm_des
     if (!tn_ok || !pick_gemm_tn(pl.dt, pl.cfg.tile_i, pl.cfg.tile_j, waves))
       return set_error(AMOS_ERR_INFEASIBLE,
                        "direct-to-LDS pipeline needs K-contiguous 16-byte aligned operands, "
-                       "K %% %d == 0, split_k 1 and a tile of 256x256, 128x128, 128x256 or 256x128", bke);
+                       "K %% %d == 0, a tile of 256x256, 128x128, 128x256 or 256x128 and, for split-K, "
+                       "the workspace that amos_workspace_bytes() names", bke);
     pl.tn_waves = waves;
   } else if (pipe == AMOS_PIPE_AUTO && tn_ok && pick_gemm_tn(pl.dt, pl.cfg.tile_i, pl.cfg.tile_j, 8)) {
     pl.tn_waves = 8;  // measured a few percent ahead of 4 waves on the 8192^3 fp16 GEMM
@@ -558,6 +593,8 @@ static int plan_gemm(Plan& pl, int op, const void* desc_any, const amos_gemm_des
     q.lda = d->lda; q.ldb = d->ldb; q.ldc = d->ldc;
     q.batch_a = sa; q.batch_b = sb; q.batch_c = sc;
     q.tiles_i = p.tiles_i; q.tiles_j = p.tiles_j;
+    q.kt_per_split = pl.split > 1 ? p.k_tiles_per_split : 0;
+    q.split_stride = 0;
   }
   return 0;
 }
@@ -762,7 +799,6 @@ static int plan_conv(Plan& pl, int op, const amos_conv_desc_t* d, const amos_ker
     ConvNchwPlan np = conv_nchw_plan(c, op, BI, BJ);
     const char* why = np.why;
     if (!why && ((uintptr_t)X & 7)) why = "activations not 8-byte aligned";
-    if (!why && cfg->split_k > 1) why = "no split-K in this pipeline";
     if (why) return set_error(AMOS_ERR_INFEASIBLE, "NCDHW-direct convolution not applicable: %s", why);
     ConvNchwParams& q = pl.nc;
     memset(&q, 0, sizeof(q));
@@ -786,7 +822,10 @@ static int plan_conv(Plan& pl, int op, const amos_conv_desc_t* d, const amos_ker
     const int es1 = pl.dt == DT_I8 ? 1 : 2;
     q.c_chunks = (int)(c.C * es1 / 64);
     q.macro_steps = q.s.T * q.c_chunks;
-    q.macro_per_split = q.macro_steps;
+    int nsplit = cfg->split_k < 1 ? 1 : cfg->split_k;
+    if (nsplit > q.macro_steps) nsplit = q.macro_steps;
+    q.macro_per_split = (q.macro_steps + nsplit - 1) / nsplit;
+    nsplit = (q.macro_steps + q.macro_per_split - 1) / q.macro_per_split;
     q.tiles_i = (int)((c.K + BI - 1) / BI);
     q.tiles_j = (int)((J + BJ - 1) / BJ);
     q.max_pos = np.max_pos;
@@ -806,12 +845,16 @@ static int plan_conv(Plan& pl, int op, const amos_conv_desc_t* d, const amos_ker
     pl.nchw_lds = np.lds;
     memset(&pl.cfg, 0, sizeof(pl.cfg));
     pl.cfg = *cfg;
-    pl.cfg.tile_i = BI; pl.cfg.tile_j = BJ; pl.cfg.split_k = 1;
+    pl.cfg.tile_i = BI; pl.cfg.tile_j = BJ; pl.cfg.split_k = nsplit;
     memset(&pl.p, 0, sizeof(pl.p));
     pl.p.out_si = (int64_t)OD * OP * OQ;     // (the fused tail's operand is laid out like the output)
     pl.p.out_batch = 0;
     pl.batch = 1;
-    pl.split = 1;
+    pl.split = nsplit;                       // (partial sums in the workspace: make_plan)
+    pl.fill_rows = 1;
+    pl.fill_cols = c.N * c.K * (int64_t)OD * OP * OQ;
+    pl.fill_ld = pl.fill_cols;
+    pl.fill_once = 1;
     return 0;
   }
   const int es = pl.dt == DT_I8 ? 1 : 2;
@@ -961,9 +1004,59 @@ static int plan_conv(Plan& pl, int op, const amos_conv_desc_t* d, const amos_ker
   return 0;
 }
 
+static int make_plan_inner(Plan& pl, int op, const void* desc, const amos_kernel_config_t* cfg,
+                           const void* in0, const void* in1, void* out, void* workspace, size_t ws_bytes);
+
 static int make_plan(Plan& pl, int op, const void* desc, const amos_kernel_config_t* cfg,
                      const void* in0, const void* in1, void* out, void* workspace = nullptr,
                      size_t ws_bytes = 0) {
+  pl.ws_base = (char*)workspace;
+  pl.ws_bytes = ws_bytes;
+  pl.part = nullptr;
+  pl.part_stride = 0;
+  pl.part_out = nullptr;
+  pl.split = 1;
+  // the pipeline's own share of the workspace: what the same configuration asks for without a split
+  {
+    amos_kernel_config_t c1;
+    if (cfg) { c1 = *cfg; c1.split_k = 1; }
+    pl.ws_own = (amos_workspace_bytes(op, desc, cfg ? &c1 : nullptr) + 255) & ~(size_t)255;
+  }
+  int rc = make_plan_inner(pl, op, desc, cfg, in0, in1, out, workspace, ws_bytes);
+  if (rc) return rc;
+  if (pl.split > 1 && split_partials_fit(pl, pl.split)) {
+    pl.part = pl.ws_base + pl.ws_own;
+    pl.part_stride = plan_out_footprint(pl);
+    if (pl.nchw) {
+      pl.part_out = pl.nc.y;
+      pl.nc.y = pl.part;
+      pl.nc.split_stride = pl.part_stride;
+    } else if (pl.conv_ups) {
+      pl.part_out = pl.cv.y;
+      pl.cv.y = pl.part;
+      pl.cv.split_stride = pl.part_stride;
+      pl.cv.atomic_out = 0;
+      pl.cv.zero_words = 0;
+      pl.cv.prep_z_blocks = 0;
+    } else if (pl.tn_waves) {
+      pl.part_out = pl.tn.c;
+      pl.tn.c = pl.part;
+      pl.tn.split_stride = pl.part_stride;
+    } else {
+      pl.part_out = pl.p.out;
+      pl.p.out = pl.part;
+      pl.p.split_stride = pl.part_stride;
+      pl.p.atomic_out = 0;
+    }
+  } else if (pl.split > 1 && (pl.tn_waves || pl.nchw)) {
+    return set_error(AMOS_ERR_WORKSPACE, "split-K of this pipeline keeps partial sums in the workspace: "
+                     "amos_workspace_bytes() of the same configuration says how much");
+  }
+  return 0;
+}
+
+static int make_plan_inner(Plan& pl, int op, const void* desc, const amos_kernel_config_t* cfg,
+                           const void* in0, const void* in1, void* out, void* workspace, size_t ws_bytes) {
   pl.tn_waves = 0;
   pl.conv_ups = 0;
   pl.fill_once = 0;
@@ -1019,7 +1112,7 @@ static int launch_tn(const Plan& pl, hipStream_t stream) {
   if (inst->scratch_bytes)
     return set_error(AMOS_ERR_INFEASIBLE, "%s was built with %d bytes of scratch memory per lane (register "
                      "spills), which its wait counts do not allow for", inst->name, inst->scratch_bytes);
-  dim3 grid((unsigned)(pl.tn.tiles_i * pl.tn.tiles_j), 1, (unsigned)pl.batch);
+  dim3 grid((unsigned)(pl.tn.tiles_i * pl.tn.tiles_j), (unsigned)pl.split, (unsigned)pl.batch);
   hipLaunchKernelGGL(inst->fn, grid, dim3(inst->threads), inst->lds, stream, pl.tn);
   HIP_TRY(hipGetLastError());
   return 0;
@@ -1096,7 +1189,28 @@ static int launch_conv_nchw(const Plan& pl, hipStream_t stream) {
   return 0;
 }
 
+static int launch_kernels(const Plan& pl, hipStream_t stream);
+
+// the kernels of the plan, then (split-K with partial sums) the launch that adds the slices
 static int launch(const Plan& pl, hipStream_t stream) {
+  int rc = launch_kernels(pl, stream);
+  if (rc || !pl.part) return rc;
+  const int64_t n = pl.fill_rows * pl.fill_cols;
+  const int blocks = (int)std::min<int64_t>((n + 255) / 256, 8192);
+  for (int64_t b = 0; b < (pl.fill_once ? 1 : pl.batch); ++b) {
+    const int64_t off = b * pl.p.out_batch * 4;
+    if (pl.dt == DT_I8)
+      hipLaunchKernelGGL(reduce_splits_kernel<int>, dim3(blocks), dim3(256), 0, stream, (int*)(pl.part_out + off),
+                         (const int*)(pl.part + off), pl.fill_rows, pl.fill_cols, pl.fill_ld, pl.split, pl.part_stride);
+    else
+      hipLaunchKernelGGL(reduce_splits_kernel<float>, dim3(blocks), dim3(256), 0, stream, (float*)(pl.part_out + off),
+                         (const float*)(pl.part + off), pl.fill_rows, pl.fill_cols, pl.fill_ld, pl.split, pl.part_stride);
+  }
+  HIP_TRY(hipGetLastError());
+  return 0;
+}
+
+static int launch_kernels(const Plan& pl, hipStream_t stream) {
   if (pl.nchw) return launch_conv_nchw(pl, stream);
   if (pl.im2col) {
     const unsigned want = (pl.icp.total + 255u) / 256u;
@@ -1151,7 +1265,7 @@ static int launch(const Plan& pl, hipStream_t stream) {
   if (attr_err != hipSuccess)
     return set_error(AMOS_ERR_HIP, "hipFuncSetAttribute(%s, %zu B LDS): %s", inst->name, inst->lds,
                      hipGetErrorString(attr_err));
-  if (pl.split > 1) {
+  if (pl.split > 1 && !pl.part) {
     int64_t n = pl.fill_rows * pl.fill_cols * pl.batch;
     int blocks = (int)((n + 255) / 256 < 4096 ? (n + 255) / 256 : 4096);
     // batched outputs are contiguous per batch only when stride_c == M*ldc; fill per batch
@@ -1172,7 +1286,7 @@ static int launch(const Plan& pl, hipStream_t stream) {
 }
 
 // fused tail operation: validate it against the planned op and hand it to whichever kernel runs
-static int plan_epilogue(Plan& pl, int op, const void* desc, const amos_epilogue_t* e) {
+static int plan_epilogue(Plan& pl, int op, const void* desc, const amos_epilogue_t* e, const void* out) {
   EpiParams ep = {nullptr, 0, 0, EPI_NONE};
   if (e && e->kind != AMOS_EPI_NONE) {
     if (e->kind != AMOS_EPI_ADD) return set_error(AMOS_ERR_UNSUPPORTED, "unknown epilogue kind %d", e->kind);
@@ -1184,6 +1298,12 @@ static int plan_epilogue(Plan& pl, int op, const void* desc, const amos_epilogue
                        "(int32 output: int32; fp32 output: fp32, fp16 or bf16)", e->dtype);
     ep.ptr = (const char*)e->operand;
     ep.dt = e->dtype == AMOS_F16 ? EPI_F16 : e->dtype == AMOS_BF16 ? EPI_BF16 : EPI_OUT_TYPE;
+    // split-K that accumulates into the output with atomics (no workspace for partial sums): the
+    // output is zeroed and added to while the first split still reads D
+    if (pl.split > 1 && !pl.part && out && ep.ptr >= (const char*)out &&
+        ep.ptr < (const char*)out + plan_out_footprint(pl) * 4)
+      return set_error(AMOS_ERR_BAD_ARG, "the epilogue operand aliases the output of a split-K launch without a "
+                       "workspace for its partial sums (amos_workspace_bytes() of the configuration)");
     if (op == AMOS_OP_GEMM || op == AMOS_OP_BGEMM) {
       const amos_gemm_desc_t& g = op == AMOS_OP_GEMM ? *(const amos_gemm_desc_t*)desc
                                                      : ((const amos_bgemm_desc_t*)desc)->g;
@@ -1213,7 +1333,7 @@ static int run_op(int op, const void* desc, const amos_kernel_config_t* cfg, con
   Plan pl;
   int rc = make_plan(pl, op, desc, cfg, in0, in1, out, workspace, ws_bytes);
   if (rc) return rc;
-  rc = plan_epilogue(pl, op, desc, epi);
+  rc = plan_epilogue(pl, op, desc, epi, out);
   if (rc) return rc;
   return launch(pl, (hipStream_t)stream);
 }
@@ -1459,7 +1579,43 @@ int amos_run_fused(int op, const void* desc, const amos_kernel_config_t* cfg,
   return run_op(op, desc, cfg, epilogue, in0, in1, out, workspace, ws_bytes, stream);
 }
 
+// elements from the first to the last element of the output a descriptor names, rounded up to 64
+static int64_t desc_out_footprint(int op, const void* desc) {
+  int64_t n = 0;
+  if (op == AMOS_OP_GEMM || op == AMOS_OP_BGEMM) {
+    const amos_gemm_desc_t& g = op == AMOS_OP_GEMM ? *(const amos_gemm_desc_t*)desc : ((const amos_bgemm_desc_t*)desc)->g;
+    const int64_t ldc = g.ldc > 0 ? g.ldc : g.N;
+    n = (g.M - 1) * ldc + g.N;
+    if (op == AMOS_OP_BGEMM) {
+      const amos_bgemm_desc_t* b = (const amos_bgemm_desc_t*)desc;
+      n += (b->batch - 1) * (b->stride_c > 0 ? b->stride_c : g.M * ldc);
+    }
+  } else if (op == AMOS_OP_CONV2D || op == AMOS_OP_CONV3D) {
+    const amos_conv_desc_t& c = *(const amos_conv_desc_t*)desc;
+    auto ext = [](int64_t in, int64_t pad, int64_t dil, int64_t k, int64_t st) {
+      const int64_t eff = (k - 1) * dil + 1;
+      return in + 2 * pad < eff || st <= 0 ? (int64_t)0 : (in + 2 * pad - eff) / st + 1;
+    };
+    const int64_t od = op == AMOS_OP_CONV2D ? 1 : ext(c.D, c.pad_d, c.dil_d, c.T, c.stride_d);
+    n = c.N * c.K * od * ext(c.H, c.pad_h, c.dil_h, c.R, c.stride_h) * ext(c.W, c.pad_w, c.dil_w, c.S, c.stride_w);
+  }
+  return n <= 0 ? 0 : (n + 63) & ~(int64_t)63;
+}
+
+static size_t workspace_bytes_unsplit(int op, const void* desc, const amos_kernel_config_t* cfg);
+
 size_t amos_workspace_bytes(int op, const void* desc, const amos_kernel_config_t* cfg) {
+  if (!desc) return 0;
+  if (!cfg || cfg->split_k <= 1) return workspace_bytes_unsplit(op, desc, cfg);
+  // split-K: behind the pipeline's own share, one slice of the output per split for the partial
+  // sums (a workspace without that room: the kernels that can accumulate with atomics do so)
+  amos_kernel_config_t c1 = *cfg;
+  c1.split_k = 1;
+  const size_t own = (workspace_bytes_unsplit(op, desc, &c1) + 255) & ~(size_t)255;
+  return own + (size_t)cfg->split_k * (size_t)desc_out_footprint(op, desc) * 4;
+}
+
+static size_t workspace_bytes_unsplit(int op, const void* desc, const amos_kernel_config_t* cfg) {
   // GEMM: room for K-contiguous copies of row-contiguous operands (a transposed A, a row-major B)
   // where the problem is large enough for the copies to pay; none otherwise (split-K accumulates
   // straight into the zero-filled output).
@@ -1577,7 +1733,7 @@ int amos_time_fused(int op, const void* desc, const amos_kernel_config_t* cfg,
   Plan pl;
   int rc = make_plan(pl, op, desc, cfg, in0, in1, out, workspace, ws_bytes);
   if (rc) return rc;
-  rc = plan_epilogue(pl, op, desc, epilogue);
+  rc = plan_epilogue(pl, op, desc, epilogue, out);
   if (rc) return rc;
   return time_launches([&] { return launch(pl, stream); }, stream, number, repeat, min_repeat_ms, out_seconds);
 }

@@ -69,7 +69,8 @@ struct ConvFpropParams {
   int macro_steps;   // T * c_chunks
   int macro_per_split;
   int tiles_i, tiles_j;
-  int atomic_out;
+  int atomic_out;        // split-K without room for partial sums: accumulate into the zeroed output
+  int64_t split_stride;  // split-K with it: blockIdx.y stores its partial sums at y + blockIdx.y * split_stride
   FastDiv fd_opq, fd_oq, fd_od, fd_wp, fd_odpq, fd_cc, fd_c, fd_slab;   // divisions by OP*OQ, OQ, OD, Wp, OD*OP*OQ, c_chunks, C, C*T*R*S
   // prepare kernel work split (in blocks)
   int prep_w_blocks, prep_x_blocks, prep_z_blocks;
@@ -533,7 +534,7 @@ __global__ __launch_bounds__(64 * NW, OCC) void amos_conv_fprop(const ConvFpropP
 
   // ---- epilogue: Y[(n*K + i)*ODPQ + (od*OPQ + opq)] ---------------------------------------------
   auto store_tile = [&](const TileGeo& q) {
-  out_t* const out = (out_t*)p.y;
+  out_t* const out = (out_t*)p.y + (int64_t)blockIdx.y * p.split_stride;
   const int ODPQ = p.OD * OPQ;
   const bool full = q.bi0 + BI <= p.K && q.bj0 + BJ <= p.J && !p.atomic_out;
   const int64_t y_si = p.y_si;

@@ -38,6 +38,8 @@ struct GemmTnParams {
   int64_t lda, ldb, ldc;
   int64_t batch_a, batch_b, batch_c;  // elements between batches
   int tiles_i, tiles_j;
+  int kt_per_split;       // split-K: blockIdx.y takes the K tiles [y * kt_per_split, (y + 1) * kt_per_split) ...
+  int64_t split_stride;   // ... and stores its partial sums at c + y * split_stride (0: no split)
   EpiParams epi;   // fused tail: C = acc + cast(D), D[i][j] at i*epi.si + j
 };
 
@@ -126,9 +128,11 @@ __global__ __launch_bounds__(64 * WI * WJ) void amos_gemm_tn(const GemmTnParams 
     }
   }
 
+  // this block's K tiles: all of them, or blockIdx.y's share of a split-K launch
+  const int kt0 = p.kt_per_split ? (int)blockIdx.y * p.kt_per_split : 0;
   auto issue_copies = [&](int kt, int stage) {
-    const char* ak = abase + (int64_t)kt * 128;
-    const char* bk = bbase + (int64_t)kt * 128;
+    const char* ak = abase + (int64_t)(kt0 + kt) * 128;
+    const char* bk = bbase + (int64_t)(kt0 + kt) * 128;
     char* s = smem + stage * STAGE;
 #pragma unroll
     for (int u = 0; u < CH; ++u) {
@@ -186,7 +190,8 @@ __global__ __launch_bounds__(64 * WI * WJ) void amos_gemm_tn(const GemmTnParams 
       for (int a = 0; a < HA; ++a) acc[h * HA + a][b] = MM::run(af[sa][a], bf[sb][b], acc[h * HA + a][b]);
   };
 
-  const int KT = p.K / BKE;
+  int KT = p.K / BKE - kt0;
+  if (p.kt_per_split && KT > p.kt_per_split) KT = p.kt_per_split;
   static_assert(NS >= 2 && (NS - 1) * CH <= 63, "stages");
 #pragma unroll
   for (int s = 0; s < NS; ++s) issue_copies(s < KT ? s : KT - 1, s);
@@ -223,7 +228,7 @@ __global__ __launch_bounds__(64 * WI * WJ) void amos_gemm_tn(const GemmTnParams 
   // (16 rows x the wave tile's width) and leaves as 16-byte stores that cover whole rows of the
   // wave tile: 64 / (4 TJ) rows x 64 TJ bytes per instruction instead of four rows x 64 bytes.
   // LDS operations of one wave complete in issue order, so the strip needs no barrier of its own.
-  out_t* const out = (out_t*)p.c + batch * p.batch_c;
+  out_t* const out = (out_t*)p.c + batch * p.batch_c + (int64_t)blockIdx.y * p.split_stride;
   constexpr int SP = TJ * 16 + 4;          // strip row pitch in elements
   constexpr int CPR = TJ * 4, RPI = 64 / CPR;   // 16-byte chunks per row, rows per store instruction
   static_assert(TJ <= 16 && (TJ & (TJ - 1)) == 0 && NW * 16 * SP * 4 <= NS * STAGE, "output strip");
@@ -237,7 +242,7 @@ __global__ __launch_bounds__(64 * WI * WJ) void amos_gemm_tn(const GemmTnParams 
 #pragma unroll
   for (int a = 0; a < TI; ++a) {
     const int i0 = bi0 + (wi * TI + a) * 16 + 4 * frag_q;
-    if (p.epi.dt != EPI_NONE) {   // the row block's loads in flight before the first addition
+    if (p.epi.dt != EPI_NONE && blockIdx.y == 0) {   // (one K split adds D) the row block's loads in flight before the first addition
       out_t dv[TJ][4];
 #pragma unroll
       for (int b = 0; b < TJ; ++b) {

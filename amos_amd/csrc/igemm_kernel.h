@@ -134,7 +134,8 @@ struct IgemmParams {
   int out_jmod;
   int64_t out_batch;
   int out_vec4;                 // out_si == 1, rows % 4 == 0, 16-byte aligned, no atomics: 4 rows per store
-  int atomic_out;               // split-K: accumulate into a zeroed output
+  int atomic_out;               // split-K without a workspace: accumulate into a zeroed output
+  int64_t split_stride;         // split-K with one: blockIdx.y stores its partial sums at out + blockIdx.y * split_stride
   EpiParams epi;                // D is indexed like the output, with its own row stride
 };
 
@@ -465,7 +466,7 @@ __global__ __launch_bounds__(256) void amos_igemm(const IgemmParams p) {
   }
 
   // ---- epilogue: accumulators straight to the final layout -----------------------
-  out_t* const out = (out_t*)p.out + batch * p.out_batch;
+  out_t* const out = (out_t*)p.out + batch * p.out_batch + (int64_t)blockIdx.y * p.split_stride;
   const bool add_d = p.epi.dt != EPI_NONE && blockIdx.y == 0;   // one K split adds D
 #pragma unroll
   for (int b = 0; b < TJ; ++b) {

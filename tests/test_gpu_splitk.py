@@ -1,0 +1,127 @@
+"""Split-K keeps its partial sums in the workspace and adds them in the order of the splits: the same
+bits on every run, for every kernel that takes a split (the register-staged implicit GEMM, the
+direct-to-LDS GEMM, the patch-staged and the NCDHW-direct convolution); the fused tail's operand may
+be the output itself; without the workspace the kernels that can do so fall back to atomics and an
+operand that aliases the output is refused."""
+import ctypes
+
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+MAX_REL, MEAN_REL = 1e-2, 1e-3
+
+
+def _rel(got, ref):
+    from oracle import cpu_oracle as co
+    return co.rel_errors(got, ref)
+
+
+def _repeat_equal(fn, runs=4):
+    first = fn()
+    torch.cuda.synchronize()
+    for _ in range(runs - 1):
+        again = fn()
+        torch.cuda.synchronize()
+        assert torch.equal(first, again), "two runs of the same split-K launch differ"
+    return first
+
+
+@pytest.mark.parametrize("name,cfg,tb", [
+    ("register-staged", dict(tile_i=64, tile_j=64, split_k=4, pipeline=1), False),
+    ("direct-to-LDS", dict(tile_i=128, tile_j=128, split_k=4, pipeline=3), True),
+    ("default pipeline", dict(tile_i=128, tile_j=128, split_k=3), True),
+])
+def test_gemm_split_k_is_deterministic(gpu, name, cfg, tb):
+    from amos_amd import _lib, ops
+    torch.manual_seed(1)
+    M, N, K = 200, 264, 4096
+    a = torch.randn(M, K, device="cuda").half()
+    b = (torch.randn(N, K, device="cuda") if tb else torch.randn(K, N, device="cuda")).half()
+    d = ops.gemm_desc(M, N, K, torch.float16, False, tb)
+    kname = ops.kernel_name(_lib.AMOS_OP_GEMM, d, cfg)
+    if name == "direct-to-LDS":
+        assert "amos_gemm_tn" in kname, kname
+    need = _lib.load().amos_workspace_bytes(_lib.AMOS_OP_GEMM, ctypes.byref(d), ctypes.byref(ops.make_config(cfg)))
+    assert need >= cfg["split_k"] * M * N * 4, "the workspace has room for one slice of the output per split"
+    got = _repeat_equal(lambda: ops.gemm(a, b, False, tb, config=cfg))
+    ref = a.double() @ (b.double().t() if tb else b.double())
+    mx, mean = _rel(got.cpu().numpy(), ref.cpu().numpy())
+    assert mx <= MAX_REL and mean <= MEAN_REL, "%s (%s): max_rel %.3e mean_rel %.3e" % (name, kname, mx, mean)
+
+
+def test_gemm_split_k_int8_equals_the_unsplit_product(gpu):
+    from amos_amd import ops
+    torch.manual_seed(2)
+    a = torch.randint(-128, 128, (96, 2048), device="cuda", dtype=torch.int8)
+    b = torch.randint(-128, 128, (160, 2048), device="cuda", dtype=torch.int8)
+    one = ops.gemm(a, b, False, True, config=dict(tile_i=128, tile_j=128, split_k=1, pipeline=3))
+    for pipe in (1, 3):
+        four = ops.gemm(a, b, False, True, config=dict(tile_i=128, tile_j=128, split_k=4, pipeline=pipe))
+        assert torch.equal(one, four)
+    assert torch.equal(one.cpu(), (a.cpu().int() @ b.cpu().int().t()))
+
+
+def test_batched_gemm_split_k(gpu):
+    from amos_amd import ops
+    torch.manual_seed(3)
+    a = torch.randn(3, 72, 1024, device="cuda").half()
+    b = torch.randn(3, 1024, 40, device="cuda").half()
+    cfg = dict(tile_i=64, tile_j=64, split_k=1, pipeline=1)
+    ref = torch.bmm(a.double(), b.double())
+    # (a batched product keeps split 1 in the register-staged kernel's plan: the call still runs)
+    got = _repeat_equal(lambda: ops.bgemm(a, b, config=dict(cfg, split_k=2)))
+    mx, mean = _rel(got.cpu().numpy(), ref.cpu().numpy())
+    assert mx <= MAX_REL and mean <= MEAN_REL
+
+
+@pytest.mark.parametrize("pipeline", ["patch", "nchw"])
+def test_conv_split_k_is_deterministic(gpu, pipeline):
+    from amos_amd import _lib, ops
+    torch.manual_seed(4)
+    x = torch.randn(2, 256, 12, 12, device="cuda").half()
+    w = (torch.randn(64, 256, 3, 3, device="cuda") * 0.05).half()
+    cfg = dict(tile_i=64, tile_j=128, split_k=2,
+               pipeline=_lib.AMOS_PIPE_NCHW if pipeline == "nchw" else _lib.AMOS_PIPE_PATCH8)
+    d = ops.conv_desc((2, 256, 1, 12, 12), (64, 256, 1, 3, 3), torch.float16, (1, 1, 1), (0, 1, 1), (1, 1, 1))
+    kname = ops.kernel_name(_lib.AMOS_OP_CONV2D, d, cfg)
+    assert ("amos_conv_nchw" if pipeline == "nchw" else "amos_conv_fprop") in kname, kname
+    got = _repeat_equal(lambda: ops.conv2d(x, w, 1, 1, 1, config=cfg))
+    ref = torch.nn.functional.conv2d(x.double(), w.double(), padding=1)
+    mx, mean = _rel(got.cpu().numpy(), ref.cpu().numpy())
+    assert mx <= MAX_REL and mean <= MEAN_REL, "%s: max_rel %.3e mean_rel %.3e" % (kname, mx, mean)
+    # the fused tail's operand may be the output itself: every read of the call is behind it when
+    # the reduction writes the output
+    out = torch.full_like(got, 0.5)
+    ops.conv2d(x, w, 1, 1, 1, out=out, add=out, config=cfg)
+    torch.cuda.synchronize()
+    assert torch.allclose(out, got + 0.5, rtol=0, atol=1e-4)
+
+
+def test_split_k_without_the_workspace(gpu):
+    """through the C ABI with a null workspace: the register-staged kernel accumulates with atomics
+    (right sums, any order) and refuses a fused-tail operand that is the output; the direct-to-LDS
+    kernel, which has no atomic path, refuses the split"""
+    from amos_amd import _lib, ops
+    lib = _lib.load()
+    torch.manual_seed(5)
+    M, N, K = 128, 128, 2048
+    a = torch.randn(M, K, device="cuda").half()
+    b = torch.randn(N, K, device="cuda").half()
+    out = torch.zeros(M, N, device="cuda")
+    d = ops.gemm_desc(M, N, K, torch.float16, False, True)
+    cfg = ops.make_config(dict(tile_i=64, tile_j=64, split_k=4, pipeline=1))
+    _lib.check(lib.amos_gemm(ctypes.byref(d), ctypes.byref(cfg), a.data_ptr(), b.data_ptr(), out.data_ptr(), None, 0, None))
+    torch.cuda.synchronize()
+    mx, mean = _rel(out.cpu().numpy(), (a.double() @ b.double().t()).cpu().numpy())
+    assert mx <= MAX_REL and mean <= MEAN_REL
+    epi = _lib.Epilogue()
+    epi.kind, epi.operand, epi.dtype, epi.ld, epi.stride = _lib.AMOS_EPI_ADD, out.data_ptr(), _lib.AMOS_F32, N, 0
+    rc = lib.amos_run_fused(_lib.AMOS_OP_GEMM, ctypes.byref(d), ctypes.byref(cfg), ctypes.byref(epi), a.data_ptr(),
+                            b.data_ptr(), out.data_ptr(), None, 0, None)
+    assert rc == _lib.AMOS_ERR_BAD_ARG and b"alias" in lib.amos_last_error()
+    tn = ops.make_config(dict(tile_i=128, tile_j=128, split_k=4, pipeline=3))
+    rc = lib.amos_gemm(ctypes.byref(d), ctypes.byref(tn), a.data_ptr(), b.data_ptr(), out.data_ptr(), None, 0, None)
+    assert rc in (_lib.AMOS_ERR_WORKSPACE, _lib.AMOS_ERR_INFEASIBLE), lib.amos_last_error()
