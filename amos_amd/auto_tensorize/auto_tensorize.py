@@ -226,20 +226,32 @@ def auto_tensorize_v4(target_dag, target, schedule_log_file, measure_opt, schedu
             realised = {}
             for pipe in (_lib.AMOS_PIPE_PATCH, _lib.AMOS_PIPE_STAGED):
                 realised.setdefault(tuple(mapping_of_pipeline(match_result, pipe)), pipe)
+            if rnd == 0:
+                # trials only for mappings that can run: the others keep weight 0
+                runnable = [_realisation(match_result, r, realised) is not None for r in all_mappings[match_id]]
+                print("Num runnable mapping:", sum(runnable), flush=True)
+                if any(runnable):
+                    weights = [w if ok else 0.0 for w, ok in zip(weights, runnable)]
+                    total = sum(weights)
+                    weights = [w / total for w in weights]
+                    mapping_weights[match_id] = weights
+                    tune_trials = [math.ceil(trials_per_matching * x) for x in weights]
+                    print("Weights of the runnable mappings", weights, flush=True)
             for mapping_id, record in enumerate(all_mappings[match_id]):
                 print("Current explored mapping:", str(record), flush=True)
                 new_state = app.apply(record, drop_output=drop_output)
                 key = record.as_key()
                 log = os.path.join(schedule_log_dir, "mapping_" + str(key) + "_" + schedule_log_file)
                 value, params = 1 / MAX_FLOAT, None
-                pipe = _equivalent_pipeline(match_result, record, realised)
-                if pipe is None:
+                how = _realisation(match_result, record, realised)
+                if how is None:
                     print("No kernel instance realises this mapping; skipped.", flush=True)
                 else:
+                    pipes, rows = how
                     if key not in cache:
                         try:
                             gen = MI355XScheduleGenerator(
-                                match_result, new_state, log_file=log,
+                                match_result, new_state, log_file=log, rows=rows,
                                 perf_percentage=perf_percentage if enable_perf_model else 1.0)
                         except NoKernelError as e:
                             print("No kernel for this compute:", e, flush=True)
@@ -247,8 +259,8 @@ def auto_tensorize_v4(target_dag, target, schedule_log_file, measure_opt, schedu
                         if gen is not None:
                             if os.path.exists(log) and os.path.getsize(log) > 0:
                                 gen.load_from_file(log)
-                            gen._candidates = gen.candidates([pipe])
-                            cache[key] = ScheduleContext(gen, MI355XScheduleApplier(match_result, gen.lowered), pipe)
+                            gen._candidates = gen.candidates(pipes)
+                            cache[key] = ScheduleContext(gen, MI355XScheduleApplier(match_result, gen.lowered), pipes[0])
                     ctx = cache.get(key)
                     if ctx is not None:
                         if tune_trials[mapping_id] and not pure_test:
@@ -268,6 +280,8 @@ def auto_tensorize_v4(target_dag, target, schedule_log_file, measure_opt, schedu
                 print(f"Round {rnd+1}, Match {match_id+1}, Mapping {mapping_id+1}: {value}/{best_value}"
                       f"({1/best_value*1e3} ms), {str(record)}, {str(params)}", flush=True)
             if not pure_test:
+                # (mappings without a kernel stay at weight 0: the update is over the runnable ones)
+                ran = [v > 1 / MAX_FLOAT for v in best_values]
                 max_value = max(best_values)
                 exp_scores = [math.exp(min(0.0, x - max_value)) for x in best_values]
                 s = sum(exp_scores)
@@ -275,7 +289,7 @@ def auto_tensorize_v4(target_dag, target, schedule_log_file, measure_opt, schedu
                 delta = [new_weights[i] - weights[i] for i in range(len(weights))]
                 new_updates = [delta[i] + momentum * updates[i] for i in range(len(updates))]
                 new_weights = [weights[i] + new_updates[i] for i in range(len(new_updates))]
-                exp_scores = [math.exp(x) for x in new_weights]
+                exp_scores = [math.exp(x) if ok or not any(ran) else 0.0 for x, ok in zip(new_weights, ran)]
                 s = sum(exp_scores)
                 mapping_weights[match_id] = [x / s for x in exp_scores]
                 weights_updates[match_id] = new_updates
@@ -290,6 +304,37 @@ def auto_tensorize_v4(target_dag, target, schedule_log_file, measure_opt, schedu
         return AutoTensorizeResult()
     return AutoTensorizeResult(best_ctx.schedule_gen, best_ctx.schedule_app, best_params, 1 / best_value,
                                mapping=best_mapping)
+
+
+def _realisation(match_result, record, realised):
+    """How a mapping runs: (pipelines, rows) or None.  `rows` names the output loops fused into the
+    rows of the implicit GEMM where that is not all of them (lowering.remap_conv2d_rows: a 2-d
+    convolution whose mapping keeps the batch loop and leaves p and / or q as time loops); the
+    reduce side decides the kernel -- channels only: the patch-staged kernels, whose window taps
+    are time loops; channels and both window loops: the register-staged kernel (im2col)."""
+    patch_family = [_lib.AMOS_PIPE_PATCH, _lib.AMOS_PIPE_PATCH8, _lib.AMOS_PIPE_NCHW]
+    pipe = _equivalent_pipeline(match_result, record, realised)
+    if pipe is not None:
+        return (patch_family if pipe == _lib.AMOS_PIPE_PATCH else [pipe]), None
+    names = {ia.var.name: [t.var.name for t in lst] for ia, lst in match_result.axis_map.items()}
+    if sorted(names) != ["i", "j", "rk"]:
+        return None
+    bits = record.vmap_choice[0]
+    i_set = sorted(set(n for n, b in zip(names["i"], bits) if b))
+    rk_set = sorted(set(n for n, b in zip(names["rk"], bits) if b))
+    spatial, reduce_all = sorted(set(names["i"])), sorted(set(names["rk"]))
+    if spatial != ["n", "p", "q"] or reduce_all != ["rc", "rr", "rs"] or "n" not in i_set:
+        return None
+    if rk_set == ["rc"]:
+        # (rows n alone: one image as wide as N*Q*S columns, whose patch of a tile no LDS holds)
+        if i_set == ["n"]:
+            return None
+        pipes = patch_family
+    elif rk_set == reduce_all:
+        pipes = [_lib.AMOS_PIPE_STAGED]
+    else:
+        return None
+    return pipes, "".join(i_set)
 
 
 def _equivalent_pipeline(match_result, record, realised):

@@ -736,6 +736,80 @@ def _lower_conv(main_op, l0, l1, iters, forms0, forms1):
     return low
 
 
+def remap_conv2d_rows(low, rows):
+    """The same convolution with only the loops in `rows` (a subset of 'n', 'p', 'q' that holds 'n')
+    fused into the rows of the implicit GEMM, the other output loops being time loops: every value
+    of such a loop is a convolution of its own, with its own copy of the input rows / columns it
+    reads (no reuse of the halo between neighbouring outputs along that loop), all of them batched
+    into one launch.  The reference reaches the same loop structure by fusing only the mapped
+    loops into the intrinsic's axis (tensorization_phases/compute_transform.py:343-499).
+
+      rows n,q (p a time loop): image n holds, for every output row p, its own R input rows, one
+                                block under the other; window R x S, stride R along H
+      rows n,p (q a time loop): the same with H and W swapped (the copied axis is the image's H):
+                                per output column q its own S input columns; window S x R
+      rows n (p, q time loops): one image of P blocks of R rows and N*Q blocks of S columns;
+                                window R x S, strides R and S
+
+    The copies are dimension-separable gathers (zero padding along the copied axis included) into
+    NHWC images; the weights are gathered into the window-major layout that goes with it and the
+    result is gathered back to NKPQ."""
+    rows = "".join(sorted(rows))
+    if rows == "npq":
+        return low
+    if low.kind != "conv2d" or low.attrs.get("layout", "nchw") != "nchw" or low.gathers or low.out_view is not None \
+            or low.constants or low.computed or len(low.attrs["x_shape"]) != 4 or rows not in ("nq", "np", "n"):
+        raise NoKernelError("no kernel for this convolution with rows %s" % rows)
+    N, C, H, W = low.attrs["x_shape"]
+    K, _, R, S = low.attrs["w_shape"]
+    (sh, sw), (ph, pw), (dh, dw) = low.attrs["stride"], low.attrs["pad"], low.attrs["dil"]
+    P = (H + 2 * ph - ((R - 1) * dh + 1)) // sh + 1
+    Q = (W + 2 * pw - ((S - 1) * dw + 1)) // sw + 1
+    src, wt = low.inputs
+    hw = H * W
+    # source offsets of the copied axes: (output index, tap) -> input row / column, -1 in the padding
+    rows_of = [(p * sh - ph + r * dh) * W if 0 <= p * sh - ph + r * dh < H else -1 for p in range(P) for r in range(R)]
+    cols_of = [q * sw - pw + s * dw if 0 <= q * sw - pw + s * dw < W else -1 for q in range(Q) for s in range(S)]
+    n_tab, c_tab = [n * C * hw for n in range(N)], [c * hw for c in range(C)]
+    c = _lib.ConvDesc()
+    c.C, c.K, c.D, c.T = C, K, 1, 1
+    c.stride_d, c.pad_d, c.dil_d = 1, 0, 1
+    c.stride_h, c.pad_h, c.dil_h = 1, 0, 1
+    c.in_dtype, c.out_dtype = low.desc.in_dtype, low.desc.out_dtype
+    c.layout = _lib.LAYOUT_CODE["nhwc"]
+    krs = C * R * S
+    if rows == "nq":
+        x_view = OperandView(src, [N, P * R, W, C], [n_tab, rows_of, list(range(W)), c_tab], src.dtype)
+        c.N, c.H, c.W, c.R, c.S = N, P * R, W, R, S
+        c.stride_h = R
+        c.stride_w, c.pad_w, c.dil_w = sw, pw, dw
+        w_view = OperandView(wt, [R, S, C, K], [[r * S for r in range(R)], list(range(S)), [cc * R * S for cc in range(C)],
+                                                [k * krs for k in range(K)]], wt.dtype)
+        o_tabs = [[n * P * Q * K for n in range(N)], list(range(K)), [p * Q * K for p in range(P)], [q * K for q in range(Q)]]
+    elif rows == "np":
+        x_view = OperandView(src, [N, Q * S, H, C], [n_tab, cols_of, [h * W for h in range(H)], c_tab], src.dtype)
+        c.N, c.H, c.W, c.R, c.S = N, Q * S, H, S, R
+        c.stride_h = S
+        c.stride_w, c.pad_w, c.dil_w = sh, ph, dh
+        w_view = OperandView(wt, [S, R, C, K], [list(range(S)), [r * S for r in range(R)], [cc * R * S for cc in range(C)],
+                                                [k * krs for k in range(K)]], wt.dtype)
+        o_tabs = [[n * Q * P * K for n in range(N)], list(range(K)), [p * K for p in range(P)], [q * P * K for q in range(Q)]]
+    else:
+        x_view = OperandView(src, [P * R, N, Q * S, C], [rows_of, n_tab, cols_of, c_tab], src.dtype)
+        c.N, c.H, c.W, c.R, c.S = 1, P * R, N * Q * S, R, S
+        c.stride_h = R
+        c.stride_w, c.pad_w, c.dil_w = S, 0, 1
+        w_view = OperandView(wt, [R, S, C, K], [[r * S for r in range(R)], list(range(S)), [cc * R * S for cc in range(C)],
+                                                [k * krs for k in range(K)]], wt.dtype)
+        o_tabs = [[n * Q * K for n in range(N)], list(range(K)), [p * N * Q * K for p in range(P)], [q * K for q in range(Q)]]
+    attrs = dict(low.attrs, layout="nhwc", rows=rows)
+    out = LoweredOp("conv2d", low.op_code, c, [src, wt], low.output, attrs)
+    out.add_input = low.add_input
+    out.gathers = {0: x_view, 1: w_view}
+    out.out_view = OperandView(None, [N, K, P, Q], o_tabs, low.output.dtype)
+    return out
+
+
 def _numel(shape):
     n = 1
     for e in shape:

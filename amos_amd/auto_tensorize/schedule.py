@@ -117,6 +117,11 @@ class MI355XScheduleGenerator(object):
         self.state = new_state
         main_op = list(intrin_match_result.main_op_map.values())[0]
         self.lowered = lower_main_op(main_op, getattr(intrin_match_result, "target_dag", None))
+        # a mapping that fuses only some of the output loops into the rows of the implicit GEMM
+        rows = kwargs.get("rows")
+        if rows is not None:
+            from .lowering import remap_conv2d_rows
+            self.lowered = remap_conv2d_rows(self.lowered, rows)
         self.log_file = log_file
         self.verbose_init = verbose_init
         self.entries = []
@@ -212,7 +217,8 @@ class MI355XScheduleGenerator(object):
             out.append(p)
 
         d = _lib.KernelConfig()
-        if lib.amos_default_config(low.op_code, ctypes.byref(low.desc), ctypes.byref(d)) == 0:
+        if lib.amos_default_config(low.op_code, ctypes.byref(low.desc), ctypes.byref(d)) == 0 and (
+                pipelines is None or d.pipeline in pipelines):
             add(KernelParams(d.tile_i, d.tile_j, d.split_k, d.pipeline))
         is_conv = low.kind in ("conv2d", "conv3d")
         pipes = pipelines if pipelines is not None else (
@@ -251,7 +257,19 @@ class MI355XScheduleGenerator(object):
         cfg = params.to_config()
         rc = _lib.load().amos_estimate_seconds(self.lowered.op_code, ctypes.byref(self.lowered.desc),
                                                ctypes.byref(cfg), ctypes.byref(sec))
-        return sec.value if rc == 0 else MAX_FLOAT
+        if rc != 0:
+            return MAX_FLOAT
+        # stages materialised around the kernel (gathers of an operand, of the result): a launch
+        # each, their bytes read and written once at about a quarter of the HBM rate
+        extra = 0.0
+        views = list(self.lowered.gathers.values()) + ([self.lowered.out_view] if self.lowered.out_view is not None else [])
+        for v in views:
+            n = 1
+            for e in v.shape:
+                n *= int(e)
+            width = {"float16": 2, "bfloat16": 2, "int8": 1}.get(v.dtype, 4)
+            extra += 3e-6 + 2.0 * n * width / 2.0e12
+        return sec.value + extra
 
 
 class MI355XScheduleApplier(object):

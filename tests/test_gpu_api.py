@@ -409,3 +409,86 @@ def test_eltwise_entry_point(gpu, dtype):
     with pytest.raises(Exception, match="stack|program"):
         ops.Eltwise(["add"], 1, tx.dtype, n)([tx])
 
+
+
+@pytest.mark.parametrize("dtype", ["float16", "int8"])
+@pytest.mark.parametrize("rows", ["npq", "nq", "np", "n"])
+def test_conv2d_mapping_classes_run_and_agree(gpu, rows, dtype):
+    """Mappings that fuse only some of the output loops into the rows of the implicit GEMM (p and / or
+    q stay time loops), with the reduce side on channels only (patch-staged kernels, window taps as
+    time loops) or on channels and both window loops (register-staged kernel): every class against
+    the oracle (the reference builds a kernel per mapping:
+    tensorization_phases/compute_transform.py:343-499)"""
+    from amos_amd import _lib
+    from amos_amd.auto_tensorize.lowering import lower_main_op, remap_conv2d_rows
+    from amos_amd.auto_tensorize.runtime import Module
+    from amos_amd.auto_tensorize.schedule import KernelParams
+    N, C, H, W, K, stride, pad, dil = 4, 64, 10, 12, 40, 1, 1, 1
+    if dtype == "int8":
+        A, B, Conv = conv2d(N, C, H, W, K, 3, 3, stride, pad, dil, dtype="int8", out_dtype="int32", exact_int=True)
+    else:
+        A, B, Conv = conv2d(N, C, H, W, K, 3, 3, stride, pad, dil)
+    dag = at.compute_dag_from_tensors([Conv])
+    main_op = [op for op in dag.op_lst if op.reduce_axis][0]
+    low = remap_conv2d_rows(lower_main_op(main_op, dag), rows)
+    rng = np.random.default_rng(3)
+    if dtype == "int8":
+        a = rng.integers(-128, 128, [int(s) for s in A.shape]).astype(np.int8)
+        b = rng.integers(-64, 64, [int(s) for s in B.shape]).astype(np.int8)
+        ref = co.lib_conv2d(a, b, "int8", stride, pad, dil)
+    else:
+        a = rng.uniform(-1, 1, [int(s) for s in A.shape]).astype(np.float16)
+        b = rng.uniform(-1, 1, [int(s) for s in B.shape]).astype(np.float16)
+        ref = co.lib_conv2d(a, b, "float16", stride, pad, dil, acc="float64")
+    ctx = tvm.context("hip", 0)
+    ran = []
+    for pipe in (_lib.AMOS_PIPE_PATCH8, _lib.AMOS_PIPE_STAGED):
+        params = KernelParams(64, 128, 1, pipe)
+        func = Module(low, params, [A, B, Conv])
+        y = tvm.nd.array(np.zeros([int(s) for s in Conv.shape], dtype=ref.dtype if dtype == "int8" else np.float32), ctx)
+        try:
+            func(tvm.nd.array(a, ctx), tvm.nd.array(b, ctx), y)
+        except _lib.AmosError as e:
+            assert pipe == _lib.AMOS_PIPE_PATCH8 and "not applicable" in str(e), str(e)
+            continue
+        ctx.sync()
+        name = func.imported_modules[0].get_source()
+        assert ("amos_conv_fprop" if pipe == _lib.AMOS_PIPE_PATCH8 else "amos_igemm") in name, name
+        if dtype == "int8":
+            assert np.array_equal(y.asnumpy(), ref), (rows, pipe)
+        else:
+            mx, mean = co.rel_errors(y.asnumpy(), ref)
+            assert mx <= 1e-2 and mean <= 1e-3, (rows, pipe, mx, mean)
+        ran.append(pipe)
+    # the register-staged kernel runs every class; the patch-staged one all but "rows n" at most
+    assert _lib.AMOS_PIPE_STAGED in ran and (rows == "n" or _lib.AMOS_PIPE_PATCH8 in ran)
+
+
+def test_v4_times_seven_mapping_classes(gpu, tmp_path, capsys):
+    # the convolution of the reference's tutorial (README.md:174-261): 20 feasible mappings
+    A, B, Conv = conv2d(16, 64, 14, 14, 64, 3, 3, 1, 1, 1)
+    opt = at.MeasureOptions(target="hip", number=3, min_repeat_ms=2)
+    res = at.auto_tensorize_v4(at.compute_dag_from_tensors([Conv]), "hip", "conv.log", opt,
+                               schedule_log_dir=str(tmp_path / "logs"), trials=60, repeat_rounds=1,
+                               search_group_size=1)
+    out = capsys.readouterr().out
+    assert res.defined()
+    assert "Num mapping: 20" in out and "Num runnable mapping: 7" in out
+    timed = set()
+    for line in out.splitlines():
+        if line.startswith("Round 1, Match 1, Mapping"):
+            value = float(line.split(": ")[1].split("/")[0])
+            if value > 1.0:   # (1 / seconds of the mapping's best schedule; 1e-10 = nothing ran)
+                timed.add(line.split('"vmap": ')[1].split("]")[0])
+    assert len(timed) == 7, out[-3000:]
+    # the winner runs and is right
+    sch, args = at.get_schedule(res.sch_app, res.params)
+    func = tvm.build(sch, args, "hip")
+    rng = np.random.default_rng(4)
+    a = rng.uniform(-1, 1, [int(s) for s in A.shape]).astype(np.float16)
+    b = rng.uniform(-1, 1, [int(s) for s in B.shape]).astype(np.float16)
+    ctx = tvm.context("hip", 0)
+    y = tvm.nd.array(np.zeros([int(s) for s in Conv.shape], dtype=np.float32), ctx)
+    func(tvm.nd.array(a, ctx), tvm.nd.array(b, ctx), y)
+    mx, mean = co.rel_errors(y.asnumpy(), co.lib_conv2d(a, b, "float16", 1, 1, 1, acc="float64"))
+    assert mx <= 1e-2 and mean <= 1e-3
