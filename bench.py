@@ -93,7 +93,7 @@ def _timed(fn):
     return time.perf_counter() - t0
 
 
-def run_all_configs(cpu=True, only=None):
+def run_all_configs(cpu=True, only=None, launches=None):
     """Every configuration of the path: GPU ms, TFLOP/s (TOP/s), % of the MFMA peak, % of the
     HBM roof for the algorithmic bytes, which roof binds, and the te_literal CPU loop nest
     (1 thread and all cores) on a slab of the same workload, linearly scaled."""
@@ -108,7 +108,10 @@ def run_all_configs(cpu=True, only=None):
 
     def gpu_time(op, desc, i0, i1, out, fused=None):
         cfg = ops.default_config(op, desc)
-        t = ops.time_op(op, desc, i0, i1, out, config=cfg, number=20, repeat=3, min_repeat_ms=100, add=fused)
+        if launches:   # (a fixed, small number of launches: runs under a profiler)
+            t = ops.time_op(op, desc, i0, i1, out, config=cfg, number=launches, repeat=1, min_repeat_ms=0, add=fused)
+        else:
+            t = ops.time_op(op, desc, i0, i1, out, config=cfg, number=20, repeat=3, min_repeat_ms=100, add=fused)
         return min(t), cfg
 
     def add(name, op, desc, hin, dtype, flop, nbytes, out_shape, cpu_fn, frac, fused_tail=False):
@@ -128,7 +131,8 @@ def run_all_configs(cpu=True, only=None):
                "gpu_us": sec * 1e6, "tflops": flop / sec / 1e12,
                "pct_mfma_peak": 100 * t_mfma / sec, "pct_hbm_roof": 100 * t_hbm / sec,
                "bound": "mfma" if t_mfma >= t_hbm else "hbm", "flop": flop, "bytes": nbytes}
-        if cfg.pipeline == _lib.AMOS_PIPE_NCHW and not fused_tail:
+        row["traffic_bytes"] = measured_traffic(row["kernel"])
+        if cfg.pipeline == _lib.AMOS_PIPE_NCHW and not fused_tail and not launches:
             # the same convolution where the owner of the weights has packed them once
             # (amos_conv_pack_weights + AMOS_FLAG_WEIGHTS_PACKED): no packing launch in the call
             lib = _lib.load()
@@ -371,6 +375,10 @@ def main():
                          "dispatcher, write JSON here")
     ap.add_argument("--networks", default="resnet18,resnet50,mobilenet_v1,bertbase,shufflenet,milstm",
                     help="the networks --network covers, comma-separated")
+    ap.add_argument("--config", default=None,
+                    help="run only the configuration whose name contains this text (C2, C3 fp16, C4 int8, C5a, "
+                         "C5b), --steps launches of it, print its row and exit: the command that the counter "
+                         "summaries under profiles/ were made with")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a 256 MiB device copy, the known-size kernel that rocprofv3's "
                          "FETCH_SIZE / WRITE_SIZE readings are scaled by")
@@ -384,6 +392,18 @@ def main():
     from amos_amd import _lib, ops
     if not torch.cuda.is_available():
         sys.exit("bench.py needs a GPU")
+    if args.config:
+        if args.calibrate_copy:
+            src = torch.empty(256 << 20, dtype=torch.uint8, device="cuda").random_()
+            dst = torch.empty_like(src)
+            for _ in range(3):
+                dst.copy_(src)
+            torch.cuda.synchronize()
+            del src, dst
+        rows = run_all_configs(cpu=False, only=(args.config,), launches=max(1, args.steps))
+        rows = [r for r in rows if " + D" not in r["config"]]
+        print(json.dumps(rows))
+        return
     n = 8192
     rng = np.random.default_rng(0)
     a = rng.uniform(-1, 1, (n, n)).astype(np.float32).astype(np.float16)

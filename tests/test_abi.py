@@ -178,3 +178,44 @@ def test_module_refuses_arrays_that_are_not_the_declared_tensors():
         mod(a.float(), b, torch.empty(32, 48))                      # float32 input wrapped by array()
     with pytest.raises(ValueError, match="device array"):
         mod(a, b, torch.empty(32, 48))                              # right shapes, but host memory
+
+
+@pytest.mark.parametrize("waves", [4, 8])
+@pytest.mark.parametrize("I,J,K", [(8192, 8192, 8192), (8000, 8100, 4096)])
+def test_gemm_tn_copy_addresses_stay_inside_operands(waves, I, J, K):
+    """The direct-to-LDS GEMM's address arithmetic (gemm_tn_kernel.h: a wave copies 1 KB chunks
+    q = wave + NW * u of a stage, lane l the 16 bytes (row 8 * q' + l / 8, swizzled chunk)),
+    evaluated on the host for the four- and the eight-wave grid of the 256x256 tile: every byte a
+    lane fetches lies inside its operand, every LDS byte it lands on inside the stage.  (The
+    four-wave instance faulted on the GPU at 8192^3 and is withdrawn; its addresses are the same
+    set as the eight-wave instance's, so the fault is not an index error of the source.  What
+    differs: its 128x128 wave tile leaves the 256 accumulator registers in scratch memory --
+    1040 bytes per lane -- and the kernel's launch code refuses instances with scratch.)"""
+    ES, BI, BJ, NS = 2, 256, 256, 2
+    NW, QA, CH = waves, BI // 8, (BI + BJ) // 8 // waves
+    lda = ldb = K
+    stage_bytes = (BI + BJ) * 128
+    a_bytes, b_bytes = I * lda * ES, J * ldb * ES
+    tiles_i, tiles_j = -(-I // BI), -(-J // BJ)
+    seen = set()
+    for tile_i, tile_j in {(0, 0), (tiles_i - 1, tiles_j - 1), (tiles_i - 1, 0), (0, tiles_j - 1)}:
+        bi0, bj0 = tile_i * BI, tile_j * BJ
+        for wave in range(NW):
+            for u in range(CH):
+                q = wave + NW * u
+                assert 0 <= q * 1024 and (q + 1) * 1024 <= stage_bytes
+                seen.add(q)
+                for lane in range(64):
+                    qq = q if q < QA else q - QA
+                    row = qq * 8 + (lane >> 3)
+                    chunk = (lane & 7) ^ ((row ^ (row >> 3)) & 7)
+                    for kt in (0, K * ES // 128 - 1):
+                        if q < QA:
+                            r = row if bi0 + row < I else I - 1 - bi0
+                            off = bi0 * lda * ES + r * lda * ES + chunk * 16 + kt * 128
+                            assert 0 <= off and off + 16 <= a_bytes
+                        else:
+                            r = row if bj0 + row < J else J - 1 - bj0
+                            off = bj0 * ldb * ES + r * ldb * ES + chunk * 16 + kt * 128
+                            assert 0 <= off and off + 16 <= b_bytes
+    assert seen == set(range((BI + BJ) // 8))
