@@ -10,6 +10,7 @@ conv3d), each timed in the same run next to the CPU loop nest on a slab of the s
 conv2d fp16 / int8, conv3d) and writes a per-config table as JSON to FILE.
 """
 import argparse
+import ctypes
 import json
 import os
 import sys
@@ -470,14 +471,21 @@ def main():
         for r in run_all_configs(cpu=not args.no_cpu, only=("C3 fp16", "C4 int8", "C5a fp16", "C5b fp16")):
             row = {k: r[k] for k in ("config", "kernel", "split_k", "gpu_us", "tflops", "pct_mfma_peak",
                                      "pct_hbm_roof", "bound")}
+            for k in ("traffic_bytes", "gpu_us_weights_packed_once"):
+                if r.get(k) is not None:
+                    row[k] = r[k]
             if "cpu" in r:
                 row["cpu"] = {k: r["cpu"][k] for k in ("threads1_tflops", "threadsN_tflops", "cores",
                                                        "extrapolated_from")}
             per_op.append(row)
+        per_op[0]["traffic_bytes"] = line["roofline"]["traffic"]
         line["config"]["per_op"] = per_op
         line["config"]["per_op_note"] = ("gpu_us: mean seconds per call by HIP events (time_evaluator loop), every "
                                          "launch of a call included; tflops: TFLOP/s (int8: TOP/s); cpu: the "
-                                         "te_literal loop nest (gcc -O3) on a slab, scaled linearly")
+                                         "te_literal loop nest (gcc -O3) on a slab, scaled linearly; traffic_bytes: HBM-side "
+                                         "bytes per launch of the main kernel from the counter summaries under profiles/; "
+                                         "gpu_us_weights_packed_once: the same convolution where the owner of the weights "
+                                         "packed them once (no packing launch in the call)")
     if args.report:
         with open(args.report, "w") as f:
             json.dump(run_all_configs(cpu=not args.no_cpu, only=args.report_only), f, indent=1)
