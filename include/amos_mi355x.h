@@ -189,7 +189,16 @@ int amos_check_config(int op, const void* desc, const amos_kernel_config_t* cfg,
                       int64_t* lds_bytes, int64_t* acc_regs);
 /* bytes of device scratch the op's fastest pipeline wants (conv: repacked weights and
  * activations; GEMM and 1x1 convolutions: K-contiguous copies of operands); calls that get less
- * fall back to the register-staged pipeline, which needs none */
+ * fall back to the register-staged pipeline, which needs none.  With cfg->split_k > 1 the figure
+ * includes, behind the pipeline's own share, one slice of the output per split: the splits store
+ * their partial sums there and a second launch adds them in the order of the splits, so that a
+ * split-K result has the same bits on every run and the fused tail's operand may be the output
+ * (the reference reduces its split through shared memory,
+ * python/tvm/auto_tensorize/tensorization_phases/schedulers/cuda_split_K.py:868-914).  A call
+ * with split_k > 1 and less workspace accumulates with atomicAdd into the zeroed output where the
+ * kernel can (AMOS_PIPE_STAGED, AMOS_PIPE_PATCH*: sums in any order, an epilogue operand that
+ * aliases the output is refused) and returns AMOS_ERR_WORKSPACE where it cannot
+ * (AMOS_PIPE_DIRECT8, AMOS_PIPE_NCHW). */
 size_t amos_workspace_bytes(int op, const void* desc, const amos_kernel_config_t* cfg);
 /* the mapper's analytical estimate (seconds per launch) for a config: wave quantisation of the
  * grid over the CUs against MFMA issue time, HBM time for the algorithmic bytes, a launch floor
