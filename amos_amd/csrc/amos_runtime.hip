@@ -1172,6 +1172,11 @@ static int launch_conv_nchw(const Plan& pl, hipStream_t stream) {
     return set_error(AMOS_ERR_HIP, "hipFuncSetAttribute(%s): %s", inst->name, hipGetErrorString(attr_err));
   if (inst->static_lds)   // the kernel addresses its dynamic LDS from byte 0
     return set_error(AMOS_ERR_HIP, "%s was built with %d bytes of static LDS", inst->name, inst->static_lds);
+  // (the loader waves decide that their loads have landed by counting vector-memory operations in
+  // flight; register spills are such operations too)
+  if (inst->scratch_bytes && pl.nchw_wmode == NCHW_W_PACKED)
+    return set_error(AMOS_ERR_INFEASIBLE, "%s was built with %d bytes of scratch memory per lane (register "
+                     "spills), which its wait counts do not allow for", inst->name, inst->scratch_bytes);
   const ConvNchwParams& q = pl.nc;
   // what the kernel assumes of its launch: the tile of the instance, whole 64-byte chunks of
   // channels, a patch that fits the LDS asked for
