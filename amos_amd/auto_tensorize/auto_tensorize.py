@@ -29,6 +29,9 @@ class AutoTensorizeResult(object):
         self.params = params
         self.perf = perf          # seconds per run
         self.mapping = mapping
+        # auto_tensorize_v4: how many of the feasible mappings a kernel could run, and how many there were
+        self.num_runnable_mappings = None
+        self.num_feasible_mappings = None
 
     def defined(self):
         return ((self.sch_gen is not None) and (self.sch_app is not None)
@@ -207,6 +210,7 @@ def auto_tensorize_v4(target_dag, target, schedule_log_file, measure_opt, schedu
             self.schedule_gen, self.schedule_app, self.pipeline = schedule_gen, schedule_app, pipeline
 
     cache = {}
+    runnable_total = 0
     best_value, best_ctx, best_params, best_mapping = 1 / MAX_FLOAT, None, None, None
     checker = MI355XProgramChecker(verbose_init=False)
     beg = time.time()
@@ -230,6 +234,7 @@ def auto_tensorize_v4(target_dag, target, schedule_log_file, measure_opt, schedu
                 # trials only for mappings that can run: the others keep weight 0
                 runnable = [_realisation(match_result, r, realised) is not None for r in all_mappings[match_id]]
                 print("Num runnable mapping:", sum(runnable), flush=True)
+                runnable_total += sum(runnable)
                 if any(runnable):
                     weights = [w if ok else 0.0 for w, ok in zip(weights, runnable)]
                     total = sum(weights)
@@ -300,10 +305,10 @@ def auto_tensorize_v4(target_dag, target, schedule_log_file, measure_opt, schedu
                 print(f"mapping {str(k)}: explored {v.schedule_gen.num_entries()} schedules", flush=True)
     if not pure_test:
         print(f"Mapping exploration uses time {(time.time() - beg)} s.", flush=True)
-    if best_ctx is None:
-        return AutoTensorizeResult()
-    return AutoTensorizeResult(best_ctx.schedule_gen, best_ctx.schedule_app, best_params, 1 / best_value,
-                               mapping=best_mapping)
+    result = AutoTensorizeResult() if best_ctx is None else AutoTensorizeResult(
+        best_ctx.schedule_gen, best_ctx.schedule_app, best_params, 1 / best_value, mapping=best_mapping)
+    result.num_runnable_mappings, result.num_feasible_mappings = runnable_total, total_mappings
+    return result
 
 
 def _realisation(match_result, record, realised):

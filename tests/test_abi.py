@@ -219,3 +219,41 @@ def test_gemm_tn_copy_addresses_stay_inside_operands(waves, I, J, K):
                             off = bj0 * ldb * ES + r * ldb * ES + chunk * 16 + kt * 128
                             assert 0 <= off and off + 16 <= b_bytes
     assert seen == set(range((BI + BJ) // 8))
+
+
+@pytest.mark.parametrize("WI,WJ", [(2, 2), (4, 2)])
+def test_gemm_tn_fragment_and_strip_offsets_stay_inside_lds(WI, WJ):
+    """the same kernel's LDS side on the host, for the withdrawn four-wave grid (2 x 2 waves, wave
+    tile 128x128: TI = TJ = 8) and the shipped eight-wave one: every 16-byte fragment read
+    (lds_chunk_offset of the block's row plus whole 64-row strides for blocks beyond the fourth)
+    lies inside its operand's half of a stage, every fragment row of the tile is read by exactly
+    one (wave, block, lane row), and the epilogue's output strips lie inside the stages"""
+    BI = BJ = 256
+    NS, NW = 2, WI * WJ
+    TI, TJ = BI // (16 * WI), BJ // (16 * WJ)
+    OPER, STAGE = BI * 128, (BI + BJ) * 128
+
+    def lds_chunk_offset(row, chunk):
+        return row * 128 + ((chunk ^ ((row ^ (row >> 3)) & 7)) << 4)
+
+    rows_a, rows_b = set(), set()
+    for wave in range(NW):
+        wi, wj = wave // WJ, wave % WJ
+        for lane in range(64):
+            frag_row, frag_q = lane & 15, lane >> 4
+            frag_chunk = (frag_q >> 1) | ((frag_q & 1) << 1)
+            for ks in range(2):
+                for ab in range(TI):
+                    off = lds_chunk_offset(wi * TI * 16 + (ab & 3) * 16 + frag_row, ks * 4 + frag_chunk) + (ab >> 2) * 64 * 128
+                    assert 0 <= off and off + 16 <= OPER
+                    assert off // 128 == wi * TI * 16 + ab * 16 + frag_row
+                    rows_a.add((off // 128, wj))
+                for b in range(TJ):
+                    off = OPER + lds_chunk_offset(wj * TJ * 16 + (b & 3) * 16 + frag_row, ks * 4 + frag_chunk) + (b >> 2) * 64 * 128
+                    assert OPER <= off and off + 16 <= STAGE
+                    assert (off - OPER) // 128 == wj * TJ * 16 + b * 16 + frag_row
+                    rows_b.add(((off - OPER) // 128, wi))
+        SP = TJ * 16 + 4
+        assert (wave + 1) * 16 * SP * 4 <= NS * STAGE
+    assert rows_a == {(r, wj) for r in range(BI) for wj in range(WJ)}
+    assert rows_b == {(r, wi) for r in range(BJ) for wi in range(WI)}

@@ -474,6 +474,7 @@ def test_v4_times_seven_mapping_classes(gpu, tmp_path, capsys):
     out = capsys.readouterr().out
     assert res.defined()
     assert "Num mapping: 20" in out and "Num runnable mapping: 7" in out
+    assert (res.num_runnable_mappings, res.num_feasible_mappings) == (7, 20)
     timed = set()
     for line in out.splitlines():
         if line.startswith("Round 1, Match 1, Mapping"):
