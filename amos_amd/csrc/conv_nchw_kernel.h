@@ -110,6 +110,43 @@ __global__ __launch_bounds__(256) void amos_conv_pack_weights_kernel(const T* __
   }
 }
 
+// The same for nine taps (conv2d, T = 1) and 16-byte aligned weights: a thread takes the 144
+// contiguous bytes of one (output channel, 16-byte chunk of channels) -- nine 16-byte loads --,
+// transposes them in registers and writes one 16-byte vector per tap; threads of neighbouring
+// chunks write neighbouring 16 bytes of a row.  A tenth of the memory instructions of the
+// element-wise kernel above (C3's weights: 2.6 instead of 4.4 us).
+template <int ES>
+__global__ __launch_bounds__(256) void amos_conv_pack_weights9_kernel(const char* __restrict__ w, char* __restrict__ out,
+                                                                      int K, int C, NchwDiv div_chunks) {
+  constexpr int CG = 16 / ES;
+  const int chunks = C / CG;
+  const int total = K * chunks;
+  for (int u = (int)(blockIdx.x * 256 + threadIdx.x); u < total; u += (int)(gridDim.x * 256)) {
+    const int k = nchw_div(u, div_chunks), cq = u - k * chunks;
+    const char* const src = w + ((int64_t)k * C + (int64_t)cq * CG) * 9 * ES;
+    unsigned raw[36];
+#pragma unroll
+    for (int i = 0; i < 9; ++i) {
+      const v4i x = *(const v4i*)(src + i * 16);
+      raw[4 * i] = x.x; raw[4 * i + 1] = x.y; raw[4 * i + 2] = x.z; raw[4 * i + 3] = x.w;
+    }
+    // byte bb of channel ci at tap `tap` is byte (ci * 9 + tap) * ES + bb of the run
+#pragma unroll
+    for (int tap = 0; tap < 9; ++tap) {
+      v4i o;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        if (ES == 2)
+          o[j] = (int)nchw_gather<ES>(raw, ((2 * j) * 9 + tap) * 2, ((2 * j) * 9 + tap) * 2 + 1, ((2 * j + 1) * 9 + tap) * 2,
+                                      ((2 * j + 1) * 9 + tap) * 2 + 1);
+        else
+          o[j] = (int)nchw_gather<ES>(raw, (4 * j) * 9 + tap, (4 * j + 1) * 9 + tap, (4 * j + 2) * 9 + tap, (4 * j + 3) * 9 + tap);
+      }
+      *(v4i*)(out + (((int64_t)k * 9 + tap) * C + (int64_t)cq * CG) * ES) = o;
+    }
+  }
+}
+
 // bytes of one patch buffer: a constant of the tile, so that the second buffer is an immediate
 // offset of every LDS access; the last 1 KB of a buffer is a dump line for stores that have no
 // position to go to (one 16-byte slot per lane)
