@@ -353,7 +353,7 @@ struct Plan {
   size_t fewc_lds;
   // convolution read straight from NCDHW / KCTRS (0 = not used)
   int nchw;
-  int nchw_wmode, nchw_pt, nchw_groups, nchw_nwl;
+  int nchw_wmode, nchw_pt, nchw_groups, nchw_nwl, nchw_lb;
   int nchw_pack;            // 1: the weights are packed into the workspace in front of the kernel
   const void* nchw_w_src;   // ... from here
   ConvNchwParams nc;
@@ -796,17 +796,28 @@ static int plan_conv(Plan& pl, int op, const amos_conv_desc_t* d, const amos_ker
   if (cfg && cfg->pipeline == AMOS_PIPE_NCHW) {
     const int BI = cfg->tile_i > 0 ? cfg->tile_i : 64;
     const int BJ = cfg->tile_j > 0 ? cfg->tile_j : 128;
-    ConvNchwPlan np = conv_nchw_plan(c, op, BI, BJ);
+    // Weights: already packed by the caller (AMOS_FLAG_WEIGHTS_PACKED), packed into the workspace by
+    // this call, or -- without a workspace -- transposed by every workgroup on its way to LDS
+    const size_t packed_bytes = (size_t)(c.K * c.C * (op == AMOS_OP_CONV2D ? 1 : c.T) * 9) * (pl.dt == DT_I8 ? 1 : 2);
+    const bool will_pack = (cfg->reserved[0] & AMOS_FLAG_WEIGHTS_PACKED) ||
+                           (workspace && ws_bytes >= packed_bytes && ((uintptr_t)workspace & 255) == 0);
+    // patch loads of 16 bytes where the shape and the tensor's address allow them, the weights are
+    // packed and one round of the loaders covers the largest tile; else of 8
+    int lb = 8;
+    ConvNchwPlan np;
+    if (will_pack && conv_nchw_load_bytes(c) == 16 && aligned16(X)) {
+      np = conv_nchw_plan(c, op, BI, BJ, 16);
+      if (!np.why && np.max_groups <= 16 * nchw_loader_waves(true, np.max_groups)) lb = 16;
+    }
+    if (lb == 8) np = conv_nchw_plan(c, op, BI, BJ, 8);
     const char* why = np.why;
     if (!why && ((uintptr_t)X & 7)) why = "activations not 8-byte aligned";
     if (why) return set_error(AMOS_ERR_INFEASIBLE, "NCDHW-direct convolution not applicable: %s", why);
     ConvNchwParams& q = pl.nc;
     memset(&q, 0, sizeof(q));
     q.x = (const char*)X; q.w = (const char*)Wt; q.y = (char*)Y;
-    conv_nchw_shape(c, op, np.Wp, &q.s);
-    // Weights: already packed by the caller (AMOS_FLAG_WEIGHTS_PACKED), packed into the workspace by
-    // this call, or -- without a workspace -- transposed by every workgroup on its way to LDS
-    const size_t packed_bytes = (size_t)(c.K * c.C * q.s.T * 9) * (pl.dt == DT_I8 ? 1 : 2);
+    conv_nchw_shape(c, op, np.Wp, &q.s, lb);
+    pl.nchw_lb = lb;
     pl.nchw_pack = 0;
     pl.nchw_w_src = Wt;
     if (cfg->reserved[0] & AMOS_FLAG_WEIGHTS_PACKED) {
@@ -1151,14 +1162,14 @@ static int launch_conv(const Plan& pl, hipStream_t stream) {
   return 0;
 }
 
-static ConvNchwInstance* pick_conv_nchw(int dt, int ti, int tj, int wmode, int pt, int nwl) {
-  if (dt == DT_F16) return pick_conv_nchw_f16(ti, tj, wmode, pt, nwl);
-  if (dt == DT_BF16) return pick_conv_nchw_bf16(ti, tj, wmode, pt, nwl);
-  return pick_conv_nchw_i8(ti, tj, wmode, pt, nwl);
+static ConvNchwInstance* pick_conv_nchw(int dt, int ti, int tj, int wmode, int pt, int nwl, int lb) {
+  if (dt == DT_F16) return pick_conv_nchw_f16(ti, tj, wmode, pt, nwl, lb);
+  if (dt == DT_BF16) return pick_conv_nchw_bf16(ti, tj, wmode, pt, nwl, lb);
+  return pick_conv_nchw_i8(ti, tj, wmode, pt, nwl, lb);
 }
 
 static int launch_conv_nchw(const Plan& pl, hipStream_t stream) {
-  ConvNchwInstance* inst = pick_conv_nchw(pl.dt, pl.cfg.tile_i, pl.cfg.tile_j, pl.nchw_wmode, pl.nchw_pt, pl.nchw_nwl);
+  ConvNchwInstance* inst = pick_conv_nchw(pl.dt, pl.cfg.tile_i, pl.cfg.tile_j, pl.nchw_wmode, pl.nchw_pt, pl.nchw_nwl, pl.nchw_lb);
   if (!inst) return set_error(AMOS_ERR_INFEASIBLE, "no NCDHW-direct convolution instance");
   hipError_t attr_err = hipSuccess;
   std::call_once(inst->once, [&] {
@@ -1184,7 +1195,10 @@ static int launch_conv_nchw(const Plan& pl, hipStream_t stream) {
       q.max_pos > nchw_max_positions(inst->bj) ||
       pl.nchw_lds != (size_t)2 * 9 * inst->bi * 64 + (size_t)2 * nchw_patch_buffer_bytes(inst->bj) ||
       inst->threads != inst->bi * 8 + 64 * pl.nchw_nwl || inst->loader_waves != pl.nchw_nwl ||
-      inst->groups_per_thread != pl.nchw_pt || pl.nchw_pt * 16 * pl.nchw_nwl < pl.nchw_groups)
+      inst->groups_per_thread != pl.nchw_pt || pl.nchw_pt * 16 * pl.nchw_nwl < pl.nchw_groups ||
+      inst->load_bytes != pl.nchw_lb || (inst->load_bytes >> (pl.dt == DT_I8 ? 0 : 1)) != (1 << q.s.pg_shift) ||
+      ((uintptr_t)q.x & (uintptr_t)(inst->load_bytes - 1)) ||
+      ((int64_t)q.s.H * q.s.W * (pl.dt == DT_I8 ? 1 : 2)) % inst->load_bytes)
     return set_error(AMOS_ERR_BAD_ARG, "inconsistent plan for %s", inst->name);
   if (pl.nchw_pack)
     launch_conv_pack_weights(pl.dt == DT_I8 ? 1 : 2, pl.nchw_w_src, (void*)q.w, q.s.K, q.s.C, q.s.T * 9, stream);
@@ -1675,7 +1689,7 @@ const char* amos_kernel_name(int op, const void* desc, const amos_kernel_config_
   static char dummy_ws[256] __attribute__((aligned(256)));
   if (make_plan(pl, op, desc, cfg, dummy, dummy, dummy, dummy_ws, (size_t)-1)) return nullptr;
   if (pl.nchw) {
-    ConvNchwInstance* ni = pick_conv_nchw(pl.dt, pl.cfg.tile_i, pl.cfg.tile_j, pl.nchw_wmode, pl.nchw_pt, pl.nchw_nwl);
+    ConvNchwInstance* ni = pick_conv_nchw(pl.dt, pl.cfg.tile_i, pl.cfg.tile_j, pl.nchw_wmode, pl.nchw_pt, pl.nchw_nwl, pl.nchw_lb);
     return ni ? ni->name : nullptr;
   }
   if (pl.dw) return depthwise_name(pl.dt, pl.dw - 1);

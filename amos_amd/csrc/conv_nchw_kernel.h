@@ -6,10 +6,10 @@
 // The matrix core wants, per lane, 16 contiguous bytes of K of one row / column.  Neither tensor
 // offers that (in NCDHW the positions are contiguous, in KCTRS the window taps):
 //   * activations are transposed in registers on their way to LDS: a loader thread fetches, for
-//     one 16-byte chunk of channels, one 8-byte run of input positions per channel (16 lanes cover
-//     128 contiguous bytes of a channel plane), turns them with byte permutes into one 16-byte
-//     vector of channels per position and stores those into the zero-padded patch
-//     [position][64 bytes of channels] of the tile;
+//     one 16-byte chunk of channels, one 8- or 16-byte run of input positions per channel (16
+//     lanes cover 128 / 256 contiguous bytes of a channel plane), turns them with byte permutes
+//     into one 16-byte vector of channels per position and stores those into the zero-padded
+//     patch [position][64 bytes of channels] of the tile;
 //   * weights come packed as [K][T*9][C] (amos_conv_pack_weights: by the same call into the
 //     workspace, or once by their owner) and are copied into LDS as they are, 16 bytes a lane,
 //     without passing through registers; or, with no workspace, from the caller's KCTRS tensor:
@@ -156,7 +156,10 @@ constexpr int nchw_max_positions(int bj) { return nchw_patch_buffer_bytes(bj) / 
 
 // BI x BJ: output channels x output positions of a workgroup; WI x WJ: the grid of its
 // matrix-core waves; NWL: its loader waves; PTL: load groups of the patch per loader thread (the
-// loaders take 16 * NWL * PTL groups); WMODE: where the weights come from -- NCHW_W_KCTRS: the caller's tensor, per channel
+// loaders take 16 * NWL * PTL groups); LB: bytes of a patch load, i.e. of a load group's run of
+// positions in one channel -- 8, or 16 where a channel plane is a whole number of 16-byte runs and
+// the tensor is 16-byte aligned (half the load instructions, which are what bounds the loaders);
+// WMODE: where the weights come from -- NCHW_W_KCTRS: the caller's tensor, per channel
 // an unaligned run of nine taps; NCHW_W_KCRS: the same where a chunk of channels is one
 // contiguous, 16-byte aligned run (conv2d with aligned weights); NCHW_W_PACKED: [K][T*9][C],
 // written by amos_conv_pack_weights (into the workspace by the same call, or once by the owner of
@@ -169,7 +172,7 @@ constexpr int nchw_max_positions(int bj) { return nchw_patch_buffer_bytes(bj) / 
 // store the operands of macro step m + 1 (their loads two macro steps ahead of their use) while
 // the WI x WJ matrix-core waves do nothing but read fragments of macro step m and multiply; the
 // two kinds meet at the one barrier per macro step.
-template <int DT, int BI, int BJ, int WI, int WJ, int PTL, int WMODE, int NWL>
+template <int DT, int BI, int BJ, int WI, int WJ, int PTL, int WMODE, int NWL, int LB>
 __global__ __launch_bounds__(64 * (WI * WJ + NWL)) void amos_conv_nchw(const ConvNchwParams p) {
   typedef Mfma16<DT> MM;
   typedef typename MM::acc_t acc_t;
@@ -178,7 +181,8 @@ __global__ __launch_bounds__(64 * (WI * WJ + NWL)) void amos_conv_nchw(const Con
   constexpr int NWM = WI * WJ, NTM = 64 * NWM, NTL = 64 * NWL, NTA = NTM + NTL;
   constexpr int TI = BI / (16 * WI), TJ = BJ / (16 * WJ);
   static_assert(TI >= 1 && TJ >= 1 && TI * WI * 16 == BI && TJ * WJ * 16 == BJ, "wave tile");
-  constexpr int PG = 8 / ES;      // input positions per 8-byte load
+  static_assert(LB == 8 || LB == 16, "patch loads of 8 or 16 bytes");
+  constexpr int PG = LB / ES;     // input positions per patch load
   constexpr int CG = 16 / ES;     // channels per 16-byte chunk
   constexpr int CK = 64 / ES;     // channels per macro step
   constexpr int RS = 9;
@@ -256,11 +260,11 @@ __global__ __launch_bounds__(64 * (WI * WJ + NWL)) void amos_conv_nchw(const Con
       w_dst = (unsigned)nchw_position_offset(row, cq);
     }
     unsigned wraw[PACKED ? 1 : WRAW];
-    typedef unsigned nchw_u2 __attribute__((ext_vector_type(2)));
     // (two staging sets with packed weights: the patch loads run two macro steps ahead; one set
     // where the weights pass through registers too and every wait is for all loads anyway)
     constexpr int SETS = PACKED ? 2 : 1;
-    nchw_u2 praw[SETS][PTL][CG] = {};
+    typedef unsigned nchw_ul __attribute__((ext_vector_type(LB / 4)));
+    nchw_ul praw[SETS][PTL][CG] = {};
 
     // weights that pass through registers: the raw taps of this thread's unit
     auto load_weights = [&](int m) __attribute__((always_inline)) {
@@ -367,8 +371,11 @@ __global__ __launch_bounds__(64 * (WI * WJ + NWL)) void amos_conv_nchw(const Con
 #pragma unroll
         for (int ci = 0; ci < CG; ++ci) {
           const char* const plane = nchw_uniform(xm0 + (int64_t)ci * DHW * ES);
-          nchw_u2 x;
-          asm volatile("s_nop 4\n\tglobal_load_dwordx2 %0, %1, %2" : "=v"(x) : "v"(off), "s"(plane) : "memory");
+          nchw_ul x;
+          if constexpr (LB == 16)
+            asm volatile("s_nop 4\n\tglobal_load_dwordx4 %0, %1, %2" : "=v"(x) : "v"(off), "s"(plane) : "memory");
+          else
+            asm volatile("s_nop 4\n\tglobal_load_dwordx2 %0, %1, %2" : "=v"(x) : "v"(off), "s"(plane) : "memory");
           praw[SET][v][ci] = x;
         }
       }
@@ -382,7 +389,7 @@ __global__ __launch_bounds__(64 * (WI * WJ + NWL)) void amos_conv_nchw(const Con
       for (int v = 0; v < PTL; ++v)
 #pragma unroll
         for (int ci = 0; ci < CG; ++ci) {
-          nchw_u2 x = praw[SET][v][ci];
+          nchw_ul x = praw[SET][v][ci];
           asm volatile("" : "+v"(x));
           praw[SET][v][ci] = x;
         }

@@ -188,46 +188,56 @@ struct ConvNchwInstance {
   int bi, bj;
   int groups_per_thread;   // load groups of the patch a loader thread may own (x 4 chunks of channels)
   int loader_waves;
+  int load_bytes;          // bytes of a patch load (8, or 16: needs 16-byte aligned channel planes)
   std::once_flag once;
   int scratch_bytes = 0;   // per-lane scratch memory of the built kernel (register spills)
   int static_lds = 0;      // must stay 0: the kernel addresses dynamic LDS from byte 0
 };
 // wmode: NCHW_W_KCTRS (0), NCHW_W_KCRS (1), NCHW_W_PACKED (2)
-ConvNchwInstance* pick_conv_nchw_f16(int ti, int tj, int wmode, int pt, int nwl);
-ConvNchwInstance* pick_conv_nchw_bf16(int ti, int tj, int wmode, int pt, int nwl);
-ConvNchwInstance* pick_conv_nchw_i8(int ti, int tj, int wmode, int pt, int nwl);
+ConvNchwInstance* pick_conv_nchw_f16(int ti, int tj, int wmode, int pt, int nwl, int lb);
+ConvNchwInstance* pick_conv_nchw_bf16(int ti, int tj, int wmode, int pt, int nwl, int lb);
+ConvNchwInstance* pick_conv_nchw_i8(int ti, int tj, int wmode, int pt, int nwl, int lb);
 void launch_conv_pack_weights(int es, const void* w, void* out, int K, int C, int TRS, hipStream_t stream);
 
 #ifdef AMOS_CONV_NCHW_KERNEL_INCLUDED
-template <int DT, int BI, int BJ, int WI, int WJ, int PTL, int WMODE, int NWL>
+template <int DT, int BI, int BJ, int WI, int WJ, int PTL, int WMODE, int NWL, int LB>
 ConvNchwInstance* conv_nchw_instance() {
   static ConvNchwInstance inst;
   static const char* dtn[] = {"f16", "bf16", "i8"};
   static const char* wmn[] = {",kctrs", ",kcrs", ",packed"};
   static std::string name = std::string("amos_conv_nchw<") + dtn[DT] + "," + std::to_string(BI) + "x" +
                             std::to_string(BJ) + "," + std::to_string(WI * WJ) + "+" + std::to_string(NWL) + "w" +
-                            wmn[WMODE] + (PTL > 1 ? ",pt" + std::to_string(PTL) + ">" : std::string(">"));
-  inst.fn = amos_conv_nchw<DT, BI, BJ, WI, WJ, PTL, WMODE, NWL>;
+                            wmn[WMODE] + (LB == 16 ? ",ld16" : "") + (PTL > 1 ? ",pt" + std::to_string(PTL) + ">" : std::string(">"));
+  inst.fn = amos_conv_nchw<DT, BI, BJ, WI, WJ, PTL, WMODE, NWL, LB>;
   inst.name = name.c_str();
   inst.threads = 64 * (WI * WJ + NWL);
   inst.bi = BI;
   inst.bj = BJ;
   inst.groups_per_thread = PTL;
   inst.loader_waves = NWL;
+  inst.load_bytes = LB;
   return &inst;
 }
 // 64-row tiles: eight matrix-core waves, 32-row tiles: four; beside them nwl loader waves, which
 // take 16 * nwl load groups of the patch per round (pt = rounds)
-template <int DT, int WMODE, int PTL, int NWL>
+template <int DT, int WMODE, int PTL, int NWL, int LB = 8>
 ConvNchwInstance* pick_conv_nchw_p(int ti, int tj) {
-  if (ti == 64 && tj == 128) return conv_nchw_instance<DT, 64, 128, 2, 4, PTL, WMODE, NWL>();
-  if (ti == 64 && tj == 256) return conv_nchw_instance<DT, 64, 256, 1, 8, PTL, WMODE, NWL>();
-  if (ti == 32 && tj == 128) return conv_nchw_instance<DT, 32, 128, 1, 4, PTL, WMODE, NWL>();
-  if (ti == 32 && tj == 256) return conv_nchw_instance<DT, 32, 256, 1, 4, PTL, WMODE, NWL>();
+  if (ti == 64 && tj == 128) return conv_nchw_instance<DT, 64, 128, 2, 4, PTL, WMODE, NWL, LB>();
+  if (ti == 64 && tj == 256) return conv_nchw_instance<DT, 64, 256, 1, 8, PTL, WMODE, NWL, LB>();
+  if (ti == 32 && tj == 128) return conv_nchw_instance<DT, 32, 128, 1, 4, PTL, WMODE, NWL, LB>();
+  if (ti == 32 && tj == 256) return conv_nchw_instance<DT, 32, 256, 1, 4, PTL, WMODE, NWL, LB>();
   return nullptr;
 }
+// lb: bytes of a patch load; 16 only with packed weights and 16-bit types, one round
 template <int DT, int WMODE>
-ConvNchwInstance* pick_conv_nchw_t(int ti, int tj, int pt, int nwl) {
+ConvNchwInstance* pick_conv_nchw_t(int ti, int tj, int pt, int nwl, int lb) {
+  if (lb == 16) {
+    if constexpr (WMODE == NCHW_W_PACKED && DT != DT_I8) {
+      if (pt == 1 && nwl == 4) return pick_conv_nchw_p<DT, WMODE, 1, 4, 16>(ti, tj);
+      if (pt == 1 && nwl == 8) return pick_conv_nchw_p<DT, WMODE, 1, 8, 16>(ti, tj);
+    }
+    return nullptr;
+  }
   if (pt == 1 && nwl == 4) return pick_conv_nchw_p<DT, WMODE, 1, 4>(ti, tj);
   if constexpr (WMODE == NCHW_W_PACKED) {
     if (pt == 1 && nwl == 8) return pick_conv_nchw_p<DT, WMODE, 1, 8>(ti, tj);
@@ -238,10 +248,10 @@ ConvNchwInstance* pick_conv_nchw_t(int ti, int tj, int pt, int nwl) {
   return nullptr;
 }
 template <int DT>
-ConvNchwInstance* pick_conv_nchw_tile(int ti, int tj, int wmode, int pt, int nwl) {
-  return wmode == NCHW_W_PACKED ? pick_conv_nchw_t<DT, NCHW_W_PACKED>(ti, tj, pt, nwl)
-         : wmode == NCHW_W_KCRS ? pick_conv_nchw_t<DT, NCHW_W_KCRS>(ti, tj, pt, nwl)
-                                : pick_conv_nchw_t<DT, NCHW_W_KCTRS>(ti, tj, pt, nwl);
+ConvNchwInstance* pick_conv_nchw_tile(int ti, int tj, int wmode, int pt, int nwl, int lb) {
+  return wmode == NCHW_W_PACKED ? pick_conv_nchw_t<DT, NCHW_W_PACKED>(ti, tj, pt, nwl, lb)
+         : wmode == NCHW_W_KCRS ? pick_conv_nchw_t<DT, NCHW_W_KCRS>(ti, tj, pt, nwl, lb)
+                                : pick_conv_nchw_t<DT, NCHW_W_KCTRS>(ti, tj, pt, nwl, lb);
 }
 #endif
 

@@ -659,7 +659,11 @@ static double estimate_seconds(const Problem& pb, int ti, int tj, int split, boo
 }
 
 // patch_pitch 0: the smallest row pitch
-void conv_nchw_shape(const amos_conv_desc_t& c, int op, int patch_pitch, NchwShape* out) {
+int conv_nchw_load_bytes(const amos_conv_desc_t& c) {
+  return c.in_dtype != AMOS_I8 && (c.H * c.W * 2) % 16 == 0 ? 16 : 8;
+}
+
+void conv_nchw_shape(const amos_conv_desc_t& c, int op, int patch_pitch, NchwShape* out, int load_bytes) {
   NchwShape& s = *out;
   const bool two_d = op == AMOS_OP_CONV2D;
   s.N = (int)c.N; s.C = (int)c.C; s.D = two_d ? 1 : (int)c.D; s.H = (int)c.H; s.W = (int)c.W; s.K = (int)c.K;
@@ -676,14 +680,14 @@ void conv_nchw_shape(const amos_conv_desc_t& c, int op, int patch_pitch, NchwSha
   s.OQ = ext(s.W, s.pw, s.dw, s.S, s.sw);
   s.J = s.N * s.OD * s.OP * s.OQ;
   s.Wp = patch_pitch > 0 ? patch_pitch : nchw_patch_pitch(s.OQ, s.S, s.sw, s.dw, s.sh, 1);
-  s.pg_shift = c.in_dtype == AMOS_I8 ? 3 : 2;
+  s.pg_shift = (c.in_dtype == AMOS_I8 ? 3 : 2) + (load_bytes == 16 ? 1 : 0);
   s.div_opq = nchw_make_div((uint32_t)(s.OP * s.OQ));
   s.div_oq = nchw_make_div((uint32_t)s.OQ);
   s.div_w = nchw_make_div((uint32_t)s.W);
   s.div_od = nchw_make_div((uint32_t)s.OD);
 }
 
-ConvNchwPlan conv_nchw_plan(const amos_conv_desc_t& c, int op, int BI, int BJ) {
+ConvNchwPlan conv_nchw_plan(const amos_conv_desc_t& c, int op, int BI, int BJ, int load_bytes) {
   ConvNchwPlan r;
   memset(&r, 0, sizeof(r));
   const int es = c.in_dtype == AMOS_I8 ? 1 : 2;
@@ -692,12 +696,13 @@ ConvNchwPlan conv_nchw_plan(const amos_conv_desc_t& c, int op, int BI, int BJ) {
   if (c.groups > 1) { r.why = "grouped convolution"; return r; }
   if (c.R != 3 || c.S != 3) { r.why = "window not 3x3"; return r; }
   if ((c.C * es) % 64) { r.why = "channels do not fill whole 64-byte chunks"; return r; }
-  if ((c.H * c.W) % (8 / es)) { r.why = "a channel plane is not a whole number of 8-byte loads"; return r; }
+  if (load_bytes != 8 && (load_bytes != 16 || es != 2)) { r.why = "patch loads of 16 bytes are for 16-bit types"; return r; }
+  if ((c.H * c.W * es) % load_bytes) { r.why = "a channel plane is not a whole number of patch loads"; return r; }
   if ((BI != 64 && BI != 32) || (BJ != 128 && BJ != 256)) { r.why = "block tile not 32 or 64 by 128 or 256"; return r; }
   // (lanes address both tensors by 32-bit byte offsets)
   if (c.N * c.C * D * c.H * c.W * es >= ((int64_t)1 << 32) || c.K * c.C * T * 9 * es >= ((int64_t)1 << 32)) { r.why = "a tensor of 4 GiB or more"; return r; }
   NchwShape s;
-  conv_nchw_shape(c, op, 0, &s);
+  conv_nchw_shape(c, op, 0, &s, load_bytes);
   if (s.OD <= 0 || s.OP <= 0 || s.OQ <= 0) { r.why = "window larger than the padded input"; return r; }
   // nine weight tiles and a patch buffer of the tile's fixed size (its last 1 KB a dump line), both twice
   const int pbuf = BJ <= 128 ? 32 * 1024 : 40 * 1024;
@@ -791,7 +796,11 @@ static double conv_patch_estimate(const amos_conv_desc_t& c, int op, const Probl
 // Returns <= 0 where the kernel does not apply.
 double conv_nchw_estimate(const amos_conv_desc_t& c, int op, const Problem& pb, int ti, int tj) {
   if ((ti != 64 && ti != 32) || (tj != 128 && tj != 256)) return -1.0;
-  const ConvNchwPlan np = conv_nchw_plan(c, op, ti, tj);
+  // (as the launch plans it: patch loads of 16 bytes where the shape allows them and one round of
+  // the loaders covers the largest tile)
+  ConvNchwPlan np = conv_nchw_plan(c, op, ti, tj, conv_nchw_load_bytes(c));
+  if (conv_nchw_load_bytes(c) == 16 && (np.why || np.max_groups > 16 * nchw_loader_waves(true, np.max_groups)))
+    np = conv_nchw_plan(c, op, ti, tj, 8);
   if (np.why) return -1.0;
   const bool i8 = pb.in_dtype == AMOS_I8;
   const double es = i8 ? 1.0 : 2.0;

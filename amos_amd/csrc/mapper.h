@@ -151,11 +151,15 @@ struct ConvNchwPlan {
   int t1;               // conv2d: a chunk's weights are one contiguous run (needs 16-byte aligned weights)
   size_t lds;           // dynamic LDS bytes of a workgroup
 };
-ConvNchwPlan conv_nchw_plan(const amos_conv_desc_t& c, int op, int BI, int BJ);
+// load_bytes: bytes of a patch load, i.e. of a load group's run of positions in one channel (8 or 16)
+ConvNchwPlan conv_nchw_plan(const amos_conv_desc_t& c, int op, int BI, int BJ, int load_bytes = 8);
+// the widest patch load the shape allows (16 for 16-bit types whose channel planes are whole
+// 16-byte runs; the tensor itself must then be 16-byte aligned, which only the launch knows)
+int conv_nchw_load_bytes(const amos_conv_desc_t& c);
 // estimated seconds of a call that packs the weights into its workspace; <= 0 where the kernel does not apply
 double conv_nchw_estimate(const amos_conv_desc_t& c, int op, const Problem& pb, int ti, int tj);
 // the kernel's geometry descriptor of a convolution (extents, patch pitch, dividers)
 struct NchwShape;
-void conv_nchw_shape(const amos_conv_desc_t& c, int op, int patch_pitch, NchwShape* out);
+void conv_nchw_shape(const amos_conv_desc_t& c, int op, int patch_pitch, NchwShape* out, int load_bytes = 8);
 
 }  // namespace amos

@@ -159,6 +159,11 @@ int main() {
       {32, 256, 1, 14, 14, 256, 1, 3, 3, 1, 1, 1, 0, 1, 1, 1, 1, 1, 2, 128, 1},    // the smallest pitch: collisions at row wraps only
       {2, 64, 5, 56, 56, 64, 3, 3, 3, 1, 1, 1, 1, 1, 1, 1, 1, 1, 2, 256, 4},
       {2, 64, 5, 56, 56, 64, 3, 3, 3, 1, 1, 1, 1, 1, 1, 1, 1, 1, 2, 256, 16},
+      {2, 64, 5, 56, 56, 64, 3, 3, 3, 1, 1, 1, 1, 1, 1, 1, 1, 1, 3, 256, 8},      // 16-bit types with 16-byte loads: 8 positions
+      {2, 64, 5, 56, 56, 64, 3, 3, 3, 1, 1, 1, 1, 1, 1, 1, 1, 1, 3, 128, 8},
+      {3, 32, 1, 6, 12, 40, 1, 3, 3, 1, 1, 1, 0, 1, 1, 1, 1, 1, 3, 128, 8},       // ... groups that straddle image rows
+      {2, 32, 1, 10, 12, 40, 1, 3, 3, 1, 2, 2, 0, 1, 1, 1, 1, 1, 3, 128, 8},      // ... strides
+      {2, 32, 3, 6, 8, 40, 3, 3, 3, 2, 1, 2, 1, 1, 0, 1, 1, 1, 3, 128, 8},        // ... mixed strides, 3-d
   };
   for (const Case& c : cases) run(c);
   // weight tiles: a bijection; a fragment read (rows r .. r+7, chunks of lane groups q and q + 2) and

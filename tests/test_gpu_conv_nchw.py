@@ -184,6 +184,44 @@ def test_conv_nchw_weight_modes_agree(gpu, dtype, tile):
         _check(got if op == _lib.AMOS_OP_CONV3D else got[:, :, 0], ref, dtype, "weight modes %s %s" % (dtype, tile))
 
 
+@pytest.mark.parametrize("tile", TILES)
+def test_conv_nchw_load_widths_agree(gpu, tile):
+    """16-bit activations whose channel planes are whole 16-byte runs are fetched with 16-byte loads
+    where the tensor is 16-byte aligned and with 8-byte loads where it is not: same bits either
+    way (the accumulation order does not depend on it), 2-d with groups that straddle image rows,
+    and 3-d"""
+    import torch
+    from amos_amd import _lib, ops
+    ti, tj = tile
+    for xs, ws, st, pd in (((3, 64, 1, 6, 12), (72, 64, 1, 3, 3), (1, 1, 1), (0, 1, 1)),
+                           ((2, 64, 3, 10, 12), (40, 64, 3, 3, 3), (1, 1, 1), (1, 1, 1))):
+        op = _lib.AMOS_OP_CONV2D if xs[2] == 1 else _lib.AMOS_OP_CONV3D
+        rng = np.random.default_rng(ti + tj + xs[3])
+        x, w = make_operand(rng, xs, "float16"), make_operand(rng, ws, "float16")
+        dw = to_device(w, "float16")
+        n = int(np.prod(xs))
+        big = torch.zeros(n + 16, dtype=torch.float16, device="cuda")
+        assert big.data_ptr() % 16 == 0
+        outs = []
+        for shift in (8, 4):   # halves: 16 and 8 bytes past an aligned address
+            dx = big[shift:shift + n].view(xs)
+            dx.copy_(to_device(x, "float16"))
+            assert dx.data_ptr() % 16 == (0 if shift == 8 else 8)
+            print("load widths", tile, xs, "shift", shift, flush=True)
+            if op == _lib.AMOS_OP_CONV2D:
+                out = _run(ops.conv2d, dx[:, :, 0], dw[:, :, 0], st[1:], pd[1:], 1, config=_cfg(_lib, tj, ti))
+            else:
+                out = _run(ops.conv3d, dx, dw, st, pd, 1, config=_cfg(_lib, tj, ti))
+            outs.append(out)
+        assert torch.equal(outs[0], outs[1])
+        d = ops.conv_desc(xs, ws, torch.float16, st, pd, (1, 1, 1))
+        c = ops.make_config(_cfg(_lib, tj, ti))
+        assert "ld16" in ops.kernel_name(op, d, c)
+        ref = (co.lib_conv2d(x[:, :, 0], w[:, :, 0], "float16", st[1:], pd[1:], 1, acc="float64") if op == _lib.AMOS_OP_CONV2D
+               else co.lib_conv3d(x, w, "float16", st, pd, 1, acc="float64"))
+        _check(outs[0].cpu().numpy(), ref, "float16", "load widths %s %s" % (tile, xs))
+
+
 def test_conv_nchw_refusals(gpu):
     import torch
     from amos_amd import _lib, ops
