@@ -799,13 +799,21 @@ static int plan_conv(Plan& pl, int op, const amos_conv_desc_t* d, const amos_ker
     // Weights: already packed by the caller (AMOS_FLAG_WEIGHTS_PACKED), packed into the workspace by
     // this call, or -- without a workspace -- transposed by every workgroup on its way to LDS
     const size_t packed_bytes = (size_t)(c.K * c.C * (op == AMOS_OP_CONV2D ? 1 : c.T) * 9) * (pl.dt == DT_I8 ? 1 : 2);
+    // (a conv2d whose weights are 16-byte aligned can read them as they are: where the mapper's
+    // model says that this costs less than the packing launch, the workspace stays unused)
+    const bool t1_direct = op == AMOS_OP_CONV2D && aligned16(Wt);
+    bool prefer_unpacked = false;
+    if (t1_direct && !(cfg->reserved[0] & AMOS_FLAG_WEIGHTS_PACKED)) {
+      Problem pb;
+      if (problem_of(op, &c, &pb) == 0) conv_nchw_estimate(c, op, pb, BI, BJ, &prefer_unpacked);
+    }
     const bool will_pack = (cfg->reserved[0] & AMOS_FLAG_WEIGHTS_PACKED) ||
-                           (workspace && ws_bytes >= packed_bytes && ((uintptr_t)workspace & 255) == 0);
+                           (!prefer_unpacked && workspace && ws_bytes >= packed_bytes && ((uintptr_t)workspace & 255) == 0);
     // patch loads of 16 bytes where the shape and the tensor's address allow them, the weights are
     // packed and one round of the loaders covers the largest tile; else of 8
     int lb = 8;
     ConvNchwPlan np;
-    if (will_pack && conv_nchw_load_bytes(c) == 16 && aligned16(X)) {
+    if ((will_pack || t1_direct) && conv_nchw_load_bytes(c) == 16 && aligned16(X)) {
       np = conv_nchw_plan(c, op, BI, BJ, 16);
       if (!np.why && np.max_groups <= 16 * nchw_loader_waves(true, np.max_groups)) lb = 16;
     }
@@ -823,7 +831,7 @@ static int plan_conv(Plan& pl, int op, const amos_conv_desc_t* d, const amos_ker
     if (cfg->reserved[0] & AMOS_FLAG_WEIGHTS_PACKED) {
       if (!aligned16(Wt)) return set_error(AMOS_ERR_BAD_ARG, "packed weights must be 16-byte aligned");
       pl.nchw_wmode = NCHW_W_PACKED;
-    } else if (workspace && ws_bytes >= packed_bytes && ((uintptr_t)workspace & 255) == 0) {
+    } else if (will_pack) {
       pl.nchw_wmode = NCHW_W_PACKED;
       pl.nchw_pack = 1;
       q.w = (const char*)workspace;
@@ -844,14 +852,14 @@ static int plan_conv(Plan& pl, int op, const amos_conv_desc_t* d, const amos_ker
     q.div_cc = nchw_make_div((uint32_t)q.c_chunks);
     q.div_odpq = nchw_make_div((uint32_t)(OD * OP * OQ));
     pl.nchw = 1;
-    // rounds of the loader waves over the patch's load groups: one with packed weights, else two
-    // at most (int8, with sixteen channels per chunk and twice the staging registers per group: one)
+    // rounds of the loader waves over the patch's load groups: two at most; one for int8 (sixteen
+    // channels per chunk) and for 16-byte loads, which take twice the staging registers per group
     const bool packed = pl.nchw_wmode == NCHW_W_PACKED;
     pl.nchw_nwl = nchw_loader_waves(packed, np.max_groups);
     const int per_round = 16 * pl.nchw_nwl;
     pl.nchw_pt = std::max(1, (np.max_groups + per_round - 1) / per_round);
     pl.nchw_groups = np.max_groups;
-    if (pl.nchw_pt > (packed || pl.dt == DT_I8 ? 1 : 2))
+    if (pl.nchw_pt > (lb == 16 || pl.dt == DT_I8 ? 1 : 2))
       return set_error(AMOS_ERR_INFEASIBLE, "NCDHW-direct convolution not applicable: input patch of a tile above the threads' load budget");
     pl.nchw_lds = np.lds;
     memset(&pl.cfg, 0, sizeof(pl.cfg));
@@ -1178,23 +1186,29 @@ static int launch_conv_nchw(const Plan& pl, hipStream_t stream) {
     hipFuncAttributes fa;
     if (attr_err == hipSuccess) attr_err = hipFuncGetAttributes(&fa, (const void*)inst->fn);
     if (attr_err == hipSuccess) { inst->scratch_bytes = (int)fa.localSizeBytes; inst->static_lds = (int)fa.sharedSizeBytes; }
+    int blocks = 0;
+    if (attr_err == hipSuccess)
+      attr_err = hipOccupancyMaxActiveBlocksPerMultiprocessor(&blocks, (const void*)inst->fn, inst->threads, 0);
+    inst->fits = blocks >= 1;
   });
   if (attr_err != hipSuccess)
     return set_error(AMOS_ERR_HIP, "hipFuncSetAttribute(%s): %s", inst->name, hipGetErrorString(attr_err));
   if (inst->static_lds)   // the kernel addresses its dynamic LDS from byte 0
     return set_error(AMOS_ERR_HIP, "%s was built with %d bytes of static LDS", inst->name, inst->static_lds);
-  // (the loader waves decide that their loads have landed by counting vector-memory operations in
-  // flight; register spills are such operations too)
-  if (inst->scratch_bytes && pl.nchw_wmode == NCHW_W_PACKED)
-    return set_error(AMOS_ERR_INFEASIBLE, "%s was built with %d bytes of scratch memory per lane (register "
-                     "spills), which its wait counts do not allow for", inst->name, inst->scratch_bytes);
+  // (the loaders' staging registers are accumulation registers named in assembly: a build whose
+  // registers no longer leave room for a workgroup on a compute unit cannot be launched)
+  if (!inst->fits)
+    return set_error(AMOS_ERR_INFEASIBLE, "%s needs more registers than a workgroup of %d threads can have",
+                     inst->name, inst->threads);
   const ConvNchwParams& q = pl.nc;
   // what the kernel assumes of its launch: the tile of the instance, whole 64-byte chunks of
   // channels, a patch that fits the LDS asked for
+  // ... and at least one macro step for every block along the reduction
   if (inst->bi != pl.cfg.tile_i || inst->bj != pl.cfg.tile_j || q.c_chunks < 1 || q.max_pos < 4 ||
+      q.macro_per_split < 1 || pl.split < 1 || (int64_t)(pl.split - 1) * q.macro_per_split >= q.macro_steps ||
       q.max_pos > nchw_max_positions(inst->bj) ||
       pl.nchw_lds != (size_t)2 * 9 * inst->bi * 64 + (size_t)2 * nchw_patch_buffer_bytes(inst->bj) ||
-      inst->threads != inst->bi * 8 + 64 * pl.nchw_nwl || inst->loader_waves != pl.nchw_nwl ||
+      inst->threads != 64 * (inst->mma_waves + pl.nchw_nwl) || inst->loader_waves != pl.nchw_nwl ||
       inst->groups_per_thread != pl.nchw_pt || pl.nchw_pt * 16 * pl.nchw_nwl < pl.nchw_groups ||
       inst->load_bytes != pl.nchw_lb || (inst->load_bytes >> (pl.dt == DT_I8 ? 0 : 1)) != (1 << q.s.pg_shift) ||
       ((uintptr_t)q.x & (uintptr_t)(inst->load_bytes - 1)) ||

@@ -41,15 +41,12 @@ namespace amos {
 constexpr int kNchwMaxSeg = 4;
 constexpr int kNchwPosBytes = 64;   // bytes of channels per patch position and macro step
 
+// Loader waves of a workgroup (beside its matrix-core waves): they fetch and transpose the patch,
+// 16 load groups (x four chunks of channels) per wave and round.
+constexpr int nchw_loader_waves(bool packed, int groups) { return (void)packed, (void)groups, 4; }
+
 // n / d for 0 <= n < 2^31 by a multiplication with a host-built constant (the extents are known
 // when the kernel is launched; a hardware-less integer division costs dozens of instructions)
-// Loader waves of a workgroup (beside its matrix-core waves): they fetch and transpose the patch,
-// 16 load groups (x four chunks of channels) per wave and round.  Four of them; eight for a patch
-// of more than 64 load groups where the weights are packed (copied without registers: the kernel
-// then fits the 128 registers that 16 waves per CU leave each) -- one round of eight waves keeps
-// twice as many loads in flight as two rounds of four.
-constexpr int nchw_loader_waves(bool packed, int groups) { return packed && groups > 64 ? 8 : 4; }
-
 struct NchwDiv {
   uint32_t magic, shift, one, d;
 };

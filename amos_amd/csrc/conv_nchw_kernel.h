@@ -196,8 +196,6 @@ __global__ __launch_bounds__(64 * (WI * WJ + NWL)) void amos_conv_nchw(const Con
   static_assert(UNITS <= NTL, "one weight unit per loader thread at most");
   // packed weights: copied in 1 KB blocks (16 rows x 64 bytes); a tap's tile is NB of them
   constexpr int NB = BI / 16;
-  constexpr int NPL = PTL * CG;   // patch loads per thread and macro step
-  static_assert(2 * NPL <= 63, "the counter of loads in flight has six bits");
   // LDS, by byte offset from 0 (the kernel has no static LDS; the host checks that):
   //   [2][9][BI * 64] weight tiles | [2][PBUF] patches, the last 1 KB of each a dump line
   constexpr unsigned PBASE = 2 * WBUF;
@@ -236,14 +234,10 @@ __global__ __launch_bounds__(64 * (WI * WJ + NWL)) void amos_conv_nchw(const Con
 
   if (wave >= NWM) {
     // ==================================== loader waves ==============================================
-    // The loaders' memory instructions are all loads into registers: "at most N loads in flight"
-    // says which loads have landed only while loads complete in the order of their issue, and a
-    // direct copy into LDS and a load into registers do not keep that order between them
-    // (measured: with both in one wave a counted wait let through loads that were still on their
-    // way).  The direct copies of packed weights are therefore issued by the matrix-core waves.
+    // (The direct copies of packed weights are issued by the matrix-core waves: a direct copy into
+    // LDS costs the issuing wave the time LDS takes to accept it.)
     const int tl = t - NTM;
     constexpr int NTP = NTL;
-    const bool patch_wave = true;
     const int tlp = tl;
     // ---- this thread's share of the weights ----------------------------------------------------
     unsigned w_src[1] = {0};   // byte offset of (row, first channel of the chunk): below 4 GiB
@@ -260,11 +254,24 @@ __global__ __launch_bounds__(64 * (WI * WJ + NWL)) void amos_conv_nchw(const Con
       w_dst = (unsigned)nchw_position_offset(row, cq);
     }
     unsigned wraw[PACKED ? 1 : WRAW];
-    // (two staging sets with packed weights: the patch loads run two macro steps ahead; one set
-    // where the weights pass through registers too and every wait is for all loads anyway)
-    constexpr int SETS = PACKED ? 2 : 1;
-    typedef unsigned nchw_ul __attribute__((ext_vector_type(LB / 4)));
-    nchw_ul praw[SETS][PTL][CG] = {};
+    // The patch loads of a macro step are on their way for a whole macro step, across the loop's
+    // back edge.  The compiler takes the result of an assembly load for present as soon as the
+    // statement is behind it and is free to copy such a register to another one at any join of
+    // the control flow -- which copies what the register held before the data arrived.  So the
+    // loads land in the 32 highest registers a wave of this workgroup size can have (v136 .. v167
+    // with twelve waves on a compute unit, v224 .. v255 with eight), named in the assembly text
+    // and far above what the compiler needs for either kind of wave -- tests/test_conv_nchw_isa.py
+    // reads the compiled code of every instance and fails if anything outside these statements
+    // touches them -- and landed() moves them into ordinary registers behind the wait; the next
+    // loads go out right after that, before the transposes, so one set of registers keeps loads
+    // in flight all the time.
+    constexpr int LW = LB / 4;            // dwords of a load
+    constexpr int NAG = PTL * CG * LW;    // staging registers the loads of a macro step fill
+    static_assert(NAG <= 32, "staging registers");
+    constexpr int SBASE = NWM + NWL == 12 ? 136 : NWM + NWL == 8 ? 224 : -1;
+    static_assert(SBASE > 0, "workgroups of eight or twelve waves");
+    typedef unsigned nchw_ul __attribute__((ext_vector_type(LW)));
+    nchw_ul praw[PTL][CG];
 
     // weights that pass through registers: the raw taps of this thread's unit
     auto load_weights = [&](int m) __attribute__((always_inline)) {
@@ -316,9 +323,7 @@ __global__ __launch_bounds__(64 * (WI * WJ + NWL)) void amos_conv_nchw(const Con
       }
     };
     // the first weights go out before the tile's geometry is worked out
-    if (m_begin < m_end) {
-      if constexpr (!PACKED) load_weights(m_begin);
-    }
+    if constexpr (!PACKED) load_weights(m_begin);
 
     const NchwTile tile = nchw_tile(s, bj0, BJ);
     // ---- this thread's load groups of the patch ------------------------------------------------
@@ -330,7 +335,7 @@ __global__ __launch_bounds__(64 * (WI * WJ + NWL)) void amos_conv_nchw(const Con
     for (int v = 0; v < PTL; ++v) {
       const int q = tlp + NTP * v;
       const int cg = q & 3, grp = q >> 2;
-      const bool on = patch_wave && grp < tile.ngroups;
+      const bool on = grp < tile.ngroups;
       int f = 0;
       const NchwSeg seg = nchw_group(s, tile, on ? grp : 0, &f);
       p_src[v] = (unsigned)((((int64_t)seg.n * s.C + cg * CG) * DHW + f) * ES);
@@ -351,53 +356,55 @@ __global__ __launch_bounds__(64 * (WI * WJ + NWL)) void amos_conv_nchw(const Con
       const int pos = i ^ (lane >> 5);
       p_sel[i] = ES == 2 ? (pos ? 0x07060302u : 0x05040100u) : ((unsigned)pos | ((unsigned)(4 + pos) << 8));
     }
-    // the patch loads of macro step m into staging set SET.  Every lane loads, from a depth
-    // clamped into the tensor: a load that some lanes skip needs its registers preset, and the
-    // compiler waits for ALL loads in flight before it writes a register that an earlier load may
-    // still own; a depth in the padding is zeroed when the vector is stored, lanes without a
-    // group store into the dump line.  As assembly, and waited for by landed<N>(): the
-    // compiler's own bookkeeping of loads in flight around the loop ends in "wait for all of
-    // them" in front of the first use, which is the wait the second staging set is there to avoid.
-    auto load_patch = [&](auto set_c, int m) __attribute__((always_inline)) {
-      constexpr int SET = decltype(set_c)::value % SETS;
+    // the patch loads of macro step m.  Every lane loads, from a depth clamped into the tensor (a
+    // depth in the padding is zeroed when the vector is stored, lanes without a group store into
+    // the dump line).
+#define AMOS_NCHW_S136 "v136", "v137", "v138", "v139", "v140", "v141", "v142", "v143", "v144", "v145", "v146", "v147", "v148", "v149", "v150", "v151", \
+                       "v152", "v153", "v154", "v155", "v156", "v157", "v158", "v159", "v160", "v161", "v162", "v163", "v164", "v165", "v166", "v167"
+#define AMOS_NCHW_S224 "v224", "v225", "v226", "v227", "v228", "v229", "v230", "v231", "v232", "v233", "v234", "v235", "v236", "v237", "v238", "v239", \
+                       "v240", "v241", "v242", "v243", "v244", "v245", "v246", "v247", "v248", "v249", "v250", "v251", "v252", "v253", "v254", "v255"
+    auto load_patch = [&](int m) __attribute__((always_inline)) {
       const int tt = nchw_div(m, p.div_cc), cc = m - tt * p.c_chunks;
       const char* const xm0 = p.x + (int64_t)cc * CK * DHW * ES;
-#pragma unroll
-      for (int v = 0; v < PTL; ++v) {
+      nchw_static_for<0, PTL>([&](auto v_c) {
+        constexpr int v = decltype(v_c)::value;
         int d = p_d0[v] + tt * s.dd;
         d = d < 0 ? 0 : d >= s.D ? s.D - 1 : d;
         // (the depth is the lane's own: its offset stays below 4 GiB like the rest of the tensor)
-        const unsigned off = p_src[v] + (unsigned)d * (unsigned)(HW * ES);
-#pragma unroll
-        for (int ci = 0; ci < CG; ++ci) {
+        const unsigned off_v = p_src[v] + (unsigned)d * (unsigned)(HW * ES);
+        nchw_static_for<0, CG>([&](auto ci_c) {
+          constexpr int ci = decltype(ci_c)::value, r0 = SBASE + (v * CG + ci) * LW;
           const char* const plane = nchw_uniform(xm0 + (int64_t)ci * DHW * ES);
-          nchw_ul x;
-          if constexpr (LB == 16)
-            asm volatile("s_nop 4\n\tglobal_load_dwordx4 %0, %1, %2" : "=v"(x) : "v"(off), "s"(plane) : "memory");
+          const unsigned off = off_v;
+          // (five wait states between the v_readfirstlane that made the address and its use)
+          if constexpr (LB == 16 && SBASE == 136)
+            asm volatile("s_nop 4\n\tglobal_load_dwordx4 v[%2:%3], %0, %1" ::"v"(off), "s"(plane), "n"(r0), "n"(r0 + 3) : "memory", AMOS_NCHW_S136);
+          else if constexpr (LB == 16)
+            asm volatile("s_nop 4\n\tglobal_load_dwordx4 v[%2:%3], %0, %1" ::"v"(off), "s"(plane), "n"(r0), "n"(r0 + 3) : "memory", AMOS_NCHW_S224);
+          else if constexpr (SBASE == 136)
+            asm volatile("s_nop 4\n\tglobal_load_dwordx2 v[%2:%3], %0, %1" ::"v"(off), "s"(plane), "n"(r0), "n"(r0 + 1) : "memory", AMOS_NCHW_S136);
           else
-            asm volatile("s_nop 4\n\tglobal_load_dwordx2 %0, %1, %2" : "=v"(x) : "v"(off), "s"(plane) : "memory");
-          praw[SET][v][ci] = x;
-        }
-      }
+            asm volatile("s_nop 4\n\tglobal_load_dwordx2 v[%2:%3], %0, %1" ::"v"(off), "s"(plane), "n"(r0), "n"(r0 + 1) : "memory", AMOS_NCHW_S224);
+        });
+      });
     };
-    // at most N of this wave's loads are still in flight (they land in the order of their
-    // issue); staging set SET is read only behind this point
-    auto landed = [&](auto n_c, auto set_c) __attribute__((always_inline)) {
-      constexpr int SET = decltype(set_c)::value % SETS;
-      asm volatile("s_waitcnt vmcnt(%0)" ::"n"(decltype(n_c)::value) : "memory");
-#pragma unroll
-      for (int v = 0; v < PTL; ++v)
-#pragma unroll
-        for (int ci = 0; ci < CG; ++ci) {
-          nchw_ul x = praw[SET][v][ci];
-          asm volatile("" : "+v"(x));
-          praw[SET][v][ci] = x;
-        }
+    // every load of this wave has landed (the compiler's own loads of unpacked weights too); the
+    // patch loads move into ordinary registers
+    auto landed = [&]() __attribute__((always_inline)) {
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      nchw_static_for<0, PTL * CG>([&](auto u_c) {
+        constexpr int u = decltype(u_c)::value;
+        nchw_static_for<0, LW>([&](auto k_c) {
+          constexpr int k = decltype(k_c)::value;
+          unsigned x;
+          asm volatile("v_mov_b32 %0, v[%1]" : "=v"(x) : "n"(SBASE + u * LW + k));
+          praw[u / CG][u % CG][k] = x;
+        });
+      });
     };
-    // the patch of macro step m out of staging set SET into patch buffer BUF: per position one
+    // the patch of macro step m out of the registers into patch buffer BUF: per position one
     // 16-byte vector of channels
-    auto store_patch = [&](auto set_c, auto buf_c, int m) __attribute__((always_inline)) {
-      constexpr int SET = decltype(set_c)::value % SETS;
+    auto store_patch = [&](auto buf_c, int m) __attribute__((always_inline)) {
       const int tt = nchw_div(m, p.div_cc);
 #pragma unroll
       for (int v = 0; v < PTL; ++v) {
@@ -408,11 +415,11 @@ __global__ __launch_bounds__(64 * (WI * WJ + NWL)) void amos_conv_nchw(const Con
 #pragma unroll
           for (int j = 0; j < 4; ++j) {
             if constexpr (ES == 2) {
-              o[j] = (int)__builtin_amdgcn_perm(praw[SET][v][2 * j + 1][i >> 1], praw[SET][v][2 * j][i >> 1], p_sel[i & 1]);
+              o[j] = (int)__builtin_amdgcn_perm(praw[v][2 * j + 1][i >> 1], praw[v][2 * j][i >> 1], p_sel[i & 1]);
             } else {
               const unsigned sel = p_sel[i & 3];
-              const unsigned lo = __builtin_amdgcn_perm(praw[SET][v][4 * j + 1][i >> 2], praw[SET][v][4 * j][i >> 2], sel);
-              const unsigned hi = __builtin_amdgcn_perm(praw[SET][v][4 * j + 3][i >> 2], praw[SET][v][4 * j + 2][i >> 2], sel);
+              const unsigned lo = __builtin_amdgcn_perm(praw[v][4 * j + 1][i >> 2], praw[v][4 * j][i >> 2], sel);
+              const unsigned hi = __builtin_amdgcn_perm(praw[v][4 * j + 3][i >> 2], praw[v][4 * j + 2][i >> 2], sel);
               o[j] = (int)__builtin_amdgcn_perm(hi, lo, 0x05040100u);
             }
           }
@@ -423,53 +430,36 @@ __global__ __launch_bounds__(64 * (WI * WJ + NWL)) void amos_conv_nchw(const Con
     };
 
     // ---- prologue: macro step m_begin into the first buffers, the loads of the next one out ------
-    if (patch_wave) {
-      if (m_begin < m_end) load_patch(NchwSet<0>{}, m_begin);
-      if (PACKED && m_begin + 1 < m_end) load_patch(NchwSet<1>{}, m_begin + 1);
-    }
+    // (every blockIdx.y has at least one macro step: the host checks that)
+    load_patch(m_begin);
     clear_patches();
     meet();
-    if (m_begin < m_end) {
-      if (patch_wave) {
-        if (PACKED && m_begin + 1 < m_end) landed(NchwSet<NPL>{}, NchwSet<0>{});
-        else landed(NchwSet<0>{}, NchwSet<0>{});
-        store_patch(NchwSet<0>{}, NchwSet<0>{}, m_begin);
-        if (!PACKED && m_begin + 1 < m_end) load_patch(NchwSet<0>{}, m_begin + 1);
-      }
-      if constexpr (!PACKED) store_weights(NchwSet<0>{});
-    }
+    landed();
+    // (unpacked weights first: the compiler waits for its own loads in front of their first use, and
+    // that wait would take the patch loads behind it along)
+    if constexpr (!PACKED) store_weights(NchwSet<0>{});
+    if (m_begin + 1 < m_end) load_patch(m_begin + 1);
+    store_patch(NchwSet<0>{}, m_begin);
     meet();
     // ---- under macro step m of the matrix-core waves: macro step m + 1 into the other buffers
-    // (last read a macro step ago), the patch out of staging set SET while the loads of m + 2 fill
-    // the other set
-    auto under = [&](auto set_c, auto buf_c, int m) __attribute__((always_inline)) {
-      constexpr int SET = decltype(set_c)::value;
-      const bool next = m + 1 < m_end, more = m + 2 < m_end;
-      if constexpr (PACKED) {
-        if (more) load_patch(NchwSet<SET ^ 1>{}, m + 2);
-        if (next) {
-          if (more) landed(NchwSet<NPL>{}, set_c);
-          else landed(NchwSet<0>{}, set_c);
-          store_patch(set_c, buf_c, m + 1);
-        }
-      } else {
-        // (the compiler's loads of the weights and the patch loads share the wave: wait for all)
-        if (next) load_weights(m + 1);
-        if (patch_wave && next) {
-          landed(NchwSet<0>{}, set_c);
-          store_patch(set_c, buf_c, m + 1);
-        }
-        if (patch_wave && more) load_patch(NchwSet<SET ^ 1>{}, m + 2);
-        if (next) store_weights(buf_c);
+    // (last read a macro step ago) while the loads of m + 2 are on their way
+    auto under = [&](auto buf_c, int m) __attribute__((always_inline)) {
+      if (m + 1 < m_end) {
+        if constexpr (!PACKED) load_weights(m + 1);
+        landed();
+        if constexpr (!PACKED) store_weights(buf_c);
+        if (m + 2 < m_end) load_patch(m + 2);
+        store_patch(buf_c, m + 1);
       }
       meet();
     };
     // macro step m_begin + r is computed from buffers r & 1; the loaders fill buffers (r + 1) & 1
-    // from staging set (r + 1) & 1
     for (int m = m_begin; m < m_end; m += 2) {
-      under(NchwSet<1>{}, NchwSet<1>{}, m);
-      if (m + 1 < m_end) under(NchwSet<0>{}, NchwSet<0>{}, m + 1);
+      under(NchwSet<1>{}, m);
+      if (m + 1 < m_end) under(NchwSet<0>{}, m + 1);
     }
+#undef AMOS_NCHW_S136
+#undef AMOS_NCHW_S224
     return;
   }
 
@@ -485,8 +475,9 @@ __global__ __launch_bounds__(64 * (WI * WJ + NWL)) void amos_conv_nchw(const Con
   //   a v_readfirstlane that may have produced the address registers and the memory instruction
   //   that reads them, one between the write of M0 and the copy that takes its LDS address from
   //   there; without them the copy can run with stale registers.
-  static_assert(NWM == 2 * NB, "two taps per round of the matrix-core waves' copies");
-  constexpr int NWC = (RS + 1) / 2;
+  static_assert(NWM % NB == 0, "a wave copies the same block of rows of every tap it takes");
+  constexpr int TPR = NWM / NB;               // taps per round of the matrix-core waves' copies
+  constexpr int NWC = (RS + TPR - 1) / TPR;
   const int wblock = wave % NB, wtap0 = wave / NB;
   unsigned w_lane = 0;
   if (PACKED) {
@@ -502,7 +493,7 @@ __global__ __launch_bounds__(64 * (WI * WJ + NWL)) void amos_conv_nchw(const Con
     const unsigned lane_off = w_lane;
 #pragma unroll
     for (int i = 0; i < NWC; ++i) {
-      const int tap = wtap0 + 2 * i;
+      const int tap = wtap0 + TPR * i;
       if (tap < RS) {
         const char* const src = nchw_uniform(wm + (int64_t)tap * s.C * ES);
         const unsigned dst = decltype(buf_c)::value * WBUF + tap * WTILE + wblock * 1024;
@@ -512,7 +503,7 @@ __global__ __launch_bounds__(64 * (WI * WJ + NWL)) void amos_conv_nchw(const Con
     }
   };
   // the first weights go out before anything else
-  if (PACKED && m_begin < m_end) copy_weights(NchwSet<0>{}, m_begin);
+  if (PACKED) copy_weights(NchwSet<0>{}, m_begin);
   const int wi = wave / WJ, wj = wave % WJ;
   const int frag_row = lane & 15, frag_q = lane >> 4;
   const NchwTile tile = nchw_tile(s, bj0, BJ);

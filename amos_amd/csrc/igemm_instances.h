@@ -188,9 +188,11 @@ struct ConvNchwInstance {
   int bi, bj;
   int groups_per_thread;   // load groups of the patch a loader thread may own (x 4 chunks of channels)
   int loader_waves;
+  int mma_waves;
   int load_bytes;          // bytes of a patch load (8, or 16: needs 16-byte aligned channel planes)
   std::once_flag once;
   int scratch_bytes = 0;   // per-lane scratch memory of the built kernel (register spills)
+  bool fits = true;        // a workgroup of `threads` fits a compute unit's registers
   int static_lds = 0;      // must stay 0: the kernel addresses dynamic LDS from byte 0
 };
 // wmode: NCHW_W_KCTRS (0), NCHW_W_KCRS (1), NCHW_W_PACKED (2)
@@ -215,6 +217,7 @@ ConvNchwInstance* conv_nchw_instance() {
   inst.bj = BJ;
   inst.groups_per_thread = PTL;
   inst.loader_waves = NWL;
+  inst.mma_waves = WI * WJ;
   inst.load_bytes = LB;
   return &inst;
 }
@@ -228,22 +231,22 @@ ConvNchwInstance* pick_conv_nchw_p(int ti, int tj) {
   if (ti == 32 && tj == 256) return conv_nchw_instance<DT, 32, 256, 1, 4, PTL, WMODE, NWL, LB>();
   return nullptr;
 }
-// lb: bytes of a patch load; 16 only with packed weights and 16-bit types, one round
+// lb: bytes of a patch load; 16 only for 16-bit types, one round, and not with weights whose taps
+// are unaligned runs (3-d without packing).  The staging
+// registers of a loader thread are pt * (16 channels' worth of loads): int8 (sixteen channels per
+// chunk) and 16-byte loads take one round only.
 template <int DT, int WMODE>
 ConvNchwInstance* pick_conv_nchw_t(int ti, int tj, int pt, int nwl, int lb) {
+  if (nwl != 4) return nullptr;
   if (lb == 16) {
-    if constexpr (WMODE == NCHW_W_PACKED && DT != DT_I8) {
-      if (pt == 1 && nwl == 4) return pick_conv_nchw_p<DT, WMODE, 1, 4, 16>(ti, tj);
-      if (pt == 1 && nwl == 8) return pick_conv_nchw_p<DT, WMODE, 1, 8, 16>(ti, tj);
+    if constexpr (WMODE != NCHW_W_KCTRS && DT != DT_I8) {
+      if (pt == 1) return pick_conv_nchw_p<DT, WMODE, 1, 4, 16>(ti, tj);
     }
     return nullptr;
   }
-  if (pt == 1 && nwl == 4) return pick_conv_nchw_p<DT, WMODE, 1, 4>(ti, tj);
-  if constexpr (WMODE == NCHW_W_PACKED) {
-    if (pt == 1 && nwl == 8) return pick_conv_nchw_p<DT, WMODE, 1, 8>(ti, tj);
-  } else if constexpr (DT != DT_I8) {
-    // (int8: sixteen channels per chunk, twice the staging registers of a load group: one round only)
-    if (pt == 2 && nwl == 4) return pick_conv_nchw_p<DT, WMODE, 2, 4>(ti, tj);
+  if (pt == 1) return pick_conv_nchw_p<DT, WMODE, 1, 4>(ti, tj);
+  if constexpr (DT != DT_I8) {
+    if (pt == 2) return pick_conv_nchw_p<DT, WMODE, 2, 4>(ti, tj);
   }
   return nullptr;
 }

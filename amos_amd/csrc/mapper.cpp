@@ -794,30 +794,46 @@ static double conv_patch_estimate(const amos_conv_desc_t& c, int op, const Probl
 // of latency that their two-step lookahead does not cover, plus ~45 per load instruction of a
 // wave, measured on 14x14 and 56x56 planes; int8 loads twice the channels per group).
 // Returns <= 0 where the kernel does not apply.
-double conv_nchw_estimate(const amos_conv_desc_t& c, int op, const Problem& pb, int ti, int tj) {
+double conv_nchw_estimate(const amos_conv_desc_t& c, int op, const Problem& pb, int ti, int tj, bool* unpacked) {
+  if (unpacked) *unpacked = false;
   if ((ti != 64 && ti != 32) || (tj != 128 && tj != 256)) return -1.0;
   // (as the launch plans it: patch loads of 16 bytes where the shape allows them and one round of
   // the loaders covers the largest tile)
-  ConvNchwPlan np = conv_nchw_plan(c, op, ti, tj, conv_nchw_load_bytes(c));
-  if (conv_nchw_load_bytes(c) == 16 && (np.why || np.max_groups > 16 * nchw_loader_waves(true, np.max_groups)))
+  int s_lb = conv_nchw_load_bytes(c);
+  ConvNchwPlan np = conv_nchw_plan(c, op, ti, tj, s_lb);
+  if (s_lb == 16 && (np.why || np.max_groups > 16 * nchw_loader_waves(true, np.max_groups))) {
+    s_lb = 8;
     np = conv_nchw_plan(c, op, ti, tj, 8);
+  }
   if (np.why) return -1.0;
   const bool i8 = pb.in_dtype == AMOS_I8;
   const double es = i8 ? 1.0 : 2.0;
   const int nwl = nchw_loader_waves(true, np.max_groups);
-  if (np.max_groups > 16 * nwl) return -1.0;
+  if (np.max_groups > 16 * nwl * (i8 || s_lb == 16 ? 1 : 2)) return -1.0;
   const int64_t T = op == AMOS_OP_CONV2D ? 1 : c.T;
   const double macro_steps = (double)T * (c.C * es / 64.0);
   const double tiles = std::ceil((double)pb.I / ti) * std::ceil((double)pb.J / tj);
   const double rounds = std::ceil(tiles / device_compute_units());
   const double flop_per_cycle = (i8 ? 2.0 : 1.0) * 3850.0 * (ti * tj >= 64 * 256 ? 0.85 : ti * tj >= 64 * 128 ? 0.72 : 0.6);
   const double mma = 2.0 * ti * tj * 9.0 * (64.0 / es) / flop_per_cycle;
-  const double load_instr = std::ceil(np.max_groups * 4.0 / 64.0) * (16.0 / es) * (i8 ? 2.0 : 1.0);
-  const double loaders = 1800.0 + 45.0 * load_instr;
-  const double prologue = 7000.0 + 40.0 * load_instr;
+  // the loaders of a macro step: a fixed part, the bytes they move and their load instructions
+  // (fitted: 64x128 tile, 24 instructions of 8 bytes a lane 2400 cycles, of 16 bytes 3500; 64x256,
+  // 32 of 16 bytes 4600)
+  const double load_instr = std::ceil(np.max_groups * 4.0 / 64.0) * (16.0 / es);
+  const double loaders = 1300.0 + 5.0 * load_instr * s_lb + 20.0 * load_instr;
+  const double prologue = 9000.0 + 40.0 * load_instr;
   const double cycles = rounds * (prologue + macro_steps * std::max(mma, loaders));
+  const double kernel = cycles / 2.4e9 + 2.5e-6;
+  // the weights: packed by a launch in front of the kernel (its cost is the dependent launch more
+  // than the copy), or -- conv2d, where a chunk's taps are one aligned run -- transposed by the
+  // loaders of every tile, some 600 cycles more per macro step
   const double pack = (double)(c.K * c.C * T * 9) * es * 2.0 / 2.5e12 + 3.5e-6;
-  return cycles / 2.4e9 + 2.5e-6 + pack;
+  const double in_kernel = rounds * macro_steps * 600.0 / 2.4e9;
+  if (op == AMOS_OP_CONV2D && in_kernel < pack) {
+    if (unpacked) *unpacked = true;
+    return kernel + in_kernel;
+  }
+  return kernel + pack;
 }
 
 }  // namespace amos

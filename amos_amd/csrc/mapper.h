@@ -156,8 +156,10 @@ ConvNchwPlan conv_nchw_plan(const amos_conv_desc_t& c, int op, int BI, int BJ, i
 // the widest patch load the shape allows (16 for 16-bit types whose channel planes are whole
 // 16-byte runs; the tensor itself must then be 16-byte aligned, which only the launch knows)
 int conv_nchw_load_bytes(const amos_conv_desc_t& c);
-// estimated seconds of a call that packs the weights into its workspace; <= 0 where the kernel does not apply
-double conv_nchw_estimate(const amos_conv_desc_t& c, int op, const Problem& pb, int ti, int tj);
+// estimated seconds of a call that brings a workspace for packed weights; <= 0 where the kernel
+// does not apply.  *unpacked: the call is better off reading the weights as they are (conv2d with
+// 16-byte aligned weights) than packing them first
+double conv_nchw_estimate(const amos_conv_desc_t& c, int op, const Problem& pb, int ti, int tj, bool* unpacked = nullptr);
 // the kernel's geometry descriptor of a convolution (extents, patch pitch, dividers)
 struct NchwShape;
 void conv_nchw_shape(const amos_conv_desc_t& c, int op, int patch_pitch, NchwShape* out, int load_bytes = 8);
