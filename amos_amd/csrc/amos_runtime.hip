@@ -789,6 +789,7 @@ static int plan_conv(Plan& pl, int op, const amos_conv_desc_t* d, const amos_ker
   amos_kernel_config_t nchw_default;
   if ((!cfg || (cfg->pipeline == AMOS_PIPE_AUTO && (cfg->tile_i <= 0 || cfg->tile_j <= 0) && cfg->split_k <= 1)) &&
       workspace && ((uintptr_t)workspace & 255) == 0 && ws_bytes >= amos_conv_packed_weights_bytes(op, &c) &&
+      ((uintptr_t)X & 7) == 0 &&   // (its 8-byte loads of the activations; other kernels take any address)
       amos_default_config(op, &c, &nchw_default) == 0 && nchw_default.pipeline == AMOS_PIPE_NCHW) {
     if (cfg) nchw_default.reserved[0] = cfg->reserved[0];
     cfg = &nchw_default;

@@ -678,6 +678,27 @@ def test_conv_defaults_when_applicable(gpu):
     assert ops.kernel_name(_lib.AMOS_OP_CONV2D, d).startswith("amos_igemm<f16,")
 
 
+def test_conv_default_with_odd_addresses(gpu):
+    """tensors that start 2 bytes past an aligned address (views into larger buffers): the default
+    config must pick a kernel that takes them, not the one whose loads want 8-byte alignment"""
+    import torch
+    from amos_amd import ops
+    rng = np.random.default_rng(5)
+    xs, ws = (4, 64, 14, 14), (64, 64, 3, 3)
+    x, w = make_operand(rng, xs, "float16"), make_operand(rng, ws, "float16")
+    ref = co.lib_conv2d(x, w, "float16", 1, 1, 1, acc="float64")
+    bx = torch.zeros(x.size + 8, dtype=torch.float16, device="cuda")
+    bw = torch.zeros(w.size + 8, dtype=torch.float16, device="cuda")
+    for sx, sw in ((1, 0), (0, 1), (1, 1), (4, 4)):
+        dx = bx[sx:sx + x.size].view(xs)
+        dw = bw[sw:sw + w.size].view(ws)
+        dx.copy_(to_device(x, "float16"))
+        dw.copy_(to_device(w, "float16"))
+        print("odd addresses", sx, sw, flush=True)
+        got = ops.conv2d(dx, dw, 1, 1, 1).cpu().numpy()
+        check_float(got, ref, "default conv2d, x + %d B, w + %d B" % (2 * sx, 2 * sw))
+
+
 def test_conv2d_config3(gpu):
     """fp16 conv2d N32 C256 14x14 K256 3x3 s1 p1; X ~ U[0,1], W ~ N(0, 0.05)"""
     from amos_amd import ops
