@@ -127,14 +127,102 @@ def get_schedule(sch_app, params):
     return sch, args
 
 
+class _TrialShares:
+    """How one matching's trial budget is divided between its mappings: a softmax over each
+    mapping's best value, moved towards with momentum between rounds (the rule of
+    auto_tensorize.py:784-811 and :1018-1035).  Mappings no kernel can run hold a share of 0."""
+    MOMENTUM = 0.8
+
+    def __init__(self, count):
+        self.shares = [1.0 / count] * count
+        self.velocity = [0.0] * count
+
+    def restrict(self, allowed):
+        """shares only for the mappings flagged in `allowed` (unless none is)"""
+        if any(allowed):
+            kept = [w if ok else 0.0 for w, ok in zip(self.shares, allowed)]
+            total = sum(kept)
+            self.shares = [w / total for w in kept]
+
+    def trials(self, budget):
+        return [math.ceil(budget * w) for w in self.shares]
+
+    def update(self, values):
+        """one round's best values (1 / MAX_FLOAT = did not run) -> new shares"""
+        ran = [v > 1 / MAX_FLOAT for v in values]
+        top = max(values)
+        target = _normalised([math.exp(min(0.0, v - top)) for v in values])
+        self.velocity = [t - w + self.MOMENTUM * u for t, w, u in zip(target, self.shares, self.velocity)]
+        moved = [w + u for w, u in zip(self.shares, self.velocity)]
+        self.shares = _normalised([math.exp(x) if ok or not any(ran) else 0.0 for x, ok in zip(moved, ran)])
+
+
+def _normalised(xs):
+    total = sum(xs)
+    return [x / total for x in xs]
+
+
+class _MappingRun:
+    """the kernel-configuration sweep of one mapping: generator, applier, first pipeline"""
+
+    def __init__(self, schedule_gen, schedule_app, pipeline):
+        self.schedule_gen, self.schedule_app, self.pipeline = schedule_gen, schedule_app, pipeline
+
+
+class _MatchingSweep:
+    """one matching of auto_tensorize_v4: its feasible mappings, their trial shares, and which
+    of them a kernel family can run"""
+
+    def __init__(self, match_result, transform_strict, transform_dump, drop_output):
+        self.match_result = match_result
+        self.drop_output = drop_output
+        probe = MappingApplier(match_result, strict=transform_strict)
+        self.mappings = []
+        for mapping in MappingGenerator(match_result).get_all():
+            try:
+                probe.apply(mapping, drop_output=drop_output)
+                self.mappings.append(mapping)
+            except RuntimeError:
+                print("Catch an infeasible mapping:", flush=True)
+                print(mapping, flush=True)
+        self.applier = MappingApplier(match_result, verbose=transform_dump, strict=transform_strict)
+        self.shares = _TrialShares(len(self.mappings)) if self.mappings else None
+        # the mappings the kernel families implement as they are: bit vector -> pipeline
+        self.realised = {}
+        for pipe in (_lib.AMOS_PIPE_PATCH, _lib.AMOS_PIPE_STAGED):
+            self.realised.setdefault(tuple(mapping_of_pipeline(match_result, pipe)), pipe)
+
+    def how(self, record):
+        return _realisation(self.match_result, record, self.realised)
+
+    def announce(self, budget):
+        print("Original weights", self.shares.shares, flush=True)
+        print("Original trials for each mapping", self.shares.trials(budget), flush=True)
+        print("Current explored matching:", str(self.match_result), flush=True)
+        print("Its axis mapping:", flush=True)
+        for i, v in self.match_result.axis_map.items():
+            print(i.var, ":", [x.var for x in v], flush=True)
+
+    def keep_runnable(self):
+        """first round: trials only for mappings that can run; returns how many can"""
+        runnable = [self.how(r) is not None for r in self.mappings]
+        print("Num runnable mapping:", sum(runnable), flush=True)
+        if any(runnable):
+            self.shares.restrict(runnable)
+            print("Weights of the runnable mappings", self.shares.shares, flush=True)
+        return sum(runnable)
+
+
 def auto_tensorize_v4(target_dag, target, schedule_log_file, measure_opt, schedule_log_dir="schedules",
                       trials=200, repeat_rounds=10, builder=None, runner=None, verbose_schedule=False,
                       transform_dump=False, transform_strict=True, search_group_size=5,
                       desired_compute_key=None, desired_shape_key=None, enable_split_K=False,
                       use_shared_store=False, drop_output=False, build_parallel=1, run_parallel=1,
                       explore_full_match=False, enable_perf_model=False, perf_percentage=0.5):
-    """explore every feasible mapping, re-weighting the trial budget between rounds by a
-    softmax with momentum over each mapping's best value (auto_tensorize.py:784-811,1018-1035)"""
+    """Explores every feasible mapping of the chosen matching(s): per round each mapping gets its
+    share of the trials (`_TrialShares`) for the kernel-configuration sweep of the kernel family
+    that can run it.  Signature and console protocol of the reference's auto_tensorize_v4
+    (python/tvm/auto_tensorize/auto_tensorize.py:661-1053)."""
     measure_opt.target = target
     _check_target(target)
     match_results = get_match_results(target_dag, target)
@@ -144,169 +232,116 @@ def auto_tensorize_v4(target_dag, target, schedule_log_file, measure_opt, schedu
     print("Possible matchings:", flush=True)
     for i, m in enumerate(match_results):
         print(i, ":", str(m), flush=True)
-    if desired_compute_key is not None:
-        match_results = [m for m in match_results if m.compute_key == desired_compute_key]
+    for wanted, attr, what in ((desired_compute_key, "compute_key", "compute"), (desired_shape_key, "shape_key", "shape")):
+        if wanted is None:
+            continue
+        match_results = [m for m in match_results if getattr(m, attr) == wanted]
         if not match_results:
-            print("No match result matches desired compute key:", desired_compute_key, flush=True)
-            return AutoTensorizeResult()
-    if desired_shape_key is not None:
-        match_results = [m for m in match_results if m.shape_key == desired_shape_key]
-        if not match_results:
-            print("No match result matches desired shape key:", desired_shape_key, flush=True)
+            print("No match result matches desired %s key:" % what, wanted, flush=True)
             return AutoTensorizeResult()
     if not explore_full_match:
-        match_result, _ = all_fit(match_results)
-        match_results = [match_result]
+        match_results = [all_fit(match_results)[0]]
 
-    all_matches, all_mappings, appliers, mapping_weights, weights_updates = [], [], [], [], []
-    momentum = 0.8
-    total_mappings = 0
-    for match_result in match_results:
-        mappings = MappingGenerator(match_result).get_all()
-        feasible = []
-        tmp_app = MappingApplier(match_result, strict=transform_strict)
-        for mapping in mappings:
-            try:
-                tmp_app.apply(mapping, drop_output=drop_output)
-                feasible.append(mapping)
-            except RuntimeError:
-                print("Catch an infeasible mapping:", flush=True)
-                print(mapping, flush=True)
-        if not feasible:
-            continue
-        all_matches.append(match_result)
-        all_mappings.append(feasible)
-        total_mappings += len(feasible)
-        mapping_weights.append([1.0 / len(feasible) for _ in feasible])
-        weights_updates.append([0.0 for _ in feasible])
-        appliers.append(MappingApplier(match_result, verbose=transform_dump, strict=transform_strict))
-    total_matchings = len(all_matches)
+    sweeps = [sw for sw in (_MatchingSweep(m, transform_strict, transform_dump, drop_output) for m in match_results)
+              if sw.mappings]
+    total_mappings = sum(len(sw.mappings) for sw in sweeps)
     if total_mappings == 0:
         print("Can't find any mappings!", flush=True)
         return AutoTensorizeResult()
 
-    pure_test = False
-    if trials == 0:
-        pure_test = True
+    pure_test = trials == 0
+    if pure_test:
         repeat_rounds = 1
         print("Pure testing mode...", flush=True)
     elif trials < total_mappings * repeat_rounds * search_group_size:
-        need = total_mappings * repeat_rounds * search_group_size
-        print(f"[Warning] Too few trials, expect at least {need} trials.", flush=True)
-        trials = need
-        print(f"Increase trials to {need}.", flush=True)
+        trials = total_mappings * repeat_rounds * search_group_size
+        print(f"[Warning] Too few trials, expect at least {trials} trials.", flush=True)
+        print(f"Increase trials to {trials}.", flush=True)
     else:
         print("Total trials:", trials, flush=True)
-    trials_per_matching = trials // repeat_rounds // total_matchings
+    budget = trials // repeat_rounds // len(sweeps)
     print("Num rounds:", repeat_rounds, flush=True)
-    print("Num matching:", total_matchings, flush=True)
+    print("Num matching:", len(sweeps), flush=True)
     print("Num mapping:", total_mappings, flush=True)
-    print("Initial trials per matching:", trials_per_matching, flush=True)
-    if not (os.path.exists(schedule_log_dir) and os.path.isdir(schedule_log_dir)):
+    print("Initial trials per matching:", budget, flush=True)
+    if not os.path.isdir(schedule_log_dir):
         os.mkdir(schedule_log_dir)
 
-    class ScheduleContext:
-        def __init__(self, schedule_gen, schedule_app, pipeline):
-            self.schedule_gen, self.schedule_app, self.pipeline = schedule_gen, schedule_app, pipeline
-
-    cache = {}
+    runs = {}            # mapping key -> _MappingRun (None: no kernel for the compute)
     runnable_total = 0
-    best_value, best_ctx, best_params, best_mapping = 1 / MAX_FLOAT, None, None, None
+    best = {"value": 1 / MAX_FLOAT, "run": None, "params": None, "mapping": None}
     checker = MI355XProgramChecker(verbose_init=False)
-    beg = time.time()
+    started = time.time()
+
+    def run_of(sweep, record, pipes, rows):
+        key = record.as_key()
+        if key not in runs:
+            log = os.path.join(schedule_log_dir, "mapping_" + str(key) + "_" + schedule_log_file)
+            try:
+                gen = MI355XScheduleGenerator(sweep.match_result, sweep.applier.apply(record, drop_output=drop_output),
+                                              log_file=log, rows=rows,
+                                              perf_percentage=perf_percentage if enable_perf_model else 1.0)
+            except NoKernelError as e:
+                print("No kernel for this compute:", e, flush=True)
+                runs[key] = None
+                return None
+            if os.path.exists(log) and os.path.getsize(log) > 0:
+                gen.load_from_file(log)
+            gen._candidates = gen.candidates(pipes)
+            runs[key] = _MappingRun(gen, MI355XScheduleApplier(sweep.match_result, gen.lowered), pipes[0])
+        return runs[key]
+
+    def explore(sweep, record, n_trials):
+        """the sweep of one mapping for this round -> (its best value so far, the parameters)"""
+        how = sweep.how(record)
+        if how is None:
+            print("No kernel instance realises this mapping; skipped.", flush=True)
+            return 1 / MAX_FLOAT, None
+        run = run_of(sweep, record, *how)
+        if run is None:
+            return 1 / MAX_FLOAT, None
+        gen = run.schedule_gen
+        if n_trials and not pure_test:
+            find_optimized_parameters(sweep.match_result, gen, run.schedule_app, measure_opt, checker, n_trials,
+                                      verbose=verbose_schedule)
+        value, params = 1 / MAX_FLOAT, None
+        if gen.has_entry():
+            entry = gen.get_best_entry()
+            params, value = entry.record, entry.value
+        elif pure_test and gen.candidates():
+            params = gen.candidates()[0]
+            value = 1.0 / gen.estimate(params)
+        if value > best["value"]:
+            best.update(value=value, run=run, params=params, mapping=record)
+        return value, params
+
     for rnd in range(repeat_rounds):
-        for match_id in range(total_matchings):
-            match_result, app = all_matches[match_id], appliers[match_id]
-            weights, updates = mapping_weights[match_id], weights_updates[match_id]
-            tune_trials = [math.ceil(trials_per_matching * x) for x in weights]
-            best_values = []
-            print("Original weights", weights, flush=True)
-            print("Original trials for each mapping", tune_trials, flush=True)
-            print("Current explored matching:", str(match_result), flush=True)
-            print("Its axis mapping:", flush=True)
-            for i, v in match_result.axis_map.items():
-                print(i.var, ":", [x.var for x in v], flush=True)
-            # the mappings the kernel family realises: pipeline -> bit vector
-            realised = {}
-            for pipe in (_lib.AMOS_PIPE_PATCH, _lib.AMOS_PIPE_STAGED):
-                realised.setdefault(tuple(mapping_of_pipeline(match_result, pipe)), pipe)
+        for match_id, sweep in enumerate(sweeps):
+            sweep.announce(budget)
             if rnd == 0:
-                # trials only for mappings that can run: the others keep weight 0
-                runnable = [_realisation(match_result, r, realised) is not None for r in all_mappings[match_id]]
-                print("Num runnable mapping:", sum(runnable), flush=True)
-                runnable_total += sum(runnable)
-                if any(runnable):
-                    weights = [w if ok else 0.0 for w, ok in zip(weights, runnable)]
-                    total = sum(weights)
-                    weights = [w / total for w in weights]
-                    mapping_weights[match_id] = weights
-                    tune_trials = [math.ceil(trials_per_matching * x) for x in weights]
-                    print("Weights of the runnable mappings", weights, flush=True)
-            for mapping_id, record in enumerate(all_mappings[match_id]):
+                runnable_total += sweep.keep_runnable()
+            per_mapping = sweep.shares.trials(budget)
+            values = []
+            for mapping_id, record in enumerate(sweep.mappings):
                 print("Current explored mapping:", str(record), flush=True)
-                new_state = app.apply(record, drop_output=drop_output)
-                key = record.as_key()
-                log = os.path.join(schedule_log_dir, "mapping_" + str(key) + "_" + schedule_log_file)
-                value, params = 1 / MAX_FLOAT, None
-                how = _realisation(match_result, record, realised)
-                if how is None:
-                    print("No kernel instance realises this mapping; skipped.", flush=True)
-                else:
-                    pipes, rows = how
-                    if key not in cache:
-                        try:
-                            gen = MI355XScheduleGenerator(
-                                match_result, new_state, log_file=log, rows=rows,
-                                perf_percentage=perf_percentage if enable_perf_model else 1.0)
-                        except NoKernelError as e:
-                            print("No kernel for this compute:", e, flush=True)
-                            gen = None
-                        if gen is not None:
-                            if os.path.exists(log) and os.path.getsize(log) > 0:
-                                gen.load_from_file(log)
-                            gen._candidates = gen.candidates(pipes)
-                            cache[key] = ScheduleContext(gen, MI355XScheduleApplier(match_result, gen.lowered), pipes[0])
-                    ctx = cache.get(key)
-                    if ctx is not None:
-                        if tune_trials[mapping_id] and not pure_test:
-                            find_optimized_parameters(match_result, ctx.schedule_gen, ctx.schedule_app,
-                                                      measure_opt, checker, tune_trials[mapping_id],
-                                                      verbose=verbose_schedule)
-                        if ctx.schedule_gen.has_entry():
-                            entry = ctx.schedule_gen.get_best_entry()
-                            params, value = entry.record, entry.value
-                        elif pure_test and ctx.schedule_gen.candidates():
-                            params = ctx.schedule_gen.candidates()[0]
-                            value = 1.0 / ctx.schedule_gen.estimate(params)
-                        if value > best_value:
-                            best_value, best_ctx, best_params, best_mapping = value, ctx, params, record
-                best_values.append(value)
-                print(f"Best record value:{best_value} (larger is better)", flush=True)
-                print(f"Round {rnd+1}, Match {match_id+1}, Mapping {mapping_id+1}: {value}/{best_value}"
-                      f"({1/best_value*1e3} ms), {str(record)}, {str(params)}", flush=True)
+                value, params = explore(sweep, record, per_mapping[mapping_id])
+                values.append(value)
+                print(f"Best record value:{best['value']} (larger is better)", flush=True)
+                print(f"Round {rnd+1}, Match {match_id+1}, Mapping {mapping_id+1}: {value}/{best['value']}"
+                      f"({1/best['value']*1e3} ms), {str(record)}, {str(params)}", flush=True)
             if not pure_test:
-                # (mappings without a kernel stay at weight 0: the update is over the runnable ones)
-                ran = [v > 1 / MAX_FLOAT for v in best_values]
-                max_value = max(best_values)
-                exp_scores = [math.exp(min(0.0, x - max_value)) for x in best_values]
-                s = sum(exp_scores)
-                new_weights = [x / s for x in exp_scores]
-                delta = [new_weights[i] - weights[i] for i in range(len(weights))]
-                new_updates = [delta[i] + momentum * updates[i] for i in range(len(updates))]
-                new_weights = [weights[i] + new_updates[i] for i in range(len(new_updates))]
-                exp_scores = [math.exp(x) if ok or not any(ran) else 0.0 for x, ok in zip(new_weights, ran)]
-                s = sum(exp_scores)
-                mapping_weights[match_id] = [x / s for x in exp_scores]
-                weights_updates[match_id] = new_updates
-                print("New weights", mapping_weights[match_id], flush=True)
+                sweep.shares.update(values)
+                print("New weights", sweep.shares.shares, flush=True)
         if not pure_test:
             print("Show mapping exploration summary:", flush=True)
-            for k, v in cache.items():
-                print(f"mapping {str(k)}: explored {v.schedule_gen.num_entries()} schedules", flush=True)
+            for k, v in runs.items():
+                if v is not None:
+                    print(f"mapping {str(k)}: explored {v.schedule_gen.num_entries()} schedules", flush=True)
     if not pure_test:
-        print(f"Mapping exploration uses time {(time.time() - beg)} s.", flush=True)
-    result = AutoTensorizeResult() if best_ctx is None else AutoTensorizeResult(
-        best_ctx.schedule_gen, best_ctx.schedule_app, best_params, 1 / best_value, mapping=best_mapping)
+        print(f"Mapping exploration uses time {(time.time() - started)} s.", flush=True)
+    run = best["run"]
+    result = AutoTensorizeResult() if run is None else AutoTensorizeResult(
+        run.schedule_gen, run.schedule_app, best["params"], 1 / best["value"], mapping=best["mapping"])
     result.num_runnable_mappings, result.num_feasible_mappings = runnable_total, total_mappings
     return result
 

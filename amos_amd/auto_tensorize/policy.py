@@ -4,28 +4,29 @@ from functools import reduce
 from .compute_transform import MappingGenerator, Record, enumerate_mappings
 
 
+def _padding_volume(match_result):
+    """padded volume minus real volume of the fused loops, by the reference's own arithmetic
+    (transform_policy.py:12-27).  Its tile count reads `(ext + intrin_extent) - 1 // intrin_extent`:
+    the division binds first, so an axis counts ext + intrin_extent "tiles" (one fewer where the
+    intrinsic extent is 1).  Kept as it is: the README's choice of matching depends on it."""
+    padded, real = 1, 1
+    for intrin_axis, target_axes in match_result.axis_map.items():
+        width = int(intrin_axis.dom.extent)
+        ext = 1
+        for axis in target_axes:
+            ext *= int(axis.dom.extent)
+        tiles = ext + width - (1 // width)
+        padded *= tiles * width
+        real *= ext
+    return padded - real
+
+
 def all_fit(match_results):
-    """Matching with the smallest padding volume, all match points switched on.  The volume
-    formula is the reference's, operator precedence included (transform_policy.py:12-27:
-    `(ext + intrin_extent) - 1 // intrin_extent`), so the same matching wins: the first
-    strict minimum in registry order."""
-    minimum_padding = -1
-    chosen_match = None
-    for match_result in match_results:
-        effective_volume = 1
-        target_volume = 1
-        for iv, tv_lst in match_result.axis_map.items():
-            intrin_extent = int(iv.dom.extent)
-            ext = reduce(lambda x, y: x * int(y.dom.extent), tv_lst, 1)
-            target_volume *= ext
-            iterations = (ext + intrin_extent) - 1 // intrin_extent
-            effective_volume *= iterations * intrin_extent
-        padding_volume = effective_volume - target_volume
-        if minimum_padding < 0 or padding_volume < minimum_padding:
-            minimum_padding = padding_volume
-            chosen_match = match_result
-    n_points = len(list(chosen_match.axis_map.values())[0])
-    return chosen_match, Record(([1] * n_points, -1))
+    """The matching with the smallest padding volume (the first one on a tie, in registry order),
+    with every match point switched on."""
+    chosen = min(match_results, key=_padding_volume)
+    n_points = len(next(iter(chosen.axis_map.values())))
+    return chosen, Record(([1] * n_points, -1))
 
 
 def first_fit(match_results):
