@@ -31,7 +31,7 @@ static int out_extent(int in, int pad, int dil, int k, int stride) {
   return in + 2 * pad < eff ? 0 : (in + 2 * pad - eff) / stride + 1;
 }
 
-static void run(const Case& c) {
+static void run(const Case& c, bool quiet = false) {
   NchwShape s;
   s.N = c.N; s.C = c.C; s.D = c.D; s.H = c.H; s.W = c.W; s.K = c.K; s.T = c.T; s.R = c.R; s.S = c.S;
   s.sd = c.sd; s.sh = c.sh; s.sw = c.sw; s.pd = c.pd; s.ph = c.ph; s.pw = c.pw; s.dd = c.dd; s.dh = c.dh; s.dw = c.dw;
@@ -130,6 +130,7 @@ static void run(const Case& c) {
             }
       }
   }
+  if (quiet) return;   // (seeded random shapes: addresses and contents only)
   if (c.align >= 8) REQUIRE(conflicts == 0, "%ld bank-group collisions in %ld fragment reads", conflicts, reads);
   printf("%5.1f %% of fragment reads and %5.1f %% of staging stores with a bank-group collision; ",
          reads ? 100.0 * conflicts / reads : 0.0, writes ? 100.0 * wconflicts / writes : 0.0);
@@ -166,6 +167,38 @@ int main() {
       {2, 32, 3, 6, 8, 40, 3, 3, 3, 2, 1, 2, 1, 1, 0, 1, 1, 1, 3, 128, 8},        // ... mixed strides, 3-d
   };
   for (const Case& c : cases) run(c);
+  // seeded random shapes (window 3x3, any stride / padding / dilation the planner accepts): every
+  // writer inside its channel plane and its buffer, every reader on the element it wants
+  {
+    unsigned long long state = 0x9e3779b97f4a7c15ull;
+    auto rnd = [&](int lo, int hi) {   // uniform in [lo, hi]
+      state = state * 6364136223846793005ull + 1442695040888963407ull;
+      return lo + (int)((state >> 33) % (unsigned long long)(hi - lo + 1));
+    };
+    int ran = 0;
+    for (int it = 0; it < 4000 && ran < 400; ++it) {
+      Case c;
+      c.N = rnd(1, 5); c.C = 32; c.K = 8; c.R = 3; c.S = 3;
+      const bool three_d = rnd(0, 2) == 0;
+      c.D = three_d ? rnd(1, 5) : 1; c.T = three_d ? 3 : 1;
+      c.H = rnd(2, 40); c.W = rnd(2, 40);
+      c.sd = three_d ? rnd(1, 2) : 1; c.sh = rnd(1, 2); c.sw = rnd(1, 2);
+      c.pd = three_d ? rnd(0, 1) : 0; c.ph = rnd(0, 2); c.pw = rnd(0, 2);
+      c.dd = 1; c.dh = rnd(1, 2); c.dw = rnd(1, 2);
+      c.pg_shift = rnd(2, 3); c.BJ = rnd(0, 1) ? 128 : 256; c.align = rnd(0, 1) ? 8 : 1;
+      if ((c.H * c.W) % (1 << c.pg_shift)) continue;
+      if (out_extent(c.D, c.pd, c.dd, c.T, c.sd) <= 0 || out_extent(c.H, c.ph, c.dh, 3, c.sh) <= 0 ||
+          out_extent(c.W, c.pw, c.dw, 3, c.sw) <= 0)
+        continue;
+      const int before = fails;
+      run(c, true);
+      if (fails != before)
+        printf("  ... in random case N%d D%d %dx%d s%d%d%d p%d%d%d d%d%d%d pg%d BJ%d align %d\n", c.N, c.D, c.H, c.W, c.sd, c.sh,
+               c.sw, c.pd, c.ph, c.pw, c.dd, c.dh, c.dw, 1 << c.pg_shift, c.BJ, c.align);
+      ++ran;
+    }
+    printf("%d seeded random shapes\n", ran);
+  }
   // weight tiles: a bijection; a fragment read (rows r .. r+7, chunks of lane groups q and q + 2) and
   // a store (lanes 4x .. 4x+3 fill row nchw_row_of_slot(x); lanes l .. l+7 with l+32 .. l+39) on
   // sixteen different slots

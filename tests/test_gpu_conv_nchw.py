@@ -264,6 +264,51 @@ def test_conv_nchw_macro_step_counts(gpu, dtype, tile):
             assert torch.equal(outs[0], outs[1])
 
 
+def test_conv_nchw_random_shapes(gpu):
+    """seeded random 3x3 convolutions (2-d and 3-d, strides, paddings, dilations, ragged channel
+    counts, every tile) through AMOS_PIPE_NCHW against the oracle; shapes the planner refuses
+    (a tile over more than four images, a patch above the loaders' budget or LDS) are skipped"""
+    from amos_amd import _lib, ops
+    rng = np.random.default_rng(20240607)
+    ran = 0
+    for it in range(220):
+        dtype = ("float16", "float16", "bfloat16", "int8")[int(rng.integers(0, 4))]
+        es = 1 if dtype == "int8" else 2
+        three_d = rng.integers(0, 3) == 0
+        N, K = int(rng.integers(1, 4)), int(rng.integers(8, 80))
+        C = int(rng.integers(1, 4)) * 64 // es
+        D = int(rng.integers(1, 4)) if three_d else 1
+        H, W = int(rng.integers(3, 21)), int(rng.integers(3, 21))
+        if (H * W * es) % 8:
+            continue
+        st = tuple(int(v) for v in rng.integers(1, 3, 3))
+        pd = tuple(int(v) for v in rng.integers(0, 3, 3))
+        dl = (1,) + tuple(int(v) for v in rng.integers(1, 3, 2))
+        if not three_d:
+            st, pd = (1,) + st[1:], (0,) + pd[1:]
+        ti, tj = TILES[int(rng.integers(0, len(TILES)))]
+        xs, ws = (N, C, D, H, W), (K, C, 3 if three_d else 1, 3, 3)
+        if min(ops.conv_out_shape(xs, ws, st, pd, dl)) <= 0:
+            continue
+        x, w = make_operand(rng, xs, dtype), make_operand(rng, ws, dtype)
+        print("random nchw", it, dtype, (ti, tj), xs, K, st, pd, dl, flush=True)
+        try:
+            if three_d:
+                got = ops.conv3d(to_device(x, dtype), to_device(w, dtype), st, pd, dl, config=_cfg(_lib, tj, ti))
+            else:
+                got = ops.conv2d(to_device(x[:, :, 0], dtype), to_device(w[:, :, 0], dtype), st[1:], pd[1:], dl[1:],
+                                 config=_cfg(_lib, tj, ti))
+        except _lib.AmosError as e:
+            assert e.code == _lib.AMOS_ERR_INFEASIBLE, str(e)
+            continue
+        kw = {} if dtype == "int8" else {"acc": "float64"}
+        ref = (co.lib_conv3d(x, w, dtype, st, pd, dl, **kw) if three_d
+               else co.lib_conv2d(x[:, :, 0], w[:, :, 0], dtype, st[1:], pd[1:], dl[1:], **kw))
+        _check(got.cpu().numpy(), ref, dtype, "random %d %s %s %s" % (it, dtype, (ti, tj), xs))
+        ran += 1
+    assert ran >= 60, ran
+
+
 def test_conv_nchw_refusals(gpu):
     import torch
     from amos_amd import _lib, ops
