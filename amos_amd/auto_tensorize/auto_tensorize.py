@@ -351,7 +351,10 @@ def _realisation(match_result, record, realised):
     rows of the implicit GEMM where that is not all of them (lowering.remap_conv2d_rows: a 2-d
     convolution whose mapping keeps the batch loop and leaves p and / or q as time loops); the
     reduce side decides the kernel -- channels only: the patch-staged kernels, whose window taps
-    are time loops; channels and both window loops: the register-staged kernel (im2col)."""
+    are time loops; channels and both window loops: the register-staged kernel (im2col); channels
+    and one window loop ("+s" / "+r" behind the rows): the patch-staged kernels on an image whose
+    channels hold that loop's taps, the other window loop staying a time loop -- the output loop
+    along the folded axis is then a row loop of necessity."""
     patch_family = [_lib.AMOS_PIPE_PATCH, _lib.AMOS_PIPE_PATCH8, _lib.AMOS_PIPE_NCHW]
     pipe = _equivalent_pipeline(match_result, record, realised)
     if pipe is not None:
@@ -372,6 +375,10 @@ def _realisation(match_result, record, realised):
         pipes = patch_family
     elif rk_set == reduce_all:
         pipes = [_lib.AMOS_PIPE_STAGED]
+    elif rk_set == ["rc", "rs"] and "q" in i_set:
+        return patch_family, "".join(i_set) + "+s"
+    elif rk_set == ["rc", "rr"] and "p" in i_set:
+        return patch_family, "".join(i_set) + "+r"
     else:
         return None
     return pipes, "".join(i_set)

@@ -751,10 +751,21 @@ def remap_conv2d_rows(low, rows):
       rows n (p, q time loops): one image of P blocks of R rows and N*Q blocks of S columns;
                                 window R x S, strides R and S
 
+    `rows` may end in "+s" or "+r": that window loop joins the channels in the reduction of the
+    implicit GEMM (rk <- {rc, rs} or {rc, rr}) while the other window loop stays a time loop.  The
+    axis of the folded loop is copied tap by tap as above -- per output column q its S input
+    columns, side by side -- and the S copies of a column then ARE S * C channels of an image of
+    width Q (the same memory, NHWC), convolved with a window R x 1; "+r" is the same with H and W
+    swapped.  The output loop of the folded axis is a row loop of necessity (q with "+s", p with
+    "+r").
+
     The copies are dimension-separable gathers (zero padding along the copied axis included) into
     NHWC images; the weights are gathered into the window-major layout that goes with it and the
     result is gathered back to NKPQ."""
+    rows, _, fold = rows.partition("+")
     rows = "".join(sorted(rows))
+    if fold:
+        return _remap_conv2d_fold(low, rows, fold)
     if rows == "npq":
         return low
     if low.kind != "conv2d" or low.attrs.get("layout", "nchw") != "nchw" or low.gathers or low.out_view is not None \
@@ -803,6 +814,59 @@ def remap_conv2d_rows(low, rows):
                                                 [k * krs for k in range(K)]], wt.dtype)
         o_tabs = [[n * Q * K for n in range(N)], list(range(K)), [p * N * Q * K for p in range(P)], [q * K for q in range(Q)]]
     attrs = dict(low.attrs, layout="nhwc", rows=rows)
+    out = LoweredOp("conv2d", low.op_code, c, [src, wt], low.output, attrs)
+    out.add_input = low.add_input
+    out.gathers = {0: x_view, 1: w_view}
+    out.out_view = OperandView(None, [N, K, P, Q], o_tabs, low.output.dtype)
+    return out
+
+
+def _remap_conv2d_fold(low, rows, fold):
+    """remap_conv2d_rows with one window loop folded into the channels: fold 's' (rows 'npq' or
+    'nq') or 'r' (rows 'npq' or 'np')"""
+    ok_rows = {"s": ("npq", "nq"), "r": ("npq", "np")}.get(fold, ())
+    if low.kind != "conv2d" or low.attrs.get("layout", "nchw") != "nchw" or low.gathers or low.out_view is not None \
+            or low.constants or low.computed or len(low.attrs["x_shape"]) != 4 or rows not in ok_rows:
+        raise NoKernelError("no kernel for this convolution with rows %s and window loop %s in the reduction" % (rows, fold))
+    N, C, H, W = low.attrs["x_shape"]
+    K, _, R, S = low.attrs["w_shape"]
+    (sh, sw), (ph, pw), (dh, dw) = low.attrs["stride"], low.attrs["pad"], low.attrs["dil"]
+    P = (H + 2 * ph - ((R - 1) * dh + 1)) // sh + 1
+    Q = (W + 2 * pw - ((S - 1) * dw + 1)) // sw + 1
+    src, wt = low.inputs
+    hw, krs = H * W, C * R * S
+    rows_of = [(p * sh - ph + r * dh) * W if 0 <= p * sh - ph + r * dh < H else -1 for p in range(P) for r in range(R)]
+    cols_of = [q * sw - pw + s * dw if 0 <= q * sw - pw + s * dw < W else -1 for q in range(Q) for s in range(S)]
+    n_tab, c_tab = [n * C * hw for n in range(N)], [c * hw for c in range(C)]
+    c = _lib.ConvDesc()
+    c.N, c.K, c.D, c.T = N, K, 1, 1
+    c.stride_d, c.pad_d, c.dil_d = 1, 0, 1
+    c.in_dtype, c.out_dtype = low.desc.in_dtype, low.desc.out_dtype
+    c.layout = _lib.LAYOUT_CODE["nhwc"]
+    c.S, c.stride_w, c.pad_w, c.dil_w = 1, 1, 0, 1     # the folded axis: one output per S * C (R * C) channels
+    if fold == "s":
+        # image [N][H or P*R][Q*S][C] = [N][.][Q][S*C]; window R x 1
+        if "p" in rows:
+            a_tab, c.H, c.stride_h, c.pad_h, c.dil_h = [h * W for h in range(H)], H, sh, ph, dh
+        else:
+            a_tab, c.H, c.stride_h, c.pad_h, c.dil_h = rows_of, P * R, R, 0, 1
+        x_view = OperandView(src, [N, c.H, Q * S, C], [n_tab, a_tab, cols_of, c_tab], src.dtype)
+        c.W, c.C, c.R = Q, S * C, R
+        w_view = OperandView(wt, [R, S, C, K], [[r * S for r in range(R)], list(range(S)), [cc * R * S for cc in range(C)],
+                                                [k * krs for k in range(K)]], wt.dtype)
+        o_tabs = [[n * P * Q * K for n in range(N)], list(range(K)), [p * Q * K for p in range(P)], [q * K for q in range(Q)]]
+    else:
+        # transposed image [N][W or Q*S][P*R][C] = [N][.][P][R*C]; window S x 1
+        if "q" in rows:
+            a_tab, c.H, c.stride_h, c.pad_h, c.dil_h = list(range(W)), W, sw, pw, dw
+        else:
+            a_tab, c.H, c.stride_h, c.pad_h, c.dil_h = cols_of, Q * S, S, 0, 1
+        x_view = OperandView(src, [N, c.H, P * R, C], [n_tab, a_tab, rows_of, c_tab], src.dtype)
+        c.W, c.C, c.R = P, R * C, S
+        w_view = OperandView(wt, [S, R, C, K], [list(range(S)), [r * S for r in range(R)], [cc * R * S for cc in range(C)],
+                                                [k * krs for k in range(K)]], wt.dtype)
+        o_tabs = [[n * Q * P * K for n in range(N)], list(range(K)), [p * K for p in range(P)], [q * P * K for q in range(Q)]]
+    attrs = dict(low.attrs, layout="nhwc", rows=rows + "+" + fold)
     out = LoweredOp("conv2d", low.op_code, c, [src, wt], low.output, attrs)
     out.add_input = low.add_input
     out.gathers = {0: x_view, 1: w_view}
