@@ -287,7 +287,11 @@ def auto_tensorize_v4(target_dag, target, schedule_log_file, measure_opt, schedu
                 return None
             if os.path.exists(log) and os.path.getsize(log) > 0:
                 gen.load_from_file(log)
-            gen._candidates = gen.candidates(pipes)
+            # a mapping the kernels implement as it is (no remapped loops) is also what the mapper's
+            # own choice and its AMOS_PIPE_AUTO resolution run -- the direct-to-LDS GEMM, the
+            # depthwise, few-channel and skinny kernels, which have no pipeline value of their own;
+            # a remapped one only gets the pipelines of its kernel family
+            gen._candidates = gen.candidates(None if rows is None else pipes)
             runs[key] = _MappingRun(gen, MI355XScheduleApplier(sweep.match_result, gen.lowered), pipes[0])
         return runs[key]
 

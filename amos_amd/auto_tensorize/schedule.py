@@ -222,7 +222,7 @@ class MI355XScheduleGenerator(object):
             add(KernelParams(d.tile_i, d.tile_j, d.split_k, d.pipeline))
         is_conv = low.kind in ("conv2d", "conv3d")
         pipes = pipelines if pipelines is not None else (
-            [_lib.AMOS_PIPE_PATCH, _lib.AMOS_PIPE_PATCH8, _lib.AMOS_PIPE_STAGED, _lib.AMOS_PIPE_AUTO] if is_conv
+            [_lib.AMOS_PIPE_NCHW, _lib.AMOS_PIPE_PATCH, _lib.AMOS_PIPE_PATCH8, _lib.AMOS_PIPE_STAGED, _lib.AMOS_PIPE_AUTO] if is_conv
             else [_lib.AMOS_PIPE_AUTO, _lib.AMOS_PIPE_STAGED])
         first = len(out)
         for pipe in pipes:

@@ -479,6 +479,28 @@ def test_v4_pure_test_mode_lists_infeasible_mappings(tmp_path, capsys):
     assert fused["rk"] in ({"rc"}, {"rc", "rr", "rs"})
 
 
+def test_v4_keeps_the_kernels_without_a_pipeline_value(tmp_path):
+    """the network dispatcher tunes every layer through auto_tensorize_v4: the mapping the kernels
+    implement as it is must keep the mapper's own choice among its candidates -- the depthwise,
+    few-channel and skinny kernels and the direct-to-LDS GEMM are reached through it alone"""
+    import contextlib
+    import io
+    from amos_amd import ops
+    from amos_amd.auto_tensorize import network as net
+    want = {"depthwise 3x3/1 32 @112": "amos_depthwise_conv", "conv 3x3/2 3->32 @224": "amos_conv_few_channels"}
+    seen = {}
+    for sg in list(net.mobilenet_v1(16))[:2] + list(net.mi_lstm(1))[:1] + list(net.bert_base(16))[:1]:
+        with contextlib.redirect_stdout(io.StringIO()):
+            res = at.auto_tensorize_v4(sg.dag, "hip", "x.log", at.MeasureOptions(target="hip"),
+                                       schedule_log_dir=str(tmp_path / "logs"), trials=0, transform_strict=False)
+        assert res.defined(), sg.note
+        low = res.sch_gen.lowered
+        seen[sg.note] = ops.kernel_name(low.op_code, low.desc, res.params.to_config())
+    for note, kernel in want.items():
+        assert kernel in seen[note], seen
+    assert any("amos_skinny_gemm" in k for k in seen.values()) and any("amos_gemm_tn" in k for k in seen.values()), seen
+
+
 def test_log_format_and_reference_fixture(tmp_path):
     from amos_amd.auto_tensorize.schedule import KernelParams, read_log
     rows = read_log(os.path.join(GOLDEN, "a100_conv2d_1_256_14_14_256_3_3_mapping_0010010.log"))
