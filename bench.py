@@ -303,7 +303,8 @@ def model_check():
         oshape = ops.conv_out_shape(xs5, ws5, st, pd, (1, 1, 1))
         y = torch.empty(oshape if op == CONV3D else (oshape[0], oshape[1], oshape[3], oshape[4]),
                         device="cuda", dtype=torch.int32 if dt == i8 else torch.float32)
-        out.append(sweep(name, fitted, op, d, x, w, y, (4, 5, 1), (1, 2, 4) if op == CONV2D else (1,)))
+        out.append(sweep(name, fitted, op, d, x, w, y, (_lib.AMOS_PIPE_NCHW, _lib.AMOS_PIPE_PATCH, _lib.AMOS_PIPE_PATCH8, _lib.AMOS_PIPE_STAGED),
+                         (1, 2, 4) if op == CONV2D else (1,)))
 
     for M, N, K in [(8192, 8192, 8192), (2048, 2048, 2048), (512, 512, 4096), (4096, 256, 1024)]:
         gemm_case(M, N, K, 0, 1, f16, True)
@@ -322,6 +323,8 @@ def model_check():
     conv_case("conv2d N8 C128 28x28 K256 3x3 f16", False, (8, 128, 28, 28), (256, 128, 3, 3), (1, 1, 1), (0, 1, 1))
     conv_case("conv2d N16 C64 56x56 K64 1x1 f16", False, (16, 64, 56, 56), (64, 64, 1, 1), (1, 1, 1), (0, 0, 0))
     conv_case("conv2d N4 C48 30x30 K96 5x5 f16", False, (4, 48, 30, 30), (96, 48, 5, 5), (1, 1, 1), (0, 2, 2))
+    conv_case("conv2d N16 C64 56x56 K64 3x3 f16", False, (16, 64, 56, 56), (64, 64, 3, 3), (1, 1, 1), (0, 1, 1))
+    conv_case("conv2d N64 C512 14x14 K512 3x3 f16", False, (64, 512, 14, 14), (512, 512, 3, 3), (1, 1, 1), (0, 1, 1))
     return out
 
 
