@@ -1189,7 +1189,9 @@ static int launch_conv_nchw(const Plan& pl, hipStream_t stream) {
     if (attr_err == hipSuccess) { inst->scratch_bytes = (int)fa.localSizeBytes; inst->static_lds = (int)fa.sharedSizeBytes; }
     int blocks = 0;
     if (attr_err == hipSuccess)
-      attr_err = hipOccupancyMaxActiveBlocksPerMultiprocessor(&blocks, (const void*)inst->fn, inst->threads, 0);
+      attr_err = hipOccupancyMaxActiveBlocksPerMultiprocessor(
+          &blocks, (const void*)inst->fn, inst->threads,
+          (size_t)2 * 9 * inst->bi * 64 + (size_t)2 * nchw_patch_buffer_bytes(inst->bj));
     inst->fits = blocks >= 1;
   });
   if (attr_err != hipSuccess)
