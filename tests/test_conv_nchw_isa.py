@@ -6,8 +6,8 @@ those registers.  This test compiles every instance to assembly (no GPU needed) 
 
   * outside the assembly statements no instruction names a staging register;
   * the assembly statements stay inside the 32 staging registers;
-  * no instance spills to scratch memory or uses accumulation registers, and its register count
-    leaves room for the waves of one workgroup on a compute unit.
+  * no instance spills to scratch memory or uses accumulation registers; its register count
+    covers the staging registers and leaves room for the waves of one workgroup on a compute unit.
 """
 import os
 import re
@@ -123,6 +123,7 @@ def test_staging_registers_belong_to_the_assembly_statements():
                 r = res.get(name)
                 assert r is not None, "%s: no resource remarks" % what
                 assert r.get("scratch", 0) == 0 and r.get("agprs", 0) == 0, "%s: %s" % (what, r)
-                assert r["vgprs"] <= rec["base"] + 32, "%s: %s" % (what, r)
+                # (the wave's register allocation covers the staging registers, and nothing above them)
+                assert max(rec["inside"]) < r["vgprs"] <= rec["base"] + 32, "%s: %s" % (what, r)
                 assert r["occupancy"] * 4 >= rec["waves"], "%s: %d waves do not fit (%s)" % (what, rec["waves"], r)
         assert total >= 60
