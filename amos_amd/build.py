@@ -20,37 +20,58 @@ def sources():
 
 
 def build(verbose=True, jobs=8):
-    """compile every translation unit (in parallel) and link the shared library"""
+    """compile every translation unit (in parallel), read the compiled code of the kernels whose
+    assembly statements own registers (isa_check) and link the shared library only if that holds"""
+    from . import isa_check
     hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
     inc = ["-I" + os.path.join(ROOT, "include"), "-I" + CSRC]
     objdir = os.path.join(HERE, "build")
     os.makedirs(objdir, exist_ok=True)
     procs, objs = [], []
+    jobs_list = []
     for src in sources():
         obj = os.path.join(objdir, os.path.basename(src) + ".o")
         objs.append(obj)
-        cmd = [hipcc] + HIP_FLAGS + inc + ["-c", src, "-o", obj]
+        jobs_list.append((src, obj, [hipcc] + HIP_FLAGS + inc + ["-c", src, "-o", obj]))
+    # the same units once more as assembly text, for the check
+    checked = []
+    for unit in isa_check.UNITS:
+        src = os.path.join(CSRC, unit)
+        asm = os.path.join(objdir, unit + ".s")
+        checked.append((unit, asm))
+        jobs_list.append((src, asm, [hipcc] + HIP_FLAGS + inc + isa_check.ASM_FLAGS + [src, "-o", asm]))
+    for src, out, cmd in jobs_list:
         if verbose:
             print(" ".join(cmd), flush=True)
         # (the compiler's output goes to a file: a pipe that nobody reads while we wait for the
         # process fills up after 64 KB of diagnostics and the compiler then blocks for good)
-        log = open(obj + ".log", "w+b")
-        procs.append((src, subprocess.Popen(cmd, stdout=log, stderr=subprocess.STDOUT), log))
-        while sum(p.poll() is None for _, p, _ in procs) >= jobs:
-            for _, p, _ in procs:
+        log = open(out + ".log", "w+b")
+        procs.append((src, out, subprocess.Popen(cmd, stdout=log, stderr=subprocess.STDOUT), log))
+        while sum(p.poll() is None for _, _, p, _ in procs) >= jobs:
+            for _, _, p, _ in procs:
                 if p.poll() is None:
                     p.wait()
                     break
-    for src, p, log in procs:
+    logs = {}
+    for src, out, p, log in procs:
         p.wait()
         log.seek(0)
-        out = log.read()
+        text = log.read().decode()
         log.close()
-        text = "\n".join(l for l in out.decode().splitlines() if "packed-fp32-ops" not in l)
+        logs[out] = text
+        shown = "\n".join(l for l in text.splitlines() if "packed-fp32-ops" not in l and "remark:" not in l)
         if p.returncode != 0:
-            raise RuntimeError("hipcc failed on %s:\n%s" % (src, text))
-        if verbose and text.strip():
-            print(text)
+            raise RuntimeError("hipcc failed on %s:\n%s" % (src, shown))
+        if verbose and shown.strip() and not out.endswith(".s"):   # (the assembly jobs' output is remarks)
+            print(shown)
+    bad = []
+    for unit, asm in checked:
+        bad += isa_check.violations(unit, asm, logs[asm])[1]
+    if bad:
+        if os.path.exists(OUT):
+            os.remove(OUT)
+        raise RuntimeError("not linking %s: the compiled code breaks the rule of amos_amd/isa_check.py\n%s"
+                           % (OUT, "\n".join(bad)))
     cmd = [hipcc, "--offload-arch=gfx950", "-shared", "-fPIC"] + objs + ["-o", OUT]
     if verbose:
         print(" ".join(cmd), flush=True)
