@@ -309,6 +309,38 @@ def test_conv_nchw_random_shapes(gpu):
     assert ran >= 60, ran
 
 
+@pytest.mark.parametrize("dtype", ["float16", "bfloat16"])
+def test_conv_nchw_two_rounds_with_packed_weights(gpu, dtype):
+    """a patch of more than 64 load groups (two rounds of the loaders, `pt2`) together with weights
+    packed by their owner: against the oracle, and the same bits as with the weights read as they are"""
+    import torch
+    from amos_amd import _lib, ops
+    lib = _lib.load()
+    xs, ws = (4, 64, 1, 14, 14), (72, 64, 1, 3, 3)
+    rng = np.random.default_rng(11)
+    x, w = make_operand(rng, xs, dtype), make_operand(rng, ws, dtype)
+    dx, dw = to_device(x, dtype), to_device(w, dtype)
+    d = ops.conv_desc(xs, ws, dx.dtype, (1, 1, 1), (0, 1, 1), (1, 1, 1))
+    oshape = ops.conv_out_shape(xs, ws, (1, 1, 1), (0, 1, 1), (1, 1, 1))
+    need = lib.amos_conv_packed_weights_bytes(_lib.AMOS_OP_CONV2D, ctypes.byref(d))
+    packed = torch.empty(need, dtype=torch.uint8, device="cuda")
+    _lib.check(lib.amos_conv_pack_weights(_lib.AMOS_OP_CONV2D, ctypes.byref(d), dw.data_ptr(), packed.data_ptr(), None))
+    outs = []
+    for flags, wptr in ((_lib.AMOS_FLAG_WEIGHTS_PACKED, packed.data_ptr()), (0, dw.data_ptr())):
+        c = ops.make_config(_cfg(_lib, 256, 64))
+        c.reserved[0] = flags
+        name = ops.kernel_name(_lib.AMOS_OP_CONV2D, d, c)
+        assert name.endswith(",pt2>") and (",packed" in name) == bool(flags), name
+        print("two rounds", dtype, name, flush=True)
+        out = torch.full(oshape, -3, dtype=torch.float32, device="cuda")
+        _lib.check(lib.amos_conv2d(ctypes.byref(d), ctypes.byref(c), dx.data_ptr(), wptr, out.data_ptr(), None, 0, None))
+        torch.cuda.synchronize()
+        outs.append(out)
+    assert torch.equal(outs[0], outs[1])
+    ref = co.lib_conv2d(x[:, :, 0], w[:, :, 0], dtype, 1, 1, 1, acc="float64")
+    _check(outs[0].cpu().numpy()[:, :, 0], ref, dtype, "two rounds, packed weights, %s" % dtype)
+
+
 def test_conv_nchw_refusals(gpu):
     import torch
     from amos_amd import _lib, ops
