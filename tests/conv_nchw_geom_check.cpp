@@ -176,7 +176,7 @@ int main() {
       return lo + (int)((state >> 33) % (unsigned long long)(hi - lo + 1));
     };
     int ran = 0;
-    for (int it = 0; it < 4000 && ran < 400; ++it) {
+    for (int it = 0; it < 40000 && ran < 3000; ++it) {
       Case c;
       c.N = rnd(1, 5); c.C = 32; c.K = 8; c.R = 3; c.S = 3;
       const bool three_d = rnd(0, 2) == 0;
