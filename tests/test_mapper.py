@@ -479,6 +479,36 @@ def test_v4_pure_test_mode_lists_infeasible_mappings(tmp_path, capsys):
     assert fused["rk"] in ({"rc"}, {"rc", "rr", "rs"})
 
 
+@pytest.mark.parametrize("rows", ["nq", "np", "n", "npq+s", "nq+s", "npq+r", "np+r"])
+@pytest.mark.parametrize("case", [(3, 4, 7, 9, 5, 1, 1, 1), (2, 3, 8, 6, 4, 2, 1, 1), (2, 2, 9, 9, 3, 1, 2, 2), (1, 5, 6, 7, 2, 2, 2, 1), (2, 3, 5, 8, 6, 1, 0, 1)])
+def test_remapped_convolutions_mean_the_same(rows, case):
+    """lowering.remap_conv2d_rows on the CPU: the gathered activations and weights, convolved as the
+    sub-convolution's descriptor says (NHWC, its window, strides and paddings) and gathered back
+    through out_view, are the original convolution -- for every class of rows and folded window
+    loop, with strides, padding and dilation (int8: exact)"""
+    from amos_amd.auto_tensorize.lowering import lower_main_op, remap_conv2d_rows
+    N, C, H, W, K, st, pd, dl = case
+    A, B, Conv = conv2d(N, C, H, W, K, 3, 3, st, pd, dl, dtype="int8", out_dtype="int32", exact_int=True)
+    dag = at.compute_dag_from_tensors([Conv])
+    main_op = [op for op in dag.op_lst if op.reduce_axis][0]
+    low = remap_conv2d_rows(lower_main_op(main_op, dag), rows)
+    rng = np.random.default_rng(7)
+    a = rng.integers(-9, 10, (N, C, H, W)).astype(np.int8)
+    b = rng.integers(-9, 10, (K, C, 3, 3)).astype(np.int8)
+    want = co.lib_conv2d(a, b, "int8", st, pd, dl)
+    d = low.desc
+    assert d.layout == _lib.LAYOUT_CODE["nhwc"]
+    # the kernel's operands: activations [N][H][W][C], weights [R][S][C][K] of the sub-convolution
+    x = apply_view(low.gathers[0], a).reshape(d.N, d.H, d.W, d.C)
+    w = apply_view(low.gathers[1], b).reshape(d.R, d.S, d.C, d.K)
+    y = co.lib_conv2d(np.transpose(x, (0, 3, 1, 2)), np.transpose(w, (3, 2, 0, 1)), "int8", (d.stride_h, d.stride_w),
+                      (d.pad_h, d.pad_w), (d.dil_h, d.dil_w))
+    kernel_out = np.ascontiguousarray(np.transpose(y, (0, 2, 3, 1)))      # what the kernel writes: NHWC
+    assert kernel_out.size == want.size
+    got = apply_view(low.out_view, kernel_out)
+    assert got.shape == want.shape and np.array_equal(got, want)
+
+
 def test_v4_keeps_the_kernels_without_a_pipeline_value(tmp_path):
     """the network dispatcher tunes every layer through auto_tensorize_v4: the mapping the kernels
     implement as it is must keep the mapper's own choice among its candidates -- the depthwise,
