@@ -170,8 +170,10 @@ typedef struct {
                               /* and transposed in registers on their way to LDS; the weights   */
                               /* are packed to [K][T*9][C] -- into the workspace by the call     */
                               /* (amos_workspace_bytes), or once by their owner                  */
-                              /* (amos_conv_pack_weights, AMOS_FLAG_WEIGHTS_PACKED) -- or,       */
-                              /* without a workspace, transposed in registers as well; tiles    */
+                              /* (amos_conv_pack_weights, AMOS_FLAG_WEIGHTS_PACKED) -- or        */
+                              /* transposed in registers as well: without a workspace, and for   */
+                              /* a conv2d with 16-byte aligned weights also with one where the   */
+                              /* mapper's model says the packing launch would cost more; tiles   */
                               /* 32 or 64 output channels x 128 or 256 output positions          */
 
 int amos_version(void);
