@@ -98,6 +98,7 @@ EXPORTS = [
     "amos_check_config", "amos_workspace_bytes", "amos_estimate_seconds", "amos_gemm", "amos_bgemm", "amos_conv2d",
     "amos_conv3d", "amos_conv2d_noalloc", "amos_conv_packed_weights_bytes", "amos_conv_pack_weights", "amos_run_fused", "amos_time", "amos_time_fused", "amos_gather", "amos_time_gather",
     "amos_eltwise", "amos_time_eltwise", "amos_kernel_name", "amos_match", "amos_enumerate_mappings",
+    "amos_mfma_ceiling",
 ]
 
 _lib = None
@@ -142,6 +143,10 @@ def load():
     lib.amos_time_fused.argtypes = [ctypes.c_int, vp, ctypes.POINTER(KernelConfig), ctypes.POINTER(Epilogue),
                                     vp, vp, vp, vp, sz, vp, ctypes.c_int, ctypes.c_int, ctypes.c_int,
                                     ctypes.POINTER(ctypes.c_double)]
+    lib.amos_mfma_ceiling.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, vp, vp, sz, vp,
+                                      ctypes.c_int, vp, ctypes.POINTER(ctypes.c_double),
+                                      ctypes.POINTER(ctypes.c_double)]
+    lib.amos_mfma_ceiling.restype = ctypes.c_int
     lib.amos_gather.argtypes = [ctypes.POINTER(GatherDesc), vp, vp, vp, vp]
     lib.amos_eltwise.argtypes = [ctypes.POINTER(EltwiseDesc), ctypes.POINTER(vp), vp, vp]
     lib.amos_eltwise.restype = ctypes.c_int

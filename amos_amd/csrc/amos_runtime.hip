@@ -219,14 +219,15 @@ __global__ void fill_zero_kernel(T* p, int64_t rows, int64_t cols, int64_t ld) {
   for (; idx < n; idx += (int64_t)gridDim.x * blockDim.x) p[(idx / cols) * ld + idx % cols] = 0;
 }
 
-// out[r][c] = part[0][r][c] + part[1][r][c] + ... in that order (split-K partial sums)
+// out[b][r][c] = part[0][b][r][c] + part[1][b][r][c] + ... in that order (split-K partial sums);
+// blockIdx.y walks the batches, `batch_stride` elements apart in the output and in every slice
 template <typename T>
 __global__ void reduce_splits_kernel(T* out, const T* part, int64_t rows, int64_t cols, int64_t ld, int nsplit,
-                                     int64_t stride) {
-  int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+                                     int64_t stride, int64_t batch_stride, int64_t nbatch) {
   const int64_t n = rows * cols;
-  for (; idx < n; idx += (int64_t)gridDim.x * blockDim.x) {
-    const int64_t off = (idx / cols) * ld + idx % cols;
+  for (int64_t b = blockIdx.y; b < nbatch; b += gridDim.y)
+  for (int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; idx < n; idx += (int64_t)gridDim.x * blockDim.x) {
+    const int64_t off = b * batch_stride + (idx / cols) * ld + idx % cols;
     T acc = part[off];
     for (int s = 1; s < nsplit; ++s) acc += part[(int64_t)s * stride + off];
     out[off] = acc;
@@ -379,6 +380,14 @@ static int64_t plan_out_footprint(const Plan& pl) {
   return (n + 63) & ~(int64_t)63;
 }
 // whether the caller's workspace has room for `split` slices of partial sums behind the pipeline's own share
+// The plan takes `bytes` from the front of the caller's workspace (operand copies, packed weights,
+// relaid activations): the slices of a split's partial sums start behind the largest such claim.
+// amos_workspace_bytes() assumes 16-byte aligned operands; a misaligned one can add a copy, and
+// the slices must not start inside it.
+static void claim_workspace(Plan& pl, int64_t bytes) {
+  const size_t b = ((size_t)(bytes > 0 ? bytes : 0) + 255) & ~(size_t)255;
+  if (b > pl.ws_own) pl.ws_own = b;
+}
 static bool split_partials_fit(const Plan& pl, int split) {
   if (!pl.ws_base || ((uintptr_t)pl.ws_base & 255) || split < 2) return false;
   return pl.ws_bytes >= pl.ws_own + (size_t)split * (size_t)plan_out_footprint(pl) * 4;
@@ -484,8 +493,10 @@ static int plan_gemm(Plan& pl, int op, const void* desc_any, const amos_gemm_des
       d->lda >= (d->trans_a ? d->M : d->K) && d->ldb >= (d->trans_b ? d->K : d->N) &&
       (d->in_dtype == AMOS_F16 || d->in_dtype == AMOS_BF16 || d->in_dtype == AMOS_I8)) {
     const GemmRepack rp = gemm_repack(*d, batch, !aligned16(A), !aligned16(B));
-    if (rp.total() > 0 && ws_bytes >= (size_t)rp.total())
+    if (rp.total() > 0 && ws_bytes >= (size_t)rp.total()) {
+      claim_workspace(pl, rp.total());
       return plan_gemm_repacked(pl, op, d, rp, batch, sa, sb, sc, cfg, A, B, C, workspace);
+    }
   }
   if (!fits_int(d->M) || !fits_int(d->N) || !fits_int(d->K) || batch <= 0)
     return set_error(AMOS_ERR_BAD_ARG, "extents must be in [1, 2^31): M=%lld N=%lld K=%lld batch=%lld",
@@ -646,7 +657,9 @@ static int plan_conv(Plan& pl, int op, const amos_conv_desc_t* d, const amos_ker
   // A pointwise convolution runs on the GEMM kernels, vector loaders and operand copies
   // included, unless the patch-staged pipeline is asked for.
   amos_bgemm_desc_t b;
-  if ((!cfg || (cfg->pipeline != AMOS_PIPE_PATCH && cfg->pipeline != AMOS_PIPE_PATCH8)) && conv_as_gemm(c, op, &b)) {
+  // (... or the NCDHW-direct one, whose planner then says why it does not apply)
+  if ((!cfg || (cfg->pipeline != AMOS_PIPE_PATCH && cfg->pipeline != AMOS_PIPE_PATCH8 && cfg->pipeline != AMOS_PIPE_NCHW)) &&
+      conv_as_gemm(c, op, &b)) {
     b.g.out_dtype = c.out_dtype;
     const bool w_first = layout == AMOS_LAYOUT_NCHW;
     return plan_gemm(pl, AMOS_OP_BGEMM, &b, &b.g, b.batch, b.stride_a, b.stride_b, b.stride_c, cfg,
@@ -660,6 +673,7 @@ static int plan_conv(Plan& pl, int op, const amos_conv_desc_t* d, const amos_ker
     const GemmRepack rp = gemm_repack(b.g, b.batch, !aligned16(Wt), false, true);
     if (ws_bytes >= (size_t)rp.total()) {
       b.g.out_dtype = c.out_dtype;
+      claim_workspace(pl, rp.total());
       return plan_gemm_repacked(pl, AMOS_OP_BGEMM, &b.g, rp, b.batch, b.stride_a, b.stride_b, b.stride_c, cfg,
                                 Wt, X, Y, workspace, &sub);
     }
@@ -704,6 +718,7 @@ static int plan_conv(Plan& pl, int op, const amos_conv_desc_t* d, const amos_ker
     char* wpad = (char*)workspace;
     char* col = wpad + ic.bytes_w;
     b.g.out_dtype = c.out_dtype;
+    claim_workspace(pl, ic.bytes_w + ic.bytes_x);
     // without a tile from the caller: the convolution's own default (the best direct tile)
     amos_kernel_config_t own;
     if (!cfg || cfg->tile_i <= 0 || cfg->tile_j <= 0) {
@@ -836,6 +851,7 @@ static int plan_conv(Plan& pl, int op, const amos_conv_desc_t* d, const amos_ker
       pl.nchw_wmode = NCHW_W_PACKED;
       pl.nchw_pack = 1;
       q.w = (const char*)workspace;
+      claim_workspace(pl, (int64_t)packed_bytes);
     } else {
       pl.nchw_wmode = (np.t1 && aligned16(Wt)) ? NCHW_W_KCRS : NCHW_W_KCTRS;
     }
@@ -964,6 +980,7 @@ static int plan_conv(Plan& pl, int op, const amos_conv_desc_t* d, const amos_ker
   }
   pl.conv_ups = 1;
   pl.conv_lds = lds;
+  claim_workspace(pl, need_ws);
   ConvFpropParams& q = pl.cv;
   memset(&q, 0, sizeof(q));
   q.x = (const char*)X; q.w = (const char*)Wt; q.y = (char*)Y;
@@ -1232,16 +1249,18 @@ static int launch(const Plan& pl, hipStream_t stream) {
   int rc = launch_kernels(pl, stream);
   if (rc || !pl.part) return rc;
   const int64_t n = pl.fill_rows * pl.fill_cols;
-  const int blocks = (int)std::min<int64_t>((n + 255) / 256, 8192);
-  for (int64_t b = 0; b < (pl.fill_once ? 1 : pl.batch); ++b) {
-    const int64_t off = b * pl.p.out_batch * 4;
-    if (pl.dt == DT_I8)
-      hipLaunchKernelGGL(reduce_splits_kernel<int>, dim3(blocks), dim3(256), 0, stream, (int*)(pl.part_out + off),
-                         (const int*)(pl.part + off), pl.fill_rows, pl.fill_cols, pl.fill_ld, pl.split, pl.part_stride);
-    else
-      hipLaunchKernelGGL(reduce_splits_kernel<float>, dim3(blocks), dim3(256), 0, stream, (float*)(pl.part_out + off),
-                         (const float*)(pl.part + off), pl.fill_rows, pl.fill_cols, pl.fill_ld, pl.split, pl.part_stride);
-  }
+  // one launch for all batches: blockIdx.y walks them
+  const int64_t nb = pl.fill_once ? 1 : pl.batch;
+  const int by = (int)std::min<int64_t>(nb, 65535);
+  const int blocks = (int)std::min<int64_t>((n + 255) / 256, std::max<int64_t>(8192 / by, 1));
+  if (pl.dt == DT_I8)
+    hipLaunchKernelGGL(reduce_splits_kernel<int>, dim3(blocks, by), dim3(256), 0, stream, (int*)pl.part_out,
+                       (const int*)pl.part, pl.fill_rows, pl.fill_cols, pl.fill_ld, pl.split, pl.part_stride,
+                       pl.p.out_batch, nb);
+  else
+    hipLaunchKernelGGL(reduce_splits_kernel<float>, dim3(blocks, by), dim3(256), 0, stream, (float*)pl.part_out,
+                       (const float*)pl.part, pl.fill_rows, pl.fill_cols, pl.fill_ld, pl.split, pl.part_stride,
+                       pl.p.out_batch, nb);
   HIP_TRY(hipGetLastError());
   return 0;
 }

@@ -2,9 +2,10 @@
 on one MI355X, next to the CPU restatement of the reference's llvm path timed in the same run.
 
   python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--report FILE] [--model-check FILE]
+  python bench.py --mfma-ceiling     (what the matrix cores sustain with nothing else in their way)
 
 A step is one launch of the GEMM over device-resident operands.  Prints ONE JSON line; its
-`config.per_op` holds the other configurations of the path (fp16 / int8 conv2d, batched GEMM,
+`per_op` holds the other configurations of the path (fp16 / int8 conv2d, batched GEMM,
 conv3d), each timed in the same run next to the CPU loop nest on a slab of the same workload.
 `--report FILE` additionally times every configuration of the path (GEMM, batched GEMM,
 conv2d fp16 / int8, conv3d) and writes a per-config table as JSON to FILE.
@@ -62,6 +63,32 @@ def measured_traffic(kernel_name):
     return None
 
 
+def mfma_ceiling(da, db, variants=None, launches=10, repeats=3):
+    """amos_mfma_ceiling over the named variants (shape, random operands, copies, reads): the
+    matrix-core instruction stream of the 8192^3 product with no wait anywhere.  da, db: device
+    fp16 [8192][8192] operands.  Returns rows with the best of `repeats` means of `launches`."""
+    import torch
+    from amos_amd import _lib
+    lib = _lib.load()
+    sink = torch.zeros(256, device="cuda")
+    variants = variants or [(16, 1, 0, 0)]
+    rows = []
+    for shape, rnd, copies, reads in variants:
+        best, flop = None, ctypes.c_double()
+        for _ in range(repeats):
+            sec = ctypes.c_double()
+            _lib.check(lib.amos_mfma_ceiling(shape, rnd, copies, reads, da.data_ptr(), db.data_ptr(),
+                                             da.numel() * da.element_size(), sink.data_ptr(), launches, None,
+                                             ctypes.byref(sec), ctypes.byref(flop)))
+            best = sec.value if best is None else min(best, sec.value)
+        rows.append({"instruction": "v_mfma_f32_16x16x32_f16" if shape == 16 else "v_mfma_f32_32x32x16_f16",
+                     "operands": "random fp16 U[-1,1]" if rnd else "small constants",
+                     "extra_traffic": " + ".join(n for n, on in (("global->LDS copies", copies), ("LDS fragment reads", reads)) if on) or "none",
+                     "us_per_launch": best * 1e6, "tflops": flop.value / best / 1e12,
+                     "frac_of_published_peak": flop.value / best / 1e12 / PEAK_F16_TFLOPS})
+    return rows
+
+
 def cpu_baseline_gemm(a, b, seconds_budget=12.0):
     """te_literal loop nest (single thread, as TVM's default schedule) on a slab of rows of the
     same 8192^3 workload, scaled linearly; plus an all-core OpenMP run of a larger slab."""
@@ -115,7 +142,7 @@ def run_all_configs(cpu=True, only=None, launches=None):
             t = ops.time_op(op, desc, i0, i1, out, config=cfg, number=launches, repeat=1, min_repeat_ms=0, add=fused)
         else:
             t = ops.time_op(op, desc, i0, i1, out, config=cfg, number=20, repeat=3, min_repeat_ms=100, add=fused)
-        return min(t), cfg
+        return sum(t) / len(t), cfg   # mean seconds per call over all repeats
 
     def add(name, op, desc, hin, dtype, flop, nbytes, out_shape, cpu_fn, frac, fused_tail=False):
         if only and not any(o in name for o in ([only] if isinstance(only, str) else only)):
@@ -133,7 +160,8 @@ def run_all_configs(cpu=True, only=None, launches=None):
         row = {"config": name, "kernel": ops.kernel_name(op, desc, cfg), "split_k": cfg.split_k,
                "gpu_us": sec * 1e6, "tflops": flop / sec / 1e12,
                "pct_mfma_peak": 100 * t_mfma / sec, "pct_hbm_roof": 100 * t_hbm / sec,
-               "bound": "mfma" if t_mfma >= t_hbm else "hbm", "flop": flop, "bytes": nbytes}
+               "bound": "mfma" if t_mfma >= t_hbm else "hbm", "frac": max(t_mfma, t_hbm) / sec,
+               "flop": flop, "bytes": nbytes}
         row["traffic_bytes"] = measured_traffic(row["kernel"])
         if cfg.pipeline == _lib.AMOS_PIPE_NCHW and not fused_tail and not launches:
             # the same convolution where the owner of the weights has packed them once
@@ -147,7 +175,7 @@ def run_all_configs(cpu=True, only=None, launches=None):
             res = (ctypes.c_double * 3)()
             _lib.check(lib.amos_time(op, ctypes.byref(desc), ctypes.byref(c2), tin[0].data_ptr(), packed.data_ptr(),
                                      out.data_ptr(), None, 0, None, 20, 3, 100, res))
-            row["gpu_us_weights_packed_once"] = min(res) * 1e6
+            row["gpu_us_weights_packed_once"] = sum(res) / len(res) * 1e6
             del packed
         if cpu and cpu_fn is not None:
             t1 = _timed(lambda: cpu_fn(1, False))
@@ -385,6 +413,10 @@ def main():
                     help="run only the configuration whose name contains this text (C2, C3 fp16, C4 int8, C5a, "
                          "C5b), --steps launches of it, print its row and exit: the command that the counter "
                          "summaries under profiles/ were made with")
+    ap.add_argument("--mfma-ceiling", action="store_true",
+                    help="only measure what the matrix cores sustain (amos_mfma_ceiling: both instruction shapes, "
+                         "constant and random operands, with and without the data movement of a 256x256x64 "
+                         "tiling), print the rows as JSON and exit")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a 256 MiB device copy, the known-size kernel that rocprofv3's "
                          "FETCH_SIZE / WRITE_SIZE readings are scaled by")
@@ -398,6 +430,16 @@ def main():
     from amos_amd import _lib, ops
     if not torch.cuda.is_available():
         sys.exit("bench.py needs a GPU")
+    if args.mfma_ceiling:
+        g = torch.Generator(device="cuda").manual_seed(0)
+        da = (torch.rand((8192, 8192), device="cuda", generator=g) * 2 - 1).half()
+        db = (torch.rand((8192, 8192), device="cuda", generator=g) * 2 - 1).half()
+        # (the clock settles under load: two passes, the second one is reported)
+        variants = [(32, 0, 0, 0), (32, 1, 0, 0), (16, 0, 0, 0), (16, 1, 0, 0), (32, 1, 1, 0), (32, 1, 0, 1),
+                    (32, 1, 1, 1), (16, 1, 1, 1), (32, 0, 1, 1)]
+        mfma_ceiling(da, db, variants, launches=20, repeats=1)
+        print(json.dumps(mfma_ceiling(da, db, variants, launches=20, repeats=3), indent=1))
+        return
     if args.config:
         if args.calibrate_copy:
             src = torch.empty(256 << 20, dtype=torch.uint8, device="cuda").random_()
@@ -449,6 +491,10 @@ def main():
     per_launch = ops.time_op(_lib.AMOS_OP_GEMM, desc, da, db, dc, config=cfg, number=args.steps,
                              repeat=1, min_repeat_ms=0)[0]
     achieved = flop / per_launch / 1e12
+    # what the matrix cores sustain on this box with the benchmark's operand values and nothing in
+    # their way (amos_mfma_ceiling, the kernel's own instruction shape), right behind the timed
+    # steps so that the chip is at the same clock
+    sustained = mfma_ceiling(da, db, [(16, 1, 0, 0)], launches=20, repeats=2)[0]["tflops"]
     line = {
         "metric": METRIC, "value": value, "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps,
         "warmup": args.warmup, "ms_per_step": ms_per_step, "higher_is_better": True,
@@ -462,7 +508,10 @@ def main():
         "roofline": {"bound": "mfma", "achieved": achieved, "peak": PEAK_F16_TFLOPS,
                      "unit": "TFLOP/s", "frac": achieved / PEAK_F16_TFLOPS,
                      "traffic": measured_traffic(ops.kernel_name(_lib.AMOS_OP_GEMM, desc, cfg)),
-                     "kernel_us": per_launch * 1e6},
+                     "kernel_us": per_launch * 1e6,
+                     "sustained_peak": sustained, "frac_of_sustained_peak": achieved / sustained,
+                     "sustained_peak_note": "amos_mfma_ceiling: v_mfma_f32_16x16x32_f16 on random fp16 U[-1,1] "
+                                            "operands, no memory traffic, same run (python bench.py --mfma-ceiling)"},
     }
     if not args.no_cpu:
         line["cpu_baseline"] = cpu_baseline_gemm(a, b)
@@ -475,14 +524,14 @@ def main():
                    "gpu_us": per_launch * 1e6, "tflops": achieved,
                    "pct_mfma_peak": 100 * achieved / PEAK_F16_TFLOPS,
                    "pct_hbm_roof": 100 * (2 * n * n * 2 + n * n * 4) / (PEAK_HBM_GBS * 1e9) / per_launch,
-                   "bound": "mfma"}]
+                   "bound": "mfma", "frac": achieved / PEAK_F16_TFLOPS}]
         if "cpu_baseline" in line:
             cb = line["cpu_baseline"]
             per_op[0]["cpu"] = {"threads1_tflops": cb["value"], "threadsN_tflops": cb["all_cores"]["value"],
                                 "cores": cb["all_cores"]["cores"], "extrapolated_from": cb["sample"].split("=")[-1]}
         for r in run_all_configs(cpu=not args.no_cpu, only=("C3 fp16", "C4 int8", "C5a fp16", "C5b fp16")):
             row = {k: r[k] for k in ("config", "kernel", "split_k", "gpu_us", "tflops", "pct_mfma_peak",
-                                     "pct_hbm_roof", "bound")}
+                                     "pct_hbm_roof", "bound", "frac")}
             for k in ("traffic_bytes", "gpu_us_weights_packed_once"):
                 if r.get(k) is not None:
                     row[k] = r[k]
@@ -491,9 +540,10 @@ def main():
                                                        "extrapolated_from")}
             per_op.append(row)
         per_op[0]["traffic_bytes"] = line["roofline"]["traffic"]
-        line["config"]["per_op"] = per_op
-        line["config"]["per_op_note"] = ("gpu_us: mean seconds per call by HIP events (time_evaluator loop), every "
-                                         "launch of a call included; tflops: TFLOP/s (int8: TOP/s); cpu: the "
+        line["per_op"] = per_op
+        line["per_op_note"] = ("gpu_us: mean seconds per call by HIP events (time_evaluator loop, mean over "
+                                         "its repeats), every launch of a call included; frac: fraction of the roof "
+                                         "that binds (bound); tflops: TFLOP/s (int8: TOP/s); cpu: the "
                                          "te_literal loop nest (gcc -O3) on a slab, scaled linearly; traffic_bytes: HBM-side "
                                          "bytes per launch of the main kernel from the counter summaries under profiles/; "
                                          "gpu_us_weights_packed_once: the same convolution where the owner of the weights "

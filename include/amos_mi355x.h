@@ -337,6 +337,28 @@ int amos_eltwise(const amos_eltwise_desc_t* desc, const void* const* inputs, voi
 int amos_time_eltwise(const amos_eltwise_desc_t* desc, const void* const* inputs, void* out, void* stream,
                       int number, int repeat, int min_repeat_ms, double* out_seconds);
 
+/*
+ * What the matrix cores sustain on this device when nothing else limits them: `launches`
+ * back-to-back launches of a measurement kernel with the matrix-core instruction stream of the
+ * 8192^3 fp16 product (256 workgroups x 4 waves, 1.0995e12 flop per launch) and no wait or barrier
+ * anywhere; mean seconds per launch by HIP events on `stream` and the flop of a launch are
+ * written out.  Synchronises the stream.
+ *   shape            16: v_mfma_f32_16x16x32_f16, 32: v_mfma_f32_32x32x16_f16
+ *   random_operands  0: small constants built in registers; 1: the operands of the instructions are
+ *                    read (once) from a and b -- the switching activity of the multipliers, and
+ *                    with it the clock the chip holds, depends on the operand values
+ *   copies / reads   add the global -> LDS copies (64 KB per K step and workgroup) / the LDS
+ *                    fragment reads (32 x 16 bytes per lane and K step) of a 256x256x64 tiling
+ * a, b: device buffers of operand_bytes each, 16-byte aligned: at least 8 MiB, with copies an
+ * [8192][8192] fp16 matrix (128 MiB); sink: 1 KiB of device memory (never written for finite
+ * operands).  The reference has no counterpart: it reports seconds per call
+ * (python/tvm/auto_tensorize/search/measure.py:175-207) and leaves the peak to its reader; the
+ * benchmark here reports this figure next to the published peak.
+ */
+int amos_mfma_ceiling(int shape, int random_operands, int copies, int reads, const void* a, const void* b,
+                      size_t operand_bytes, void* sink, int launches, void* stream, double* out_seconds,
+                      double* out_flop);
+
 /* name of the kernel instance a (desc, cfg) pair dispatches to, e.g.
  * "amos_igemm<f16,vec,vec,256x256>"; replaces func.imported_modules[0].get_source()
  * as the way to see what was chosen (reference: README.md:340). */

@@ -125,3 +125,47 @@ def test_split_k_without_the_workspace(gpu):
     tn = ops.make_config(dict(tile_i=128, tile_j=128, split_k=4, pipeline=3))
     rc = lib.amos_gemm(ctypes.byref(d), ctypes.byref(tn), a.data_ptr(), b.data_ptr(), out.data_ptr(), None, 0, None)
     assert rc in (_lib.AMOS_ERR_WORKSPACE, _lib.AMOS_ERR_INFEASIBLE), lib.amos_last_error()
+
+
+@pytest.mark.parametrize("extra", [0, 64 << 20])
+def test_split_k_slices_stay_clear_of_the_copy_of_a_misaligned_operand(gpu, extra):
+    """A 2-byte offset A makes the plan copy A as well as the row-major B, which
+    amos_workspace_bytes() (aligned operands) does not count: the slices of the partial sums must
+    start behind BOTH copies, whatever the size of the workspace the caller brings."""
+    from amos_amd import _lib, ops
+    lib = _lib.load()
+    torch.manual_seed(6)
+    M = N = K = 2048
+    abuf = torch.randn(M * K + 8, device="cuda").half()
+    a = abuf[1:1 + M * K].view(M, K)
+    assert a.data_ptr() % 16 == 2
+    b = torch.randn(K, N, device="cuda").half()
+    d = ops.gemm_desc(M, N, K, torch.float16, False, False)
+    cfg = ops.make_config(dict(tile_i=128, tile_j=128, split_k=2))
+    need = lib.amos_workspace_bytes(_lib.AMOS_OP_GEMM, ctypes.byref(d), ctypes.byref(cfg))
+    ws = torch.empty(need + extra, dtype=torch.uint8, device="cuda")
+    ref = (a.double() @ b.double()).cpu().numpy()
+    outs = []
+    for _ in range(3):
+        out = torch.empty(M, N, device="cuda")
+        _lib.check(lib.amos_gemm(ctypes.byref(d), ctypes.byref(cfg), a.data_ptr(), b.data_ptr(), out.data_ptr(),
+                                 ws.data_ptr(), ws.numel(), None))
+        torch.cuda.synchronize()
+        outs.append(out)
+        mx, mean = _rel(out.cpu().numpy(), ref)
+        assert mx <= MAX_REL and mean <= MEAN_REL, "max_rel %.3e mean_rel %.3e" % (mx, mean)
+    if extra:   # room for the slices behind both copies: the deterministic reduction runs
+        assert torch.equal(outs[0], outs[1]) and torch.equal(outs[0], outs[2])
+
+
+def test_batched_split_k_reduces_every_batch_in_one_launch(gpu):
+    """direct-to-LDS batched product with a split: one reduction launch walks all batches"""
+    from amos_amd import ops
+    torch.manual_seed(7)
+    a = torch.randn(5, 128, 1024, device="cuda").half()
+    b = torch.randn(5, 136, 1024, device="cuda").half()
+    cfg = dict(tile_i=128, tile_j=128, split_k=4, pipeline=3)
+    got = _repeat_equal(lambda: ops.bgemm(a, b, False, True, config=cfg))
+    ref = torch.bmm(a.double(), b.double().transpose(1, 2))
+    mx, mean = _rel(got.cpu().numpy(), ref.cpu().numpy())
+    assert mx <= MAX_REL and mean <= MEAN_REL
