@@ -271,7 +271,6 @@ __global__ __launch_bounds__(64 * (WI * WJ + NWL)) void amos_conv_nchw(const Con
     constexpr int SBASE = NWM + NWL == 12 ? 136 : NWM + NWL == 8 ? 224 : -1;
     static_assert(SBASE > 0, "workgroups of eight or twelve waves");
     typedef unsigned nchw_ul __attribute__((ext_vector_type(LW)));
-    nchw_ul praw[PTL][CG];
 
     // weights that pass through registers: the raw taps of this thread's unit
     auto load_weights = [&](int m) __attribute__((always_inline)) {
@@ -327,10 +326,18 @@ __global__ __launch_bounds__(64 * (WI * WJ + NWL)) void amos_conv_nchw(const Con
 
     const NchwTile tile = nchw_tile(s, bj0, BJ);
     // ---- this thread's load groups of the patch ------------------------------------------------
+    // First what the loads need (a wave issues an instruction every five to seven cycles when it
+    // is alone on its SIMD, every nine to seventeen next to two waves of matrix-core work: the
+    // length of this stretch is the time to the first load), then the loads, then -- while they
+    // are on their way -- where the positions go in LDS.
     unsigned p_src[PTL];      // byte offset of (image, first channel of the chunk, depth 0, group): below 4 GiB
     int p_d0[PTL];            // input depth at depth tap 0
     unsigned p_dst[PTL][PG];  // LDS addresses (first buffer) of the group's positions; the dump line
                               // for positions that are not part of the window
+    const unsigned plane_bytes = (unsigned)(DHW * ES);
+    // byte selectors that pick position i (lower half of the wave) or i ^ 1 (upper half) out of a
+    // staging dword: 16-bit types hold two positions per dword, int8 four
+    unsigned p_sel[ES == 2 ? 2 : 4];
 #pragma unroll
     for (int v = 0; v < PTL; ++v) {
       const int q = tlp + NTP * v;
@@ -340,32 +347,24 @@ __global__ __launch_bounds__(64 * (WI * WJ + NWL)) void amos_conv_nchw(const Con
       const NchwSeg seg = nchw_group(s, tile, on ? grp : 0, &f);
       p_src[v] = (unsigned)((((int64_t)seg.n * s.C + cg * CG) * DHW + f) * ES);
       p_d0[v] = seg.d0;
-#pragma unroll
-      for (int i = 0; i < PG; ++i) {
-        // (the upper half of a wave stores its positions in the order 1, 0, 3, 2, ...: see the bank
-        // conflict notes of the geometry header)
-        const int off = on ? nchw_writer_offset(s, seg, f + (i ^ (lane >> 5)), cg) : -1;
-        p_dst[v][i] = PBASE + (off >= 0 ? (unsigned)off : DUMP + (unsigned)lane * 16);
-      }
     }
-    // byte selectors that pick position i (lower half of the wave) or i ^ 1 (upper half) out of a
-    // staging dword: 16-bit types hold two positions per dword, int8 four
-    unsigned p_sel[ES == 2 ? 2 : 4];
-#pragma unroll
-    for (int i = 0; i < (ES == 2 ? 2 : 4); ++i) {
-      const int pos = i ^ (lane >> 5);
-      p_sel[i] = ES == 2 ? (pos ? 0x07060302u : 0x05040100u) : ((unsigned)pos | ((unsigned)(4 + pos) << 8));
-    }
-    // the patch loads of macro step m.  Every lane loads, from a depth clamped into the tensor (a
-    // depth in the padding is zeroed when the vector is stored, lanes without a group store into
-    // the dump line).
 #define AMOS_NCHW_S136 "v136", "v137", "v138", "v139", "v140", "v141", "v142", "v143", "v144", "v145", "v146", "v147", "v148", "v149", "v150", "v151", \
                        "v152", "v153", "v154", "v155", "v156", "v157", "v158", "v159", "v160", "v161", "v162", "v163", "v164", "v165", "v166", "v167"
 #define AMOS_NCHW_S224 "v224", "v225", "v226", "v227", "v228", "v229", "v230", "v231", "v232", "v233", "v234", "v235", "v236", "v237", "v238", "v239", \
                        "v240", "v241", "v242", "v243", "v244", "v245", "v246", "v247", "v248", "v249", "v250", "v251", "v252", "v253", "v254", "v255"
-    auto load_patch = [&](int m) __attribute__((always_inline)) {
+    // the patch loads of macro step m.  Every lane loads, from a depth clamped into the tensor (a
+    // depth in the padding stores zeros instead, lanes without a group store into the dump line).
+    // One scalar base per macro step (the chunk of channels), per load the lane's offset plus the
+    // channel's plane: two instructions a load.
+    // Where a macro step's loads take half of the staging registers or less there are two sets: the
+    // loads of macro step m + 2 go out (into the other set) BEFORE macro step m + 1 is transposed
+    // out of its set, a transposition longer on their way; else one set, and the loads follow the
+    // permutes that read it.
+    constexpr bool TWO_SETS = NAG <= 16 && PACKED;   // (unpacked weights: their loads go first, measured)
+    auto load_patch = [&](auto set_c, int m) __attribute__((always_inline)) {
+      constexpr int SB = SBASE + (TWO_SETS ? decltype(set_c)::value * 16 : 0);
       const int tt = nchw_div(m, p.div_cc), cc = m - tt * p.c_chunks;
-      const char* const xm0 = p.x + (int64_t)cc * CK * DHW * ES;
+      const char* const base = nchw_uniform(p.x + (int64_t)cc * CK * DHW * ES);
       nchw_static_for<0, PTL>([&](auto v_c) {
         constexpr int v = decltype(v_c)::value;
         int d = p_d0[v] + tt * s.dd;
@@ -373,83 +372,122 @@ __global__ __launch_bounds__(64 * (WI * WJ + NWL)) void amos_conv_nchw(const Con
         // (the depth is the lane's own: its offset stays below 4 GiB like the rest of the tensor)
         const unsigned off_v = p_src[v] + (unsigned)d * (unsigned)(HW * ES);
         nchw_static_for<0, CG>([&](auto ci_c) {
-          constexpr int ci = decltype(ci_c)::value, r0 = SBASE + (v * CG + ci) * LW;
-          const char* const plane = nchw_uniform(xm0 + (int64_t)ci * DHW * ES);
-          const unsigned off = off_v;
-          // (five wait states between the v_readfirstlane that made the address and its use)
-          if constexpr (LB == 16 && SBASE == 136)
-            asm volatile("s_nop 4\n\tglobal_load_dwordx4 v[%2:%3], %0, %1" ::"v"(off), "s"(plane), "n"(r0), "n"(r0 + 3) : "memory", AMOS_NCHW_S136);
-          else if constexpr (LB == 16)
-            asm volatile("s_nop 4\n\tglobal_load_dwordx4 v[%2:%3], %0, %1" ::"v"(off), "s"(plane), "n"(r0), "n"(r0 + 3) : "memory", AMOS_NCHW_S224);
-          else if constexpr (SBASE == 136)
-            asm volatile("s_nop 4\n\tglobal_load_dwordx2 v[%2:%3], %0, %1" ::"v"(off), "s"(plane), "n"(r0), "n"(r0 + 1) : "memory", AMOS_NCHW_S136);
-          else
-            asm volatile("s_nop 4\n\tglobal_load_dwordx2 v[%2:%3], %0, %1" ::"v"(off), "s"(plane), "n"(r0), "n"(r0 + 1) : "memory", AMOS_NCHW_S224);
+          constexpr int ci = decltype(ci_c)::value, r0 = SB + (v * CG + ci) * LW;
+          const unsigned off = off_v + (unsigned)ci * plane_bytes;
+          const char* const plane = base;
+          // (five wait states between the v_readfirstlane that may have made the base and its first
+          // use; the compiler cannot insert them inside a statement)
+#define AMOS_NCHW_LOAD(width, last, clobbers)                                                                                   \
+  if constexpr (v == 0 && ci == 0)                                                                                              \
+    asm volatile("s_nop 4\n\tglobal_load_" width " v[%2:%3], %0, %1" ::"v"(off), "s"(plane), "n"(r0), "n"(r0 + last) : "memory", clobbers); \
+  else                                                                                                                          \
+    asm volatile("global_load_" width " v[%2:%3], %0, %1" ::"v"(off), "s"(plane), "n"(r0), "n"(r0 + last) : "memory", clobbers)
+          if constexpr (LB == 16 && SBASE == 136) { AMOS_NCHW_LOAD("dwordx4", 3, AMOS_NCHW_S136); }
+          else if constexpr (LB == 16) { AMOS_NCHW_LOAD("dwordx4", 3, AMOS_NCHW_S224); }
+          else if constexpr (SBASE == 136) { AMOS_NCHW_LOAD("dwordx2", 1, AMOS_NCHW_S136); }
+          else { AMOS_NCHW_LOAD("dwordx2", 1, AMOS_NCHW_S224); }
+#undef AMOS_NCHW_LOAD
         });
       });
     };
-    // every load of this wave has landed (the compiler's own loads of unpacked weights too); the
-    // patch loads move into ordinary registers
-    auto landed = [&]() __attribute__((always_inline)) {
-      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-      nchw_static_for<0, PTL * CG>([&](auto u_c) {
-        constexpr int u = decltype(u_c)::value;
-        nchw_static_for<0, LW>([&](auto k_c) {
-          constexpr int k = decltype(k_c)::value;
-          unsigned x;
-          asm volatile("v_mov_b32 %0, v[%1]" : "=v"(x) : "n"(SBASE + u * LW + k));
-          praw[u / CG][u % CG][k] = x;
-        });
-      });
-    };
-    // the patch of macro step m out of the registers into patch buffer BUF: per position one
-    // 16-byte vector of channels
-    auto store_patch = [&](auto buf_c, int m) __attribute__((always_inline)) {
+    // every load of this wave has landed (the compiler's own loads of unpacked weights too)
+    auto landed = [&]() __attribute__((always_inline)) { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); };
+    // dword `k` of channel `c` of load group `v`, out of the staging registers, as an operand of
+    // an assembly statement: "v[n]"
+    // The patch of macro step m out of the staging registers into patch buffer BUF: per position
+    // one 16-byte vector of channels.  The byte permutes read the staging registers where the
+    // loads left them (assembly: the compiler does not know these registers), so the next loads
+    // go out behind them.  A group whose depth lies in the padding stores zeros.
+    auto store_patch = [&](auto buf_c, auto set_c, int m) __attribute__((always_inline)) {
+      constexpr int SB = SBASE + (TWO_SETS ? decltype(set_c)::value * 16 : 0);
       const int tt = nchw_div(m, p.div_cc);
-#pragma unroll
-      for (int v = 0; v < PTL; ++v) {
+      nchw_static_for<0, PTL>([&](auto v_c) {
+        constexpr int v = decltype(v_c)::value;
         const bool ok = (unsigned)(p_d0[v] + tt * s.dd) < (unsigned)s.D;
+        if (ok) {
+          nchw_static_for<0, PG>([&](auto i_c) {
+            constexpr int i = decltype(i_c)::value;
+            unsigned o[4];
+            nchw_static_for<0, 4>([&](auto j_c) {
+              constexpr int j = decltype(j_c)::value;
+              if constexpr (ES == 2) {
+                const unsigned sel = p_sel[i & 1];
+                unsigned x;   // (an assembly operand cannot name a variable of an enclosing lambda)
+                asm volatile("v_perm_b32 %0, v[%1], v[%2], %3" : "=v"(x)
+                             : "n"(SB + (v * CG + 2 * j + 1) * LW + (i >> 1)), "n"(SB + (v * CG + 2 * j) * LW + (i >> 1)), "v"(sel));
+                o[j] = x;
+              } else {
+                const unsigned sel = p_sel[i & 3];
+                unsigned lo, hi;
+                asm volatile("v_perm_b32 %0, v[%1], v[%2], %3" : "=v"(lo)
+                             : "n"(SB + (v * CG + 4 * j + 1) * LW + (i >> 2)), "n"(SB + (v * CG + 4 * j) * LW + (i >> 2)), "v"(sel));
+                asm volatile("v_perm_b32 %0, v[%1], v[%2], %3" : "=v"(hi)
+                             : "n"(SB + (v * CG + 4 * j + 3) * LW + (i >> 2)), "n"(SB + (v * CG + 4 * j + 2) * LW + (i >> 2)), "v"(sel));
+                o[j] = __builtin_amdgcn_perm(hi, lo, 0x05040100u);
+              }
+            });
+            *(v4i*)AMOS_LDS_ADDR(p_dst[v][i] + decltype(buf_c)::value * PBUF) = v4i{(int)o[0], (int)o[1], (int)o[2], (int)o[3]};
+          });
+        } else {
 #pragma unroll
-        for (int i = 0; i < PG; ++i) {
-          v4i o;
-#pragma unroll
-          for (int j = 0; j < 4; ++j) {
-            if constexpr (ES == 2) {
-              o[j] = (int)__builtin_amdgcn_perm(praw[v][2 * j + 1][i >> 1], praw[v][2 * j][i >> 1], p_sel[i & 1]);
-            } else {
-              const unsigned sel = p_sel[i & 3];
-              const unsigned lo = __builtin_amdgcn_perm(praw[v][4 * j + 1][i >> 2], praw[v][4 * j][i >> 2], sel);
-              const unsigned hi = __builtin_amdgcn_perm(praw[v][4 * j + 3][i >> 2], praw[v][4 * j + 2][i >> 2], sel);
-              o[j] = (int)__builtin_amdgcn_perm(hi, lo, 0x05040100u);
-            }
-          }
-          if (!ok) o = v4i{0, 0, 0, 0};
-          *(v4i*)AMOS_LDS_ADDR(p_dst[v][i] + decltype(buf_c)::value * PBUF) = o;
+          for (int i = 0; i < PG; ++i) *(v4i*)AMOS_LDS_ADDR(p_dst[v][i] + decltype(buf_c)::value * PBUF) = v4i{0, 0, 0, 0};
         }
-      }
+      });
     };
 
-    // ---- prologue: macro step m_begin into the first buffers, the loads of the next one out ------
+    // ---- prologue: the first loads, then the rest of the set-up while they are on their way -------
     // (every blockIdx.y has at least one macro step: the host checks that)
-    load_patch(m_begin);
+    load_patch(NchwSet<0>{}, m_begin);
+    {
+      // (the thread index passes through an empty assembly statement: what depends on it stays
+      // behind the loads instead of being merged with the arithmetic in front of them)
+      int tl2 = tlp;
+      asm volatile("" : "+v"(tl2));
+      const int hi_half = (tl2 >> 5) & 1;
+#pragma unroll
+      for (int i = 0; i < (ES == 2 ? 2 : 4); ++i) {
+        const int pos = i ^ hi_half;
+        p_sel[i] = ES == 2 ? (pos ? 0x07060302u : 0x05040100u) : ((unsigned)pos | ((unsigned)(4 + pos) << 8));
+      }
+#pragma unroll
+      for (int v = 0; v < PTL; ++v) {
+        const int q = tl2 + NTP * v;
+        const int cg = q & 3, grp = q >> 2;
+        const bool on = grp < tile.ngroups;
+        int f = 0;
+        const NchwSeg seg = nchw_group(s, tile, on ? grp : 0, &f);
+#pragma unroll
+        for (int i = 0; i < PG; ++i) {
+          // (the upper half of a wave stores its positions in the order 1, 0, 3, 2, ...: see the bank
+          // conflict notes of the geometry header)
+          const int off = on ? nchw_writer_offset(s, seg, f + (i ^ hi_half), cg) : -1;
+          p_dst[v][i] = PBASE + (off >= 0 ? (unsigned)off : DUMP + (unsigned)(tl2 & 63) * 16);
+        }
+      }
+    }
     clear_patches();
     meet();
     landed();
     // (unpacked weights first: the compiler waits for its own loads in front of their first use, and
     // that wait would take the patch loads behind it along)
     if constexpr (!PACKED) store_weights(NchwSet<0>{});
-    if (m_begin + 1 < m_end) load_patch(m_begin + 1);
-    store_patch(NchwSet<0>{}, m_begin);
+    if (TWO_SETS && m_begin + 1 < m_end) load_patch(NchwSet<1>{}, m_begin + 1);
+    store_patch(NchwSet<0>{}, NchwSet<0>{}, m_begin);
+    if (!TWO_SETS && m_begin + 1 < m_end) load_patch(NchwSet<1>{}, m_begin + 1);
     meet();
     // ---- under macro step m of the matrix-core waves: macro step m + 1 into the other buffers
-    // (last read a macro step ago) while the loads of m + 2 are on their way
+    // (last read a macro step ago), then the loads of m + 2 go out.  Unpacked weights: their loads
+    // are on their way while the patch is transposed.
     auto under = [&](auto buf_c, int m) __attribute__((always_inline)) {
+      // (buffer and staging set of macro step m_begin + r: r & 1)
+      constexpr int BUF = decltype(buf_c)::value;
       if (m + 1 < m_end) {
-        if constexpr (!PACKED) load_weights(m + 1);
         landed();
+        if (TWO_SETS && m + 2 < m_end) load_patch(NchwSet<BUF ^ 1>{}, m + 2);
+        if constexpr (!PACKED) load_weights(m + 1);
+        store_patch(buf_c, buf_c, m + 1);
         if constexpr (!PACKED) store_weights(buf_c);
-        if (m + 2 < m_end) load_patch(m + 2);
-        store_patch(buf_c, m + 1);
+        if (!TWO_SETS && m + 2 < m_end) load_patch(NchwSet<BUF ^ 1>{}, m + 2);
       }
       meet();
     };
@@ -553,6 +591,20 @@ __global__ __launch_bounds__(64 * (WI * WJ + NWL)) void amos_conv_nchw(const Con
       for (int a = 0; a < TI; ++a) acc[a][b] = MM::run(af[slot][a], bf[slot][b], acc[a][b]);
   };
 
+  // Every address is worked out HERE, while the loaders' first loads are on their way: left to
+  // itself the compiler sinks this arithmetic (some 150 instructions, a wave's instructions issue
+  // 5-7 cycles apart) behind the barriers to its first use, into the one stretch of the
+  // kernel where the loaders have delivered and every other wave waits for the first result.
+#pragma unroll
+  for (int a = 0; a < TI; ++a) asm volatile("" : "+v"(a_addr[0][a]), "+v"(a_addr[1][a]));
+#pragma unroll
+  for (int b = 0; b < TJ; ++b)
+#pragma unroll
+    for (int tap = 0; tap < RS; ++tap) asm volatile("" : "+v"(b_addr[tap][b]));
+#pragma unroll
+  for (int a = 0; a < TI; ++a)
+#pragma unroll
+    for (int b = 0; b < TJ; ++b) asm volatile("" : "+v"(acc[a][b]));
   clear_patches();
   meet();
   if (PACKED) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // the first macro step's weights
@@ -562,8 +614,7 @@ __global__ __launch_bounds__(64 * (WI * WJ + NWL)) void amos_conv_nchw(const Con
   auto macro_step = [&](auto buf_c, int m) __attribute__((always_inline)) {
     constexpr int BUF = decltype(buf_c)::value;
     if (PACKED && m + 1 < m_end) copy_weights(NchwSet<BUF ^ 1>{}, m + 1);
-    read_frags(buf_c, NchwSet<0>{});
-    if (NF > 2) read_frags(buf_c, NchwSet<1>{});
+    nchw_static_for<0, NF - 1>([&](auto tap_c) { read_frags(buf_c, tap_c); });
     __builtin_amdgcn_sched_barrier(0);
     nchw_static_for<0, RS>([&](auto tap_c) {
       constexpr int tap = decltype(tap_c)::value;
@@ -586,6 +637,43 @@ __global__ __launch_bounds__(64 * (WI * WJ + NWL)) void amos_conv_nchw(const Con
   out_t* const out = (out_t*)p.y + (int64_t)blockIdx.y * p.split_stride;
   const int ODPQ = s.OD * s.OP * s.OQ;
   const bool add_d = p.epi.dt != EPI_NONE && blockIdx.y == 0;
+  // Where four consecutive output positions are one aligned 16-byte run of the result (an image's
+  // positions a multiple of four, the tensor 16-byte aligned) and there is no fused tail, a 16-row
+  // block of the wave tile goes through an LDS strip of the wave (the operand buffers are free
+  // behind the last barrier; LDS operations of one wave complete in issue order, so the strip needs
+  // no barrier of its own) and leaves as 16-byte stores that cover whole rows of the wave tile:
+  // 64 / (4 TJ) rows x 64 TJ bytes per instruction instead of four rows x 64 bytes.
+  constexpr int SP = TJ * 16 + 4;                 // strip row pitch in elements
+  constexpr int CPR = TJ * 4, RPI = 64 / CPR;     // 16-byte chunks per row, rows per store instruction
+  static_assert((TJ & (TJ - 1)) == 0 && TJ <= 16 && NWM * 16 * SP * 4 <= 2 * WBUF, "output strip");
+  const bool strips = !add_d && (ODPQ & 3) == 0 && (((uintptr_t)out) & 15) == 0;
+  if (strips) {
+    out_t* const strip = (out_t*)AMOS_LDS_ADDR(wave * (16 * SP * 4));
+    // this lane's four positions of the wave tile's row: one image, one 16-byte run
+    const int j4 = bj0 + wj * TJ * 16 + (lane % CPR) * 4;
+    const int jc = j4 < s.J ? j4 : 0;
+    const int n = nchw_div(jc, p.div_odpq);
+    const int64_t coff = (int64_t)n * s.K * ODPQ + (jc - n * ODPQ);
+#pragma unroll
+    for (int a = 0; a < TI; ++a) {
+#pragma unroll
+      for (int b = 0; b < TJ; ++b)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) strip[(4 * frag_q + r) * SP + b * 16 + frag_row] = acc[a][b][r];
+      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+      acc_t v[TJ];
+#pragma unroll
+      for (int x = 0; x < TJ; ++x) v[x] = *(const acc_t*)(strip + (x * RPI + lane / CPR) * SP + (lane % CPR) * 4);
+      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+#pragma unroll
+      for (int x = 0; x < TJ; ++x) {
+        const int i = bi0 + (wi * TI + a) * 16 + x * RPI + lane / CPR;
+        // (J is a multiple of four here: the four positions are inside the tensor together)
+        if (i < s.K && j4 < s.J) *(acc_t*)(out + coff + (int64_t)i * ODPQ) = v[x];
+      }
+    }
+    return;
+  }
 #pragma unroll
   for (int b = 0; b < TJ; ++b) {
     const int j = bj0 + (wj * TJ + b) * 16 + frag_row;
