@@ -1224,7 +1224,7 @@ static int launch_conv_nchw(const Plan& pl, hipStream_t stream) {
   // what the kernel assumes of its launch: the tile of the instance, whole 64-byte chunks of
   // channels, a patch that fits the LDS asked for
   // ... and at least one macro step for every block along the reduction
-  if (inst->bi != pl.cfg.tile_i || inst->bj != pl.cfg.tile_j || q.c_chunks < 1 || q.max_pos < 4 ||
+  if (inst->bi * inst->halves != pl.cfg.tile_i || inst->bj != pl.cfg.tile_j || q.c_chunks < 1 || q.max_pos < 4 ||
       q.macro_per_split < 1 || pl.split < 1 || (int64_t)(pl.split - 1) * q.macro_per_split >= q.macro_steps ||
       q.max_pos > nchw_max_positions(inst->bj) ||
       pl.nchw_lds != (size_t)2 * 9 * inst->bi * 64 + (size_t)2 * nchw_patch_buffer_bytes(inst->bj) ||

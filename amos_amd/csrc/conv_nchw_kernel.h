@@ -172,7 +172,14 @@ constexpr int nchw_max_positions(int bj) { return nchw_patch_buffer_bytes(bj) / 
 // store the operands of macro step m + 1 (their loads two macro steps ahead of their use) while
 // the WI x WJ matrix-core waves do nothing but read fragments of macro step m and multiply; the
 // two kinds meet at the one barrier per macro step.
-template <int DT, int BI, int BJ, int WI, int WJ, int PTL, int WMODE, int NWL, int LB>
+//
+// HV: halves of output channels.  With HV = 2 a workgroup computes 2 * BI output channels of its
+// positions: every macro step's patch serves two weight halves one after the other (sequence step
+// q = macro step * HV + half; the weight buffers alternate with q, the patch buffers with the
+// macro step), at twice the accumulators.  Half as many workgroups, each with one set-up, one
+// patch and one round of patch loads for twice the work: for shapes whose tiles would otherwise
+// take two rounds of the compute units with the second one half empty.
+template <int DT, int BI, int BJ, int WI, int WJ, int PTL, int WMODE, int NWL, int LB, int HV = 1>
 __global__ __launch_bounds__(64 * (WI * WJ + NWL)) void amos_conv_nchw(const ConvNchwParams p) {
   typedef Mfma16<DT> MM;
   typedef typename MM::acc_t acc_t;
@@ -215,13 +222,15 @@ __global__ __launch_bounds__(64 * (WI * WJ + NWL)) void amos_conv_nchw(const Con
     logical = x * per + (x < rem ? x : rem) + (wg >> 3);
   }
   const int tile_j = logical / p.tiles_i, tile_i = logical - tile_j * p.tiles_i;
-  const int bi0 = tile_i * BI, bj0 = tile_j * BJ;
+  const int bi0 = tile_i * BI * HV, bj0 = tile_j * BJ;
+  static_assert(HV == 1 || HV == 2, "one or two halves of output channels");
   const int HW = s.H * s.W;
   const int64_t DHW = (int64_t)s.D * HW;
   const int TRS = s.T * RS;
   const int m_begin = blockIdx.y * p.macro_per_split;
   int m_end = m_begin + p.macro_per_split;
   if (m_end > p.macro_steps) m_end = p.macro_steps;
+  const int nq = (m_end - m_begin) * HV;   // sequence steps: (macro step, half of the output channels)
 
   // both kinds of waves: clear the patch buffers (padding positions are never written), meet
   auto clear_patches = [&]() __attribute__((always_inline)) {
@@ -240,7 +249,7 @@ __global__ __launch_bounds__(64 * (WI * WJ + NWL)) void amos_conv_nchw(const Con
     constexpr int NTP = NTL;
     const int tlp = tl;
     // ---- this thread's share of the weights ----------------------------------------------------
-    unsigned w_src[1] = {0};   // byte offset of (row, first channel of the chunk): below 4 GiB
+    unsigned w_src[HV] = {0};  // byte offset of (row, first channel of the chunk) per half: below 4 GiB
     unsigned w_dst = 0;        // LDS address inside a tap's tile of the first buffer
     bool w_on = !PACKED;
     if (!PACKED) {
@@ -249,8 +258,11 @@ __global__ __launch_bounds__(64 * (WI * WJ + NWL)) void amos_conv_nchw(const Con
       // (lanes 4x .. 4x+3 of a wave take row nchw_row_of_slot(x) of their sixteen: no bank conflicts)
       const int cq = u & 3, row = ((u >> 6) * 16 + nchw_row_of_slot((u >> 2) & 15)) & (BI - 1);
       w_on = u >= 0;
-      const int k = bi0 + row < s.K ? bi0 + row : s.K - 1;
-      w_src[0] = (unsigned)((((int64_t)k * s.C + cq * CG) * TRS) * ES);
+#pragma unroll
+      for (int h = 0; h < HV; ++h) {
+        const int k = bi0 + h * BI + row < s.K ? bi0 + h * BI + row : s.K - 1;
+        w_src[h] = (unsigned)((((int64_t)k * s.C + cq * CG) * TRS) * ES);
+      }
       w_dst = (unsigned)nchw_position_offset(row, cq);
     }
     unsigned wraw[PACKED ? 1 : WRAW];
@@ -273,10 +285,10 @@ __global__ __launch_bounds__(64 * (WI * WJ + NWL)) void amos_conv_nchw(const Con
     typedef unsigned nchw_ul __attribute__((ext_vector_type(LW)));
 
     // weights that pass through registers: the raw taps of this thread's unit
-    auto load_weights = [&](int m) __attribute__((always_inline)) {
+    auto load_weights = [&](int m, auto half_c) __attribute__((always_inline)) {
       if (!w_on) return;
       const int tt = nchw_div(m, p.div_cc), cc = m - tt * p.c_chunks;
-      const char* const src = p.w + ((int64_t)cc * CK * TRS + tt * RS) * ES + w_src[0];
+      const char* const src = p.w + ((int64_t)cc * CK * TRS + tt * RS) * ES + w_src[decltype(half_c)::value];
       if (T1) {
 #pragma unroll
         for (int i = 0; i < 9; ++i) {
@@ -322,7 +334,7 @@ __global__ __launch_bounds__(64 * (WI * WJ + NWL)) void amos_conv_nchw(const Con
       }
     };
     // the first weights go out before the tile's geometry is worked out
-    if constexpr (!PACKED) load_weights(m_begin);
+    if constexpr (!PACKED) load_weights(m_begin, NchwSet<0>{});
 
     const NchwTile tile = nchw_tile(s, bj0, BJ);
     // ---- this thread's load groups of the patch ------------------------------------------------
@@ -475,27 +487,34 @@ __global__ __launch_bounds__(64 * (WI * WJ + NWL)) void amos_conv_nchw(const Con
     store_patch(NchwSet<0>{}, NchwSet<0>{}, m_begin);
     if (!TWO_SETS && m_begin + 1 < m_end) load_patch(NchwSet<1>{}, m_begin + 1);
     meet();
-    // ---- under macro step m of the matrix-core waves: macro step m + 1 into the other buffers
-    // (last read a macro step ago), then the loads of m + 2 go out.  Unpacked weights: their loads
-    // are on their way while the patch is transposed.
-    auto under = [&](auto buf_c, int m) __attribute__((always_inline)) {
-      // (buffer and staging set of macro step m_begin + r: r & 1)
-      constexpr int BUF = decltype(buf_c)::value;
-      if (m + 1 < m_end) {
-        landed();
-        if (TWO_SETS && m + 2 < m_end) load_patch(NchwSet<BUF ^ 1>{}, m + 2);
-        if constexpr (!PACKED) load_weights(m + 1);
-        store_patch(buf_c, buf_c, m + 1);
-        if constexpr (!PACKED) store_weights(buf_c);
-        if (!TWO_SETS && m + 2 < m_end) load_patch(NchwSet<BUF ^ 1>{}, m + 2);
+    // ---- under sequence step q of the matrix-core waves: step q + 1 into the other weight buffer
+    // and, where it starts a macro step, that macro step's patch into the other patch buffer (last
+    // read a macro step ago); then the loads of the macro step after that go out.  Unpacked
+    // weights: their loads are on their way while the patch is transposed.
+    // U = (q + 1) % (2 * HV): weight buffer U & 1, patch buffer and staging set (U / HV) & 1, half U % HV
+    auto under = [&](auto u_c, int q) __attribute__((always_inline)) {
+      constexpr int U = decltype(u_c)::value, WB = U & 1, PB = (U / HV) & 1, HALF = U % HV;
+      if (q + 1 < nq) {
+        const int m1 = m_begin + (q + 1) / HV;   // the macro step of sequence step q + 1
+        if constexpr (HALF == 0) {
+          landed();
+          if (TWO_SETS && m1 + 1 < m_end) load_patch(NchwSet<PB ^ 1>{}, m1 + 1);
+          if constexpr (!PACKED) load_weights(m1, NchwSet<0>{});
+          store_patch(NchwSet<PB>{}, NchwSet<PB>{}, m1);
+          if constexpr (!PACKED) store_weights(NchwSet<WB>{});
+          if (!TWO_SETS && m1 + 1 < m_end) load_patch(NchwSet<PB ^ 1>{}, m1 + 1);
+        } else if constexpr (!PACKED) {
+          load_weights(m1, NchwSet<HALF>{});
+          store_weights(NchwSet<WB>{});
+        }
       }
       meet();
     };
-    // macro step m_begin + r is computed from buffers r & 1; the loaders fill buffers (r + 1) & 1
-    for (int m = m_begin; m < m_end; m += 2) {
-      under(NchwSet<1>{}, m);
-      if (m + 1 < m_end) under(NchwSet<0>{}, m + 1);
-    }
+    for (int q = 0; q < nq; q += 2 * HV)
+      nchw_static_for<0, 2 * HV>([&](auto u_c) {
+        constexpr int u = decltype(u_c)::value;
+        if (q + u < nq) under(NchwSet<(u + 1) % (2 * HV)>{}, q + u);
+      });
 #undef AMOS_NCHW_S136
 #undef AMOS_NCHW_S224
     return;
@@ -517,18 +536,21 @@ __global__ __launch_bounds__(64 * (WI * WJ + NWL)) void amos_conv_nchw(const Con
   constexpr int TPR = NWM / NB;               // taps per round of the matrix-core waves' copies
   constexpr int NWC = (RS + TPR - 1) / TPR;
   const int wblock = wave % NB, wtap0 = wave / NB;
-  unsigned w_lane = 0;
+  unsigned w_lane[HV] = {0};
   if (PACKED) {
     int row16, cq;
     nchw_unit_of_slot(lane, &row16, &cq);
     const int row = wblock * 16 + row16;
-    const int k = bi0 + row < s.K ? bi0 + row : s.K - 1;
-    w_lane = (unsigned)(((int64_t)k * TRS * s.C) * ES + cq * 16);
+#pragma unroll
+    for (int h = 0; h < HV; ++h) {
+      const int k = bi0 + h * BI + row < s.K ? bi0 + h * BI + row : s.K - 1;
+      w_lane[h] = (unsigned)(((int64_t)k * TRS * s.C) * ES + cq * 16);
+    }
   }
-  auto copy_weights = [&](auto buf_c, int m) __attribute__((always_inline)) {
+  auto copy_weights = [&](auto buf_c, int m, auto half_c) __attribute__((always_inline)) {
     const int tt = nchw_div(m, p.div_cc), cc = m - tt * p.c_chunks;
     const char* const wm = p.w + ((int64_t)tt * RS * s.C + (int64_t)cc * CK) * ES;
-    const unsigned lane_off = w_lane;
+    const unsigned lane_off = w_lane[decltype(half_c)::value];
 #pragma unroll
     for (int i = 0; i < NWC; ++i) {
       const int tap = wtap0 + TPR * i;
@@ -541,7 +563,7 @@ __global__ __launch_bounds__(64 * (WI * WJ + NWL)) void amos_conv_nchw(const Con
     }
   };
   // the first weights go out before anything else
-  if (PACKED) copy_weights(NchwSet<0>{}, m_begin);
+  if (PACKED) copy_weights(NchwSet<0>{}, m_begin, NchwSet<0>{});
   const int wi = wave / WJ, wj = wave % WJ;
   const int frag_row = lane & 15, frag_q = lane >> 4;
   const NchwTile tile = nchw_tile(s, bj0, BJ);
@@ -565,30 +587,33 @@ __global__ __launch_bounds__(64 * (WI * WJ + NWL)) void amos_conv_nchw(const Con
       b_addr[tap][b] = PBASE + (unsigned)nchw_reader_offset(s, column, tap / 3, tap % 3, nchw_frag_chunk(frag_q));
   }
 
-  acc_t acc[TI][TJ];
+  acc_t acc[HV][TI][TJ];
 #pragma unroll
-  for (int a = 0; a < TI; ++a)
+  for (int h = 0; h < HV; ++h)
 #pragma unroll
-    for (int b = 0; b < TJ; ++b)
+    for (int a = 0; a < TI; ++a)
 #pragma unroll
-      for (int r = 0; r < 4; ++r) acc[a][b][r] = 0;
+      for (int b = 0; b < TJ; ++b)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) acc[h][a][b][r] = 0;
 
   // operand fragments are read NF - 1 taps ahead: a batch of LDS reads takes some 200 cycles to
   // come back, a tap's matrix-core work of a wave 64
   constexpr int NF = TI * TJ >= 8 ? 2 : 3;
   v4i af[NF][TI], bf[NF][TJ];
-  auto read_frags = [&](auto buf_c, auto tap_c) __attribute__((always_inline)) {
-    constexpr int BUF = decltype(buf_c)::value, tap = decltype(tap_c)::value, slot = tap % NF;
+  auto read_frags = [&](auto wb_c, auto pb_c, auto tap_c) __attribute__((always_inline)) {
+    constexpr int WB = decltype(wb_c)::value, PB = decltype(pb_c)::value, tap = decltype(tap_c)::value, slot = tap % NF;
 #pragma unroll
-    for (int a = 0; a < TI; ++a) af[slot][a] = *(const v4i*)AMOS_LDS_ADDR(a_addr[BUF][a] + tap * WTILE);
+    for (int a = 0; a < TI; ++a) af[slot][a] = *(const v4i*)AMOS_LDS_ADDR(a_addr[WB][a] + tap * WTILE);
 #pragma unroll
-    for (int b = 0; b < TJ; ++b) bf[slot][b] = *(const v4i*)AMOS_LDS_ADDR(b_addr[tap][b] + BUF * PBUF);
+    for (int b = 0; b < TJ; ++b) bf[slot][b] = *(const v4i*)AMOS_LDS_ADDR(b_addr[tap][b] + PB * PBUF);
   };
-  auto mma = [&](int slot) __attribute__((always_inline)) {
+  auto mma = [&](auto half_c, int slot) __attribute__((always_inline)) {
+    constexpr int h = decltype(half_c)::value;
 #pragma unroll
     for (int b = 0; b < TJ; ++b)
 #pragma unroll
-      for (int a = 0; a < TI; ++a) acc[a][b] = MM::run(af[slot][a], bf[slot][b], acc[a][b]);
+      for (int a = 0; a < TI; ++a) acc[h][a][b] = MM::run(af[slot][a], bf[slot][b], acc[h][a][b]);
   };
 
   // Every address is worked out HERE, while the loaders' first loads are on their way: left to
@@ -602,36 +627,41 @@ __global__ __launch_bounds__(64 * (WI * WJ + NWL)) void amos_conv_nchw(const Con
 #pragma unroll
     for (int tap = 0; tap < RS; ++tap) asm volatile("" : "+v"(b_addr[tap][b]));
 #pragma unroll
-  for (int a = 0; a < TI; ++a)
+  for (int h = 0; h < HV; ++h)
 #pragma unroll
-    for (int b = 0; b < TJ; ++b) asm volatile("" : "+v"(acc[a][b]));
+    for (int a = 0; a < TI; ++a)
+#pragma unroll
+      for (int b = 0; b < TJ; ++b) asm volatile("" : "+v"(acc[h][a][b]));
   clear_patches();
   meet();
   if (PACKED) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // the first macro step's weights
   meet();
-  // One macro step: nine taps out of buffers BUF, then the barrier behind which the loaders have
-  // the other buffers ready and may overwrite these
-  auto macro_step = [&](auto buf_c, int m) __attribute__((always_inline)) {
-    constexpr int BUF = decltype(buf_c)::value;
-    if (PACKED && m + 1 < m_end) copy_weights(NchwSet<BUF ^ 1>{}, m + 1);
-    nchw_static_for<0, NF - 1>([&](auto tap_c) { read_frags(buf_c, tap_c); });
+  // One sequence step: nine taps out of weight buffer U & 1 and patch buffer (U / HV) & 1 into the
+  // accumulators of half U % HV, then the barrier behind which the loaders have the next step's
+  // buffers ready and may overwrite what this one has read
+  auto seq_step = [&](auto u_c, int q) __attribute__((always_inline)) {
+    constexpr int U = decltype(u_c)::value, WB = U & 1, PB = (U / HV) & 1, HALF = U % HV;
+    constexpr int U1 = (U + 1) % (2 * HV);
+    if (PACKED && q + 1 < nq) copy_weights(NchwSet<(U1 & 1)>{}, m_begin + (q + 1) / HV, NchwSet<U1 % HV>{});
+    nchw_static_for<0, NF - 1>([&](auto tap_c) { read_frags(NchwSet<WB>{}, NchwSet<PB>{}, tap_c); });
     __builtin_amdgcn_sched_barrier(0);
     nchw_static_for<0, RS>([&](auto tap_c) {
       constexpr int tap = decltype(tap_c)::value;
       // (the order is pinned: left to itself the scheduler moves a tap's fragment reads next to
       // its matrix-core instructions, and every tap then waits for LDS)
-      if constexpr (tap + NF - 1 < RS) read_frags(buf_c, NchwSet<tap + NF - 1>{});
+      if constexpr (tap + NF - 1 < RS) read_frags(NchwSet<WB>{}, NchwSet<PB>{}, NchwSet<tap + NF - 1>{});
       __builtin_amdgcn_sched_barrier(0);
-      mma(tap % NF);
+      mma(NchwSet<HALF>{}, tap % NF);
       __builtin_amdgcn_sched_barrier(0);
     });
     if (PACKED) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // this wave's copies have landed
     meet();
-    };
-  for (int m = m_begin; m < m_end; m += 2) {
-    macro_step(NchwSet<0>{}, m);
-    if (m + 1 < m_end) macro_step(NchwSet<1>{}, m + 1);
-  }
+  };
+  for (int q = 0; q < nq; q += 2 * HV)
+    nchw_static_for<0, 2 * HV>([&](auto u_c) {
+      constexpr int u = decltype(u_c)::value;
+      if (q + u < nq) seq_step(u_c, q + u);
+    });
 
   // ---- epilogue: Y[(n * K + i) * ODPQ + s], a lane holds column j of rows 4 * frag_q + r ----------
   out_t* const out = (out_t*)p.y + (int64_t)blockIdx.y * p.split_stride;
@@ -655,11 +685,12 @@ __global__ __launch_bounds__(64 * (WI * WJ + NWL)) void amos_conv_nchw(const Con
     const int n = nchw_div(jc, p.div_odpq);
     const int64_t coff = (int64_t)n * s.K * ODPQ + (jc - n * ODPQ);
 #pragma unroll
-    for (int a = 0; a < TI; ++a) {
+    for (int ha = 0; ha < HV * TI; ++ha) {
+      const int h = ha / TI, a = ha % TI;
 #pragma unroll
       for (int b = 0; b < TJ; ++b)
 #pragma unroll
-        for (int r = 0; r < 4; ++r) strip[(4 * frag_q + r) * SP + b * 16 + frag_row] = acc[a][b][r];
+        for (int r = 0; r < 4; ++r) strip[(4 * frag_q + r) * SP + b * 16 + frag_row] = acc[h][a][b][r];
       asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
       acc_t v[TJ];
 #pragma unroll
@@ -667,7 +698,7 @@ __global__ __launch_bounds__(64 * (WI * WJ + NWL)) void amos_conv_nchw(const Con
       asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
 #pragma unroll
       for (int x = 0; x < TJ; ++x) {
-        const int i = bi0 + (wi * TI + a) * 16 + x * RPI + lane / CPR;
+        const int i = bi0 + h * BI + (wi * TI + a) * 16 + x * RPI + lane / CPR;
         // (J is a multiple of four here: the four positions are inside the tensor together)
         if (i < s.K && j4 < s.J) *(acc_t*)(out + coff + (int64_t)i * ODPQ) = v[x];
       }
@@ -681,18 +712,19 @@ __global__ __launch_bounds__(64 * (WI * WJ + NWL)) void amos_conv_nchw(const Con
     const int n = nchw_div(jc, p.div_odpq);
     const int64_t coff = (int64_t)n * s.K * ODPQ + (jc - n * ODPQ);
 #pragma unroll
-    for (int a = 0; a < TI; ++a) {
-      const int i0 = bi0 + (wi * TI + a) * 16 + 4 * frag_q;
+    for (int ha = 0; ha < HV * TI; ++ha) {
+      const int h = ha / TI, a = ha % TI;
+      const int i0 = bi0 + h * BI + (wi * TI + a) * 16 + 4 * frag_q;
       if (add_d) {
         out_t dv[4];
 #pragma unroll
         for (int r = 0; r < 4; ++r) dv[r] = epi_value<out_t>(p.epi, coff + (int64_t)(i0 + r < s.K ? i0 + r : s.K - 1) * ODPQ);
 #pragma unroll
-        for (int r = 0; r < 4; ++r) acc[a][b][r] += dv[r];
+        for (int r = 0; r < 4; ++r) acc[h][a][b][r] += dv[r];
       }
 #pragma unroll
       for (int r = 0; r < 4; ++r)
-        if (i0 + r < s.K && j < s.J) out[coff + (int64_t)(i0 + r) * ODPQ] = acc[a][b][r];
+        if (i0 + r < s.K && j < s.J) out[coff + (int64_t)(i0 + r) * ODPQ] = acc[h][a][b][r];
     }
   }
 }

@@ -190,6 +190,7 @@ struct ConvNchwInstance {
   int loader_waves;
   int mma_waves;
   int load_bytes;          // bytes of a patch load (8, or 16: needs 16-byte aligned channel planes)
+  int halves;              // halves of output channels a workgroup computes (bi rows each)
   std::once_flag once;
   int scratch_bytes = 0;   // per-lane scratch memory of the built kernel (register spills)
   bool fits = true;        // a workgroup of `threads` fits a compute unit's registers
@@ -202,15 +203,16 @@ ConvNchwInstance* pick_conv_nchw_i8(int ti, int tj, int wmode, int pt, int nwl, 
 void launch_conv_pack_weights(int es, const void* w, void* out, int K, int C, int TRS, hipStream_t stream);
 
 #ifdef AMOS_CONV_NCHW_KERNEL_INCLUDED
-template <int DT, int BI, int BJ, int WI, int WJ, int PTL, int WMODE, int NWL, int LB>
+template <int DT, int BI, int BJ, int WI, int WJ, int PTL, int WMODE, int NWL, int LB, int HV = 1>
 ConvNchwInstance* conv_nchw_instance() {
   static ConvNchwInstance inst;
   static const char* dtn[] = {"f16", "bf16", "i8"};
   static const char* wmn[] = {",kctrs", ",kcrs", ",packed"};
-  static std::string name = std::string("amos_conv_nchw<") + dtn[DT] + "," + std::to_string(BI) + "x" +
+  static std::string name = std::string("amos_conv_nchw<") + dtn[DT] + "," + (HV > 1 ? std::to_string(HV) + "x" : std::string()) + std::to_string(BI) + "x" +
                             std::to_string(BJ) + "," + std::to_string(WI * WJ) + "+" + std::to_string(NWL) + "w" +
                             wmn[WMODE] + (LB == 16 ? ",ld16" : "") + (PTL > 1 ? ",pt" + std::to_string(PTL) + ">" : std::string(">"));
-  inst.fn = amos_conv_nchw<DT, BI, BJ, WI, WJ, PTL, WMODE, NWL, LB>;
+  inst.fn = amos_conv_nchw<DT, BI, BJ, WI, WJ, PTL, WMODE, NWL, LB, HV>;
+  inst.halves = HV;
   inst.name = name.c_str();
   inst.threads = 64 * (WI * WJ + NWL);
   inst.bi = BI;
@@ -229,6 +231,9 @@ ConvNchwInstance* pick_conv_nchw_p(int ti, int tj) {
   if (ti == 64 && tj == 256) return conv_nchw_instance<DT, 64, 256, 1, 8, PTL, WMODE, NWL, LB>();
   if (ti == 32 && tj == 128) return conv_nchw_instance<DT, 32, 128, 1, 4, PTL, WMODE, NWL, LB>();
   if (ti == 32 && tj == 256) return conv_nchw_instance<DT, 32, 256, 1, 4, PTL, WMODE, NWL, LB>();
+  // 128 rows: two halves of 64 that share every macro step's patch
+  if (ti == 128 && tj == 256) return conv_nchw_instance<DT, 64, 256, 1, 8, PTL, WMODE, NWL, LB, 2>();
+  if (ti == 128 && tj == 128) return conv_nchw_instance<DT, 64, 128, 2, 4, PTL, WMODE, NWL, LB, 2>();
   return nullptr;
 }
 // lb: bytes of a patch load; 16 only for 16-bit types, one round, and not with weights whose taps

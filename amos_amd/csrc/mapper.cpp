@@ -698,7 +698,8 @@ ConvNchwPlan conv_nchw_plan(const amos_conv_desc_t& c, int op, int BI, int BJ, i
   if ((c.C * es) % 64) { r.why = "channels do not fill whole 64-byte chunks"; return r; }
   if (load_bytes != 8 && (load_bytes != 16 || es != 2)) { r.why = "patch loads of 16 bytes are for 16-bit types"; return r; }
   if ((c.H * c.W * es) % load_bytes) { r.why = "a channel plane is not a whole number of patch loads"; return r; }
-  if ((BI != 64 && BI != 32) || (BJ != 128 && BJ != 256)) { r.why = "block tile not 32 or 64 by 128 or 256"; return r; }
+  // (128 rows: two halves of 64 that share every macro step's patch)
+  if ((BI != 128 && BI != 64 && BI != 32) || (BJ != 128 && BJ != 256)) { r.why = "block tile not 32, 64 or 128 by 128 or 256"; return r; }
   // (lanes address both tensors by 32-bit byte offsets)
   if (c.N * c.C * D * c.H * c.W * es >= ((int64_t)1 << 32) || c.K * c.C * T * 9 * es >= ((int64_t)1 << 32)) { r.why = "a tensor of 4 GiB or more"; return r; }
   NchwShape s;
@@ -748,7 +749,7 @@ ConvNchwPlan conv_nchw_plan(const amos_conv_desc_t& c, int op, int BI, int BJ, i
   // launch plan decides and refuses what is above the loaders' budget)
   r.groups_per_thread = 0;
   if (r.max_pos > pos_limit) { r.why = "input patch of a tile does not fit its LDS buffer"; return r; }
-  r.lds = (size_t)2 * 9 * BI * 64 + (size_t)2 * pbuf;
+  r.lds = (size_t)2 * 9 * (BI == 128 ? 64 : BI) * 64 + (size_t)2 * pbuf;
   r.t1 = T == 1;
   return r;
 }
@@ -796,7 +797,9 @@ static double conv_patch_estimate(const amos_conv_desc_t& c, int op, const Probl
 // Returns <= 0 where the kernel does not apply.
 double conv_nchw_estimate(const amos_conv_desc_t& c, int op, const Problem& pb, int ti, int tj, bool* unpacked) {
   if (unpacked) *unpacked = false;
-  if ((ti != 64 && ti != 32) || (tj != 128 && tj != 256)) return -1.0;
+  if ((ti != 128 && ti != 64 && ti != 32) || (tj != 128 && tj != 256)) return -1.0;
+  const int halves = ti == 128 ? 2 : 1;   // a 128-row workgroup: two sequence steps of 64 rows per macro step
+  const int tr = ti / halves;
   // (as the launch plans it: patch loads of 16 bytes where the shape allows them and one round of
   // the loaders covers the largest tile)
   int s_lb = conv_nchw_load_bytes(c);
@@ -814,15 +817,16 @@ double conv_nchw_estimate(const amos_conv_desc_t& c, int op, const Problem& pb, 
   const double macro_steps = (double)T * (c.C * es / 64.0);
   const double tiles = std::ceil((double)pb.I / ti) * std::ceil((double)pb.J / tj);
   const double rounds = std::ceil(tiles / device_compute_units());
-  const double flop_per_cycle = (i8 ? 2.0 : 1.0) * 3850.0 * (ti * tj >= 64 * 256 ? 0.85 : ti * tj >= 64 * 128 ? 0.72 : 0.6);
-  const double mma = 2.0 * ti * tj * 9.0 * (64.0 / es) / flop_per_cycle;
+  const double flop_per_cycle = (i8 ? 2.0 : 1.0) * 3850.0 * (tr * tj >= 64 * 256 ? 0.85 : tr * tj >= 64 * 128 ? 0.72 : 0.6);
+  const double mma = 2.0 * tr * tj * 9.0 * (64.0 / es) / flop_per_cycle;
   // the loaders of a macro step: a fixed part, the bytes they move and their load instructions
   // (fitted: 64x128 tile, 24 instructions of 8 bytes a lane 2400 cycles, of 16 bytes 3500; 64x256,
   // 32 of 16 bytes 4600)
   const double load_instr = std::ceil(np.max_groups * 4.0 / 64.0) * (16.0 / es);
   const double loaders = 1300.0 + 5.0 * load_instr * s_lb + 20.0 * load_instr;
   const double prologue = 9000.0 + 40.0 * load_instr;
-  const double cycles = rounds * (prologue + macro_steps * std::max(mma, loaders));
+  // (the second half of a macro step has no patch to bring in: its weights only; twice the stores)
+  const double cycles = rounds * (prologue + (halves - 1) * 2500.0 + macro_steps * (std::max(mma, loaders) + (halves - 1) * std::max(mma, 900.0)));
   const double kernel = cycles / 2.4e9 + 2.5e-6;
   // the weights: packed by a launch in front of the kernel (its cost is the dependent launch more
   // than the copy), or -- conv2d, where a chunk's taps are one aligned run -- transposed by the
@@ -1012,7 +1016,7 @@ int amos_default_config(int op, const void* desc, amos_kernel_config_t* result) 
   if (op == AMOS_OP_CONV2D || op == AMOS_OP_CONV3D) {
     const amos_conv_desc_t& c = *(const amos_conv_desc_t*)desc;
     if (patch_best < 1e30 && best >= staged_bar) best = patch_best;   // (the estimate of what was chosen)
-    for (int ti : {64, 32})
+    for (int ti : {64, 32, 128})
       for (int tj : {128, 256}) {
         const double s = conv_nchw_estimate(c, op, pb, ti, tj);
         if (s > 0 && s < best * 0.97) {

@@ -7,7 +7,13 @@ nothing the compiler generates touches those registers: an address the compiler 
 would be overwritten by a load that lands, and the next access through it faults.  So the build
 refuses to link a library, and a test fails, unless for every instance
 
-  * no instruction outside the assembly statements names a staging register;
+  * no compiler-generated instruction names a staging register between a staging load and the wait
+    for it: followed along the kernel's labels and branches from every assembly statement that
+    loads into a staging register up to the next assembly statement `s_waitcnt vmcnt(0)` -- the
+    stretch in which the data lands.  (A value the compiler keeps across a staging load cannot sit
+    in one of these registers: the load statements declare them clobbered.  Code outside those
+    stretches -- the matrix-core waves' in particular, other waves with registers of their own --
+    may use every register the workgroup size leaves it.)
   * the assembly statements stay inside the 32 staging registers;
   * the instance neither spills to scratch memory nor uses accumulation registers, its register
     count covers the staging registers and leaves room for the waves of one workgroup on a
@@ -34,23 +40,19 @@ def vregs(text):
     return out
 
 
-def instances(asm_path):
-    """{kernel symbol: {targs, waves, base (first staging register), outside: instructions outside
-    assembly statements that name a staging register, inside: staging registers the assembly
-    statements name}}"""
-    found, name, inasm = {}, None, False
-    for line in open(asm_path):
-        m = re.match(r"^(_ZN4amos14amos_conv_nchw\w+):", line)
+_LABEL = re.compile(r"^(\.LBB\d+_\d+):")
+_BRANCH = re.compile(r"^\s*(s_branch|s_cbranch_\w+)\s+(\.LBB\d+_\d+)")
+
+
+def _blocks(lines):
+    """basic blocks of one kernel's assembly text: [{label, code: [(text, inside an assembly
+    statement)], succ: [block indices]}]"""
+    blocks, cur, inasm = [], {"label": None, "code": [], "targets": [], "falls": True}, False
+    for line in lines:
+        m = _LABEL.match(line)
         if m:
-            name = m.group(1)
-            t = [int(x) for x in re.findall(r"Li(\d+)E", name)]
-            waves = t[3] * t[4] + t[7]          # WI * WJ matrix-core waves + NWL loader waves
-            found[name] = {"targs": t, "waves": waves, "base": {12: 136, 8: 224}.get(waves, -1), "outside": [], "inside": set()}
-            continue
-        if name is None:
-            continue
-        if line.startswith(".Lfunc_end"):
-            name = None
+            blocks.append(cur)
+            cur = {"label": m.group(1), "code": [], "targets": [], "falls": True}
             continue
         if "ASMSTART" in line:
             inasm = True
@@ -61,12 +63,90 @@ def instances(asm_path):
         code = line.split(";")[0].strip()
         if not code or code.startswith("."):
             continue
+        if not cur["falls"]:   # code behind an unconditional branch without a label: its own block
+            blocks.append(cur)
+            cur = {"label": None, "code": [], "targets": [], "falls": True}
+        cur["code"].append((code, inasm))
+        b = _BRANCH.match(code)
+        if b:
+            cur["targets"].append(b.group(2))
+            if b.group(1) == "s_branch":
+                cur["falls"] = False
+        elif code.startswith("s_endpgm"):
+            cur["falls"] = False
+    blocks.append(cur)
+    index = {b["label"]: i for i, b in enumerate(blocks) if b["label"]}
+    for i, b in enumerate(blocks):
+        b["succ"] = [index[t] for t in b["targets"] if t in index]
+        if b["falls"] and i + 1 < len(blocks):
+            b["succ"].append(i + 1)
+    return blocks
+
+
+def instances(asm_path):
+    """{kernel symbol: {targs, waves, base (first staging register), outside: compiler-generated
+    instructions between a staging load and its wait that name a staging register, inside: staging
+    registers the assembly statements name}}"""
+    found, name, body = {}, None, []
+
+    def finish():
         rec = found[name]
-        high = {r for r in vregs(code) if r >= rec["base"]}
-        if inasm:
-            rec["inside"] |= high
-        elif high:
-            rec["outside"].append(code)
+        base = rec["base"]
+        blocks = _blocks(body)
+        index = {b["label"]: i for i, b in enumerate(blocks) if b["label"]}
+        is_load = lambda code, inasm: inasm and "load" in code and any(r >= base for r in vregs(code))
+        is_wait = lambda code, inasm: inasm and code.replace(" ", "") == "s_waitcntvmcnt(0)"
+        for b in blocks:
+            for code, inasm in b["code"]:
+                if inasm:
+                    rec["inside"] |= {r for r in vregs(code) if r >= base}
+        # from behind every staging load, forward until the wait
+        seen_block_starts, todo, flagged = set(), [], []
+        for i, b in enumerate(blocks):
+            for k, (code, inasm) in enumerate(b["code"]):
+                if is_load(code, inasm):
+                    todo.append((i, k + 1))
+        done = set()
+        while todo:
+            i, k = todo.pop()
+            if (i, k) in done:
+                continue
+            done.add((i, k))
+            stopped = False
+            follow = []
+            for code, inasm in blocks[i]["code"][k:]:
+                if is_wait(code, inasm):
+                    stopped = True
+                    break
+                if not inasm and any(r >= base for r in vregs(code)):
+                    flagged.append(code)
+                b = _BRANCH.match(code)
+                if b and b.group(2) in index:      # a branch in front of the wait leaves the block
+                    follow.append(index[b.group(2)])
+            if not stopped:
+                follow = blocks[i]["succ"]
+            for j in follow:
+                if j not in seen_block_starts:
+                    seen_block_starts.add(j)
+                    todo.append((j, 0))
+        rec["outside"] = flagged
+
+    for line in open(asm_path):
+        m = re.match(r"^(_ZN4amos14amos_conv_nchw\w+):", line)
+        if m:
+            name = m.group(1)
+            t = [int(x) for x in re.findall(r"Li(\d+)E", name)]
+            waves = t[3] * t[4] + t[7]          # WI * WJ matrix-core waves + NWL loader waves
+            found[name] = {"targs": t, "waves": waves, "base": {12: 136, 8: 224}.get(waves, -1), "outside": [], "inside": set()}
+            body = []
+            continue
+        if name is None:
+            continue
+        if line.startswith(".Lfunc_end"):
+            finish()
+            name = None
+            continue
+        body.append(line)
     return found
 
 

@@ -41,14 +41,21 @@ def test_staging_registers_belong_to_the_assembly_statements():
             total += n
             bad += b
         assert not bad, "\n".join(bad)
-        assert total >= 60
+        assert total >= 100
 
 
 def test_the_check_sees_a_violation(tmp_path):
     """doctored code: a compiler-generated instruction that names a staging register, an assembly
     statement outside the staging range, a spill -- each must be reported"""
     sym = "_ZN4amos14amos_conv_nchwILi0ELi64ELi128ELi2ELi4ELi1ELi2ELi4ELi8EEEvNS_14ConvNchwParamsE"
-    good = "%s:\n\tv_mov_b32_e32 v5, 0\n\t;;#ASMSTART\n\tglobal_load_dwordx2 v[136:137], v5, s[0:1]\n\t;;#ASMEND\n.Lfunc_end0:\n" % sym
+    # a staging load, compiler code behind it (HERE), the wait, code behind the wait (AFTER), and a
+    # block that only the matrix-core waves run (a branch around the loaders' code: OTHER)
+    good = ("%s:\n\ts_cbranch_scc1 .LBB0_2\n\tv_mov_b32_e32 v5, 0\n"
+            "\t;;#ASMSTART\n\tglobal_load_dwordx2 v[136:137], v5, s[0:1]\n\t;;#ASMEND\n"
+            "\tv_mov_b32_e32 v6, 1\n"                                      # HERE
+            "\t;;#ASMSTART\n\ts_waitcnt vmcnt(0)\n\t;;#ASMEND\n"
+            "\tv_mov_b32_e32 v7, 2\n\ts_endpgm\n"                         # AFTER
+            ".LBB0_2:\n\tv_mov_b32_e32 v8, 3\n\ts_endpgm\n.Lfunc_end0:\n" % sym)   # OTHER
     log = "remark: Function Name: %s\nremark:     VGPRs: 168\nremark:     AGPRs: 0\nremark:     ScratchSize [bytes/lane]: 0\nremark:     Occupancy [waves/SIMD]: 3\n" % sym
 
     def run(asm, remarks=log):
@@ -57,8 +64,16 @@ def test_the_check_sees_a_violation(tmp_path):
         return isa_check.violations("x", str(path), remarks)[1]
 
     assert run(good) == []
-    assert any("names a staging register" in b for b in run(good.replace("v_mov_b32_e32 v5, 0", "v_add_u32_e32 v140, v5, v5")))
-    assert any("names a staging register" in b for b in run(good.replace("v_mov_b32_e32 v5, 0", "ds_read_b128 v[134:137], v5")))
+    # between the load and its wait: reported, whether the register is written or read, alone or in a range
+    assert any("names a staging register" in b for b in run(good.replace("v_mov_b32_e32 v6, 1", "v_add_u32_e32 v140, v5, v5")))
+    assert any("names a staging register" in b for b in run(good.replace("v_mov_b32_e32 v6, 1", "ds_read_b128 v[134:137], v5")))
+    # ... also where the stretch runs through a branch target
+    assert any("names a staging register" in b
+               for b in run(good.replace("v_mov_b32_e32 v6, 1", "s_cbranch_scc0 .LBB0_2").replace("v_mov_b32_e32 v8, 3", "v_mov_b32_e32 v150, 3")))
+    # behind the wait, and in code that no path from a staging load reaches before a wait: the
+    # data has landed / these are other waves' registers
+    assert run(good.replace("v_mov_b32_e32 v7, 2", "v_mov_b32_e32 v140, 2")) == []
+    assert run(good.replace("v_mov_b32_e32 v8, 3", "v_mov_b32_e32 v150, 3")) == []
     assert any("assembly names" in b for b in run(good.replace("v[136:137]", "v[0xa6:0xa9]")))
     assert any("scratch" in b for b in run(good, log.replace("ScratchSize [bytes/lane]: 0", "ScratchSize [bytes/lane]: 16")))
     assert any("register count" in b for b in run(good, log.replace("VGPRs: 168", "VGPRs: 124")))

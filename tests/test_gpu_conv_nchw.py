@@ -28,7 +28,7 @@ def _cfg(_lib, tj, ti=64):
     return dict(tile_i=ti, tile_j=tj, split_k=1, pipeline=_lib.AMOS_PIPE_NCHW)
 
 
-TILES = [(64, 128), (64, 256), (32, 128), (32, 256)]
+TILES = [(64, 128), (64, 256), (32, 128), (32, 256), (128, 128), (128, 256)]
 
 
 def _run(fn, *args, **kw):
