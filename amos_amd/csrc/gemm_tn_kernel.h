@@ -106,9 +106,27 @@ __global__ __launch_bounds__(64 * WI * WJ) void amos_gemm_tn(const GemmTnParams 
   const int wi = wave / WJ, wj = wave % WJ;
 
   int tile_i, tile_j;
-  block_to_tile(blockIdx.x, gridDim.x, p.tiles_i, p.tiles_j, tile_i, tile_j);
+  int64_t batch = blockIdx.z;
+  // A batch of small products (its tiles fewer than the chip's workgroup slots): workgroups are
+  // dealt round-robin to the 8 XCDs in launch order (x fastest, then z), which spreads the tiles
+  // of one batch over all XCDs -- every L2 then fetches that batch's row and column panels.  Where
+  // the counts allow it, XCD x takes whole batches x, x + 8, ...: its s-th workgroup is tile
+  // s % T of batch x + 8 * (s / T), and a batch's panels are fetched by one L2 only.
+  if (gridDim.z > 1 && gridDim.y == 1 && (gridDim.z & 7) == 0) {
+    const unsigned T = gridDim.x, L = blockIdx.x + T * blockIdx.z;
+    const unsigned xcd = L & 7, sq = L >> 3;
+    const unsigned tile = sq % T;
+    batch = xcd + 8 * (sq / T);
+    const int per_group = 8 * p.tiles_j;   // (the walk of block_to_tile without its own XCD permutation)
+    const int gidx = (int)tile / per_group, first_i = gidx * 8;
+    const int rows_here = p.tiles_i - first_i < 8 ? p.tiles_i - first_i : 8;
+    const int in_group = (int)tile - gidx * per_group;
+    tile_i = first_i + in_group % rows_here;
+    tile_j = in_group / rows_here;
+  } else {
+    block_to_tile(blockIdx.x, gridDim.x, p.tiles_i, p.tiles_j, tile_i, tile_j);
+  }
   const int bi0 = tile_i * BI, bj0 = tile_j * BJ;
-  const int64_t batch = blockIdx.z;
   const char* const abase = p.a + (batch * p.batch_a + (int64_t)bi0 * p.lda) * ES;
   const char* const bbase = p.b + (batch * p.batch_b + (int64_t)bj0 * p.ldb) * ES;
 
