@@ -250,9 +250,10 @@ __global__ __launch_bounds__(64 * WI * WJ) void amos_gemm_tn(const GemmTnParams 
   constexpr int SP = TJ * 16 + 4;          // strip row pitch in elements
   constexpr int CPR = TJ * 4, RPI = 64 / CPR;   // 16-byte chunks per row, rows per store instruction
   static_assert(TJ <= 16 && (TJ & (TJ - 1)) == 0 && NW * 16 * SP * 4 <= NS * STAGE, "output strip");
-  // (wave tiles 32 columns wide keep the direct stores: the store-bound 192 x (512x512x64) batched
-  // product measured 2 % slower through the strip, the 64- and 128-column tiles 4-5 % faster)
-  const bool vec_out = TJ >= 4 && ((((uintptr_t)out) & 15) | (uintptr_t)(p.ldc & 3) | (uintptr_t)(p.J & 3)) == 0;
+  // (measured: the 64- and 128-column wave tiles 4-5 % faster through the strip; the 32-column
+  // tile of the store-bound 192 x (512x512x64) batched product 2 % faster once an XCD's workgroups
+  // write one batch's rows instead of eight batches')
+  const bool vec_out = TJ >= 2 && ((((uintptr_t)out) & 15) | (uintptr_t)(p.ldc & 3) | (uintptr_t)(p.J & 3)) == 0;
   out_t* const strip = (out_t*)(smem + wave * (16 * SP * 4));
   // the last K steps re-issue copies of the final tile: they (any wave's) must have landed, and
   // every wave must be done with its fragment reads, before the stages are reused
