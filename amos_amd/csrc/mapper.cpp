@@ -852,6 +852,23 @@ int amos_check_config(int op, const void* desc, const amos_kernel_config_t* cfg,
   int rc = problem_of(op, desc, &pb);
   if (rc) return rc;
   if (!cfg) return set_error(AMOS_ERR_BAD_ARG, "null config");
+  // the NCDHW-direct convolution has tiles of its own (32 / 64 / 128 rows by 128 / 256 positions):
+  // its planner says whether the shape and the tile go together and how much LDS a workgroup takes
+  if ((op == AMOS_OP_CONV2D || op == AMOS_OP_CONV3D) && cfg->pipeline == AMOS_PIPE_NCHW) {
+    const amos_conv_desc_t& c = *(const amos_conv_desc_t*)desc;
+    int lb = conv_nchw_load_bytes(c);
+    ConvNchwPlan np = conv_nchw_plan(c, op, cfg->tile_i, cfg->tile_j, lb);
+    if (np.why && lb == 16) np = conv_nchw_plan(c, op, cfg->tile_i, cfg->tile_j, 8);
+    if (np.why) return set_error(AMOS_ERR_INFEASIBLE, "NCDHW-direct convolution not applicable: %s", np.why);
+    if (lds_bytes) *lds_bytes = (int64_t)np.lds;
+    // (accumulators of a matrix-core wave: its share of the tile, four bytes an element, 64 lanes)
+    const int waves = cfg->tile_i >= 64 ? 8 : 4;
+    if (acc_regs) *acc_regs = (int64_t)cfg->tile_i * cfg->tile_j / (64 * waves);
+    if ((int64_t)np.lds > Gfx950::kLdsBytes)
+      return set_error(AMOS_ERR_INFEASIBLE, "LDS over budget: %lld (required) vs. %d (given)", (long long)np.lds, Gfx950::kLdsBytes);
+    if (cfg->split_k < 0) return set_error(AMOS_ERR_BAD_ARG, "negative split_k");
+    return 0;
+  }
   bool known = false;
   for (auto& t : kTiles) known |= (t[0] == cfg->tile_i && t[1] == cfg->tile_j);
   if (!known)

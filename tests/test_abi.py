@@ -71,6 +71,43 @@ def test_check_config_budget():
     assert lib.amos_check_config(0, ctypes.byref(d), ctypes.byref(bad), None, None) == _lib.AMOS_ERR_INFEASIBLE
 
 
+def test_check_config_and_estimate_know_the_ncdhw_direct_tiles():
+    """every tile the NCDHW-direct convolution is built for passes amos_check_config and gets an
+    estimate (the sweep skips what has none), the default of the benchmark's convolutions among
+    them; a tile it is not built for and a shape it does not take are refused with a reason"""
+    from amos_amd import ops
+    import torch
+    lib = _lib.load()
+    c3 = ops.conv_desc((32, 256, 1, 14, 14), (256, 256, 1, 3, 3), torch.float16, (1, 1, 1), (0, 1, 1), (1, 1, 1))
+    c4 = ops.conv_desc((64, 128, 1, 28, 28), (128, 128, 1, 3, 3), torch.int8, (1, 1, 1), (0, 1, 1), (1, 1, 1))
+    lds, regs, est = ctypes.c_int64(), ctypes.c_int64(), ctypes.c_double()
+    for d in (c3, c4):
+        for ti, tj in [(32, 128), (32, 256), (64, 128), (64, 256), (128, 128), (128, 256)]:
+            cfg = _lib.KernelConfig(ti, tj, 1, _lib.AMOS_PIPE_NCHW)
+            rc = lib.amos_check_config(_lib.AMOS_OP_CONV2D, ctypes.byref(d), ctypes.byref(cfg), ctypes.byref(lds), ctypes.byref(regs))
+            if rc != 0:   # (a tile whose patch does not fit: said so, not "no kernel instance")
+                assert b"NCDHW-direct" in lib.amos_last_error(), lib.amos_last_error()
+                continue
+            rows = 64 if ti == 128 else ti
+            assert lds.value == 2 * 9 * rows * 64 + 2 * (32 if tj <= 128 else 40) * 1024 and regs.value > 0
+            assert lib.amos_estimate_seconds(_lib.AMOS_OP_CONV2D, ctypes.byref(d), ctypes.byref(cfg), ctypes.byref(est)) == 0
+            assert 1e-6 < est.value < 1e-3
+        dflt = _lib.KernelConfig()
+        assert lib.amos_default_config(_lib.AMOS_OP_CONV2D, ctypes.byref(d), ctypes.byref(dflt)) == 0
+        assert dflt.pipeline == _lib.AMOS_PIPE_NCHW
+        assert lib.amos_check_config(_lib.AMOS_OP_CONV2D, ctypes.byref(d), ctypes.byref(dflt), None, None) == 0
+    bad = _lib.KernelConfig(96, 128, 1, _lib.AMOS_PIPE_NCHW)
+    assert lib.amos_check_config(_lib.AMOS_OP_CONV2D, ctypes.byref(c3), ctypes.byref(bad), None, None) == _lib.AMOS_ERR_INFEASIBLE
+    five = ops.conv_desc((32, 256, 1, 14, 14), (256, 256, 1, 5, 5), torch.float16, (1, 1, 1), (0, 2, 2), (1, 1, 1))
+    ok = _lib.KernelConfig(64, 128, 1, _lib.AMOS_PIPE_NCHW)
+    assert lib.amos_check_config(_lib.AMOS_OP_CONV2D, ctypes.byref(five), ctypes.byref(ok), None, None) == _lib.AMOS_ERR_INFEASIBLE
+    assert b"3x3" in lib.amos_last_error()
+    # a pointwise convolution asked to run on this pipeline is refused too, not run as a matrix product
+    one = ops.conv_desc((4, 64, 1, 14, 14), (64, 64, 1, 1, 1), torch.float16, (1, 1, 1), (0, 0, 0), (1, 1, 1))
+    assert lib.amos_kernel_name(_lib.AMOS_OP_CONV2D, ctypes.byref(one), ctypes.byref(ok)) is None
+    assert b"3x3" in lib.amos_last_error()
+
+
 def test_default_config_is_a_compiled_instance():
     lib = _lib.load()
     cfg = _lib.KernelConfig()
