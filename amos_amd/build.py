@@ -32,7 +32,8 @@ def build(verbose=True, jobs=8):
     for src in sources():
         obj = os.path.join(objdir, os.path.basename(src) + ".o")
         objs.append(obj)
-        jobs_list.append((src, obj, [hipcc] + HIP_FLAGS + inc + ["-c", src, "-o", obj]))
+        remarks = ["-Rpass-analysis=kernel-resource-usage"] if src.endswith(".hip") else []
+        jobs_list.append((src, obj, [hipcc] + HIP_FLAGS + inc + remarks + ["-c", src, "-o", obj]))
     # the same units once more as assembly text, for the check
     checked = []
     for unit in isa_check.UNITS:
@@ -67,6 +68,9 @@ def build(verbose=True, jobs=8):
     bad = []
     for unit, asm in checked:
         bad += isa_check.violations(unit, asm, logs[asm])[1]
+    # kernels that count their own memory waits must not spill: scratch traffic uses the same counter
+    for obj in objs:
+        bad += isa_check.spills(os.path.basename(obj), logs[obj])
     if bad:
         if os.path.exists(OUT):
             os.remove(OUT)

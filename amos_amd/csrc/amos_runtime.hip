@@ -4,7 +4,9 @@
 
 #include <cstdarg>
 #include <cstdio>
+#include <cstdlib>
 #include <cstring>
+#include <atomic>
 #include <mutex>
 #include <string>
 
@@ -1244,8 +1246,66 @@ static int launch_conv_nchw(const Plan& pl, hipStream_t stream) {
 
 static int launch_kernels(const Plan& pl, hipStream_t stream);
 
-// the kernels of the plan, then (split-K with partial sums) the launch that adds the slices
+// Ticket counters of the in-kernel split-K reduction (SplitFinish): the library's own, one array per
+// GPU, zero when the module is loaded and put back to zero by the workgroup that draws a tile's
+// last ticket.  A launch takes a run of counters of its own from a rotating position, so launches
+// that overlap on one GPU (other streams, other threads) do not share counters as long as fewer
+// than kTicketSlots tiles are in flight at once.
+constexpr int kTicketSlots = 1 << 16;
+static __device__ unsigned g_split_tickets[kTicketSlots];
+constexpr int kTicketMaxDevices = 64;
+static unsigned* g_ticket_ptr[kTicketMaxDevices];
+static std::mutex g_ticket_mutex;
+static std::atomic<unsigned> g_ticket_next{0};
+static unsigned* tickets_for(int64_t n) {
+  if (n <= 0 || n > kTicketSlots / 8) return nullptr;
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kTicketMaxDevices) return nullptr;
+  unsigned* base;
+  {
+    std::lock_guard<std::mutex> lock(g_ticket_mutex);
+    if (!g_ticket_ptr[dev] && hipGetSymbolAddress((void**)&g_ticket_ptr[dev], HIP_SYMBOL(g_split_tickets)) != hipSuccess) {
+      g_ticket_ptr[dev] = nullptr;
+      (void)hipGetLastError();
+    }
+    base = g_ticket_ptr[dev];
+  }
+  if (!base) return nullptr;
+  for (;;) {
+    const unsigned start = g_ticket_next.fetch_add((unsigned)n) % kTicketSlots;
+    if (start + n <= kTicketSlots) return base + start;   // (a run that would wrap is skipped)
+  }
+}
+
+// The in-kernel reduction is opt-in (environment AMOS_SPLIT_IN_KERNEL=1, read once): without it
+// every split adds its slices with the launch of its own below, the path every test has run on.
+static bool split_in_kernel() {
+  static const bool on = [] {
+    const char* v = getenv("AMOS_SPLIT_IN_KERNEL");
+    return v && v[0] == '1';
+  }();
+  return on;
+}
+
+// the kernels of the plan; split-K with partial sums: a launch of its own adds the slices, or --
+// opted in, no more tiles than there are counters, a kernel with that tail -- the last workgroup
+// of every tile does
 static int launch(const Plan& pl, hipStream_t stream) {
+  if (pl.part && split_in_kernel()) {
+    const bool own_tail = pl.nchw || pl.tn_waves || (pl.conv_ups && !(pl.conv_w9 == 2)) ||
+                          (!pl.conv_ups && !pl.skinny && !pl.dw && !pl.fewc);
+    const int64_t tiles = pl.nchw ? (int64_t)pl.nc.tiles_i * pl.nc.tiles_j
+                          : pl.conv_ups ? (int64_t)pl.cv.tiles_i * pl.cv.tiles_j
+                          : pl.tn_waves ? (int64_t)pl.tn.tiles_i * pl.tn.tiles_j * pl.batch
+                                        : (int64_t)pl.p.tiles_i * pl.p.tiles_j * pl.batch;
+    unsigned* const tk = own_tail ? tickets_for(tiles) : nullptr;
+    if (tk) {
+      Plan armed = pl;
+      const SplitFinish fin = {tk, pl.part_out, pl.split, pl.part_stride};
+      armed.p.fin = armed.tn.fin = armed.cv.fin = armed.nc.fin = fin;
+      return launch_kernels(armed, stream);
+    }
+  }
   int rc = launch_kernels(pl, stream);
   if (rc || !pl.part) return rc;
   const int64_t n = pl.fill_rows * pl.fill_cols;
@@ -1370,6 +1430,9 @@ static int plan_epilogue(Plan& pl, int op, const void* desc, const amos_epilogue
       ep.batch = pl.p.out_batch;
     }
   }
+  // (no in-kernel reduction of a split unless the launch arms it)
+  const SplitFinish no_fin = {nullptr, nullptr, 0, 0};
+  pl.p.fin = no_fin; pl.tn.fin = no_fin; pl.cv.fin = no_fin; pl.nc.fin = no_fin;
   pl.p.epi = ep;
   pl.tn.epi = ep;
   pl.cv.epi = ep;

@@ -76,6 +76,7 @@ struct ConvFpropParams {
   int prep_w_blocks, prep_x_blocks, prep_z_blocks;
   int64_t zero_words;
   EpiParams epi;     // fused tail: Y = acc + cast(D), D laid out like Y
+  SplitFinish fin;   // split-K: the last workgroup of a tile adds the slices
   // tensor layouts (AMOS_LAYOUT_*): 0 = NCDHW / KCTRS / NKDPQ, 1 = NDHWC / TRSCK / NDPQK,
   // 2 = DHWNC / TRSCK / DPQNK.  Output element (i, j), j = n*ODPQ + s, at i*y_si + n*y_sn + s*y_ss.
   int layout;
@@ -892,6 +893,18 @@ __global__ __launch_bounds__(64 * NW, OCC) void amos_conv_fprop(const ConvFpropP
   if constexpr (!PERSIST) store_tile(geo);
   // the re-fetched tiles of the last steps still target this block's LDS
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  if constexpr (!PERSIST) {
+    if (p.fin.tickets) {
+      const int ODPQ = p.OD * OPQ;
+      split_finish<out_t>(p.fin, blockIdx.x, (const out_t*)p.y, (int)threadIdx.x, (int)blockDim.x, BI, BJ,
+                          (lds_flag_t)(size_t)0, [&](int r, int c) -> int64_t {
+                            const int i = geo.bi0 + r, j = geo.bj0 + c;
+                            if (i >= p.K || j >= p.J) return -1;
+                            const int n = fast_div(j, p.fd_odpq);
+                            return (int64_t)n * p.y_sn + (int64_t)(j - n * ODPQ) * p.y_ss + (int64_t)i * p.y_si;
+                          });
+    }
+  }
 }
 
 }  // namespace amos

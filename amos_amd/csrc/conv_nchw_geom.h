@@ -30,7 +30,7 @@
 #pragma once
 #include <stdint.h>
 
-#if defined(__HIPCC__) || defined(__CUDACC__)
+#if defined(__HIPCC__)
 #define AMOS_HD __host__ __device__ __forceinline__
 #else
 #define AMOS_HD inline

@@ -51,6 +51,7 @@ struct ConvNchwParams {
   int64_t split_stride;  // elements between the partial outputs of the split-K blocks
   NchwDiv div_cc, div_odpq;
   EpiParams epi;         // fused tail: Y = acc + cast(D), D laid out like Y
+  SplitFinish fin;       // split-K: the last workgroup of a tile adds the slices
 };
 
 #define AMOS_LDS_ADDR(off) ((__attribute__((address_space(3))) char*)(size_t)(off))
@@ -703,8 +704,7 @@ __global__ __launch_bounds__(64 * (WI * WJ + NWL)) void amos_conv_nchw(const Con
         if (i < s.K && j4 < s.J) *(acc_t*)(out + coff + (int64_t)i * ODPQ) = v[x];
       }
     }
-    return;
-  }
+  } else {
 #pragma unroll
   for (int b = 0; b < TJ; ++b) {
     const int j = bj0 + (wj * TJ + b) * 16 + frag_row;
@@ -726,6 +726,17 @@ __global__ __launch_bounds__(64 * (WI * WJ + NWL)) void amos_conv_nchw(const Con
       for (int r = 0; r < 4; ++r)
         if (i0 + r < s.K && j < s.J) out[coff + (int64_t)(i0 + r) * ODPQ] = acc[h][a][b][r];
     }
+  }
+  }
+  if (p.fin.tickets) {
+    // (the loader waves have left: the matrix-core waves' threads are the workgroup now)
+    split_finish<out_t>(p.fin, blockIdx.x, (const out_t*)p.y, t, NTM, BI * HV, BJ, (lds_flag_t)(size_t)0,
+                        [&](int r, int c) -> int64_t {
+                          const int i = bi0 + r, j = bj0 + c;
+                          if (i >= s.K || j >= s.J) return -1;
+                          const int n = nchw_div(j, p.div_odpq);
+                          return ((int64_t)n * s.K + i) * ODPQ + (j - n * ODPQ);
+                        });
   }
 }
 

@@ -99,6 +99,46 @@ __device__ __forceinline__ int epi_value<int>(const EpiParams& e, int64_t idx) {
   return ((const int*)e.ptr)[idx];
 }
 
+// Split-K without a second launch: every split stores its partial tile into its own slice (as
+// for the reduction launch), then takes a ticket of the tile; the workgroup that draws the last
+// one adds the slices IN THE ORDER OF THE SPLITS -- the same bits whichever workgroup that is --
+// and writes the output.  The counters are the library's own, zero between launches (the last
+// arrival puts its counter back).  (The reference reduces a split inside one kernel as well,
+// through shared memory: python/tvm/auto_tensorize/tensorization_phases/schedulers/cuda_split_K.py:868-914.)
+struct SplitFinish {
+  unsigned* tickets;     // nullptr: a launch of its own adds the slices
+  char* out;             // the output proper (the kernel's own output pointer names the slices)
+  int nsplit;
+  int64_t slice_stride;  // elements between the slices
+};
+// Called by every thread of the workgroup behind its last store, `flag` a pointer to an LDS word
+// nobody else uses any more -- IN THE LDS ADDRESS SPACE where it is made from a byte offset: the
+// compiler folds a cast of LDS offset 0 to a generic pointer into the null pointer, and the
+// access into one of global address 0.  elem(r, c) gives the element offset of row r, column c of
+// the workgroup's rows x cols tile in the output (the same in every slice), or a negative value
+// outside the tensor.
+typedef volatile __attribute__((address_space(3))) unsigned* lds_flag_t;
+template <typename T, typename Flag, typename Elem>
+__device__ __forceinline__ void split_finish(const SplitFinish& f, unsigned tile_id, const T* slices, int tid, int nthreads,
+                                             int rows, int cols, Flag flag, Elem elem) {
+  __threadfence();   // this workgroup's slice, visible to every other one before the ticket is
+  __syncthreads();
+  if (tid == 0) *flag = atomicAdd(f.tickets + tile_id, 1u) == (unsigned)(f.nsplit - 1) ? 1u : 0u;
+  __syncthreads();
+  if (!*flag) return;
+  __threadfence();   // ... and theirs to this one behind it
+  T* const out = (T*)f.out;
+  for (int idx = tid; idx < rows * cols; idx += nthreads) {
+    const int r = idx / cols, c = idx - r * cols;
+    const int64_t at = elem(r, c);
+    if (at < 0) continue;
+    T acc = slices[at];
+    for (int sp = 1; sp < f.nsplit; ++sp) acc += slices[(int64_t)sp * f.slice_stride + at];
+    out[at] = acc;
+  }
+  if (tid == 0) atomicExch(f.tickets + tile_id, 0u);
+}
+
 template <int N> struct NSlots { static constexpr int value = N; };
 
 struct ConvGeom {
@@ -137,6 +177,7 @@ struct IgemmParams {
   int atomic_out;               // split-K without a workspace: accumulate into a zeroed output
   int64_t split_stride;         // split-K with one: blockIdx.y stores its partial sums at out + blockIdx.y * split_stride
   EpiParams epi;                // D is indexed like the output, with its own row stride
+  SplitFinish fin;              // split-K with slices: the last workgroup of a tile adds them
 };
 
 __device__ __forceinline__ int lds_chunk_offset(int row, int chunk) {
@@ -508,6 +549,16 @@ __global__ __launch_bounds__(256) void amos_igemm(const IgemmParams p) {
         }
       }
     }
+  }
+  if (p.fin.tickets) {
+    split_finish<out_t>(p.fin, (unsigned)(batch * gridDim.x + blockIdx.x), (const out_t*)p.out, t, 256, BI, BJ, (lds_flag_t)smem,
+                        [&](int r, int c) -> int64_t {
+                          const int i = bi0 + r, j = bj0 + c;
+                          if (i >= p.I || j >= p.J) return -1;
+                          const int jo = j / p.out_jmod;
+                          return batch * p.out_batch + (int64_t)i * p.out_si + (int64_t)jo * p.out_sjo +
+                                 (int64_t)(j - jo * p.out_jmod) * p.out_sj;
+                        });
   }
 }
 

@@ -830,9 +830,9 @@ double conv_nchw_estimate(const amos_conv_desc_t& c, int op, const Problem& pb, 
   const double kernel = cycles / 2.4e9 + 2.5e-6;
   // the weights: packed by a launch in front of the kernel (its cost is the dependent launch more
   // than the copy), or -- conv2d, where a chunk's taps are one aligned run -- transposed by the
-  // loaders of every tile, some 600 cycles more per macro step
+  // loaders of every tile, some 600 cycles more per macro step and 64 rows
   const double pack = (double)(c.K * c.C * T * 9) * es * 2.0 / 2.5e12 + 3.5e-6;
-  const double in_kernel = rounds * macro_steps * 600.0 / 2.4e9;
+  const double in_kernel = rounds * macro_steps * 600.0 * halves / 2.4e9;
   if (op == AMOS_OP_CONV2D && in_kernel < pack) {
     if (unpacked) *unpacked = true;
     return kernel + in_kernel;

@@ -17,7 +17,11 @@ refuses to link a library, and a test fails, unless for every instance
   * the assembly statements stay inside the 32 staging registers;
   * the instance neither spills to scratch memory nor uses accumulation registers, its register
     count covers the staging registers and leaves room for the waves of one workgroup on a
-    compute unit.
+    compute unit;
+  * no instruction accesses memory through a generic ("flat") address: the kernel names global
+    memory and the LDS in their own address spaces.  (An LDS byte offset turned into a generic
+    pointer is what this catches: the compiler folds offset 0 into the null pointer, and the
+    access becomes one of global address 0 -- a memory fault.)
 """
 import re
 
@@ -100,6 +104,8 @@ def instances(asm_path):
             for code, inasm in b["code"]:
                 if inasm:
                     rec["inside"] |= {r for r in vregs(code) if r >= base}
+                if re.match(r"flat_(load|store|atomic)", code):
+                    rec["flat"].append(code)
         # from behind every staging load, forward until the wait
         seen_block_starts, todo, flagged = set(), [], []
         for i, b in enumerate(blocks):
@@ -137,7 +143,7 @@ def instances(asm_path):
             name = m.group(1)
             t = [int(x) for x in re.findall(r"Li(\d+)E", name)]
             waves = t[3] * t[4] + t[7]          # WI * WJ matrix-core waves + NWL loader waves
-            found[name] = {"targs": t, "waves": waves, "base": {12: 136, 8: 224}.get(waves, -1), "outside": [], "inside": set()}
+            found[name] = {"targs": t, "waves": waves, "base": {12: 136, 8: 224}.get(waves, -1), "outside": [], "inside": set(), "flat": []}
             body = []
             continue
         if name is None:
@@ -165,6 +171,22 @@ def resources(log_text):
     return rows
 
 
+# Kernels whose pipelines wait for their own global -> LDS copies and global loads by count
+# (s_waitcnt vmcnt(n), n > 0): a register spill's scratch access counts on the same counter, so a
+# spilling instance would wait for the wrong accesses.  The build refuses such an instance; the
+# library refuses to launch one as well (amos_runtime.hip: launch_tn, launch_conv).
+NO_SCRATCH = ("amos_gemm_tn", "amos_conv_fprop", "amos_conv_nchw")
+
+
+def spills(unit, log_text):
+    """[what is wrong] for one translation unit's resource remarks"""
+    bad = []
+    for name, r in resources(log_text).items():
+        if any(("%d%s" % (len(k), k)) in name for k in NO_SCRATCH) and r.get("scratch", 0):
+            bad.append("%s: %s spills %d bytes per lane to scratch memory" % (unit, name, r["scratch"]))
+    return bad
+
+
 def violations(unit, asm_path, log_text):
     """(number of instances read, [what is wrong]) for one translation unit"""
     bad = []
@@ -179,6 +201,8 @@ def violations(unit, asm_path, log_text):
             continue
         if rec["outside"]:
             bad.append("%s: compiler-generated code names a staging register: %s" % (what, rec["outside"][:3]))
+        if rec["flat"]:
+            bad.append("%s: memory accessed through a generic address: %s" % (what, rec["flat"][:3]))
         if not rec["inside"]:
             bad.append("%s: no staging register in its assembly statements" % what)
             continue

@@ -38,12 +38,33 @@ def kernel_source_hash(files):
     return h.hexdigest()[:12]
 
 
+def stale_summaries():
+    """{configuration: record} of the `stale_json:` lines under profiles/: configurations whose
+    default kernel has changed since its counters were read and has not been profiled again (the
+    record names the kernel that ships now and why there is no reading of it)"""
+    out = {}
+    pdir = os.path.join(ROOT, "profiles")
+    for fn in sorted(os.listdir(pdir)) if os.path.isdir(pdir) else []:
+        if fn.endswith(".md"):
+            for line in open(os.path.join(pdir, fn)):
+                if line.startswith("stale_json:"):
+                    try:
+                        rec = json.loads(line[len("stale_json:"):])
+                        out[rec["config"]] = rec
+                    except (ValueError, KeyError):
+                        continue
+    return out
+
+
 def measured_traffic(kernel_name):
     """HBM bytes per launch of `kernel_name` from the counter summaries under profiles/: a summary
     carries a line `traffic_json: {...}` with the kernel's name, the two counter readings (KiB per
     dispatch), the factors a plain copy of known size gave for them, and the hash of the kernel's
     sources at the time of the run.  Returns None when no summary names this kernel or its sources
-    have changed since (the figure would describe a kernel that no longer ships)."""
+    have changed since (the figure would describe a kernel that no longer ships).  A summary may
+    carry its figure over to ONE later state of the sources (`carried_to`: that state's hash and
+    the reason why the change cannot have moved the kernel's memory traffic), for changes that
+    leave the measured instance's loop and addresses as they were."""
     pdir = os.path.join(ROOT, "profiles")
     if not os.path.isdir(pdir):
         return None
@@ -55,7 +76,10 @@ def measured_traffic(kernel_name):
                 continue
             try:
                 rec = json.loads(line[len("traffic_json:"):])
-                if rec["kernel"] != kernel_name or rec["source_hash"] != kernel_source_hash(rec["sources"]):
+                if rec["kernel"] != kernel_name:
+                    continue
+                now = kernel_source_hash(rec["sources"])
+                if now != rec["source_hash"] and now != rec.get("carried_to", {}).get("source_hash"):
                     continue
                 return (rec["fetch_kib"] * rec["fetch_scale"] + rec["write_kib"] * rec["write_scale"]) * 1024.0
             except (ValueError, KeyError, OSError):

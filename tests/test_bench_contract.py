@@ -27,7 +27,15 @@ def test_counter_summaries_match_the_kernel_sources():
         "C5a": (_lib.AMOS_OP_BGEMM, ops.bgemm_desc(192, 512, 512, 64, torch.float16, False, True)),
         "C5b": (_lib.AMOS_OP_CONV3D, ops.conv_desc((8, 64, 16, 56, 56), (64, 64, 3, 3, 3), torch.float16, (1, 1, 1), (1, 1, 1), (1, 1, 1))),
     }
+    stale = bench.stale_summaries()
     for name, (op, desc) in configs.items():
         kernel = ops.kernel_name(op, desc)      # the default configuration's kernel, as bench.py runs it
         traffic = bench.measured_traffic(kernel)
+        if traffic is None and name != "C2":
+            # A kernel that changed after its counters were read and could not be profiled again:
+            # the summary must say so, naming the kernel that ships now (bench.py then reports no
+            # traffic for it).  The headline kernel (roofline.traffic) has no such way out.
+            assert name in stale and stale[name]["kernel_now"] == kernel and stale[name]["why"], \
+                "%s: neither a current counter summary nor a stale_json line for %s" % (name, kernel)
+            continue
         assert traffic is not None and traffic > 0, "%s: no current counter summary for %s" % (name, kernel)

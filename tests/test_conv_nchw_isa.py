@@ -78,3 +78,21 @@ def test_the_check_sees_a_violation(tmp_path):
     assert any("scratch" in b for b in run(good, log.replace("ScratchSize [bytes/lane]: 0", "ScratchSize [bytes/lane]: 16")))
     assert any("register count" in b for b in run(good, log.replace("VGPRs: 168", "VGPRs: 124")))
     assert any("do not fit" in b for b in run(good, log.replace("Occupancy [waves/SIMD]: 3", "Occupancy [waves/SIMD]: 2")))
+    # an access through a generic address, anywhere in the kernel (an LDS offset of 0 turned into a
+    # generic pointer is the null pointer: the access goes to global address 0)
+    assert any("generic address" in b for b in run(good.replace("v_mov_b32_e32 v8, 3", "flat_store_dword v[2:3], v1 sc0 sc1")))
+    assert any("generic address" in b for b in run(good.replace("v_mov_b32_e32 v7, 2", "flat_load_dword v1, v[2:3]")))
+
+
+def test_a_spilling_instance_of_a_wait_counting_kernel_is_refused():
+    """the build reads every unit's resource remarks: scratch memory in a kernel that waits for its
+    own copies by count is a reason not to link, in any other kernel it is not"""
+    remark = ("remark: Function Name: %s\nremark:     VGPRs: 128\nremark:     AGPRs: 0\n"
+              "remark:     ScratchSize [bytes/lane]: %d\nremark:     Occupancy [waves/SIMD]: 4\n")
+    tn = "_ZN4amos12amos_gemm_tnILi0ELi256ELi256ELi2ELi2ELi3EEEvNS_12GemmTnParamsE"
+    other = "_ZN4amos10amos_igemmILi0ELi0ELi0ELi1ELi1EEEvNS_11IgemmParamsE"
+    assert isa_check.spills("x", remark % (tn, 0) + remark % (other, 24)) == []
+    bad = isa_check.spills("x", remark % (tn, 24) + remark % (other, 0))
+    assert len(bad) == 1 and "amos_gemm_tn" in bad[0] and "24 bytes" in bad[0]
+    for k in ("_ZN4amos15amos_conv_fpropILi0EEEvNS_15ConvFpropParamsE", "_ZN4amos14amos_conv_nchwILi0EEEvNS_14ConvNchwParamsE"):
+        assert len(isa_check.spills("x", remark % (k, 8))) == 1

@@ -535,7 +535,9 @@ def test_default_convolution_kernels():
     """what the mapper's model picks for the benchmark convolutions and a few network layers (the
     plan is host code: no GPU needed): the NCDHW-direct kernel with the weights read as they are
     where the packing launch would cost more than the transposes, packed where it would not, 16-byte
-    patch loads where a channel plane is whole 16-byte runs, the patch-staged kernel for int8"""
+    patch loads where a channel plane is whole 16-byte runs; for the int8 benchmark shape the
+    128-row workgroups (two halves of 64 output channels on one patch: its tiles in one round of
+    the compute units)"""
     import torch
     from amos_amd import _lib, ops
 
@@ -545,9 +547,9 @@ def test_default_convolution_kernels():
     assert name((32, 256, 1, 14, 14), (256, 256, 1, 3, 3)) == "amos_conv_nchw<f16,64x128,8+4w,kcrs>"
     assert name((8, 64, 16, 56, 56), (64, 64, 3, 3, 3), op=_lib.AMOS_OP_CONV3D, pad=(1, 1, 1)) == \
         "amos_conv_nchw<f16,64x256,8+4w,packed,ld16>"
-    assert name((64, 128, 1, 28, 28), (128, 128, 1, 3, 3), torch.int8).startswith("amos_conv_fprop<i8,")
+    assert name((64, 128, 1, 28, 28), (128, 128, 1, 3, 3), torch.int8) == "amos_conv_nchw<i8,2x64x256,8+4w,kcrs>"
     assert name((16, 64, 1, 56, 56), (64, 64, 1, 3, 3)) == "amos_conv_nchw<f16,64x256,8+4w,kcrs,ld16>"
-    assert name((64, 512, 1, 14, 14), (512, 512, 1, 3, 3)) == "amos_conv_nchw<f16,64x256,8+4w,packed,pt2>"
+    assert name((64, 512, 1, 14, 14), (512, 512, 1, 3, 3)) == "amos_conv_nchw<f16,2x64x256,8+4w,packed,pt2>"
     # a channel count that does not fill 64-byte chunks, a 5x5 window: not this kernel's
     assert not name((2, 24, 1, 14, 14), (40, 24, 1, 3, 3)).startswith("amos_conv_nchw")
     assert not name((4, 64, 1, 30, 30), (96, 64, 1, 5, 5), pad=(0, 2, 2)).startswith("amos_conv_nchw")
