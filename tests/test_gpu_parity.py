@@ -663,9 +663,9 @@ def test_conv_layouts(gpu, layout, dtype, case):
 
 
 def test_conv_defaults_when_applicable(gpu):
-    """the kernel that reads the activations as they are for the fp16 3x3 benchmark shapes, the
-    patch-staged one for the int8 shape (as measured and as the planner's model says), the
-    register-staged one where neither applies"""
+    """the kernel that reads the activations as they are for the 3x3 benchmark shapes (the int8 one
+    with 128-row workgroups: one round of the compute units, as measured and as the planner's model
+    says), the register-staged one where neither it nor the patch-staged kernel applies"""
     import torch
     from amos_amd import _lib, ops
     d = ops.conv_desc((32, 256, 1, 14, 14), (256, 256, 1, 3, 3), torch.float16, (1, 1, 1), (0, 1, 1), (1, 1, 1))
@@ -673,7 +673,7 @@ def test_conv_defaults_when_applicable(gpu):
     d = ops.conv_desc((8, 64, 16, 56, 56), (64, 64, 3, 3, 3), torch.float16, (1, 1, 1), (1, 1, 1), (1, 1, 1))
     assert ops.kernel_name(_lib.AMOS_OP_CONV3D, d).startswith("amos_conv_nchw<f16,64x256,")
     d = ops.conv_desc((64, 128, 1, 28, 28), (128, 128, 1, 3, 3), torch.int8, (1, 1, 1), (0, 1, 1), (1, 1, 1))
-    assert ops.kernel_name(_lib.AMOS_OP_CONV2D, d).startswith("amos_conv_fprop<i8,")
+    assert ops.kernel_name(_lib.AMOS_OP_CONV2D, d) == "amos_conv_nchw<i8,2x64x256,8+4w,kcrs>"
     d = ops.conv_desc((2, 24, 1, 14, 14), (40, 24, 1, 3, 3), torch.float16, (1, 1, 1), (0, 1, 1), (1, 1, 1))
     assert ops.kernel_name(_lib.AMOS_OP_CONV2D, d).startswith("amos_igemm<f16,")
 
