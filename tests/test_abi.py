@@ -294,3 +294,68 @@ def test_gemm_tn_fragment_and_strip_offsets_stay_inside_lds(WI, WJ):
         assert (wave + 1) * 16 * SP * 4 <= NS * STAGE
     assert rows_a == {(r, wj) for r in range(BI) for wj in range(WJ)}
     assert rows_b == {(r, wi) for r in range(BJ) for wi in range(WI)}
+
+
+@pytest.mark.parametrize("WI,WJ,BI,BJ,NS", [(4, 2, 256, 256, 2), (2, 4, 128, 128, 2), (2, 4, 128, 256, 3), (4, 2, 256, 128, 3)])
+def test_gemm_tn_output_strips_cover_every_element_once(WI, WJ, BI, BJ, NS):
+    """the epilogue of every shipped direct-to-LDS instance on the host (gemm_tn_kernel.h): a wave
+    writes a 16-row block of accumulators into its LDS strip in the matrix core's layout (lane l:
+    column l % 16, rows 4 * (l / 16) + r) and reads it back as 16-byte pieces (TJ instructions of
+    64 / (4 TJ) rows x the wave tile's width).  Every element of the block tile must leave in
+    exactly one piece, from the strip slot it was written to, and the strips of the eight waves
+    must fit the LDS stages they reuse"""
+    NW = WI * WJ
+    TI, TJ = BI // (16 * WI), BJ // (16 * WJ)
+    assert TJ >= 2 and TJ & (TJ - 1) == 0
+    SP, CPR = TJ * 16 + 4, TJ * 4
+    RPI = 64 // CPR
+    assert NW * 16 * SP * 4 <= NS * (BI + BJ) * 128
+    stored = {}
+    for wave in range(NW):
+        wi, wj = wave // WJ, wave % WJ
+        for a in range(TI):
+            slot_of = {}                        # strip slot -> (row, column) of the tile written there
+            for lane in range(64):
+                frag_row, frag_q = lane & 15, lane >> 4
+                for b in range(TJ):
+                    for r in range(4):
+                        slot = (4 * frag_q + r) * SP + b * 16 + frag_row
+                        assert slot not in slot_of and slot < 16 * SP
+                        slot_of[slot] = ((wi * TI + a) * 16 + 4 * frag_q + r, (wj * TJ + b) * 16 + frag_row)
+            for lane in range(64):
+                for n in range(TJ):
+                    base = (n * RPI + lane // CPR) * SP + (lane % CPR) * 4
+                    i = (wi * TI + a) * 16 + n * RPI + lane // CPR
+                    j = wj * TJ * 16 + (lane % CPR) * 4
+                    for e in range(4):
+                        assert slot_of[base + e] == (i, j + e)
+                        assert (i, j + e) not in stored
+                        stored[(i, j + e)] = wave
+    assert len(stored) == BI * BJ
+
+
+@pytest.mark.parametrize("tiles_i,tiles_j,batches", [(4, 4, 192), (1, 1, 8), (9, 3, 16), (8, 5, 24), (17, 2, 8), (3, 7, 40)])
+def test_gemm_tn_batches_go_to_xcds_whole(tiles_i, tiles_j, batches):
+    """the workgroup renumbering of a batched launch (gemm_tn_kernel.h; gridDim = (T, 1, batches),
+    batches a multiple of 8) on the host: workgroups reach the 8 XCDs round-robin in launch order
+    L = x + T * z; XCD L % 8 takes tile (L / 8) % T of batch L % 8 + 8 * ((L / 8) / T).  Every
+    (batch, tile) must be computed exactly once, every tile index must lie inside the tile grid,
+    and all tiles of a batch must run on one XCD"""
+    T = tiles_i * tiles_j
+    seen, xcd_of_batch = set(), {}
+    for z in range(batches):
+        for x in range(T):
+            L = x + T * z
+            xcd, sq = L & 7, L >> 3
+            tile, batch = sq % T, xcd + 8 * (sq // T)
+            per_group = 8 * tiles_j
+            gidx = tile // per_group
+            first_i = gidx * 8
+            rows_here = min(tiles_i - first_i, 8)
+            in_group = tile - gidx * per_group
+            ti, tj = first_i + in_group % rows_here, in_group // rows_here
+            assert 0 <= batch < batches and 0 <= ti < tiles_i and 0 <= tj < tiles_j
+            assert (batch, ti, tj) not in seen
+            seen.add((batch, ti, tj))
+            assert xcd_of_batch.setdefault(batch, xcd) == xcd
+    assert len(seen) == batches * T

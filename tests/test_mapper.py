@@ -998,3 +998,52 @@ def test_variance_lowering():
     got = (lhs @ low.constants[1].astype(np.float64)).reshape(-1)
     assert lhs.shape == (C, N * H * W) and np.allclose(got, want, rtol=1e-3)
 
+
+
+def dilated_conv2d_as_scripted(N, C, H, W, K, R, S, stride, padding, dilation, in_dtype="float16", out_dtype="float32"):
+    """the compute of benchmark/amos/mapping_dilatedconv2d_tensorcore.py:7-44 as it is spelled there:
+    the reduce axes rr, rs run over the DILATED window's extents kH, kW (the tutorial's conv2d runs
+    them over R, S) and index the filter B[k, rc, rr, rs] with them"""
+    kH, kW = (R - 1) * dilation + 1, (S - 1) * dilation + 1
+    pH, pW = H + 2 * padding, W + 2 * padding
+    A = te.placeholder([N, C, H, W], dtype=in_dtype, name="A")
+    B = te.placeholder([K, C, R, S], dtype=in_dtype, name="B")
+    Pad = te.compute([N, C, pH, pW], lambda n, c, h, w: tir.if_then_else(
+        tir.all(h >= padding, h - padding < H, w >= padding, w - padding < W),
+        A[n, c, h - padding, w - padding], tir.const(0.0, A.dtype)), name="Pad")
+    rc, rr, rs = te.reduce_axis([0, C], name="rc"), te.reduce_axis([0, kH], name="rr"), te.reduce_axis([0, kW], name="rs")
+    P, Q = (pH - kH) // stride + 1, (pW - kW) // stride + 1
+    Conv = te.compute([N, K, P, Q], lambda n, k, p, q: te.sum(
+        (Pad[n, rc, p * stride + rr * dilation, q * stride + rs * dilation] * B[k, rc, rr, rs]).astype(out_dtype),
+        axis=[rc, rr, rs]), name="Conv")
+    return A, B, Conv
+
+
+def test_dilated_conv_script_lowers_at_its_own_shapes():
+    """every shape mapping_dilatedconv2d_tensorcore.py:122-129 runs has a 1x1 window (dilation 2 of
+    one tap: kH = kW = 1 = R = S), where the script's spelling IS a convolution -- a pointwise one,
+    whatever the dilation; with a wider window the same spelling indexes the filter past its
+    extent (rr up to (R - 1) * dilation), which no convolution descriptor means: refused"""
+    from amos_amd.auto_tensorize.lowering import NoKernelError, lower_main_op
+    shapes_b1 = [(256, 56, 56, 512), (256, 56, 56, 128), (512, 28, 28, 1024), (512, 28, 28, 256), (1024, 14, 14, 2048),
+                 (1024, 14, 14, 512)]
+    for C, H, W, K in shapes_b1:
+        A, B, Conv = dilated_conv2d_as_scripted(1, C, H, W, K, 1, 1, 1, 0, 2)
+        low = lower_main_op(Conv.op, at.compute_dag_from_tensors([Conv]))
+        d = low.desc
+        assert low.kind == "conv2d" and (d.N, d.C, d.H, d.W, d.K, d.R, d.S) == (1, C, H, W, K, 1, 1)
+        assert [int(x) for x in Conv.shape] == [1, K, H, W]
+        name = _lib.load().amos_kernel_name(low.op_code, __import__("ctypes").byref(d), None)
+        assert name is not None and (b"amos_gemm_tn" in name or b"amos_igemm" in name), name   # a matrix product
+    # the interpreter agrees with the oracle's convolution on a small instance of the same spelling
+    from oracle import cpu_oracle as co, te_interp
+    rng = np.random.default_rng(3)
+    A, B, Conv = dilated_conv2d_as_scripted(2, 8, 5, 6, 4, 1, 1, 1, 0, 2)
+    a = rng.uniform(-1, 1, (2, 8, 5, 6)).astype(np.float16)
+    b = rng.uniform(-1, 1, (4, 8, 1, 1)).astype(np.float16)
+    got = te_interp.evaluate(Conv, {"A": a, "B": b})
+    ref = co.te_literal_conv2d(a, b, "float16", 1, 0, 1)
+    assert np.allclose(got, ref, atol=1e-3, rtol=1e-3)
+    A, B, Conv = dilated_conv2d_as_scripted(1, 64, 14, 14, 64, 3, 3, 1, 2, 2)
+    with pytest.raises(NoKernelError, match="reduce extent 5 differs from the kernel window 3"):
+        lower_main_op(Conv.op, at.compute_dag_from_tensors([Conv]))
