@@ -3,7 +3,9 @@
 // matrix-core instructions of a 128x128 wave tile x 512 K steps of 64 = 1.0995e12 flop per launch)
 // and, optionally, the data movement a 256x256x64 tiling needs next to them -- global -> LDS
 // copies (64 KB per K step and workgroup) and LDS fragment reads (32 x 16 bytes per lane and K
-// step) -- with no wait or barrier anywhere.  The operands of the matrix-core instructions never
+// step) -- with no barrier and no wait for a copy anywhere; a read's data is consumed (XORed into
+// a running value) behind the next two (32x32x16) / four (16x16x32) matrix-core instructions, so a
+// wave has one read in flight and waits for it only if LDS takes longer than those take to issue.  The operands of the matrix-core instructions never
 // change: either small constants or random fp16 values read once from the caller's buffers, which
 // is what decides the clock the chip holds (the switching activity of the multipliers).
 //
