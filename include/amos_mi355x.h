@@ -340,9 +340,10 @@ int amos_time_eltwise(const amos_eltwise_desc_t* desc, const void* const* inputs
 /*
  * What the matrix cores sustain on this device when nothing else limits them: `launches`
  * back-to-back launches of a measurement kernel with the matrix-core instruction stream of the
- * 8192^3 fp16 product (256 workgroups x 4 waves, 1.0995e12 flop per launch) and no wait or barrier
- * anywhere; mean seconds per launch by HIP events on `stream` and the flop of a launch are
- * written out.  Synchronises the stream.
+ * 8192^3 fp16 product (256 workgroups x 4 waves, 1.0995e12 flop per launch), no barrier and no
+ * wait for a copy anywhere (a wave keeps one LDS read in flight and consumes it behind the next
+ * two to four matrix-core instructions); mean seconds per launch by HIP events on `stream` and the
+ * flop of a launch are written out.  Synchronises the stream.
  *   shape            16: v_mfma_f32_16x16x32_f16, 32: v_mfma_f32_32x32x16_f16
  *   random_operands  0: small constants built in registers; 1: the operands of the instructions are
  *                    read (once) from a and b -- the switching activity of the multipliers, and

@@ -359,3 +359,22 @@ def test_gemm_tn_batches_go_to_xcds_whole(tiles_i, tiles_j, batches):
             seen.add((batch, ti, tj))
             assert xcd_of_batch.setdefault(batch, xcd) == xcd
     assert len(seen) == batches * T
+
+
+def test_mfma_ceiling_refuses_bad_arguments_before_any_launch():
+    """amos_mfma_ceiling checks its arguments on the host: an instruction shape it does not have,
+    null buffers, buffers too small for the variant asked for (8 MiB per operand without the
+    copies, a whole 8192 x 8192 fp16 matrix with them), a misaligned buffer"""
+    import ctypes
+    lib = _lib.load()
+    sec, flop = ctypes.c_double(), ctypes.c_double()
+    buf = ctypes.create_string_buffer(64)          # (never dereferenced: every call below is refused)
+    a = ctypes.addressof(buf) & ~15
+    big = 8192 * 8192 * 2
+    cases = [(8, 0, 0, 0, a, a, big, a, 1), (16, 0, 0, 0, None, a, big, a, 1), (16, 0, 0, 0, a, a, big, None, 1),
+             (16, 0, 0, 0, a, a, big, a, 0), (16, 1, 0, 0, a, a, (8 << 20) - 1, a, 1), (32, 1, 1, 0, a, a, big - 1, a, 1),
+             (32, 1, 0, 0, a + 2, a, big, a, 1)]
+    for shape, rnd, copies, reads, pa, pb, nbytes, sink, launches in cases:
+        rc = lib.amos_mfma_ceiling(shape, rnd, copies, reads, pa, pb, nbytes, sink, launches, None,
+                                   ctypes.byref(sec), ctypes.byref(flop))
+        assert rc == _lib.AMOS_ERR_BAD_ARG and b"amos_mfma_ceiling" in lib.amos_last_error(), (shape, rnd, copies, nbytes)
