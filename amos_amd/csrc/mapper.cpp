@@ -14,6 +14,8 @@
 #include <cmath>
 #include <cstring>
 #include <mutex>
+#include <string>
+#include <unordered_map>
 #include <vector>
 
 #include "conv_nchw_geom.h"
@@ -951,7 +953,36 @@ int amos_estimate_seconds(int op, const void* desc, const amos_kernel_config_t* 
   return 0;
 }
 
+// The choice is a function of the operator, its descriptor and the device's compute units, and
+// costs some 150 evaluations of the model: a call that names no configuration would pay that on
+// the host every time (tens of microseconds, more than many of the kernels take).  The last few
+// hundred choices are therefore kept, keyed by the descriptor's bytes.
+static int default_config_of(int op, const void* desc, amos_kernel_config_t* result);
+
 int amos_default_config(int op, const void* desc, amos_kernel_config_t* result) {
+  const size_t n = op == AMOS_OP_GEMM ? sizeof(amos_gemm_desc_t) : op == AMOS_OP_BGEMM ? sizeof(amos_bgemm_desc_t)
+                   : (op == AMOS_OP_CONV2D || op == AMOS_OP_CONV3D) ? sizeof(amos_conv_desc_t) : 0;
+  if (!desc || !result || n == 0) return default_config_of(op, desc, result);
+  static std::mutex mu;
+  static std::unordered_map<std::string, amos_kernel_config_t> kept;
+  std::string key((const char*)desc, n);
+  const int tag[2] = {op, device_compute_units()};
+  key.append((const char*)tag, sizeof(tag));
+  {
+    std::lock_guard<std::mutex> lock(mu);
+    auto it = kept.find(key);
+    if (it != kept.end()) { *result = it->second; return 0; }
+  }
+  const int rc = default_config_of(op, desc, result);
+  if (rc == 0) {
+    std::lock_guard<std::mutex> lock(mu);
+    if (kept.size() >= 512) kept.clear();
+    kept[key] = *result;
+  }
+  return rc;
+}
+
+static int default_config_of(int op, const void* desc, amos_kernel_config_t* result) {
   Problem pb;
   int rc = problem_of(op, desc, &pb);
   if (rc) return rc;

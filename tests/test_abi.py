@@ -378,3 +378,37 @@ def test_mfma_ceiling_refuses_bad_arguments_before_any_launch():
         rc = lib.amos_mfma_ceiling(shape, rnd, copies, reads, pa, pb, nbytes, sink, launches, None,
                                    ctypes.byref(sec), ctypes.byref(flop))
         assert rc == _lib.AMOS_ERR_BAD_ARG and b"amos_mfma_ceiling" in lib.amos_last_error(), (shape, rnd, copies, nbytes)
+
+
+def test_default_config_is_kept_per_descriptor():
+    """amos_default_config keeps its last choices keyed by the descriptor: the same answer on every
+    call (a call that names no configuration asks for it every time), each descriptor its own, and
+    repeated calls at a cost far below the ~150 model evaluations of a first call"""
+    import ctypes
+    import time
+    import torch
+    from amos_amd import ops
+    lib = _lib.load()
+    descs = [(_lib.AMOS_OP_GEMM, ops.gemm_desc(m, 512, 1024, torch.float16, False, True)) for m in (64, 512, 4096, 8192)]
+    descs += [(_lib.AMOS_OP_CONV2D, ops.conv_desc((n, 128, 1, 28, 28), (128, 128, 1, 3, 3), dt, (1, 1, 1), (0, 1, 1), (1, 1, 1)))
+              for n in (1, 16, 64) for dt in (torch.float16, torch.int8)]
+    descs.append((_lib.AMOS_OP_BGEMM, ops.bgemm_desc(192, 512, 512, 64, torch.float16, False, True)))
+    first = []
+    for op, d in descs:
+        c = _lib.KernelConfig()
+        assert lib.amos_default_config(op, ctypes.byref(d), ctypes.byref(c)) == 0
+        first.append((c.tile_i, c.tile_j, c.split_k, c.pipeline))
+    assert len(set(first)) > 3                      # (the shapes do not all get one answer)
+    t0 = time.perf_counter()
+    for _ in range(50):
+        for (op, d), want in zip(descs, first):
+            c = _lib.KernelConfig()
+            assert lib.amos_default_config(op, ctypes.byref(d), ctypes.byref(c)) == 0
+            assert (c.tile_i, c.tile_j, c.split_k, c.pipeline) == want
+    per_call = (time.perf_counter() - t0) / (50 * len(descs))
+    assert per_call < 20e-6, per_call
+    # an invalid descriptor is refused every time (errors are not kept)
+    bad = ops.gemm_desc(64, 64, 64, torch.float16, False, True)
+    bad.M = -1
+    for _ in range(2):
+        assert lib.amos_default_config(_lib.AMOS_OP_GEMM, ctypes.byref(bad), ctypes.byref(_lib.KernelConfig())) != 0
