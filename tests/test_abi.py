@@ -412,3 +412,62 @@ def test_default_config_is_kept_per_descriptor():
     bad.M = -1
     for _ in range(2):
         assert lib.amos_default_config(_lib.AMOS_OP_GEMM, ctypes.byref(bad), ctypes.byref(_lib.KernelConfig())) != 0
+
+
+def test_planner_is_consistent_with_itself_on_random_shapes():
+    """seeded random GEMMs, batched GEMMs and convolutions (2-d, 3-d, grouped, depthwise; windows
+    1 to 7, strides, paddings): amos_default_config's choice passes amos_check_config, has a kernel
+    instance (as does a null configuration), an estimate and a sane workspace size"""
+    import ctypes
+    import torch
+    from amos_amd import ops
+    lib = _lib.load()
+    import numpy as np
+    rng = np.random.default_rng(7)
+    checked = 0
+    for _ in range(500):
+        kind = int(rng.integers(0, 4))
+        dt = [torch.float16, torch.bfloat16, torch.int8][int(rng.integers(0, 3))]
+        if kind == 0:
+            M, N, K = [int(x) for x in rng.choice([1, 3, 8, 17, 64, 96, 128, 200, 512, 1000, 2048, 4096, 8192], 3)]
+            op, d = _lib.AMOS_OP_GEMM, ops.gemm_desc(M, N, K, dt, bool(rng.integers(0, 2)), bool(rng.integers(0, 2)))
+            what = ("gemm", M, N, K, dt)
+        elif kind == 1:
+            B = int(rng.choice([1, 2, 8, 16, 24, 192]))
+            M, N, K = [int(x) for x in rng.choice([8, 64, 128, 512, 1024], 3)]
+            op, d = _lib.AMOS_OP_BGEMM, ops.bgemm_desc(B, M, N, K, dt, bool(rng.integers(0, 2)), bool(rng.integers(0, 2)))
+            what = ("bgemm", B, M, N, K, dt)
+        else:
+            three = kind == 3
+            n, C = int(rng.choice([1, 2, 8, 16, 32, 64])), int(rng.choice([3, 16, 24, 32, 64, 96, 128, 256, 512]))
+            K = int(rng.choice([8, 32, 64, 72, 128, 256, 512]))
+            H = int(rng.choice([7, 14, 28, 56, 112]))
+            W = H if rng.integers(0, 2) else int(rng.choice([7, 9, 14, 30]))
+            D = int(rng.choice([1, 4, 16])) if three else 1
+            R = int(rng.choice([1, 3, 5, 7]))
+            T = int(rng.choice([1, 3])) if three else 1
+            st, pd = int(rng.choice([1, 2])), int(rng.choice([0, 1, R // 2]))
+            groups = 1
+            if rng.integers(0, 6) == 0 and C % 4 == 0 and K % 4 == 0:
+                groups = 4
+            if rng.integers(0, 8) == 0:
+                groups, K = C, C
+            xs, ws = (n, C, D, H, W), (K, C // groups, T, R, R)
+            stride, pad = (st if three else 1, st, st), (pd if three else 0, pd, pd)
+            if min(ops.conv_out_shape(xs, ws, stride, pad, (1, 1, 1))) <= 0:
+                continue
+            op = _lib.AMOS_OP_CONV3D if three else _lib.AMOS_OP_CONV2D
+            d = ops.conv_desc(xs, ws, dt, stride, pad, (1, 1, 1), groups)
+            what = ("conv", xs, ws, st, pd, groups, dt)
+        c = _lib.KernelConfig()
+        assert lib.amos_default_config(op, ctypes.byref(d), ctypes.byref(c)) == 0, (what, lib.amos_last_error())
+        cfg = (c.tile_i, c.tile_j, c.split_k, c.pipeline)
+        assert lib.amos_kernel_name(op, ctypes.byref(d), ctypes.byref(c)) is not None, (what, cfg, lib.amos_last_error())
+        assert lib.amos_kernel_name(op, ctypes.byref(d), None) is not None, (what, lib.amos_last_error())
+        assert lib.amos_check_config(op, ctypes.byref(d), ctypes.byref(c), None, None) >= 0, (what, cfg, lib.amos_last_error())
+        est = ctypes.c_double()
+        assert lib.amos_estimate_seconds(op, ctypes.byref(d), ctypes.byref(c), ctypes.byref(est)) == 0 and 0 < est.value < 10, (what, cfg)
+        assert 0 <= lib.amos_workspace_bytes(op, ctypes.byref(d), ctypes.byref(c)) < (64 << 30), (what, cfg)
+        assert 0 <= lib.amos_workspace_bytes(op, ctypes.byref(d), None) < (64 << 30), what
+        checked += 1
+    assert checked > 400
