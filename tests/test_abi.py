@@ -471,3 +471,42 @@ def test_planner_is_consistent_with_itself_on_random_shapes():
         assert 0 <= lib.amos_workspace_bytes(op, ctypes.byref(d), None) < (64 << 30), what
         checked += 1
     assert checked > 400
+
+
+@pytest.mark.parametrize("BI,BJ,WI,WJ,HV", [(64, 128, 2, 4, 1), (64, 256, 1, 8, 1), (32, 128, 1, 4, 1), (32, 256, 1, 4, 1),
+                                            (64, 128, 2, 4, 2), (64, 256, 1, 8, 2)])
+def test_conv_nchw_output_strips_cover_every_element_once(BI, BJ, WI, WJ, HV):
+    """the strip epilogue of every NCDHW-direct instance on the host (conv_nchw_kernel.h): per
+    16-row block and half of the output channels a matrix-core wave writes its accumulators into
+    its LDS strip in the matrix core's layout and reads them back as 16-byte pieces of whole rows.
+    Every element of the (HV * BI) x BJ tile leaves exactly once, from the slot it was written to;
+    the eight (four) strips fit the two weight buffers they reuse"""
+    NWM = WI * WJ
+    TI, TJ = BI // (16 * WI), BJ // (16 * WJ)
+    assert TJ & (TJ - 1) == 0 and TJ <= 16
+    SP, CPR = TJ * 16 + 4, TJ * 4
+    RPI = 64 // CPR
+    assert NWM * 16 * SP * 4 <= 2 * 9 * BI * 64
+    stored = set()
+    for wave in range(NWM):
+        wi, wj = wave // WJ, wave % WJ
+        for ha in range(HV * TI):
+            h, a = ha // TI, ha % TI
+            slot_of = {}
+            for lane in range(64):
+                frag_row, frag_q = lane & 15, lane >> 4
+                for b in range(TJ):
+                    for r in range(4):
+                        slot = (4 * frag_q + r) * SP + b * 16 + frag_row
+                        assert slot not in slot_of and slot < 16 * SP
+                        slot_of[slot] = (h * BI + (wi * TI + a) * 16 + 4 * frag_q + r, (wj * TJ + b) * 16 + frag_row)
+            for lane in range(64):
+                for x in range(TJ):
+                    base = (x * RPI + lane // CPR) * SP + (lane % CPR) * 4
+                    i = h * BI + (wi * TI + a) * 16 + x * RPI + lane // CPR
+                    j4 = wj * TJ * 16 + (lane % CPR) * 4
+                    for e in range(4):
+                        assert slot_of[base + e] == (i, j4 + e)
+                        assert (i, j4 + e) not in stored
+                        stored.add((i, j4 + e))
+    assert len(stored) == HV * BI * BJ
