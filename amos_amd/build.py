@@ -11,6 +11,10 @@ OUT = os.path.join(HERE, "libamos_mi355x.so")
 # -packed-fp32-ops is switched off: the compiler must not form v_pk_*_f32
 HIP_FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-Xclang", "-target-feature",
              "-Xclang", "-packed-fp32-ops", "-Wno-unused-command-line-argument"]
+# AMOS_BUILD_SPLIT_IN_KERNEL=1 in the environment of the build compiles the split-K tails into the
+# kernels (igemm_kernel.h: split_finish); the default library does not have them
+if os.environ.get("AMOS_BUILD_SPLIT_IN_KERNEL") == "1":
+    HIP_FLAGS.append("-DAMOS_SPLIT_IN_KERNEL=1")
 
 
 def sources():

@@ -1246,6 +1246,7 @@ static int launch_conv_nchw(const Plan& pl, hipStream_t stream) {
 
 static int launch_kernels(const Plan& pl, hipStream_t stream);
 
+#if AMOS_SPLIT_IN_KERNEL
 // Ticket counters of the in-kernel split-K reduction (SplitFinish): the library's own, one array per
 // GPU, zero when the module is loaded and put back to zero by the workgroup that draws a tile's
 // last ticket.  A launch takes a run of counters of its own from a rotating position, so launches
@@ -1277,8 +1278,9 @@ static unsigned* tickets_for(int64_t n) {
   }
 }
 
-// The in-kernel reduction is opt-in (environment AMOS_SPLIT_IN_KERNEL=1, read once): without it
-// every split adds its slices with the launch of its own below, the path every test has run on.
+// In a library built with the tails (-DAMOS_SPLIT_IN_KERNEL=1) the in-kernel reduction is still
+// opt-in (environment AMOS_SPLIT_IN_KERNEL=1, read once): without it every split adds its slices
+// with the launch of its own below, the path every test has run on.
 static bool split_in_kernel() {
   static const bool on = [] {
     const char* v = getenv("AMOS_SPLIT_IN_KERNEL");
@@ -1286,11 +1288,13 @@ static bool split_in_kernel() {
   }();
   return on;
 }
+#endif
 
 // the kernels of the plan; split-K with partial sums: a launch of its own adds the slices, or --
 // opted in, no more tiles than there are counters, a kernel with that tail -- the last workgroup
 // of every tile does
 static int launch(const Plan& pl, hipStream_t stream) {
+#if AMOS_SPLIT_IN_KERNEL
   if (pl.part && split_in_kernel()) {
     const bool own_tail = pl.nchw || pl.tn_waves || (pl.conv_ups && !(pl.conv_w9 == 2)) ||
                           (!pl.conv_ups && !pl.skinny && !pl.dw && !pl.fewc);
@@ -1306,6 +1310,7 @@ static int launch(const Plan& pl, hipStream_t stream) {
       return launch_kernels(armed, stream);
     }
   }
+#endif
   int rc = launch_kernels(pl, stream);
   if (rc || !pl.part) return rc;
   const int64_t n = pl.fill_rows * pl.fill_cols;
@@ -1430,9 +1435,11 @@ static int plan_epilogue(Plan& pl, int op, const void* desc, const amos_epilogue
       ep.batch = pl.p.out_batch;
     }
   }
+#if AMOS_SPLIT_IN_KERNEL
   // (no in-kernel reduction of a split unless the launch arms it)
   const SplitFinish no_fin = {nullptr, nullptr, 0, 0};
   pl.p.fin = no_fin; pl.tn.fin = no_fin; pl.cv.fin = no_fin; pl.nc.fin = no_fin;
+#endif
   pl.p.epi = ep;
   pl.tn.epi = ep;
   pl.cv.epi = ep;

@@ -76,7 +76,9 @@ struct ConvFpropParams {
   int prep_w_blocks, prep_x_blocks, prep_z_blocks;
   int64_t zero_words;
   EpiParams epi;     // fused tail: Y = acc + cast(D), D laid out like Y
+#if AMOS_SPLIT_IN_KERNEL
   SplitFinish fin;   // split-K: the last workgroup of a tile adds the slices
+#endif
   // tensor layouts (AMOS_LAYOUT_*): 0 = NCDHW / KCTRS / NKDPQ, 1 = NDHWC / TRSCK / NDPQK,
   // 2 = DHWNC / TRSCK / DPQNK.  Output element (i, j), j = n*ODPQ + s, at i*y_si + n*y_sn + s*y_ss.
   int layout;
@@ -893,6 +895,7 @@ __global__ __launch_bounds__(64 * NW, OCC) void amos_conv_fprop(const ConvFpropP
   if constexpr (!PERSIST) store_tile(geo);
   // the re-fetched tiles of the last steps still target this block's LDS
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+#if AMOS_SPLIT_IN_KERNEL
   if constexpr (!PERSIST) {
     if (p.fin.tickets) {
       const int ODPQ = p.OD * OPQ;
@@ -905,6 +908,7 @@ __global__ __launch_bounds__(64 * NW, OCC) void amos_conv_fprop(const ConvFpropP
                           });
     }
   }
+#endif
 }
 
 }  // namespace amos

@@ -51,7 +51,9 @@ struct ConvNchwParams {
   int64_t split_stride;  // elements between the partial outputs of the split-K blocks
   NchwDiv div_cc, div_odpq;
   EpiParams epi;         // fused tail: Y = acc + cast(D), D laid out like Y
+#if AMOS_SPLIT_IN_KERNEL
   SplitFinish fin;       // split-K: the last workgroup of a tile adds the slices
+#endif
 };
 
 #define AMOS_LDS_ADDR(off) ((__attribute__((address_space(3))) char*)(size_t)(off))
@@ -728,6 +730,7 @@ __global__ __launch_bounds__(64 * (WI * WJ + NWL)) void amos_conv_nchw(const Con
     }
   }
   }
+#if AMOS_SPLIT_IN_KERNEL
   if (p.fin.tickets) {
     // (the loader waves have left: the matrix-core waves' threads are the workgroup now)
     split_finish<out_t>(p.fin, blockIdx.x, (const out_t*)p.y, t, NTM, BI * HV, BJ, (lds_flag_t)(size_t)0,
@@ -738,6 +741,7 @@ __global__ __launch_bounds__(64 * (WI * WJ + NWL)) void amos_conv_nchw(const Con
                           return ((int64_t)n * s.K + i) * ODPQ + (j - n * ODPQ);
                         });
   }
+#endif
 }
 
 }  // namespace amos

@@ -41,7 +41,9 @@ struct GemmTnParams {
   int kt_per_split;       // split-K: blockIdx.y takes the K tiles [y * kt_per_split, (y + 1) * kt_per_split) ...
   int64_t split_stride;   // ... and stores its partial sums at c + y * split_stride (0: no split)
   EpiParams epi;   // fused tail: C = acc + cast(D), D[i][j] at i*epi.si + j
+#if AMOS_SPLIT_IN_KERNEL
   SplitFinish fin; // split-K: the last workgroup of a tile adds the slices
+#endif
 };
 
 #define AMOS_GLOBAL_PTR(p) ((const __attribute__((address_space(1))) void*)(p))
@@ -308,6 +310,7 @@ __global__ __launch_bounds__(64 * WI * WJ) void amos_gemm_tn(const GemmTnParams 
     }
   }
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+#if AMOS_SPLIT_IN_KERNEL
   if (p.fin.tickets) {
     // (the tile index is taken from the launch grid, whatever walk mapped it to (tile_i, tile_j))
     split_finish<out_t>(p.fin, (unsigned)(blockIdx.z * gridDim.x + blockIdx.x), (const out_t*)p.c, t, 64 * NW, BI, BJ,
@@ -316,6 +319,7 @@ __global__ __launch_bounds__(64 * WI * WJ) void amos_gemm_tn(const GemmTnParams 
                           return i < p.I && j < p.J ? batch * p.batch_c + (int64_t)i * p.ldc + j : (int64_t)-1;
                         });
   }
+#endif
 }
 
 }  // namespace amos

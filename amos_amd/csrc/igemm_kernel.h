@@ -99,6 +99,12 @@ __device__ __forceinline__ int epi_value<int>(const EpiParams& e, int64_t idx) {
   return ((const int*)e.ptr)[idx];
 }
 
+// (Compiled in only with -DAMOS_SPLIT_IN_KERNEL=1: the default build's kernels are, instruction for
+// instruction, the ones without this tail.)
+#ifndef AMOS_SPLIT_IN_KERNEL
+#define AMOS_SPLIT_IN_KERNEL 0
+#endif
+#if AMOS_SPLIT_IN_KERNEL
 // Split-K without a second launch: every split stores its partial tile into its own slice (as
 // for the reduction launch), then takes a ticket of the tile; the workgroup that draws the last
 // one adds the slices IN THE ORDER OF THE SPLITS -- the same bits whichever workgroup that is --
@@ -138,6 +144,7 @@ __device__ __forceinline__ void split_finish(const SplitFinish& f, unsigned tile
   }
   if (tid == 0) atomicExch(f.tickets + tile_id, 0u);
 }
+#endif
 
 template <int N> struct NSlots { static constexpr int value = N; };
 
@@ -177,7 +184,9 @@ struct IgemmParams {
   int atomic_out;               // split-K without a workspace: accumulate into a zeroed output
   int64_t split_stride;         // split-K with one: blockIdx.y stores its partial sums at out + blockIdx.y * split_stride
   EpiParams epi;                // D is indexed like the output, with its own row stride
+#if AMOS_SPLIT_IN_KERNEL
   SplitFinish fin;              // split-K with slices: the last workgroup of a tile adds them
+#endif
 };
 
 __device__ __forceinline__ int lds_chunk_offset(int row, int chunk) {
@@ -550,6 +559,7 @@ __global__ __launch_bounds__(256) void amos_igemm(const IgemmParams p) {
       }
     }
   }
+#if AMOS_SPLIT_IN_KERNEL
   if (p.fin.tickets) {
     split_finish<out_t>(p.fin, (unsigned)(batch * gridDim.x + blockIdx.x), (const out_t*)p.out, t, 256, BI, BJ, (lds_flag_t)smem,
                         [&](int r, int c) -> int64_t {
@@ -560,6 +570,7 @@ __global__ __launch_bounds__(256) void amos_igemm(const IgemmParams p) {
                                  (int64_t)(j - jo * p.out_jmod) * p.out_sj;
                         });
   }
+#endif
 }
 
 template <int TI, int TJ>

@@ -194,10 +194,11 @@ for _ in range(2):   # the second pass finds every ticket counter back at zero
 '''
 
 
-@pytest.mark.skip(reason="AMOS_SPLIT_IN_KERNEL=1 (the last workgroup of a tile adds the slices, no second launch) is off by "
-                         "default and has not run on a GPU since its LDS flag word is named in the LDS address space: the "
-                         "first build cast LDS offset 0 to a generic pointer, which the compiler folds to the null pointer "
-                         "(a store to global address 0)")
+@pytest.mark.skip(reason="the in-kernel reduction (the last workgroup of a tile adds the slices, no second launch) is compiled "
+                         "in only with AMOS_BUILD_SPLIT_IN_KERNEL=1 and armed only with AMOS_SPLIT_IN_KERNEL=1; it has not run "
+                         "on a GPU since its LDS flag word is named in the LDS address space: the first build cast LDS "
+                         "offset 0 to a generic pointer, which the compiler folds to the null pointer (a store to global "
+                         "address 0)")
 def test_split_k_reduced_inside_the_kernel_gives_the_same_bits(gpu):
     """both reductions add the slices in the order of the splits: the same bits, on every kernel
     with that tail, also on a second pass (the counters are put back to zero)"""
